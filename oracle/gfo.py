@@ -1,0 +1,253 @@
+"""ctypes binding of the CPU oracle (libgfo.so) and of the compiled reference
+(_ref/libguffin_ref.so).  TEST INFRASTRUCTURE ONLY: imported by tests/,
+__graft_entry__.smoke() and the cpu_baseline leg of bench.py, never by guffin_amd.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+Q8_0, Q4_K, Q6_K = 0, 1, 2
+BLOCK_BYTES = {Q8_0: 34, Q4_K: 144, Q6_K: 210}
+BLOCK_ELEMS = {Q8_0: 32, Q4_K: 256, Q6_K: 256}
+
+token_logit = np.dtype([("token", np.uint32), ("logit", np.float32)])
+
+
+class SamplerOptions(C.Structure):
+    _fields_ = [("temperature", C.c_float), ("top_k", C.c_uint32), ("top_p", C.c_float),
+                ("min_p", C.c_float), ("repetition_penalty", C.c_float)]
+
+
+class Prepared(C.Structure):
+    _fields_ = [("count", C.c_uint32), ("pad", C.c_uint32), ("total_sampling_weight", C.c_double),
+                ("token", C.c_uint32 * 256), ("probability", C.c_double * 256),
+                ("sampling_weight", C.c_double * 256)]
+
+
+class DraftLaw(C.Structure):
+    _fields_ = [("count", C.c_uint32), ("pad", C.c_uint32), ("ids", C.c_uint32 * 256),
+                ("cdf", C.c_uint64 * 257)]
+
+
+class SpecResult(C.Structure):
+    _fields_ = [("accepted", C.c_uint32), ("token", C.c_uint32), ("next_root", C.c_uint32),
+                ("status", C.c_uint32), ("acceptance_probability", C.c_double),
+                ("residual_total", C.c_double), ("residual_count", C.c_uint32), ("pad", C.c_uint32)]
+
+
+class ModelConfig(C.Structure):
+    _fields_ = [(n, C.c_uint32) for n in
+                ("hidden", "ffn", "q_heads", "kv_heads", "head_dim", "layers", "vocab",
+                 "sliding_window", "global_period")] + \
+               [(n, C.c_float) for n in ("local_base", "global_base", "global_scale", "eps")] + \
+               [("ring_local", C.c_uint32), ("ring_global", C.c_uint32)]
+
+
+class Layer(C.Structure):
+    _fields_ = [("dtype", C.c_int * 7), ("w", C.c_void_p * 7), ("norm", C.c_void_p * 6),
+                ("ring_k", C.c_void_p), ("ring_v", C.c_void_p)]
+
+
+def build(force=False):
+    """Compile libgfo.so (and the reference library when the checkout is present)."""
+    if force or not os.path.exists(os.path.join(HERE, "libgfo.so")):
+        subprocess.check_call(["make", "-C", HERE, "-j8"], stdout=subprocess.DEVNULL)
+
+
+_lib = None
+_ref = None
+
+
+def _ptr(a):
+    return a.ctypes.data_as(C.c_void_p) if a is not None else None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        build()
+        _lib = C.CDLL(os.path.join(HERE, "libgfo.so"))
+        _lib.gfo_f16_to_f32.restype = C.c_float
+        _lib.gfo_f16_to_f32.argtypes = [C.c_uint16]
+        _lib.gfo_f32_to_f16_rne.restype = C.c_uint16
+        _lib.gfo_f32_to_f16_rne.argtypes = [C.c_float]
+        _lib.gfo_exp_f32.restype = C.c_float
+        _lib.gfo_exp_f32.argtypes = [C.c_float]
+        _lib.gfo_argmax.restype = C.c_uint32
+        _lib.gfo_draft_select.restype = C.c_uint32
+        _lib.gfo_draft_select_full.restype = C.c_uint32
+    return _lib
+
+
+def ref():
+    """The compiled reference, or None when oracle/_ref was not built."""
+    global _ref
+    if _ref is None:
+        path = os.path.join(HERE, "_ref", "libguffin_ref.so")
+        if not os.path.exists(path):
+            return None
+        _ref = C.CDLL(path)
+        _ref.gfr_f16_to_f32.restype = C.c_float
+        _ref.gfr_f16_to_f32.argtypes = [C.c_uint16]
+        _ref.gfr_argmax.restype = C.c_uint32
+        _ref.gfr_select_draft_token.restype = C.c_uint32
+    return _ref
+
+
+# ---- thin numpy wrappers -------------------------------------------------
+def _u8(a):
+    a = np.ascontiguousarray(a, dtype=np.uint8)
+    return a
+
+
+def dequant(dtype, blocks, which=None):
+    blocks = _u8(blocks)
+    n = blocks.size // BLOCK_BYTES[dtype]
+    out = np.empty(n * BLOCK_ELEMS[dtype], np.float32)
+    if which is None:
+        lib().gfo_dequant(dtype, _ptr(blocks), C.c_uint64(n), _ptr(out))
+    else:
+        assert which.gfr_dequant(dtype, _ptr(blocks), C.c_uint64(n), _ptr(out)) == 0
+    return out
+
+
+def gemv(dtype, w, x, N, threads=1, as_written=False, which=None):
+    w = _u8(w)
+    x = np.ascontiguousarray(x, np.float32).reshape(-1, x.shape[-1])
+    rows, K = x.shape
+    assert w.size == N * (K // BLOCK_ELEMS[dtype]) * BLOCK_BYTES[dtype]
+    y = np.empty((rows, N), np.float32)
+    if which is not None:
+        assert which.gfr_gemv(dtype, _ptr(w), _ptr(x), _ptr(y), rows, K, N) == 0
+    elif as_written:
+        lib().gfo_gemv_as_written(dtype, _ptr(w), _ptr(x), _ptr(y), rows, K, N)
+    else:
+        lib().gfo_gemv_mt(dtype, _ptr(w), _ptr(x), _ptr(y), rows, K, N, threads)
+    return y
+
+
+def rms_norm(x, gamma, eps=1e-6, residual=None):
+    x = np.ascontiguousarray(x, np.float32)
+    rows, width = x.reshape(-1, x.shape[-1]).shape
+    y = np.empty_like(x)
+    g = np.ascontiguousarray(gamma, np.float32)
+    if residual is None:
+        lib().gfo_rms_norm(_ptr(x), _ptr(g), _ptr(y), rows, width, C.c_float(eps))
+    else:
+        r = np.ascontiguousarray(residual, np.float32)
+        lib().gfo_rms_norm_add(_ptr(x), _ptr(g), _ptr(r), _ptr(y), rows, width, C.c_float(eps))
+    return y
+
+
+def rope_neox(x, positions, heads, head_dim, rope_dim, base, scale=1.0):
+    x = np.ascontiguousarray(x, np.float32)
+    rows = x.shape[0]
+    pos = np.ascontiguousarray(positions, np.uint32)
+    y = np.empty_like(x)
+    lib().gfo_rope_neox(_ptr(x), _ptr(y), _ptr(pos), rows, heads, head_dim, rope_dim,
+                        C.c_float(base), C.c_float(scale))
+    return y
+
+
+def kv_store_f16(raw_k, raw_v, positions, heads, head_dim, rope_dim, base, scale=1.0):
+    raw_k = np.ascontiguousarray(raw_k, np.float32)
+    raw_v = np.ascontiguousarray(raw_v, np.float32)
+    rows = raw_k.shape[0]
+    pos = np.ascontiguousarray(positions, np.uint32)
+    k = np.empty(raw_k.shape, np.uint16)
+    v = np.empty(raw_v.shape, np.uint16)
+    lib().gfo_kv_store_f16(_ptr(raw_k), _ptr(raw_v), _ptr(pos), _ptr(k), _ptr(v), rows, heads,
+                           head_dim, rope_dim, C.c_float(base), C.c_float(scale))
+    return k, v
+
+
+def geglu(gate, up):
+    gate = np.ascontiguousarray(gate, np.float32)
+    up = np.ascontiguousarray(up, np.float32)
+    out = np.empty_like(gate)
+    lib().gfo_geglu(_ptr(gate), _ptr(up), _ptr(out), C.c_uint64(gate.size))
+    return out
+
+
+def embed(dtype, w, tokens, width, scale):
+    w = _u8(w)
+    tokens = np.ascontiguousarray(tokens, np.uint32)
+    out = np.empty((tokens.size, width), np.float32)
+    lib().gfo_embed(dtype, _ptr(w), _ptr(tokens), _ptr(out), tokens.size, width, C.c_float(scale))
+    return out
+
+
+def attention(q, ring_k, ring_v, priv_k, priv_v, schedule, ancestors, row_mask, q_heads, kv_heads,
+              head_dim, scale):
+    q = np.ascontiguousarray(q, np.float32)
+    rows = q.shape[0]
+    out = np.empty_like(q)
+    sched = np.ascontiguousarray(schedule, np.uint32)
+    anc = np.ascontiguousarray(ancestors, np.uint32)
+    lib().gfo_attention(_ptr(q), _ptr(ring_k), _ptr(ring_v), _ptr(priv_k), _ptr(priv_v),
+                        _ptr(sched), _ptr(anc), _ptr(out), rows, row_mask, q_heads, kv_heads,
+                        head_dim, C.c_float(scale))
+    return out
+
+
+def select_candidates(logits, k, history=()):
+    logits = np.ascontiguousarray(logits, np.float32)
+    hist = np.ascontiguousarray(history, np.uint32)
+    out = np.zeros(k + hist.size, token_logit)
+    n = lib().gfo_select_candidates(_ptr(logits), logits.size, k, _ptr(hist), hist.size, _ptr(out))
+    if n < 0:
+        raise ValueError("non-finite selected logit")
+    return out[:n]
+
+
+def prepare(cands, opt, history=(), which=None):
+    cands = np.ascontiguousarray(cands, token_logit)
+    hist = np.ascontiguousarray(history, np.uint32)
+    out = Prepared()
+    fn = lib().gfo_prepare_token_distribution if which is None else which.gfr_prepare_token_distribution
+    rc = fn(_ptr(cands), cands.size, C.byref(opt), _ptr(hist), hist.size, C.byref(out))
+    return rc, out
+
+
+def draft_law_compact(logits, opt):
+    logits = np.ascontiguousarray(logits, np.float32)
+    law = DraftLaw()
+    rc = lib().gfo_draft_law_compact(_ptr(logits), logits.size, C.byref(opt), C.byref(law))
+    return rc, law
+
+
+def draft_law_full(logits, opt):
+    logits = np.ascontiguousarray(logits, np.float32)
+    cdf = np.zeros(logits.size + 1, np.uint64)
+    rc = lib().gfo_draft_law_full(_ptr(logits), logits.size, C.byref(opt), _ptr(cdf))
+    return rc, cdf
+
+
+def spec_accept(row0, row1, law, proposal, opt, u_accept, u_residual, u_next, which=None):
+    row0 = np.ascontiguousarray(row0, token_logit)
+    row1 = np.ascontiguousarray(row1, token_logit)
+    out = SpecResult()
+    fn = lib().gfo_spec_accept if which is None else which.gfr_spec_accept
+    rc = fn(_ptr(row0), row0.size, _ptr(row1), row1.size, C.byref(law), C.c_uint32(proposal),
+            C.byref(opt), C.c_double(u_accept), C.c_double(u_residual), C.c_double(u_next),
+            C.byref(out))
+    return rc, out
+
+
+def philox(counter, key):
+    c = (C.c_uint32 * 4)(*counter)
+    k = (C.c_uint32 * 2)(*key)
+    o = (C.c_uint32 * 4)()
+    lib().gfo_philox4x32_10(c, k, o)
+    return list(o)
+
+
+def step_draws(seed, step):
+    w = C.c_uint32()
+    a, r, n = C.c_double(), C.c_double(), C.c_double()
+    lib().gfo_step_draws(C.c_uint64(seed), C.c_uint64(step), C.byref(w), C.byref(a), C.byref(r),
+                         C.byref(n))
+    return w.value, a.value, r.value, n.value

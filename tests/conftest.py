@@ -1,0 +1,25 @@
+import os
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
+
+
+@pytest.fixture(scope="session")
+def gfo():
+    from oracle import gfo as module
+    module.build()
+    return module
+
+
+@pytest.fixture(scope="session")
+def ref(gfo):
+    """The compiled reference sources; None where oracle/_ref was not built."""
+    return gfo.ref()
