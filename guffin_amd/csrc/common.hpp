@@ -1,0 +1,105 @@
+// Shared device helpers for the gfx950 kernels of the H1 step.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/guffin_hip.h"
+
+namespace guffin {
+
+constexpr int kWave = 64;
+
+// ---- error plumbing (host) -------------------------------------------------
+void set_last_error(const char* message);
+int fail(int code, const char* message);
+int check_launch(const char* what);
+
+inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
+
+// ---- typed loads at the alignment a GGUF block stream guarantees ------------
+struct __attribute__((packed, aligned(4))) U4a4 { uint32_t x, y, z, w; };
+struct __attribute__((packed, aligned(2))) U4a2 { uint32_t x, y, z, w; };
+struct __attribute__((packed, aligned(2))) U2a2 { uint32_t x, y; };
+struct __attribute__((packed, aligned(4))) F4a4 { float x, y, z, w; };
+
+__device__ __forceinline__ uint4 ld16_a4(const uint8_t* p) {
+    const U4a4 t = *reinterpret_cast<const U4a4*>(p);
+    return make_uint4(t.x, t.y, t.z, t.w);
+}
+__device__ __forceinline__ uint4 ld16_a2(const uint8_t* p) {
+    const U4a2 t = *reinterpret_cast<const U4a2*>(p);
+    return make_uint4(t.x, t.y, t.z, t.w);
+}
+__device__ __forceinline__ uint2 ld8_a2(const uint8_t* p) {
+    const U2a2 t = *reinterpret_cast<const U2a2*>(p);
+    return make_uint2(t.x, t.y);
+}
+__device__ __forceinline__ float4 ldf4_a4(const float* p) {
+    const F4a4 t = *reinterpret_cast<const F4a4*>(p);
+    return make_float4(t.x, t.y, t.z, t.w);
+}
+__device__ __forceinline__ uint32_t ld_u16(const uint8_t* p) { return *reinterpret_cast<const uint16_t*>(p); }
+
+// fp16 bits -> fp32, exact (IEEE widening, subnormals included)
+__device__ __forceinline__ float h2f(uint32_t bits) {
+    return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<unsigned short>(bits)));
+}
+
+// Hides a value from the optimiser so that a following (v >> 8k) & 0xFF selects
+// v_cvt_f32_ubyteK instead of being re-derived from the unmasked source.
+__device__ __forceinline__ uint32_t opaque(uint32_t v) {
+    asm volatile("" : "+v"(v));
+    return v;
+}
+__device__ __forceinline__ float ub0(uint32_t v) { return static_cast<float>(v & 0xFFu); }
+__device__ __forceinline__ float ub1(uint32_t v) { return static_cast<float>((v >> 8) & 0xFFu); }
+__device__ __forceinline__ float ub2(uint32_t v) { return static_cast<float>((v >> 16) & 0xFFu); }
+__device__ __forceinline__ float ub3(uint32_t v) { return static_cast<float>(v >> 24); }
+__device__ __forceinline__ float sb0(uint32_t v) { return static_cast<float>(static_cast<int8_t>(v)); }
+__device__ __forceinline__ float sb1(uint32_t v) { return static_cast<float>(static_cast<int8_t>(v >> 8)); }
+__device__ __forceinline__ float sb2(uint32_t v) { return static_cast<float>(static_cast<int8_t>(v >> 16)); }
+__device__ __forceinline__ float sb3(uint32_t v) { return static_cast<float>(static_cast<int8_t>(v >> 24)); }
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int s = 32; s > 0; s >>= 1) v += __shfl_xor(v, s, kWave);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int s = 32; s > 0; s >>= 1) v = fmaxf(v, __shfl_xor(v, s, kWave));
+    return v;
+}
+
+// Reduces NV per-lane values across the 64 lanes with NV-1 + (6 - log2 NV) exchanges
+// instead of 6*NV: at each level the upper half-wave keeps one half of the values and
+// the lower half-wave the other.  Afterwards v[0] on lane l holds the wave total of
+// value index l >> (6 - log2 NV); the summation order is fixed, so results repeat.
+template <int NV>
+__device__ __forceinline__ void wave_reduce_multi(float (&v)[NV], int lane) {
+    static_assert(NV >= 1 && NV <= 64 && (NV & (NV - 1)) == 0, "NV must be a power of two");
+    int stride = 32;
+#pragma unroll
+    for (int m = NV; m > 1; m >>= 1) {
+        const int half = m >> 1;
+        const bool upper = (lane & stride) != 0;
+#pragma unroll
+        for (int i = 0; i < half; ++i) {
+            const float send = upper ? v[i] : v[i + half];
+            const float keep = upper ? v[i + half] : v[i];
+            v[i] = keep + __shfl_xor(send, stride, kWave);
+        }
+        stride >>= 1;
+    }
+#pragma unroll
+    for (; stride > 0; stride >>= 1) v[0] += __shfl_xor(v[0], stride, kWave);
+}
+
+template <int NV>
+__device__ __forceinline__ constexpr int reduce_multi_shift() {
+    int s = 6, n = NV;
+    while (n > 1) { n >>= 1; --s; }
+    return s;
+}
+
+}  // namespace guffin
