@@ -29,6 +29,7 @@ int check_launch(const char* what) {
 
 int gemv_init(int cu_count);
 int ops_init(int cu_count);
+void gemv_packed_init(int cu_count);
 
 }  // namespace guffin
 
@@ -53,5 +54,6 @@ extern "C" int guffin_hip_init(int device) {
     }
     if (gemv_init(prop.multiProcessorCount) != 0 || ops_init(prop.multiProcessorCount) != 0)
         return fail(GUFFIN_E_HIP, "init: could not raise a kernel's dynamic LDS limit");
+    gemv_packed_init(prop.multiProcessorCount);
     return GUFFIN_OK;
 }

@@ -1,0 +1,434 @@
+// Wave-tile weight layout and the dequant-GEMV that streams it (gfx950, wavefront 64).
+//
+// Role in the reference: the Metal backend re-lays K-quant weights once at upload into a
+// "columns8" order for its SIMD-group loads and keeps that repack lossless
+// (src/tensor/kquant_packing.hpp:9-23, src/tensor/kquant_packing.cpp).  This file is the
+// CDNA counterpart: a lossless repack into 64-column wave tiles plus the GEMV kernels
+// (replacing src/tensor/backends/metal/metal_kernels.mm:551-750, 788-922, 267-436) that
+// consume it.
+//
+// Tile = 64 adjacent output columns x one block along K.  Inside a tile every 16-byte
+// piece of a block is stored lane-major: piece p of column l sits at p*1024 + l*16, so a
+// wave reads each piece with one fully coalesced 1 KiB load and lane l ends up with its
+// own column's bytes.  Tiles of one column group are consecutive along K.
+//   Q4_K  9216 B : piece 0 = {d, dmin, 12 scale bytes}, pieces 1..8 = quants
+//   Q6_K 13440 B : pieces 0..7 = ql, 8..11 = qh, 12 = 16 int8 scales, then 64 x fp16 d
+//   Q8_0  2176 B : pieces 0..1 = quants, then 64 x fp16 d
+//
+// GEMV: lane l owns output column 64*tile + l for a slice of K.  All lanes walk the same
+// k, so activations are wave-uniform and are read through the scalar cache straight into
+// FMA operands; no LDS, no barrier, no cross-lane reduction.  Quants are spread into
+// 16-bit fields and fed to v_fma_mix_f32 as fp16 subnormals (an integer n < 1024 in a
+// half is exactly n*2^-24), which replaces convert+FMA by one FMA per weight per row with
+// bit-identical products; the 2^24 is folded into the block scale.  The offset terms
+// (-dmin*m for Q4_K, -32 for Q6_K, -128 for the biased Q8_0 bytes) use per-16 / per-32
+// activation sums supplied by the producer of x.  K is cut into S slices across
+// workgroups; slice partials go to [S][rows][N] and are summed in slice order by the
+// consumer (or by reduce_partials below), so results are deterministic and a row's
+// arithmetic does not depend on how many rows are computed.
+#include "common.hpp"
+
+namespace guffin {
+namespace {
+
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+
+constexpr uint32_t kTileCols = 64;
+
+__host__ __device__ constexpr uint32_t block_bytes(int dtype) {
+    return dtype == GUFFIN_Q8_0 ? 34u : dtype == GUFFIN_Q4_K ? 144u : 210u;
+}
+__host__ __device__ constexpr uint32_t block_elems(int dtype) { return dtype == GUFFIN_Q8_0 ? 32u : 256u; }
+
+// offset of canonical block byte `o` (even) of lane `l` inside its tile
+template <int DTYPE>
+__device__ __forceinline__ uint32_t tile_offset(uint32_t o, uint32_t l) {
+    if constexpr (DTYPE == GUFFIN_Q4_K) {
+        return (o >> 4) * 1024u + l * 16u + (o & 15u);
+    } else if constexpr (DTYPE == GUFFIN_Q6_K) {
+        return o < 208u ? (o >> 4) * 1024u + l * 16u + (o & 15u) : 13312u + l * 2u + (o - 208u);
+    } else {
+        if (o < 2u) return 2048u + l * 2u + o;
+        const uint32_t q = o - 2u;
+        return (q >> 4) * 1024u + l * 16u + (q & 15u);
+    }
+}
+
+// One thread moves one 16-bit word (every field of every block is 2-byte aligned on both sides).
+template <int DTYPE, bool TO_TILES>
+__global__ void repack_kernel(const uint16_t* __restrict__ src, uint16_t* __restrict__ dst,
+                              uint32_t nblk, uint64_t total_words) {
+    constexpr uint32_t BB = block_bytes(DTYPE), WPB = BB / 2;
+    const uint64_t stride = uint64_t(gridDim.x) * blockDim.x;
+    for (uint64_t i = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x; i < total_words; i += stride) {
+        // canonical word index -> (column, block, word in block)
+        const uint64_t blk = i / WPB;
+        const uint32_t wd = static_cast<uint32_t>(i - blk * WPB);
+        const uint64_t col = blk / nblk;
+        const uint32_t b = static_cast<uint32_t>(blk - col * nblk);
+        const uint64_t tile = (col / kTileCols) * nblk + b;
+        const uint32_t lane = static_cast<uint32_t>(col % kTileCols);
+        const uint64_t t = tile * (uint64_t(kTileCols) * WPB) + tile_offset<DTYPE>(wd * 2u, lane) / 2u;
+        if (TO_TILES) dst[t] = src[i];
+        else dst[i] = src[t];
+    }
+}
+
+// xsums[r][0 .. K/16) = sums of 16 consecutive activations, xsums[r][K/16 .. 3K/32) = sums of 32.
+__global__ void group_sums_kernel(const float* __restrict__ x, float* __restrict__ xsums, uint32_t K, uint32_t rows) {
+    const uint32_t n16 = K / 16, per_row = n16 + K / 32;
+    for (uint32_t g = blockIdx.x * blockDim.x + threadIdx.x; g < rows * n16; g += gridDim.x * blockDim.x) {
+        const uint32_t r = g / n16, i = g - r * n16;
+        const float* p = x + size_t(r) * K + i * 16u;
+        float s = 0.f;
+#pragma unroll
+        for (int k = 0; k < 16; ++k) s += p[k];
+        xsums[r * per_row + i] = s;
+        // the 32-sum is the sum of its two 16-sums, taken by the even thread of the pair
+        const float other = __shfl_xor(s, 1, kWave);
+        if ((i & 1u) == 0) xsums[r * per_row + n16 + (i >> 1)] = s + other;
+    }
+}
+
+__global__ void reduce_partials_kernel(const float* __restrict__ part, float* __restrict__ y, uint32_t S, uint32_t count) {
+    for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < count; i += gridDim.x * blockDim.x) {
+        float t = part[i];
+        for (uint32_t s = 1; s < S; ++s) t += part[size_t(s) * count + i];
+        y[i] = t;
+    }
+}
+
+// ---- fp16-subnormal FMA helpers -------------------------------------------------------
+// `packed` holds two integers < 1024 in its 16-bit halves; adds lo*x0 + hi*x1 (times 2^-24).
+__device__ __forceinline__ void mix2(float& acc, uint32_t packed, float x0, float x1) {
+    const half2_t h = __builtin_bit_cast(half2_t, packed);
+    acc = fmaf(static_cast<float>(h.x), x0, acc);
+    acc = fmaf(static_cast<float>(h.y), x1, acc);
+}
+// bytes {0,2} and {1,3} of v as 16-bit fields
+__device__ __forceinline__ uint32_t even_bytes(uint32_t v) { return __builtin_amdgcn_perm(0u, v, 0x0c020c00u); }
+__device__ __forceinline__ uint32_t odd_bytes(uint32_t v) { return __builtin_amdgcn_perm(0u, v, 0x0c030c01u); }
+
+constexpr float kTwo24 = 16777216.0f;      // 2^24: undoes the subnormal scale
+constexpr float kTwo20 = 1048576.0f;       // 2^20: same for fields holding 16*q
+
+// =======================================================================================
+// Q4_K
+// =======================================================================================
+struct Q4Tile { uint4 hdr; uint4 q[8]; };
+
+__device__ __forceinline__ void load_tile(Q4Tile& t, const uint8_t* p) {
+    t.hdr = *reinterpret_cast<const uint4*>(p);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) t.q[i] = *reinterpret_cast<const uint4*>(p + 1024 * (i + 1));
+}
+
+template <int R>
+__device__ __forceinline__ void compute_tile(const Q4Tile& t, const float* __restrict__ x, const float* __restrict__ xs32,
+                                             uint32_t K, uint32_t per_row, float (&acc)[R]) {
+    // x, xs32 point at this block's 256 activations / 8 group sums of row 0
+    const float d = h2f(t.hdr.x & 0xFFFFu), dmin = h2f(t.hdr.x >> 16);
+    const uint32_t s0 = t.hdr.y, s1 = t.hdr.z, s2 = t.hdr.w;
+    const uint32_t sc_a = s0 & 0x3F3F3F3Fu, mn_a = s1 & 0x3F3F3F3Fu;
+    const uint32_t sc_b = (s2 & 0x0F0F0F0Fu) | ((s0 >> 2) & 0x30303030u);
+    const uint32_t mn_b = ((s2 >> 4) & 0x0F0F0F0Fu) | ((s1 >> 2) & 0x30303030u);
+    const float d_lo = d * kTwo24, d_hi = d * kTwo20;
+    float mt[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) mt[r] = 0.f;
+#pragma unroll
+    for (int J = 0; J < 4; ++J) {  // sub-block of 64: groups 2J (low nibbles) and 2J+1 (high)
+        float plo[R], phi[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) { plo[r] = 0.f; phi[r] = 0.f; }
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+            const uint4 qv = t.q[2 * J + half];
+            const uint32_t qd[4] = {qv.x, qv.y, qv.z, qv.w};
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const uint32_t w = qd[k], w8 = w >> 8;
+                const uint32_t a = w & 0x000F000Fu, b = w & 0x00F000F0u;    // bytes 0,2: low / 16*high
+                const uint32_t c = w8 & 0x000F000Fu, e = w8 & 0x00F000F0u;  // bytes 1,3
+                const int e0 = 64 * J + 16 * half + 4 * k;
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    const float* xr = x + size_t(r) * K;
+                    mix2(plo[r], a, xr[e0], xr[e0 + 2]);
+                    mix2(plo[r], c, xr[e0 + 1], xr[e0 + 3]);
+                    mix2(phi[r], b, xr[e0 + 32], xr[e0 + 34]);
+                    mix2(phi[r], e, xr[e0 + 33], xr[e0 + 35]);
+                }
+            }
+        }
+        const uint32_t scw = J < 2 ? sc_a : sc_b, mnw = J < 2 ? mn_a : mn_b;
+        const float sc_lo = (J & 1) ? ub2(scw) : ub0(scw), sc_hi = (J & 1) ? ub3(scw) : ub1(scw);
+        const float mn_lo = (J & 1) ? ub2(mnw) : ub0(mnw), mn_hi = (J & 1) ? ub3(mnw) : ub1(mnw);
+        const float f_lo = d_lo * sc_lo, f_hi = d_hi * sc_hi;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            acc[r] = fmaf(f_lo, plo[r], acc[r]);
+            acc[r] = fmaf(f_hi, phi[r], acc[r]);
+            mt[r] = fmaf(mn_lo, xs32[r * per_row + 2 * J], mt[r]);
+            mt[r] = fmaf(mn_hi, xs32[r * per_row + 2 * J + 1], mt[r]);
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) acc[r] = fmaf(-dmin, mt[r], acc[r]);
+}
+
+// =======================================================================================
+// Q6_K
+// =======================================================================================
+struct Q6Tile { uint4 ql[8]; uint4 qh[4]; uint4 sc; uint32_t d; };
+
+__device__ __forceinline__ void load_tile(Q6Tile& t, const uint8_t* p, uint32_t lane) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) t.ql[i] = *reinterpret_cast<const uint4*>(p + 1024 * i);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) t.qh[i] = *reinterpret_cast<const uint4*>(p + 8192 + 1024 * i);
+    t.sc = *reinterpret_cast<const uint4*>(p + 12288);
+    t.d = *reinterpret_cast<const uint16_t*>(p - lane * 16 + 13312 + lane * 2);
+}
+
+template <int R>
+__device__ __forceinline__ void compute_tile(const Q6Tile& t, const float* __restrict__ x, const float* __restrict__ xs16,
+                                             uint32_t K, uint32_t per_row, float (&acc)[R]) {
+    const float d24 = h2f(t.d) * kTwo24;
+    const float bias = -32.0f / kTwo24;  // sum (q-32) x = sum q x - 32 sum x, in the subnormal scale
+    const uint32_t scw[4] = {t.sc.x, t.sc.y, t.sc.z, t.sc.w};
+#pragma unroll
+    for (int p = 0; p < 8; ++p) {  // ql piece p: half h, 16-byte run tt
+        const int h = p >> 2, tt = p & 3;
+        const uint4 qlv = t.ql[p], qhv = t.qh[h * 2 + (tt & 1)];
+        const uint32_t ql[4] = {qlv.x, qlv.y, qlv.z, qlv.w}, qh[4] = {qhv.x, qhv.y, qhv.z, qhv.w};
+        const int s_lo = 2 * (tt >> 1), s_hi = 4 + 2 * (tt >> 1);
+        const int e_lo = h * 128 + 32 * (tt >> 1) + 16 * (tt & 1), e_hi = e_lo + 64;
+        const int g_lo = h * 8 + tt, g_hi = g_lo + 4;  // 16-element scale groups
+        float plo[R], phi[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            plo[r] = bias * xs16[r * per_row + g_lo];
+            phi[r] = bias * xs16[r * per_row + g_hi];
+        }
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const uint32_t vlo = (ql[k] & 0x0F0F0F0Fu) | (((qh[k] >> s_lo) & 0x03030303u) << 4);
+            const uint32_t vhi = ((ql[k] >> 4) & 0x0F0F0F0Fu) | (((qh[k] >> s_hi) & 0x03030303u) << 4);
+            const uint32_t a = even_bytes(vlo), c = odd_bytes(vlo), b = even_bytes(vhi), e = odd_bytes(vhi);
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                const float* xr = x + size_t(r) * K;
+                mix2(plo[r], a, xr[e_lo + 4 * k], xr[e_lo + 4 * k + 2]);
+                mix2(plo[r], c, xr[e_lo + 4 * k + 1], xr[e_lo + 4 * k + 3]);
+                mix2(phi[r], b, xr[e_hi + 4 * k], xr[e_hi + 4 * k + 2]);
+                mix2(phi[r], e, xr[e_hi + 4 * k + 1], xr[e_hi + 4 * k + 3]);
+            }
+        }
+        const uint32_t wlo = scw[g_lo >> 2], whi = scw[g_hi >> 2];
+        const float f_lo = d24 * ((g_lo & 3) == 0 ? sb0(wlo) : (g_lo & 3) == 1 ? sb1(wlo) : (g_lo & 3) == 2 ? sb2(wlo) : sb3(wlo));
+        const float f_hi = d24 * ((g_hi & 3) == 0 ? sb0(whi) : (g_hi & 3) == 1 ? sb1(whi) : (g_hi & 3) == 2 ? sb2(whi) : sb3(whi));
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            acc[r] = fmaf(f_lo, plo[r], acc[r]);
+            acc[r] = fmaf(f_hi, phi[r], acc[r]);
+        }
+    }
+}
+
+// =======================================================================================
+// Q8_0
+// =======================================================================================
+struct Q8Tile { uint4 q[2]; uint32_t d; };
+
+__device__ __forceinline__ void load_tile(Q8Tile& t, const uint8_t* p, uint32_t lane) {
+    t.q[0] = *reinterpret_cast<const uint4*>(p);
+    t.q[1] = *reinterpret_cast<const uint4*>(p + 1024);
+    t.d = *reinterpret_cast<const uint16_t*>(p - lane * 16 + 2048 + lane * 2);
+}
+
+template <int R>
+__device__ __forceinline__ void compute_tile(const Q8Tile& t, const float* __restrict__ x, const float* __restrict__ xs32,
+                                             uint32_t K, uint32_t per_row, float (&acc)[R]) {
+    const float d24 = h2f(t.d) * kTwo24;
+    const float bias = -128.0f / kTwo24;  // bytes are biased to q+128
+    float p[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) p[r] = bias * xs32[r * per_row];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const uint32_t qd[4] = {t.q[i].x, t.q[i].y, t.q[i].z, t.q[i].w};
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const uint32_t u = qd[k] ^ 0x80808080u;
+            const uint32_t a = even_bytes(u), c = odd_bytes(u);
+            const int e0 = 16 * i + 4 * k;
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                const float* xr = x + size_t(r) * K;
+                mix2(p[r], a, xr[e0], xr[e0 + 2]);
+                mix2(p[r], c, xr[e0 + 1], xr[e0 + 3]);
+            }
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) acc[r] = fmaf(d24, p[r], acc[r]);
+}
+
+// =======================================================================================
+// The streaming kernel: one wave = one (column tile, k-slice)
+// =======================================================================================
+template <int DTYPE, int R>
+__global__ void __launch_bounds__(64)
+gemv_packed_kernel(const uint8_t* __restrict__ wt, const float* __restrict__ x, const float* __restrict__ xsums,
+                   float* __restrict__ part, uint32_t K, uint32_t N, uint32_t nblk, uint32_t bps) {
+    constexpr uint32_t TB = kTileCols * block_bytes(DTYPE), BE = block_elems(DTYPE);
+    const uint32_t lane = threadIdx.x, ct = blockIdx.x, slice = blockIdx.y;
+    const uint32_t b0 = slice * bps, b1 = b0 + bps < nblk ? b0 + bps : nblk;
+    const uint32_t n16 = K / 16, per_row = n16 + K / 32;
+    // Q6_K consumes 16-sums (16 per block), Q4_K 32-sums (8 per block), Q8_0 one 32-sum per block
+    const float* xs = DTYPE == GUFFIN_Q6_K ? xsums : xsums + n16;
+    constexpr uint32_t sums_per_block = DTYPE == GUFFIN_Q6_K ? 16 : DTYPE == GUFFIN_Q4_K ? 8 : 1;
+    const uint8_t* tp = wt + (size_t(ct) * nblk + b0) * TB + lane * 16;
+    float acc[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) acc[r] = 0.f;
+
+    if constexpr (DTYPE == GUFFIN_Q4_K) {
+        Q4Tile cur, nxt;
+        if (b0 < b1) load_tile(cur, tp);
+        for (uint32_t b = b0; b < b1; ++b) {
+            if (b + 1 < b1) load_tile(nxt, tp + size_t(b + 1 - b0) * TB);
+            compute_tile<R>(cur, x + size_t(b) * BE, xs + b * sums_per_block, K, per_row, acc);
+            cur = nxt;
+        }
+    } else if constexpr (DTYPE == GUFFIN_Q6_K) {
+        Q6Tile cur, nxt;
+        if (b0 < b1) load_tile(cur, tp, lane);
+        for (uint32_t b = b0; b < b1; ++b) {
+            if (b + 1 < b1) load_tile(nxt, tp + size_t(b + 1 - b0) * TB, lane);
+            compute_tile<R>(cur, x + size_t(b) * BE, xs + b * sums_per_block, K, per_row, acc);
+            cur = nxt;
+        }
+    } else {
+        Q8Tile cur, nxt;
+        if (b0 < b1) load_tile(cur, tp, lane);
+        for (uint32_t b = b0; b < b1; ++b) {
+            if (b + 1 < b1) load_tile(nxt, tp + size_t(b + 1 - b0) * TB, lane);
+            compute_tile<R>(cur, x + size_t(b) * BE, xs + b * sums_per_block, K, per_row, acc);
+            cur = nxt;
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) part[(size_t(slice) * R + r) * N + ct * kTileCols + lane] = acc[r];
+}
+
+int g_cus = 256;
+
+// k-slices: about four waves per SIMD over the whole chip (fine grains balance the
+// SIMDs and let compute start while later slices are still streaming); matrices with
+// more tiles than that walk K inside the wave with the next tile's loads in flight.
+uint32_t choose_slices(int dtype, uint32_t K, uint32_t N) {
+    const uint32_t nblk = K / block_elems(dtype), tiles = N / kTileCols;
+    const uint32_t target_waves = g_cus * 4 * 4;
+    uint32_t S = (target_waves + tiles - 1) / tiles;
+    if (S > nblk) S = nblk;
+    if (S > 64) S = 64;
+    if (S < 1) S = 1;
+    const uint32_t bps = (nblk + S - 1) / S;
+    return (nblk + bps - 1) / bps;  // no empty slices
+}
+
+template <int DTYPE>
+int launch_packed(hipStream_t s, const uint8_t* w, const float* x, const float* xsums, float* part,
+                  uint32_t rows, uint32_t K, uint32_t N, uint32_t S) {
+    const uint32_t nblk = K / block_elems(DTYPE), bps = (nblk + S - 1) / S;
+    const dim3 grid(N / kTileCols, S);
+    if (rows == 2)
+        hipLaunchKernelGGL((gemv_packed_kernel<DTYPE, 2>), grid, dim3(64), 0, s, w, x, xsums, part, K, N, nblk, bps);
+    else
+        hipLaunchKernelGGL((gemv_packed_kernel<DTYPE, 1>), grid, dim3(64), 0, s, w, x, xsums, part, K, N, nblk, bps);
+    return check_launch("gemv_packed");
+}
+
+}  // namespace
+
+void gemv_packed_init(int cu_count) { g_cus = cu_count > 0 ? cu_count : 256; }
+
+}  // namespace guffin
+
+using namespace guffin;
+
+static int check_packed_shape(const char* what, int dtype, uint32_t K, uint32_t N) {
+    if (dtype < GUFFIN_Q8_0 || dtype > GUFFIN_Q6_K) return fail(GUFFIN_E_ARG, what);
+    if (K == 0 || N == 0 || K % block_elems(dtype) != 0 || N % kTileCols != 0) return fail(GUFFIN_E_SHAPE, what);
+    return GUFFIN_OK;
+}
+
+extern "C" uint64_t guffin_hip_packed_bytes(int dtype, uint32_t K, uint32_t N) {
+    if (check_packed_shape("packed_bytes: need K % block == 0 and N % 64 == 0", dtype, K, N)) return 0;
+    return uint64_t(N) * (K / block_elems(dtype)) * block_bytes(dtype);
+}
+
+static int repack_common(void* stream, int dtype, const void* src, void* dst, uint32_t K, uint32_t N, bool to_tiles) {
+    if (!src || !dst) return fail(GUFFIN_E_ARG, "repack: null pointer");
+    if (int rc = check_packed_shape("repack: need K % block == 0 and N % 64 == 0", dtype, K, N)) return rc;
+    if ((reinterpret_cast<uintptr_t>(to_tiles ? dst : src) & 15u) || (reinterpret_cast<uintptr_t>(to_tiles ? src : dst) & 1u))
+        return fail(GUFFIN_E_ALIGN, "repack: tiles must be 16-byte aligned, the canonical stream 2-byte aligned");
+    const uint32_t nblk = K / block_elems(dtype);
+    const uint64_t words = uint64_t(N) * nblk * block_bytes(dtype) / 2;
+    const uint32_t grid = static_cast<uint32_t>(words / 256 < 262144 ? (words + 255) / 256 : 262144);
+    const uint16_t* s16 = static_cast<const uint16_t*>(src);
+    uint16_t* d16 = static_cast<uint16_t*>(dst);
+    hipStream_t s = as_stream(stream);
+#define GUFFIN_REPACK(DT)                                                                                   \
+    if (to_tiles) hipLaunchKernelGGL((repack_kernel<DT, true>), dim3(grid), dim3(256), 0, s, s16, d16, nblk, words); \
+    else hipLaunchKernelGGL((repack_kernel<DT, false>), dim3(grid), dim3(256), 0, s, s16, d16, nblk, words)
+    if (dtype == GUFFIN_Q4_K) { GUFFIN_REPACK(GUFFIN_Q4_K); }
+    else if (dtype == GUFFIN_Q6_K) { GUFFIN_REPACK(GUFFIN_Q6_K); }
+    else { GUFFIN_REPACK(GUFFIN_Q8_0); }
+#undef GUFFIN_REPACK
+    return check_launch("repack");
+}
+
+extern "C" int guffin_hip_repack(void* stream, int dtype, const void* canonical, void* tiles, uint32_t K, uint32_t N) {
+    return repack_common(stream, dtype, canonical, tiles, K, N, true);
+}
+
+extern "C" int guffin_hip_unpack(void* stream, int dtype, const void* tiles, void* canonical, uint32_t K, uint32_t N) {
+    return repack_common(stream, dtype, tiles, canonical, K, N, false);
+}
+
+extern "C" int guffin_hip_group_sums(void* stream, const float* x, float* xsums, uint32_t rows, uint32_t K) {
+    if (!x || !xsums) return fail(GUFFIN_E_ARG, "group_sums: null pointer");
+    if (rows == 0 || K == 0 || K % 32 != 0) return fail(GUFFIN_E_SHAPE, "group_sums: K must be a positive multiple of 32");
+    const uint32_t n = rows * (K / 16);
+    hipLaunchKernelGGL(group_sums_kernel, dim3((n + 255) / 256), dim3(256), 0, as_stream(stream), x, xsums, K, rows);
+    return check_launch("group_sums");
+}
+
+extern "C" uint32_t guffin_hip_gemv_packed_slices(int dtype, uint32_t K, uint32_t N) {
+    if (check_packed_shape("gemv_packed_slices: need K % block == 0 and N % 64 == 0", dtype, K, N)) return 0;
+    return choose_slices(dtype, K, N);
+}
+
+extern "C" int guffin_hip_gemv_packed(void* stream, int dtype, const void* tiles, const float* x, const float* xsums,
+                                      float* partials, float* y, uint32_t rows, uint32_t K, uint32_t N) {
+    if (!tiles || !x || !xsums || !partials) return fail(GUFFIN_E_ARG, "gemv_packed: null pointer");
+    if (int rc = check_packed_shape("gemv_packed: need K % block == 0 and N % 64 == 0", dtype, K, N)) return rc;
+    if (rows == 0 || rows > 2) return fail(GUFFIN_E_SHAPE, "gemv_packed: rows must be 1 or 2");
+    if (reinterpret_cast<uintptr_t>(tiles) & 15u) return fail(GUFFIN_E_ALIGN, "gemv_packed: tiles must be 16-byte aligned");
+    if ((reinterpret_cast<uintptr_t>(x) & 3u) || (reinterpret_cast<uintptr_t>(xsums) & 3u) || (reinterpret_cast<uintptr_t>(partials) & 3u))
+        return fail(GUFFIN_E_ALIGN, "gemv_packed: fp32 pointers must be 4-byte aligned");
+    const uint32_t S = choose_slices(dtype, K, N);
+    const uint8_t* w = static_cast<const uint8_t*>(tiles);
+    hipStream_t s = as_stream(stream);
+    int rc;
+    if (dtype == GUFFIN_Q4_K) rc = launch_packed<GUFFIN_Q4_K>(s, w, x, xsums, partials, rows, K, N, S);
+    else if (dtype == GUFFIN_Q6_K) rc = launch_packed<GUFFIN_Q6_K>(s, w, x, xsums, partials, rows, K, N, S);
+    else rc = launch_packed<GUFFIN_Q8_0>(s, w, x, xsums, partials, rows, K, N, S);
+    if (rc || !y) return rc;
+    const uint32_t count = rows * N;
+    hipLaunchKernelGGL(reduce_partials_kernel, dim3((count + 255) / 256), dim3(256), 0, s, partials, y, S, count);
+    return check_launch("reduce_partials");
+}

@@ -68,3 +68,45 @@ def gemv(dtype, w, x, N, out=None):
         out = torch.empty((rows, N), dtype=torch.float32, device=x.device)
     check(lib().guffin_hip_gemv(_stream(), dtype, _p(w), _p(x), _p(out), rows, K, N))
     return out
+
+
+def packed_bytes(dtype, K, N):
+    lib().guffin_hip_packed_bytes.restype = C.c_uint64
+    return lib().guffin_hip_packed_bytes(dtype, K, N)
+
+
+def repack(dtype, canonical, K, N):
+    tiles = torch.empty_like(canonical)
+    check(lib().guffin_hip_repack(_stream(), dtype, _p(canonical), _p(tiles), K, N))
+    return tiles
+
+
+def unpack(dtype, tiles, K, N):
+    canonical = torch.empty_like(tiles)
+    check(lib().guffin_hip_unpack(_stream(), dtype, _p(tiles), _p(canonical), K, N))
+    return canonical
+
+
+def group_sums(x, out=None):
+    rows, K = x.shape
+    if out is None:
+        out = torch.empty((rows, K // 16 + K // 32), dtype=torch.float32, device=x.device)
+    check(lib().guffin_hip_group_sums(_stream(), _p(x), _p(out), rows, K))
+    return out
+
+
+def gemv_packed_slices(dtype, K, N):
+    lib().guffin_hip_gemv_packed_slices.restype = C.c_uint32
+    return lib().guffin_hip_gemv_packed_slices(dtype, K, N)
+
+
+def gemv_packed(dtype, tiles, x, xsums, N, partials=None, out=None, reduce=True):
+    rows, K = x.shape
+    S = gemv_packed_slices(dtype, K, N)
+    if partials is None:
+        partials = torch.empty((S, rows, N), dtype=torch.float32, device=x.device)
+    if reduce and out is None:
+        out = torch.empty((rows, N), dtype=torch.float32, device=x.device)
+    check(lib().guffin_hip_gemv_packed(_stream(), dtype, _p(tiles), _p(x), _p(xsums), _p(partials),
+                                       _p(out) if reduce else C.c_void_p(0), rows, K, N))
+    return out if reduce else partials

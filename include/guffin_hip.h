@@ -74,6 +74,29 @@ int guffin_hip_gemv_q6k(void* stream, const void* w, const float* x, float* y,
 int guffin_hip_gemv_q80(void* stream, const void* w, const float* x, float* y,
                         uint32_t rows, uint32_t K, uint32_t N);
 
+/* ---- wave-tile weights (lossless repack) and the GEMV that streams them ------------------
+ * The reference re-lays K-quant weights at upload into a layout its GPU loads coalesce on
+ * and keeps the repack lossless (src/tensor/kquant_packing.hpp:9-23; round trip pinned in
+ * tests/tensor/tensor_tests.cpp:3193-3283).  This is the gfx950 counterpart: tiles of 64
+ * adjacent output columns x one block, every 16-byte piece stored lane-major.  Same byte
+ * count as the canonical stream; N must be a multiple of 64. */
+uint64_t guffin_hip_packed_bytes(int dtype, uint32_t K, uint32_t N);
+int guffin_hip_repack(void* stream, int dtype, const void* canonical, void* tiles, uint32_t K, uint32_t N);
+int guffin_hip_unpack(void* stream, int dtype, const void* tiles, void* canonical, uint32_t K, uint32_t N);
+
+/* Per-row sums of 16 and of 32 consecutive activations: xsums is [rows][K/16 + K/32]
+ * (16-sums first).  The reference's producers emit the same kind of receipt for its Q4_K
+ * kernels (src/tensor/backends/metal/metal_kernels.mm:16-27, "Q4 sums"). */
+int guffin_hip_group_sums(void* stream, const float* x, float* xsums, uint32_t rows, uint32_t K);
+
+/* Number of k-slices S the packed GEMV cuts this shape into (size of the partials buffer). */
+uint32_t guffin_hip_gemv_packed_slices(int dtype, uint32_t K, uint32_t N);
+/* Same operator as guffin_hip_gemv on repacked weights.  rows in {1, 2}.  Slice partials are
+ * written to partials[S][rows][N]; if y is non-null they are summed in slice order into
+ * y[rows][N] by a second small launch, otherwise the consumer does that sum. */
+int guffin_hip_gemv_packed(void* stream, int dtype, const void* tiles, const float* x, const float* xsums,
+                           float* partials, float* y, uint32_t rows, uint32_t K, uint32_t N);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,142 @@
+"""GPU parity of the wave-tile repack and the packed GEMV.
+
+Bars: repack -> unpack restores every byte (the reference pins its own repack the same
+way, tests/tensor/tensor_tests.cpp:3193-3283); packed GEMV within 1e-3 relative of the
+oracle's sequential fp32 sums; rows of a 2-row call bit-equal to 1-row calls; the packed
+and canonical-layout kernels agree to fp32 rounding.
+"""
+import numpy as np
+import pytest
+
+from guffin_amd import synth
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def hip():
+    from guffin_amd import hip as module
+    module.init(0)
+    return module
+
+
+def dev(a):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+@pytest.mark.parametrize("dtype,K,N", [(0, 640, 128), (1, 768, 192), (2, 512, 64), (1, 3840, 2048), (2, 3840, 256)])
+def test_repack_round_trip_is_lossless(hip, dtype, K, N):
+    w = synth.make_weight(dtype, K, N, seed=50 + dtype)
+    wd = dev(w)
+    tiles = hip.repack(dtype, wd, K, N)
+    assert hip.packed_bytes(dtype, K, N) == w.size
+    back = hip.unpack(dtype, tiles, K, N).cpu().numpy()
+    assert np.array_equal(back, w)
+    t = tiles.cpu().numpy()
+    assert not np.array_equal(t, w)
+    # spot-check the documented tile layout: 16-byte piece p of column l at p*1024 + l*16
+    bb = synth.BLOCK_BYTES[dtype]
+    nblk = K // synth.BLOCK_ELEMS[dtype]
+    col, b = 70 % N, nblk - 1
+    tile = t[((col // 64) * nblk + b) * 64 * bb:][:64 * bb]
+    blk = w[(col * nblk + b) * bb:][:bb]
+    lane = col % 64
+    if dtype == 1:
+        assert np.array_equal(tile[3 * 1024 + lane * 16:][:16], blk[48:64])
+    elif dtype == 2:
+        assert np.array_equal(tile[9 * 1024 + lane * 16:][:16], blk[144:160])
+        assert np.array_equal(tile[13312 + lane * 2:][:2], blk[208:210])
+    else:
+        assert np.array_equal(tile[1024 + lane * 16:][:16], blk[18:34])
+        assert np.array_equal(tile[2048 + lane * 2:][:2], blk[0:2])
+
+
+def test_group_sums(hip):
+    x = synth.make_activation(2, 3840, seed=60)
+    s = hip.group_sums(dev(x)).cpu().numpy()
+    want16 = x.reshape(2, -1, 16).astype(np.float64).sum(-1)
+    want32 = x.reshape(2, -1, 32).astype(np.float64).sum(-1)
+    assert s.shape == (2, 240 + 120)
+    assert np.allclose(s[:, :240], want16, rtol=0, atol=2e-5)
+    assert np.allclose(s[:, 240:], want32, rtol=0, atol=3e-5)
+
+
+SHAPES = [
+    (1, 3840, 4096), (1, 3840, 2048), (2, 3840, 2048), (1, 4096, 3840), (1, 3840, 15360),
+    (2, 15360, 3840), (1, 15360, 3840), (0, 640, 1024), (0, 1024, 640), (0, 2048, 640),
+    (0, 640, 2048), (1, 256, 64), (2, 256, 64), (0, 32, 64), (2, 768, 128),
+]
+
+
+@pytest.mark.parametrize("dtype,K,N", SHAPES)
+@pytest.mark.parametrize("rows", [1, 2])
+def test_packed_gemv_parity(hip, gfo, dtype, K, N, rows):
+    w = synth.make_weight(dtype, K, N, seed=7)
+    x = synth.make_activation(rows, K, seed=8)
+    wd, xd = dev(w), dev(x)
+    tiles = hip.repack(dtype, wd, K, N)
+    y = hip.gemv_packed(dtype, tiles, xd, hip.group_sums(xd), N).cpu().numpy()
+    ref = gfo.gemv(dtype, w, x, N, threads=8)
+    scale = np.sqrt((ref.astype(np.float64) ** 2).mean(axis=1, keepdims=True))
+    err = np.abs(y.astype(np.float64) - ref)
+    assert np.all(err <= 1e-3 * scale), float((err / scale).max())
+    # and against the canonical-layout kernel: both are fp32 sums of the same products
+    yc = hip.gemv(dtype, wd, xd, N).cpu().numpy()
+    assert np.all(np.abs(y.astype(np.float64) - yc) <= 2e-5 * scale)
+
+
+@pytest.mark.parametrize("dtype,K,N", [(1, 3840, 2048), (2, 3840, 2048), (2, 15360, 512), (0, 640, 1024), (1, 15360, 256)])
+def test_packed_two_row_rows_equal_one_row_calls(hip, dtype, K, N):
+    w = hip.repack(dtype, dev(synth.make_weight(dtype, K, N, 9)), K, N)
+    x = synth.make_activation(2, K, 10)
+    xd = dev(x)
+    both = hip.gemv_packed(dtype, w, xd, hip.group_sums(xd), N).cpu().numpy()
+    for r in range(2):
+        xr = dev(x[r:r + 1])
+        one = hip.gemv_packed(dtype, w, xr, hip.group_sums(xr), N).cpu().numpy()
+        assert np.array_equal(one[0].view(np.uint32), both[r].view(np.uint32))
+    again = hip.gemv_packed(dtype, w, xd, hip.group_sums(xd), N).cpu().numpy()
+    assert np.array_equal(again.view(np.uint32), both.view(np.uint32))
+
+
+@pytest.mark.parametrize("dtype", [0, 1, 2])
+def test_packed_unit_vectors_recover_columns(hip, gfo, dtype):
+    K, N = 256, 64
+    w = synth.make_weight(dtype, K, N, 30)
+    dense = gfo.dequant(dtype, w).reshape(N, K)
+    tiles = hip.repack(dtype, dev(w), K, N)
+    for k in (0, 17, 33, 100, 255):
+        x = np.zeros((1, K), np.float32)
+        x[0, k] = 1.0
+        xd = dev(x)
+        y = hip.gemv_packed(dtype, tiles, xd, hip.group_sums(xd), N).cpu().numpy()[0]
+        assert np.allclose(y, dense[:, k], rtol=2e-6, atol=2e-6), k
+
+
+def test_packed_partials_sum_in_slice_order(hip):
+    dtype, K, N = 1, 3840, 1024
+    w = hip.repack(dtype, dev(synth.make_weight(dtype, K, N, 11)), K, N)
+    xd = dev(synth.make_activation(2, K, 12))
+    xs = hip.group_sums(xd)
+    S = hip.gemv_packed_slices(dtype, K, N)
+    assert 1 <= S <= K // 256
+    parts = hip.gemv_packed(dtype, w, xd, xs, N, reduce=False).cpu().numpy()
+    y = hip.gemv_packed(dtype, w, xd, xs, N).cpu().numpy()
+    total = parts[0].copy()
+    for s in range(1, S):
+        total = total + parts[s]
+    assert np.array_equal(total.view(np.uint32), y.view(np.uint32))
+
+
+def test_packed_rejects_bad_arguments(hip):
+    import torch
+    w = torch.zeros(144 * 64, dtype=torch.uint8, device="cuda")
+    x = torch.zeros((1, 256), dtype=torch.float32, device="cuda")
+    with pytest.raises(hip.GuffinError):
+        hip.repack(1, w, 256, 60)          # N not a multiple of 64
+    with pytest.raises(hip.GuffinError):
+        hip.gemv_packed(1, w, torch.zeros((3, 256), dtype=torch.float32, device="cuda"),
+                        torch.zeros((3, 24), dtype=torch.float32, device="cuda"), 64)
+    with pytest.raises(hip.GuffinError):
+        hip.gemv_packed(1, w[8:], x, torch.zeros((1, 24), dtype=torch.float32, device="cuda"), 64)
