@@ -1,0 +1,295 @@
+// GQA decode / verify attention over an fp16 KV cache (gfx950).
+//
+// Replaces MetalCommandContext::encode_verifier_attention and its partition reducer
+// (src/tensor/backends/metal/metal_command_context.hpp:267,
+//  src/tensor/backends/metal/metal_kernels.mm:3061-3382); CPU definition
+// src/tensor/ops/attention.cpp:482-618 with softmax.cpp:42-71.
+//
+// Token list of a query row, in order: `base_count` committed tokens read from the ring
+// at slot (base_first + t) & ring_mask, then the row's ancestors among the private rows
+// of this verify pass.  All rows of a pass (<= 2) and the `group` query heads that share a
+// KV head are served by one workgroup, so each K/V row is read once per KV head and
+// partition: the rows' lists are merged into one virtual list (union of the ring ranges,
+// then every private row) with a per-row validity mask.
+//
+// Workgroup = (partition of TP consecutive virtual tokens, KV head), 256 threads.
+//   pass 1  scores: 16 lanes split the head dimension of one token (coalesced 512-byte K
+//           rows), four tokens per wave at a time; fp16 keys enter v_fma_mix_f32 directly;
+//           a 4-step exchange inside each 16-lane group finishes the dot product.
+//   softmax per query over the partition in LDS (max, exp, sum).
+//   pass 2  values: a wave owns every fourth token, a lane four output dims; no cross-lane
+//           reduction, the four waves are merged through LDS.
+// Partitions emit (max, denominator, unnormalised output); a second kernel merges them in
+// partition order.  fp32 throughout, keys/values stay fp16 in memory.
+#include "common.hpp"
+
+namespace guffin {
+namespace {
+
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+
+constexpr int kMaxRows = 2;
+
+struct AttnArgs {
+    const float* q;              // [rows][q_heads][hd]
+    const uint16_t* ring_k; const uint16_t* ring_v;   // [cap][kv_heads][hd]
+    const uint16_t* priv_k; const uint16_t* priv_v;   // [private rows][kv_heads][hd]
+    const uint32_t* schedule;    // [rows][4]
+    const uint32_t* ancestors;
+    float* part_out;             // [rows][q_heads][partitions][hd]
+    float* part_ml;              // [rows][q_heads][partitions][2]
+    uint32_t rows, q_heads, kv_heads, hd, ring_mask, tp, partitions, private_rows;
+    float scale;
+};
+
+__device__ __forceinline__ float dot2(float acc, uint32_t packed_half2, float a, float b) {
+    const half2_t h = __builtin_bit_cast(half2_t, packed_half2);
+    acc = fmaf(static_cast<float>(h.x), a, acc);
+    return fmaf(static_cast<float>(h.y), b, acc);
+}
+
+template <int ROWS, int GROUP, int HD>
+__global__ void __launch_bounds__(256) attn_partial_kernel(AttnArgs a) {
+    static_assert(HD == 256, "head dimension 256 (16 lanes x 16 dims)");
+    constexpr int NQ = ROWS * GROUP;
+    extern __shared__ float lds[];
+    float* sc = lds;                          // [NQ][tp] scores, then probabilities
+    float* merge = lds + NQ * a.tp;           // [4][NQ][HD]
+    __shared__ float s_max[NQ], s_sum[NQ];
+
+    const uint32_t part = blockIdx.x, kvh = blockIdx.y;
+    const uint32_t lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    constexpr uint32_t group = GROUP;
+    const uint32_t row_stride = a.kv_heads * HD;  // in halves
+
+    // merged virtual token list
+    uint32_t u_first = 0xFFFFFFFFu, u_end = 0;
+    uint32_t bfirst[ROWS], bend[ROWS], amask[ROWS];
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) {
+        bfirst[r] = 0; bend[r] = 0; amask[r] = 0;
+        {
+            const uint32_t* s = a.schedule + 4 * r;
+            bfirst[r] = s[0]; bend[r] = s[0] + s[1];
+            if (s[1]) { u_first = min(u_first, s[0]); u_end = max(u_end, s[0] + s[1]); }
+            for (uint32_t i = 0; i < s[3]; ++i) amask[r] |= 1u << a.ancestors[s[2] + i];
+        }
+    }
+    if (u_end == 0) { u_first = 0; }
+    const uint32_t n_ring = u_end - u_first, n_total = n_ring + a.private_rows;
+    const uint32_t t0 = part * a.tp, t1 = min(t0 + a.tp, n_total);
+
+    // ---- pass 1: scores ------------------------------------------------------------
+    {
+        const uint32_t slot = lane >> 4, seg = lane & 15;  // token slot in the wave, 16-dim segment
+        float qv[NQ][16];
+#pragma unroll
+        for (int n = 0; n < NQ; ++n) {
+            const uint32_t r = n / group, g = n % group;
+            const float* qp = a.q + (size_t(r) * a.q_heads + kvh * group + g) * HD + seg * 16;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) qv[n][i] = qp[i] * a.scale;
+        }
+        for (uint32_t t = t0 + wv * 4 + slot; t < t0 + a.tp; t += 16) {
+            float s[NQ];
+#pragma unroll
+            for (int n = 0; n < NQ; ++n) s[n] = 0.f;
+            const bool in_range = t < t1;
+            uint32_t pos = 0, prow = 0;
+            bool is_priv = false;
+            if (in_range) {
+                is_priv = t >= n_ring;
+                pos = u_first + t; prow = t - n_ring;
+                const uint16_t* kp = is_priv ? a.priv_k + size_t(prow) * row_stride
+                                             : a.ring_k + size_t(pos & a.ring_mask) * row_stride;
+                kp += kvh * HD + seg * 16;
+                const uint4 k0 = *reinterpret_cast<const uint4*>(kp), k1 = *reinterpret_cast<const uint4*>(kp + 8);
+                const uint32_t kw[8] = {k0.x, k0.y, k0.z, k0.w, k1.x, k1.y, k1.z, k1.w};
+#pragma unroll
+                for (int n = 0; n < NQ; ++n)
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) s[n] = dot2(s[n], kw[i], qv[n][2 * i], qv[n][2 * i + 1]);
+            }
+#pragma unroll
+            for (int n = 0; n < NQ; ++n) {
+                s[n] += __shfl_xor(s[n], 8, kWave);
+                s[n] += __shfl_xor(s[n], 4, kWave);
+                s[n] += __shfl_xor(s[n], 2, kWave);
+                s[n] += __shfl_xor(s[n], 1, kWave);
+            }
+            if (seg == 0) {
+#pragma unroll
+                for (int n = 0; n < NQ; ++n) {
+                    const uint32_t r = n / group;
+                    const bool valid = in_range && (is_priv ? ((amask[r] >> prow) & 1u) != 0
+                                                            : (pos >= bfirst[r] && pos < bend[r]));
+                    sc[n * a.tp + (t - t0)] = valid ? s[n] : -INFINITY;
+                }
+            }
+        }
+    }
+    __syncthreads();
+
+    // ---- softmax over the partition, one wave per query ----------------------------------
+    for (uint32_t n = wv; n < NQ; n += 4) {
+        float m = -INFINITY;
+        for (uint32_t i = lane; i < a.tp; i += 64) m = fmaxf(m, sc[n * a.tp + i]);
+        m = wave_max(m);
+        float l = 0.f;
+        for (uint32_t i = lane; i < a.tp; i += 64) {
+            const float v = sc[n * a.tp + i];
+            const float p = v == -INFINITY ? 0.f : expf(v - m);
+            sc[n * a.tp + i] = p;
+            l += p;
+        }
+        l = wave_sum(l);
+        if (lane == 0) { s_max[n] = m; s_sum[n] = l; }
+    }
+    __syncthreads();
+
+    // ---- pass 2: values -------------------------------------------------------------------
+    {
+        float acc[NQ][4];
+#pragma unroll
+        for (int n = 0; n < NQ; ++n)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[n][i] = 0.f;
+        for (uint32_t t = t0 + wv; t < t1; t += 4) {
+            const bool is_priv = t >= n_ring;
+            const uint16_t* vp = is_priv ? a.priv_v + size_t(t - n_ring) * row_stride
+                                         : a.ring_v + size_t((u_first + t) & a.ring_mask) * row_stride;
+            const uint2 vv = *reinterpret_cast<const uint2*>(vp + kvh * HD + lane * 4);
+#pragma unroll
+            for (int n = 0; n < NQ; ++n) {
+                const float p = sc[n * a.tp + (t - t0)];
+                const half2_t h0 = __builtin_bit_cast(half2_t, vv.x), h1 = __builtin_bit_cast(half2_t, vv.y);
+                acc[n][0] = fmaf(static_cast<float>(h0.x), p, acc[n][0]);
+                acc[n][1] = fmaf(static_cast<float>(h0.y), p, acc[n][1]);
+                acc[n][2] = fmaf(static_cast<float>(h1.x), p, acc[n][2]);
+                acc[n][3] = fmaf(static_cast<float>(h1.y), p, acc[n][3]);
+            }
+        }
+#pragma unroll
+        for (int n = 0; n < NQ; ++n)
+            *reinterpret_cast<float4*>(merge + (wv * NQ + n) * HD + lane * 4) =
+                make_float4(acc[n][0], acc[n][1], acc[n][2], acc[n][3]);
+    }
+    __syncthreads();
+    for (uint32_t i = threadIdx.x; i < NQ * HD; i += 256) {
+        const uint32_t n = i / HD, d = i % HD;
+        const float v = (merge[(0 * NQ + n) * HD + d] + merge[(1 * NQ + n) * HD + d])
+            + (merge[(2 * NQ + n) * HD + d] + merge[(3 * NQ + n) * HD + d]);
+        const uint32_t r = n / group, g = n % group, head = kvh * group + g;
+        const size_t slot = (size_t(r) * a.q_heads + head) * a.partitions + part;
+        a.part_out[slot * HD + d] = v;
+        if (d == 0) { a.part_ml[slot * 2] = s_max[n]; a.part_ml[slot * 2 + 1] = s_sum[n]; }
+    }
+}
+
+// out[row][head][:] = sum_p e^(m_p - M) acc_p / sum_p e^(m_p - M) l_p, partitions in order
+__global__ void __launch_bounds__(256)
+attn_merge_kernel(const float* __restrict__ part_out, const float* __restrict__ part_ml, float* __restrict__ out,
+                  float* __restrict__ out_sums, uint32_t partitions, uint32_t hd, uint32_t q_heads,
+                  uint32_t* __restrict__ status) {
+    const uint32_t rh = blockIdx.x;  // row * q_heads + head
+    const float* ml = part_ml + size_t(rh) * partitions * 2;
+    float M = -INFINITY;
+    for (uint32_t p = 0; p < partitions; ++p) if (ml[2 * p + 1] > 0.f) M = fmaxf(M, ml[2 * p]);
+    float denom = 0.f;
+    for (uint32_t p = 0; p < partitions; ++p) if (ml[2 * p + 1] > 0.f) denom += expf(ml[2 * p] - M) * ml[2 * p + 1];
+    __shared__ float rowbuf[1024];
+    bool bad = false;
+    for (uint32_t d = threadIdx.x; d < hd; d += blockDim.x) {
+        float acc = 0.f;
+        for (uint32_t p = 0; p < partitions; ++p)
+            if (ml[2 * p + 1] > 0.f) acc = fmaf(expf(ml[2 * p] - M), part_out[(size_t(rh) * partitions + p) * hd + d], acc);
+        const float v = acc / denom;
+        bad |= !isfinite(v);
+        out[size_t(rh) * hd + d] = v;
+        rowbuf[d] = v;
+    }
+    if (bad && status) atomicOr(status, GUFFIN_STATUS_NONFINITE);
+    if (out_sums) {
+        __syncthreads();
+        // group sums of the attention output row [q_heads*hd] feed the o-projection GEMV
+        const uint32_t row = rh / q_heads, head = rh % q_heads, width = q_heads * hd;
+        float* sums = out_sums + size_t(row) * (width / 16 + width / 32);
+        for (uint32_t g = threadIdx.x; g < hd / 16; g += blockDim.x) {
+            float s = 0.f;
+            for (int k = 0; k < 16; ++k) s += rowbuf[g * 16 + k];
+            sums[head * (hd / 16) + g] = s;
+        }
+        for (uint32_t g = threadIdx.x; g < hd / 32; g += blockDim.x) {
+            float s0 = 0.f, s1 = 0.f;
+            for (int k = 0; k < 16; ++k) { s0 += rowbuf[g * 32 + k]; s1 += rowbuf[g * 32 + 16 + k]; }
+            sums[width / 16 + head * (hd / 32) + g] = s0 + s1;
+        }
+    }
+}
+
+template <int ROWS, int GROUP>
+int launch_partial(hipStream_t s, const AttnArgs& a) {
+    constexpr int NQ = ROWS * GROUP;
+    const size_t lds = (size_t(NQ) * a.tp + size_t(4) * NQ * 256) * sizeof(float);
+    hipLaunchKernelGGL((attn_partial_kernel<ROWS, GROUP, 256>), dim3(a.partitions, a.kv_heads), dim3(256), lds, s, a);
+    return check_launch("attention_partial");
+}
+
+}  // namespace
+}  // namespace guffin
+
+using namespace guffin;
+
+extern "C" uint32_t guffin_hip_attention_partitions(uint32_t max_tokens, uint32_t kv_heads) {
+    // tokens per partition: aim at >= 256 workgroups, between 32 and 128 tokens each
+    if (max_tokens == 0 || kv_heads == 0) return 0;
+    uint32_t tp = 128;
+    while (tp > 32 && ((max_tokens + tp - 1) / tp) * kv_heads < 256) tp >>= 1;
+    return (max_tokens + tp - 1) / tp;
+}
+
+extern "C" int guffin_hip_attention_decode(void* stream, const float* q, const void* ring_k, const void* ring_v,
+                                           const void* priv_k, const void* priv_v, const uint32_t* schedule,
+                                           const uint32_t* ancestors, float* out, float* out_sums,
+                                           float* partial_out, float* partial_ml, uint32_t rows,
+                                           uint32_t private_rows, uint32_t max_tokens, uint32_t ring_mask,
+                                           uint32_t q_heads, uint32_t kv_heads, uint32_t head_dim, float scale,
+                                           uint32_t* status) {
+    if (!q || !ring_k || !ring_v || !priv_k || !priv_v || !schedule || !ancestors || !out || !partial_out || !partial_ml)
+        return fail(GUFFIN_E_ARG, "attention_decode: null pointer");
+    if (rows == 0 || rows > kMaxRows || private_rows > 32) return fail(GUFFIN_E_SHAPE, "attention_decode: rows must be 1 or 2, private rows <= 32");
+    if (head_dim != 256) return fail(GUFFIN_E_SHAPE, "attention_decode: head_dim must be 256");
+    if (kv_heads == 0 || q_heads % kv_heads != 0) return fail(GUFFIN_E_SHAPE, "attention_decode: q_heads must be a multiple of kv_heads");
+    if ((ring_mask & (ring_mask + 1)) != 0) return fail(GUFFIN_E_ARG, "attention_decode: ring capacity must be a power of two");
+    if (max_tokens == 0) return fail(GUFFIN_E_SHAPE, "attention_decode: max_tokens must cover every row's token list");
+    if (!(scale > 0.f)) return fail(GUFFIN_E_ARG, "attention_decode: scale must be positive");
+    if ((reinterpret_cast<uintptr_t>(ring_k) & 15u) || (reinterpret_cast<uintptr_t>(ring_v) & 15u)
+        || (reinterpret_cast<uintptr_t>(priv_k) & 15u) || (reinterpret_cast<uintptr_t>(priv_v) & 15u))
+        return fail(GUFFIN_E_ALIGN, "attention_decode: KV rows must be 16-byte aligned");
+    const uint32_t group = q_heads / kv_heads;
+    AttnArgs a {};
+    a.q = q;
+    a.ring_k = static_cast<const uint16_t*>(ring_k); a.ring_v = static_cast<const uint16_t*>(ring_v);
+    a.priv_k = static_cast<const uint16_t*>(priv_k); a.priv_v = static_cast<const uint16_t*>(priv_v);
+    a.schedule = schedule; a.ancestors = ancestors; a.part_out = partial_out; a.part_ml = partial_ml;
+    a.rows = rows; a.q_heads = q_heads; a.kv_heads = kv_heads; a.hd = head_dim; a.ring_mask = ring_mask;
+    a.partitions = guffin_hip_attention_partitions(max_tokens, kv_heads);
+    a.tp = (max_tokens + a.partitions - 1) / a.partitions;
+    a.tp = (a.tp + 15u) & ~15u;  // whole rounds of 16 tokens per workgroup
+    a.private_rows = private_rows; a.scale = scale;
+    hipStream_t s = as_stream(stream);
+    int rc;
+    switch (group * 10 + rows) {
+        case 11: rc = launch_partial<1, 1>(s, a); break;
+        case 12: rc = launch_partial<2, 1>(s, a); break;
+        case 21: rc = launch_partial<1, 2>(s, a); break;
+        case 22: rc = launch_partial<2, 2>(s, a); break;
+        case 41: rc = launch_partial<1, 4>(s, a); break;
+        case 42: rc = launch_partial<2, 4>(s, a); break;
+        default: return fail(GUFFIN_E_SHAPE, "attention_decode: q_heads / kv_heads must be 1, 2 or 4");
+    }
+    if (rc) return rc;
+    hipLaunchKernelGGL(attn_merge_kernel, dim3(rows * q_heads), dim3(256), 0, s, partial_out, partial_ml, out,
+                       out_sums, a.partitions, head_dim, q_heads, status);
+    return check_launch("attention_merge");
+}

@@ -1,3 +1,487 @@
-// placeholder translation unit filled in with the per-layer operators
+// Per-layer operators of the Gemma-3 block graph on gfx950: RMS norms, NeoX RoPE,
+// fp16 KV narrowing, GeGLU, embedding gather, KV publication.
+//
+// Reference behaviour:
+//   rms_norm / rms_norm_add / head_rms_norm  src/tensor/backends/metal/metal_kernels.mm:1915-2158
+//                                            (CPU: src/tensor/ops/normalization.cpp:70-99)
+//   rope by positions, kv store              metal_kernels.mm:2406-2486 (CPU angle in double:
+//                                            src/tensor/ops/rope.cpp:109-117, 242-283)
+//   gelu_tanh * up                           metal_kernels.mm:1827-1843 (CPU: ops/elementwise.cpp:79-94)
+//   embedding                                metal_kernels.mm:452-474, src/engine/gemma3_draft.mm:61-71
+//   kv scatter (publish private rows)        metal_kernels.mm:2519-2557
+//
+// Every operator that produces a GEMV input can also emit the per-16 / per-32 activation
+// sums the packed GEMV consumes, and every operator that consumes a GEMV output can sum
+// `planes` k-slice partial planes (stride plane_stride floats) while it loads.
 #include "common.hpp"
-namespace guffin { int ops_init(int) { return 0; } }
+
+namespace guffin {
+namespace {
+
+__device__ __forceinline__ float block_sum(float v, float* scratch) {
+    v = wave_sum(v);
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
+    __syncthreads();  // scratch may still be read from a previous call
+    if (lane == 0) scratch[wv] = v;
+    __syncthreads();
+    float t = 0.f;
+    for (int i = 0; i < nw; ++i) t += scratch[i];  // same order on every thread
+    return t;
+}
+
+__device__ __forceinline__ float load_planes(const float* p, uint32_t planes, size_t plane_stride) {
+    float v = p[0];
+    for (uint32_t s = 1; s < planes; ++s) v += p[s * plane_stride];
+    return v;
+}
+
+// 16-sums and 32-sums of a row that lives in LDS (`row`, `width` floats), written to sums[]
+__device__ __forceinline__ void emit_group_sums(const float* row, float* sums, uint32_t width) {
+    const uint32_t n16 = width / 16;
+    for (uint32_t g = threadIdx.x; g < n16; g += blockDim.x) {
+        float s = 0.f;
+#pragma unroll
+        for (int k = 0; k < 16; ++k) s += row[g * 16 + k];
+        sums[g] = s;
+    }
+    for (uint32_t g = threadIdx.x; g < width / 32; g += blockDim.x) {
+        float a = 0.f, b = 0.f;
+#pragma unroll
+        for (int k = 0; k < 16; ++k) { a += row[g * 32 + k]; b += row[g * 32 + 16 + k]; }
+        sums[n16 + g] = a + b;  // the sum of the two 16-sums, as group_sums_kernel forms it
+    }
+}
+
+// y = x * rsqrt(mean(x^2) + eps) * gamma [+ residual]; one workgroup per row.
+// x may be `planes` partial planes.  Optional outputs: y_sums (group sums of y).
+__global__ void __launch_bounds__(256)
+rms_norm_kernel(const float* __restrict__ x, uint32_t planes, size_t plane_stride,
+                const float* __restrict__ gamma, const float* __restrict__ residual,
+                float* __restrict__ y, float* __restrict__ y_sums, uint32_t width, float eps,
+                uint32_t* __restrict__ status) {
+    extern __shared__ float lds[];  // [width] row image + [4] scratch
+    float* row = lds;
+    float* scratch = lds + width;
+    const uint32_t r = blockIdx.x;
+    const float* xr = x + size_t(r) * width;
+    float ss = 0.f;
+    for (uint32_t c = threadIdx.x; c < width; c += blockDim.x) {
+        const float v = load_planes(xr + c, planes, plane_stride);
+        row[c] = v;
+        ss = fmaf(v, v, ss);
+    }
+    const float total = block_sum(ss, scratch);
+    const float inv = 1.0f / sqrtf(total / static_cast<float>(width) + eps);
+    bool bad = false;
+    for (uint32_t c = threadIdx.x; c < width; c += blockDim.x) {
+        float v = row[c] * inv * gamma[c];
+        if (residual) v += residual[size_t(r) * width + c];
+        bad |= !isfinite(v);
+        row[c] = v;
+        y[size_t(r) * width + c] = v;
+    }
+    if (bad && status) atomicOr(status, GUFFIN_STATUS_NONFINITE);
+    if (y_sums) {
+        __syncthreads();
+        emit_group_sums(row, y_sums + size_t(r) * (width / 16 + width / 32), width);
+    }
+}
+
+// Fused tail of one sub-block and head of the next:
+//   out_residual = residual + rms(x, gamma_post);  out_norm = rms(out_residual, gamma_next)
+// (reference order: encode_rms_norm_add then encode_rms_norm, gemma_target_runtime.cpp:156-173, 201-213)
+__global__ void __launch_bounds__(256)
+rms_norm_add_norm_kernel(const float* __restrict__ x, uint32_t planes, size_t plane_stride,
+                         const float* __restrict__ gamma_post, const float* __restrict__ residual,
+                         float* __restrict__ out_residual, const float* __restrict__ gamma_next,
+                         float* __restrict__ out_norm, float* __restrict__ out_sums, uint32_t width,
+                         float eps, uint32_t* __restrict__ status) {
+    extern __shared__ float lds[];
+    float* row = lds;
+    float* scratch = lds + width;
+    const uint32_t r = blockIdx.x;
+    const float* xr = x + size_t(r) * width;
+    float ss = 0.f;
+    for (uint32_t c = threadIdx.x; c < width; c += blockDim.x) {
+        const float v = load_planes(xr + c, planes, plane_stride);
+        row[c] = v;
+        ss = fmaf(v, v, ss);
+    }
+    float total = block_sum(ss, scratch);
+    float inv = 1.0f / sqrtf(total / static_cast<float>(width) + eps);
+    ss = 0.f;
+    bool bad = false;
+    for (uint32_t c = threadIdx.x; c < width; c += blockDim.x) {
+        const float v = row[c] * inv * gamma_post[c] + residual[size_t(r) * width + c];
+        bad |= !isfinite(v);
+        row[c] = v;
+        out_residual[size_t(r) * width + c] = v;
+        ss = fmaf(v, v, ss);
+    }
+    total = block_sum(ss, scratch);
+    inv = 1.0f / sqrtf(total / static_cast<float>(width) + eps);
+    for (uint32_t c = threadIdx.x; c < width; c += blockDim.x) {
+        const float v = row[c] * inv * gamma_next[c];
+        row[c] = v;
+        out_norm[size_t(r) * width + c] = v;
+    }
+    if (bad && status) atomicOr(status, GUFFIN_STATUS_NONFINITE);
+    if (out_sums) {
+        __syncthreads();
+        emit_group_sums(row, out_sums + size_t(r) * (width / 16 + width / 32), width);
+    }
+}
+
+// Per-head RMS norm over head_dim (one wave per (row, head)); in place allowed.
+__global__ void __launch_bounds__(64)
+head_rms_norm_kernel(const float* __restrict__ x, const float* __restrict__ gamma, float* __restrict__ y,
+                     uint32_t head_dim, float eps) {
+    const size_t base = size_t(blockIdx.x) * head_dim;
+    float ss = 0.f;
+    for (uint32_t c = threadIdx.x; c < head_dim; c += 64) { const float v = x[base + c]; ss = fmaf(v, v, ss); }
+    ss = wave_sum(ss);
+    const float inv = 1.0f / sqrtf(ss / static_cast<float>(head_dim) + eps);
+    for (uint32_t c = threadIdx.x; c < head_dim; c += 64) y[base + c] = x[base + c] * inv * gamma[c];
+}
+
+__device__ __forceinline__ void rope_sincos(uint32_t position, uint32_t pair, uint32_t rope_dim, float base,
+                                            float scale, float& c, float& s) {
+    // angle in double, as the CPU operator forms it (rope.cpp:109-117), times the layer's frequency scale
+    const double exponent = static_cast<double>(2u * pair) / static_cast<double>(rope_dim);
+    const double angle = static_cast<double>(position) / pow(static_cast<double>(base), exponent)
+        * static_cast<double>(scale);
+    c = static_cast<float>(cos(angle));
+    s = static_cast<float>(sin(angle));
+}
+
+// Fused q/k head norm + NeoX RoPE + fp16 KV narrowing for `rows` new tokens:
+//   q_out = rope(headnorm(q_raw)) fp32;  k_out = f16(rope(headnorm(k_raw)));  v_out = f16(v_raw)
+// One wave per (row, head); q heads first, then k heads, then v heads.  Any of the three
+// sections can be disabled with a null pointer; q_norm/k_norm null skips the head norm.
+// Inputs may be `planes` partial planes of a GEMV.
+struct QkvArgs {
+    const float* q_raw; const float* k_raw; const float* v_raw;
+    uint32_t planes; size_t q_plane_stride, k_plane_stride, v_plane_stride;
+    const float* q_norm; const float* k_norm;
+    const uint32_t* positions;
+    float* q_out; uint16_t* k_out; uint16_t* v_out;
+    uint32_t rows, q_heads, kv_heads, head_dim, rope_dim;
+    float base, scale, eps;
+    uint32_t* status;
+};
+
+__global__ void __launch_bounds__(64) qkv_post_kernel(QkvArgs a) {
+    extern __shared__ float lds[];  // [head_dim]
+    const uint32_t per_row = a.q_heads + 2 * a.kv_heads;
+    const uint32_t r = blockIdx.x / per_row, h = blockIdx.x % per_row, lane = threadIdx.x;
+    const bool is_q = h < a.q_heads, is_k = !is_q && h < a.q_heads + a.kv_heads;
+    const uint32_t hh = is_q ? h : is_k ? h - a.q_heads : h - a.q_heads - a.kv_heads;
+    const uint32_t heads = is_q ? a.q_heads : a.kv_heads;
+    const float* src = is_q ? a.q_raw : is_k ? a.k_raw : a.v_raw;
+    if (!src) return;
+    const size_t stride = is_q ? a.q_plane_stride : is_k ? a.k_plane_stride : a.v_plane_stride;
+    const size_t off = (size_t(r) * heads + hh) * a.head_dim;
+    float ss = 0.f;
+    for (uint32_t c = lane; c < a.head_dim; c += 64) {
+        const float v = load_planes(src + off + c, a.planes, stride);
+        lds[c] = v;
+        ss = fmaf(v, v, ss);
+    }
+    bool bad = false;
+    if (!is_q && !is_k) {  // V: narrow only
+        for (uint32_t c = lane; c < a.head_dim; c += 64) {
+            const _Float16 hv = static_cast<_Float16>(lds[c]);
+            bad |= !isfinite(static_cast<float>(hv));
+            a.v_out[off + c] = __builtin_bit_cast(uint16_t, hv);
+        }
+        if (bad && a.status) atomicOr(a.status, GUFFIN_STATUS_KV_NONFINITE);
+        return;
+    }
+    const float* gamma = is_q ? a.q_norm : a.k_norm;
+    if (gamma) {
+        ss = wave_sum(ss);
+        const float inv = 1.0f / sqrtf(ss / static_cast<float>(a.head_dim) + a.eps);
+        for (uint32_t c = lane; c < a.head_dim; c += 64) lds[c] = lds[c] * inv * gamma[c];
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const uint32_t half = a.rope_dim / 2, pos = a.positions[r];
+    for (uint32_t c = lane; c < a.head_dim; c += 64) {
+        float v = lds[c];
+        if (c < a.rope_dim) {
+            const uint32_t pair = c % half;
+            float cs, sn;
+            rope_sincos(pos, pair, a.rope_dim, a.base, a.scale, cs, sn);
+            const float first = lds[pair], second = lds[pair + half];
+            v = c < half ? __fsub_rn(__fmul_rn(first, cs), __fmul_rn(second, sn))
+                         : __fadd_rn(__fmul_rn(first, sn), __fmul_rn(second, cs));
+        }
+        if (is_q) {
+            a.q_out[off + c] = v;
+        } else {
+            const _Float16 hv = static_cast<_Float16>(v);  // round-to-nearest-even, after rotation
+            bad |= !isfinite(static_cast<float>(hv));
+            a.k_out[off + c] = __builtin_bit_cast(uint16_t, hv);
+        }
+    }
+    if (bad && a.status) atomicOr(a.status, GUFFIN_STATUS_KV_NONFINITE);
+}
+
+// out = gelu_tanh(gate) * up, element-wise; gate/up may be partial planes.  One workgroup
+// per row when sums are requested (row image in LDS), grid-stride otherwise.
+__device__ __forceinline__ float geglu_value(float g, float u) {
+    constexpr float k0 = 0.7978845608028654f, k1 = 0.044715f;
+    const float inner = __fmul_rn(k0, __fadd_rn(g, __fmul_rn(__fmul_rn(__fmul_rn(k1, g), g), g)));
+    const float t = tanhf(inner);
+    return __fmul_rn(__fmul_rn(__fmul_rn(0.5f, g), __fadd_rn(1.0f, t)), u);
+}
+
+__global__ void __launch_bounds__(256)
+geglu_kernel(const float* __restrict__ gate, const float* __restrict__ up, uint32_t planes, size_t plane_stride,
+             float* __restrict__ out, float* __restrict__ out_sums, uint32_t width) {
+    extern __shared__ float lds[];  // [chunk] when sums are requested
+    // grid: (chunks_per_row, rows); a chunk is a multiple of 32 columns
+    const uint32_t chunk = (width + gridDim.x - 1) / gridDim.x;
+    const uint32_t c0 = blockIdx.x * chunk, c1 = c0 + chunk < width ? c0 + chunk : width;
+    const size_t rbase = size_t(blockIdx.y) * width;
+    for (uint32_t c = c0 + threadIdx.x; c < c1; c += blockDim.x) {
+        const float g = load_planes(gate + rbase + c, planes, plane_stride);
+        const float u = load_planes(up + rbase + c, planes, plane_stride);
+        const float v = geglu_value(g, u);
+        out[rbase + c] = v;
+        if (out_sums) lds[c - c0] = v;
+    }
+    if (out_sums) {
+        __syncthreads();
+        float* sums = out_sums + size_t(blockIdx.y) * (width / 16 + width / 32);
+        const uint32_t n16 = width / 16;
+        for (uint32_t g = threadIdx.x; g < (c1 - c0) / 16; g += blockDim.x) {
+            float s = 0.f;
+#pragma unroll
+            for (int k = 0; k < 16; ++k) s += lds[g * 16 + k];
+            sums[c0 / 16 + g] = s;
+        }
+        for (uint32_t g = threadIdx.x; g < (c1 - c0) / 32; g += blockDim.x) {
+            float a = 0.f, b = 0.f;
+#pragma unroll
+            for (int k = 0; k < 16; ++k) { a += lds[g * 32 + k]; b += lds[g * 32 + 16 + k]; }
+            sums[n16 + c0 / 32 + g] = a + b;
+        }
+    }
+}
+
+// out[r, :] = dequant(row tokens[r] of W) * scale; canonical block stream (one row = width/elems blocks)
+template <int DTYPE>
+__global__ void __launch_bounds__(256)
+embed_kernel(const uint8_t* __restrict__ w, const uint32_t* __restrict__ tokens, float* __restrict__ out,
+             uint32_t width, float scale, uint32_t vocab, uint32_t* __restrict__ status) {
+    constexpr uint32_t be = DTYPE == GUFFIN_Q8_0 ? 32 : 256;
+    constexpr uint32_t bb = DTYPE == GUFFIN_Q8_0 ? 34 : DTYPE == GUFFIN_Q4_K ? 144 : 210;
+    uint32_t token = tokens[blockIdx.x];
+    if (token >= vocab) {
+        if (threadIdx.x == 0 && status) atomicOr(status, GUFFIN_STATUS_BAD_TOKEN);
+        token = 0;
+    }
+    const uint8_t* row = w + size_t(token) * (width / be) * bb;
+    bool bad = false;
+    for (uint32_t c = threadIdx.x; c < width; c += blockDim.x) {
+        const uint8_t* b = row + size_t(c / be) * bb;
+        const uint32_t i = c % be;
+        float v;
+        if constexpr (DTYPE == GUFFIN_Q8_0) {
+            v = __fmul_rn(h2f(ld_u16(b)), static_cast<float>(static_cast<int8_t>(b[2 + i])));
+        } else if constexpr (DTYPE == GUFFIN_Q6_K) {
+            const uint32_t half = i >> 7, rr = i & 127, l = rr & 31;
+            const uint32_t lo_byte = b[half * 64 + ((rr >> 5) & 1) * 32 + l];
+            const uint32_t lo = rr < 64 ? (lo_byte & 0x0Fu) : (lo_byte >> 4);
+            const uint32_t hi = (b[128 + half * 32 + l] >> ((rr >> 5) * 2)) & 3u;
+            const int q = static_cast<int>(lo | (hi << 4)) - 32;
+            const float sc = static_cast<float>(static_cast<int8_t>(b[192 + (i >> 4)]));
+            v = __fmul_rn(__fmul_rn(h2f(ld_u16(b + 208)), sc), static_cast<float>(q));
+        } else {
+            const float d = h2f(ld_u16(b)), dmin = h2f(ld_u16(b + 2));
+            const uint8_t* s = b + 4;
+            const uint32_t g = i >> 5;
+            uint32_t sc, mn;
+            if (g < 4) { sc = s[g] & 63u; mn = s[g + 4] & 63u; }
+            else { sc = (s[g + 4] & 0x0Fu) | ((s[g - 4] >> 6) << 4); mn = (s[g + 4] >> 4) | ((s[g] >> 6) << 4); }
+            const uint32_t byte = b[16 + (i >> 6) * 32 + (i & 31)];
+            const uint32_t q = (i & 63) < 32 ? (byte & 0x0Fu) : (byte >> 4);
+            v = __fsub_rn(__fmul_rn(__fmul_rn(d, static_cast<float>(sc)), static_cast<float>(q)),
+                          __fmul_rn(dmin, static_cast<float>(mn)));
+        }
+        v = __fmul_rn(v, scale);
+        bad |= !isfinite(v);
+        out[size_t(blockIdx.x) * width + c] = v;
+    }
+    if (bad && status) atomicOr(status, GUFFIN_STATUS_NONFINITE);
+}
+
+// ring[(position + i) & mask] = private[selected[i]] for both K and V (16-bit elements)
+__global__ void kv_scatter_kernel(const uint16_t* __restrict__ priv_k, const uint16_t* __restrict__ priv_v,
+                                  const uint32_t* __restrict__ selected, uint16_t* __restrict__ ring_k,
+                                  uint16_t* __restrict__ ring_v, uint32_t position, uint32_t rows,
+                                  uint32_t row_width, uint32_t mask) {
+    const uint32_t i = blockIdx.y;
+    if (i >= rows) return;
+    // when more rows than ring slots are published only the newest owner of a slot writes it
+    if (rows > mask + 1 && i + mask + 1 < rows) return;
+    const size_t src = size_t(selected[i]) * row_width, dst = size_t((position + i) & mask) * row_width;
+    for (uint32_t c = blockIdx.x * blockDim.x + threadIdx.x; c < row_width; c += gridDim.x * blockDim.x) {
+        ring_k[dst + c] = priv_k[src + c];
+        ring_v[dst + c] = priv_v[src + c];
+    }
+}
+
+bool aligned4(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 3u) == 0; }
+
+}  // namespace
+
+int ops_init(int) {
+    int rc = 0;
+    rc |= hipFuncSetAttribute(reinterpret_cast<const void*>(rms_norm_kernel),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess;
+    rc |= hipFuncSetAttribute(reinterpret_cast<const void*>(rms_norm_add_norm_kernel),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess;
+    return rc;
+}
+
+}  // namespace guffin
+
+using namespace guffin;
+
+extern "C" int guffin_hip_rms_norm(void* stream, const float* x, uint32_t planes, uint64_t plane_stride,
+                                   const float* gamma, const float* residual, float* y, float* y_sums,
+                                   uint32_t rows, uint32_t width, float eps, uint32_t* status) {
+    if (!x || !gamma || !y) return fail(GUFFIN_E_ARG, "rms_norm: null pointer");
+    if (rows == 0 || width == 0 || planes == 0) return fail(GUFFIN_E_SHAPE, "rms_norm: empty shape");
+    if (y_sums && width % 32 != 0) return fail(GUFFIN_E_SHAPE, "rms_norm: group sums need width % 32 == 0");
+    if (!(eps > 0.f)) return fail(GUFFIN_E_ARG, "rms_norm: epsilon must be positive");
+    if (!aligned4(x) || !aligned4(y) || !aligned4(gamma)) return fail(GUFFIN_E_ALIGN, "rms_norm: fp32 pointers must be 4-byte aligned");
+    const size_t lds = (size_t(width) + 8) * 4;
+    if (lds > 160 * 1024) return fail(GUFFIN_E_CAPACITY, "rms_norm: row does not fit in LDS");
+    hipLaunchKernelGGL(rms_norm_kernel, dim3(rows), dim3(256), lds, as_stream(stream), x, planes,
+                       static_cast<size_t>(plane_stride), gamma, residual, y, y_sums, width, eps, status);
+    return check_launch("rms_norm");
+}
+
+extern "C" int guffin_hip_rms_norm_add_norm(void* stream, const float* x, uint32_t planes, uint64_t plane_stride,
+                                            const float* gamma_post, const float* residual, float* out_residual,
+                                            const float* gamma_next, float* out_norm, float* out_sums,
+                                            uint32_t rows, uint32_t width, float eps, uint32_t* status) {
+    if (!x || !gamma_post || !residual || !out_residual || !gamma_next || !out_norm)
+        return fail(GUFFIN_E_ARG, "rms_norm_add_norm: null pointer");
+    if (rows == 0 || width == 0 || planes == 0) return fail(GUFFIN_E_SHAPE, "rms_norm_add_norm: empty shape");
+    if (out_sums && width % 32 != 0) return fail(GUFFIN_E_SHAPE, "rms_norm_add_norm: group sums need width % 32 == 0");
+    if (!(eps > 0.f)) return fail(GUFFIN_E_ARG, "rms_norm_add_norm: epsilon must be positive");
+    const size_t lds = (size_t(width) + 8) * 4;
+    if (lds > 160 * 1024) return fail(GUFFIN_E_CAPACITY, "rms_norm_add_norm: row does not fit in LDS");
+    hipLaunchKernelGGL(rms_norm_add_norm_kernel, dim3(rows), dim3(256), lds, as_stream(stream), x, planes,
+                       static_cast<size_t>(plane_stride), gamma_post, residual, out_residual, gamma_next,
+                       out_norm, out_sums, width, eps, status);
+    return check_launch("rms_norm_add_norm");
+}
+
+extern "C" int guffin_hip_head_rms_norm(void* stream, const float* x, const float* gamma, float* y,
+                                        uint32_t rows, uint32_t heads, uint32_t head_dim, float eps) {
+    if (!x || !gamma || !y) return fail(GUFFIN_E_ARG, "head_rms_norm: null pointer");
+    if (rows == 0 || heads == 0 || head_dim == 0) return fail(GUFFIN_E_SHAPE, "head_rms_norm: empty shape");
+    if (!(eps > 0.f)) return fail(GUFFIN_E_ARG, "head_rms_norm: epsilon must be positive");
+    hipLaunchKernelGGL(head_rms_norm_kernel, dim3(rows * heads), dim3(64), 0, as_stream(stream), x, gamma, y, head_dim, eps);
+    return check_launch("head_rms_norm");
+}
+
+static int launch_qkv(void* stream, const QkvArgs& a) {
+    if (!a.positions) return fail(GUFFIN_E_ARG, "rope/kv: null positions");
+    if (a.rows == 0 || a.head_dim == 0 || a.head_dim > 4096) return fail(GUFFIN_E_SHAPE, "rope/kv: bad head shape");
+    if (a.rope_dim > a.head_dim || (a.rope_dim & 1u)) return fail(GUFFIN_E_SHAPE, "rope/kv: rope_dim must be even and <= head_dim");
+    if (a.rope_dim && !(a.base > 0.f)) return fail(GUFFIN_E_ARG, "rope/kv: frequency base must be positive");
+    const uint32_t blocks = a.rows * (a.q_heads + 2 * a.kv_heads);
+    if (blocks == 0) return fail(GUFFIN_E_SHAPE, "rope/kv: no heads");
+    hipLaunchKernelGGL(qkv_post_kernel, dim3(blocks), dim3(64), a.head_dim * sizeof(float), as_stream(stream), a);
+    return check_launch("qkv_post");
+}
+
+extern "C" int guffin_hip_rope_neox(void* stream, const float* in, const uint32_t* positions, float* out,
+                                    uint32_t rows, uint32_t heads, uint32_t head_dim, uint32_t rope_dim,
+                                    float freq_base, float freq_scale) {
+    if (!in || !out) return fail(GUFFIN_E_ARG, "rope_neox: null pointer");
+    QkvArgs a {};
+    a.q_raw = in; a.planes = 1; a.positions = positions; a.q_out = out;
+    a.rows = rows; a.q_heads = heads; a.kv_heads = 0; a.head_dim = head_dim; a.rope_dim = rope_dim;
+    a.base = freq_base; a.scale = freq_scale; a.eps = 1e-6f;
+    return launch_qkv(stream, a);
+}
+
+extern "C" int guffin_hip_kv_store_f16(void* stream, const float* raw_k, const float* raw_v, const uint32_t* positions,
+                                       void* out_k, void* out_v, uint32_t rows, uint32_t heads, uint32_t head_dim,
+                                       uint32_t rope_dim, float freq_base, float freq_scale, uint32_t* status) {
+    if (!raw_k || !raw_v || !out_k || !out_v) return fail(GUFFIN_E_ARG, "kv_store_f16: null pointer");
+    QkvArgs a {};
+    a.k_raw = raw_k; a.v_raw = raw_v; a.planes = 1; a.positions = positions;
+    a.k_out = static_cast<uint16_t*>(out_k); a.v_out = static_cast<uint16_t*>(out_v);
+    a.rows = rows; a.q_heads = 0; a.kv_heads = heads; a.head_dim = head_dim; a.rope_dim = rope_dim;
+    a.base = freq_base; a.scale = freq_scale; a.eps = 1e-6f; a.status = status;
+    return launch_qkv(stream, a);
+}
+
+extern "C" int guffin_hip_qkv_post(void* stream, const float* q_raw, const float* k_raw, const float* v_raw,
+                                   uint32_t planes, uint64_t q_plane_stride, uint64_t k_plane_stride,
+                                   uint64_t v_plane_stride, const float* q_norm, const float* k_norm,
+                                   const uint32_t* positions, float* q_out, void* k_out, void* v_out,
+                                   uint32_t rows, uint32_t q_heads, uint32_t kv_heads, uint32_t head_dim,
+                                   uint32_t rope_dim, float freq_base, float freq_scale, float eps, uint32_t* status) {
+    if (!q_raw || !k_raw || !v_raw || !q_out || !k_out || !v_out) return fail(GUFFIN_E_ARG, "qkv_post: null pointer");
+    if (planes == 0) return fail(GUFFIN_E_SHAPE, "qkv_post: planes must be >= 1");
+    if (!(eps > 0.f)) return fail(GUFFIN_E_ARG, "qkv_post: epsilon must be positive");
+    QkvArgs a {};
+    a.q_raw = q_raw; a.k_raw = k_raw; a.v_raw = v_raw; a.planes = planes;
+    a.q_plane_stride = q_plane_stride; a.k_plane_stride = k_plane_stride; a.v_plane_stride = v_plane_stride;
+    a.q_norm = q_norm; a.k_norm = k_norm; a.positions = positions;
+    a.q_out = q_out; a.k_out = static_cast<uint16_t*>(k_out); a.v_out = static_cast<uint16_t*>(v_out);
+    a.rows = rows; a.q_heads = q_heads; a.kv_heads = kv_heads; a.head_dim = head_dim; a.rope_dim = rope_dim;
+    a.base = freq_base; a.scale = freq_scale; a.eps = eps; a.status = status;
+    return launch_qkv(stream, a);
+}
+
+extern "C" int guffin_hip_geglu(void* stream, const float* gate, const float* up, uint32_t planes, uint64_t plane_stride,
+                                float* out, float* out_sums, uint32_t rows, uint32_t width) {
+    if (!gate || !up || !out) return fail(GUFFIN_E_ARG, "geglu: null pointer");
+    if (rows == 0 || width == 0 || planes == 0) return fail(GUFFIN_E_SHAPE, "geglu: empty shape");
+    if (out_sums && width % 32 != 0) return fail(GUFFIN_E_SHAPE, "geglu: group sums need width % 32 == 0");
+    // chunks of 512 columns (a multiple of 32) per workgroup
+    const uint32_t chunk = 512, chunks = (width + chunk - 1) / chunk;
+    const uint32_t per = out_sums ? chunk : (width + chunks - 1) / chunks;
+    const uint32_t gx = (width + per - 1) / per;
+    hipLaunchKernelGGL(geglu_kernel, dim3(gx, rows), dim3(256), out_sums ? per * sizeof(float) : 0, as_stream(stream),
+                       gate, up, planes, static_cast<size_t>(plane_stride), out, out_sums, width);
+    return check_launch("geglu");
+}
+
+extern "C" int guffin_hip_embed(void* stream, int dtype, const void* w, const uint32_t* tokens, float* out,
+                                uint32_t rows, uint32_t width, float scale, uint32_t vocab, uint32_t* status) {
+    if (!w || !tokens || !out) return fail(GUFFIN_E_ARG, "embed: null pointer");
+    if (dtype < GUFFIN_Q8_0 || dtype > GUFFIN_Q6_K) return fail(GUFFIN_E_ARG, "embed: unknown dtype");
+    const uint32_t be = dtype == GUFFIN_Q8_0 ? 32u : 256u;
+    if (rows == 0 || width == 0 || width % be != 0 || vocab == 0) return fail(GUFFIN_E_SHAPE, "embed: bad shape");
+    if (reinterpret_cast<uintptr_t>(w) & 1u) return fail(GUFFIN_E_ALIGN, "embed: weights must be 2-byte aligned");
+    const uint8_t* wb = static_cast<const uint8_t*>(w);
+    hipStream_t s = as_stream(stream);
+    if (dtype == GUFFIN_Q8_0) hipLaunchKernelGGL(embed_kernel<GUFFIN_Q8_0>, dim3(rows), dim3(256), 0, s, wb, tokens, out, width, scale, vocab, status);
+    else if (dtype == GUFFIN_Q4_K) hipLaunchKernelGGL(embed_kernel<GUFFIN_Q4_K>, dim3(rows), dim3(256), 0, s, wb, tokens, out, width, scale, vocab, status);
+    else hipLaunchKernelGGL(embed_kernel<GUFFIN_Q6_K>, dim3(rows), dim3(256), 0, s, wb, tokens, out, width, scale, vocab, status);
+    return check_launch("embed");
+}
+
+extern "C" int guffin_hip_kv_scatter(void* stream, const void* priv_k, const void* priv_v, const uint32_t* selected,
+                                     void* ring_k, void* ring_v, uint32_t position, uint32_t rows,
+                                     uint32_t row_width, uint32_t ring_mask) {
+    if (!priv_k || !priv_v || !selected || !ring_k || !ring_v) return fail(GUFFIN_E_ARG, "kv_scatter: null pointer");
+    if (rows == 0 || row_width == 0) return fail(GUFFIN_E_SHAPE, "kv_scatter: empty shape");
+    if ((ring_mask & (ring_mask + 1)) != 0) return fail(GUFFIN_E_ARG, "kv_scatter: ring capacity must be a power of two");
+    hipLaunchKernelGGL(kv_scatter_kernel, dim3((row_width + 255) / 256, rows), dim3(256), 0, as_stream(stream),
+                       static_cast<const uint16_t*>(priv_k), static_cast<const uint16_t*>(priv_v), selected,
+                       static_cast<uint16_t*>(ring_k), static_cast<uint16_t*>(ring_v), position, rows, row_width, ring_mask);
+    return check_launch("kv_scatter");
+}

@@ -110,3 +110,120 @@ def gemv_packed(dtype, tiles, x, xsums, N, partials=None, out=None, reduce=True)
     check(lib().guffin_hip_gemv_packed(_stream(), dtype, _p(tiles), _p(x), _p(xsums), _p(partials),
                                        _p(out) if reduce else C.c_void_p(0), rows, K, N))
     return out if reduce else partials
+
+
+def _f32(shape, like):
+    return torch.empty(shape, dtype=torch.float32, device=like.device)
+
+
+def _planes(x, planes):
+    """(planes, plane_stride) of a [planes, ...] tensor or a plain one."""
+    if planes is None:
+        return 1, 0
+    return planes, x[0].numel()
+
+
+def new_status(device="cuda"):
+    return torch.zeros(1, dtype=torch.int32, device=device)
+
+
+def rms_norm(x, gamma, eps=1e-6, residual=None, planes=None, want_sums=False, status=None):
+    pl, stride = _planes(x, planes)
+    shape = x.shape[1:] if planes else x.shape
+    rows, width = shape
+    y = _f32((rows, width), x)
+    sums = _f32((rows, width // 16 + width // 32), x) if want_sums else None
+    check(lib().guffin_hip_rms_norm(_stream(), _p(x), pl, C.c_uint64(stride), _p(gamma), _p(residual),
+                                    _p(y), _p(sums), rows, width, C.c_float(eps), _p(status)))
+    return (y, sums) if want_sums else y
+
+
+def rms_norm_add_norm(x, gamma_post, residual, gamma_next, eps=1e-6, planes=None, want_sums=False, status=None):
+    pl, stride = _planes(x, planes)
+    shape = x.shape[1:] if planes else x.shape
+    rows, width = shape
+    out_res, out_norm = _f32((rows, width), x), _f32((rows, width), x)
+    sums = _f32((rows, width // 16 + width // 32), x) if want_sums else None
+    check(lib().guffin_hip_rms_norm_add_norm(_stream(), _p(x), pl, C.c_uint64(stride), _p(gamma_post),
+                                             _p(residual), _p(out_res), _p(gamma_next), _p(out_norm), _p(sums),
+                                             rows, width, C.c_float(eps), _p(status)))
+    return out_res, out_norm, sums
+
+
+def head_rms_norm(x, gamma, heads, head_dim, eps=1e-6):
+    y = torch.empty_like(x)
+    check(lib().guffin_hip_head_rms_norm(_stream(), _p(x), _p(gamma), _p(y), x.shape[0], heads, head_dim,
+                                         C.c_float(eps)))
+    return y
+
+
+def rope_neox(x, positions, heads, head_dim, rope_dim, base, scale=1.0):
+    y = torch.empty_like(x)
+    check(lib().guffin_hip_rope_neox(_stream(), _p(x), _p(positions), _p(y), x.shape[0], heads, head_dim,
+                                     rope_dim, C.c_float(base), C.c_float(scale)))
+    return y
+
+
+def kv_store_f16(raw_k, raw_v, positions, heads, head_dim, rope_dim, base, scale=1.0, status=None):
+    k = torch.empty(raw_k.shape, dtype=torch.float16, device=raw_k.device)
+    v = torch.empty(raw_v.shape, dtype=torch.float16, device=raw_v.device)
+    check(lib().guffin_hip_kv_store_f16(_stream(), _p(raw_k), _p(raw_v), _p(positions), _p(k), _p(v),
+                                        raw_k.shape[0], heads, head_dim, rope_dim, C.c_float(base),
+                                        C.c_float(scale), _p(status)))
+    return k, v
+
+
+def qkv_post(q_raw, k_raw, v_raw, q_norm, k_norm, positions, rows, q_heads, kv_heads, head_dim, rope_dim, base,
+             scale=1.0, eps=1e-6, planes=None, status=None):
+    pl = planes or 1
+    strides = [t[0].numel() if planes else 0 for t in (q_raw, k_raw, v_raw)]
+    q = _f32((rows, q_heads * head_dim), q_raw)
+    k = torch.empty((rows, kv_heads * head_dim), dtype=torch.float16, device=q_raw.device)
+    v = torch.empty_like(k)
+    check(lib().guffin_hip_qkv_post(_stream(), _p(q_raw), _p(k_raw), _p(v_raw), pl, C.c_uint64(strides[0]),
+                                    C.c_uint64(strides[1]), C.c_uint64(strides[2]), _p(q_norm), _p(k_norm),
+                                    _p(positions), _p(q), _p(k), _p(v), rows, q_heads, kv_heads, head_dim,
+                                    rope_dim, C.c_float(base), C.c_float(scale), C.c_float(eps), _p(status)))
+    return q, k, v
+
+
+def geglu(gate, up, planes=None, want_sums=False):
+    pl, stride = _planes(gate, planes)
+    rows, width = gate.shape[1:] if planes else gate.shape
+    out = _f32((rows, width), gate)
+    sums = _f32((rows, width // 16 + width // 32), gate) if want_sums else None
+    check(lib().guffin_hip_geglu(_stream(), _p(gate), _p(up), pl, C.c_uint64(stride), _p(out), _p(sums), rows, width))
+    return (out, sums) if want_sums else out
+
+
+def embed(dtype, w, tokens, width, scale, vocab, status=None):
+    out = _f32((tokens.numel(), width), w)
+    check(lib().guffin_hip_embed(_stream(), dtype, _p(w), _p(tokens), _p(out), tokens.numel(), width,
+                                 C.c_float(scale), vocab, _p(status)))
+    return out
+
+
+def kv_scatter(priv_k, priv_v, selected, ring_k, ring_v, position, row_width, ring_mask):
+    check(lib().guffin_hip_kv_scatter(_stream(), _p(priv_k), _p(priv_v), _p(selected), _p(ring_k), _p(ring_v),
+                                      position, selected.numel(), row_width, ring_mask))
+
+
+def attention_partitions(max_tokens, kv_heads):
+    lib().guffin_hip_attention_partitions.restype = C.c_uint32
+    return lib().guffin_hip_attention_partitions(max_tokens, kv_heads)
+
+
+def attention_decode(q, ring_k, ring_v, priv_k, priv_v, schedule, ancestors, max_tokens, ring_mask, q_heads,
+                     kv_heads, head_dim, scale, want_sums=False, status=None):
+    rows = q.shape[0]
+    P = attention_partitions(max_tokens, kv_heads)
+    out = torch.empty_like(q)
+    width = q_heads * head_dim
+    sums = _f32((rows, width // 16 + width // 32), q) if want_sums else None
+    part_out = _f32((rows * q_heads * P * head_dim,), q)
+    part_ml = _f32((rows * q_heads * P * 2,), q)
+    check(lib().guffin_hip_attention_decode(_stream(), _p(q), _p(ring_k), _p(ring_v), _p(priv_k), _p(priv_v),
+                                            _p(schedule), _p(ancestors), _p(out), _p(sums), _p(part_out),
+                                            _p(part_ml), rows, priv_k.shape[0], max_tokens, ring_mask, q_heads,
+                                            kv_heads, head_dim, C.c_float(scale), _p(status)))
+    return (out, sums) if want_sums else out

@@ -97,6 +97,81 @@ uint32_t guffin_hip_gemv_packed_slices(int dtype, uint32_t K, uint32_t N);
 int guffin_hip_gemv_packed(void* stream, int dtype, const void* tiles, const float* x, const float* xsums,
                            float* partials, float* y, uint32_t rows, uint32_t K, uint32_t N);
 
+/* ---- per-layer operators -----------------------------------------------------------------
+ * Inputs produced by a packed GEMV may be given as `planes` k-slice partial planes
+ * (`plane_stride` floats apart) that the operator sums in slice order while loading; plain
+ * tensors pass planes = 1.  Outputs that feed a packed GEMV can also emit their group sums
+ * (`*_sums`, layout of guffin_hip_group_sums; pass NULL to skip). */
+
+/* y = x * rsqrt(mean(x^2) + eps) * gamma (+ residual if non-null).  Replaces encode_rms_norm
+ * (metal_command_context.hpp:128) and encode_rms_norm_add (:137); CPU definition
+ * src/tensor/ops/normalization.cpp:70-99.  status: GUFFIN_STATUS_NONFINITE on a non-finite output. */
+int guffin_hip_rms_norm(void* stream, const float* x, uint32_t planes, uint64_t plane_stride,
+                        const float* gamma, const float* residual, float* y, float* y_sums,
+                        uint32_t rows, uint32_t width, float eps, uint32_t* status);
+/* out_residual = residual + rms(x, gamma_post); out_norm = rms(out_residual, gamma_next): the
+ * encode_rms_norm_add + encode_rms_norm pair at the joints of a block
+ * (src/engine/gemma_target_runtime.cpp:156-173, 201-213 then :60-66 of the next block). */
+int guffin_hip_rms_norm_add_norm(void* stream, const float* x, uint32_t planes, uint64_t plane_stride,
+                                 const float* gamma_post, const float* residual, float* out_residual,
+                                 const float* gamma_next, float* out_norm, float* out_sums,
+                                 uint32_t rows, uint32_t width, float eps, uint32_t* status);
+/* Per-head RMS norm over head_dim, in place allowed.  Replaces encode_head_rms_norm (:119). */
+int guffin_hip_head_rms_norm(void* stream, const float* x, const float* gamma, float* y,
+                             uint32_t rows, uint32_t heads, uint32_t head_dim, float eps);
+/* Split-half (NeoX) RoPE with one absolute position per row: theta = pos / base^(2i/rope_dim) * scale.
+ * Replaces encode_verifier_rope (:239); CPU definition src/tensor/ops/rope.cpp:242-283. */
+int guffin_hip_rope_neox(void* stream, const float* in, const uint32_t* positions, float* out,
+                         uint32_t rows, uint32_t heads, uint32_t head_dim, uint32_t rope_dim,
+                         float freq_base, float freq_scale);
+/* K = f16(rope(raw_k)), V = f16(raw_v), round-to-nearest-even after rotation, into private
+ * rows [rows][heads*head_dim].  Replaces encode_verifier_kv_store (:250; bit contract
+ * tests/tensor/gemma3_metal_tests.cpp:87-128).  status: GUFFIN_STATUS_KV_NONFINITE. */
+int guffin_hip_kv_store_f16(void* stream, const float* raw_k, const float* raw_v, const uint32_t* positions,
+                            void* out_k, void* out_v, uint32_t rows, uint32_t heads, uint32_t head_dim,
+                            uint32_t rope_dim, float freq_base, float freq_scale, uint32_t* status);
+/* The three steps between the QKV GEMVs and attention in one launch: q/k head norms
+ * (NULL gamma skips), RoPE on q and k, fp16 narrowing of k and v
+ * (src/engine/gemma_target_runtime.cpp:92-124). */
+int guffin_hip_qkv_post(void* stream, const float* q_raw, const float* k_raw, const float* v_raw,
+                        uint32_t planes, uint64_t q_plane_stride, uint64_t k_plane_stride,
+                        uint64_t v_plane_stride, const float* q_norm, const float* k_norm,
+                        const uint32_t* positions, float* q_out, void* k_out, void* v_out,
+                        uint32_t rows, uint32_t q_heads, uint32_t kv_heads, uint32_t head_dim,
+                        uint32_t rope_dim, float freq_base, float freq_scale, float eps, uint32_t* status);
+/* out = 0.5 g (1 + tanh(0.7978845608 (g + 0.044715 g^3))) * up.  Replaces
+ * encode_gelu_tanh_multiply (:313); CPU definition src/tensor/ops/elementwise.cpp:79-94, 50-63. */
+int guffin_hip_geglu(void* stream, const float* gate, const float* up, uint32_t planes, uint64_t plane_stride,
+                     float* out, float* out_sums, uint32_t rows, uint32_t width);
+/* out[r,:] = dequant(row tokens[r] of the [vocab x width] canonical block stream) * scale.
+ * Replaces encode_embedding (:75) and the drafter's gd_embed (src/engine/gemma3_draft.mm:61-71).
+ * A token >= vocab sets GUFFIN_STATUS_BAD_TOKEN and reads row 0. */
+int guffin_hip_embed(void* stream, int dtype, const void* w, const uint32_t* tokens, float* out,
+                     uint32_t rows, uint32_t width, float scale, uint32_t vocab, uint32_t* status);
+/* ring[(position + i) & ring_mask] = private[selected[i]] for K and V (fp16 rows of row_width
+ * elements).  Replaces encode_verifier_kv_scatter (:290). */
+int guffin_hip_kv_scatter(void* stream, const void* priv_k, const void* priv_v, const uint32_t* selected,
+                          void* ring_k, void* ring_v, uint32_t position, uint32_t rows,
+                          uint32_t row_width, uint32_t ring_mask);
+
+/* ---- GQA decode / verify attention over the fp16 KV cache -----------------------------------
+ * Replaces encode_verifier_attention (:267) and its partition reducer; CPU definition
+ * src/tensor/ops/attention.cpp:482-618 + softmax.cpp:42-71 (no logit softcap: Gemma 3).
+ * schedule: 4 u32 per row {base_first_position, base_token_count, ancestor_offset, ancestor_count}
+ * (metal_kernels.mm:129-134); row r attends ring slots (base_first+t)&ring_mask for t<base_count,
+ * then private rows ancestors[ancestor_offset + i].  rows in {1,2}; head_dim 256;
+ * q_heads/kv_heads in {1,2,4}.  max_tokens >= (union of the rows' ring ranges) + private_rows.
+ * partial_out holds rows*q_heads*P*head_dim floats and partial_ml rows*q_heads*P*2 floats with
+ * P = guffin_hip_attention_partitions(max_tokens, kv_heads). */
+uint32_t guffin_hip_attention_partitions(uint32_t max_tokens, uint32_t kv_heads);
+int guffin_hip_attention_decode(void* stream, const float* q, const void* ring_k, const void* ring_v,
+                                const void* priv_k, const void* priv_v, const uint32_t* schedule,
+                                const uint32_t* ancestors, float* out, float* out_sums,
+                                float* partial_out, float* partial_ml, uint32_t rows,
+                                uint32_t private_rows, uint32_t max_tokens, uint32_t ring_mask,
+                                uint32_t q_heads, uint32_t kv_heads, uint32_t head_dim, float scale,
+                                uint32_t* status);
+
 #ifdef __cplusplus
 }
 #endif

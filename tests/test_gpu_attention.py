@@ -1,0 +1,110 @@
+"""GPU parity of the GQA decode/verify attention against the CPU oracle and closed forms.
+
+The reference checks its kernel against a double-precision softmax at 2e-7 on a
+tree + wrapped-ring case (tests/tensor/gemma3_metal_tests.cpp:746-833); the oracle here
+follows the CPU operators (fp32 dots, double exp), so the bar is a few fp32 ulps of the
+value scale.
+"""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def hip():
+    from guffin_amd import hip as module
+    module.init(0)
+    return module
+
+
+def dev(a):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def contiguous_schedule(position, rows, window):
+    sched = []
+    for row in range(rows):
+        p = position + row
+        ws = p + 1 - window if (window and p >= window) else 0
+        base_start = min(position, ws)
+        private_start = max(ws - position, 0) if ws > position else 0
+        sched.append([base_start, position - base_start, private_start, row + 1 - private_start])
+    return np.array(sched, np.uint32)
+
+
+def run_case(hip, gfo, rows, q_heads, kv_heads, cap, position, window, seed, sigma_v=1.0):
+    hd = 256
+    rng = np.random.default_rng(seed)
+    ring_k = rng.normal(0, 1, (cap, kv_heads * hd)).astype(np.float16)
+    ring_v = rng.normal(0, sigma_v, (cap, kv_heads * hd)).astype(np.float16)
+    pk = rng.normal(0, 1, (rows, kv_heads * hd)).astype(np.float16)
+    pv = rng.normal(0, sigma_v, (rows, kv_heads * hd)).astype(np.float16)
+    q = rng.normal(0, 1, (rows, q_heads * hd)).astype(np.float32)
+    sched = contiguous_schedule(position, rows, window)
+    anc = np.arange(rows, dtype=np.uint32)
+    want = gfo.attention(q, ring_k.view(np.uint16), ring_v.view(np.uint16), pk.view(np.uint16),
+                         pv.view(np.uint16), sched, anc, cap - 1, q_heads, kv_heads, hd, 0.0625)
+    union = int(max(s[0] + s[1] for s in sched) - min(s[0] for s in sched if s[1]) if any(s[1] for s in sched) else 0)
+    out, sums = hip.attention_decode(dev(q), dev(ring_k), dev(ring_v), dev(pk), dev(pv), dev(sched), dev(anc),
+                                     union + rows, cap - 1, q_heads, kv_heads, hd, 0.0625, want_sums=True)
+    out = out.cpu().numpy()
+    err = np.max(np.abs(out - want))
+    assert err <= 3e-6 * sigma_v * 4, err
+    o64 = out.astype(np.float64)
+    ref_sums = np.concatenate([o64.reshape(rows, -1, 16).sum(-1), o64.reshape(rows, -1, 32).sum(-1)], axis=1)
+    assert np.allclose(sums.cpu().numpy(), ref_sums, rtol=0, atol=1e-4 * sigma_v)
+    return out
+
+
+@pytest.mark.parametrize("rows,q_heads,kv_heads,cap,position,window", [
+    (2, 16, 8, 1024, 8190, 1024),   # target local layer: wrapped ring, window drops the oldest token for row 1
+    (2, 16, 8, 8192, 8190, 0),      # target global layer
+    (1, 16, 8, 1024, 500, 1024),    # single row, ring not yet wrapped
+    (1, 4, 1, 512, 4096, 512),      # drafter local
+    (1, 4, 1, 8192, 4096, 0),       # drafter global
+    (2, 4, 2, 64, 5, 0),            # tiny: one partition, mostly masked
+    (2, 2, 2, 64, 0, 0),            # empty prefix: only the private rows
+])
+def test_attention_matches_oracle(hip, gfo, rows, q_heads, kv_heads, cap, position, window):
+    run_case(hip, gfo, rows, q_heads, kv_heads, cap, position, window, seed=rows * 100 + q_heads)
+
+
+def test_attention_large_values_keep_relative_accuracy(hip, gfo):
+    run_case(hip, gfo, 2, 16, 8, 1024, 3000, 1024, seed=77, sigma_v=200.0)
+
+
+def test_attention_closed_forms(hip):
+    import torch
+    hd, cap, q_heads, kv_heads = 256, 64, 4, 2
+    rng = np.random.default_rng(3)
+    q = rng.normal(0, 1, (1, q_heads * hd)).astype(np.float32)
+    ring_k = np.ones((cap, kv_heads * hd), np.float16)            # uniform keys -> uniform weights
+    ring_v = rng.normal(0, 1, (cap, kv_heads * hd)).astype(np.float16)
+    pk = np.ones((1, kv_heads * hd), np.float16)
+    pv = rng.normal(0, 1, (1, kv_heads * hd)).astype(np.float16)
+    sched = np.array([[60, 9, 0, 1]], np.uint32)                   # ring slots 60..63, 0..4 then self
+    out = hip.attention_decode(dev(q), dev(ring_k), dev(ring_v), dev(pk), dev(pv), dev(sched),
+                               dev(np.array([0], np.uint32)), 10, cap - 1, q_heads, kv_heads, hd, 0.0625).cpu().numpy()
+    slots = [(60 + t) & 63 for t in range(9)]
+    mean = np.concatenate([ring_v[slots], pv]).astype(np.float64).mean(0).reshape(kv_heads, hd)
+    want = np.repeat(mean, 2, axis=0).reshape(1, -1)
+    assert np.max(np.abs(out - want)) < 1e-6
+    # a single attended token returns its value row exactly
+    sched1 = np.array([[0, 0, 0, 1]], np.uint32)
+    out1 = hip.attention_decode(dev(q), dev(ring_k), dev(ring_v), dev(pk), dev(pv), dev(sched1),
+                                dev(np.array([0], np.uint32)), 1, cap - 1, q_heads, kv_heads, hd, 0.0625).cpu().numpy()
+    want1 = np.repeat(pv.astype(np.float32).reshape(kv_heads, hd), 2, axis=0).reshape(1, -1)
+    assert np.array_equal(out1, want1)
+
+
+def test_attention_rejects_bad_shapes(hip):
+    import torch
+    z = torch.zeros(4096, dtype=torch.float32, device="cuda")
+    h = torch.zeros((4, 512), dtype=torch.float16, device="cuda")
+    s = torch.zeros(8, dtype=torch.int32, device="cuda")
+    with pytest.raises(hip.GuffinError):   # head_dim 128 unsupported
+        hip.attention_decode(z[:256].view(1, 256), h, h, h[:1], h[:1], s, s, 4, 3, 2, 2, 128, 0.1)
+    with pytest.raises(hip.GuffinError):   # ring capacity not a power of two
+        hip.attention_decode(z[:1024].view(1, 1024), h, h, h[:1], h[:1], s, s, 4, 2, 4, 2, 256, 0.1)
