@@ -30,6 +30,7 @@ int check_launch(const char* what) {
 int gemv_init(int cu_count);
 int ops_init(int cu_count);
 void gemv_packed_init(int cu_count);
+int head_init();
 
 }  // namespace guffin
 
@@ -52,7 +53,7 @@ extern "C" int guffin_hip_init(int device) {
         std::snprintf(buf, sizeof(buf), "init: code object is gfx950 only, device is %s", prop.gcnArchName);
         return fail(GUFFIN_E_HIP, buf);
     }
-    if (gemv_init(prop.multiProcessorCount) != 0 || ops_init(prop.multiProcessorCount) != 0)
+    if (gemv_init(prop.multiProcessorCount) != 0 || ops_init(prop.multiProcessorCount) != 0 || head_init() != 0)
         return fail(GUFFIN_E_HIP, "init: could not raise a kernel's dynamic LDS limit");
     gemv_packed_init(prop.multiProcessorCount);
     return GUFFIN_OK;

@@ -1,0 +1,244 @@
+// Output-head selection over the 262144-entry logits rows (gfx950).
+//
+// Replaces encode_token_candidates / encode_target_token_candidates and their tile-sort,
+// merge-tree and finalize kernels (src/tensor/backends/metal/metal_command_context.hpp:326-345,
+// src/tensor/backends/metal/metal_kernels.mm:3444-3884), and the CPU argmax
+// (src/tensor/ops/reduction.cpp:93-117).  Order everywhere: higher logit first, then lower
+// token id (src/engine/sampling.cpp:25-30, metal_kernels.mm:171-173).
+//
+// An entry is one 64-bit key {ordered(logit) : 32 | ~token : 32}; descending key order is the
+// candidate order and keys are unique, so selection is a pure comparison network and the
+// result is exact including ties.
+//   stage 1  every workgroup sorts a 2048-logit tile in LDS (bitonic) and keeps its best R
+//   stage 2  one workgroup per row merges the G*R survivors (bitonic, in rounds if needed),
+//            writes the best `retain`, then appends the logits of the history tokens
+// A global top-R entry is necessarily a top-R entry of its own tile, so the two stages lose
+// nothing.
+#include "common.hpp"
+
+namespace guffin {
+namespace {
+
+constexpr uint32_t kTile = 2048;          // logits per stage-1 workgroup
+constexpr uint32_t kMergeCap = 16384;     // keys a stage-2 round sorts in LDS (128 KiB)
+
+__device__ __forceinline__ uint64_t make_key(float logit, uint32_t token) {
+    const uint32_t b = __float_as_uint(logit + 0.0f);  // -0 orders as +0, as a float comparison does
+    const uint32_t ordered = (b & 0x80000000u) ? ~b : (b | 0x80000000u);
+    return (uint64_t(ordered) << 32) | (0xFFFFFFFFu - token);
+}
+[[maybe_unused]] __device__ __forceinline__ float key_logit(uint64_t key) {
+    const uint32_t o = static_cast<uint32_t>(key >> 32);
+    return __uint_as_float((o & 0x80000000u) ? (o & 0x7FFFFFFFu) : ~o);
+}
+__device__ __forceinline__ uint32_t key_token(uint64_t key) { return 0xFFFFFFFFu - static_cast<uint32_t>(key); }
+
+// descending bitonic sort of n (power of two) keys in LDS by all threads of the workgroup
+__device__ __forceinline__ void bitonic_desc(uint64_t* keys, uint32_t n) {
+    for (uint32_t width = 2; width <= n; width <<= 1) {
+        for (uint32_t stride = width >> 1; stride > 0; stride >>= 1) {
+            __syncthreads();
+            for (uint32_t i = threadIdx.x; i < n / 2; i += blockDim.x) {
+                const uint32_t lo = 2 * i - (i & (stride - 1));   // index with the `stride` bit clear
+                const uint32_t hi = lo + stride;
+                const bool descending = (lo & width) == 0;
+                const uint64_t a = keys[lo], b = keys[hi];
+                if ((a < b) == descending) { keys[lo] = b; keys[hi] = a; }
+            }
+        }
+    }
+    __syncthreads();
+}
+
+__global__ void __launch_bounds__(1024)
+topk_tile_kernel(const float* __restrict__ logits, uint64_t* __restrict__ survivors, uint32_t vocab,
+                 uint32_t keep, float divisor, uint32_t* __restrict__ status) {
+    __shared__ uint64_t keys[kTile];
+    const uint32_t tile = blockIdx.x, row = blockIdx.y;
+    const float* lr = logits + size_t(row) * vocab;
+    bool bad = false;
+    for (uint32_t i = threadIdx.x; i < kTile; i += blockDim.x) {
+        const uint32_t t = tile * kTile + i;
+        uint64_t k = 0;  // below every real key
+        if (t < vocab) {
+            const float v = lr[t] / divisor;  // IEEE division: the drafter's score = logit / T
+            bad |= !isfinite(v) || !isfinite(lr[t]);
+            k = make_key(v, t);
+        }
+        keys[i] = k;
+    }
+    if (bad && status) atomicOr(status + row, GUFFIN_STATUS_NONFINITE);
+    bitonic_desc(keys, kTile);
+    uint64_t* out = survivors + (size_t(row) * gridDim.x + tile) * keep;
+    for (uint32_t i = threadIdx.x; i < keep; i += blockDim.x) out[i] = keys[i];
+}
+
+struct Candidates {  // layout of one row of the result (sampling.hpp:57-61 plus a status word)
+    uint32_t count;
+    uint32_t status;
+    struct { uint32_t token; float logit; } values[384];
+};
+
+__global__ void __launch_bounds__(1024)
+topk_merge_kernel(const float* __restrict__ logits, const uint64_t* __restrict__ survivors, uint32_t n_survivors,
+                  uint32_t vocab, uint32_t retain, float divisor, const uint32_t* __restrict__ history,
+                  const uint32_t* __restrict__ history_count, Candidates* __restrict__ result,
+                  uint32_t* __restrict__ status) {
+    extern __shared__ uint64_t keys[];  // kMergeCap
+    const uint32_t row = blockIdx.x;
+    const uint64_t* src = survivors + size_t(row) * n_survivors;
+    // round 0 sorts the first chunk; later rounds merge the running best `retain` with the next chunk
+    uint32_t done = 0, have = 0;
+    while (done < n_survivors) {
+        const uint32_t room = kMergeCap - have;
+        const uint32_t take = n_survivors - done < room ? n_survivors - done : room;
+        uint32_t n = 1;
+        while (n < have + take) n <<= 1;
+        for (uint32_t i = threadIdx.x; i < n - have; i += blockDim.x) keys[have + i] = i < take ? src[done + i] : 0;
+        bitonic_desc(keys, n);
+        done += take;
+        have = retain < n ? retain : n;
+    }
+    Candidates& out = result[row];
+    const uint32_t hc = history_count ? history_count[row] : 0;
+    for (uint32_t i = threadIdx.x; i < retain; i += blockDim.x) {
+        const uint32_t token = key_token(keys[i]);
+        out.values[i].token = token;
+        out.values[i].logit = logits[size_t(row) * vocab + token] / divisor;  // the native value, not the key's
+    }
+    uint32_t st = 0;
+    for (uint32_t i = threadIdx.x; i < hc; i += blockDim.x) {
+        const uint32_t token = history[row * 64 + i];
+        if (token >= vocab) {
+            st |= GUFFIN_STATUS_BAD_TOKEN;
+            out.values[retain + i].token = 0xFFFFFFFFu;
+            out.values[retain + i].logit = -INFINITY;
+        } else {
+            const float v = logits[size_t(row) * vocab + token] / divisor;
+            if (!isfinite(v)) st |= GUFFIN_STATUS_NONFINITE;
+            out.values[retain + i].token = token;
+            out.values[retain + i].logit = v;
+        }
+    }
+    if (st && status) atomicOr(status + row, st);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        out.count = retain + hc;
+        out.status = status ? status[row] : 0;
+    }
+}
+
+// ---- greedy argmax ---------------------------------------------------------------------
+__global__ void __launch_bounds__(256)
+argmax_tile_kernel(const float* __restrict__ logits, uint64_t* __restrict__ partial, uint32_t vocab,
+                   uint32_t* __restrict__ status) {
+    __shared__ uint64_t best[4];
+    const uint32_t row = blockIdx.y;
+    const float* lr = logits + size_t(row) * vocab;
+    uint64_t k = 0;
+    bool bad = false;
+    for (uint32_t t = blockIdx.x * blockDim.x + threadIdx.x; t < vocab; t += gridDim.x * blockDim.x) {
+        const float v = lr[t];
+        bad |= !isfinite(v);
+        const uint64_t c = make_key(v, t);
+        k = c > k ? c : k;
+    }
+    if (bad && status) atomicOr(status + row, GUFFIN_STATUS_NONFINITE);
+#pragma unroll
+    for (int s = 32; s > 0; s >>= 1) {
+        const uint64_t o = __shfl_xor(k, s, kWave);
+        k = o > k ? o : k;
+    }
+    if ((threadIdx.x & 63) == 0) best[threadIdx.x >> 6] = k;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int i = 1; i < 4; ++i) k = best[i] > k ? best[i] : k;
+        partial[size_t(row) * gridDim.x + blockIdx.x] = k;
+    }
+}
+
+__global__ void __launch_bounds__(256)
+argmax_final_kernel(const uint64_t* __restrict__ partial, uint32_t n, uint32_t* __restrict__ token,
+                    float* __restrict__ logit) {
+    __shared__ uint64_t best[4];
+    const uint32_t row = blockIdx.x;
+    uint64_t k = 0;
+    for (uint32_t i = threadIdx.x; i < n; i += blockDim.x) {
+        const uint64_t c = partial[size_t(row) * n + i];
+        k = c > k ? c : k;
+    }
+#pragma unroll
+    for (int s = 32; s > 0; s >>= 1) {
+        const uint64_t o = __shfl_xor(k, s, kWave);
+        k = o > k ? o : k;
+    }
+    if ((threadIdx.x & 63) == 0) best[threadIdx.x >> 6] = k;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int i = 1; i < 4; ++i) k = best[i] > k ? best[i] : k;
+        token[row] = key_token(k);
+        if (logit) logit[row] = key_logit(k);
+    }
+}
+
+}  // namespace
+
+int head_init() {
+    return hipFuncSetAttribute(reinterpret_cast<const void*>(topk_merge_kernel),
+                               hipFuncAttributeMaxDynamicSharedMemorySize, kMergeCap * 8) != hipSuccess;
+}
+
+}  // namespace guffin
+
+using namespace guffin;
+
+extern "C" uint64_t guffin_hip_select_workspace_bytes(uint32_t rows, uint32_t vocab, uint32_t retain) {
+    const uint64_t tiles = (uint64_t(vocab) + kTile - 1) / kTile;
+    const uint64_t keep = retain < kTile ? retain : kTile;
+    return rows * tiles * keep * 8;
+}
+
+namespace guffin {
+int select_candidates_scaled(hipStream_t s, const float* logits, uint32_t rows, uint32_t vocab, uint32_t retain,
+                             float divisor, const uint32_t* history, const uint32_t* history_count,
+                             void* workspace, void* result, uint32_t* status);
+}
+
+extern "C" int guffin_hip_select_candidates(void* stream, const float* logits, uint32_t rows, uint32_t vocab,
+                                            uint32_t retain, const uint32_t* history, const uint32_t* history_count,
+                                            void* workspace, void* result, uint32_t* status) {
+    return select_candidates_scaled(as_stream(stream), logits, rows, vocab, retain, 1.0f, history, history_count,
+                                    workspace, result, status);
+}
+
+int guffin::select_candidates_scaled(hipStream_t s, const float* logits, uint32_t rows, uint32_t vocab,
+                                     uint32_t retain, float divisor, const uint32_t* history,
+                                     const uint32_t* history_count, void* workspace, void* result, uint32_t* status) {
+    if (!logits || !workspace || !result) return fail(GUFFIN_E_ARG, "select_candidates: null pointer");
+    if (rows == 0 || vocab == 0) return fail(GUFFIN_E_SHAPE, "select_candidates: empty shape");
+    if (retain == 0 || retain > 320) return fail(GUFFIN_E_CAPACITY, "select_candidates: retain must be in [1, 320] (top_k <= 256 plus 64 history tokens)");
+    if ((history == nullptr) != (history_count == nullptr)) return fail(GUFFIN_E_ARG, "select_candidates: history and its counts come together");
+    if (reinterpret_cast<uintptr_t>(workspace) & 7u) return fail(GUFFIN_E_ALIGN, "select_candidates: workspace must be 8-byte aligned");
+    const uint32_t keep = retain < vocab ? retain : vocab;
+    const uint32_t tiles = (vocab + kTile - 1) / kTile;
+    uint64_t* surv = static_cast<uint64_t*>(workspace);
+    hipLaunchKernelGGL(topk_tile_kernel, dim3(tiles, rows), dim3(1024), 0, s, logits, surv, vocab, keep, divisor, status);
+    if (int rc = check_launch("select_candidates(tile)")) return rc;
+    hipLaunchKernelGGL(topk_merge_kernel, dim3(rows), dim3(1024), kMergeCap * 8, s, logits, surv, tiles * keep, vocab,
+                       keep, divisor, history, history_count, static_cast<Candidates*>(result), status);
+    return check_launch("select_candidates(merge)");
+}
+
+extern "C" int guffin_hip_argmax(void* stream, const float* logits, uint32_t rows, uint32_t vocab, void* workspace,
+                                 uint32_t* token, float* logit, uint32_t* status) {
+    if (!logits || !workspace || !token) return fail(GUFFIN_E_ARG, "argmax: null pointer");
+    if (rows == 0 || vocab == 0) return fail(GUFFIN_E_SHAPE, "argmax: empty shape");
+    if (reinterpret_cast<uintptr_t>(workspace) & 7u) return fail(GUFFIN_E_ALIGN, "argmax: workspace must be 8-byte aligned");
+    const uint32_t blocks = vocab / 1024 < 1 ? 1 : (vocab / 1024 > 256 ? 256 : vocab / 1024);
+    hipStream_t s = as_stream(stream);
+    uint64_t* part = static_cast<uint64_t*>(workspace);  // rows * 256 keys at most
+    hipLaunchKernelGGL(argmax_tile_kernel, dim3(blocks, rows), dim3(256), 0, s, logits, part, vocab, status);
+    if (int rc = check_launch("argmax(tile)")) return rc;
+    hipLaunchKernelGGL(argmax_final_kernel, dim3(rows), dim3(256), 0, s, part, blocks, token, logit);
+    return check_launch("argmax(final)");
+}

@@ -1,0 +1,508 @@
+// Proposal law of the drafter and lossless accept / residual sampling (gfx950).
+//
+// Reference behaviour:
+//   compact proposal law (integer 2^32-mass CDF)   src/engine/gemma3_draft.mm:191-294, 995-1070
+//   gather of q on p's support                     src/engine/gemma3_draft.mm:1528-1581
+//   target law p (all double)                      src/engine/sampling.cpp:394-499
+//   validation / Neumaier total                    src/engine/sampling.cpp:117-158
+//   accept min(1,p/q), residual max(p-q,0)         src/engine/sampling.cpp:561-656
+//   inverse-CDF selections                         src/engine/sampling.cpp:247-257, 501-514
+//   draw consumption order                         src/engine/sampling.cpp:896-934
+// The reference evaluates the target law and the accept test on the host from a compact
+// read-back; here both run on the device in the same fp64 operation order (sequential sums
+// are taken by one lane in the reference's order), so decisions depend only on the inputs and
+// the draws.  Draws come from Philox4x32-10 keyed (seed, step) unless injected.
+#include "common.hpp"
+
+namespace guffin {
+namespace {
+
+constexpr uint32_t kMaxTopK = 256, kMaxCandidates = 384;
+constexpr uint64_t kMassTotal = uint64_t{1} << 32;
+
+struct Candidates { uint32_t count; uint32_t status; struct { uint32_t token; float logit; } values[384]; };
+struct DraftLaw { uint32_t count; uint32_t pad; uint32_t ids[256]; uint64_t cdf[257]; };
+struct SamplerOptions { float temperature; uint32_t top_k; float top_p; float min_p; float repetition_penalty; };
+struct StepDraws { uint32_t word; uint32_t pad; double u_accept, u_residual, u_next; };
+struct SpecResult {
+    uint32_t accepted, token, next_root, status;
+    double acceptance_probability, residual_total;
+    uint32_t residual_count, proposal;
+};
+
+// ---- Philox4x32-10 ----------------------------------------------------------------------
+__device__ __forceinline__ void philox(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, uint32_t k0, uint32_t k1,
+                                       uint32_t (&out)[4]) {
+#pragma unroll
+    for (int round = 0; round < 10; ++round) {
+        const uint64_t p0 = uint64_t{0xD2511F53u} * c0, p1 = uint64_t{0xCD9E8D57u} * c2;
+        const uint32_t n0 = static_cast<uint32_t>(p1 >> 32) ^ c1 ^ k0, n1 = static_cast<uint32_t>(p1);
+        const uint32_t n2 = static_cast<uint32_t>(p0 >> 32) ^ c3 ^ k1, n3 = static_cast<uint32_t>(p0);
+        c0 = n0; c1 = n1; c2 = n2; c3 = n3;
+        k0 += 0x9E3779B9u; k1 += 0xBB67AE85u;
+    }
+    out[0] = c0; out[1] = c1; out[2] = c2; out[3] = c3;
+}
+__device__ __forceinline__ double unit_double(uint32_t hi, uint32_t lo) {
+    return static_cast<double>(((uint64_t{hi} << 32) | lo) >> 11) * 0x1.0p-53;
+}
+// word, u_accept from counter (step, 0); u_residual, u_next from counter (step, 1)
+__device__ __forceinline__ StepDraws step_draws(uint64_t seed, uint64_t step) {
+    uint32_t a[4], b[4];
+    const uint32_t k0 = static_cast<uint32_t>(seed), k1 = static_cast<uint32_t>(seed >> 32);
+    const uint32_t s0 = static_cast<uint32_t>(step), s1 = static_cast<uint32_t>(step >> 32);
+    philox(s0, s1, 0, 0, k0, k1, a);
+    philox(s0, s1, 1, 0, k0, k1, b);
+    StepDraws d;
+    d.word = a[0]; d.pad = 0;
+    d.u_accept = unit_double(a[1], a[2]);
+    d.u_residual = unit_double(b[0], b[1]);
+    d.u_next = unit_double(b[2], b[3]);
+    return d;
+}
+
+// exp for the law's f32 weights from IEEE-exact operations only (fma, floor, exponent
+// scaling), so the integer CDF is reproducible bit for bit on any conforming machine.
+__device__ __forceinline__ float law_exp(float x) {
+    if (!(x > -86.0f)) return x != x ? x : 0.0f;
+    if (x > 88.0f) return INFINITY;
+    const float kf = floorf(fmaf(x, 1.44269502162933349609375f, 0.5f));
+    float r = fmaf(kf, -0.693145751953125f, x);
+    r = fmaf(kf, -1.428606765330187045037746429443359375e-06f, r);
+    float p = 1.0f / 5040.0f;
+    p = fmaf(p, r, 1.0f / 720.0f);
+    p = fmaf(p, r, 1.0f / 120.0f);
+    p = fmaf(p, r, 1.0f / 24.0f);
+    p = fmaf(p, r, 1.0f / 6.0f);
+    p = fmaf(p, r, 0.5f);
+    p = fmaf(p, r, 1.0f);
+    p = fmaf(p, r, 1.0f);
+    const int k = static_cast<int>(kf);
+    return __fmul_rn(p, __uint_as_float(static_cast<uint32_t>(k + 127) << 23));
+}
+
+__device__ __forceinline__ bool options_valid(const SamplerOptions& o) {
+    return isfinite(o.temperature) && o.temperature >= 0.f && o.top_k >= 1 && o.top_k <= kMaxTopK
+        && isfinite(o.top_p) && o.top_p > 0.f && o.top_p <= 1.f && isfinite(o.min_p) && o.min_p >= 0.f
+        && o.min_p <= 1.f && isfinite(o.repetition_penalty) && o.repetition_penalty > 0.f;
+}
+
+// bitonic sort of n (power of two) 64-bit keys in LDS, ascending or descending
+__device__ __forceinline__ void bitonic(uint64_t* keys, uint32_t n, bool desc) {
+    for (uint32_t width = 2; width <= n; width <<= 1)
+        for (uint32_t stride = width >> 1; stride > 0; stride >>= 1) {
+            __syncthreads();
+            for (uint32_t i = threadIdx.x; i < n / 2; i += blockDim.x) {
+                const uint32_t lo = 2 * i - (i & (stride - 1)), hi = lo + stride;
+                const bool first_dir = (lo & width) == 0;
+                const uint64_t a = keys[lo], b = keys[hi];
+                if (((a < b) == desc) == first_dir) { keys[lo] = b; keys[hi] = a; }
+            }
+        }
+    __syncthreads();
+}
+
+__device__ __forceinline__ uint64_t score_key(float score, uint32_t token) {
+    const uint32_t b = __float_as_uint(score + 0.0f);
+    const uint32_t ordered = (b & 0x80000000u) ? ~b : (b | 0x80000000u);
+    return (uint64_t(ordered) << 32) | (0xFFFFFFFFu - token);
+}
+
+// =========================================================================================
+// Compact proposal law from the best 257 scores (sorted, score = logit / T)
+// =========================================================================================
+__global__ void __launch_bounds__(256)
+draft_law_kernel(const Candidates* __restrict__ top, SamplerOptions opt, uint64_t seed, uint64_t step,
+                 const StepDraws* __restrict__ injected, DraftLaw* __restrict__ law,
+                 uint32_t* __restrict__ proposal, uint32_t* __restrict__ status) {
+    __shared__ uint64_t keys[256];
+    __shared__ float score[256], weight[256];
+    __shared__ uint32_t s_n;
+    const uint32_t t = threadIdx.x;
+    const uint32_t avail = top->count;
+    if (t == 0) {
+        uint32_t st = 0, n = 0;
+        if (!options_valid(opt) || opt.temperature <= 0.f || opt.top_k > 64 || avail < 1) st = GUFFIN_STATUS_LAW_INVALID;
+        if (top->status & GUFFIN_STATUS_NONFINITE) st = GUFFIN_STATUS_LAW_INVALID | GUFFIN_STATUS_NONFINITE;
+        if (!st) {
+            const uint32_t k = opt.top_k < avail ? opt.top_k : avail;
+            const float cutoff = top->values[k - 1].logit;
+            // entries are sorted by (score desc, token asc): the support is a prefix
+            while (n < avail && !(top->values[n].logit < cutoff)) ++n;
+            if (n > 256) st = GUFFIN_STATUS_LAW_INVALID | 32u;  // support overflow: needs the full-vocabulary law
+        }
+        s_n = st ? 0 : n;
+        if (st) { atomicOr(status, st); law->count = 0; *proposal = 0xFFFFFFFFu; }
+    }
+    __syncthreads();
+    const uint32_t n = s_n;
+    if (n == 0) return;
+    score[t] = t < n ? top->values[t].logit : -INFINITY;
+    weight[t] = t < n ? law_exp(top->values[t].logit - top->values[0].logit) : 0.f;
+    __syncthreads();
+    if (t == 0) {  // descending-tail top-p / min-p in the reference's sequential order
+        float total = 0.f, tail = 0.f;
+        for (uint32_t j = n; j > 0; --j) total = __fadd_rn(total, weight[j - 1]);
+        for (uint32_t j = n; j > 0; --j) {
+            const uint32_t i = j - 1;
+            tail = __fadd_rn(tail, weight[i]);
+            const bool keep = i == 0
+                || ((opt.top_p >= 1.0f || __fdiv_rn(tail, total) > __fsub_rn(1.0f, opt.top_p))
+                    && (opt.min_p <= 0.0f || weight[i] >= opt.min_p));
+            if (!keep) score[i] = -INFINITY;
+        }
+    }
+    __syncthreads();
+    // ascending token id; the score rides in the low half of the key
+    keys[t] = t < n ? (uint64_t(top->values[t].token) << 32) | __float_as_uint(score[t]) : ~uint64_t{0};
+    bitonic(keys, 256, false);
+    const float s = __uint_as_float(static_cast<uint32_t>(keys[t]));
+    score[t] = t < n ? s : -INFINITY;
+    __syncthreads();
+    if (t == 0) {
+        float maximum = -INFINITY;
+        for (uint32_t i = 0; i < n; ++i) maximum = fmaxf(maximum, score[i]);
+        weight[0] = maximum;  // broadcast slot
+    }
+    __syncthreads();
+    const float maximum = weight[0];
+    __syncthreads();
+    weight[t] = t < n ? law_exp(__fsub_rn(score[t], maximum)) : 0.f;
+    __syncthreads();
+    if (t == 0) {
+        float total = 0.f;
+        for (uint32_t i = 0; i < n; ++i) total = __fadd_rn(total, weight[i]);
+        uint32_t st = 0;
+        if (!(total > 0.f) || !isfinite(total)) st = GUFFIN_STATUS_LAW_INVALID;
+        const StepDraws d = injected ? *injected : step_draws(seed, step);
+        float prefix = 0.f;
+        uint64_t last = 0;
+        uint32_t chosen = 0xFFFFFFFFu;
+        law->count = n; law->pad = 0; law->cdf[0] = 0;
+        for (uint32_t i = 0; i < n && !st; ++i) {
+            law->ids[i] = static_cast<uint32_t>(keys[i] >> 32);
+            prefix = __fadd_rn(prefix, weight[i]);
+            float scaled = __fmul_rn(__fdiv_rn(prefix, total), 4294967296.0f);
+            scaled = fminf(fmaxf(scaled, 0.0f), 4294967296.0f);
+            const uint64_t next = static_cast<uint64_t>(scaled);
+            law->cdf[i + 1] = next;
+            if (next < last || next > kMassTotal) st = GUFFIN_STATUS_LAW_INVALID;
+            if (uint64_t(d.word) >= last && uint64_t(d.word) < next) chosen = law->ids[i];
+            last = next;
+        }
+        if (!st && last != kMassTotal) st = GUFFIN_STATUS_LAW_INVALID;
+        if (st) { atomicOr(status, st); chosen = 0xFFFFFFFFu; }
+        *proposal = chosen;
+    }
+}
+
+// =========================================================================================
+// Target law (prepare_token_distribution) — whole workgroup, 512 threads
+// =========================================================================================
+struct Prepared {
+    uint32_t count;
+    double total;
+    uint32_t token[kMaxTopK];
+    double weight[kMaxTopK];
+};
+
+struct Scratch {
+    uint64_t keys[512];
+    float logit[512];
+    double w[kMaxTopK];
+    int err;
+};
+
+// returns 0 or a negative error; result in `out` (shared); uses all threads
+__device__ int prepare_distribution(const Candidates* cand, const SamplerOptions& opt, const uint32_t* history,
+                                    uint32_t history_count, Scratch& sc, Prepared& out) {
+    const uint32_t t = threadIdx.x, n = cand->count;
+    if (t == 0) sc.err = (!options_valid(opt) ? -1 : (n == 0 || n > kMaxCandidates) ? -2 : history_count > 64 ? -3 : 0);
+    __syncthreads();
+    if (sc.err) return sc.err;
+    const uint32_t request_top_k = opt.temperature == 0.f ? 1u : opt.top_k;
+    // dedup (a later duplicate must carry the same logit), repetition penalty, sort key
+    uint64_t key = 0;
+    if (t < n) {
+        const uint32_t token = cand->values[t].token;
+        float logit = cand->values[t].logit;
+        bool dup = false;
+        if (!isfinite(logit)) atomicMin(&sc.err, -4);
+        for (uint32_t j = 0; j < t; ++j)
+            if (cand->values[j].token == token) {
+                dup = true;
+                if (cand->values[j].logit != logit) atomicMin(&sc.err, -5);
+            }
+        if (!dup) {
+            for (uint32_t h = 0; h < history_count; ++h)
+                if (history[h] == token) {
+                    logit = logit < 0.f ? __fmul_rn(logit, opt.repetition_penalty) : __fdiv_rn(logit, opt.repetition_penalty);
+                    break;
+                }
+            key = score_key(logit, token);
+            sc.logit[t] = logit;
+        }
+    }
+    if (t < 512) sc.keys[t] = key;
+    __syncthreads();
+    if (sc.err) return sc.err;
+    bitonic(sc.keys, 512, true);
+    // unique count = number of non-zero keys (a real key is never 0: ordered(logit) has a set bit)
+    uint32_t mine = (t < 512 && sc.keys[t] != 0) ? 1u : 0u;
+    const uint32_t unique = __syncthreads_count(mine);
+    if (unique < request_top_k) return -6;
+    uint32_t count = unique < request_top_k ? unique : request_top_k;
+    // logits back from the sorted keys
+    if (t < count) {
+        const uint32_t o = static_cast<uint32_t>(sc.keys[t] >> 32);
+        sc.logit[t] = __uint_as_float((o & 0x80000000u) ? (o & 0x7FFFFFFFu) : ~o);
+        out.token[t] = 0xFFFFFFFFu - static_cast<uint32_t>(sc.keys[t]);
+    }
+    __syncthreads();
+    if (opt.temperature == 0.f) {
+        if (t == 0) { out.count = 1; out.total = 1.0; out.weight[0] = 1.0; }
+        __syncthreads();
+        return 0;
+    }
+    const float max_logit = sc.logit[0];
+    if (t < count) sc.w[t] = exp(static_cast<double>(__fsub_rn(sc.logit[t], max_logit)));
+    __syncthreads();
+    if (t == 0) {
+        double total = 0.0;
+        for (uint32_t i = 0; i < count; ++i) total += sc.w[i];
+        double retained = 0.0;
+        uint32_t kept = 0;
+        do {
+            retained += sc.w[kept++];
+        } while (kept < count && retained / total < static_cast<double>(opt.top_p));
+        uint32_t c = kept;
+        if (opt.min_p > 0.f) {
+            uint32_t m = 1;
+            while (m < c && sc.w[m] >= static_cast<double>(opt.min_p)) ++m;
+            c = m;
+        }
+        out.count = c;
+    }
+    __syncthreads();
+    count = out.count;
+    if (t < count)
+        out.weight[t] = exp(static_cast<double>(__fsub_rn(sc.logit[t], max_logit)) / static_cast<double>(opt.temperature));
+    __syncthreads();
+    if (t == 0) {
+        double norm = 0.0;
+        for (uint32_t i = 0; i < count; ++i) norm += out.weight[i];
+        out.total = norm;
+        sc.err = (!isfinite(norm) || norm <= 0.0) ? -7 : 0;
+    }
+    __syncthreads();
+    return sc.err;
+}
+
+// Neumaier-compensated total with the reference's consistency checks; one lane.
+__device__ double validated_total(const Prepared& p) {
+    if (p.count == 0 || p.count > kMaxTopK || !isfinite(p.total) || p.total <= 0.0) return -1.0;
+    double total = 0.0, correction = 0.0;
+    for (uint32_t i = 0; i < p.count; ++i) {
+        const double w = p.weight[i];
+        const double prob = w / p.total;  // the stored probability is exactly this quotient
+        if (!isfinite(prob) || prob < 0.0 || prob > 1.0 || !isfinite(w) || w < 0.0) return -1.0;
+        const double sum = total + w;
+        correction += total >= w ? (total - sum) + w : (w - sum) + total;
+        total = sum;
+    }
+    total += correction;
+    const double tol = static_cast<double>(p.count) * 2.220446049250313e-16 * total;
+    if (!isfinite(total) || total <= 0.0 || fabs(total - p.total) > tol) return -1.0;
+    return total;
+}
+
+__device__ uint32_t select_prepared(const Prepared& p, double draw) {
+    double cumulative = 0.0;
+    for (uint32_t i = 0; i < p.count; ++i) {
+        cumulative += p.weight[i];
+        if (draw < cumulative) return p.token[i];
+    }
+    return p.token[p.count - 1];
+}
+
+__device__ uint64_t law_mass(const DraftLaw* law, uint32_t token, uint64_t* begin) {
+    uint32_t lo = 0, hi = law->count;
+    while (lo < hi) {
+        const uint32_t mid = (lo + hi) >> 1;
+        if (law->ids[mid] < token) lo = mid + 1; else hi = mid;
+    }
+    if (lo == law->count || law->ids[lo] != token) { if (begin) *begin = 0; return 0; }
+    if (begin) *begin = law->cdf[lo];
+    return law->cdf[lo + 1] - law->cdf[lo];
+}
+
+__global__ void __launch_bounds__(512)
+spec_accept_kernel(const Candidates* __restrict__ rows, const DraftLaw* __restrict__ law,
+                   const uint32_t* __restrict__ proposal_ptr, SamplerOptions opt, uint64_t seed, uint64_t step,
+                   const StepDraws* __restrict__ injected, SpecResult* __restrict__ result,
+                   uint32_t* __restrict__ status) {
+    __shared__ Scratch sc;
+    __shared__ Prepared target, residual;
+    __shared__ uint64_t q[kMaxTopK];
+    __shared__ int s_code;
+    __shared__ uint32_t s_accepted;
+    const uint32_t t = threadIdx.x;
+    const uint32_t proposal = *proposal_ptr;
+    const StepDraws d = injected ? *injected : step_draws(seed, step);
+    if (t == 0) {
+        result->accepted = 0; result->token = 0xFFFFFFFFu; result->next_root = 0xFFFFFFFFu; result->status = 0;
+        result->acceptance_probability = 0.0; result->residual_total = 0.0; result->residual_count = 0;
+        result->proposal = proposal;
+    }
+    int rc = prepare_distribution(&rows[0], opt, nullptr, 0, sc, target);
+    if (!rc && t < target.count) q[t] = law_mass(law, target.token[t], nullptr);
+    __syncthreads();
+    if (t == 0) {
+        int code = rc;
+        auto unit = [](double u) { return isfinite(u) && u >= 0.0 && u < 1.0; };
+        if (!code && (!unit(d.u_accept) || !unit(d.u_residual) || !unit(d.u_next))) code = -20;
+        double normalization = 0.0;
+        if (!code) { normalization = validated_total(target); if (normalization < 0.0) code = -21; }
+        uint64_t begin = 0, proposal_mass = 0;
+        if (!code) {
+            proposal_mass = law_mass(law, proposal, &begin);
+            if (proposal_mass == 0 || proposal_mass > kMassTotal || begin > kMassTotal - proposal_mass) code = -22;
+        }
+        bool in_target = false;
+        if (!code) {
+            uint64_t gathered = 0;
+            for (uint32_t i = 0; i < target.count && !code; ++i) {
+                if (q[i] > kMassTotal - gathered) code = -23;
+                gathered += q[i];
+                if (target.token[i] == proposal) in_target = true;
+            }
+            if (!code && !in_target && proposal_mass > kMassTotal - gathered) code = -24;
+        }
+        uint32_t accepted = 0;
+        if (!code) {
+            const double proposed = static_cast<double>(proposal_mass) / static_cast<double>(kMassTotal);
+            double acceptance = 0.0;
+            residual.count = 0; residual.total = 0.0;
+            for (uint32_t i = 0; i < target.count; ++i) {
+                const double p = target.weight[i] / normalization;
+                if (target.token[i] == proposal) acceptance = fmin(1.0, p / proposed);
+                const double diff = p - static_cast<double>(q[i]) / static_cast<double>(kMassTotal);
+                if (diff <= 0.0) continue;
+                residual.token[residual.count] = target.token[i];
+                residual.weight[residual.count] = diff;
+                ++residual.count;
+                residual.total += diff;
+            }
+            if (residual.count == 0 && acceptance < 1.0) code = -25;
+            result->acceptance_probability = acceptance;
+            result->residual_total = residual.total;
+            result->residual_count = residual.count;
+            if (!code) {
+                if (d.u_accept < acceptance) {
+                    accepted = 1;
+                    result->accepted = 1; result->token = proposal; result->next_root = proposal;
+                } else if (validated_total(residual) < 0.0) {
+                    code = -26;
+                } else {
+                    const uint32_t tok = select_prepared(residual, d.u_residual * residual.total);
+                    result->token = tok; result->next_root = tok;
+                }
+            }
+        }
+        s_code = code;
+        s_accepted = accepted;
+    }
+    __syncthreads();
+    if (s_code == 0 && s_accepted) {
+        // a fully accepted chain leaves row 1's candidates to seed the next root
+        rc = prepare_distribution(&rows[1], opt, nullptr, 0, sc, target);
+        if (t == 0) {
+            if (rc) s_code = rc - 100;
+            else result->next_root = opt.temperature == 0.f ? target.token[0]
+                                                             : select_prepared(target, d.u_next * target.total);
+        }
+    }
+    __syncthreads();
+    if (t == 0 && s_code != 0) {
+        result->status = static_cast<uint32_t>(-s_code);
+        result->token = 0xFFFFFFFFu; result->next_root = 0xFFFFFFFFu; result->accepted = 0;
+        if (status) atomicOr(status, GUFFIN_STATUS_LAW_INVALID);
+    }
+}
+
+}  // namespace
+
+int select_candidates_scaled(hipStream_t s, const float* logits, uint32_t rows, uint32_t vocab, uint32_t retain,
+                             float divisor, const uint32_t* history, const uint32_t* history_count,
+                             void* workspace, void* result, uint32_t* status);
+
+}  // namespace guffin
+
+using namespace guffin;
+
+extern "C" uint64_t guffin_hip_draft_law_workspace_bytes(uint32_t vocab) {
+    // survivors of the 257-best selection plus the sorted candidate row
+    const uint64_t tiles = (uint64_t(vocab) + 2047) / 2048;
+    return tiles * 257 * 8 + sizeof(Candidates) + 16;
+}
+
+extern "C" int guffin_hip_draft_law(void* stream, const float* logits, uint32_t vocab, const void* options,
+                                    uint64_t seed, uint64_t step, const void* injected_draws, void* workspace,
+                                    void* law, uint32_t* proposal, uint32_t* status) {
+    if (!logits || !options || !workspace || !law || !proposal || !status) return fail(GUFFIN_E_ARG, "draft_law: null pointer");
+    if (vocab < 1) return fail(GUFFIN_E_SHAPE, "draft_law: empty vocabulary");
+    if (reinterpret_cast<uintptr_t>(workspace) & 7u) return fail(GUFFIN_E_ALIGN, "draft_law: workspace must be 8-byte aligned");
+    const SamplerOptions opt = *static_cast<const SamplerOptions*>(options);
+    if (!(opt.temperature > 0.f) || opt.top_k == 0 || opt.top_k > 64)
+        return fail(GUFFIN_E_ARG, "draft_law: the compact law needs temperature > 0 and top_k in [1, 64]");
+    hipStream_t s = as_stream(stream);
+    const uint64_t tiles = (uint64_t(vocab) + 2047) / 2048;
+    uint8_t* ws = static_cast<uint8_t*>(workspace);
+    Candidates* top = reinterpret_cast<Candidates*>(ws + ((tiles * 257 * 8 + 15) & ~uint64_t{15}));
+    // the k-th best score and every tie with it: the best 257 scores decide both
+    if (int rc = select_candidates_scaled(s, logits, 1, vocab, vocab < 257 ? vocab : 257, opt.temperature, nullptr,
+                                          nullptr, ws, top, status))
+        return rc;
+    hipLaunchKernelGGL(draft_law_kernel, dim3(1), dim3(256), 0, s, top, opt, seed, step,
+                       static_cast<const StepDraws*>(injected_draws), static_cast<DraftLaw*>(law), proposal, status);
+    return check_launch("draft_law");
+}
+
+extern "C" int guffin_hip_spec_accept(void* stream, const void* target_candidates, const void* law,
+                                      const uint32_t* proposal, const void* options, uint64_t seed, uint64_t step,
+                                      const void* injected_draws, void* result, uint32_t* status) {
+    if (!target_candidates || !law || !proposal || !options || !result) return fail(GUFFIN_E_ARG, "spec_accept: null pointer");
+    const SamplerOptions opt = *static_cast<const SamplerOptions*>(options);
+    hipLaunchKernelGGL(spec_accept_kernel, dim3(1), dim3(512), 0, as_stream(stream),
+                       static_cast<const Candidates*>(target_candidates), static_cast<const DraftLaw*>(law), proposal,
+                       opt, seed, step, static_cast<const StepDraws*>(injected_draws),
+                       static_cast<SpecResult*>(result), status);
+    return check_launch("spec_accept");
+}
+
+extern "C" int guffin_hip_step_draws(uint64_t seed, uint64_t step, void* out_draws_host) {
+    // host restatement of the device draw schedule, for callers that log or inject draws
+    if (!out_draws_host) return fail(GUFFIN_E_ARG, "step_draws: null pointer");
+    auto round = [](uint32_t (&c)[4], uint32_t (&k)[2]) {
+        const uint64_t p0 = uint64_t{0xD2511F53u} * c[0], p1 = uint64_t{0xCD9E8D57u} * c[2];
+        const uint32_t n0 = static_cast<uint32_t>(p1 >> 32) ^ c[1] ^ k[0], n1 = static_cast<uint32_t>(p1);
+        const uint32_t n2 = static_cast<uint32_t>(p0 >> 32) ^ c[3] ^ k[1], n3 = static_cast<uint32_t>(p0);
+        c[0] = n0; c[1] = n1; c[2] = n2; c[3] = n3;
+        k[0] += 0x9E3779B9u; k[1] += 0xBB67AE85u;
+    };
+    StepDraws d {};
+    uint32_t out[2][4];
+    for (uint32_t block = 0; block < 2; ++block) {
+        uint32_t c[4] = {static_cast<uint32_t>(step), static_cast<uint32_t>(step >> 32), block, 0};
+        uint32_t k[2] = {static_cast<uint32_t>(seed), static_cast<uint32_t>(seed >> 32)};
+        for (int r = 0; r < 10; ++r) round(c, k);
+        for (int i = 0; i < 4; ++i) out[block][i] = c[i];
+    }
+    auto unit = [](uint32_t hi, uint32_t lo) { return static_cast<double>(((uint64_t{hi} << 32) | lo) >> 11) * 0x1.0p-53; };
+    d.word = out[0][0];
+    d.u_accept = unit(out[0][1], out[0][2]);
+    d.u_residual = unit(out[1][0], out[1][1]);
+    d.u_next = unit(out[1][2], out[1][3]);
+    *static_cast<StepDraws*>(out_draws_host) = d;
+    return GUFFIN_OK;
+}

@@ -227,3 +227,83 @@ def attention_decode(q, ring_k, ring_v, priv_k, priv_v, schedule, ancestors, max
                                             _p(part_ml), rows, priv_k.shape[0], max_tokens, ring_mask, q_heads,
                                             kv_heads, head_dim, C.c_float(scale), _p(status)))
     return (out, sums) if want_sums else out
+
+
+# ---- head selection, proposal law, acceptance ------------------------------------------
+import numpy as _np
+
+token_logit = _np.dtype([("token", _np.uint32), ("logit", _np.float32)])
+candidates_dtype = _np.dtype([("count", _np.uint32), ("status", _np.uint32), ("values", token_logit, (384,))])
+law_dtype = _np.dtype([("count", _np.uint32), ("pad", _np.uint32), ("ids", _np.uint32, (256,)),
+                       ("cdf", _np.uint64, (257,))])
+result_dtype = _np.dtype([("accepted", _np.uint32), ("token", _np.uint32), ("next_root", _np.uint32),
+                          ("status", _np.uint32), ("acceptance_probability", _np.float64),
+                          ("residual_total", _np.float64), ("residual_count", _np.uint32),
+                          ("proposal", _np.uint32)])
+draws_dtype = _np.dtype([("word", _np.uint32), ("pad", _np.uint32), ("u_accept", _np.float64),
+                         ("u_residual", _np.float64), ("u_next", _np.float64)])
+
+
+class SamplerOptions(C.Structure):
+    _fields_ = [("temperature", C.c_float), ("top_k", C.c_uint32), ("top_p", C.c_float),
+                ("min_p", C.c_float), ("repetition_penalty", C.c_float)]
+
+
+def _bytes(n, device="cuda"):
+    return torch.zeros(int(n), dtype=torch.uint8, device=device)
+
+
+def select_candidates(logits, retain, history=None, history_count=None, status=None, result=None):
+    rows, vocab = logits.shape
+    lib().guffin_hip_select_workspace_bytes.restype = C.c_uint64
+    ws = _bytes(lib().guffin_hip_select_workspace_bytes(rows, vocab, retain))
+    if result is None:
+        result = _bytes(rows * candidates_dtype.itemsize)
+    if status is None:
+        status = torch.zeros(rows, dtype=torch.int32, device=logits.device)
+    check(lib().guffin_hip_select_candidates(_stream(), _p(logits), rows, vocab, retain, _p(history),
+                                             _p(history_count), _p(ws), _p(result), _p(status)))
+    return result, status
+
+
+def candidates_to_numpy(result):
+    return result.cpu().numpy().view(candidates_dtype)
+
+
+def argmax(logits, status=None):
+    rows, vocab = logits.shape
+    ws = _bytes(rows * 256 * 8)
+    token = torch.zeros(rows, dtype=torch.int32, device=logits.device)
+    logit = torch.zeros(rows, dtype=torch.float32, device=logits.device)
+    check(lib().guffin_hip_argmax(_stream(), _p(logits), rows, vocab, _p(ws), _p(token), _p(logit), _p(status)))
+    return token, logit
+
+
+def draft_law(logits, options, seed=0, step=0, draws=None, law=None, proposal=None, status=None, workspace=None):
+    vocab = logits.numel()
+    lib().guffin_hip_draft_law_workspace_bytes.restype = C.c_uint64
+    if workspace is None:
+        workspace = _bytes(lib().guffin_hip_draft_law_workspace_bytes(vocab))
+    if law is None:
+        law = _bytes(law_dtype.itemsize)
+    if proposal is None:
+        proposal = torch.zeros(1, dtype=torch.int32, device=logits.device)
+    if status is None:
+        status = torch.zeros(1, dtype=torch.int32, device=logits.device)
+    check(lib().guffin_hip_draft_law(_stream(), _p(logits), vocab, C.byref(options), C.c_uint64(seed),
+                                     C.c_uint64(step), _p(draws), _p(workspace), _p(law), _p(proposal), _p(status)))
+    return law, proposal, status
+
+
+def spec_accept(cands, law, proposal, options, seed=0, step=0, draws=None, result=None, status=None):
+    if result is None:
+        result = _bytes(result_dtype.itemsize)
+    check(lib().guffin_hip_spec_accept(_stream(), _p(cands), _p(law), _p(proposal), C.byref(options),
+                                       C.c_uint64(seed), C.c_uint64(step), _p(draws), _p(result), _p(status)))
+    return result
+
+
+def step_draws(seed, step):
+    out = _np.zeros(1, draws_dtype)
+    check(lib().guffin_hip_step_draws(C.c_uint64(seed), C.c_uint64(step), out.ctypes.data_as(C.c_void_p)))
+    return out[0]

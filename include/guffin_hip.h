@@ -172,6 +172,56 @@ int guffin_hip_attention_decode(void* stream, const float* q, const void* ring_k
                                 uint32_t q_heads, uint32_t kv_heads, uint32_t head_dim, float scale,
                                 uint32_t* status);
 
+/* ---- output-head selection ---------------------------------------------------------------
+ * Per row the best `retain` (= top_k + history count, the reference's base_candidate_count)
+ * logits by (logit desc, token asc), then the logits of the row's history tokens.  Replaces
+ * encode_token_candidates[_width_two] / encode_target_token_candidates (:326-345) and
+ * read_token_candidates; order src/engine/sampling.cpp:25-30.
+ * result: per row { u32 count; u32 status; {u32 token; f32 logit} values[384]; }
+ * (CompactTokenCandidates, include/local_gguf_engine/engine/sampling.hpp:57-61, plus the status).
+ * history: [rows][64] token ids with history_count[rows] (both NULL for none).
+ * status: one u32 per row; GUFFIN_STATUS_NONFINITE if the row holds a non-finite logit,
+ * GUFFIN_STATUS_BAD_TOKEN for a history token outside the vocabulary. */
+uint64_t guffin_hip_select_workspace_bytes(uint32_t rows, uint32_t vocab, uint32_t retain);
+int guffin_hip_select_candidates(void* stream, const float* logits, uint32_t rows, uint32_t vocab,
+                                 uint32_t retain, const uint32_t* history, const uint32_t* history_count,
+                                 void* workspace, void* result, uint32_t* status);
+/* Greedy token per row, strict '>' so the lowest id wins ties (src/tensor/ops/reduction.cpp:93-117).
+ * workspace: rows * 256 * 8 bytes.  logit may be NULL. */
+int guffin_hip_argmax(void* stream, const float* logits, uint32_t rows, uint32_t vocab, void* workspace,
+                      uint32_t* token, float* logit, uint32_t* status);
+
+/* ---- proposal law and lossless acceptance ---------------------------------------------------
+ * options: { f32 temperature; u32 top_k; f32 top_p; f32 min_p; f32 repetition_penalty; }
+ * draws:   { u32 word; u32 pad; f64 u_accept; f64 u_residual; f64 u_next; } — when the injected
+ *          pointer is NULL the kernels derive them from Philox4x32-10 with key = seed and
+ *          counters (step, 0) -> {word, u_accept}, (step, 1) -> {u_residual, u_next}, 53-bit
+ *          uniforms in [0,1).  The reference draws from mt19937_64 streams
+ *          (src/engine/sampling.cpp:45-60); the consumption pattern is kept (:896-934).
+ *
+ * guffin_hip_draft_law builds the drafter's compact proposal law from full-vocabulary logits:
+ * score = logit / T, support = every token scoring >= the top_k-th best (<= 256 entries, else
+ * status bit 32 is raised), descending-tail top-p / min-p, f32 prefix / total * 2^32 -> u64 bins
+ * in ascending token id (src/engine/gemma3_draft.mm:191-294), and selects the proposal with
+ * the step's 32-bit word.  law: { u32 count; u32 pad; u32 ids[256]; u64 cdf[257]; }. */
+uint64_t guffin_hip_draft_law_workspace_bytes(uint32_t vocab);
+int guffin_hip_draft_law(void* stream, const float* logits, uint32_t vocab, const void* options,
+                         uint64_t seed, uint64_t step, const void* injected_draws, void* workspace,
+                         void* law, uint32_t* proposal, uint32_t* status);
+/* One accept / residual decision (src/engine/sampling.cpp:394-499, 561-656):
+ * target law p from row 0 of target_candidates (two rows of the select result), q gathered
+ * from `law` on p's support, accept iff u_accept < min(1, p(x)/q(x)), else inverse-CDF draw
+ * from norm(max(p-q, 0)) with u_residual; on acceptance the next root is drawn from row 1's
+ * law with u_next (src/engine/chain_chat.mm:524-533).
+ * result: { u32 accepted, token, next_root, status; f64 acceptance_probability,
+ *           residual_total; u32 residual_count, proposal; }; status != 0 mirrors the reference's
+ * throws and also sets GUFFIN_STATUS_LAW_INVALID in *status. */
+int guffin_hip_spec_accept(void* stream, const void* target_candidates, const void* law,
+                           const uint32_t* proposal, const void* options, uint64_t seed, uint64_t step,
+                           const void* injected_draws, void* result, uint32_t* status);
+/* Host evaluation of the draw schedule above (out: the draws struct). */
+int guffin_hip_step_draws(uint64_t seed, uint64_t step, void* out_draws_host);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,218 @@
+"""GPU parity of head selection, the proposal law and lossless acceptance.
+
+Bars: candidate lists, argmax ids, integer CDF bins, proposals and accept / residual /
+next-root decisions bit-exact against the CPU oracle given the same logits and draws.
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+TOTAL = 1 << 32
+VOCAB = 262144
+
+
+@pytest.fixture(scope="module")
+def hip():
+    from guffin_amd import hip as module
+    module.init(0)
+    return module
+
+
+def dev(a):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def opts(mod, t=1.0, k=64, p=0.95, m=0.0, r=1.0):
+    return mod.SamplerOptions(t, k, p, m, r)
+
+
+def test_step_draws_match_oracle_schedule(hip, gfo):
+    for seed, step in ((0, 0), (7, 5), (2 ** 40 + 3, 2 ** 33 + 9)):
+        d = hip.step_draws(seed, step)
+        w, a, r, n = gfo.step_draws(seed, step)
+        assert (int(d["word"]), float(d["u_accept"]), float(d["u_residual"]), float(d["u_next"])) == (w, a, r, n)
+
+
+def test_selection_reference_tie_and_history_case(hip):
+    logits = np.full((1, 1025), -2.0, np.float32)
+    logits[0, 1000] = logits[0, 1001] = 101.0
+    logits[0, 1010] = 100.0
+    logits[0, 7] = -99.75
+    hist = np.zeros((1, 64), np.uint32)
+    hist[0, 0] = 7
+    res, status = hip.select_candidates(dev(logits), 3, dev(hist), dev(np.array([1], np.uint32)))
+    c = hip.candidates_to_numpy(res)[0]
+    assert c["count"] == 4 and int(status[0]) == 0
+    assert list(c["values"]["token"][:4]) == [1000, 1001, 1010, 7]
+    assert list(c["values"]["logit"][:4]) == [101.0, 101.0, 100.0, -99.75]
+    tok, lg = hip.argmax(dev(logits))
+    assert int(tok[0]) == 1000 and float(lg[0]) == 101.0
+
+
+@pytest.mark.parametrize("retain", [1, 64, 257, 320])
+def test_selection_matches_oracle_on_full_vocabulary(hip, gfo, retain):
+    rng = np.random.default_rng(retain)
+    logits = rng.normal(0, 3, (2, VOCAB)).astype(np.float32)
+    logits[0, rng.integers(0, VOCAB, 4000)] = logits[0, 12345]      # many exact ties
+    logits[1, :500] = logits[1].max() + 1.0                          # a tie plateau at the top
+    res, status = hip.select_candidates(dev(logits), retain)
+    c = hip.candidates_to_numpy(res)
+    for row in range(2):
+        want = gfo.select_candidates(logits[row], retain)
+        assert c[row]["count"] == retain
+        assert np.array_equal(c[row]["values"]["token"][:retain], want["token"])
+        assert np.array_equal(c[row]["values"]["logit"][:retain].view(np.uint32), want["logit"].view(np.uint32))
+    tok, _ = hip.argmax(dev(logits))
+    assert [int(t) for t in tok] == [gfo.lib().gfo_argmax(logits[r].ctypes, VOCAB) for r in range(2)]
+
+
+def test_selection_flags_non_finite_logits(hip):
+    logits = np.zeros((2, 4096), np.float32)
+    logits[1, 77] = np.inf
+    _, status = hip.select_candidates(dev(logits), 8)
+    assert int(status[0]) == 0 and int(status[1]) & 2
+
+
+def law_np(hip, law):
+    return law.cpu().numpy().view(hip.law_dtype)[0]
+
+
+def check_law(hip, gfo, logits, o_gpu, o_cpu, word):
+    import torch
+    draws = np.zeros(1, hip.draws_dtype)
+    draws["word"] = word
+    draws["u_accept"], draws["u_residual"], draws["u_next"] = 0.5, 0.5, 0.5
+    law, proposal, status = hip.draft_law(dev(logits), o_gpu, draws=dev(draws.view(np.uint8)))
+    rc, want = gfo.draft_law_compact(logits, o_cpu)
+    if rc != 0:
+        assert int(status[0]) & 16
+        return None
+    got = law_np(hip, law)
+    assert int(status[0]) == 0
+    assert got["count"] == want.count
+    assert list(got["ids"][:want.count]) == [want.ids[i] for i in range(want.count)]
+    assert list(got["cdf"][:want.count + 1]) == [want.cdf[i] for i in range(want.count + 1)]
+    assert int(proposal[0]) & 0xFFFFFFFF == gfo.lib().gfo_draft_select(C.byref(want), C.c_uint32(word))
+    return got
+
+
+def test_draft_law_bit_exact_against_oracle(hip, gfo):
+    rng = np.random.default_rng(5)
+    for trial in range(12):
+        logits = rng.normal(0, 2, VOCAB).astype(np.float32)
+        k = int(rng.choice([1, 8, 40, 64]))
+        t = float(rng.choice([0.7, 1.0, 1.3]))
+        p = float(rng.choice([0.5, 0.9, 0.95, 1.0]))
+        m = float(rng.choice([0.0, 0.05]))
+        got = check_law(hip, gfo, logits, opts(hip, t, k, p, m), opts(gfo, t, k, p, m),
+                        int(rng.integers(0, 2 ** 32)))
+        assert got is not None and int(got["cdf"][got["count"]]) == TOTAL
+
+
+def test_draft_law_reference_fixtures(hip, gfo):
+    # tests/engine/gemma3_draft_tests.cpp:332-362 (48 candidates in different tiles, cutoff ties)
+    logits = np.full(VOCAB, -100.0, np.float32)
+    for i in range(48):
+        logits[37 + i * 4099] = 4.0 - i * 0.07 if i < 38 else 1.34
+    got = check_law(hip, gfo, logits, opts(hip, 1.0, 40, 0.87, 0.05), opts(gfo, 1.0, 40, 0.87, 0.05), 123456789)
+    assert got is not None
+    # :366-375 cutoff ties: 256 stay compact, 257 overflow, 64 compact
+    for count in (256, 257, 64):
+        logits = np.full(VOCAB, -100.0, np.float32)
+        logits[:count] = 0.0
+        got = check_law(hip, gfo, logits, opts(hip, 1.0, 1, 1.0, 0.0), opts(gfo, 1.0, 1, 1.0, 0.0), 0xFFFFFFFF)
+        if count == 257:
+            assert got is None
+        else:
+            mass = int(got["cdf"][count]) - int(got["cdf"][count - 1])
+            assert abs(mass / TOTAL - 1.0 / count) < 1e-6
+    bad = np.zeros(VOCAB, np.float32)
+    bad[5] = np.nan
+    _, _, status = hip.draft_law(dev(bad), opts(hip, 1.0, 4, 1.0, 0.0))
+    assert int(status[0]) & 16
+
+
+def run_steps(hip, gfo, p_logits, q_logits, steps, seed, o_gpu, o_cpu):
+    """steps of draft-law + accept on the GPU against the oracle; returns (accepted, rejected)."""
+    import torch
+    sets = p_logits.shape[0]
+    cands, laws_cpu, cands_cpu = [], [], []
+    for s in range(sets):
+        res, status = hip.select_candidates(dev(p_logits[s]), o_gpu.top_k)
+        assert int(status.abs().sum()) == 0
+        cands.append(res)
+        rc, law = gfo.draft_law_compact(q_logits[s], o_cpu)
+        assert rc == 0
+        laws_cpu.append(law)
+        c = hip.candidates_to_numpy(res)
+        for row in range(2):   # the GPU's selection equals the oracle's on the same logits
+            want = gfo.select_candidates(p_logits[s, row], o_gpu.top_k)
+            assert np.array_equal(c[row]["values"]["token"][:want.size], want["token"])
+        cands_cpu.append([gfo.select_candidates(p_logits[s, r], o_gpu.top_k) for r in range(2)])
+    q_dev = [dev(q_logits[s]) for s in range(sets)]
+    results = torch.zeros(steps * hip.result_dtype.itemsize, dtype=torch.uint8, device="cuda")
+    law = torch.zeros(hip.law_dtype.itemsize, dtype=torch.uint8, device="cuda")
+    proposal = torch.zeros(1, dtype=torch.int32, device="cuda")
+    status = torch.zeros(1, dtype=torch.int32, device="cuda")
+    lib = hip.lib()
+    lib.guffin_hip_draft_law_workspace_bytes.restype = C.c_uint64
+    ws = torch.zeros(lib.guffin_hip_draft_law_workspace_bytes(VOCAB), dtype=torch.uint8, device="cuda")
+    size = hip.result_dtype.itemsize
+    for step in range(steps):
+        s = step % sets
+        hip.draft_law(q_dev[s], o_gpu, seed=seed, step=step, law=law, proposal=proposal, status=status, workspace=ws)
+        hip.spec_accept(cands[s], law, proposal, o_gpu, seed=seed, step=step,
+                        result=results[step * size:(step + 1) * size], status=status)
+    got = results.cpu().numpy().view(hip.result_dtype)
+    assert int(status[0]) == 0
+    accepted = rejected = 0
+    for step in range(steps):
+        s = step % sets
+        word, ua, ur, un = gfo.step_draws(seed, step)
+        prop = gfo.lib().gfo_draft_select(C.byref(laws_cpu[s]), C.c_uint32(word))
+        rc, want = gfo.spec_accept(cands_cpu[s][0], cands_cpu[s][1], laws_cpu[s], prop, o_cpu, ua, ur, un)
+        assert rc == 0 and got[step]["status"] == 0, (step, rc, got[step]["status"])
+        assert got[step]["proposal"] == prop
+        assert (got[step]["accepted"], got[step]["token"], got[step]["next_root"]) == \
+            (want.accepted, want.token, want.next_root), step
+        assert got[step]["residual_count"] == want.residual_count
+        # the laws' doubles agree to a few ulp (device exp vs libm exp); decisions are exact
+        assert abs(got[step]["acceptance_probability"] - want.acceptance_probability) <= 1e-14
+        accepted += want.accepted
+        rejected += 1 - want.accepted
+    return accepted, rejected
+
+
+def test_ten_thousand_seeded_steps_bit_exact(hip, gfo):
+    """Config 3: T=1, top-k 64, top-p 0.95, drafter logits N(0,4) independent of the target."""
+    rng = np.random.default_rng(2024)
+    sets = 8
+    p_logits = rng.normal(0, 3, (sets, 2, VOCAB)).astype(np.float32)
+    q_logits = rng.normal(0, 2, (sets, VOCAB)).astype(np.float32)
+    a, r = run_steps(hip, gfo, p_logits, q_logits, 10000, 0, opts(hip), opts(gfo))
+    assert a + r == 10000
+
+
+def test_correlated_drafter_mixes_accepts_and_rejections(hip, gfo):
+    rng = np.random.default_rng(99)
+    sets = 8
+    p_logits = rng.normal(0, 3, (sets, 2, VOCAB)).astype(np.float32)
+    q_logits = (p_logits[:, 0] + rng.normal(0, 1.0, (sets, VOCAB))).astype(np.float32)
+    a, r = run_steps(hip, gfo, p_logits, q_logits, 3000, 17, opts(hip), opts(gfo))
+    assert a > 300 and r > 300, (a, r)
+    a2, r2 = run_steps(hip, gfo, p_logits, q_logits, 500, 18, opts(hip, 0.8, 40, 0.9, 0.05), opts(gfo, 0.8, 40, 0.9, 0.05))
+    assert a2 + r2 == 500
+
+
+def test_spec_accept_fails_closed(hip, gfo):
+    import torch
+    rng = np.random.default_rng(3)
+    p = rng.normal(0, 3, (2, 4096)).astype(np.float32)
+    res, _ = hip.select_candidates(dev(p), 64)
+    law, proposal, status = hip.draft_law(dev(rng.normal(0, 2, 4096).astype(np.float32)), opts(hip))
+    bad_prop = torch.full((1,), 5000, dtype=torch.int32, device="cuda")   # not in q's support
+    out = hip.spec_accept(res, law, bad_prop, opts(hip), status=status).cpu().numpy().view(hip.result_dtype)[0]
+    assert out["status"] == 22 and int(status[0]) & 16
