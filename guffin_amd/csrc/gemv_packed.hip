@@ -279,11 +279,12 @@ __device__ __forceinline__ void compute_tile(const Q8Tile& t, const float* __res
 // The streaming kernel: one wave = one (column tile, k-slice)
 // =======================================================================================
 template <int DTYPE, int R>
-__global__ void __launch_bounds__(64)
-gemv_packed_kernel(const uint8_t* __restrict__ wt, const float* __restrict__ x, const float* __restrict__ xsums,
-                   float* __restrict__ part, uint32_t K, uint32_t N, uint32_t nblk, uint32_t bps) {
+__device__ __forceinline__ void run_tile_slice(const uint8_t* __restrict__ wt, const float* __restrict__ x,
+                                               const float* __restrict__ xsums, float* __restrict__ part,
+                                               uint32_t K, uint32_t N, uint32_t nblk, uint32_t bps,
+                                               uint32_t ct, uint32_t slice) {
     constexpr uint32_t TB = kTileCols * block_bytes(DTYPE), BE = block_elems(DTYPE);
-    const uint32_t lane = threadIdx.x, ct = blockIdx.x, slice = blockIdx.y;
+    const uint32_t lane = threadIdx.x;
     const uint32_t b0 = slice * bps, b1 = b0 + bps < nblk ? b0 + bps : nblk;
     const uint32_t n16 = K / 16, per_row = n16 + K / 32;
     // Q6_K consumes 16-sums (16 per block), Q4_K 32-sums (8 per block), Q8_0 one 32-sum per block
@@ -321,6 +322,33 @@ gemv_packed_kernel(const uint8_t* __restrict__ wt, const float* __restrict__ x, 
     }
 #pragma unroll
     for (int r = 0; r < R; ++r) part[(size_t(slice) * R + r) * N + ct * kTileCols + lane] = acc[r];
+}
+
+template <int DTYPE, int R>
+__global__ void __launch_bounds__(64)
+gemv_packed_kernel(const uint8_t* __restrict__ wt, const float* __restrict__ x, const float* __restrict__ xsums,
+                   float* __restrict__ part, uint32_t K, uint32_t N, uint32_t nblk, uint32_t bps) {
+    run_tile_slice<DTYPE, R>(wt, x, xsums, part, K, N, nblk, bps, blockIdx.x, blockIdx.y);
+}
+
+// Several matrices that share the activation rows (q/k/v, gate/up) in one launch: the
+// column tiles of all matrices are laid side by side along grid x.
+struct PackedMat { const uint8_t* tiles; float* part; uint32_t N, dtype, S, bps, tile_end; };
+struct MultiArgs { PackedMat m[3]; const float* x; const float* xsums; uint32_t K, count; };
+
+template <int R>
+__global__ void __launch_bounds__(64) gemv_packed_multi_kernel(MultiArgs a) {
+    uint32_t which = 0, first = 0;
+    while (which + 1 < a.count && blockIdx.x >= a.m[which].tile_end) { first = a.m[which].tile_end; ++which; }
+    const PackedMat& m = a.m[which];
+    if (blockIdx.y >= m.S) return;
+    const uint32_t ct = blockIdx.x - first;
+    if (m.dtype == GUFFIN_Q4_K)
+        run_tile_slice<GUFFIN_Q4_K, R>(m.tiles, a.x, a.xsums, m.part, a.K, m.N, a.K / 256, m.bps, ct, blockIdx.y);
+    else if (m.dtype == GUFFIN_Q6_K)
+        run_tile_slice<GUFFIN_Q6_K, R>(m.tiles, a.x, a.xsums, m.part, a.K, m.N, a.K / 256, m.bps, ct, blockIdx.y);
+    else
+        run_tile_slice<GUFFIN_Q8_0, R>(m.tiles, a.x, a.xsums, m.part, a.K, m.N, a.K / 32, m.bps, ct, blockIdx.y);
 }
 
 int g_cus = 256;
@@ -410,6 +438,31 @@ extern "C" int guffin_hip_group_sums(void* stream, const float* x, float* xsums,
 extern "C" uint32_t guffin_hip_gemv_packed_slices(int dtype, uint32_t K, uint32_t N) {
     if (check_packed_shape("gemv_packed_slices: need K % block == 0 and N % 64 == 0", dtype, K, N)) return 0;
     return choose_slices(dtype, K, N);
+}
+
+extern "C" int guffin_hip_gemv_packed_multi(void* stream, uint32_t count, const int* dtypes, const void* const* tiles,
+                                            const uint32_t* N, float* const* partials, const float* x,
+                                            const float* xsums, uint32_t rows, uint32_t K) {
+    if (!dtypes || !tiles || !N || !partials || !x || !xsums) return fail(GUFFIN_E_ARG, "gemv_packed_multi: null pointer");
+    if (count == 0 || count > 3) return fail(GUFFIN_E_SHAPE, "gemv_packed_multi: 1 to 3 matrices");
+    if (rows == 0 || rows > 2) return fail(GUFFIN_E_SHAPE, "gemv_packed_multi: rows must be 1 or 2");
+    MultiArgs a {};
+    a.x = x; a.xsums = xsums; a.K = K; a.count = count;
+    uint32_t tile_end = 0, max_s = 1;
+    for (uint32_t i = 0; i < count; ++i) {
+        if (!tiles[i] || !partials[i]) return fail(GUFFIN_E_ARG, "gemv_packed_multi: null pointer");
+        if (int rc = check_packed_shape("gemv_packed_multi: need K % block == 0 and N % 64 == 0", dtypes[i], K, N[i])) return rc;
+        if (reinterpret_cast<uintptr_t>(tiles[i]) & 15u) return fail(GUFFIN_E_ALIGN, "gemv_packed_multi: tiles must be 16-byte aligned");
+        const uint32_t S = choose_slices(dtypes[i], K, N[i]), nblk = K / block_elems(dtypes[i]);
+        tile_end += N[i] / kTileCols;
+        a.m[i] = PackedMat {static_cast<const uint8_t*>(tiles[i]), partials[i], N[i], static_cast<uint32_t>(dtypes[i]),
+                            S, (nblk + S - 1) / S, tile_end};
+        if (S > max_s) max_s = S;
+    }
+    const dim3 grid(tile_end, max_s);
+    if (rows == 2) hipLaunchKernelGGL(gemv_packed_multi_kernel<2>, grid, dim3(64), 0, as_stream(stream), a);
+    else hipLaunchKernelGGL(gemv_packed_multi_kernel<1>, grid, dim3(64), 0, as_stream(stream), a);
+    return check_launch("gemv_packed_multi");
 }
 
 extern "C" int guffin_hip_gemv_packed(void* stream, int dtype, const void* tiles, const float* x, const float* xsums,

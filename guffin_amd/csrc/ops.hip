@@ -161,7 +161,7 @@ __device__ __forceinline__ void rope_sincos(uint32_t position, uint32_t pair, ui
 // Inputs may be `planes` partial planes of a GEMV.
 struct QkvArgs {
     const float* q_raw; const float* k_raw; const float* v_raw;
-    uint32_t planes; size_t q_plane_stride, k_plane_stride, v_plane_stride;
+    uint32_t q_planes, k_planes, v_planes; size_t q_plane_stride, k_plane_stride, v_plane_stride;
     const float* q_norm; const float* k_norm;
     const uint32_t* positions;
     float* q_out; uint16_t* k_out; uint16_t* v_out;
@@ -180,10 +180,11 @@ __global__ void __launch_bounds__(64) qkv_post_kernel(QkvArgs a) {
     const float* src = is_q ? a.q_raw : is_k ? a.k_raw : a.v_raw;
     if (!src) return;
     const size_t stride = is_q ? a.q_plane_stride : is_k ? a.k_plane_stride : a.v_plane_stride;
+    const uint32_t planes = is_q ? a.q_planes : is_k ? a.k_planes : a.v_planes;
     const size_t off = (size_t(r) * heads + hh) * a.head_dim;
     float ss = 0.f;
     for (uint32_t c = lane; c < a.head_dim; c += 64) {
-        const float v = load_planes(src + off + c, a.planes, stride);
+        const float v = load_planes(src + off + c, planes, stride);
         lds[c] = v;
         ss = fmaf(v, v, ss);
     }
@@ -408,7 +409,7 @@ extern "C" int guffin_hip_rope_neox(void* stream, const float* in, const uint32_
                                     float freq_base, float freq_scale) {
     if (!in || !out) return fail(GUFFIN_E_ARG, "rope_neox: null pointer");
     QkvArgs a {};
-    a.q_raw = in; a.planes = 1; a.positions = positions; a.q_out = out;
+    a.q_raw = in; a.q_planes = 1; a.positions = positions; a.q_out = out;
     a.rows = rows; a.q_heads = heads; a.kv_heads = 0; a.head_dim = head_dim; a.rope_dim = rope_dim;
     a.base = freq_base; a.scale = freq_scale; a.eps = 1e-6f;
     return launch_qkv(stream, a);
@@ -419,7 +420,7 @@ extern "C" int guffin_hip_kv_store_f16(void* stream, const float* raw_k, const f
                                        uint32_t rope_dim, float freq_base, float freq_scale, uint32_t* status) {
     if (!raw_k || !raw_v || !out_k || !out_v) return fail(GUFFIN_E_ARG, "kv_store_f16: null pointer");
     QkvArgs a {};
-    a.k_raw = raw_k; a.v_raw = raw_v; a.planes = 1; a.positions = positions;
+    a.k_raw = raw_k; a.v_raw = raw_v; a.k_planes = a.v_planes = 1; a.positions = positions;
     a.k_out = static_cast<uint16_t*>(out_k); a.v_out = static_cast<uint16_t*>(out_v);
     a.rows = rows; a.q_heads = 0; a.kv_heads = heads; a.head_dim = head_dim; a.rope_dim = rope_dim;
     a.base = freq_base; a.scale = freq_scale; a.eps = 1e-6f; a.status = status;
@@ -427,16 +428,17 @@ extern "C" int guffin_hip_kv_store_f16(void* stream, const float* raw_k, const f
 }
 
 extern "C" int guffin_hip_qkv_post(void* stream, const float* q_raw, const float* k_raw, const float* v_raw,
-                                   uint32_t planes, uint64_t q_plane_stride, uint64_t k_plane_stride,
+                                   uint32_t q_planes, uint32_t k_planes, uint32_t v_planes,
+                                   uint64_t q_plane_stride, uint64_t k_plane_stride,
                                    uint64_t v_plane_stride, const float* q_norm, const float* k_norm,
                                    const uint32_t* positions, float* q_out, void* k_out, void* v_out,
                                    uint32_t rows, uint32_t q_heads, uint32_t kv_heads, uint32_t head_dim,
                                    uint32_t rope_dim, float freq_base, float freq_scale, float eps, uint32_t* status) {
     if (!q_raw || !k_raw || !v_raw || !q_out || !k_out || !v_out) return fail(GUFFIN_E_ARG, "qkv_post: null pointer");
-    if (planes == 0) return fail(GUFFIN_E_SHAPE, "qkv_post: planes must be >= 1");
+    if (q_planes == 0 || k_planes == 0 || v_planes == 0) return fail(GUFFIN_E_SHAPE, "qkv_post: planes must be >= 1");
     if (!(eps > 0.f)) return fail(GUFFIN_E_ARG, "qkv_post: epsilon must be positive");
     QkvArgs a {};
-    a.q_raw = q_raw; a.k_raw = k_raw; a.v_raw = v_raw; a.planes = planes;
+    a.q_raw = q_raw; a.k_raw = k_raw; a.v_raw = v_raw; a.q_planes = q_planes; a.k_planes = k_planes; a.v_planes = v_planes;
     a.q_plane_stride = q_plane_stride; a.k_plane_stride = k_plane_stride; a.v_plane_stride = v_plane_stride;
     a.q_norm = q_norm; a.k_norm = k_norm; a.positions = positions;
     a.q_out = q_out; a.k_out = static_cast<uint16_t*>(k_out); a.v_out = static_cast<uint16_t*>(v_out);

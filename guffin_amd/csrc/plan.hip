@@ -1,0 +1,353 @@
+// Host side of the H1 step above the kernel C ABI: the Gemma-3 block graph for a few
+// contiguous rows, and one speculative cycle (draft 1 token, verify 2 rows, accept).
+//
+// Mirrors, in structure and operator order:
+//   encode_gemma_target_blocks            src/engine/gemma_target_runtime.cpp:13-221
+//   stage_contiguous_rows                 src/engine/gemma_target_runtime.cpp:238-271
+//   run_gemma_target_width_two_verifier   src/engine/gemma_target_runtime.cpp:457-519
+//   Gemma3DraftPlan forward / project     src/engine/gemma3_draft.mm:888-993
+//   one H1 cycle                          src/engine/standalone_chat.cpp:508-615,
+//                                         src/engine/chain_chat.mm:245-543
+// Like the reference's command context it allocates nothing: weights, KV rings and the
+// scratch arena are the caller's; everything is enqueued in order on one HIP stream, so a
+// caller can capture a whole step into a HIP graph.
+#include "common.hpp"
+
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+
+namespace guffin {
+namespace {
+
+struct Arena {
+    uint8_t* base; uint64_t used, capacity;
+    template <typename T> T* take(uint64_t count) {
+        used = (used + 255) & ~uint64_t{255};
+        T* p = base ? reinterpret_cast<T*>(base + used) : nullptr;
+        used += count * sizeof(T);
+        return p;
+    }
+};
+
+struct Scratch {
+    float *x, *x1, *u, *us, *q, *a, *as, *h, *hs;
+    float *part_a, *part_b, *part_c;          // GEMV partial planes (largest users: gate / up / down)
+    float *attn_out, *attn_ml;
+    uint32_t *positions, *ancestors, *schedule;
+    uint64_t bytes;
+};
+
+uint32_t slices(int dtype, uint32_t K, uint32_t N) { return guffin_hip_gemv_packed_slices(dtype, K, N); }
+uint64_t sums_len(uint32_t width) { return width / 16 + width / 32; }
+
+bool is_local(const guffin_model_desc& m, uint32_t layer) {
+    return m.global_period > 1 && (layer % m.global_period) != m.global_period - 1;
+}
+
+// longest token list an attention call of this model can see at `position` with `rows` rows
+uint32_t max_tokens_for(const guffin_model_desc& m, uint32_t layer, uint32_t position, uint32_t rows) {
+    if (is_local(m, layer)) {
+        const uint32_t w = m.sliding_window;
+        return (position < w ? position : w) + rows;
+    }
+    return position + rows;
+}
+
+Scratch layout(const guffin_model_desc& m, uint32_t rows, uint32_t position, uint8_t* base) {
+    Arena ar {base, 0, 0};
+    const uint32_t H = m.hidden, F = m.ffn, QW = m.q_heads * m.head_dim, KW = m.kv_heads * m.head_dim;
+    Scratch s {};
+    s.x = ar.take<float>(uint64_t(rows) * H);
+    s.x1 = ar.take<float>(uint64_t(rows) * H);
+    s.u = ar.take<float>(uint64_t(rows) * H);
+    s.us = ar.take<float>(rows * sums_len(H));
+    s.q = ar.take<float>(uint64_t(rows) * QW);
+    s.a = ar.take<float>(uint64_t(rows) * QW);
+    s.as = ar.take<float>(rows * sums_len(QW));
+    s.h = ar.take<float>(uint64_t(rows) * F);
+    s.hs = ar.take<float>(rows * sums_len(F));
+    // partial planes: a <- q / o / gate / down, b <- k / up, c <- v
+    uint64_t pa = 0, pb = 0, pc = 0;
+    for (uint32_t l = 0; l < m.layer_count; ++l) {
+        const guffin_layer_desc& L = m.layers[l];
+        auto need = [&](int i, uint32_t K, uint32_t N) { return uint64_t(slices(L.dtype[i], K, N)) * rows * N; };
+        pa = std::max({pa, need(0, H, QW), need(3, QW, H), need(4, H, F), need(6, F, H)});
+        pb = std::max({pb, need(1, H, KW), need(5, H, F)});
+        pc = std::max(pc, need(2, H, KW));
+    }
+    s.part_a = ar.take<float>(pa);
+    s.part_b = ar.take<float>(pb);
+    s.part_c = ar.take<float>(pc);
+    uint32_t max_parts = 1;
+    for (uint32_t l = 0; l < m.layer_count; ++l)
+        max_parts = std::max(max_parts, guffin_hip_attention_partitions(max_tokens_for(m, l, position, rows), m.kv_heads));
+    s.attn_out = ar.take<float>(uint64_t(rows) * m.q_heads * max_parts * m.head_dim);
+    s.attn_ml = ar.take<float>(uint64_t(rows) * m.q_heads * max_parts * 2);
+    s.positions = ar.take<uint32_t>(rows);
+    s.ancestors = ar.take<uint32_t>(rows);
+    s.schedule = ar.take<uint32_t>(uint64_t(m.layer_count) * rows * 4);
+    s.bytes = (ar.used + 255) & ~uint64_t{255};
+    return s;
+}
+
+// positions, ancestors and the per-layer attention schedule of `rows` contiguous rows
+__global__ void stage_rows_kernel(uint32_t* positions, uint32_t* ancestors, uint32_t* schedule, uint32_t rows,
+                                  uint32_t position, uint32_t layers, uint32_t window, uint32_t global_period) {
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < rows) { positions[i] = position + i; ancestors[i] = i; }
+    if (i >= layers * rows) return;
+    const uint32_t layer = i / rows, row = i % rows, p = position + row;
+    const bool local = global_period > 1 && (layer % global_period) != global_period - 1;
+    const uint32_t window_start = (local && p >= window) ? p + 1 - window : 0;
+    const uint32_t base_start = position < window_start ? position : window_start;
+    const uint32_t private_start = window_start > position ? window_start - position : 0;
+    uint32_t* s = schedule + 4 * i;
+    s[0] = base_start; s[1] = position - base_start; s[2] = private_start; s[3] = row + 1 - private_start;
+}
+
+int validate_model(const guffin_model_desc* m) {
+    if (!m || !m->layers || !m->embed_rows || !m->out_norm) return fail(GUFFIN_E_ARG, "forward: null model field");
+    if (m->head_dim != 256) return fail(GUFFIN_E_SHAPE, "forward: head_dim must be 256");
+    if (m->hidden % 64 || m->ffn % 64 || m->kv_heads == 0 || m->q_heads % m->kv_heads)
+        return fail(GUFFIN_E_SHAPE, "forward: widths must be multiples of 64 and q_heads a multiple of kv_heads");
+    if ((m->ring_local & (m->ring_local - 1)) || (m->ring_global & (m->ring_global - 1)) || !m->ring_local || !m->ring_global)
+        return fail(GUFFIN_E_ARG, "forward: ring capacities must be powers of two");
+    return GUFFIN_OK;
+}
+
+#define GUFFIN_TRY(expr) do { if (int rc_ = (expr)) return rc_; } while (0)
+
+int forward_rows(hipStream_t stream, const guffin_model_desc& m, const uint32_t* tokens, uint32_t rows,
+                 uint32_t position, const Scratch& s, void* priv_k, void* priv_v, float* out_hidden,
+                 float* out_hidden_sums, uint32_t* status) {
+    void* st = stream;
+    const uint32_t H = m.hidden, F = m.ffn, QW = m.q_heads * m.head_dim, KW = m.kv_heads * m.head_dim;
+    const float attn_scale = 1.0f / std::sqrt(static_cast<float>(m.head_dim));
+    const uint32_t n_sched = m.layer_count * rows;
+    hipLaunchKernelGGL(stage_rows_kernel, dim3((n_sched + 63) / 64), dim3(64), 0, stream, s.positions, s.ancestors,
+                       s.schedule, rows, position, m.layer_count, m.sliding_window, m.global_period);
+    GUFFIN_TRY(check_launch("stage_rows"));
+    GUFFIN_TRY(guffin_hip_embed(st, m.embed_dtype, m.embed_rows, tokens, s.x, rows, H,
+                                std::sqrt(static_cast<float>(H)), m.vocab, status));
+    GUFFIN_TRY(guffin_hip_rms_norm(st, s.x, 1, 0, m.layers[0].norm[0], nullptr, s.u, s.us, rows, H, m.eps, status));
+    for (uint32_t l = 0; l < m.layer_count; ++l) {
+        const guffin_layer_desc& L = m.layers[l];
+        const bool local = is_local(m, l);
+        const float base = local ? m.local_base : m.global_base, scale = local ? 1.0f : m.global_scale;
+        const uint32_t ring_mask = (local ? m.ring_local : m.ring_global) - 1;
+        uint16_t* pk = static_cast<uint16_t*>(priv_k) + size_t(l) * rows * KW;
+        uint16_t* pv = static_cast<uint16_t*>(priv_v) + size_t(l) * rows * KW;
+        {   // q, k, v projections of the normalised rows
+            const int dt[3] = {L.dtype[0], L.dtype[1], L.dtype[2]};
+            const void* tl[3] = {L.tiles[0], L.tiles[1], L.tiles[2]};
+            const uint32_t n[3] = {QW, KW, KW};
+            float* parts[3] = {s.part_a, s.part_b, s.part_c};
+            GUFFIN_TRY(guffin_hip_gemv_packed_multi(st, 3, dt, tl, n, parts, s.u, s.us, rows, H));
+            GUFFIN_TRY(guffin_hip_qkv_post(st, s.part_a, s.part_b, s.part_c, slices(dt[0], H, QW), slices(dt[1], H, KW),
+                                           slices(dt[2], H, KW), uint64_t(rows) * QW, uint64_t(rows) * KW,
+                                           uint64_t(rows) * KW, L.norm[1], L.norm[2], s.positions, s.q, pk, pv, rows,
+                                           m.q_heads, m.kv_heads, m.head_dim, m.head_dim, base, scale, m.eps, status));
+        }
+        GUFFIN_TRY(guffin_hip_attention_decode(st, s.q, L.ring_k, L.ring_v, pk, pv, s.schedule + size_t(l) * rows * 4,
+                                               s.ancestors, s.a, s.as, s.attn_out, s.attn_ml, rows, rows,
+                                               max_tokens_for(m, l, position, rows), ring_mask, m.q_heads, m.kv_heads,
+                                               m.head_dim, attn_scale, status));
+        GUFFIN_TRY(guffin_hip_gemv_packed(st, L.dtype[3], L.tiles[3], s.a, s.as, s.part_a, nullptr, rows, QW, H));
+        // x1 = x + rms(o, post_attention_norm); u = rms(x1, ffn_norm)
+        GUFFIN_TRY(guffin_hip_rms_norm_add_norm(st, s.part_a, slices(L.dtype[3], QW, H), uint64_t(rows) * H, L.norm[3],
+                                                s.x, s.x1, L.norm[4], s.u, s.us, rows, H, m.eps, status));
+        {
+            const int dt[2] = {L.dtype[4], L.dtype[5]};
+            const void* tl[2] = {L.tiles[4], L.tiles[5]};
+            const uint32_t n[2] = {F, F};
+            float* parts[2] = {s.part_a, s.part_b};
+            GUFFIN_TRY(guffin_hip_gemv_packed_multi(st, 2, dt, tl, n, parts, s.u, s.us, rows, H));
+            if (slices(dt[0], H, F) != slices(dt[1], H, F)) return fail(GUFFIN_E_SHAPE, "forward: gate and up must use the same block type");
+            GUFFIN_TRY(guffin_hip_geglu(st, s.part_a, s.part_b, slices(dt[0], H, F), uint64_t(rows) * F, s.h, s.hs, rows, F));
+        }
+        GUFFIN_TRY(guffin_hip_gemv_packed(st, L.dtype[6], L.tiles[6], s.h, s.hs, s.part_a, nullptr, rows, F, H));
+        // x = x1 + rms(down, post_ffw_norm); u = rms(x, next block's attn_norm | output_norm)
+        const bool last = l + 1 == m.layer_count;
+        const float* gamma_next = last ? m.out_norm : m.layers[l + 1].norm[0];
+        GUFFIN_TRY(guffin_hip_rms_norm_add_norm(st, s.part_a, slices(L.dtype[6], F, H), uint64_t(rows) * H, L.norm[5],
+                                                s.x1, s.x, gamma_next, last ? out_hidden : s.u,
+                                                last ? out_hidden_sums : s.us, rows, H, m.eps, status));
+    }
+    return GUFFIN_OK;
+}
+
+// publishes the verified rows: row 0 always, row 1 if the proposal was accepted
+__global__ void commit_rows_kernel(const uint16_t* priv_k, const uint16_t* priv_v, uint16_t* const* ring_k,
+                                   uint16_t* const* ring_v, const uint32_t* accepted, uint32_t position, uint32_t rows,
+                                   uint32_t row_width, uint32_t mask_local, uint32_t mask_global, uint32_t global_period) {
+    const uint32_t layer = blockIdx.y, row = blockIdx.z;
+    const uint32_t publish = accepted ? 1u + (*accepted != 0u) : rows;
+    if (row >= publish || row >= rows) return;
+    const bool local = global_period > 1 && (layer % global_period) != global_period - 1;
+    const uint32_t mask = local ? mask_local : mask_global;
+    const size_t src = (size_t(layer) * rows + row) * row_width, dst = size_t((position + row) & mask) * row_width;
+    for (uint32_t c = blockIdx.x * blockDim.x + threadIdx.x; c < row_width; c += gridDim.x * blockDim.x) {
+        ring_k[layer][dst + c] = priv_k[src + c];
+        ring_v[layer][dst + c] = priv_v[src + c];
+    }
+}
+
+__global__ void set_token_kernel(const uint32_t* src, uint32_t* dst) { *dst = *src; }
+
+}  // namespace
+}  // namespace guffin
+
+using namespace guffin;
+
+extern "C" uint64_t guffin_hip_forward_scratch_bytes(const guffin_model_desc* model, uint32_t rows, uint32_t position) {
+    if (validate_model(model) || rows == 0 || rows > 2) return 0;
+    return layout(*model, rows, position, nullptr).bytes;
+}
+
+extern "C" int guffin_hip_forward_rows(void* stream, const guffin_model_desc* model, const uint32_t* tokens,
+                                       uint32_t rows, uint32_t position, void* scratch, uint64_t scratch_bytes,
+                                       void* priv_k, void* priv_v, float* out_hidden, float* out_hidden_sums,
+                                       uint32_t* status) {
+    GUFFIN_TRY(validate_model(model));
+    if (!tokens || !scratch || !priv_k || !priv_v || !out_hidden || !status) return fail(GUFFIN_E_ARG, "forward_rows: null pointer");
+    if (rows == 0 || rows > 2) return fail(GUFFIN_E_SHAPE, "forward_rows: rows must be 1 or 2");
+    if (reinterpret_cast<uintptr_t>(scratch) & 255u) return fail(GUFFIN_E_ALIGN, "forward_rows: scratch must be 256-byte aligned");
+    const Scratch s = layout(*model, rows, position, static_cast<uint8_t*>(scratch));
+    if (s.bytes > scratch_bytes) return fail(GUFFIN_E_CAPACITY, "forward_rows: scratch arena too small");
+    return forward_rows(as_stream(stream), *model, tokens, rows, position, s, priv_k, priv_v, out_hidden,
+                        out_hidden_sums, status);
+}
+
+extern "C" int guffin_hip_commit_rows(void* stream, const guffin_model_desc* model, const void* priv_k,
+                                      const void* priv_v, void* const* ring_k_table, void* const* ring_v_table,
+                                      const uint32_t* accepted, uint32_t position, uint32_t rows) {
+    GUFFIN_TRY(validate_model(model));
+    if (!priv_k || !priv_v || !ring_k_table || !ring_v_table) return fail(GUFFIN_E_ARG, "commit_rows: null pointer");
+    if (rows == 0 || rows > 2) return fail(GUFFIN_E_SHAPE, "commit_rows: rows must be 1 or 2");
+    const uint32_t KW = model->kv_heads * model->head_dim;
+    hipLaunchKernelGGL(commit_rows_kernel, dim3((KW + 255) / 256, model->layer_count, rows), dim3(256), 0,
+                       as_stream(stream), static_cast<const uint16_t*>(priv_k), static_cast<const uint16_t*>(priv_v),
+                       reinterpret_cast<uint16_t* const*>(ring_k_table), reinterpret_cast<uint16_t* const*>(ring_v_table),
+                       accepted, position, rows, KW, model->ring_local - 1, model->ring_global - 1, model->global_period);
+    return check_launch("commit_rows");
+}
+
+// ---- one H1 cycle ---------------------------------------------------------------------
+extern "C" uint64_t guffin_hip_h1_scratch_bytes(const guffin_h1_desc* d) {
+    if (!d || validate_model(d->target) || validate_model(d->drafter)) return 0;
+    Arena ar {nullptr, 0, 0};
+    const uint64_t V = d->target->vocab;
+    ar.take<uint8_t>(guffin_hip_forward_scratch_bytes(d->drafter, 1, d->drafter_position));
+    ar.take<uint8_t>(guffin_hip_forward_scratch_bytes(d->target, 2, d->target_position));
+    ar.take<float>(d->drafter->hidden + sums_len(d->drafter->hidden));                 // drafter hidden + sums
+    ar.take<float>(2 * (d->target->hidden + sums_len(d->target->hidden)));             // target hidden + sums
+    ar.take<float>(uint64_t(slices(d->drafter->head_dtype, d->drafter->hidden, d->drafter->vocab)) * d->drafter->vocab);
+    ar.take<float>(d->drafter->vocab);                                                  // q logits
+    ar.take<float>(uint64_t(slices(d->target->head_dtype, d->target->hidden, V)) * 2 * V);
+    ar.take<float>(2 * V);                                                              // p logits
+    ar.take<uint8_t>(guffin_hip_draft_law_workspace_bytes(d->drafter->vocab));
+    ar.take<uint8_t>(guffin_hip_select_workspace_bytes(2, V, d->top_k));
+    ar.take<uint8_t>(4096 + 2 * 3088);                                                  // law, candidates
+    ar.take<uint32_t>(16);
+    return (ar.used + 255) & ~uint64_t{255};
+}
+
+extern "C" int guffin_hip_h1_step(void* stream, const guffin_h1_desc* d, const uint32_t* root_token, void* scratch,
+                                  uint64_t scratch_bytes, void* drafter_priv_k, void* drafter_priv_v,
+                                  void* target_priv_k, void* target_priv_v, void* result, uint32_t* status) {
+    if (!d || !root_token || !scratch || !result || !status) return fail(GUFFIN_E_ARG, "h1_step: null pointer");
+    GUFFIN_TRY(validate_model(d->target));
+    GUFFIN_TRY(validate_model(d->drafter));
+    if (!d->target->head_tiles || !d->drafter->head_tiles) return fail(GUFFIN_E_ARG, "h1_step: models need packed head weights");
+    if (d->drafter->vocab != d->target->vocab) return fail(GUFFIN_E_SHAPE, "h1_step: drafter and target vocabularies must coincide");
+    if (reinterpret_cast<uintptr_t>(scratch) & 255u) return fail(GUFFIN_E_ALIGN, "h1_step: scratch must be 256-byte aligned");
+    if (guffin_hip_h1_scratch_bytes(d) > scratch_bytes) return fail(GUFFIN_E_CAPACITY, "h1_step: scratch arena too small");
+    const guffin_model_desc& T = *d->target;
+    const guffin_model_desc& D = *d->drafter;
+    const uint64_t V = T.vocab;
+    Arena ar {static_cast<uint8_t*>(scratch), 0, scratch_bytes};
+    const uint64_t d_bytes = guffin_hip_forward_scratch_bytes(&D, 1, d->drafter_position);
+    const uint64_t t_bytes = guffin_hip_forward_scratch_bytes(&T, 2, d->target_position);
+    uint8_t* d_scratch = ar.take<uint8_t>(d_bytes);
+    uint8_t* t_scratch = ar.take<uint8_t>(t_bytes);
+    float* d_hidden = ar.take<float>(D.hidden + sums_len(D.hidden));
+    float* t_hidden = ar.take<float>(2 * (T.hidden + sums_len(T.hidden)));
+    float* q_parts = ar.take<float>(uint64_t(slices(D.head_dtype, D.hidden, D.vocab)) * D.vocab);
+    float* q_logits = ar.take<float>(D.vocab);
+    float* p_parts = ar.take<float>(uint64_t(slices(T.head_dtype, T.hidden, V)) * 2 * V);
+    float* p_logits = ar.take<float>(2 * V);
+    uint8_t* law_ws = ar.take<uint8_t>(guffin_hip_draft_law_workspace_bytes(D.vocab));
+    uint8_t* sel_ws = ar.take<uint8_t>(guffin_hip_select_workspace_bytes(2, V, d->top_k));
+    uint8_t* small = ar.take<uint8_t>(4096 + 2 * 3088);
+    uint32_t* words = ar.take<uint32_t>(16);
+    void* law = small;
+    void* cands = small + 4096;
+    uint32_t* tokens = words;          // [root, proposal]
+    uint32_t* sel_status = words + 4;  // per-row selection status
+    hipStream_t s = as_stream(stream);
+
+    struct { float temperature; uint32_t top_k; float top_p, min_p, repetition_penalty; } opt
+        = {d->temperature, d->top_k, d->top_p, d->min_p, 1.0f};
+
+    // 1. drafter: ingest the root, project, build the proposal law, pick x with the step's word
+    hipLaunchKernelGGL(set_token_kernel, dim3(1), dim3(1), 0, s, root_token, tokens);
+    GUFFIN_TRY(check_launch("set_token"));
+    GUFFIN_TRY(guffin_hip_forward_rows(stream, &D, tokens, 1, d->drafter_position, d_scratch, d_bytes, drafter_priv_k,
+                                       drafter_priv_v, d_hidden, d_hidden + D.hidden, status));
+    GUFFIN_TRY(guffin_hip_gemv_packed(stream, D.head_dtype, D.head_tiles, d_hidden, d_hidden + D.hidden, q_parts,
+                                      q_logits, 1, D.hidden, D.vocab));
+    GUFFIN_TRY(guffin_hip_draft_law(stream, q_logits, D.vocab, &opt, d->seed, d->step, nullptr, law_ws, law,
+                                    tokens + 1, status));
+    // 2. target: rows [root, x] together, head, candidates of both rows
+    GUFFIN_TRY(guffin_hip_forward_rows(stream, &T, tokens, 2, d->target_position, t_scratch, t_bytes, target_priv_k,
+                                       target_priv_v, t_hidden, t_hidden + 2 * T.hidden, status));
+    GUFFIN_TRY(guffin_hip_gemv_packed(stream, T.head_dtype, T.head_tiles, t_hidden, t_hidden + 2 * T.hidden, p_parts,
+                                      p_logits, 2, T.hidden, V));
+    GUFFIN_TRY(guffin_hip_select_candidates(stream, p_logits, 2, V, d->top_k, nullptr, nullptr, sel_ws, cands, sel_status));
+    // 3. accept x or draw from the residual; on acceptance draw the next root from row 1
+    GUFFIN_TRY(guffin_hip_spec_accept(stream, cands, law, tokens + 1, &opt, d->seed, d->step, nullptr, result, status));
+    // 4. publish: the target keeps row 0, and row 1 if x was accepted; the drafter keeps the root
+    if (d->target_ring_k && d->target_ring_v) {
+        GUFFIN_TRY(guffin_hip_commit_rows(stream, &T, target_priv_k, target_priv_v, d->target_ring_k, d->target_ring_v,
+                                          static_cast<const uint32_t*>(result), d->target_position, 2));
+    }
+    if (d->drafter_ring_k && d->drafter_ring_v) {
+        GUFFIN_TRY(guffin_hip_commit_rows(stream, &D, drafter_priv_k, drafter_priv_v, d->drafter_ring_k,
+                                          d->drafter_ring_v, nullptr, d->drafter_position, 1));
+    }
+    return GUFFIN_OK;
+}
+
+// debug / test access to the intermediate buffers of the last step laid out in `scratch`
+extern "C" int guffin_hip_h1_buffers(const guffin_h1_desc* d, void* scratch, float** drafter_hidden,
+                                     float** target_hidden, float** q_logits, float** p_logits, void** law,
+                                     void** candidates, uint32_t** tokens) {
+    if (!d || !scratch) return fail(GUFFIN_E_ARG, "h1_buffers: null pointer");
+    GUFFIN_TRY(validate_model(d->target));
+    GUFFIN_TRY(validate_model(d->drafter));
+    const guffin_model_desc& T = *d->target;
+    const guffin_model_desc& D = *d->drafter;
+    const uint64_t V = T.vocab;
+    Arena ar {static_cast<uint8_t*>(scratch), 0, 0};
+    ar.take<uint8_t>(guffin_hip_forward_scratch_bytes(&D, 1, d->drafter_position));
+    ar.take<uint8_t>(guffin_hip_forward_scratch_bytes(&T, 2, d->target_position));
+    float* dh = ar.take<float>(D.hidden + sums_len(D.hidden));
+    float* th = ar.take<float>(2 * (T.hidden + sums_len(T.hidden)));
+    ar.take<float>(uint64_t(slices(D.head_dtype, D.hidden, D.vocab)) * D.vocab);
+    float* ql = ar.take<float>(D.vocab);
+    ar.take<float>(uint64_t(slices(T.head_dtype, T.hidden, V)) * 2 * V);
+    float* pl = ar.take<float>(2 * V);
+    ar.take<uint8_t>(guffin_hip_draft_law_workspace_bytes(D.vocab));
+    ar.take<uint8_t>(guffin_hip_select_workspace_bytes(2, V, d->top_k));
+    uint8_t* small = ar.take<uint8_t>(4096 + 2 * 3088);
+    uint32_t* words = ar.take<uint32_t>(16);
+    if (drafter_hidden) *drafter_hidden = dh;
+    if (target_hidden) *target_hidden = th;
+    if (q_logits) *q_logits = ql;
+    if (p_logits) *p_logits = pl;
+    if (law) *law = small;
+    if (candidates) *candidates = small + 4096;
+    if (tokens) *tokens = words;
+    return GUFFIN_OK;
+}

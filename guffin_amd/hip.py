@@ -180,7 +180,7 @@ def qkv_post(q_raw, k_raw, v_raw, q_norm, k_norm, positions, rows, q_heads, kv_h
     q = _f32((rows, q_heads * head_dim), q_raw)
     k = torch.empty((rows, kv_heads * head_dim), dtype=torch.float16, device=q_raw.device)
     v = torch.empty_like(k)
-    check(lib().guffin_hip_qkv_post(_stream(), _p(q_raw), _p(k_raw), _p(v_raw), pl, C.c_uint64(strides[0]),
+    check(lib().guffin_hip_qkv_post(_stream(), _p(q_raw), _p(k_raw), _p(v_raw), pl, pl, pl, C.c_uint64(strides[0]),
                                     C.c_uint64(strides[1]), C.c_uint64(strides[2]), _p(q_norm), _p(k_norm),
                                     _p(positions), _p(q), _p(k), _p(v), rows, q_heads, kv_heads, head_dim,
                                     rope_dim, C.c_float(base), C.c_float(scale), C.c_float(eps), _p(status)))

@@ -1,0 +1,335 @@
+"""Synthetic Gemma-3 shaped models for the H1 step: descriptors, seeded weights, KV rings.
+
+Shapes follow BASELINE's configurations: the 12B target (48 blocks, hidden 3840, FFN 15360,
+16 query / 8 KV heads of 256, sliding window 1024 on 5 of every 6 blocks, Q4_K projections
+with Q6_K v_proj / down_proj and a tied Q6_K head) and the 270M drafter (18 blocks, hidden 640,
+FFN 2048, 4 query / 1 KV head, window 512, Q8_0 everywhere).  Layer policy and RoPE bases:
+reference src/engine/model.cpp:607-619, tests/support/gemma3_target_test_support.hpp:37-38.
+"""
+import ctypes as C
+from dataclasses import dataclass, field, replace
+
+import numpy as np
+import torch
+
+from . import hip, synth
+
+Q8_0, Q4_K, Q6_K = 0, 1, 2
+
+
+class LayerDesc(C.Structure):
+    _fields_ = [("dtype", C.c_int32 * 7), ("tiles", C.c_void_p * 7), ("norm", C.c_void_p * 6),
+                ("ring_k", C.c_void_p), ("ring_v", C.c_void_p)]
+
+
+class ModelDesc(C.Structure):
+    _fields_ = [(n, C.c_uint32) for n in ("hidden", "ffn", "q_heads", "kv_heads", "head_dim", "layer_count",
+                                           "vocab", "sliding_window", "global_period")] + \
+               [(n, C.c_float) for n in ("local_base", "global_base", "global_scale", "eps")] + \
+               [("ring_local", C.c_uint32), ("ring_global", C.c_uint32),
+                ("embed_dtype", C.c_int32), ("embed_rows", C.c_void_p),
+                ("head_dtype", C.c_int32), ("head_tiles", C.c_void_p),
+                ("out_norm", C.c_void_p), ("layers", C.POINTER(LayerDesc))]
+
+
+class H1Desc(C.Structure):
+    _fields_ = [("target", C.POINTER(ModelDesc)), ("drafter", C.POINTER(ModelDesc)),
+                ("target_position", C.c_uint32), ("drafter_position", C.c_uint32),
+                ("temperature", C.c_float), ("top_k", C.c_uint32), ("top_p", C.c_float), ("min_p", C.c_float),
+                ("seed", C.c_uint64), ("step", C.c_uint64),
+                ("target_ring_k", C.c_void_p), ("target_ring_v", C.c_void_p),
+                ("drafter_ring_k", C.c_void_p), ("drafter_ring_v", C.c_void_p)]
+
+
+@dataclass(frozen=True)
+class Shape:
+    hidden: int
+    ffn: int
+    q_heads: int
+    kv_heads: int
+    head_dim: int
+    layers: int
+    vocab: int
+    sliding_window: int
+    global_period: int
+    local_base: float
+    global_base: float
+    global_scale: float
+    ring_local: int
+    ring_global: int
+    dtypes: tuple = (Q4_K, Q4_K, Q6_K, Q4_K, Q4_K, Q4_K, Q6_K)   # q k v o gate up down
+    embed_dtype: int = Q6_K
+    eps: float = 1e-6
+
+    @property
+    def q_width(self):
+        return self.q_heads * self.head_dim
+
+    @property
+    def kv_width(self):
+        return self.kv_heads * self.head_dim
+
+    def is_local(self, layer):
+        return self.global_period > 1 and layer % self.global_period != self.global_period - 1
+
+    def proj_shapes(self):
+        """(K, N) of q, k, v, o, gate, up, down."""
+        H, F, QW, KW = self.hidden, self.ffn, self.q_width, self.kv_width
+        return [(H, QW), (H, KW), (H, KW), (QW, H), (H, F), (H, F), (F, H)]
+
+    def layer_weight_bytes(self):
+        return sum(synth.weight_bytes(d, K, N) for d, (K, N) in zip(self.dtypes, self.proj_shapes()))
+
+    def head_bytes(self):
+        return synth.weight_bytes(self.embed_dtype, self.hidden, self.vocab)
+
+
+GEMMA3_12B = Shape(3840, 15360, 16, 8, 256, 48, 262144, 1024, 6, 1e4, 1e6, 0.125, 1024, 8192)
+GEMMA3_270M = Shape(640, 2048, 4, 1, 256, 18, 262144, 512, 6, 1e4, 1e6, 1.0, 512, 8192,
+                    dtypes=(Q8_0,) * 7, embed_dtype=Q8_0)
+
+
+def tiny(shape, layers, vocab):
+    return replace(shape, layers=layers, vocab=vocab)
+
+
+class HostModel:
+    """Canonical-layout numpy weights (what the CPU oracle consumes)."""
+
+    def __init__(self, shape, seed, position, gamma_sigma=0.1):
+        self.shape = shape
+        rng = np.random.Generator(np.random.PCG64(seed))
+        self.w = []      # [layer][7] canonical uint8
+        self.norm = []   # [layer][6] float32
+        self.ring_k, self.ring_v = [], []
+        s = 1000 * seed
+        for l in range(shape.layers):
+            self.w.append([synth.make_weight(d, K, N, s + 16 * l + i)
+                           for i, (d, (K, N)) in enumerate(zip(shape.dtypes, shape.proj_shapes()))])
+            widths = [shape.hidden, shape.head_dim, shape.head_dim, shape.hidden, shape.hidden, shape.hidden]
+            self.norm.append([(1.0 + rng.normal(0, gamma_sigma, w)).astype(np.float32) for w in widths])
+            cap = shape.ring_local if shape.is_local(l) else shape.ring_global
+            k = np.zeros((cap, shape.kv_width), np.float16)
+            v = np.zeros((cap, shape.kv_width), np.float16)
+            filled = min(position, cap)
+            # positions position-filled .. position-1 live at slot p & (cap-1)
+            slots = (np.arange(position - filled, position) & (cap - 1))
+            k[slots] = rng.normal(0, 1, (filled, shape.kv_width)).astype(np.float16)
+            v[slots] = rng.normal(0, 1, (filled, shape.kv_width)).astype(np.float16)
+            self.ring_k.append(k)
+            self.ring_v.append(v)
+        self.embed = synth.make_weight(shape.embed_dtype, shape.hidden, shape.vocab, s + 999)
+        self.out_norm = (1.0 + rng.normal(0, gamma_sigma, shape.hidden)).astype(np.float32)
+
+    def oracle_config(self, gfo):
+        sh = self.shape
+        return gfo.ModelConfig(sh.hidden, sh.ffn, sh.q_heads, sh.kv_heads, sh.head_dim, sh.layers, sh.vocab,
+                               sh.sliding_window, sh.global_period, sh.local_base, sh.global_base,
+                               sh.global_scale, sh.eps, sh.ring_local, sh.ring_global)
+
+    def oracle_layers(self, gfo):
+        arr = (gfo.Layer * self.shape.layers)()
+        for l in range(self.shape.layers):
+            for i in range(7):
+                arr[l].dtype[i] = self.shape.dtypes[i]
+                arr[l].w[i] = self.w[l][i].ctypes.data
+            for i in range(6):
+                arr[l].norm[i] = self.norm[l][i].ctypes.data
+            arr[l].ring_k = self.ring_k[l].ctypes.data
+            arr[l].ring_v = self.ring_v[l].ctypes.data
+        return arr
+
+    def oracle_forward(self, gfo, tokens, position, threads=8):
+        sh = self.shape
+        rows = len(tokens)
+        tok = np.asarray(tokens, np.uint32)
+        pk = np.zeros((sh.layers, rows, sh.kv_width), np.uint16)
+        pv = np.zeros_like(pk)
+        out = np.zeros((rows, sh.hidden), np.float32)
+        cfg = self.oracle_config(gfo)
+        layers = self.oracle_layers(gfo)
+        gfo.lib().gfo_forward_rows(C.byref(cfg), layers, sh.embed_dtype, self.embed.ctypes.data_as(C.c_void_p),
+                                   self.out_norm.ctypes.data_as(C.c_void_p), tok.ctypes.data_as(C.c_void_p),
+                                   rows, position, pk.ctypes.data_as(C.c_void_p), pv.ctypes.data_as(C.c_void_p),
+                                   out.ctypes.data_as(C.c_void_p), threads)
+        return out, pk, pv
+
+
+class DeviceModel:
+    """Device weights as wave tiles plus the descriptor the C ABI takes."""
+
+    def __init__(self, shape):
+        self.shape = shape
+        self.keep = []            # tensors kept alive
+        self.layers = (LayerDesc * shape.layers)()
+        self.desc = ModelDesc()
+        self.ring_k, self.ring_v = [], []
+
+    def _finish(self, embed_rows, head_tiles, out_norm):
+        sh, d = self.shape, self.desc
+        for name in ("hidden", "ffn", "q_heads", "kv_heads", "head_dim", "vocab", "sliding_window",
+                     "global_period", "local_base", "global_base", "global_scale", "eps", "ring_local", "ring_global"):
+            setattr(d, name, getattr(sh, name))
+        d.layer_count = sh.layers
+        d.embed_dtype = d.head_dtype = sh.embed_dtype
+        d.embed_rows = embed_rows.data_ptr()
+        d.head_tiles = head_tiles.data_ptr()
+        d.out_norm = out_norm.data_ptr()
+        d.layers = C.cast(self.layers, C.POINTER(LayerDesc))
+        self.keep += [embed_rows, head_tiles, out_norm]
+        self.ring_k_table = torch.tensor([t.data_ptr() for t in self.ring_k], dtype=torch.int64, device="cuda")
+        self.ring_v_table = torch.tensor([t.data_ptr() for t in self.ring_v], dtype=torch.int64, device="cuda")
+        return self
+
+    @classmethod
+    def from_host(cls, host):
+        self = cls(host.shape)
+        sh = host.shape
+        for l in range(sh.layers):
+            for i, (dt, (K, N)) in enumerate(zip(sh.dtypes, sh.proj_shapes())):
+                canonical = torch.from_numpy(host.w[l][i]).cuda()
+                tiles = hip.repack(dt, canonical, K, N)
+                self.keep.append(tiles)
+                self.layers[l].dtype[i] = dt
+                self.layers[l].tiles[i] = tiles.data_ptr()
+            for i in range(6):
+                g = torch.from_numpy(host.norm[l][i]).cuda()
+                self.keep.append(g)
+                self.layers[l].norm[i] = g.data_ptr()
+            rk, rv = torch.from_numpy(host.ring_k[l]).cuda(), torch.from_numpy(host.ring_v[l]).cuda()
+            self.ring_k.append(rk)
+            self.ring_v.append(rv)
+            self.layers[l].ring_k, self.layers[l].ring_v = rk.data_ptr(), rv.data_ptr()
+        embed = torch.from_numpy(host.embed).cuda()
+        head = hip.repack(sh.embed_dtype, embed, sh.hidden, sh.vocab)
+        torch.cuda.synchronize()
+        return self._finish(embed, head, torch.from_numpy(host.out_norm).cuda())
+
+    @classmethod
+    def random(cls, shape, seed, position):
+        """Weights drawn on the device (full-size benchmark: no host copy of the 7 GB)."""
+        self = cls(shape)
+        gen = torch.Generator(device="cuda")
+        gen.manual_seed(seed)
+
+        def blocks(dt, K, N):
+            nb = N * (K // synth.BLOCK_ELEMS[dt])
+            raw = torch.randint(0, 256, (nb, synth.BLOCK_BYTES[dt]), dtype=torch.uint8, device="cuda", generator=gen)
+            d = torch.randn(nb, device="cuda", generator=gen).mul_(0.02).abs_().to(torch.float16).view(torch.uint8).view(nb, 2)
+            if dt == Q4_K:
+                raw[:, 0:2] = d
+                raw[:, 2:4] = torch.randn(nb, device="cuda", generator=gen).mul_(0.02).abs_().to(torch.float16).view(torch.uint8).view(nb, 2)
+            elif dt == Q6_K:
+                raw[:, 208:210] = d
+            else:
+                raw[:, 0:2] = d
+                q = raw[:, 2:]
+                q[q == 0x80] = 0x81
+            return raw.view(-1)
+
+        for l in range(shape.layers):
+            for i, (dt, (K, N)) in enumerate(zip(shape.dtypes, shape.proj_shapes())):
+                tiles = hip.repack(dt, blocks(dt, K, N), K, N)
+                self.keep.append(tiles)
+                self.layers[l].dtype[i] = dt
+                self.layers[l].tiles[i] = tiles.data_ptr()
+            widths = [shape.hidden, shape.head_dim, shape.head_dim, shape.hidden, shape.hidden, shape.hidden]
+            for i, w in enumerate(widths):
+                g = torch.ones(w, dtype=torch.float32, device="cuda")
+                self.keep.append(g)
+                self.layers[l].norm[i] = g.data_ptr()
+            cap = shape.ring_local if shape.is_local(l) else shape.ring_global
+            rk = torch.randn((cap, shape.kv_width), device="cuda", generator=gen).to(torch.float16)
+            rv = torch.randn((cap, shape.kv_width), device="cuda", generator=gen).to(torch.float16)
+            self.ring_k.append(rk)
+            self.ring_v.append(rv)
+            self.layers[l].ring_k, self.layers[l].ring_v = rk.data_ptr(), rv.data_ptr()
+        embed = blocks(shape.embed_dtype, shape.hidden, shape.vocab)
+        head = hip.repack(shape.embed_dtype, embed, shape.hidden, shape.vocab)
+        torch.cuda.synchronize()
+        return self._finish(embed, head, torch.ones(shape.hidden, dtype=torch.float32, device="cuda"))
+
+    def private_rows(self, rows):
+        sh = self.shape
+        return (torch.zeros((sh.layers, rows, sh.kv_width), dtype=torch.float16, device="cuda"),
+                torch.zeros((sh.layers, rows, sh.kv_width), dtype=torch.float16, device="cuda"))
+
+    def forward(self, tokens, position, status=None):
+        """Runs len(tokens) rows; returns (hidden, hidden_sums, priv_k, priv_v)."""
+        sh = self.shape
+        rows = tokens.numel()
+        lib = hip.lib()
+        lib.guffin_hip_forward_scratch_bytes.restype = C.c_uint64
+        nbytes = lib.guffin_hip_forward_scratch_bytes(C.byref(self.desc), rows, position)
+        if nbytes == 0:
+            raise hip.GuffinError(-1, lib.guffin_hip_last_error().decode())
+        scratch = torch.zeros(nbytes, dtype=torch.uint8, device="cuda")
+        pk, pv = self.private_rows(rows)
+        hidden = torch.zeros((rows, sh.hidden), dtype=torch.float32, device="cuda")
+        sums = torch.zeros((rows, sh.hidden // 16 + sh.hidden // 32), dtype=torch.float32, device="cuda")
+        if status is None:
+            status = hip.new_status()
+        hip.check(lib.guffin_hip_forward_rows(hip._stream(), C.byref(self.desc), hip._p(tokens), rows, position,
+                                              hip._p(scratch), C.c_uint64(nbytes), hip._p(pk), hip._p(pv),
+                                              hip._p(hidden), hip._p(sums), hip._p(status)))
+        return hidden, sums, pk, pv, status
+
+
+class H1Plan:
+    """One speculative cycle: buffers, descriptor and the call into guffin_hip_h1_step."""
+
+    def __init__(self, target, drafter, target_position, drafter_position, temperature=1.0, top_k=64,
+                 top_p=0.95, min_p=0.0, seed=0, publish=True):
+        self.target, self.drafter = target, drafter
+        d = self.desc = H1Desc()
+        d.target, d.drafter = C.pointer(target.desc), C.pointer(drafter.desc)
+        d.target_position, d.drafter_position = target_position, drafter_position
+        d.temperature, d.top_k, d.top_p, d.min_p = temperature, top_k, top_p, min_p
+        d.seed, d.step = seed, 0
+        if publish:
+            d.target_ring_k, d.target_ring_v = target.ring_k_table.data_ptr(), target.ring_v_table.data_ptr()
+            d.drafter_ring_k, d.drafter_ring_v = drafter.ring_k_table.data_ptr(), drafter.ring_v_table.data_ptr()
+        lib = hip.lib()
+        lib.guffin_hip_h1_scratch_bytes.restype = C.c_uint64
+        self.nbytes = lib.guffin_hip_h1_scratch_bytes(C.byref(d))
+        if self.nbytes == 0:
+            raise hip.GuffinError(-1, lib.guffin_hip_last_error().decode())
+        self.scratch = torch.zeros(self.nbytes, dtype=torch.uint8, device="cuda")
+        self.d_pk, self.d_pv = drafter.private_rows(1)
+        self.t_pk, self.t_pv = target.private_rows(2)
+        self.result = torch.zeros(hip.result_dtype.itemsize, dtype=torch.uint8, device="cuda")
+        self.status = hip.new_status()
+        self.root = torch.zeros(1, dtype=torch.int32, device="cuda")
+
+    def step(self, step=None):
+        if step is not None:
+            self.desc.step = step
+        hip.check(hip.lib().guffin_hip_h1_step(hip._stream(), C.byref(self.desc), hip._p(self.root),
+                                               hip._p(self.scratch), C.c_uint64(self.nbytes), hip._p(self.d_pk),
+                                               hip._p(self.d_pv), hip._p(self.t_pk), hip._p(self.t_pv),
+                                               hip._p(self.result), hip._p(self.status)))
+
+    def read_result(self):
+        return self.result.cpu().numpy().view(hip.result_dtype)[0]
+
+    def buffers(self):
+        """Views of the step's intermediates inside the scratch arena."""
+        ptrs = [C.c_void_p() for _ in range(7)]
+        hip.check(hip.lib().guffin_hip_h1_buffers(C.byref(self.desc), hip._p(self.scratch),
+                                                  *[C.byref(p) for p in ptrs]))
+        base = self.scratch.data_ptr()
+        T, D = self.target.shape, self.drafter.shape
+
+        def view(ptr, count, dtype):
+            off = ptr.value - base
+            return self.scratch[off:off + count * torch.tensor([], dtype=dtype).element_size()].view(dtype)
+
+        return {
+            "drafter_hidden": view(ptrs[0], D.hidden, torch.float32),
+            "target_hidden": view(ptrs[1], 2 * T.hidden, torch.float32).view(2, T.hidden),
+            "q_logits": view(ptrs[2], D.vocab, torch.float32),
+            "p_logits": view(ptrs[3], 2 * T.vocab, torch.float32).view(2, T.vocab),
+            "law": view(ptrs[4], hip.law_dtype.itemsize, torch.uint8),
+            "candidates": view(ptrs[5], 2 * hip.candidates_dtype.itemsize, torch.uint8),
+            "tokens": view(ptrs[6], 2, torch.int32),
+        }

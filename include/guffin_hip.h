@@ -97,6 +97,12 @@ uint32_t guffin_hip_gemv_packed_slices(int dtype, uint32_t K, uint32_t N);
 int guffin_hip_gemv_packed(void* stream, int dtype, const void* tiles, const float* x, const float* xsums,
                            float* partials, float* y, uint32_t rows, uint32_t K, uint32_t N);
 
+/* Up to three matrices that share the activation rows (q/k/v, gate/up) in one launch.  Each
+ * matrix i writes partials[i] as [S_i][rows][N_i] with S_i = guffin_hip_gemv_packed_slices. */
+int guffin_hip_gemv_packed_multi(void* stream, uint32_t count, const int* dtypes, const void* const* tiles,
+                                 const uint32_t* N, float* const* partials, const float* x,
+                                 const float* xsums, uint32_t rows, uint32_t K);
+
 /* ---- per-layer operators -----------------------------------------------------------------
  * Inputs produced by a packed GEMV may be given as `planes` k-slice partial planes
  * (`plane_stride` floats apart) that the operator sums in slice order while loading; plain
@@ -134,7 +140,8 @@ int guffin_hip_kv_store_f16(void* stream, const float* raw_k, const float* raw_v
  * (NULL gamma skips), RoPE on q and k, fp16 narrowing of k and v
  * (src/engine/gemma_target_runtime.cpp:92-124). */
 int guffin_hip_qkv_post(void* stream, const float* q_raw, const float* k_raw, const float* v_raw,
-                        uint32_t planes, uint64_t q_plane_stride, uint64_t k_plane_stride,
+                        uint32_t q_planes, uint32_t k_planes, uint32_t v_planes,
+                        uint64_t q_plane_stride, uint64_t k_plane_stride,
                         uint64_t v_plane_stride, const float* q_norm, const float* k_norm,
                         const uint32_t* positions, float* q_out, void* k_out, void* v_out,
                         uint32_t rows, uint32_t q_heads, uint32_t kv_heads, uint32_t head_dim,
@@ -221,6 +228,71 @@ int guffin_hip_spec_accept(void* stream, const void* target_candidates, const vo
                            const void* injected_draws, void* result, uint32_t* status);
 /* Host evaluation of the draw schedule above (out: the draws struct). */
 int guffin_hip_step_draws(uint64_t seed, uint64_t step, void* out_draws_host);
+
+/* ---- block graph and one H1 cycle ---------------------------------------------------------
+ * Descriptors of a Gemma-3 shaped decoder whose projection weights are wave tiles
+ * (guffin_hip_repack).  All pointers are device pointers except `layers`, a host array.
+ * The layer policy follows src/engine/model.cpp:607-619: layer l is local (sliding window,
+ * local_base, scale 1) iff l % global_period != global_period - 1, else global. */
+typedef struct guffin_layer_desc {
+    int32_t dtype[7];          /* q, k, v, o, gate, up, down */
+    const void* tiles[7];
+    const float* norm[6];      /* attn_norm, q_norm, k_norm, post_attention_norm, ffn_norm, post_ffw_norm */
+    void* ring_k; void* ring_v; /* fp16 [ring capacity][kv_heads * head_dim] */
+} guffin_layer_desc;
+
+typedef struct guffin_model_desc {
+    uint32_t hidden, ffn, q_heads, kv_heads, head_dim, layer_count, vocab, sliding_window, global_period;
+    float local_base, global_base, global_scale, eps;
+    uint32_t ring_local, ring_global;         /* ring capacities, powers of two */
+    int32_t embed_dtype; const void* embed_rows;   /* canonical [vocab] rows of `hidden` weights */
+    int32_t head_dtype; const void* head_tiles;    /* the same (tied) matrix as wave tiles, may be NULL */
+    const float* out_norm;
+    const guffin_layer_desc* layers;
+} guffin_model_desc;
+
+/* Runs `rows` (1 or 2) contiguous tokens at absolute `position` through every block:
+ * embedding * sqrt(hidden), per block the operator order of encode_gemma_target_blocks
+ * (src/engine/gemma_target_runtime.cpp:13-221; drafter: src/engine/gemma3_draft.mm:888-972),
+ * attention schedule of stage_contiguous_rows (:238-271), final output norm.  New K/V stay in
+ * the private rows priv_k / priv_v [layer][row][kv_heads*head_dim] fp16; the rings are only read.
+ * out_hidden [rows][hidden]; out_hidden_sums (group sums for the head GEMV) may be NULL. */
+uint64_t guffin_hip_forward_scratch_bytes(const guffin_model_desc* model, uint32_t rows, uint32_t position);
+int guffin_hip_forward_rows(void* stream, const guffin_model_desc* model, const uint32_t* tokens,
+                            uint32_t rows, uint32_t position, void* scratch, uint64_t scratch_bytes,
+                            void* priv_k, void* priv_v, float* out_hidden, float* out_hidden_sums,
+                            uint32_t* status);
+/* Publishes private rows into the rings of every layer at slot (position + row) & mask: all
+ * `rows` when accepted is NULL, else row 0 and, if *accepted != 0, row 1 (provisional commit,
+ * src/engine/chain_chat.mm:473-479).  ring_k_table / ring_v_table: device arrays of the
+ * per-layer ring pointers. */
+int guffin_hip_commit_rows(void* stream, const guffin_model_desc* model, const void* priv_k,
+                           const void* priv_v, void* const* ring_k_table, void* const* ring_v_table,
+                           const uint32_t* accepted, uint32_t position, uint32_t rows);
+
+/* One H1 cycle (src/engine/standalone_chat.cpp:508-615, src/engine/chain_chat.mm:245-543):
+ * the drafter ingests the pending root at drafter_position, projects through its tied head,
+ * builds its proposal law and picks x with the step's word; the target evaluates rows
+ * [root, x] at target_position, the head produces both rows' logits, the best top_k of each
+ * row are selected and row 0 decides accept / residual; the verified rows are published.
+ * result: the guffin_hip_spec_accept result.  The ring tables may be NULL to skip publication. */
+typedef struct guffin_h1_desc {
+    const guffin_model_desc* target;
+    const guffin_model_desc* drafter;
+    uint32_t target_position, drafter_position;
+    float temperature; uint32_t top_k; float top_p, min_p;
+    uint64_t seed, step;
+    void* const* target_ring_k; void* const* target_ring_v;
+    void* const* drafter_ring_k; void* const* drafter_ring_v;
+} guffin_h1_desc;
+uint64_t guffin_hip_h1_scratch_bytes(const guffin_h1_desc* desc);
+int guffin_hip_h1_step(void* stream, const guffin_h1_desc* desc, const uint32_t* root_token, void* scratch,
+                       uint64_t scratch_bytes, void* drafter_priv_k, void* drafter_priv_v,
+                       void* target_priv_k, void* target_priv_v, void* result, uint32_t* status);
+/* Addresses, inside `scratch`, of the step's intermediate results (for tests and diagnostics). */
+int guffin_hip_h1_buffers(const guffin_h1_desc* desc, void* scratch, float** drafter_hidden,
+                          float** target_hidden, float** q_logits, float** p_logits, void** law,
+                          void** candidates, uint32_t** tokens);
 
 #ifdef __cplusplus
 }

@@ -1,0 +1,166 @@
+"""GPU parity of the block graph and of one whole H1 cycle against the CPU oracle.
+
+Bars: hidden rows and logits within 1e-3 of the oracle relative to the row's RMS (the oracle
+runs the CPU operators in their sequential fp32 order; fp16 K/V bits may differ on rare
+rounding ties, tolerated at 2^-10 as the reference's own stack test does,
+tests/engine/gemma3_target_runtime_tests.cpp:310-327); proposal, accept / reject decision,
+emitted token and next root bit-exact against the oracle evaluated on the GPU's own logits
+with the same Philox draws.
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def hip():
+    from guffin_amd import hip as module
+    module.init(0)
+    return module
+
+
+def dev(a):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def rel_rms(got, want):
+    want = want.astype(np.float64)
+    scale = np.sqrt((want ** 2).mean(axis=-1, keepdims=True)) + 1e-30
+    return float(np.max(np.abs(got.astype(np.float64) - want) / scale))
+
+
+def check_private_rows(got, want, frac=0.97):
+    import torch
+    g = got.view(torch.int16).cpu().numpy().view(np.uint16)
+    same = np.mean(g == want)
+    assert same >= frac, same
+    d = np.abs(g.view(np.float16).astype(np.float32) - want.view(np.float16).astype(np.float32))
+    scale = np.abs(want.view(np.float16).astype(np.float32)).max()
+    assert d.max() <= 2.0 ** -9 * scale + 1e-6
+
+
+@pytest.mark.parametrize("kind,rows,position", [("drafter", 1, 700), ("drafter", 2, 5), ("target", 2, 1500), ("target", 1, 0)])
+def test_forward_rows_matches_oracle(hip, gfo, kind, rows, position):
+    import torch
+    from dataclasses import replace
+    from guffin_amd import model
+    if kind == "drafter":
+        shape = replace(model.GEMMA3_270M, layers=7, vocab=4096, ring_global=1024)
+    else:
+        shape = replace(model.GEMMA3_12B, layers=6, vocab=2048, ring_global=2048)
+    host = model.HostModel(shape, seed=3, position=position)
+    devm = model.DeviceModel.from_host(host)
+    tokens = np.array([17, 1999][:rows], np.uint32)
+    want, wk, wv = host.oracle_forward(gfo, tokens, position, threads=8)
+    hidden, sums, pk, pv, status = devm.forward(dev(tokens), position)
+    assert int(status.item()) == 0
+    assert rel_rms(hidden.cpu().numpy(), want) <= 1e-3
+    check_private_rows(pk, wk)
+    check_private_rows(pv, wv)
+    h = hidden.cpu().numpy().astype(np.float64)
+    ref_sums = np.concatenate([h.reshape(rows, -1, 16).sum(-1), h.reshape(rows, -1, 32).sum(-1)], axis=1)
+    assert np.allclose(sums.cpu().numpy(), ref_sums, rtol=0, atol=1e-4 * np.abs(h).max() * 4)
+
+
+def oracle_cycle(hip, gfo, plan, bufs, seed, step, top_k, opt_cpu):
+    """The oracle's decision for this cycle, evaluated on the GPU's logits."""
+    q_logits = bufs["q_logits"].cpu().numpy()
+    p_logits = bufs["p_logits"].cpu().numpy()
+    rc, law = gfo.draft_law_compact(q_logits, opt_cpu)
+    assert rc == 0
+    word, ua, ur, un = gfo.step_draws(seed, step)
+    proposal = gfo.lib().gfo_draft_select(C.byref(law), C.c_uint32(word))
+    r0 = gfo.select_candidates(p_logits[0], top_k)
+    r1 = gfo.select_candidates(p_logits[1], top_k)
+    rc, want = gfo.spec_accept(r0, r1, law, proposal, opt_cpu, ua, ur, un)
+    assert rc == 0
+    return proposal, want, law
+
+
+def run_h1(hip, gfo, t_shape, d_shape, t_pos, d_pos, steps, seed, threads=8):
+    import torch
+    from guffin_amd import model
+    t_host = model.HostModel(t_shape, seed=11, position=t_pos)
+    d_host = model.HostModel(d_shape, seed=12, position=d_pos)
+    target = model.DeviceModel.from_host(t_host)
+    drafter = model.DeviceModel.from_host(d_host)
+    plan = model.H1Plan(target, drafter, t_pos, d_pos, seed=seed, publish=False)
+    opt_cpu = gfo.SamplerOptions(1.0, 64, 0.95, 0.0, 1.0)
+    root = 123
+    plan.root.fill_(root)
+    accepted = 0
+    for step in range(steps):
+        plan.step(step)
+        torch.cuda.synchronize()
+        bufs = plan.buffers()
+        res = plan.read_result()
+        assert int(plan.status.item()) == 0 and res["status"] == 0
+        proposal, want, _ = oracle_cycle(hip, gfo, plan, bufs, seed, step, 64, opt_cpu)
+        assert res["proposal"] == proposal
+        assert (res["accepted"], res["token"], res["next_root"]) == (want.accepted, want.token, want.next_root)
+        assert abs(res["acceptance_probability"] - want.acceptance_probability) <= 1e-13
+        accepted += int(res["accepted"])
+        if step == 0:
+            # numerical parity of both forwards and both heads against the CPU path
+            dh, _, _ = d_host.oracle_forward(gfo, [root], d_pos, threads=threads)
+            assert rel_rms(bufs["drafter_hidden"].cpu().numpy()[None, :], dh) <= 1e-3
+            ql = gfo.gemv(d_shape.embed_dtype, d_host.embed, dh, d_shape.vocab, threads=threads)
+            assert rel_rms(bufs["q_logits"].cpu().numpy()[None, :], ql) <= 1e-3
+            toks = bufs["tokens"].cpu().numpy().view(np.uint32)
+            assert toks[0] == root and toks[1] == proposal
+            th, wk, wv = t_host.oracle_forward(gfo, toks, t_pos, threads=threads)
+            assert rel_rms(bufs["target_hidden"].cpu().numpy(), th) <= 1e-3
+            pl = gfo.gemv(t_shape.embed_dtype, t_host.embed, th, t_shape.vocab, threads=threads)
+            assert rel_rms(bufs["p_logits"].cpu().numpy(), pl) <= 1e-3
+            check_private_rows(plan.t_pk, wk)
+            check_private_rows(plan.t_pv, wv)
+    return accepted, plan, target, drafter, t_host
+
+
+def test_h1_cycle_small_models(hip, gfo):
+    from dataclasses import replace
+    from guffin_amd import model
+    t_shape = replace(model.GEMMA3_12B, layers=3, vocab=16384, ring_global=2048)
+    d_shape = replace(model.GEMMA3_270M, layers=4, vocab=16384, ring_global=2048)
+    run_h1(hip, gfo, t_shape, d_shape, 1300, 1300, steps=12, seed=5)
+
+
+def test_h1_commit_publishes_verified_rows(hip, gfo):
+    import torch
+    from dataclasses import replace
+    from guffin_amd import model
+    t_shape = replace(model.GEMMA3_12B, layers=6, vocab=4096, ring_global=2048)
+    d_shape = replace(model.GEMMA3_270M, layers=6, vocab=4096, ring_global=2048)
+    t_pos = 1030
+    target = model.DeviceModel.from_host(model.HostModel(t_shape, seed=21, position=t_pos))
+    drafter = model.DeviceModel.from_host(model.HostModel(d_shape, seed=22, position=t_pos))
+    before = [(k.clone(), v.clone()) for k, v in zip(target.ring_k, target.ring_v)]
+    plan = model.H1Plan(target, drafter, t_pos, t_pos, seed=9, publish=True)
+    plan.root.fill_(77)
+    plan.step(0)
+    torch.cuda.synchronize()
+    res = plan.read_result()
+    publish = 1 + int(res["accepted"])
+    for l in range(t_shape.layers):
+        cap = t_shape.ring_local if t_shape.is_local(l) else t_shape.ring_global
+        for row in range(2):
+            slot = (t_pos + row) & (cap - 1)
+            if row < publish:
+                assert torch.equal(target.ring_k[l][slot], plan.t_pk[l, row])
+                assert torch.equal(target.ring_v[l][slot], plan.t_pv[l, row])
+            else:
+                assert torch.equal(target.ring_k[l][slot], before[l][0][slot])
+        untouched = [s for s in range(cap) if s not in ((t_pos) & (cap - 1), (t_pos + 1) & (cap - 1))][:50]
+        assert torch.equal(target.ring_k[l][untouched], before[l][0][untouched])
+    cap = d_shape.ring_local
+    assert torch.equal(drafter.ring_k[0][t_pos & (cap - 1)], plan.d_pk[0, 0])
+
+
+def test_h1_cycle_full_size_models(hip, gfo):
+    """Config 4 shapes: the 48-block 12B target at an 8192-token context with the 18-block drafter."""
+    from guffin_amd import model
+    accepted, plan, *_ = run_h1(hip, gfo, model.GEMMA3_12B, model.GEMMA3_270M, 8190, 4096, steps=2, seed=1, threads=16)
