@@ -1,0 +1,203 @@
+#!/usr/bin/env python3
+"""Benchmark of the H1 speculative decode step on one MI355X.
+
+Workload (BASELINE.json config 4): one H1 cycle of the Gemma-3-12B-shaped Q4_K_M target
+(48 blocks, 2-row verify at an 8192-token fp16 KV context, tied Q6_K 262144 head, top-64
+selection, lossless accept) with the 270M-shaped Q8_0 drafter (1 row, 4096-token context),
+seeded random weights drawn on the device.  A step is one whole cycle replayed as a HIP
+graph; `value` is the mean step latency in microseconds with every input resident in HBM.
+
+Extra objects on the JSON line:
+  roofline      the dominant kernel (2-row Q4_K gate+up GEMV of one block, 66.4 MB of weights
+                per launch): algorithmic bytes / mean launch duration, measured with HIP events
+                around a graph of 48 back-to-back launches over the 48 blocks' own weights
+                (3.2 GB, far beyond the caches) on the launch stream.
+  cpu_baseline  the reference's own CPU row dot (oracle/_ref) or the oracle port timed on the
+                host cores on a bounded sample (one block's seven GEMVs at 2 rows, a column
+                subset), extrapolated to a whole step by weight count.  Reported, not a target.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+
+
+def step_bytes(T, D, t_pos, d_pos):
+    """Algorithmic HBM bytes of one cycle: weights once per GEMV, activations in/out, KV once per KV head."""
+    def model(sh, rows, pos):
+        w = sh.layers * sh.layer_weight_bytes() + sh.head_bytes()
+        kv = 0
+        for l in range(sh.layers):
+            tokens = min(pos, sh.sliding_window) if sh.is_local(l) else pos
+            kv += tokens * sh.kv_width * 2 * 2
+        act = sh.layers * rows * 4 * (2 * sh.hidden * 4 + 2 * sh.q_width + 2 * sh.kv_width + 3 * sh.ffn)
+        logits = rows * sh.vocab * 4 * 2
+        norms = sh.layers * (4 * sh.hidden + 2 * sh.head_dim) * 4
+        return w + kv + act + logits + norms
+    return model(T, 2, t_pos) + model(D, 1, d_pos)
+
+
+def cpu_baseline(T, D, budget_s=20.0):
+    """Times the CPU path on a bounded sample and extrapolates to one step by weight count."""
+    import numpy as np
+    from guffin_amd import synth
+    from oracle import gfo
+    gfo.build()
+    ref = gfo.ref()
+    kind = "reference" if ref is not None else "port"
+    cores = 1 if ref is not None else (os.cpu_count() or 1)
+    shapes = list(zip(T.dtypes, T.proj_shapes()))
+    # calibrate on a small slice, then size the sample to the budget
+    dt, (K, N) = shapes[0]
+    w = synth.make_weight(dt, K, 64, 1)
+    x = synth.make_activation(2, K, 2)
+    t0 = time.perf_counter()
+    gfo.gemv(dt, w, x, 64, threads=cores, which=ref)
+    per_weight = (time.perf_counter() - t0) / (K * 64)
+    layer_weights = sum(K * N for _, (K, N) in shapes)
+    frac = min(1.0, budget_s / (per_weight * layer_weights * 1.3))
+    done_weights, elapsed = 0, 0.0
+    for i, (dt, (K, N)) in enumerate(shapes):
+        n = max(64, int(N * frac) // 64 * 64)
+        w = synth.make_weight(dt, K, n, 10 + i)
+        x = synth.make_activation(2, K, 20 + i)
+        t0 = time.perf_counter()
+        gfo.gemv(dt, w, x, n, threads=cores, which=ref)
+        elapsed += time.perf_counter() - t0
+        done_weights += K * n
+    step_weights = (T.layers * layer_weights + T.hidden * T.vocab
+                    + 0.5 * (D.layers * sum(K * N for K, N in D.proj_shapes()) + D.hidden * D.vocab))  # drafter: 1 row
+    value_us = elapsed / done_weights * step_weights * 1e6
+    return {
+        "value": round(value_us, 1), "unit": "us", "cores": cores, "kind": kind,
+        "sample": "one 12B block's 7 GEMVs at 2 rows, first %.1f%% of each matrix's columns (%.2f s of CPU work), "
+                  "scaled to the step's weight count; %s" % (
+                      100 * frac, elapsed,
+                      "reference dot_q4_k_row_f32 / dot_q6_k_row_f32 (src/tensor/quantization.cpp), single thread"
+                      if ref is not None else "oracle gfo_gemv_mt on all host threads"),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--layers", type=int, default=0, help="debug: truncate the target to this many blocks")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs the H1 step on ONE GPU; --gpus %d is not supported "
+              "(no collectives or sharding are part of it)" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from dataclasses import replace
+    from guffin_amd import hip, model
+    hip.init(0)
+
+    T, D = model.GEMMA3_12B, model.GEMMA3_270M
+    if args.layers:
+        T = replace(T, layers=args.layers)
+    t_pos, d_pos = 8190, 4096
+    target = model.DeviceModel.random(T, seed=0, position=t_pos)
+    drafter = model.DeviceModel.random(D, seed=1, position=d_pos)
+    plan = model.H1Plan(target, drafter, t_pos, d_pos, temperature=1.0, top_k=64, top_p=0.95, min_p=0.0,
+                        seed=0, publish=True)
+    plan.root.fill_(2)
+
+    # eager once (validates the path end to end), then capture the whole cycle as a HIP graph
+    plan.step(0)
+    torch.cuda.synchronize()
+    first = plan.read_result()
+    if int(plan.status.item()) != 0 or first["status"] != 0:
+        raise RuntimeError("H1 step failed: device status %d, law status %d" % (int(plan.status.item()), first["status"]))
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        plan.step(0)
+    for _ in range(args.warmup):
+        graph.replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        graph.replay()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    replayed = plan.read_result()
+    if (replayed["accepted"], replayed["token"], replayed["next_root"]) != (first["accepted"], first["token"], first["next_root"]):
+        raise RuntimeError("graph replay changed the step's decision")
+
+    # ---- roofline of the dominant kernel: 2-row Q4_K gate+up GEMV, one launch per block -----
+    import ctypes as C
+    H, F = T.hidden, T.ffn
+    x = torch.randn(2, H, device="cuda")
+    xs = hip.group_sums(x)
+    lib = hip.lib()
+    lib.guffin_hip_gemv_packed_multi_slices.restype = C.c_uint32
+    S = lib.guffin_hip_gemv_packed_multi_slices(2, (C.c_int * 2)(T.dtypes[4], T.dtypes[5]), (C.c_uint32 * 2)(F, F), H)
+    pg = torch.empty(S, 2, F, device="cuda")
+    pu = torch.empty(S, 2, F, device="cuda")
+
+    def launch_all():
+        for l in range(T.layers):
+            L = target.layers[l]
+            dt = (C.c_int * 2)(L.dtype[4], L.dtype[5])
+            tiles = (C.c_void_p * 2)(L.tiles[4], L.tiles[5])
+            n = (C.c_uint32 * 2)(F, F)
+            parts = (C.c_void_p * 2)(pg.data_ptr(), pu.data_ptr())
+            hip.check(lib.guffin_hip_gemv_packed_multi(hip._stream(), 2, dt, tiles, n, parts, hip._p(x), hip._p(xs), 2, H))
+
+    launch_all()
+    torch.cuda.synchronize()
+    kgraph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(kgraph):
+        launch_all()
+    for _ in range(3):
+        kgraph.replay()
+    stream = torch.cuda.current_stream()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    reps = 10
+    e0.record(stream)
+    for _ in range(reps):
+        kgraph.replay()
+    e1.record(stream)
+    torch.cuda.synchronize()
+    launch_us = e0.elapsed_time(e1) * 1e3 / (reps * T.layers)
+    from guffin_amd import synth
+    kernel_bytes = 2 * synth.weight_bytes(T.dtypes[4], H, F) + 2 * (H + H // 16 + H // 32) * 4 + 2 * S * 2 * F * 4
+    achieved = kernel_bytes / launch_us / 1e3  # GB/s
+
+    total_bytes = step_bytes(T, D, t_pos, d_pos)
+    line = {
+        "metric": "h1_step_latency_us", "value": round(ms_per_step * 1e3, 1), "unit": "us",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": "config 4: full Gemma-3-12B-shaped Q4_K_M H1 step (270M Q8_0 drafter 1 row @4096 ctx, "
+                        "48-block 2-row verify @8192-token fp16 KV, Q6_K 262144 head, top-64 select, lossless accept)",
+            "target_blocks": T.layers, "rows": 2, "kv_context": t_pos + 2, "vocab": T.vocab,
+            "step_algorithmic_bytes": total_bytes,
+            "step_hbm_frac": round(total_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+            "accepted": int(first["accepted"]),
+        },
+        "roofline": {
+            "kernel": "gemv_packed_multi_kernel<2, 2> (Q4_K gate+up, 2 rows, K=3840, N=2x15360)",
+            "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+            "bytes_per_launch": kernel_bytes, "launch_us": round(launch_us, 3),
+        },
+    }
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline(T, D)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

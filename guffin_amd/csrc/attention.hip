@@ -17,8 +17,8 @@
 //           rows), four tokens per wave at a time; fp16 keys enter v_fma_mix_f32 directly;
 //           a 4-step exchange inside each 16-lane group finishes the dot product.
 //   softmax per query over the partition in LDS (max, exp, sum).
-//   pass 2  values: a wave owns every fourth token, a lane four output dims; no cross-lane
-//           reduction, the four waves are merged through LDS.
+//   pass 2  values: a half wave owns one token (a lane eight output dims, 16-byte loads);
+//           halves are combined by one lane exchange, the four waves through LDS.
 // Partitions emit (max, denominator, unnormalised output); a second kernel merges them in
 // partition order.  fp32 throughout, keys/values stay fp16 in memory.
 #include "common.hpp"
@@ -90,40 +90,49 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(AttnArgs a) {
 #pragma unroll
             for (int i = 0; i < 16; ++i) qv[n][i] = qp[i] * a.scale;
         }
-        for (uint32_t t = t0 + wv * 4 + slot; t < t0 + a.tp; t += 16) {
-            float s[NQ];
+        // four rounds of loads are issued before their dot products so that a wave keeps
+        // 16 key rows (8 KB) in flight
+        constexpr int U = 4;
+        for (uint32_t tb = t0 + wv * 4 + slot; tb < t0 + a.tp; tb += 16 * U) {
+            uint4 k0[U], k1[U];
 #pragma unroll
-            for (int n = 0; n < NQ; ++n) s[n] = 0.f;
-            const bool in_range = t < t1;
-            uint32_t pos = 0, prow = 0;
-            bool is_priv = false;
-            if (in_range) {
-                is_priv = t >= n_ring;
-                pos = u_first + t; prow = t - n_ring;
-                const uint16_t* kp = is_priv ? a.priv_k + size_t(prow) * row_stride
-                                             : a.ring_k + size_t(pos & a.ring_mask) * row_stride;
-                kp += kvh * HD + seg * 16;
-                const uint4 k0 = *reinterpret_cast<const uint4*>(kp), k1 = *reinterpret_cast<const uint4*>(kp + 8);
-                const uint32_t kw[8] = {k0.x, k0.y, k0.z, k0.w, k1.x, k1.y, k1.z, k1.w};
-#pragma unroll
-                for (int n = 0; n < NQ; ++n)
-#pragma unroll
-                    for (int i = 0; i < 8; ++i) s[n] = dot2(s[n], kw[i], qv[n][2 * i], qv[n][2 * i + 1]);
+            for (int u = 0; u < U; ++u) {
+                const uint32_t t = tb + 16 * u;
+                k0[u] = make_uint4(0, 0, 0, 0); k1[u] = k0[u];
+                if (t < t1) {
+                    const bool is_priv = t >= n_ring;
+                    const uint16_t* kp = is_priv ? a.priv_k + size_t(t - n_ring) * row_stride
+                                                 : a.ring_k + size_t((u_first + t) & a.ring_mask) * row_stride;
+                    kp += kvh * HD + seg * 16;
+                    k0[u] = *reinterpret_cast<const uint4*>(kp); k1[u] = *reinterpret_cast<const uint4*>(kp + 8);
+                }
             }
 #pragma unroll
-            for (int n = 0; n < NQ; ++n) {
-                s[n] += __shfl_xor(s[n], 8, kWave);
-                s[n] += __shfl_xor(s[n], 4, kWave);
-                s[n] += __shfl_xor(s[n], 2, kWave);
-                s[n] += __shfl_xor(s[n], 1, kWave);
-            }
-            if (seg == 0) {
+            for (int u = 0; u < U; ++u) {
+                const uint32_t t = tb + 16 * u;
+                if (t >= t0 + a.tp) break;
+                const bool in_range = t < t1, is_priv = t >= n_ring;
+                const uint32_t pos = u_first + t, prow = t - n_ring;
+                const uint32_t kw[8] = {k0[u].x, k0[u].y, k0[u].z, k0[u].w, k1[u].x, k1[u].y, k1[u].z, k1[u].w};
+                float s[NQ];
 #pragma unroll
                 for (int n = 0; n < NQ; ++n) {
-                    const uint32_t r = n / group;
-                    const bool valid = in_range && (is_priv ? ((amask[r] >> prow) & 1u) != 0
-                                                            : (pos >= bfirst[r] && pos < bend[r]));
-                    sc[n * a.tp + (t - t0)] = valid ? s[n] : -INFINITY;
+                    s[n] = 0.f;
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) s[n] = dot2(s[n], kw[i], qv[n][2 * i], qv[n][2 * i + 1]);
+                    s[n] += __shfl_xor(s[n], 8, kWave);
+                    s[n] += __shfl_xor(s[n], 4, kWave);
+                    s[n] += __shfl_xor(s[n], 2, kWave);
+                    s[n] += __shfl_xor(s[n], 1, kWave);
+                }
+                if (seg == 0) {
+#pragma unroll
+                    for (int n = 0; n < NQ; ++n) {
+                        const uint32_t r = n / group;
+                        const bool valid = in_range && (is_priv ? ((amask[r] >> prow) & 1u) != 0
+                                                                : (pos >= bfirst[r] && pos < bend[r]));
+                        sc[n * a.tp + (t - t0)] = valid ? s[n] : -INFINITY;
+                    }
                 }
             }
         }
@@ -148,31 +157,56 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(AttnArgs a) {
     __syncthreads();
 
     // ---- pass 2: values -------------------------------------------------------------------
+    // A half wave covers one value row (32 lanes x 8 dims, 16-byte loads), a wave two tokens
+    // per round, four rounds in flight; halves are combined by a lane exchange, waves via LDS.
     {
-        float acc[NQ][4];
+        constexpr int U = 4;
+        const uint32_t hsel = lane >> 5, dl = (lane & 31) * 8;
+        float acc[NQ][8];
 #pragma unroll
         for (int n = 0; n < NQ; ++n)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) acc[n][i] = 0.f;
-        for (uint32_t t = t0 + wv; t < t1; t += 4) {
-            const bool is_priv = t >= n_ring;
-            const uint16_t* vp = is_priv ? a.priv_v + size_t(t - n_ring) * row_stride
-                                         : a.ring_v + size_t((u_first + t) & a.ring_mask) * row_stride;
-            const uint2 vv = *reinterpret_cast<const uint2*>(vp + kvh * HD + lane * 4);
+            for (int i = 0; i < 8; ++i) acc[n][i] = 0.f;
+        for (uint32_t tb = t0 + wv * 2 + hsel; tb < t1; tb += 8 * U) {
+            uint4 vv[U];
 #pragma unroll
-            for (int n = 0; n < NQ; ++n) {
-                const float p = sc[n * a.tp + (t - t0)];
-                const half2_t h0 = __builtin_bit_cast(half2_t, vv.x), h1 = __builtin_bit_cast(half2_t, vv.y);
-                acc[n][0] = fmaf(static_cast<float>(h0.x), p, acc[n][0]);
-                acc[n][1] = fmaf(static_cast<float>(h0.y), p, acc[n][1]);
-                acc[n][2] = fmaf(static_cast<float>(h1.x), p, acc[n][2]);
-                acc[n][3] = fmaf(static_cast<float>(h1.y), p, acc[n][3]);
+            for (int u = 0; u < U; ++u) {
+                const uint32_t t = tb + 8 * u;
+                vv[u] = make_uint4(0, 0, 0, 0);
+                if (t < t1) {
+                    const bool is_priv = t >= n_ring;
+                    const uint16_t* vp = is_priv ? a.priv_v + size_t(t - n_ring) * row_stride
+                                                 : a.ring_v + size_t((u_first + t) & a.ring_mask) * row_stride;
+                    vv[u] = *reinterpret_cast<const uint4*>(vp + kvh * HD + dl);
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const uint32_t t = tb + 8 * u;
+                if (t >= t1) break;
+                const uint32_t w4[4] = {vv[u].x, vv[u].y, vv[u].z, vv[u].w};
+#pragma unroll
+                for (int n = 0; n < NQ; ++n) {
+                    const float p = sc[n * a.tp + (t - t0)];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const half2_t h = __builtin_bit_cast(half2_t, w4[i]);
+                        acc[n][2 * i] = fmaf(static_cast<float>(h.x), p, acc[n][2 * i]);
+                        acc[n][2 * i + 1] = fmaf(static_cast<float>(h.y), p, acc[n][2 * i + 1]);
+                    }
+                }
             }
         }
 #pragma unroll
-        for (int n = 0; n < NQ; ++n)
-            *reinterpret_cast<float4*>(merge + (wv * NQ + n) * HD + lane * 4) =
-                make_float4(acc[n][0], acc[n][1], acc[n][2], acc[n][3]);
+        for (int n = 0; n < NQ; ++n) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc[n][i] += __shfl_xor(acc[n][i], 32, kWave);
+            if (hsel == 0) {
+                float* mp = merge + (wv * NQ + n) * HD + dl;
+                *reinterpret_cast<float4*>(mp) = make_float4(acc[n][0], acc[n][1], acc[n][2], acc[n][3]);
+                *reinterpret_cast<float4*>(mp + 4) = make_float4(acc[n][4], acc[n][5], acc[n][6], acc[n][7]);
+            }
+        }
     }
     __syncthreads();
     for (uint32_t i = threadIdx.x; i < NQ * HD; i += 256) {
@@ -186,23 +220,42 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(AttnArgs a) {
     }
 }
 
-// out[row][head][:] = sum_p e^(m_p - M) acc_p / sum_p e^(m_p - M) l_p, partitions in order
+// out[row][head][:] = sum_p e^(m_p - M) acc_p / sum_p e^(m_p - M) l_p, partitions in order.
+// The partition weights are formed once, in parallel, in LDS; each thread then owns one
+// output dimension and walks the partitions with independent loads.
 __global__ void __launch_bounds__(256)
 attn_merge_kernel(const float* __restrict__ part_out, const float* __restrict__ part_ml, float* __restrict__ out,
                   float* __restrict__ out_sums, uint32_t partitions, uint32_t hd, uint32_t q_heads,
                   uint32_t* __restrict__ status) {
-    const uint32_t rh = blockIdx.x;  // row * q_heads + head
-    const float* ml = part_ml + size_t(rh) * partitions * 2;
-    float M = -INFINITY;
-    for (uint32_t p = 0; p < partitions; ++p) if (ml[2 * p + 1] > 0.f) M = fmaxf(M, ml[2 * p]);
-    float denom = 0.f;
-    for (uint32_t p = 0; p < partitions; ++p) if (ml[2 * p + 1] > 0.f) denom += expf(ml[2 * p] - M) * ml[2 * p + 1];
+    extern __shared__ float wgt[];  // [partitions]
+    __shared__ float red[4];
     __shared__ float rowbuf[1024];
+    const uint32_t rh = blockIdx.x;  // row * q_heads + head
+    const uint32_t lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const float* ml = part_ml + size_t(rh) * partitions * 2;
+    float m = -INFINITY;
+    for (uint32_t p = threadIdx.x; p < partitions; p += 256) if (ml[2 * p + 1] > 0.f) m = fmaxf(m, ml[2 * p]);
+    m = wave_max(m);
+    if (lane == 0) red[wv] = m;
+    __syncthreads();
+    const float M = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    for (uint32_t p = threadIdx.x; p < partitions; p += 256)
+        wgt[p] = ml[2 * p + 1] > 0.f ? expf(ml[2 * p] - M) : 0.f;
+    __syncthreads();
+    float denom = 0.f;
+    for (uint32_t p = 0; p < partitions; ++p) denom = fmaf(wgt[p], ml[2 * p + 1], denom);
     bool bad = false;
+    const float* po = part_out + size_t(rh) * partitions * hd;
     for (uint32_t d = threadIdx.x; d < hd; d += blockDim.x) {
         float acc = 0.f;
-        for (uint32_t p = 0; p < partitions; ++p)
-            if (ml[2 * p + 1] > 0.f) acc = fmaf(expf(ml[2 * p] - M), part_out[(size_t(rh) * partitions + p) * hd + d], acc);
+        uint32_t p = 0;
+        for (; p + 4 <= partitions; p += 4) {
+            const float v0 = po[size_t(p) * hd + d], v1 = po[size_t(p + 1) * hd + d], v2 = po[size_t(p + 2) * hd + d],
+                        v3 = po[size_t(p + 3) * hd + d];
+            acc = fmaf(wgt[p], v0, acc); acc = fmaf(wgt[p + 1], v1, acc);
+            acc = fmaf(wgt[p + 2], v2, acc); acc = fmaf(wgt[p + 3], v3, acc);
+        }
+        for (; p < partitions; ++p) acc = fmaf(wgt[p], po[size_t(p) * hd + d], acc);
         const float v = acc / denom;
         bad |= !isfinite(v);
         out[size_t(rh) * hd + d] = v;
@@ -289,7 +342,7 @@ extern "C" int guffin_hip_attention_decode(void* stream, const float* q, const v
         default: return fail(GUFFIN_E_SHAPE, "attention_decode: q_heads / kv_heads must be 1, 2 or 4");
     }
     if (rc) return rc;
-    hipLaunchKernelGGL(attn_merge_kernel, dim3(rows * q_heads), dim3(256), 0, s, partial_out, partial_ml, out,
+    hipLaunchKernelGGL(attn_merge_kernel, dim3(rows * q_heads), dim3(256), a.partitions * sizeof(float), s, partial_out, partial_ml, out,
                        out_sums, a.partitions, head_dim, q_heads, status);
     return check_launch("attention_merge");
 }

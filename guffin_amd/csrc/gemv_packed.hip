@@ -17,15 +17,16 @@
 //
 // GEMV: lane l owns output column 64*tile + l for a slice of K.  All lanes walk the same
 // k, so activations are wave-uniform and are read through the scalar cache straight into
-// FMA operands; no LDS, no barrier, no cross-lane reduction.  Quants are spread into
+// FMA operands; no cross-lane reduction, LDS only to combine the waves of a workgroup.  Quants are spread into
 // 16-bit fields and fed to v_fma_mix_f32 as fp16 subnormals (an integer n < 1024 in a
 // half is exactly n*2^-24), which replaces convert+FMA by one FMA per weight per row with
 // bit-identical products; the 2^24 is folded into the block scale.  The offset terms
 // (-dmin*m for Q4_K, -32 for Q6_K, -128 for the biased Q8_0 bytes) use per-16 / per-32
-// activation sums supplied by the producer of x.  K is cut into S slices across
-// workgroups; slice partials go to [S][rows][N] and are summed in slice order by the
-// consumer (or by reduce_partials below), so results are deterministic and a row's
-// arithmetic does not depend on how many rows are computed.
+// activation sums supplied by the producer of x.  K is cut into slices: up to 16 slices are
+// the waves of one workgroup and are combined in wave order through LDS, the remaining
+// S "planes" go to [S][rows][N] and are summed in plane order by the consumer (or by
+// reduce_partials below), so results are deterministic and a row's arithmetic does not
+// depend on how many rows are computed.
 #include "common.hpp"
 
 namespace guffin {
@@ -278,23 +279,20 @@ __device__ __forceinline__ void compute_tile(const Q8Tile& t, const float* __res
 // =======================================================================================
 // The streaming kernel: one wave = one (column tile, k-slice)
 // =======================================================================================
+// One wave: blocks [b0, b1) of column tile `ct`; returns the per-lane column sums.
 template <int DTYPE, int R>
-__device__ __forceinline__ void run_tile_slice(const uint8_t* __restrict__ wt, const float* __restrict__ x,
-                                               const float* __restrict__ xsums, float* __restrict__ part,
-                                               uint32_t K, uint32_t N, uint32_t nblk, uint32_t bps,
-                                               uint32_t ct, uint32_t slice) {
+__device__ __forceinline__ void run_blocks(const uint8_t* __restrict__ wt, const float* __restrict__ x,
+                                           const float* __restrict__ xsums, uint32_t K, uint32_t nblk,
+                                           uint32_t ct, uint32_t b0, uint32_t b1, float (&acc)[R]) {
     constexpr uint32_t TB = kTileCols * block_bytes(DTYPE), BE = block_elems(DTYPE);
-    const uint32_t lane = threadIdx.x;
-    const uint32_t b0 = slice * bps, b1 = b0 + bps < nblk ? b0 + bps : nblk;
+    const uint32_t lane = threadIdx.x & 63;
     const uint32_t n16 = K / 16, per_row = n16 + K / 32;
     // Q6_K consumes 16-sums (16 per block), Q4_K 32-sums (8 per block), Q8_0 one 32-sum per block
     const float* xs = DTYPE == GUFFIN_Q6_K ? xsums : xsums + n16;
     constexpr uint32_t sums_per_block = DTYPE == GUFFIN_Q6_K ? 16 : DTYPE == GUFFIN_Q4_K ? 8 : 1;
     const uint8_t* tp = wt + (size_t(ct) * nblk + b0) * TB + lane * 16;
-    float acc[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) acc[r] = 0.f;
-
     if constexpr (DTYPE == GUFFIN_Q4_K) {
         Q4Tile cur, nxt;
         if (b0 < b1) load_tile(cur, tp);
@@ -320,62 +318,109 @@ __device__ __forceinline__ void run_tile_slice(const uint8_t* __restrict__ wt, c
             cur = nxt;
         }
     }
-#pragma unroll
-    for (int r = 0; r < R; ++r) part[(size_t(slice) * R + r) * N + ct * kTileCols + lane] = acc[r];
 }
 
-template <int DTYPE, int R>
-__global__ void __launch_bounds__(64)
-gemv_packed_kernel(const uint8_t* __restrict__ wt, const float* __restrict__ x, const float* __restrict__ xsums,
-                   float* __restrict__ part, uint32_t K, uint32_t N, uint32_t nblk, uint32_t bps) {
-    run_tile_slice<DTYPE, R>(wt, x, xsums, part, K, N, nblk, bps, blockIdx.x, blockIdx.y);
-}
-
-// Several matrices that share the activation rows (q/k/v, gate/up) in one launch: the
-// column tiles of all matrices are laid side by side along grid x.
-struct PackedMat { const uint8_t* tiles; float* part; uint32_t N, dtype, S, bps, tile_end; };
-struct MultiArgs { PackedMat m[3]; const float* x; const float* xsums; uint32_t K, count; };
+// Workgroup = W waves over consecutive k-slices of one column tile; the W per-lane sums are
+// combined through LDS in wave order and written as one plane.  grid = (tiles, planes).
+struct PackedCfg { uint32_t K, nblk, bps, W; };
 
 template <int R>
-__global__ void __launch_bounds__(64) gemv_packed_multi_kernel(MultiArgs a) {
-    uint32_t which = 0, first = 0;
-    while (which + 1 < a.count && blockIdx.x >= a.m[which].tile_end) { first = a.m[which].tile_end; ++which; }
-    const PackedMat& m = a.m[which];
-    if (blockIdx.y >= m.S) return;
-    const uint32_t ct = blockIdx.x - first;
-    if (m.dtype == GUFFIN_Q4_K)
-        run_tile_slice<GUFFIN_Q4_K, R>(m.tiles, a.x, a.xsums, m.part, a.K, m.N, a.K / 256, m.bps, ct, blockIdx.y);
-    else if (m.dtype == GUFFIN_Q6_K)
-        run_tile_slice<GUFFIN_Q6_K, R>(m.tiles, a.x, a.xsums, m.part, a.K, m.N, a.K / 256, m.bps, ct, blockIdx.y);
-    else
-        run_tile_slice<GUFFIN_Q8_0, R>(m.tiles, a.x, a.xsums, m.part, a.K, m.N, a.K / 32, m.bps, ct, blockIdx.y);
+__device__ __forceinline__ void finish_tile(float (&acc)[R], float* __restrict__ part, uint32_t N, uint32_t ct,
+                                            uint32_t plane, uint32_t W) {
+    __shared__ float red[16 * 2 * 64];
+    const uint32_t lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    if (W == 1) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) part[(size_t(plane) * R + r) * N + ct * kTileCols + lane] = acc[r];
+        return;
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) red[(wv * R + r) * 64 + lane] = acc[r];
+    __syncthreads();
+    if (threadIdx.x < R * 64) {
+        const uint32_t r = threadIdx.x >> 6;
+        float t = red[r * 64 + lane];
+        for (uint32_t w = 1; w < W; ++w) t += red[(w * R + r) * 64 + lane];
+        part[(size_t(plane) * R + r) * N + ct * kTileCols + lane] = t;
+    }
+}
+
+// Q6_K tiles need more than the 128 registers a 16-wave workgroup leaves each lane.
+constexpr uint32_t max_waves(int dtype) { return dtype == GUFFIN_Q6_K ? 8 : 16; }
+constexpr int kMixed = 3;  // Q4_K and Q6_K matrices in one launch
+
+template <int DTYPE, int R>
+__global__ void __launch_bounds__(64 * max_waves(DTYPE))
+gemv_packed_kernel(const uint8_t* __restrict__ wt, const float* __restrict__ x, const float* __restrict__ xsums,
+                   float* __restrict__ part, uint32_t N, PackedCfg c) {
+    const uint32_t slice = blockIdx.y * c.W + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t b0 = min(slice * c.bps, c.nblk), b1 = min(b0 + c.bps, c.nblk);
+    float acc[R];
+    run_blocks<DTYPE, R>(wt, x, xsums, c.K, c.nblk, blockIdx.x, b0, b1, acc);
+    finish_tile<R>(acc, part, N, blockIdx.x, blockIdx.y, c.W);
+}
+
+// Several matrices that share the activation rows (q/k/v, gate/up) in one launch: the column
+// tiles of all matrices sit side by side along grid x.  COUNT also names the instantiation
+// so that profiles tell q/k/v (3) from gate/up (2).
+struct MultiMeta { uint32_t N[3], dtype[3], tile_end[3]; };
+
+template <int R, int COUNT, int MODE>
+__global__ void __launch_bounds__(64 * max_waves(MODE == kMixed ? GUFFIN_Q6_K : MODE))
+gemv_packed_multi_kernel(const uint8_t* __restrict__ t0, const uint8_t* __restrict__ t1, const uint8_t* __restrict__ t2,
+                         float* __restrict__ p0, float* __restrict__ p1, float* __restrict__ p2,
+                         const float* __restrict__ x, const float* __restrict__ xsums, MultiMeta m, PackedCfg c) {
+    uint32_t which = 0;
+    if (COUNT > 1 && blockIdx.x >= m.tile_end[0]) which = 1;
+    if (COUNT > 2 && blockIdx.x >= m.tile_end[1]) which = 2;
+    const uint32_t first = which == 0 ? 0 : m.tile_end[which - 1];
+    const uint8_t* __restrict__ wt = which == 0 ? t0 : which == 1 ? t1 : t2;
+    float* __restrict__ part = which == 0 ? p0 : which == 1 ? p1 : p2;
+    const uint32_t ct = blockIdx.x - first, N = m.N[which];
+    [[maybe_unused]] const uint32_t dtype = m.dtype[which];
+    const uint32_t slice = blockIdx.y * c.W + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t b0 = min(slice * c.bps, c.nblk), b1 = min(b0 + c.bps, c.nblk);
+    float acc[R];
+    if constexpr (MODE == kMixed) {
+        if (dtype == GUFFIN_Q4_K) run_blocks<GUFFIN_Q4_K, R>(wt, x, xsums, c.K, c.nblk, ct, b0, b1, acc);
+        else run_blocks<GUFFIN_Q6_K, R>(wt, x, xsums, c.K, c.nblk, ct, b0, b1, acc);
+    } else {
+        run_blocks<MODE, R>(wt, x, xsums, c.K, c.nblk, ct, b0, b1, acc);
+    }
+    finish_tile<R>(acc, part, N, ct, blockIdx.y, c.W);
 }
 
 int g_cus = 256;
 
-// k-slices: about four waves per SIMD over the whole chip (fine grains balance the
-// SIMDs and let compute start while later slices are still streaming); matrices with
-// more tiles than that walk K inside the wave with the next tile's loads in flight.
-uint32_t choose_slices(int dtype, uint32_t K, uint32_t N) {
-    const uint32_t nblk = K / block_elems(dtype), tiles = N / kTileCols;
-    const uint32_t target_waves = g_cus * 4 * 4;
-    uint32_t S = (target_waves + tiles - 1) / tiles;
-    if (S > nblk) S = nblk;
-    if (S > 64) S = 64;
-    if (S < 1) S = 1;
-    const uint32_t bps = (nblk + S - 1) / S;
-    return (nblk + bps - 1) / bps;  // no empty slices
+// Work split of a launch over `tiles` column tiles of `nblk` blocks each: blocks per wave so
+// that the chip holds about four waves per SIMD, waves per workgroup (k-slices reduced in LDS,
+// at most max_w) and planes (k-slices left to the consumer), preferring one workgroup per CU.
+struct Split { uint32_t bps, W, planes; };
+Split choose_split(uint32_t nblk, uint32_t tiles, uint32_t max_w) {
+    const uint64_t units = uint64_t(tiles) * nblk, target_waves = uint64_t(g_cus) * 16;
+    uint32_t bps = static_cast<uint32_t>((units + target_waves - 1) / target_waves);
+    if (bps < 1) bps = 1;
+    const uint32_t wpt = (nblk + bps - 1) / bps;  // waves per tile
+    uint32_t planes = (wpt + max_w - 1) / max_w;
+    if (tiles * planes * 4 < uint32_t(g_cus) * 3) {  // fewer workgroups than 3/4 of the CUs: split further
+        uint32_t want = (g_cus + tiles - 1) / tiles;
+        if (want > wpt) want = wpt;
+        if (want > planes) planes = want;
+    }
+    uint32_t W = (wpt + planes - 1) / planes;
+    planes = (wpt + W - 1) / W;
+    return {bps, W, planes};
 }
 
 template <int DTYPE>
 int launch_packed(hipStream_t s, const uint8_t* w, const float* x, const float* xsums, float* part,
-                  uint32_t rows, uint32_t K, uint32_t N, uint32_t S) {
-    const uint32_t nblk = K / block_elems(DTYPE), bps = (nblk + S - 1) / S;
-    const dim3 grid(N / kTileCols, S);
-    if (rows == 2)
-        hipLaunchKernelGGL((gemv_packed_kernel<DTYPE, 2>), grid, dim3(64), 0, s, w, x, xsums, part, K, N, nblk, bps);
-    else
-        hipLaunchKernelGGL((gemv_packed_kernel<DTYPE, 1>), grid, dim3(64), 0, s, w, x, xsums, part, K, N, nblk, bps);
+                  uint32_t rows, uint32_t K, uint32_t N) {
+    const uint32_t nblk = K / block_elems(DTYPE);
+    const Split sp = choose_split(nblk, N / kTileCols, max_waves(DTYPE));
+    const PackedCfg c {K, nblk, sp.bps, sp.W};
+    const dim3 grid(N / kTileCols, sp.planes), block(sp.W * 64);
+    if (rows == 2) hipLaunchKernelGGL((gemv_packed_kernel<DTYPE, 2>), grid, block, 0, s, w, x, xsums, part, N, c);
+    else hipLaunchKernelGGL((gemv_packed_kernel<DTYPE, 1>), grid, block, 0, s, w, x, xsums, part, N, c);
     return check_launch("gemv_packed");
 }
 
@@ -437,31 +482,67 @@ extern "C" int guffin_hip_group_sums(void* stream, const float* x, float* xsums,
 
 extern "C" uint32_t guffin_hip_gemv_packed_slices(int dtype, uint32_t K, uint32_t N) {
     if (check_packed_shape("gemv_packed_slices: need K % block == 0 and N % 64 == 0", dtype, K, N)) return 0;
-    return choose_slices(dtype, K, N);
+    return choose_split(K / block_elems(dtype), N / kTileCols, max_waves(dtype)).planes;
+}
+
+static int multi_split(const char* what, uint32_t count, const int* dtypes, const uint32_t* N, uint32_t K, Split* out, int* mode) {
+    if (!dtypes || !N) return fail(GUFFIN_E_ARG, what);
+    if (count == 0 || count > 3) return fail(GUFFIN_E_SHAPE, "gemv_packed_multi: 1 to 3 matrices");
+    uint32_t tiles = 0;
+    *mode = dtypes[0];
+    for (uint32_t i = 0; i < count; ++i) {
+        if (int rc = check_packed_shape("gemv_packed_multi: need K % block == 0 and N % 64 == 0", dtypes[i], K, N[i])) return rc;
+        if (dtypes[i] != dtypes[0]) *mode = kMixed;
+        if (block_elems(dtypes[i]) != block_elems(dtypes[0]))
+            return fail(GUFFIN_E_SHAPE, "gemv_packed_multi: matrices of one launch must share the block length");
+        tiles += N[i] / kTileCols;
+    }
+    *out = choose_split(K / block_elems(dtypes[0]), tiles, max_waves(*mode == kMixed ? GUFFIN_Q6_K : *mode));
+    return GUFFIN_OK;
+}
+
+extern "C" uint32_t guffin_hip_gemv_packed_multi_slices(uint32_t count, const int* dtypes, const uint32_t* N, uint32_t K) {
+    Split sp {};
+    int mode = 0;
+    if (multi_split("gemv_packed_multi_slices: null pointer", count, dtypes, N, K, &sp, &mode)) return 0;
+    return sp.planes;
 }
 
 extern "C" int guffin_hip_gemv_packed_multi(void* stream, uint32_t count, const int* dtypes, const void* const* tiles,
                                             const uint32_t* N, float* const* partials, const float* x,
                                             const float* xsums, uint32_t rows, uint32_t K) {
-    if (!dtypes || !tiles || !N || !partials || !x || !xsums) return fail(GUFFIN_E_ARG, "gemv_packed_multi: null pointer");
-    if (count == 0 || count > 3) return fail(GUFFIN_E_SHAPE, "gemv_packed_multi: 1 to 3 matrices");
+    if (!tiles || !partials || !x || !xsums) return fail(GUFFIN_E_ARG, "gemv_packed_multi: null pointer");
     if (rows == 0 || rows > 2) return fail(GUFFIN_E_SHAPE, "gemv_packed_multi: rows must be 1 or 2");
-    MultiArgs a {};
-    a.x = x; a.xsums = xsums; a.K = K; a.count = count;
-    uint32_t tile_end = 0, max_s = 1;
+    Split sp {};
+    int mode = 0;
+    if (int rc = multi_split("gemv_packed_multi: null pointer", count, dtypes, N, K, &sp, &mode)) return rc;
+    if (count == 1) {
+        if (!tiles[0] || !partials[0]) return fail(GUFFIN_E_ARG, "gemv_packed_multi: null pointer");
+        return guffin_hip_gemv_packed(stream, dtypes[0], tiles[0], x, xsums, partials[0], nullptr, rows, K, N[0]);
+    }
+    MultiMeta m {};
+    const uint8_t* t[3] = {nullptr, nullptr, nullptr};
+    float* p[3] = {nullptr, nullptr, nullptr};
+    uint32_t tile_end = 0;
     for (uint32_t i = 0; i < count; ++i) {
         if (!tiles[i] || !partials[i]) return fail(GUFFIN_E_ARG, "gemv_packed_multi: null pointer");
-        if (int rc = check_packed_shape("gemv_packed_multi: need K % block == 0 and N % 64 == 0", dtypes[i], K, N[i])) return rc;
         if (reinterpret_cast<uintptr_t>(tiles[i]) & 15u) return fail(GUFFIN_E_ALIGN, "gemv_packed_multi: tiles must be 16-byte aligned");
-        const uint32_t S = choose_slices(dtypes[i], K, N[i]), nblk = K / block_elems(dtypes[i]);
         tile_end += N[i] / kTileCols;
-        a.m[i] = PackedMat {static_cast<const uint8_t*>(tiles[i]), partials[i], N[i], static_cast<uint32_t>(dtypes[i]),
-                            S, (nblk + S - 1) / S, tile_end};
-        if (S > max_s) max_s = S;
+        m.N[i] = N[i]; m.dtype[i] = static_cast<uint32_t>(dtypes[i]); m.tile_end[i] = tile_end;
+        t[i] = static_cast<const uint8_t*>(tiles[i]); p[i] = partials[i];
     }
-    const dim3 grid(tile_end, max_s);
-    if (rows == 2) hipLaunchKernelGGL(gemv_packed_multi_kernel<2>, grid, dim3(64), 0, as_stream(stream), a);
-    else hipLaunchKernelGGL(gemv_packed_multi_kernel<1>, grid, dim3(64), 0, as_stream(stream), a);
+    for (uint32_t i = count; i < 3; ++i) { t[i] = t[0]; p[i] = p[0]; m.tile_end[i] = tile_end; m.N[i] = m.N[0]; m.dtype[i] = m.dtype[0]; }
+    const PackedCfg c {K, K / block_elems(dtypes[0]), sp.bps, sp.W};
+    const dim3 grid(tile_end, sp.planes), block(sp.W * 64);
+    hipStream_t s = as_stream(stream);
+#define GUFFIN_MULTI(R_, C_, M_) hipLaunchKernelGGL((gemv_packed_multi_kernel<R_, C_, M_>), grid, block, 0, s, t[0], t[1], t[2], p[0], p[1], p[2], x, xsums, m, c)
+#define GUFFIN_MULTI_MODE(R_, C_) do { \
+        if (mode == GUFFIN_Q4_K) GUFFIN_MULTI(R_, C_, GUFFIN_Q4_K); else if (mode == GUFFIN_Q6_K) GUFFIN_MULTI(R_, C_, GUFFIN_Q6_K); \
+        else if (mode == GUFFIN_Q8_0) GUFFIN_MULTI(R_, C_, GUFFIN_Q8_0); else GUFFIN_MULTI(R_, C_, kMixed); } while (0)
+    if (rows == 2) { if (count == 3) GUFFIN_MULTI_MODE(2, 3); else GUFFIN_MULTI_MODE(2, 2); }
+    else { if (count == 3) GUFFIN_MULTI_MODE(1, 3); else GUFFIN_MULTI_MODE(1, 2); }
+#undef GUFFIN_MULTI_MODE
+#undef GUFFIN_MULTI
     return check_launch("gemv_packed_multi");
 }
 
@@ -473,13 +554,13 @@ extern "C" int guffin_hip_gemv_packed(void* stream, int dtype, const void* tiles
     if (reinterpret_cast<uintptr_t>(tiles) & 15u) return fail(GUFFIN_E_ALIGN, "gemv_packed: tiles must be 16-byte aligned");
     if ((reinterpret_cast<uintptr_t>(x) & 3u) || (reinterpret_cast<uintptr_t>(xsums) & 3u) || (reinterpret_cast<uintptr_t>(partials) & 3u))
         return fail(GUFFIN_E_ALIGN, "gemv_packed: fp32 pointers must be 4-byte aligned");
-    const uint32_t S = choose_slices(dtype, K, N);
+    const uint32_t S = choose_split(K / block_elems(dtype), N / kTileCols, max_waves(dtype)).planes;
     const uint8_t* w = static_cast<const uint8_t*>(tiles);
     hipStream_t s = as_stream(stream);
     int rc;
-    if (dtype == GUFFIN_Q4_K) rc = launch_packed<GUFFIN_Q4_K>(s, w, x, xsums, partials, rows, K, N, S);
-    else if (dtype == GUFFIN_Q6_K) rc = launch_packed<GUFFIN_Q6_K>(s, w, x, xsums, partials, rows, K, N, S);
-    else rc = launch_packed<GUFFIN_Q8_0>(s, w, x, xsums, partials, rows, K, N, S);
+    if (dtype == GUFFIN_Q4_K) rc = launch_packed<GUFFIN_Q4_K>(s, w, x, xsums, partials, rows, K, N);
+    else if (dtype == GUFFIN_Q6_K) rc = launch_packed<GUFFIN_Q6_K>(s, w, x, xsums, partials, rows, K, N);
+    else rc = launch_packed<GUFFIN_Q8_0>(s, w, x, xsums, partials, rows, K, N);
     if (rc || !y) return rc;
     const uint32_t count = rows * N;
     hipLaunchKernelGGL(reduce_partials_kernel, dim3((count + 255) / 256), dim3(256), 0, s, partials, y, S, count);

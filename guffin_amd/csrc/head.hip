@@ -10,8 +10,8 @@
 // candidate order and keys are unique, so selection is a pure comparison network and the
 // result is exact including ties.
 //   stage 1  every workgroup sorts a 2048-logit tile in LDS (bitonic) and keeps its best R
-//   stage 2  one workgroup per row merges the G*R survivors (bitonic, in rounds if needed),
-//            writes the best `retain`, then appends the logits of the history tokens
+//   stage 2  one workgroup per row picks the best `retain` of the G*R survivors (radix select
+//            plus a rank sort), then appends the logits of the history tokens
 // A global top-R entry is necessarily a top-R entry of its own tile, so the two stages lose
 // nothing.
 #include "common.hpp"
@@ -20,7 +20,6 @@ namespace guffin {
 namespace {
 
 constexpr uint32_t kTile = 2048;          // logits per stage-1 workgroup
-constexpr uint32_t kMergeCap = 16384;     // keys a stage-2 round sorts in LDS (128 KiB)
 
 __device__ __forceinline__ uint64_t make_key(float logit, uint32_t token) {
     const uint32_t b = __float_as_uint(logit + 0.0f);  // -0 orders as +0, as a float comparison does
@@ -79,26 +78,78 @@ struct Candidates {  // layout of one row of the result (sampling.hpp:57-61 plus
     struct { uint32_t token; float logit; } values[384];
 };
 
+// Stage 2: exact selection of the best `retain` of n unique keys by an 8-pass radix select
+// (one byte per pass, most significant first: a 256-bin histogram in LDS, then the bin that
+// holds the retain-th largest key), followed by a rank sort of the selected keys.
 __global__ void __launch_bounds__(1024)
 topk_merge_kernel(const float* __restrict__ logits, const uint64_t* __restrict__ survivors, uint32_t n_survivors,
                   uint32_t vocab, uint32_t retain, float divisor, const uint32_t* __restrict__ history,
                   const uint32_t* __restrict__ history_count, Candidates* __restrict__ result,
                   uint32_t* __restrict__ status) {
-    extern __shared__ uint64_t keys[];  // kMergeCap
-    const uint32_t row = blockIdx.x;
+    __shared__ uint32_t hist[256];
+    __shared__ uint64_t sel[512];
+    __shared__ uint64_t keys[512];  // selected keys in candidate order
+    __shared__ uint32_t s_bin, s_above, s_count;
+    const uint32_t row = blockIdx.x, lane = threadIdx.x & 63;
     const uint64_t* src = survivors + size_t(row) * n_survivors;
-    // round 0 sorts the first chunk; later rounds merge the running best `retain` with the next chunk
-    uint32_t done = 0, have = 0;
-    while (done < n_survivors) {
-        const uint32_t room = kMergeCap - have;
-        const uint32_t take = n_survivors - done < room ? n_survivors - done : room;
-        uint32_t n = 1;
-        while (n < have + take) n <<= 1;
-        for (uint32_t i = threadIdx.x; i < n - have; i += blockDim.x) keys[have + i] = i < take ? src[done + i] : 0;
-        bitonic_desc(keys, n);
-        done += take;
-        have = retain < n ? retain : n;
+    uint64_t prefix = 0;
+    uint32_t remaining = retain;  // rank of the wanted key among the keys that match `prefix`
+    for (int pass = 0; pass < 8; ++pass) {
+        const int shift = 56 - 8 * pass;
+        for (uint32_t i = threadIdx.x; i < 256; i += blockDim.x) hist[i] = 0;
+        __syncthreads();
+        for (uint32_t i = threadIdx.x; i < n_survivors; i += blockDim.x) {
+            const uint64_t k = src[i];
+            if (pass == 0 || (k >> (shift + 8)) == prefix) atomicAdd(&hist[(k >> shift) & 255u], 1u);
+        }
+        __syncthreads();
+        if (threadIdx.x < 64) {  // lane l owns bins 255-4l .. 252-4l, highest first
+            uint32_t c[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) c[j] = hist[255 - 4 * lane - j];
+            const uint32_t mine = c[0] + c[1] + c[2] + c[3];
+            uint32_t incl = mine;
+#pragma unroll
+            for (int d = 1; d < 64; d <<= 1) {
+                const uint32_t o = __shfl_up(incl, d, kWave);
+                if (lane >= uint32_t(d)) incl += o;
+            }
+            uint32_t above = incl - mine;
+            if (above < remaining && remaining <= incl) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    if (remaining <= above + c[j]) { s_bin = 255 - 4 * lane - j; s_above = above; break; }
+                    above += c[j];
+                }
+            }
+        }
+        __syncthreads();
+        prefix = (prefix << 8) | s_bin;
+        remaining -= s_above;
+        __syncthreads();
     }
+    // `prefix` is the retain-th largest key; keys above it are taken, then `remaining` copies of it
+    // (more than one only for the zero padding of a short last tile)
+    if (threadIdx.x == 0) s_count = 0;
+    __syncthreads();
+    for (uint32_t i = threadIdx.x; i < n_survivors; i += blockDim.x) {
+        const uint64_t k = src[i];
+        if (k > prefix) sel[atomicAdd(&s_count, 1u)] = k;
+    }
+    __syncthreads();
+    const uint32_t above_total = s_count;
+    for (uint32_t i = threadIdx.x; i < remaining; i += blockDim.x) sel[above_total + i] = prefix;
+    __syncthreads();
+    for (uint32_t i = threadIdx.x; i < retain; i += blockDim.x) {
+        const uint64_t k = sel[i];
+        uint32_t rank = 0;
+        for (uint32_t j = 0; j < retain; ++j) {
+            const uint64_t o = sel[j];
+            rank += (o > k) || (o == k && j < i);
+        }
+        keys[rank] = k;
+    }
+    __syncthreads();
     Candidates& out = result[row];
     const uint32_t hc = history_count ? history_count[row] : 0;
     for (uint32_t i = threadIdx.x; i < retain; i += blockDim.x) {
@@ -183,10 +234,7 @@ argmax_final_kernel(const uint64_t* __restrict__ partial, uint32_t n, uint32_t* 
 
 }  // namespace
 
-int head_init() {
-    return hipFuncSetAttribute(reinterpret_cast<const void*>(topk_merge_kernel),
-                               hipFuncAttributeMaxDynamicSharedMemorySize, kMergeCap * 8) != hipSuccess;
-}
+int head_init() { return 0; }
 
 }  // namespace guffin
 
@@ -224,7 +272,7 @@ int guffin::select_candidates_scaled(hipStream_t s, const float* logits, uint32_
     uint64_t* surv = static_cast<uint64_t*>(workspace);
     hipLaunchKernelGGL(topk_tile_kernel, dim3(tiles, rows), dim3(1024), 0, s, logits, surv, vocab, keep, divisor, status);
     if (int rc = check_launch("select_candidates(tile)")) return rc;
-    hipLaunchKernelGGL(topk_merge_kernel, dim3(rows), dim3(1024), kMergeCap * 8, s, logits, surv, tiles * keep, vocab,
+    hipLaunchKernelGGL(topk_merge_kernel, dim3(rows), dim3(1024), 0, s, logits, surv, tiles * keep, vocab,
                        keep, divisor, history, history_count, static_cast<Candidates*>(result), status);
     return check_launch("select_candidates(merge)");
 }

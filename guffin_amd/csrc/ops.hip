@@ -29,9 +29,17 @@ __device__ __forceinline__ float block_sum(float v, float* scratch) {
     return t;
 }
 
+// Sum of `planes` partial planes in plane order; loads are issued four at a time so that the
+// adds, not the memory latency, form the dependent chain.
 __device__ __forceinline__ float load_planes(const float* p, uint32_t planes, size_t plane_stride) {
     float v = p[0];
-    for (uint32_t s = 1; s < planes; ++s) v += p[s * plane_stride];
+    uint32_t s = 1;
+    for (; s + 4 <= planes; s += 4) {
+        const float a = p[s * plane_stride], b = p[(s + 1) * plane_stride], c = p[(s + 2) * plane_stride],
+                    d = p[(s + 3) * plane_stride];
+        v += a; v += b; v += c; v += d;
+    }
+    for (; s < planes; ++s) v += p[s * plane_stride];
     return v;
 }
 
@@ -52,24 +60,55 @@ __device__ __forceinline__ void emit_group_sums(const float* row, float* sums, u
     }
 }
 
+// Loads the row (summing partial planes) into LDS and returns this thread's share of the
+// squared sum.  Four columns per thread are in flight at a time, plane loads in batches of
+// four, so a row of a few thousand columns costs two or three memory round trips.
+__device__ __forceinline__ float stage_row(const float* __restrict__ xr, uint32_t planes, size_t plane_stride,
+                                           float* row, uint32_t width) {
+    float ss = 0.f;
+    const uint32_t step = blockDim.x;
+    for (uint32_t c0 = threadIdx.x; c0 < width; c0 += 4 * step) {
+        float v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) v[u] = c0 + u * step < width ? xr[c0 + u * step] : 0.f;
+        uint32_t s = 1;
+        for (; s + 4 <= planes; s += 4) {
+            float t[4][4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+#pragma unroll
+                for (int k = 0; k < 4; ++k) t[u][k] = c0 + u * step < width ? xr[(s + k) * plane_stride + c0 + u * step] : 0.f;
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+#pragma unroll
+                for (int k = 0; k < 4; ++k) v[u] += t[u][k];
+        }
+        for (; s < planes; ++s) {
+            float t[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) t[u] = c0 + u * step < width ? xr[s * plane_stride + c0 + u * step] : 0.f;
+#pragma unroll
+            for (int u = 0; u < 4; ++u) v[u] += t[u];
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+            if (c0 + u * step < width) { row[c0 + u * step] = v[u]; ss = fmaf(v[u], v[u], ss); }
+    }
+    return ss;
+}
+
 // y = x * rsqrt(mean(x^2) + eps) * gamma [+ residual]; one workgroup per row.
 // x may be `planes` partial planes.  Optional outputs: y_sums (group sums of y).
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(1024)
 rms_norm_kernel(const float* __restrict__ x, uint32_t planes, size_t plane_stride,
                 const float* __restrict__ gamma, const float* __restrict__ residual,
                 float* __restrict__ y, float* __restrict__ y_sums, uint32_t width, float eps,
                 uint32_t* __restrict__ status) {
-    extern __shared__ float lds[];  // [width] row image + [4] scratch
+    extern __shared__ float lds[];  // [width] row image + [16] scratch
     float* row = lds;
     float* scratch = lds + width;
     const uint32_t r = blockIdx.x;
-    const float* xr = x + size_t(r) * width;
-    float ss = 0.f;
-    for (uint32_t c = threadIdx.x; c < width; c += blockDim.x) {
-        const float v = load_planes(xr + c, planes, plane_stride);
-        row[c] = v;
-        ss = fmaf(v, v, ss);
-    }
+    const float ss = stage_row(x + size_t(r) * width, planes, plane_stride, row, width);
     const float total = block_sum(ss, scratch);
     const float inv = 1.0f / sqrtf(total / static_cast<float>(width) + eps);
     bool bad = false;
@@ -90,7 +129,7 @@ rms_norm_kernel(const float* __restrict__ x, uint32_t planes, size_t plane_strid
 // Fused tail of one sub-block and head of the next:
 //   out_residual = residual + rms(x, gamma_post);  out_norm = rms(out_residual, gamma_next)
 // (reference order: encode_rms_norm_add then encode_rms_norm, gemma_target_runtime.cpp:156-173, 201-213)
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(1024)
 rms_norm_add_norm_kernel(const float* __restrict__ x, uint32_t planes, size_t plane_stride,
                          const float* __restrict__ gamma_post, const float* __restrict__ residual,
                          float* __restrict__ out_residual, const float* __restrict__ gamma_next,
@@ -100,13 +139,7 @@ rms_norm_add_norm_kernel(const float* __restrict__ x, uint32_t planes, size_t pl
     float* row = lds;
     float* scratch = lds + width;
     const uint32_t r = blockIdx.x;
-    const float* xr = x + size_t(r) * width;
-    float ss = 0.f;
-    for (uint32_t c = threadIdx.x; c < width; c += blockDim.x) {
-        const float v = load_planes(xr + c, planes, plane_stride);
-        row[c] = v;
-        ss = fmaf(v, v, ss);
-    }
+    float ss = stage_row(x + size_t(r) * width, planes, plane_stride, row, width);
     float total = block_sum(ss, scratch);
     float inv = 1.0f / sqrtf(total / static_cast<float>(width) + eps);
     ss = 0.f;
@@ -159,7 +192,18 @@ __device__ __forceinline__ void rope_sincos(uint32_t position, uint32_t pair, ui
 // One wave per (row, head); q heads first, then k heads, then v heads.  Any of the three
 // sections can be disabled with a null pointer; q_norm/k_norm null skips the head norm.
 // Inputs may be `planes` partial planes of a GEMV.
+// cos/sin of every (row, pair) once per forward pass: table[row][pair] = {cos, sin}
+__global__ void rope_table_kernel(const uint32_t* positions, float2* table, uint32_t rows, uint32_t rope_dim,
+                                  float base, float scale) {
+    const uint32_t half = rope_dim / 2, i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= rows * half) return;
+    float c, s;
+    rope_sincos(positions[i / half], i % half, rope_dim, base, scale, c, s);
+    table[i] = make_float2(c, s);
+}
+
 struct QkvArgs {
+    const float2* rope_table;  // optional [rows][rope_dim/2] from rope_table_kernel; else computed here
     const float* q_raw; const float* k_raw; const float* v_raw;
     uint32_t q_planes, k_planes, v_planes; size_t q_plane_stride, k_plane_stride, v_plane_stride;
     const float* q_norm; const float* k_norm;
@@ -207,17 +251,8 @@ __global__ void __launch_bounds__(64) qkv_post_kernel(QkvArgs a) {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    const uint32_t half = a.rope_dim / 2, pos = a.positions[r];
-    for (uint32_t c = lane; c < a.head_dim; c += 64) {
-        float v = lds[c];
-        if (c < a.rope_dim) {
-            const uint32_t pair = c % half;
-            float cs, sn;
-            rope_sincos(pos, pair, a.rope_dim, a.base, a.scale, cs, sn);
-            const float first = lds[pair], second = lds[pair + half];
-            v = c < half ? __fsub_rn(__fmul_rn(first, cs), __fmul_rn(second, sn))
-                         : __fadd_rn(__fmul_rn(first, sn), __fmul_rn(second, cs));
-        }
+    const uint32_t half = a.rope_dim / 2, pos = a.rope_table ? 0u : a.positions[r];
+    auto emit = [&](uint32_t c, float v) {
         if (is_q) {
             a.q_out[off + c] = v;
         } else {
@@ -225,7 +260,16 @@ __global__ void __launch_bounds__(64) qkv_post_kernel(QkvArgs a) {
             bad |= !isfinite(static_cast<float>(hv));
             a.k_out[off + c] = __builtin_bit_cast(uint16_t, hv);
         }
+    };
+    for (uint32_t pair = lane; pair < half; pair += 64) {
+        float cs, sn;
+        if (a.rope_table) { const float2 t = a.rope_table[size_t(r) * half + pair]; cs = t.x; sn = t.y; }
+        else rope_sincos(pos, pair, a.rope_dim, a.base, a.scale, cs, sn);
+        const float first = lds[pair], second = lds[pair + half];
+        emit(pair, __fsub_rn(__fmul_rn(first, cs), __fmul_rn(second, sn)));
+        emit(pair + half, __fadd_rn(__fmul_rn(first, sn), __fmul_rn(second, cs)));
     }
+    for (uint32_t c = a.rope_dim + lane; c < a.head_dim; c += 64) emit(c, lds[c]);
     if (bad && a.status) atomicOr(a.status, GUFFIN_STATUS_KV_NONFINITE);
 }
 
@@ -335,6 +379,12 @@ __global__ void kv_scatter_kernel(const uint16_t* __restrict__ priv_k, const uin
     }
 }
 
+// one thread per four columns, whole waves, at most 1024 threads
+uint32_t norm_threads(uint32_t width) {
+    const uint32_t t = ((width + 3) / 4 + 63) / 64 * 64;
+    return t < 64 ? 64 : t > 1024 ? 1024 : t;
+}
+
 bool aligned4(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 3u) == 0; }
 
 }  // namespace
@@ -360,9 +410,9 @@ extern "C" int guffin_hip_rms_norm(void* stream, const float* x, uint32_t planes
     if (y_sums && width % 32 != 0) return fail(GUFFIN_E_SHAPE, "rms_norm: group sums need width % 32 == 0");
     if (!(eps > 0.f)) return fail(GUFFIN_E_ARG, "rms_norm: epsilon must be positive");
     if (!aligned4(x) || !aligned4(y) || !aligned4(gamma)) return fail(GUFFIN_E_ALIGN, "rms_norm: fp32 pointers must be 4-byte aligned");
-    const size_t lds = (size_t(width) + 8) * 4;
+    const size_t lds = (size_t(width) + 16) * 4;
     if (lds > 160 * 1024) return fail(GUFFIN_E_CAPACITY, "rms_norm: row does not fit in LDS");
-    hipLaunchKernelGGL(rms_norm_kernel, dim3(rows), dim3(256), lds, as_stream(stream), x, planes,
+    hipLaunchKernelGGL(rms_norm_kernel, dim3(rows), dim3(norm_threads(width)), lds, as_stream(stream), x, planes,
                        static_cast<size_t>(plane_stride), gamma, residual, y, y_sums, width, eps, status);
     return check_launch("rms_norm");
 }
@@ -376,9 +426,9 @@ extern "C" int guffin_hip_rms_norm_add_norm(void* stream, const float* x, uint32
     if (rows == 0 || width == 0 || planes == 0) return fail(GUFFIN_E_SHAPE, "rms_norm_add_norm: empty shape");
     if (out_sums && width % 32 != 0) return fail(GUFFIN_E_SHAPE, "rms_norm_add_norm: group sums need width % 32 == 0");
     if (!(eps > 0.f)) return fail(GUFFIN_E_ARG, "rms_norm_add_norm: epsilon must be positive");
-    const size_t lds = (size_t(width) + 8) * 4;
+    const size_t lds = (size_t(width) + 16) * 4;
     if (lds > 160 * 1024) return fail(GUFFIN_E_CAPACITY, "rms_norm_add_norm: row does not fit in LDS");
-    hipLaunchKernelGGL(rms_norm_add_norm_kernel, dim3(rows), dim3(256), lds, as_stream(stream), x, planes,
+    hipLaunchKernelGGL(rms_norm_add_norm_kernel, dim3(rows), dim3(norm_threads(width)), lds, as_stream(stream), x, planes,
                        static_cast<size_t>(plane_stride), gamma_post, residual, out_residual, gamma_next,
                        out_norm, out_sums, width, eps, status);
     return check_launch("rms_norm_add_norm");
@@ -394,10 +444,10 @@ extern "C" int guffin_hip_head_rms_norm(void* stream, const float* x, const floa
 }
 
 static int launch_qkv(void* stream, const QkvArgs& a) {
-    if (!a.positions) return fail(GUFFIN_E_ARG, "rope/kv: null positions");
+    if (!a.positions && !a.rope_table) return fail(GUFFIN_E_ARG, "rope/kv: null positions");
     if (a.rows == 0 || a.head_dim == 0 || a.head_dim > 4096) return fail(GUFFIN_E_SHAPE, "rope/kv: bad head shape");
     if (a.rope_dim > a.head_dim || (a.rope_dim & 1u)) return fail(GUFFIN_E_SHAPE, "rope/kv: rope_dim must be even and <= head_dim");
-    if (a.rope_dim && !(a.base > 0.f)) return fail(GUFFIN_E_ARG, "rope/kv: frequency base must be positive");
+    if (a.rope_dim && !a.rope_table && !(a.base > 0.f)) return fail(GUFFIN_E_ARG, "rope/kv: frequency base must be positive");
     const uint32_t blocks = a.rows * (a.q_heads + 2 * a.kv_heads);
     if (blocks == 0) return fail(GUFFIN_E_SHAPE, "rope/kv: no heads");
     hipLaunchKernelGGL(qkv_post_kernel, dim3(blocks), dim3(64), a.head_dim * sizeof(float), as_stream(stream), a);
@@ -433,8 +483,10 @@ extern "C" int guffin_hip_qkv_post(void* stream, const float* q_raw, const float
                                    uint64_t v_plane_stride, const float* q_norm, const float* k_norm,
                                    const uint32_t* positions, float* q_out, void* k_out, void* v_out,
                                    uint32_t rows, uint32_t q_heads, uint32_t kv_heads, uint32_t head_dim,
-                                   uint32_t rope_dim, float freq_base, float freq_scale, float eps, uint32_t* status) {
+                                   uint32_t rope_dim, float freq_base, float freq_scale, float eps,
+                                   const float* rope_table, uint32_t* status) {
     if (!q_raw || !k_raw || !v_raw || !q_out || !k_out || !v_out) return fail(GUFFIN_E_ARG, "qkv_post: null pointer");
+    if (!rope_table && !positions) return fail(GUFFIN_E_ARG, "qkv_post: need positions or a rope table");
     if (q_planes == 0 || k_planes == 0 || v_planes == 0) return fail(GUFFIN_E_SHAPE, "qkv_post: planes must be >= 1");
     if (!(eps > 0.f)) return fail(GUFFIN_E_ARG, "qkv_post: epsilon must be positive");
     QkvArgs a {};
@@ -444,7 +496,19 @@ extern "C" int guffin_hip_qkv_post(void* stream, const float* q_raw, const float
     a.q_out = q_out; a.k_out = static_cast<uint16_t*>(k_out); a.v_out = static_cast<uint16_t*>(v_out);
     a.rows = rows; a.q_heads = q_heads; a.kv_heads = kv_heads; a.head_dim = head_dim; a.rope_dim = rope_dim;
     a.base = freq_base; a.scale = freq_scale; a.eps = eps; a.status = status;
+    a.rope_table = reinterpret_cast<const float2*>(rope_table);
     return launch_qkv(stream, a);
+}
+
+extern "C" int guffin_hip_rope_table(void* stream, const uint32_t* positions, float* table, uint32_t rows,
+                                     uint32_t rope_dim, float freq_base, float freq_scale) {
+    if (!positions || !table) return fail(GUFFIN_E_ARG, "rope_table: null pointer");
+    if (rows == 0 || rope_dim == 0 || rope_dim % 2) return fail(GUFFIN_E_SHAPE, "rope_table: rope_dim must be even and rows >= 1");
+    if (reinterpret_cast<uintptr_t>(table) & 7u) return fail(GUFFIN_E_ALIGN, "rope_table: table must be 8-byte aligned");
+    const uint32_t n = rows * (rope_dim / 2);
+    hipLaunchKernelGGL(rope_table_kernel, dim3((n + 63) / 64), dim3(64), 0, as_stream(stream), positions,
+                       reinterpret_cast<float2*>(table), rows, rope_dim, freq_base, freq_scale);
+    return check_launch("rope_table");
 }
 
 extern "C" int guffin_hip_geglu(void* stream, const float* gate, const float* up, uint32_t planes, uint64_t plane_stride,

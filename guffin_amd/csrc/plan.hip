@@ -34,12 +34,21 @@ struct Scratch {
     float *x, *x1, *u, *us, *q, *a, *as, *h, *hs;
     float *part_a, *part_b, *part_c;          // GEMV partial planes (largest users: gate / up / down)
     float *attn_out, *attn_ml;
+    float *rope_local, *rope_global;          // [rows][head_dim/2][2] cos/sin per frequency base
     uint32_t *positions, *ancestors, *schedule;
     uint64_t bytes;
 };
 
 uint32_t slices(int dtype, uint32_t K, uint32_t N) { return guffin_hip_gemv_packed_slices(dtype, K, N); }
 uint64_t sums_len(uint32_t width) { return width / 16 + width / 32; }
+uint32_t qkv_slices(const guffin_layer_desc& L, uint32_t H, uint32_t QW, uint32_t KW) {
+    const uint32_t n[3] = {QW, KW, KW};
+    return guffin_hip_gemv_packed_multi_slices(3, L.dtype, n, H);
+}
+uint32_t ffn_slices(const guffin_layer_desc& L, uint32_t H, uint32_t F) {
+    const uint32_t n[2] = {F, F};
+    return guffin_hip_gemv_packed_multi_slices(2, L.dtype + 4, n, H);
+}
 
 bool is_local(const guffin_model_desc& m, uint32_t layer) {
     return m.global_period > 1 && (layer % m.global_period) != m.global_period - 1;
@@ -72,9 +81,10 @@ Scratch layout(const guffin_model_desc& m, uint32_t rows, uint32_t position, uin
     for (uint32_t l = 0; l < m.layer_count; ++l) {
         const guffin_layer_desc& L = m.layers[l];
         auto need = [&](int i, uint32_t K, uint32_t N) { return uint64_t(slices(L.dtype[i], K, N)) * rows * N; };
-        pa = std::max({pa, need(0, H, QW), need(3, QW, H), need(4, H, F), need(6, F, H)});
-        pb = std::max({pb, need(1, H, KW), need(5, H, F)});
-        pc = std::max(pc, need(2, H, KW));
+        const uint64_t sq = qkv_slices(L, H, QW, KW), sf = ffn_slices(L, H, F);
+        pa = std::max({pa, sq * rows * QW, need(3, QW, H), sf * rows * F, need(6, F, H)});
+        pb = std::max({pb, sq * rows * KW, sf * rows * F});
+        pc = std::max(pc, sq * rows * KW);
     }
     s.part_a = ar.take<float>(pa);
     s.part_b = ar.take<float>(pb);
@@ -84,6 +94,8 @@ Scratch layout(const guffin_model_desc& m, uint32_t rows, uint32_t position, uin
         max_parts = std::max(max_parts, guffin_hip_attention_partitions(max_tokens_for(m, l, position, rows), m.kv_heads));
     s.attn_out = ar.take<float>(uint64_t(rows) * m.q_heads * max_parts * m.head_dim);
     s.attn_ml = ar.take<float>(uint64_t(rows) * m.q_heads * max_parts * 2);
+    s.rope_local = ar.take<float>(uint64_t(rows) * m.head_dim);
+    s.rope_global = ar.take<float>(uint64_t(rows) * m.head_dim);
     s.positions = ar.take<uint32_t>(rows);
     s.ancestors = ar.take<uint32_t>(rows);
     s.schedule = ar.take<uint32_t>(uint64_t(m.layer_count) * rows * 4);
@@ -128,6 +140,8 @@ int forward_rows(hipStream_t stream, const guffin_model_desc& m, const uint32_t*
     hipLaunchKernelGGL(stage_rows_kernel, dim3((n_sched + 63) / 64), dim3(64), 0, stream, s.positions, s.ancestors,
                        s.schedule, rows, position, m.layer_count, m.sliding_window, m.global_period);
     GUFFIN_TRY(check_launch("stage_rows"));
+    GUFFIN_TRY(guffin_hip_rope_table(st, s.positions, s.rope_local, rows, m.head_dim, m.local_base, 1.0f));
+    GUFFIN_TRY(guffin_hip_rope_table(st, s.positions, s.rope_global, rows, m.head_dim, m.global_base, m.global_scale));
     GUFFIN_TRY(guffin_hip_embed(st, m.embed_dtype, m.embed_rows, tokens, s.x, rows, H,
                                 std::sqrt(static_cast<float>(H)), m.vocab, status));
     GUFFIN_TRY(guffin_hip_rms_norm(st, s.x, 1, 0, m.layers[0].norm[0], nullptr, s.u, s.us, rows, H, m.eps, status));
@@ -144,10 +158,12 @@ int forward_rows(hipStream_t stream, const guffin_model_desc& m, const uint32_t*
             const uint32_t n[3] = {QW, KW, KW};
             float* parts[3] = {s.part_a, s.part_b, s.part_c};
             GUFFIN_TRY(guffin_hip_gemv_packed_multi(st, 3, dt, tl, n, parts, s.u, s.us, rows, H));
-            GUFFIN_TRY(guffin_hip_qkv_post(st, s.part_a, s.part_b, s.part_c, slices(dt[0], H, QW), slices(dt[1], H, KW),
-                                           slices(dt[2], H, KW), uint64_t(rows) * QW, uint64_t(rows) * KW,
+            const uint32_t sq = qkv_slices(L, H, QW, KW);
+            if (sq == 0) return fail(GUFFIN_E_SHAPE, "forward: q, k and v must share the block length");
+            GUFFIN_TRY(guffin_hip_qkv_post(st, s.part_a, s.part_b, s.part_c, sq, sq, sq, uint64_t(rows) * QW, uint64_t(rows) * KW,
                                            uint64_t(rows) * KW, L.norm[1], L.norm[2], s.positions, s.q, pk, pv, rows,
-                                           m.q_heads, m.kv_heads, m.head_dim, m.head_dim, base, scale, m.eps, status));
+                                           m.q_heads, m.kv_heads, m.head_dim, m.head_dim, base, scale, m.eps,
+                                           local ? s.rope_local : s.rope_global, status));
         }
         GUFFIN_TRY(guffin_hip_attention_decode(st, s.q, L.ring_k, L.ring_v, pk, pv, s.schedule + size_t(l) * rows * 4,
                                                s.ancestors, s.a, s.as, s.attn_out, s.attn_ml, rows, rows,
@@ -163,8 +179,7 @@ int forward_rows(hipStream_t stream, const guffin_model_desc& m, const uint32_t*
             const uint32_t n[2] = {F, F};
             float* parts[2] = {s.part_a, s.part_b};
             GUFFIN_TRY(guffin_hip_gemv_packed_multi(st, 2, dt, tl, n, parts, s.u, s.us, rows, H));
-            if (slices(dt[0], H, F) != slices(dt[1], H, F)) return fail(GUFFIN_E_SHAPE, "forward: gate and up must use the same block type");
-            GUFFIN_TRY(guffin_hip_geglu(st, s.part_a, s.part_b, slices(dt[0], H, F), uint64_t(rows) * F, s.h, s.hs, rows, F));
+            GUFFIN_TRY(guffin_hip_geglu(st, s.part_a, s.part_b, ffn_slices(L, H, F), uint64_t(rows) * F, s.h, s.hs, rows, F));
         }
         GUFFIN_TRY(guffin_hip_gemv_packed(st, L.dtype[6], L.tiles[6], s.h, s.hs, s.part_a, nullptr, rows, F, H));
         // x = x1 + rms(down, post_ffw_norm); u = rms(x, next block's attn_norm | output_norm)

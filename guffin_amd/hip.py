@@ -174,7 +174,7 @@ def kv_store_f16(raw_k, raw_v, positions, heads, head_dim, rope_dim, base, scale
 
 
 def qkv_post(q_raw, k_raw, v_raw, q_norm, k_norm, positions, rows, q_heads, kv_heads, head_dim, rope_dim, base,
-             scale=1.0, eps=1e-6, planes=None, status=None):
+             scale=1.0, eps=1e-6, planes=None, status=None, table=None):
     pl = planes or 1
     strides = [t[0].numel() if planes else 0 for t in (q_raw, k_raw, v_raw)]
     q = _f32((rows, q_heads * head_dim), q_raw)
@@ -183,8 +183,34 @@ def qkv_post(q_raw, k_raw, v_raw, q_norm, k_norm, positions, rows, q_heads, kv_h
     check(lib().guffin_hip_qkv_post(_stream(), _p(q_raw), _p(k_raw), _p(v_raw), pl, pl, pl, C.c_uint64(strides[0]),
                                     C.c_uint64(strides[1]), C.c_uint64(strides[2]), _p(q_norm), _p(k_norm),
                                     _p(positions), _p(q), _p(k), _p(v), rows, q_heads, kv_heads, head_dim,
-                                    rope_dim, C.c_float(base), C.c_float(scale), C.c_float(eps), _p(status)))
+                                    rope_dim, C.c_float(base), C.c_float(scale), C.c_float(eps), _p(table),
+                                    _p(status)))
     return q, k, v
+
+
+def rope_table(positions, rope_dim, base, scale=1.0):
+    rows = positions.numel()
+    table = torch.empty((rows, rope_dim // 2, 2), dtype=torch.float32, device=positions.device)
+    check(lib().guffin_hip_rope_table(_stream(), _p(positions), _p(table), rows, rope_dim, C.c_float(base),
+                                      C.c_float(scale)))
+    return table
+
+
+def gemv_packed_multi(dtypes, tiles, x, xsums, Ns):
+    """Several matrices over the same activation rows in one launch; returns one [S, rows, N_i] tensor each."""
+    rows, K = x.shape
+    count = len(dtypes)
+    dt = (C.c_int * count)(*dtypes)
+    n = (C.c_uint32 * count)(*Ns)
+    lib().guffin_hip_gemv_packed_multi_slices.restype = C.c_uint32
+    S = lib().guffin_hip_gemv_packed_multi_slices(count, dt, n, K)
+    if S == 0:
+        raise GuffinError(-2, lib().guffin_hip_last_error().decode())
+    parts = [torch.empty((S, rows, N), dtype=torch.float32, device=x.device) for N in Ns]
+    tl = (C.c_void_p * count)(*[t.data_ptr() for t in tiles])
+    pp = (C.c_void_p * count)(*[p.data_ptr() for p in parts])
+    check(lib().guffin_hip_gemv_packed_multi(_stream(), count, dt, tl, n, pp, _p(x), _p(xsums), rows, K))
+    return parts
 
 
 def geglu(gate, up, planes=None, want_sums=False):

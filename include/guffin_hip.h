@@ -98,7 +98,9 @@ int guffin_hip_gemv_packed(void* stream, int dtype, const void* tiles, const flo
                            float* partials, float* y, uint32_t rows, uint32_t K, uint32_t N);
 
 /* Up to three matrices that share the activation rows (q/k/v, gate/up) in one launch.  Each
- * matrix i writes partials[i] as [S_i][rows][N_i] with S_i = guffin_hip_gemv_packed_slices. */
+ * matrix i writes partials[i] as [S][rows][N_i] with the one S = guffin_hip_gemv_packed_multi_slices
+ * of the launch.  All matrices must share the block length (Q4_K and Q6_K mix, Q8_0 does not). */
+uint32_t guffin_hip_gemv_packed_multi_slices(uint32_t count, const int* dtypes, const uint32_t* N, uint32_t K);
 int guffin_hip_gemv_packed_multi(void* stream, uint32_t count, const int* dtypes, const void* const* tiles,
                                  const uint32_t* N, float* const* partials, const float* x,
                                  const float* xsums, uint32_t rows, uint32_t K);
@@ -136,16 +138,23 @@ int guffin_hip_rope_neox(void* stream, const float* in, const uint32_t* position
 int guffin_hip_kv_store_f16(void* stream, const float* raw_k, const float* raw_v, const uint32_t* positions,
                             void* out_k, void* out_v, uint32_t rows, uint32_t heads, uint32_t head_dim,
                             uint32_t rope_dim, float freq_base, float freq_scale, uint32_t* status);
+/* cos and sin of every (row, pair) angle, table[rows][rope_dim/2][2] = {cos, sin}, formed in
+ * double exactly as guffin_hip_rope_neox forms them (src/tensor/ops/rope.cpp:109-117); a
+ * forward pass fills one table per frequency base and hands it to every block's qkv_post. */
+int guffin_hip_rope_table(void* stream, const uint32_t* positions, float* table, uint32_t rows,
+                          uint32_t rope_dim, float freq_base, float freq_scale);
 /* The three steps between the QKV GEMVs and attention in one launch: q/k head norms
  * (NULL gamma skips), RoPE on q and k, fp16 narrowing of k and v
- * (src/engine/gemma_target_runtime.cpp:92-124). */
+ * (src/engine/gemma_target_runtime.cpp:92-124).  rope_table (optional) replaces positions,
+ * freq_base and freq_scale by a table from guffin_hip_rope_table. */
 int guffin_hip_qkv_post(void* stream, const float* q_raw, const float* k_raw, const float* v_raw,
                         uint32_t q_planes, uint32_t k_planes, uint32_t v_planes,
                         uint64_t q_plane_stride, uint64_t k_plane_stride,
                         uint64_t v_plane_stride, const float* q_norm, const float* k_norm,
                         const uint32_t* positions, float* q_out, void* k_out, void* v_out,
                         uint32_t rows, uint32_t q_heads, uint32_t kv_heads, uint32_t head_dim,
-                        uint32_t rope_dim, float freq_base, float freq_scale, float eps, uint32_t* status);
+                        uint32_t rope_dim, float freq_base, float freq_scale, float eps,
+                        const float* rope_table, uint32_t* status);
 /* out = 0.5 g (1 + tanh(0.7978845608 (g + 0.044715 g^3))) * up.  Replaces
  * encode_gelu_tanh_multiply (:313); CPU definition src/tensor/ops/elementwise.cpp:79-94, 50-63. */
 int guffin_hip_geglu(void* stream, const float* gate, const float* up, uint32_t planes, uint64_t plane_stride,

@@ -129,6 +129,45 @@ def test_packed_partials_sum_in_slice_order(hip):
     assert np.array_equal(total.view(np.uint32), y.view(np.uint32))
 
 
+MULTI = [
+    ((1, 1, 2), 3840, (4096, 2048, 2048)),   # 12B q/k/v with a Q6_K value projection
+    ((1, 1, 1), 3840, (4096, 2048, 2048)),
+    ((1, 1), 3840, (15360, 15360)),          # 12B gate/up
+    ((2, 2), 768, (128, 64)),
+    ((0, 0, 0), 640, (1024, 256, 256)),      # 270M q/k/v
+    ((0, 0), 640, (2048, 2048)),
+]
+
+
+@pytest.mark.parametrize("dtypes,K,Ns", MULTI)
+@pytest.mark.parametrize("rows", [1, 2])
+def test_packed_multi_matches_single_launches(hip, gfo, dtypes, K, Ns, rows):
+    x = synth.make_activation(rows, K, seed=40)
+    xd = dev(x)
+    xs = hip.group_sums(xd)
+    ws = [synth.make_weight(dt, K, N, seed=41 + i) for i, (dt, N) in enumerate(zip(dtypes, Ns))]
+    tiles = [hip.repack(dt, dev(w), K, N) for dt, w, N in zip(dtypes, ws, Ns)]
+    parts = hip.gemv_packed_multi(dtypes, tiles, xd, xs, Ns)
+    assert len({p.shape[0] for p in parts}) == 1            # one slice count per launch
+    for dt, w, t, N, p in zip(dtypes, ws, tiles, Ns, parts):
+        assert p.shape[1:] == (rows, N)
+        y = p.cpu().numpy().astype(np.float64).sum(axis=0)
+        ref = gfo.gemv(dt, w, x, N, threads=8)
+        scale = np.sqrt((ref.astype(np.float64) ** 2).mean(axis=1, keepdims=True))
+        assert np.all(np.abs(y - ref) <= 1e-3 * scale)
+        single = hip.gemv_packed(dt, t, xd, xs, N).cpu().numpy()
+        assert np.all(np.abs(y - single) <= 2e-5 * scale)
+
+
+def test_packed_multi_rejects_mixed_block_lengths(hip):
+    import torch
+    x = torch.zeros((1, 256), dtype=torch.float32, device="cuda")
+    xs = hip.group_sums(x)
+    t = torch.zeros(144 * 64, dtype=torch.uint8, device="cuda")
+    with pytest.raises(hip.GuffinError):
+        hip.gemv_packed_multi((1, 0), [t, t], x, xs, (64, 64))
+
+
 def test_packed_rejects_bad_arguments(hip):
     import torch
     w = torch.zeros(144 * 64, dtype=torch.uint8, device="cuda")

@@ -157,6 +157,15 @@ def test_qkv_post_fuses_headnorm_rope_and_narrowing(hip, gfo):
     assert np.mean(gk == want_k) > 0.995
     d = np.abs(gk.view(np.float16).astype(np.float32) - want_k.view(np.float16).astype(np.float32))
     assert d.max() <= 2.0 ** -9 * np.abs(want_q).max()
+    # a precomputed angle table gives the same bits as angles formed in the kernel
+    table = hip.rope_table(dev(pos), hd, 1e4, 1.0)
+    q2, k2, v2 = hip.qkv_post(dev(qp), dev(kp), dev(vp), dev(qn), dev(kn), None, rows, qh, kvh, hd, hd, 1e4,
+                              planes=planes, table=table)
+    assert torch.equal(q2.view(torch.int32), q.view(torch.int32))
+    assert torch.equal(k2.view(torch.int16), k.view(torch.int16)) and torch.equal(v2.view(torch.int16), v.view(torch.int16))
+    tb = table.cpu().numpy().astype(np.float64)
+    ang = pos[:, None].astype(np.float64) / 1e4 ** (2.0 * np.arange(hd // 2) / hd)
+    assert np.max(np.abs(tb[..., 0] - np.cos(ang))) <= 6e-8 and np.max(np.abs(tb[..., 1] - np.sin(ang))) <= 6e-8
 
 
 @pytest.mark.parametrize("rows,width", [(1, 2048), (2, 15360)])
