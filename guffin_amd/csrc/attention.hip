@@ -22,6 +22,7 @@
 // Partitions emit (max, denominator, unnormalised output); a second kernel merges them in
 // partition order.  fp32 throughout, keys/values stay fp16 in memory.
 #include "common.hpp"
+#include "receipt.hpp"
 
 namespace guffin {
 namespace {
@@ -264,19 +265,8 @@ attn_merge_kernel(const float* __restrict__ part_out, const float* __restrict__ 
     if (bad && status) atomicOr(status, GUFFIN_STATUS_NONFINITE);
     if (out_sums) {
         __syncthreads();
-        // group sums of the attention output row [q_heads*hd] feed the o-projection GEMV
-        const uint32_t row = rh / q_heads, head = rh % q_heads, width = q_heads * hd;
-        float* sums = out_sums + size_t(row) * (width / 16 + width / 32);
-        for (uint32_t g = threadIdx.x; g < hd / 16; g += blockDim.x) {
-            float s = 0.f;
-            for (int k = 0; k < 16; ++k) s += rowbuf[g * 16 + k];
-            sums[head * (hd / 16) + g] = s;
-        }
-        for (uint32_t g = threadIdx.x; g < hd / 32; g += blockDim.x) {
-            float s0 = 0.f, s1 = 0.f;
-            for (int k = 0; k < 16; ++k) { s0 += rowbuf[g * 32 + k]; s1 += rowbuf[g * 32 + 16 + k]; }
-            sums[width / 16 + head * (hd / 32) + g] = s0 + s1;
-        }
+        // receipt of the attention output row [q_heads*hd], the o-projection's input
+        emit_receipt(rowbuf, (rh % q_heads) * hd, hd, rh / q_heads, gridDim.x / q_heads, q_heads * hd, out_sums);
     }
 }
 
@@ -312,6 +302,7 @@ extern "C" int guffin_hip_attention_decode(void* stream, const float* q, const v
         return fail(GUFFIN_E_ARG, "attention_decode: null pointer");
     if (rows == 0 || rows > kMaxRows || private_rows > 32) return fail(GUFFIN_E_SHAPE, "attention_decode: rows must be 1 or 2, private rows <= 32");
     if (head_dim != 256) return fail(GUFFIN_E_SHAPE, "attention_decode: head_dim must be 256");
+    if (reinterpret_cast<uintptr_t>(out_sums) & 255u) return fail(GUFFIN_E_ALIGN, "attention_decode: the receipt must be 256-byte aligned");
     if (kv_heads == 0 || q_heads % kv_heads != 0) return fail(GUFFIN_E_SHAPE, "attention_decode: q_heads must be a multiple of kv_heads");
     if ((ring_mask & (ring_mask + 1)) != 0) return fail(GUFFIN_E_ARG, "attention_decode: ring capacity must be a power of two");
     if (max_tokens == 0) return fail(GUFFIN_E_SHAPE, "attention_decode: max_tokens must cover every row's token list");

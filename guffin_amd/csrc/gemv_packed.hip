@@ -28,6 +28,7 @@
 // reduce_partials below), so results are deterministic and a row's arithmetic does not
 // depend on how many rows are computed.
 #include "common.hpp"
+#include "receipt.hpp"
 
 namespace guffin {
 namespace {
@@ -45,7 +46,12 @@ __host__ __device__ constexpr uint32_t block_elems(int dtype) { return dtype == 
 template <int DTYPE>
 __device__ __forceinline__ uint32_t tile_offset(uint32_t o, uint32_t l) {
     if constexpr (DTYPE == GUFFIN_Q4_K) {
-        return (o >> 4) * 1024u + l * 16u + (o & 15u);
+        // matrix-core tile: the 16-byte header is piece 8 of lane l; quant byte q = o - 16 belongs
+        // to 32-byte chunk ch, k-slice s = (q % 32) / 8; column l = 16*cg + j feeds lane 16*s + j
+        // of column group cg, piece 2*cg + ch/2, as bytes (ch % 2)*8 + q % 8
+        if (o < 16u) return 8u * 1024u + l * 16u + o;
+        const uint32_t q = o - 16u, ch = q >> 5, s = (q & 31u) >> 3, cg = l >> 4, j = l & 15u;
+        return (2u * cg + (ch >> 1)) * 1024u + (16u * s + j) * 16u + (ch & 1u) * 8u + (q & 7u);
     } else if constexpr (DTYPE == GUFFIN_Q6_K) {
         return o < 208u ? (o >> 4) * 1024u + l * 16u + (o & 15u) : 13312u + l * 2u + (o - 208u);
     } else {
@@ -75,20 +81,9 @@ __global__ void repack_kernel(const uint16_t* __restrict__ src, uint16_t* __rest
     }
 }
 
-// xsums[r][0 .. K/16) = sums of 16 consecutive activations, xsums[r][K/16 .. 3K/32) = sums of 32.
-__global__ void group_sums_kernel(const float* __restrict__ x, float* __restrict__ xsums, uint32_t K, uint32_t rows) {
-    const uint32_t n16 = K / 16, per_row = n16 + K / 32;
-    for (uint32_t g = blockIdx.x * blockDim.x + threadIdx.x; g < rows * n16; g += gridDim.x * blockDim.x) {
-        const uint32_t r = g / n16, i = g - r * n16;
-        const float* p = x + size_t(r) * K + i * 16u;
-        float s = 0.f;
-#pragma unroll
-        for (int k = 0; k < 16; ++k) s += p[k];
-        xsums[r * per_row + i] = s;
-        // the 32-sum is the sum of its two 16-sums, taken by the even thread of the pair
-        const float other = __shfl_xor(s, 1, kWave);
-        if ((i & 1u) == 0) xsums[r * per_row + n16 + (i >> 1)] = s + other;
-    }
+// One workgroup per row writes the row's activation receipt (sums, multipliers, image).
+__global__ void __launch_bounds__(256) group_sums_kernel(const float* __restrict__ x, void* __restrict__ receipt, uint32_t K, uint32_t rows) {
+    emit_receipt(x + size_t(blockIdx.x) * K, 0, K, blockIdx.x, rows, K, receipt);
 }
 
 __global__ void reduce_partials_kernel(const float* __restrict__ part, float* __restrict__ y, uint32_t S, uint32_t count) {
@@ -111,67 +106,79 @@ __device__ __forceinline__ uint32_t even_bytes(uint32_t v) { return __builtin_am
 __device__ __forceinline__ uint32_t odd_bytes(uint32_t v) { return __builtin_amdgcn_perm(0u, v, 0x0c030c01u); }
 
 constexpr float kTwo24 = 16777216.0f;      // 2^24: undoes the subnormal scale
-constexpr float kTwo20 = 1048576.0f;       // 2^20: same for fields holding 16*q
 
 // =======================================================================================
 // Q4_K
 // =======================================================================================
-struct Q4Tile { uint4 hdr; uint4 q[8]; };
+// Matrix-core path.  A wave covers 64 columns x one 256-element block as four column groups
+// of 16; lane (j = lane % 16, s = lane / 16) holds, for every column group, the bytes 8s..8s+7
+// of each 32-byte quant chunk of column 16*cg + j, and owns column `lane` for the scales and
+// the result.  For each 32-element sub-block and column group one v_mfma_f32_16x16x32_f16
+// multiplies the activation image (A: 16 rows = the 4 variants hi/lo x row, repeated; lane
+// (i, s) holds variant i % 4, k-slice s) with the nibbles as fp16 subnormals (B: q * 2^-24,
+// or 16q * 2^-24 for high nibbles, both exact).  Every lane group then holds the four variant
+// sums of the 16 columns of that group; lane group g keeps those of column group g and scales
+// them by d*sc of its own column in fp32.  The -dmin*m term uses the 32-sums.
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+
+struct Q4Tile { uint4 q[8]; uint4 hdr; };
 
 __device__ __forceinline__ void load_tile(Q4Tile& t, const uint8_t* p) {
-    t.hdr = *reinterpret_cast<const uint4*>(p);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) t.q[i] = *reinterpret_cast<const uint4*>(p + 1024 * (i + 1));
+    for (int i = 0; i < 8; ++i) t.q[i] = *reinterpret_cast<const uint4*>(p + 1024 * i);
+    t.hdr = *reinterpret_cast<const uint4*>(p + 8192);
 }
 
+__device__ __forceinline__ half8_t as_half8(uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
+    return __builtin_bit_cast(half8_t, make_uint4(a, b, c, d));
+}
+
+// image: this block's 8 groups of the activation image, already offset for this lane;
+// mult / xs32: this block's 8 multipliers / 32-sums of row 0 (rows `per_mult` / `per_row` apart)
 template <int R>
-__device__ __forceinline__ void compute_tile(const Q4Tile& t, const float* __restrict__ x, const float* __restrict__ xs32,
-                                             uint32_t K, uint32_t per_row, float (&acc)[R]) {
-    // x, xs32 point at this block's 256 activations / 8 group sums of row 0
+__device__ __forceinline__ void compute_tile(const Q4Tile& t, const uint8_t* __restrict__ image,
+                                             const float* __restrict__ mult, uint32_t per_mult,
+                                             const float* __restrict__ xs32, uint32_t per_row,
+                                             uint32_t lane_group, float (&acc)[R]) {
     const float d = h2f(t.hdr.x & 0xFFFFu), dmin = h2f(t.hdr.x >> 16);
     const uint32_t s0 = t.hdr.y, s1 = t.hdr.z, s2 = t.hdr.w;
     const uint32_t sc_a = s0 & 0x3F3F3F3Fu, mn_a = s1 & 0x3F3F3F3Fu;
     const uint32_t sc_b = (s2 & 0x0F0F0F0Fu) | ((s0 >> 2) & 0x30303030u);
     const uint32_t mn_b = ((s2 >> 4) & 0x0F0F0F0Fu) | ((s1 >> 2) & 0x30303030u);
-    const float d_lo = d * kTwo24, d_hi = d * kTwo20;
+    const float d_hi = d * 0.0625f;  // high nibbles enter as 16*q
     float mt[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) mt[r] = 0.f;
+    half8_t a[8];
 #pragma unroll
-    for (int J = 0; J < 4; ++J) {  // sub-block of 64: groups 2J (low nibbles) and 2J+1 (high)
-        float plo[R], phi[R];
+    for (int g = 0; g < 8; ++g) a[g] = __builtin_bit_cast(half8_t, *reinterpret_cast<const uint4*>(image + 256 * g));
+    const float4_t zero = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int r = 0; r < R; ++r) { plo[r] = 0.f; phi[r] = 0.f; }
+    for (int ch = 0; ch < 4; ++ch) {  // 32-byte chunk: sub-blocks 2ch (low nibbles) and 2ch+1 (high)
+        float4_t lo = zero, hi = zero;
 #pragma unroll
-        for (int half = 0; half < 2; ++half) {
-            const uint4 qv = t.q[2 * J + half];
-            const uint32_t qd[4] = {qv.x, qv.y, qv.z, qv.w};
-#pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                const uint32_t w = qd[k], w8 = w >> 8;
-                const uint32_t a = w & 0x000F000Fu, b = w & 0x00F000F0u;    // bytes 0,2: low / 16*high
-                const uint32_t c = w8 & 0x000F000Fu, e = w8 & 0x00F000F0u;  // bytes 1,3
-                const int e0 = 64 * J + 16 * half + 4 * k;
-#pragma unroll
-                for (int r = 0; r < R; ++r) {
-                    const float* xr = x + size_t(r) * K;
-                    mix2(plo[r], a, xr[e0], xr[e0 + 2]);
-                    mix2(plo[r], c, xr[e0 + 1], xr[e0 + 3]);
-                    mix2(phi[r], b, xr[e0 + 32], xr[e0 + 34]);
-                    mix2(phi[r], e, xr[e0 + 33], xr[e0 + 35]);
-                }
-            }
+        for (int cg = 0; cg < 4; ++cg) {
+            const uint4 piece = t.q[2 * cg + (ch >> 1)];
+            const uint32_t w0 = (ch & 1) ? piece.z : piece.x, w1 = (ch & 1) ? piece.w : piece.y;
+            const uint32_t v0 = w0 >> 8, v1 = w1 >> 8;
+            const half8_t blo = as_half8(w0 & 0x000F000Fu, v0 & 0x000F000Fu, w1 & 0x000F000Fu, v1 & 0x000F000Fu);
+            const half8_t bhi = as_half8(w0 & 0x00F000F0u, v0 & 0x00F000F0u, w1 & 0x00F000F0u, v1 & 0x00F000F0u);
+            const float4_t dlo = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[2 * ch], blo, zero, 0, 0, 0);
+            const float4_t dhi = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[2 * ch + 1], bhi, zero, 0, 0, 0);
+            if (lane_group == uint32_t(cg)) { lo = dlo; hi = dhi; }
         }
-        const uint32_t scw = J < 2 ? sc_a : sc_b, mnw = J < 2 ? mn_a : mn_b;
-        const float sc_lo = (J & 1) ? ub2(scw) : ub0(scw), sc_hi = (J & 1) ? ub3(scw) : ub1(scw);
-        const float mn_lo = (J & 1) ? ub2(mnw) : ub0(mnw), mn_hi = (J & 1) ? ub3(mnw) : ub1(mnw);
-        const float f_lo = d_lo * sc_lo, f_hi = d_hi * sc_hi;
+        const uint32_t scw = ch < 2 ? sc_a : sc_b, mnw = ch < 2 ? mn_a : mn_b;
+        const float sc_lo = (ch & 1) ? ub2(scw) : ub0(scw), sc_hi = (ch & 1) ? ub3(scw) : ub1(scw);
+        const float mn_lo = (ch & 1) ? ub2(mnw) : ub0(mnw), mn_hi = (ch & 1) ? ub3(mnw) : ub1(mnw);
+        const float f_lo = d * sc_lo, f_hi = d_hi * sc_hi;
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            acc[r] = fmaf(f_lo, plo[r], acc[r]);
-            acc[r] = fmaf(f_hi, phi[r], acc[r]);
-            mt[r] = fmaf(mn_lo, xs32[r * per_row + 2 * J], mt[r]);
-            mt[r] = fmaf(mn_hi, xs32[r * per_row + 2 * J + 1], mt[r]);
+            const float m_lo = mult[r * per_mult + 2 * ch], m_hi = mult[r * per_mult + 2 * ch + 1];
+            acc[r] = fmaf(f_lo * m_lo, lo[2 * r] + lo[2 * r + 1], acc[r]);
+            acc[r] = fmaf(f_hi * m_hi, hi[2 * r] + hi[2 * r + 1], acc[r]);
+            mt[r] = fmaf(mn_lo, xs32[r * per_row + 2 * ch], mt[r]);
+            mt[r] = fmaf(mn_hi, xs32[r * per_row + 2 * ch + 1], mt[r]);
         }
     }
 #pragma unroll
@@ -294,11 +301,16 @@ __device__ __forceinline__ void run_blocks(const uint8_t* __restrict__ wt, const
 #pragma unroll
     for (int r = 0; r < R; ++r) acc[r] = 0.f;
     if constexpr (DTYPE == GUFFIN_Q4_K) {
+        const ReceiptLayout L = receipt_layout(R, K);
+        const uint8_t* blob = reinterpret_cast<const uint8_t*>(xsums);
+        const float* mult = reinterpret_cast<const float*>(blob + L.mult_off);
+        // lane (i = lane % 16, s = lane / 16) of the A operand: variant i % 4, k-slice s
+        const uint8_t* image = blob + L.image_off + (lane & 3u) * 64u + (lane >> 4) * 16u;
         Q4Tile cur, nxt;
         if (b0 < b1) load_tile(cur, tp);
         for (uint32_t b = b0; b < b1; ++b) {
             if (b + 1 < b1) load_tile(nxt, tp + size_t(b + 1 - b0) * TB);
-            compute_tile<R>(cur, x + size_t(b) * BE, xs + b * sums_per_block, K, per_row, acc);
+            compute_tile<R>(cur, image + size_t(b) * 2048u, mult + b * 8u, K / 32, xs + b * 8u, per_row, lane >> 4, acc);
             cur = nxt;
         }
     } else if constexpr (DTYPE == GUFFIN_Q6_K) {
@@ -474,10 +486,15 @@ extern "C" int guffin_hip_unpack(void* stream, int dtype, const void* tiles, voi
 
 extern "C" int guffin_hip_group_sums(void* stream, const float* x, float* xsums, uint32_t rows, uint32_t K) {
     if (!x || !xsums) return fail(GUFFIN_E_ARG, "group_sums: null pointer");
-    if (rows == 0 || K == 0 || K % 32 != 0) return fail(GUFFIN_E_SHAPE, "group_sums: K must be a positive multiple of 32");
-    const uint32_t n = rows * (K / 16);
-    hipLaunchKernelGGL(group_sums_kernel, dim3((n + 255) / 256), dim3(256), 0, as_stream(stream), x, xsums, K, rows);
+    if (rows == 0 || rows > 2 || K == 0 || K % 32 != 0) return fail(GUFFIN_E_SHAPE, "group_sums: K must be a positive multiple of 32, rows 1 or 2");
+    if (reinterpret_cast<uintptr_t>(xsums) & 255u) return fail(GUFFIN_E_ALIGN, "group_sums: the receipt must be 256-byte aligned");
+    hipLaunchKernelGGL(group_sums_kernel, dim3(rows), dim3(256), 0, as_stream(stream), x, xsums, K, rows);
     return check_launch("group_sums");
+}
+
+extern "C" uint64_t guffin_hip_receipt_bytes(uint32_t rows, uint32_t K) {
+    if (rows == 0 || rows > 2 || K == 0 || K % 32 != 0) return 0;
+    return receipt_layout(rows, K).bytes;
 }
 
 extern "C" uint32_t guffin_hip_gemv_packed_slices(int dtype, uint32_t K, uint32_t N) {

@@ -14,6 +14,7 @@
 // sums the packed GEMV consumes, and every operator that consumes a GEMV output can sum
 // `planes` k-slice partial planes (stride plane_stride floats) while it loads.
 #include "common.hpp"
+#include "receipt.hpp"
 
 namespace guffin {
 namespace {
@@ -41,23 +42,6 @@ __device__ __forceinline__ float load_planes(const float* p, uint32_t planes, si
     }
     for (; s < planes; ++s) v += p[s * plane_stride];
     return v;
-}
-
-// 16-sums and 32-sums of a row that lives in LDS (`row`, `width` floats), written to sums[]
-__device__ __forceinline__ void emit_group_sums(const float* row, float* sums, uint32_t width) {
-    const uint32_t n16 = width / 16;
-    for (uint32_t g = threadIdx.x; g < n16; g += blockDim.x) {
-        float s = 0.f;
-#pragma unroll
-        for (int k = 0; k < 16; ++k) s += row[g * 16 + k];
-        sums[g] = s;
-    }
-    for (uint32_t g = threadIdx.x; g < width / 32; g += blockDim.x) {
-        float a = 0.f, b = 0.f;
-#pragma unroll
-        for (int k = 0; k < 16; ++k) { a += row[g * 32 + k]; b += row[g * 32 + 16 + k]; }
-        sums[n16 + g] = a + b;  // the sum of the two 16-sums, as group_sums_kernel forms it
-    }
 }
 
 // Loads the row (summing partial planes) into LDS and returns this thread's share of the
@@ -122,7 +106,7 @@ rms_norm_kernel(const float* __restrict__ x, uint32_t planes, size_t plane_strid
     if (bad && status) atomicOr(status, GUFFIN_STATUS_NONFINITE);
     if (y_sums) {
         __syncthreads();
-        emit_group_sums(row, y_sums + size_t(r) * (width / 16 + width / 32), width);
+        emit_receipt(row, 0, width, r, gridDim.x, width, y_sums);
     }
 }
 
@@ -161,7 +145,7 @@ rms_norm_add_norm_kernel(const float* __restrict__ x, uint32_t planes, size_t pl
     if (bad && status) atomicOr(status, GUFFIN_STATUS_NONFINITE);
     if (out_sums) {
         __syncthreads();
-        emit_group_sums(row, out_sums + size_t(r) * (width / 16 + width / 32), width);
+        emit_receipt(row, 0, width, r, gridDim.x, width, out_sums);
     }
 }
 
@@ -299,20 +283,7 @@ geglu_kernel(const float* __restrict__ gate, const float* __restrict__ up, uint3
     }
     if (out_sums) {
         __syncthreads();
-        float* sums = out_sums + size_t(blockIdx.y) * (width / 16 + width / 32);
-        const uint32_t n16 = width / 16;
-        for (uint32_t g = threadIdx.x; g < (c1 - c0) / 16; g += blockDim.x) {
-            float s = 0.f;
-#pragma unroll
-            for (int k = 0; k < 16; ++k) s += lds[g * 16 + k];
-            sums[c0 / 16 + g] = s;
-        }
-        for (uint32_t g = threadIdx.x; g < (c1 - c0) / 32; g += blockDim.x) {
-            float a = 0.f, b = 0.f;
-#pragma unroll
-            for (int k = 0; k < 16; ++k) { a += lds[g * 32 + k]; b += lds[g * 32 + 16 + k]; }
-            sums[n16 + c0 / 32 + g] = a + b;
-        }
+        emit_receipt(lds, c0, c1 - c0, blockIdx.y, gridDim.y, width, out_sums);
     }
 }
 
@@ -407,7 +378,8 @@ extern "C" int guffin_hip_rms_norm(void* stream, const float* x, uint32_t planes
                                    uint32_t rows, uint32_t width, float eps, uint32_t* status) {
     if (!x || !gamma || !y) return fail(GUFFIN_E_ARG, "rms_norm: null pointer");
     if (rows == 0 || width == 0 || planes == 0) return fail(GUFFIN_E_SHAPE, "rms_norm: empty shape");
-    if (y_sums && width % 32 != 0) return fail(GUFFIN_E_SHAPE, "rms_norm: group sums need width % 32 == 0");
+    if (y_sums && (width % 32 != 0 || rows > 2)) return fail(GUFFIN_E_SHAPE, "rms_norm: a receipt needs width % 32 == 0 and rows <= 2");
+    if (reinterpret_cast<uintptr_t>(y_sums) & 255u) return fail(GUFFIN_E_ALIGN, "rms_norm: the receipt must be 256-byte aligned");
     if (!(eps > 0.f)) return fail(GUFFIN_E_ARG, "rms_norm: epsilon must be positive");
     if (!aligned4(x) || !aligned4(y) || !aligned4(gamma)) return fail(GUFFIN_E_ALIGN, "rms_norm: fp32 pointers must be 4-byte aligned");
     const size_t lds = (size_t(width) + 16) * 4;
@@ -424,7 +396,8 @@ extern "C" int guffin_hip_rms_norm_add_norm(void* stream, const float* x, uint32
     if (!x || !gamma_post || !residual || !out_residual || !gamma_next || !out_norm)
         return fail(GUFFIN_E_ARG, "rms_norm_add_norm: null pointer");
     if (rows == 0 || width == 0 || planes == 0) return fail(GUFFIN_E_SHAPE, "rms_norm_add_norm: empty shape");
-    if (out_sums && width % 32 != 0) return fail(GUFFIN_E_SHAPE, "rms_norm_add_norm: group sums need width % 32 == 0");
+    if (out_sums && (width % 32 != 0 || rows > 2)) return fail(GUFFIN_E_SHAPE, "rms_norm_add_norm: a receipt needs width % 32 == 0 and rows <= 2");
+    if (reinterpret_cast<uintptr_t>(out_sums) & 255u) return fail(GUFFIN_E_ALIGN, "rms_norm_add_norm: the receipt must be 256-byte aligned");
     if (!(eps > 0.f)) return fail(GUFFIN_E_ARG, "rms_norm_add_norm: epsilon must be positive");
     const size_t lds = (size_t(width) + 16) * 4;
     if (lds > 160 * 1024) return fail(GUFFIN_E_CAPACITY, "rms_norm_add_norm: row does not fit in LDS");
@@ -515,7 +488,8 @@ extern "C" int guffin_hip_geglu(void* stream, const float* gate, const float* up
                                 float* out, float* out_sums, uint32_t rows, uint32_t width) {
     if (!gate || !up || !out) return fail(GUFFIN_E_ARG, "geglu: null pointer");
     if (rows == 0 || width == 0 || planes == 0) return fail(GUFFIN_E_SHAPE, "geglu: empty shape");
-    if (out_sums && width % 32 != 0) return fail(GUFFIN_E_SHAPE, "geglu: group sums need width % 32 == 0");
+    if (out_sums && (width % 32 != 0 || rows > 2)) return fail(GUFFIN_E_SHAPE, "geglu: a receipt needs width % 32 == 0 and rows <= 2");
+    if (reinterpret_cast<uintptr_t>(out_sums) & 255u) return fail(GUFFIN_E_ALIGN, "geglu: the receipt must be 256-byte aligned");
     // chunks of 512 columns (a multiple of 32) per workgroup
     const uint32_t chunk = 512, chunks = (width + chunk - 1) / chunk;
     const uint32_t per = out_sums ? chunk : (width + chunks - 1) / chunks;

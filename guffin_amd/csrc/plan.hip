@@ -12,6 +12,7 @@
 // scratch arena are the caller's; everything is enqueued in order on one HIP stream, so a
 // caller can capture a whole step into a HIP graph.
 #include "common.hpp"
+#include "receipt.hpp"
 
 #include <algorithm>
 #include <cmath>
@@ -40,7 +41,11 @@ struct Scratch {
 };
 
 uint32_t slices(int dtype, uint32_t K, uint32_t N) { return guffin_hip_gemv_packed_slices(dtype, K, N); }
-uint64_t sums_len(uint32_t width) { return width / 16 + width / 32; }
+// floats in the activation receipt of `rows` rows of `width`
+uint64_t receipt_floats(uint32_t rows, uint32_t width) { return receipt_layout(rows, width).bytes / 4; }
+// floats from the start of a [rows][width] block to its receipt (256-byte aligned) and the total
+uint64_t hidden_receipt_offset(uint32_t rows, uint32_t width) { return (uint64_t(rows) * width + 63) & ~uint64_t{63}; }
+uint64_t hidden_with_receipt(uint32_t rows, uint32_t width) { return hidden_receipt_offset(rows, width) + receipt_floats(rows, width); }
 uint32_t qkv_slices(const guffin_layer_desc& L, uint32_t H, uint32_t QW, uint32_t KW) {
     const uint32_t n[3] = {QW, KW, KW};
     return guffin_hip_gemv_packed_multi_slices(3, L.dtype, n, H);
@@ -70,12 +75,12 @@ Scratch layout(const guffin_model_desc& m, uint32_t rows, uint32_t position, uin
     s.x = ar.take<float>(uint64_t(rows) * H);
     s.x1 = ar.take<float>(uint64_t(rows) * H);
     s.u = ar.take<float>(uint64_t(rows) * H);
-    s.us = ar.take<float>(rows * sums_len(H));
+    s.us = ar.take<float>(receipt_floats(rows, H));
     s.q = ar.take<float>(uint64_t(rows) * QW);
     s.a = ar.take<float>(uint64_t(rows) * QW);
-    s.as = ar.take<float>(rows * sums_len(QW));
+    s.as = ar.take<float>(receipt_floats(rows, QW));
     s.h = ar.take<float>(uint64_t(rows) * F);
-    s.hs = ar.take<float>(rows * sums_len(F));
+    s.hs = ar.take<float>(receipt_floats(rows, F));
     // partial planes: a <- q / o / gate / down, b <- k / up, c <- v
     uint64_t pa = 0, pb = 0, pc = 0;
     for (uint32_t l = 0; l < m.layer_count; ++l) {
@@ -255,8 +260,8 @@ extern "C" uint64_t guffin_hip_h1_scratch_bytes(const guffin_h1_desc* d) {
     const uint64_t V = d->target->vocab;
     ar.take<uint8_t>(guffin_hip_forward_scratch_bytes(d->drafter, 1, d->drafter_position));
     ar.take<uint8_t>(guffin_hip_forward_scratch_bytes(d->target, 2, d->target_position));
-    ar.take<float>(d->drafter->hidden + sums_len(d->drafter->hidden));                 // drafter hidden + sums
-    ar.take<float>(2 * (d->target->hidden + sums_len(d->target->hidden)));             // target hidden + sums
+    ar.take<float>(hidden_with_receipt(1, d->drafter->hidden));                 // drafter hidden + sums
+    ar.take<float>(hidden_with_receipt(2, d->target->hidden));             // target hidden + sums
     ar.take<float>(uint64_t(slices(d->drafter->head_dtype, d->drafter->hidden, d->drafter->vocab)) * d->drafter->vocab);
     ar.take<float>(d->drafter->vocab);                                                  // q logits
     ar.take<float>(uint64_t(slices(d->target->head_dtype, d->target->hidden, V)) * 2 * V);
@@ -286,8 +291,8 @@ extern "C" int guffin_hip_h1_step(void* stream, const guffin_h1_desc* d, const u
     const uint64_t t_bytes = guffin_hip_forward_scratch_bytes(&T, 2, d->target_position);
     uint8_t* d_scratch = ar.take<uint8_t>(d_bytes);
     uint8_t* t_scratch = ar.take<uint8_t>(t_bytes);
-    float* d_hidden = ar.take<float>(D.hidden + sums_len(D.hidden));
-    float* t_hidden = ar.take<float>(2 * (T.hidden + sums_len(T.hidden)));
+    float* d_hidden = ar.take<float>(hidden_with_receipt(1, D.hidden));
+    float* t_hidden = ar.take<float>(hidden_with_receipt(2, T.hidden));
     float* q_parts = ar.take<float>(uint64_t(slices(D.head_dtype, D.hidden, D.vocab)) * D.vocab);
     float* q_logits = ar.take<float>(D.vocab);
     float* p_parts = ar.take<float>(uint64_t(slices(T.head_dtype, T.hidden, V)) * 2 * V);
@@ -309,15 +314,15 @@ extern "C" int guffin_hip_h1_step(void* stream, const guffin_h1_desc* d, const u
     hipLaunchKernelGGL(set_token_kernel, dim3(1), dim3(1), 0, s, root_token, tokens);
     GUFFIN_TRY(check_launch("set_token"));
     GUFFIN_TRY(guffin_hip_forward_rows(stream, &D, tokens, 1, d->drafter_position, d_scratch, d_bytes, drafter_priv_k,
-                                       drafter_priv_v, d_hidden, d_hidden + D.hidden, status));
-    GUFFIN_TRY(guffin_hip_gemv_packed(stream, D.head_dtype, D.head_tiles, d_hidden, d_hidden + D.hidden, q_parts,
+                                       drafter_priv_v, d_hidden, d_hidden + hidden_receipt_offset(1, D.hidden), status));
+    GUFFIN_TRY(guffin_hip_gemv_packed(stream, D.head_dtype, D.head_tiles, d_hidden, d_hidden + hidden_receipt_offset(1, D.hidden), q_parts,
                                       q_logits, 1, D.hidden, D.vocab));
     GUFFIN_TRY(guffin_hip_draft_law(stream, q_logits, D.vocab, &opt, d->seed, d->step, nullptr, law_ws, law,
                                     tokens + 1, status));
     // 2. target: rows [root, x] together, head, candidates of both rows
     GUFFIN_TRY(guffin_hip_forward_rows(stream, &T, tokens, 2, d->target_position, t_scratch, t_bytes, target_priv_k,
-                                       target_priv_v, t_hidden, t_hidden + 2 * T.hidden, status));
-    GUFFIN_TRY(guffin_hip_gemv_packed(stream, T.head_dtype, T.head_tiles, t_hidden, t_hidden + 2 * T.hidden, p_parts,
+                                       target_priv_v, t_hidden, t_hidden + hidden_receipt_offset(2, T.hidden), status));
+    GUFFIN_TRY(guffin_hip_gemv_packed(stream, T.head_dtype, T.head_tiles, t_hidden, t_hidden + hidden_receipt_offset(2, T.hidden), p_parts,
                                       p_logits, 2, T.hidden, V));
     GUFFIN_TRY(guffin_hip_select_candidates(stream, p_logits, 2, V, d->top_k, nullptr, nullptr, sel_ws, cands, sel_status));
     // 3. accept x or draw from the residual; on acceptance draw the next root from row 1
@@ -347,8 +352,8 @@ extern "C" int guffin_hip_h1_buffers(const guffin_h1_desc* d, void* scratch, flo
     Arena ar {static_cast<uint8_t*>(scratch), 0, 0};
     ar.take<uint8_t>(guffin_hip_forward_scratch_bytes(&D, 1, d->drafter_position));
     ar.take<uint8_t>(guffin_hip_forward_scratch_bytes(&T, 2, d->target_position));
-    float* dh = ar.take<float>(D.hidden + sums_len(D.hidden));
-    float* th = ar.take<float>(2 * (T.hidden + sums_len(T.hidden)));
+    float* dh = ar.take<float>(hidden_with_receipt(1, D.hidden));
+    float* th = ar.take<float>(hidden_with_receipt(2, T.hidden));
     ar.take<float>(uint64_t(slices(D.head_dtype, D.hidden, D.vocab)) * D.vocab);
     float* ql = ar.take<float>(D.vocab);
     ar.take<float>(uint64_t(slices(T.head_dtype, T.hidden, V)) * 2 * V);

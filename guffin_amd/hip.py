@@ -87,10 +87,39 @@ def unpack(dtype, tiles, K, N):
     return canonical
 
 
+def receipt_bytes(rows, K):
+    lib().guffin_hip_receipt_bytes.restype = C.c_uint64
+    n = lib().guffin_hip_receipt_bytes(rows, K)
+    if n == 0:
+        raise GuffinError(-2, "receipt: K must be a positive multiple of 32 and rows 1 or 2")
+    return n
+
+
+def _receipt(rows, K, device):
+    """New receipt blob; the returned [rows, K/16 + K/32] view of its sums starts at the blob's first byte."""
+    blob = torch.zeros(receipt_bytes(rows, K) // 4, dtype=torch.float32, device=device)
+    n = K // 16 + K // 32
+    return blob[:rows * n].view(rows, n)
+
+
+def receipt_parts(sums, rows, K):
+    """(mult [rows, K/32] float32, image [K/32, 4, 32] float16) of the receipt whose sums view is given."""
+    n = K // 16 + K // 32
+    nbytes = receipt_bytes(rows, K)
+    blob = torch.empty(0, dtype=torch.uint8, device=sums.device).set_(sums.untyped_storage(), sums.storage_offset() * 4,
+                                                                      (nbytes,), (1,))
+    mult_off = (rows * n * 4 + 255) // 256 * 256
+    img_off = (mult_off + rows * (K // 32) * 4 + 255) // 256 * 256
+    mult = blob[mult_off:mult_off + rows * (K // 32) * 4].view(torch.float32).view(rows, K // 32)
+    image = blob[img_off:img_off + (K // 32) * 256].view(torch.float16).view(K // 32, 4, 32)
+    return mult, image
+
+
 def group_sums(x, out=None):
+    """Activation receipt of x (sums, multipliers, matrix-core image); returns its sums view."""
     rows, K = x.shape
     if out is None:
-        out = torch.empty((rows, K // 16 + K // 32), dtype=torch.float32, device=x.device)
+        out = _receipt(rows, K, x.device)
     check(lib().guffin_hip_group_sums(_stream(), _p(x), _p(out), rows, K))
     return out
 
@@ -132,7 +161,7 @@ def rms_norm(x, gamma, eps=1e-6, residual=None, planes=None, want_sums=False, st
     shape = x.shape[1:] if planes else x.shape
     rows, width = shape
     y = _f32((rows, width), x)
-    sums = _f32((rows, width // 16 + width // 32), x) if want_sums else None
+    sums = _receipt(rows, width, x.device) if want_sums else None
     check(lib().guffin_hip_rms_norm(_stream(), _p(x), pl, C.c_uint64(stride), _p(gamma), _p(residual),
                                     _p(y), _p(sums), rows, width, C.c_float(eps), _p(status)))
     return (y, sums) if want_sums else y
@@ -143,7 +172,7 @@ def rms_norm_add_norm(x, gamma_post, residual, gamma_next, eps=1e-6, planes=None
     shape = x.shape[1:] if planes else x.shape
     rows, width = shape
     out_res, out_norm = _f32((rows, width), x), _f32((rows, width), x)
-    sums = _f32((rows, width // 16 + width // 32), x) if want_sums else None
+    sums = _receipt(rows, width, x.device) if want_sums else None
     check(lib().guffin_hip_rms_norm_add_norm(_stream(), _p(x), pl, C.c_uint64(stride), _p(gamma_post),
                                              _p(residual), _p(out_res), _p(gamma_next), _p(out_norm), _p(sums),
                                              rows, width, C.c_float(eps), _p(status)))
@@ -217,7 +246,7 @@ def geglu(gate, up, planes=None, want_sums=False):
     pl, stride = _planes(gate, planes)
     rows, width = gate.shape[1:] if planes else gate.shape
     out = _f32((rows, width), gate)
-    sums = _f32((rows, width // 16 + width // 32), gate) if want_sums else None
+    sums = _receipt(rows, width, gate.device) if want_sums else None
     check(lib().guffin_hip_geglu(_stream(), _p(gate), _p(up), pl, C.c_uint64(stride), _p(out), _p(sums), rows, width))
     return (out, sums) if want_sums else out
 
@@ -245,7 +274,7 @@ def attention_decode(q, ring_k, ring_v, priv_k, priv_v, schedule, ancestors, max
     P = attention_partitions(max_tokens, kv_heads)
     out = torch.empty_like(q)
     width = q_heads * head_dim
-    sums = _f32((rows, width // 16 + width // 32), q) if want_sums else None
+    sums = _receipt(rows, width, q.device) if want_sums else None
     part_out = _f32((rows * q_heads * P * head_dim,), q)
     part_ml = _f32((rows * q_heads * P * 2,), q)
     check(lib().guffin_hip_attention_decode(_stream(), _p(q), _p(ring_k), _p(ring_v), _p(priv_k), _p(priv_v),

@@ -266,7 +266,7 @@ class DeviceModel:
         scratch = torch.zeros(nbytes, dtype=torch.uint8, device="cuda")
         pk, pv = self.private_rows(rows)
         hidden = torch.zeros((rows, sh.hidden), dtype=torch.float32, device="cuda")
-        sums = torch.zeros((rows, sh.hidden // 16 + sh.hidden // 32), dtype=torch.float32, device="cuda")
+        sums = hip._receipt(rows, sh.hidden, "cuda")
         if status is None:
             status = hip.new_status()
         hip.check(lib.guffin_hip_forward_rows(hip._stream(), C.byref(self.desc), hip._p(tokens), rows, position,

@@ -84,9 +84,18 @@ uint64_t guffin_hip_packed_bytes(int dtype, uint32_t K, uint32_t N);
 int guffin_hip_repack(void* stream, int dtype, const void* canonical, void* tiles, uint32_t K, uint32_t N);
 int guffin_hip_unpack(void* stream, int dtype, const void* tiles, void* canonical, uint32_t K, uint32_t N);
 
-/* Per-row sums of 16 and of 32 consecutive activations: xsums is [rows][K/16 + K/32]
- * (16-sums first).  The reference's producers emit the same kind of receipt for its Q4_K
- * kernels (src/tensor/backends/metal/metal_kernels.mm:16-27, "Q4 sums"). */
+/* Activation receipt of rows x K activations (K % 32 == 0, rows 1 or 2): one 256-byte aligned
+ * blob of guffin_hip_receipt_bytes(rows, K) bytes holding
+ *   float sums[rows][K/16 + K/32]   sums of 16 and of 32 consecutive activations (16-sums first);
+ *                                   the reference's producers emit the same kind of receipt for its
+ *                                   Q4_K kernels (src/tensor/backends/metal/metal_kernels.mm:16-27)
+ *   float mult[rows][K/32]          at the next 256-byte boundary: 2^(E+24) per 32-group
+ *   half  image[K/32][4][32]        at the next 256-byte boundary: variants {row0 hi, row0 lo,
+ *                                   row1 hi, row1 lo} of x * 2^-E (hi + lo exact to 22 bits), the
+ *                                   matrix-core operand of the packed Q4_K GEMV; inside a group the
+ *                                   halves of elements 8s..8s+7 sit at 8s + {0,2,1,3,4,6,5,7}
+ * Every operator below that has an `*_sums` output writes this whole blob. */
+uint64_t guffin_hip_receipt_bytes(uint32_t rows, uint32_t K);
 int guffin_hip_group_sums(void* stream, const float* x, float* xsums, uint32_t rows, uint32_t K);
 
 /* Number of k-slices S the packed GEMV cuts this shape into (size of the partials buffer). */

@@ -35,7 +35,7 @@ def test_repack_round_trip_is_lossless(hip, dtype, K, N):
     assert np.array_equal(back, w)
     t = tiles.cpu().numpy()
     assert not np.array_equal(t, w)
-    # spot-check the documented tile layout: 16-byte piece p of column l at p*1024 + l*16
+    # spot-check the documented tile layouts
     bb = synth.BLOCK_BYTES[dtype]
     nblk = K // synth.BLOCK_ELEMS[dtype]
     col, b = 70 % N, nblk - 1
@@ -43,7 +43,12 @@ def test_repack_round_trip_is_lossless(hip, dtype, K, N):
     blk = w[(col * nblk + b) * bb:][:bb]
     lane = col % 64
     if dtype == 1:
-        assert np.array_equal(tile[3 * 1024 + lane * 16:][:16], blk[48:64])
+        # matrix-core tile: header = piece 8 of the column's lane; quant chunk ch, k-slice s of
+        # column 16*cg + j = bytes (ch % 2)*8.. of piece 2*cg + ch/2, lane 16*s + j
+        assert np.array_equal(tile[8 * 1024 + lane * 16:][:16], blk[0:16])
+        cg, j, ch, sl = lane // 16, lane % 16, 1, 2
+        assert np.array_equal(tile[(2 * cg + ch // 2) * 1024 + (16 * sl + j) * 16 + (ch % 2) * 8:][:8],
+                              blk[16 + 32 * ch + 8 * sl:][:8])
     elif dtype == 2:
         assert np.array_equal(tile[9 * 1024 + lane * 16:][:16], blk[144:160])
         assert np.array_equal(tile[13312 + lane * 2:][:2], blk[208:210])
