@@ -234,6 +234,13 @@ attn_merge_kernel(const float* __restrict__ part_out, const float* __restrict__ 
     const uint32_t rh = blockIdx.x;  // row * q_heads + head
     const uint32_t lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
     const float* ml = part_ml + size_t(rh) * partitions * 2;
+    const float* po = part_out + size_t(rh) * partitions * hd;
+    // the first partitions' outputs are requested before the weights exist
+    constexpr int PF = 16;
+    const uint32_t d0 = threadIdx.x;
+    float pre[PF];
+#pragma unroll
+    for (int p = 0; p < PF; ++p) pre[p] = (uint32_t(p) < partitions && d0 < hd) ? po[size_t(p) * hd + d0] : 0.f;
     float m = -INFINITY;
     for (uint32_t p = threadIdx.x; p < partitions; p += 256) if (ml[2 * p + 1] > 0.f) m = fmaxf(m, ml[2 * p]);
     m = wave_max(m);
@@ -246,10 +253,14 @@ attn_merge_kernel(const float* __restrict__ part_out, const float* __restrict__ 
     float denom = 0.f;
     for (uint32_t p = 0; p < partitions; ++p) denom = fmaf(wgt[p], ml[2 * p + 1], denom);
     bool bad = false;
-    const float* po = part_out + size_t(rh) * partitions * hd;
     for (uint32_t d = threadIdx.x; d < hd; d += blockDim.x) {
         float acc = 0.f;
         uint32_t p = 0;
+        if (d == d0) {
+#pragma unroll
+            for (int q = 0; q < PF; ++q) if (uint32_t(q) < partitions) acc = fmaf(wgt[q], pre[q], acc);
+            p = partitions < PF ? partitions : PF;
+        }
         for (; p + 4 <= partitions; p += 4) {
             const float v0 = po[size_t(p) * hd + d], v1 = po[size_t(p + 1) * hd + d], v2 = po[size_t(p + 2) * hd + d],
                         v3 = po[size_t(p + 3) * hd + d];

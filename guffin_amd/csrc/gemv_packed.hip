@@ -7,26 +7,28 @@
 // (replacing src/tensor/backends/metal/metal_kernels.mm:551-750, 788-922, 267-436) that
 // consume it.
 //
-// Tile = 64 adjacent output columns x one block along K.  Inside a tile every 16-byte
-// piece of a block is stored lane-major: piece p of column l sits at p*1024 + l*16, so a
-// wave reads each piece with one fully coalesced 1 KiB load and lane l ends up with its
-// own column's bytes.  Tiles of one column group are consecutive along K.
-//   Q4_K  9216 B : piece 0 = {d, dmin, 12 scale bytes}, pieces 1..8 = quants
-//   Q6_K 13440 B : pieces 0..7 = ql, 8..11 = qh, 12 = 16 int8 scales, then 64 x fp16 d
-//   Q8_0  2176 B : pieces 0..1 = quants, then 64 x fp16 d
+// Tile = 64 adjacent output columns x one block along K, tiles of one column group
+// consecutive along K, same byte count as the GGUF stream.  Inside a tile the quant bytes are
+// laid out for the matrix core: the wave treats the 64 columns as four groups of 16; lane
+// (j = lane % 16, s = lane / 16) holds, for each group, the bytes of elements 8s..8s+7 of every
+// 32-element run of column 16*group + j, in 16-byte pieces stored lane-major (piece p of lane l
+// at p*1024 + l*16, one coalesced 1 KiB load per piece).  Scales and d/dmin sit behind the
+// quant pieces indexed by column (tile_offset below is the exact map; unpack inverts it).
+//   Q4_K  9216 B : pieces 0..7 quants, piece 8 = {d, dmin, 12 scale bytes} of column `lane`
+//   Q6_K 13440 B : pieces 0..7 ql, 8..11 qh, piece 12 = 16 int8 scales, then 64 x fp16 d
+//   Q8_0  2176 B : pieces 0..1 quants, then 64 x fp16 d
 //
-// GEMV: lane l owns output column 64*tile + l for a slice of K.  All lanes walk the same
-// k, so activations are wave-uniform and are read through the scalar cache straight into
-// FMA operands; no cross-lane reduction, LDS only to combine the waves of a workgroup.  Quants are spread into
-// 16-bit fields and fed to v_fma_mix_f32 as fp16 subnormals (an integer n < 1024 in a
-// half is exactly n*2^-24), which replaces convert+FMA by one FMA per weight per row with
-// bit-identical products; the 2^24 is folded into the block scale.  The offset terms
-// (-dmin*m for Q4_K, -32 for Q6_K, -128 for the biased Q8_0 bytes) use per-16 / per-32
-// activation sums supplied by the producer of x.  K is cut into slices: up to 16 slices are
-// the waves of one workgroup and are combined in wave order through LDS, the remaining
-// S "planes" go to [S][rows][N] and are summed in plane order by the consumer (or by
-// reduce_partials below), so results are deterministic and a row's arithmetic does not
-// depend on how many rows are computed.
+// GEMV: one v_mfma_f32_16x16x32_f16 per 32 elements and column group.  B = the quants as fp16
+// subnormals (an integer n < 1024 in a half is exactly n*2^-24, and the matrix core honours
+// subnormal inputs), A = the activation image of the producer's receipt (hi/lo fp16 split of
+// x * 2^-E per 32-group, four variants = two rows), so every product is exact and sums are
+// fp32.  Block scales are applied to the per-group sums in fp32 by the lane that owns the
+// column; the offset terms (-dmin*m for Q4_K, -32 for Q6_K, -128 for the biased Q8_0 bytes)
+// use the receipt's 16- / 32-sums.  K is cut into slices: up to 16 slices are the waves of
+// one workgroup, combined in wave order through LDS; the remaining S "planes" go to
+// [S][rows][N] and are summed in plane order by the consumer (or by reduce_partials below).
+// The split depends on the shape only, and a row's arithmetic does not depend on how many
+// rows are computed, so results are deterministic and 2-row rows equal 1-row calls bit for bit.
 #include "common.hpp"
 #include "receipt.hpp"
 
@@ -53,11 +55,24 @@ __device__ __forceinline__ uint32_t tile_offset(uint32_t o, uint32_t l) {
         const uint32_t q = o - 16u, ch = q >> 5, s = (q & 31u) >> 3, cg = l >> 4, j = l & 15u;
         return (2u * cg + (ch >> 1)) * 1024u + (16u * s + j) * 16u + (ch & 1u) * 8u + (q & 7u);
     } else if constexpr (DTYPE == GUFFIN_Q6_K) {
-        return o < 208u ? (o >> 4) * 1024u + l * 16u + (o & 15u) : 13312u + l * 2u + (o - 208u);
+        // ql byte o: half n = o/64, run m = (o%64)/32, k-slice s = (o%32)/8 -> piece 2*cg + n, lane
+        // 16*s + j, byte 8*m + o%8.  qh byte o-128: half n, k-slice s -> piece 8 + cg, byte 8*n + o%8.
+        // Scales: piece 12 of the column's lane; d: after the pieces.
+        const uint32_t cg = l >> 4, j = l & 15u;
+        if (o < 128u) {
+            const uint32_t n = o >> 6, m = (o & 63u) >> 5, s = (o & 31u) >> 3;
+            return (2u * cg + n) * 1024u + (16u * s + j) * 16u + 8u * m + (o & 7u);
+        }
+        if (o < 192u) {
+            const uint32_t q = o - 128u, n = q >> 5, s = (q & 31u) >> 3;
+            return (8u + cg) * 1024u + (16u * s + j) * 16u + 8u * n + (q & 7u);
+        }
+        return o < 208u ? 12288u + l * 16u + (o - 192u) : 13312u + l * 2u + (o - 208u);
     } else {
+        // Q8_0: quant byte q = o - 2, k-slice s = q/8 -> piece cg/2, lane 16*s + j, byte 8*(cg%2) + q%8
         if (o < 2u) return 2048u + l * 2u + o;
-        const uint32_t q = o - 2u;
-        return (q >> 4) * 1024u + l * 16u + (q & 15u);
+        const uint32_t q = o - 2u, cg = l >> 4, j = l & 15u, s = q >> 3;
+        return (cg >> 1) * 1024u + (16u * s + j) * 16u + 8u * (cg & 1u) + (q & 7u);
     }
 }
 
@@ -94,18 +109,10 @@ __global__ void reduce_partials_kernel(const float* __restrict__ part, float* __
     }
 }
 
-// ---- fp16-subnormal FMA helpers -------------------------------------------------------
-// `packed` holds two integers < 1024 in its 16-bit halves; adds lo*x0 + hi*x1 (times 2^-24).
-__device__ __forceinline__ void mix2(float& acc, uint32_t packed, float x0, float x1) {
-    const half2_t h = __builtin_bit_cast(half2_t, packed);
-    acc = fmaf(static_cast<float>(h.x), x0, acc);
-    acc = fmaf(static_cast<float>(h.y), x1, acc);
-}
 // bytes {0,2} and {1,3} of v as 16-bit fields
 __device__ __forceinline__ uint32_t even_bytes(uint32_t v) { return __builtin_amdgcn_perm(0u, v, 0x0c020c00u); }
 __device__ __forceinline__ uint32_t odd_bytes(uint32_t v) { return __builtin_amdgcn_perm(0u, v, 0x0c030c01u); }
 
-constexpr float kTwo24 = 16777216.0f;      // 2^24: undoes the subnormal scale
 
 // =======================================================================================
 // Q4_K
@@ -188,65 +195,116 @@ __device__ __forceinline__ void compute_tile(const Q4Tile& t, const uint8_t* __r
 // =======================================================================================
 // Q6_K
 // =======================================================================================
-struct Q6Tile { uint4 ql[8]; uint4 qh[4]; uint4 sc; uint32_t d; };
+// Same operand scheme as Q4_K with two differences.  A scale covers 16 elements, so the A rows
+// of one 32-element MFMA are split: rows 0-3 carry the variants with the second 16 elements
+// zeroed, rows 4-7 the other half (rows 8-15 repeat them); lane group g then holds the sums of
+// k-half g % 2.  Lane (j, g) owns columns 32*(g/2) + j and + 16 for that k-half, keeps column
+// groups 2*(g/2) and 2*(g/2)+1, and the two k-halves are added across lanes at the end.
+struct Q6Tile { uint4 ql[8]; uint4 qh[4]; uint4 sc[2]; uint32_t d[2]; };
 
 __device__ __forceinline__ void load_tile(Q6Tile& t, const uint8_t* p, uint32_t lane) {
 #pragma unroll
     for (int i = 0; i < 8; ++i) t.ql[i] = *reinterpret_cast<const uint4*>(p + 1024 * i);
 #pragma unroll
     for (int i = 0; i < 4; ++i) t.qh[i] = *reinterpret_cast<const uint4*>(p + 8192 + 1024 * i);
-    t.sc = *reinterpret_cast<const uint4*>(p + 12288);
-    t.d = *reinterpret_cast<const uint16_t*>(p - lane * 16 + 13312 + lane * 2);
+    const uint8_t* base = p - lane * 16;
+    const uint32_t col = 32u * (lane >> 5) + (lane & 15u);
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+        t.sc[c] = *reinterpret_cast<const uint4*>(base + 12288 + (col + 16 * c) * 16);
+        t.d[c] = *reinterpret_cast<const uint16_t*>(base + 13312 + (col + 16 * c) * 2);
+    }
+}
+
+__device__ __forceinline__ float sbyte(uint32_t w, int i) {
+    return i == 0 ? sb0(w) : i == 1 ? sb1(w) : i == 2 ? sb2(w) : sb3(w);
 }
 
 template <int R>
-__device__ __forceinline__ void compute_tile(const Q6Tile& t, const float* __restrict__ x, const float* __restrict__ xs16,
-                                             uint32_t K, uint32_t per_row, float (&acc)[R]) {
-    const float d24 = h2f(t.d) * kTwo24;
-    const float bias = -32.0f / kTwo24;  // sum (q-32) x = sum q x - 32 sum x, in the subnormal scale
-    const uint32_t scw[4] = {t.sc.x, t.sc.y, t.sc.z, t.sc.w};
+__device__ __forceinline__ void compute_tile(const Q6Tile& t, const uint8_t* __restrict__ image, uint32_t keep,
+                                             const float* __restrict__ mult, uint32_t per_mult,
+                                             const float* __restrict__ xs16, uint32_t per_row,
+                                             uint32_t lane, float (&acc)[2][R]) {
+    const uint32_t khalf = (lane >> 4) & 1u;
+    const bool upper = lane >= 32;
+    const float4_t zero = {0.f, 0.f, 0.f, 0.f};
+    float part[2][R], off[2][R];
 #pragma unroll
-    for (int p = 0; p < 8; ++p) {  // ql piece p: half h, 16-byte run tt
-        const int h = p >> 2, tt = p & 3;
-        const uint4 qlv = t.ql[p], qhv = t.qh[h * 2 + (tt & 1)];
-        const uint32_t ql[4] = {qlv.x, qlv.y, qlv.z, qlv.w}, qh[4] = {qhv.x, qhv.y, qhv.z, qhv.w};
-        const int s_lo = 2 * (tt >> 1), s_hi = 4 + 2 * (tt >> 1);
-        const int e_lo = h * 128 + 32 * (tt >> 1) + 16 * (tt & 1), e_hi = e_lo + 64;
-        const int g_lo = h * 8 + tt, g_hi = g_lo + 4;  // 16-element scale groups
-        float plo[R], phi[R];
+    for (int c = 0; c < 2; ++c)
 #pragma unroll
-        for (int r = 0; r < R; ++r) {
-            plo[r] = bias * xs16[r * per_row + g_lo];
-            phi[r] = bias * xs16[r * per_row + g_hi];
-        }
+        for (int r = 0; r < R; ++r) { part[c][r] = 0.f; off[c][r] = 0.f; }
 #pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            const uint32_t vlo = (ql[k] & 0x0F0F0F0Fu) | (((qh[k] >> s_lo) & 0x03030303u) << 4);
-            const uint32_t vhi = ((ql[k] >> 4) & 0x0F0F0F0Fu) | (((qh[k] >> s_hi) & 0x03030303u) << 4);
-            const uint32_t a = even_bytes(vlo), c = odd_bytes(vlo), b = even_bytes(vhi), e = odd_bytes(vhi);
+    for (int g = 0; g < 8; ++g) {  // 32-element group: half n, quadrant qd
+        const int n = g >> 2, qd = g & 3;
+        uint4 av = *reinterpret_cast<const uint4*>(image + 256 * g);
+        av.x &= keep; av.y &= keep; av.z &= keep; av.w &= keep;
+        const half8_t a = __builtin_bit_cast(half8_t, av);
+        float4_t D[4];
 #pragma unroll
-            for (int r = 0; r < R; ++r) {
-                const float* xr = x + size_t(r) * K;
-                mix2(plo[r], a, xr[e_lo + 4 * k], xr[e_lo + 4 * k + 2]);
-                mix2(plo[r], c, xr[e_lo + 4 * k + 1], xr[e_lo + 4 * k + 3]);
-                mix2(phi[r], b, xr[e_hi + 4 * k], xr[e_hi + 4 * k + 2]);
-                mix2(phi[r], e, xr[e_hi + 4 * k + 1], xr[e_hi + 4 * k + 3]);
+        for (int cg = 0; cg < 4; ++cg) {
+            const uint4 lq = t.ql[2 * cg + n], hq = t.qh[cg];
+            const uint32_t w0 = (qd & 1) ? lq.z : lq.x, w1 = (qd & 1) ? lq.w : lq.y;
+            const uint32_t h0 = n ? hq.z : hq.x, h1 = n ? hq.w : hq.y;
+            const int ls = qd >= 2 ? 4 : 0;  // nibble shift
+            uint32_t b[4];
+#pragma unroll
+            for (int k = 0; k < 2; ++k) {
+                const uint32_t w = k ? w1 : w0, h = k ? h1 : h0;
+                const uint32_t lo0 = (w >> ls) & 0x000F000Fu, lo1 = (w >> (ls + 8)) & 0x000F000Fu;
+                // 2-bit field of quadrant qd moved to bits 4-5 of each half
+                const uint32_t hs0 = qd == 0 ? h << 4 : qd == 1 ? h << 2 : qd == 2 ? h : h >> 2;
+                const uint32_t hs1 = h >> (4 + 2 * qd);
+                b[2 * k] = (hs0 & 0x00300030u) | lo0;
+                b[2 * k + 1] = (hs1 & 0x00300030u) | lo1;
             }
+            D[cg] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, as_half8(b[0], b[1], b[2], b[3]), zero, 0, 0, 0);
         }
-        const uint32_t wlo = scw[g_lo >> 2], whi = scw[g_hi >> 2];
-        const float f_lo = d24 * ((g_lo & 3) == 0 ? sb0(wlo) : (g_lo & 3) == 1 ? sb1(wlo) : (g_lo & 3) == 2 ? sb2(wlo) : sb3(wlo));
-        const float f_hi = d24 * ((g_hi & 3) == 0 ? sb0(whi) : (g_hi & 3) == 1 ? sb1(whi) : (g_hi & 3) == 2 ? sb2(whi) : sb3(whi));
+        const float4_t da = upper ? D[2] : D[0], db = upper ? D[3] : D[1];
+        // int8 scale of 16-element group 2g + khalf for the lane's two columns
+        const int word = g >> 1;  // scales 4*word .. 4*word+3 hold groups 2g-(g&1)*2 ...
+        float sc[2];
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+            const uint32_t wv = word == 0 ? t.sc[c].x : word == 1 ? t.sc[c].y : word == 2 ? t.sc[c].z : t.sc[c].w;
+            const float s_even = sbyte(wv, 2 * (g & 1)), s_odd = sbyte(wv, 2 * (g & 1) + 1);
+            sc[c] = khalf ? s_odd : s_even;
+        }
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            acc[r] = fmaf(f_lo, plo[r], acc[r]);
-            acc[r] = fmaf(f_hi, phi[r], acc[r]);
+            const float m = mult[r * per_mult + g];
+            const float s16 = khalf ? xs16[r * per_row + 2 * g + 1] : xs16[r * per_row + 2 * g];
+            part[0][r] = fmaf(sc[0] * m, da[2 * r] + da[2 * r + 1], part[0][r]);
+            part[1][r] = fmaf(sc[1] * m, db[2 * r] + db[2 * r + 1], part[1][r]);
+            off[0][r] = fmaf(sc[0], s16, off[0][r]);
+            off[1][r] = fmaf(sc[1], s16, off[1][r]);
         }
+    }
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+        const float d = h2f(t.d[c]);
+#pragma unroll
+        for (int r = 0; r < R; ++r) acc[c][r] = fmaf(d, fmaf(-32.0f, off[c][r], part[c][r]), acc[c][r]);
+    }
+}
+
+// adds the two k-halves and hands every lane the sum of its own column
+template <int R>
+__device__ __forceinline__ void q6_gather(const float (&acc2)[2][R], uint32_t lane, float (&acc)[R]) {
+    const uint32_t src = 32u * (lane >> 5) + (lane & 15u);  // lane (j, group 2*(q/2)) holds column 16q + j as a (q even) or b
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const float a = acc2[0][r] + __shfl_xor(acc2[0][r], 16, kWave);
+        const float b = acc2[1][r] + __shfl_xor(acc2[1][r], 16, kWave);
+        const float ga = __shfl(a, src, kWave), gb = __shfl(b, src, kWave);
+        acc[r] = ((lane >> 4) & 1u) ? gb : ga;
     }
 }
 
 // =======================================================================================
 // Q8_0
 // =======================================================================================
+// One 32-element block per MFMA and column group; the int8 quants enter biased by 128 as fp16
+// subnormals, the bias comes back through the 32-sum.
 struct Q8Tile { uint4 q[2]; uint32_t d; };
 
 __device__ __forceinline__ void load_tile(Q8Tile& t, const uint8_t* p, uint32_t lane) {
@@ -256,31 +314,27 @@ __device__ __forceinline__ void load_tile(Q8Tile& t, const uint8_t* p, uint32_t 
 }
 
 template <int R>
-__device__ __forceinline__ void compute_tile(const Q8Tile& t, const float* __restrict__ x, const float* __restrict__ xs32,
-                                             uint32_t K, uint32_t per_row, float (&acc)[R]) {
-    const float d24 = h2f(t.d) * kTwo24;
-    const float bias = -128.0f / kTwo24;  // bytes are biased to q+128
-    float p[R];
+__device__ __forceinline__ void compute_tile(const Q8Tile& t, const uint8_t* __restrict__ image,
+                                             const float* __restrict__ mult, uint32_t per_mult,
+                                             const float* __restrict__ xs32, uint32_t per_row,
+                                             uint32_t lane_group, float (&acc)[R]) {
+    const half8_t a = __builtin_bit_cast(half8_t, *reinterpret_cast<const uint4*>(image));
+    const float4_t zero = {0.f, 0.f, 0.f, 0.f};
+    float4_t own = zero;
 #pragma unroll
-    for (int r = 0; r < R; ++r) p[r] = bias * xs32[r * per_row];
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-        const uint32_t qd[4] = {t.q[i].x, t.q[i].y, t.q[i].z, t.q[i].w};
-#pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            const uint32_t u = qd[k] ^ 0x80808080u;
-            const uint32_t a = even_bytes(u), c = odd_bytes(u);
-            const int e0 = 16 * i + 4 * k;
-#pragma unroll
-            for (int r = 0; r < R; ++r) {
-                const float* xr = x + size_t(r) * K;
-                mix2(p[r], a, xr[e0], xr[e0 + 2]);
-                mix2(p[r], c, xr[e0 + 1], xr[e0 + 3]);
-            }
-        }
+    for (int cg = 0; cg < 4; ++cg) {
+        const uint4 piece = t.q[cg >> 1];
+        const uint32_t w0 = ((cg & 1) ? piece.z : piece.x) ^ 0x80808080u, w1 = ((cg & 1) ? piece.w : piece.y) ^ 0x80808080u;
+        const float4_t d4 = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+            a, as_half8(even_bytes(w0), odd_bytes(w0), even_bytes(w1), odd_bytes(w1)), zero, 0, 0, 0);
+        if (lane_group == uint32_t(cg)) own = d4;
     }
+    const float d = h2f(t.d);
 #pragma unroll
-    for (int r = 0; r < R; ++r) acc[r] = fmaf(d24, p[r], acc[r]);
+    for (int r = 0; r < R; ++r) {
+        const float v = fmaf(mult[r * per_mult], own[2 * r] + own[2 * r + 1], -128.0f * xs32[r * per_row]);
+        acc[r] = fmaf(d, v, acc[r]);
+    }
 }
 
 // =======================================================================================
@@ -291,21 +345,20 @@ template <int DTYPE, int R>
 __device__ __forceinline__ void run_blocks(const uint8_t* __restrict__ wt, const float* __restrict__ x,
                                            const float* __restrict__ xsums, uint32_t K, uint32_t nblk,
                                            uint32_t ct, uint32_t b0, uint32_t b1, float (&acc)[R]) {
-    constexpr uint32_t TB = kTileCols * block_bytes(DTYPE), BE = block_elems(DTYPE);
+    constexpr uint32_t TB = kTileCols * block_bytes(DTYPE);
     const uint32_t lane = threadIdx.x & 63;
     const uint32_t n16 = K / 16, per_row = n16 + K / 32;
     // Q6_K consumes 16-sums (16 per block), Q4_K 32-sums (8 per block), Q8_0 one 32-sum per block
     const float* xs = DTYPE == GUFFIN_Q6_K ? xsums : xsums + n16;
-    constexpr uint32_t sums_per_block = DTYPE == GUFFIN_Q6_K ? 16 : DTYPE == GUFFIN_Q4_K ? 8 : 1;
     const uint8_t* tp = wt + (size_t(ct) * nblk + b0) * TB + lane * 16;
 #pragma unroll
     for (int r = 0; r < R; ++r) acc[r] = 0.f;
+    const ReceiptLayout L = receipt_layout(R, K);
+    const uint8_t* blob = reinterpret_cast<const uint8_t*>(xsums);
+    const float* mult = reinterpret_cast<const float*>(blob + L.mult_off);
+    // lane (i = lane % 16, s = lane / 16) of the A operand: variant i % 4, k-slice s
+    const uint8_t* image = blob + L.image_off + (lane & 3u) * 64u + (lane >> 4) * 16u;
     if constexpr (DTYPE == GUFFIN_Q4_K) {
-        const ReceiptLayout L = receipt_layout(R, K);
-        const uint8_t* blob = reinterpret_cast<const uint8_t*>(xsums);
-        const float* mult = reinterpret_cast<const float*>(blob + L.mult_off);
-        // lane (i = lane % 16, s = lane / 16) of the A operand: variant i % 4, k-slice s
-        const uint8_t* image = blob + L.image_off + (lane & 3u) * 64u + (lane >> 4) * 16u;
         Q4Tile cur, nxt;
         if (b0 < b1) load_tile(cur, tp);
         for (uint32_t b = b0; b < b1; ++b) {
@@ -314,19 +367,25 @@ __device__ __forceinline__ void run_blocks(const uint8_t* __restrict__ wt, const
             cur = nxt;
         }
     } else if constexpr (DTYPE == GUFFIN_Q6_K) {
-        Q6Tile cur, nxt;
-        if (b0 < b1) load_tile(cur, tp, lane);
+        // A rows 0-3 / 8-11 see the first 16 elements of a group, rows 4-7 / 12-15 the second 16
+        const uint32_t keep = (((lane & 15u) >> 2) & 1u) == (lane >> 5) ? 0xFFFFFFFFu : 0u;
+        float acc2[2][R];
+#pragma unroll
+        for (int c = 0; c < 2; ++c)
+#pragma unroll
+            for (int r = 0; r < R; ++r) acc2[c][r] = 0.f;
+        Q6Tile cur;
         for (uint32_t b = b0; b < b1; ++b) {
-            if (b + 1 < b1) load_tile(nxt, tp + size_t(b + 1 - b0) * TB, lane);
-            compute_tile<R>(cur, x + size_t(b) * BE, xs + b * sums_per_block, K, per_row, acc);
-            cur = nxt;
+            load_tile(cur, tp + size_t(b - b0) * TB, lane);
+            compute_tile<R>(cur, image + size_t(b) * 2048u, keep, mult + b * 8u, K / 32, xs + b * 16u, per_row, lane, acc2);
         }
+        q6_gather<R>(acc2, lane, acc);
     } else {
         Q8Tile cur, nxt;
         if (b0 < b1) load_tile(cur, tp, lane);
         for (uint32_t b = b0; b < b1; ++b) {
             if (b + 1 < b1) load_tile(nxt, tp + size_t(b + 1 - b0) * TB, lane);
-            compute_tile<R>(cur, x + size_t(b) * BE, xs + b * sums_per_block, K, per_row, acc);
+            compute_tile<R>(cur, image + size_t(b) * 256u, mult + b, K / 32, xs + b, per_row, lane >> 4, acc);
             cur = nxt;
         }
     }

@@ -92,29 +92,47 @@ topk_merge_kernel(const float* __restrict__ logits, const uint64_t* __restrict__
     __shared__ uint32_t s_bin, s_above, s_count;
     const uint32_t row = blockIdx.x, lane = threadIdx.x & 63;
     const uint64_t* src = survivors + size_t(row) * n_survivors;
+    // up to 8 keys per thread stay in registers; longer survivor lists are re-read from memory
+    constexpr int kMine = 8;
+    const bool cached = n_survivors <= kMine * blockDim.x;
+    uint64_t mine[kMine];
+#pragma unroll
+    for (int u = 0; u < kMine; ++u) {
+        const uint32_t i = threadIdx.x + u * blockDim.x;
+        mine[u] = cached && i < n_survivors ? src[i] : 0;
+    }
     uint64_t prefix = 0;
     uint32_t remaining = retain;  // rank of the wanted key among the keys that match `prefix`
     for (int pass = 0; pass < 8; ++pass) {
         const int shift = 56 - 8 * pass;
         for (uint32_t i = threadIdx.x; i < 256; i += blockDim.x) hist[i] = 0;
         __syncthreads();
-        for (uint32_t i = threadIdx.x; i < n_survivors; i += blockDim.x) {
-            const uint64_t k = src[i];
-            if (pass == 0 || (k >> (shift + 8)) == prefix) atomicAdd(&hist[(k >> shift) & 255u], 1u);
+        if (cached) {
+#pragma unroll
+            for (int u = 0; u < kMine; ++u) {
+                const uint64_t k = mine[u];
+                if (threadIdx.x + u * blockDim.x < n_survivors && (pass == 0 || (k >> (shift + 8)) == prefix))
+                    atomicAdd(&hist[(k >> shift) & 255u], 1u);
+            }
+        } else {
+            for (uint32_t i = threadIdx.x; i < n_survivors; i += blockDim.x) {
+                const uint64_t k = src[i];
+                if (pass == 0 || (k >> (shift + 8)) == prefix) atomicAdd(&hist[(k >> shift) & 255u], 1u);
+            }
         }
         __syncthreads();
         if (threadIdx.x < 64) {  // lane l owns bins 255-4l .. 252-4l, highest first
             uint32_t c[4];
 #pragma unroll
             for (int j = 0; j < 4; ++j) c[j] = hist[255 - 4 * lane - j];
-            const uint32_t mine = c[0] + c[1] + c[2] + c[3];
-            uint32_t incl = mine;
+            const uint32_t own = c[0] + c[1] + c[2] + c[3];
+            uint32_t incl = own;
 #pragma unroll
             for (int d = 1; d < 64; d <<= 1) {
                 const uint32_t o = __shfl_up(incl, d, kWave);
                 if (lane >= uint32_t(d)) incl += o;
             }
-            uint32_t above = incl - mine;
+            uint32_t above = incl - own;
             if (above < remaining && remaining <= incl) {
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
@@ -126,15 +144,20 @@ topk_merge_kernel(const float* __restrict__ logits, const uint64_t* __restrict__
         __syncthreads();
         prefix = (prefix << 8) | s_bin;
         remaining -= s_above;
-        __syncthreads();
     }
     // `prefix` is the retain-th largest key; keys above it are taken, then `remaining` copies of it
     // (more than one only for the zero padding of a short last tile)
     if (threadIdx.x == 0) s_count = 0;
     __syncthreads();
-    for (uint32_t i = threadIdx.x; i < n_survivors; i += blockDim.x) {
-        const uint64_t k = src[i];
-        if (k > prefix) sel[atomicAdd(&s_count, 1u)] = k;
+    if (cached) {
+#pragma unroll
+        for (int u = 0; u < kMine; ++u)
+            if (threadIdx.x + u * blockDim.x < n_survivors && mine[u] > prefix) sel[atomicAdd(&s_count, 1u)] = mine[u];
+    } else {
+        for (uint32_t i = threadIdx.x; i < n_survivors; i += blockDim.x) {
+            const uint64_t k = src[i];
+            if (k > prefix) sel[atomicAdd(&s_count, 1u)] = k;
+        }
     }
     __syncthreads();
     const uint32_t above_total = s_count;

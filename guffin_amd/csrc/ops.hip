@@ -92,17 +92,33 @@ rms_norm_kernel(const float* __restrict__ x, uint32_t planes, size_t plane_strid
     float* row = lds;
     float* scratch = lds + width;
     const uint32_t r = blockIdx.x;
+    // operands of the second pass are requested before the first reduction
+    constexpr int PF = 4;
+    float gm[PF], rs[PF];
+#pragma unroll
+    for (int u = 0; u < PF; ++u) {
+        const uint32_t c = threadIdx.x + u * blockDim.x;
+        gm[u] = c < width ? gamma[c] : 0.f;
+        rs[u] = (residual && c < width) ? residual[size_t(r) * width + c] : 0.f;
+    }
     const float ss = stage_row(x + size_t(r) * width, planes, plane_stride, row, width);
     const float total = block_sum(ss, scratch);
     const float inv = 1.0f / sqrtf(total / static_cast<float>(width) + eps);
     bool bad = false;
-    for (uint32_t c = threadIdx.x; c < width; c += blockDim.x) {
-        float v = row[c] * inv * gamma[c];
-        if (residual) v += residual[size_t(r) * width + c];
+    auto second = [&](uint32_t c, float g, float res) {
+        float v = row[c] * inv * g;
+        if (residual) v += res;
         bad |= !isfinite(v);
         row[c] = v;
         y[size_t(r) * width + c] = v;
+    };
+#pragma unroll
+    for (int u = 0; u < PF; ++u) {
+        const uint32_t c = threadIdx.x + u * blockDim.x;
+        if (c < width) second(c, gm[u], rs[u]);
     }
+    for (uint32_t c = threadIdx.x + PF * blockDim.x; c < width; c += blockDim.x)
+        second(c, gamma[c], residual ? residual[size_t(r) * width + c] : 0.f);
     if (bad && status) atomicOr(status, GUFFIN_STATUS_NONFINITE);
     if (y_sums) {
         __syncthreads();
@@ -123,25 +139,49 @@ rms_norm_add_norm_kernel(const float* __restrict__ x, uint32_t planes, size_t pl
     float* row = lds;
     float* scratch = lds + width;
     const uint32_t r = blockIdx.x;
+    // operands of the second and third pass are requested before the first reduction
+    constexpr int PF = 4;
+    float gp[PF], rs[PF], gn[PF];
+#pragma unroll
+    for (int u = 0; u < PF; ++u) {
+        const uint32_t c = threadIdx.x + u * blockDim.x;
+        const bool in = c < width;
+        gp[u] = in ? gamma_post[c] : 0.f;
+        rs[u] = in ? residual[size_t(r) * width + c] : 0.f;
+        gn[u] = in ? gamma_next[c] : 0.f;
+    }
     float ss = stage_row(x + size_t(r) * width, planes, plane_stride, row, width);
     float total = block_sum(ss, scratch);
     float inv = 1.0f / sqrtf(total / static_cast<float>(width) + eps);
     ss = 0.f;
     bool bad = false;
-    for (uint32_t c = threadIdx.x; c < width; c += blockDim.x) {
-        const float v = row[c] * inv * gamma_post[c] + residual[size_t(r) * width + c];
+    auto second = [&](uint32_t c, float g, float res) {
+        const float v = row[c] * inv * g + res;
         bad |= !isfinite(v);
         row[c] = v;
         out_residual[size_t(r) * width + c] = v;
         ss = fmaf(v, v, ss);
+    };
+#pragma unroll
+    for (int u = 0; u < PF; ++u) {
+        const uint32_t c = threadIdx.x + u * blockDim.x;
+        if (c < width) second(c, gp[u], rs[u]);
     }
+    for (uint32_t c = threadIdx.x + PF * blockDim.x; c < width; c += blockDim.x)
+        second(c, gamma_post[c], residual[size_t(r) * width + c]);
     total = block_sum(ss, scratch);
     inv = 1.0f / sqrtf(total / static_cast<float>(width) + eps);
-    for (uint32_t c = threadIdx.x; c < width; c += blockDim.x) {
-        const float v = row[c] * inv * gamma_next[c];
+    auto third = [&](uint32_t c, float g) {
+        const float v = row[c] * inv * g;
         row[c] = v;
         out_norm[size_t(r) * width + c] = v;
+    };
+#pragma unroll
+    for (int u = 0; u < PF; ++u) {
+        const uint32_t c = threadIdx.x + u * blockDim.x;
+        if (c < width) third(c, gn[u]);
     }
+    for (uint32_t c = threadIdx.x + PF * blockDim.x; c < width; c += blockDim.x) third(c, gamma_next[c]);
     if (bad && status) atomicOr(status, GUFFIN_STATUS_NONFINITE);
     if (out_sums) {
         __syncthreads();

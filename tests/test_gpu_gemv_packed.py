@@ -50,10 +50,18 @@ def test_repack_round_trip_is_lossless(hip, dtype, K, N):
         assert np.array_equal(tile[(2 * cg + ch // 2) * 1024 + (16 * sl + j) * 16 + (ch % 2) * 8:][:8],
                               blk[16 + 32 * ch + 8 * sl:][:8])
     elif dtype == 2:
-        assert np.array_equal(tile[9 * 1024 + lane * 16:][:16], blk[144:160])
+        # ql byte (half n, run m, k-slice s): piece 2*cg + n, lane 16*s + j, byte 8*m; qh (half n,
+        # k-slice s): piece 8 + cg, byte 8*n; scales piece 12 and d behind the pieces, by column
+        cg, j, n, m, sl = lane // 16, lane % 16, 1, 1, 3
+        assert np.array_equal(tile[(2 * cg + n) * 1024 + (16 * sl + j) * 16 + 8 * m:][:8],
+                              blk[64 * n + 32 * m + 8 * sl:][:8])
+        assert np.array_equal(tile[(8 + cg) * 1024 + (16 * sl + j) * 16 + 8 * n:][:8], blk[128 + 32 * n + 8 * sl:][:8])
+        assert np.array_equal(tile[12288 + lane * 16:][:16], blk[192:208])
         assert np.array_equal(tile[13312 + lane * 2:][:2], blk[208:210])
     else:
-        assert np.array_equal(tile[1024 + lane * 16:][:16], blk[18:34])
+        # quant k-slice s: piece cg/2, lane 16*s + j, byte 8*(cg % 2); d behind the pieces
+        cg, j, sl = lane // 16, lane % 16, 2
+        assert np.array_equal(tile[(cg // 2) * 1024 + (16 * sl + j) * 16 + 8 * (cg % 2):][:8], blk[2 + 8 * sl:][:8])
         assert np.array_equal(tile[2048 + lane * 2:][:2], blk[0:2])
 
 
