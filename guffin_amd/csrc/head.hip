@@ -78,6 +78,20 @@ struct Candidates {  // layout of one row of the result (sampling.hpp:57-61 plus
     struct { uint32_t token; float logit; } values[384];
 };
 
+// Adds one to hist[bin] for every lane with `valid`; lanes of a wave that hit the same bin are
+// counted with one atomic (keys cluster in a few bins, and same-address LDS atomics serialise).
+__device__ __forceinline__ void hist_add(uint32_t* hist, bool valid, uint32_t bin, uint32_t lane) {
+    uint64_t todo = __ballot(valid);
+    for (int it = 0; it < 8 && todo; ++it) {
+        const int leader = __ffsll(static_cast<long long>(todo)) - 1;
+        const uint32_t b0 = __shfl(bin, leader, kWave);
+        const uint64_t same = __ballot(valid && bin == b0) & todo;
+        if (lane == uint32_t(leader)) atomicAdd(&hist[b0], static_cast<uint32_t>(__popcll(same)));
+        todo &= ~same;
+    }
+    if ((todo >> lane) & 1u) atomicAdd(&hist[bin], 1u);
+}
+
 // Stage 2: exact selection of the best `retain` of n unique keys by an 8-pass radix select
 // (one byte per pass, most significant first: a 256-bin histogram in LDS, then the bin that
 // holds the retain-th largest key), followed by a rank sort of the selected keys.
@@ -111,13 +125,15 @@ topk_merge_kernel(const float* __restrict__ logits, const uint64_t* __restrict__
 #pragma unroll
             for (int u = 0; u < kMine; ++u) {
                 const uint64_t k = mine[u];
-                if (threadIdx.x + u * blockDim.x < n_survivors && (pass == 0 || (k >> (shift + 8)) == prefix))
-                    atomicAdd(&hist[(k >> shift) & 255u], 1u);
+                hist_add(hist, threadIdx.x + u * blockDim.x < n_survivors && (pass == 0 || (k >> (shift + 8)) == prefix),
+                         static_cast<uint32_t>(k >> shift) & 255u, lane);
             }
         } else {
-            for (uint32_t i = threadIdx.x; i < n_survivors; i += blockDim.x) {
-                const uint64_t k = src[i];
-                if (pass == 0 || (k >> (shift + 8)) == prefix) atomicAdd(&hist[(k >> shift) & 255u], 1u);
+            for (uint32_t i0 = 0; i0 < n_survivors; i0 += blockDim.x) {  // whole waves stay converged
+                const uint32_t i = i0 + threadIdx.x;
+                const uint64_t k = i < n_survivors ? src[i] : 0;
+                hist_add(hist, i < n_survivors && (pass == 0 || (k >> (shift + 8)) == prefix),
+                         static_cast<uint32_t>(k >> shift) & 255u, lane);
             }
         }
         __syncthreads();
