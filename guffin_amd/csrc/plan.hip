@@ -253,6 +253,106 @@ extern "C" int guffin_hip_commit_rows(void* stream, const guffin_model_desc* mod
     return check_launch("commit_rows");
 }
 
+// ---- prefill: a run of rows through every block --------------------------------------------
+namespace guffin {
+namespace {
+
+struct PrefillScratch {
+    float *x, *x1, *u, *q, *kraw, *vraw, *a, *gate, *up, *h, *o;
+    float *rope_local, *rope_global;
+    uint16_t *run_k, *run_v;
+    uint8_t* image;
+    uint32_t* positions;
+    uint64_t bytes;
+};
+
+PrefillScratch prefill_layout(const guffin_model_desc& m, uint32_t rows, uint8_t* base) {
+    Arena ar {base, 0, 0};
+    const uint64_t H = m.hidden, F = m.ffn, QW = uint64_t(m.q_heads) * m.head_dim, KW = uint64_t(m.kv_heads) * m.head_dim;
+    PrefillScratch s {};
+    s.x = ar.take<float>(rows * H); s.x1 = ar.take<float>(rows * H); s.u = ar.take<float>(rows * H);
+    s.o = ar.take<float>(rows * H);
+    s.q = ar.take<float>(rows * QW); s.a = ar.take<float>(rows * QW);
+    s.kraw = ar.take<float>(rows * KW); s.vraw = ar.take<float>(rows * KW);
+    s.gate = ar.take<float>(rows * F); s.up = ar.take<float>(rows * F); s.h = ar.take<float>(rows * F);
+    s.rope_local = ar.take<float>(uint64_t(rows) * m.head_dim);
+    s.rope_global = ar.take<float>(uint64_t(rows) * m.head_dim);
+    s.run_k = ar.take<uint16_t>(rows * KW); s.run_v = ar.take<uint16_t>(rows * KW);
+    const uint32_t widest = std::max({m.hidden, m.ffn, m.q_heads * m.head_dim});
+    s.image = ar.take<uint8_t>(guffin_hip_prefill_image_bytes(rows, widest));
+    s.positions = ar.take<uint32_t>(rows);
+    s.bytes = (ar.used + 255) & ~uint64_t{255};
+    return s;
+}
+
+__global__ void fill_positions_kernel(uint32_t* positions, uint32_t rows, uint32_t position) {
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < rows) positions[i] = position + i;
+}
+
+}  // namespace
+}  // namespace guffin
+
+extern "C" uint64_t guffin_hip_prefill_scratch_bytes(const guffin_model_desc* model, uint32_t rows) {
+    if (!model || rows == 0 || guffin::validate_model(model)) return 0;
+    return guffin::prefill_layout(*model, rows, nullptr).bytes;
+}
+
+extern "C" int guffin_hip_prefill_rows(void* stream, const guffin_model_desc* model, const uint32_t* tokens,
+                                       uint32_t rows, uint32_t position, void* scratch, uint64_t scratch_bytes,
+                                       float* out_hidden, uint32_t* status) {
+    using namespace guffin;
+    if (!tokens || !scratch || !out_hidden || !status) return fail(GUFFIN_E_ARG, "prefill_rows: null pointer");
+    GUFFIN_TRY(validate_model(model));
+    if (rows == 0) return fail(GUFFIN_E_SHAPE, "prefill_rows: no rows");
+    if (reinterpret_cast<uintptr_t>(scratch) & 255u) return fail(GUFFIN_E_ALIGN, "prefill_rows: scratch must be 256-byte aligned");
+    const guffin_model_desc& m = *model;
+    const PrefillScratch s = prefill_layout(m, rows, static_cast<uint8_t*>(scratch));
+    if (s.bytes > scratch_bytes) return fail(GUFFIN_E_CAPACITY, "prefill_rows: scratch arena too small");
+    hipStream_t hs = as_stream(stream);
+    const uint32_t H = m.hidden, F = m.ffn, QW = m.q_heads * m.head_dim, KW = m.kv_heads * m.head_dim;
+    const float attn_scale = 1.0f / std::sqrt(static_cast<float>(m.head_dim));
+    hipLaunchKernelGGL(fill_positions_kernel, dim3((rows + 255) / 256), dim3(256), 0, hs, s.positions, rows, position);
+    GUFFIN_TRY(check_launch("prefill positions"));
+    GUFFIN_TRY(guffin_hip_rope_table(stream, s.positions, s.rope_local, rows, m.head_dim, m.local_base, 1.0f));
+    GUFFIN_TRY(guffin_hip_rope_table(stream, s.positions, s.rope_global, rows, m.head_dim, m.global_base, m.global_scale));
+    GUFFIN_TRY(guffin_hip_embed(stream, m.embed_dtype, m.embed_rows, tokens, s.x, rows, H,
+                                std::sqrt(static_cast<float>(H)), m.vocab, status));
+    GUFFIN_TRY(guffin_hip_rms_norm(stream, s.x, 1, 0, m.layers[0].norm[0], nullptr, s.u, nullptr, rows, H, m.eps, status));
+    for (uint32_t l = 0; l < m.layer_count; ++l) {
+        const guffin_layer_desc& L = m.layers[l];
+        const bool local = is_local(m, l);
+        const float base = local ? m.local_base : m.global_base, scale = local ? 1.0f : m.global_scale;
+        const uint32_t ring_mask = (local ? m.ring_local : m.ring_global) - 1;
+        GUFFIN_TRY(guffin_hip_prefill_pack(stream, s.u, s.image, rows, H));
+        GUFFIN_TRY(guffin_hip_prefill_gemm(stream, L.dtype[0], L.tiles[0], s.image, s.q, rows, H, QW));
+        GUFFIN_TRY(guffin_hip_prefill_gemm(stream, L.dtype[1], L.tiles[1], s.image, s.kraw, rows, H, KW));
+        GUFFIN_TRY(guffin_hip_prefill_gemm(stream, L.dtype[2], L.tiles[2], s.image, s.vraw, rows, H, KW));
+        GUFFIN_TRY(guffin_hip_qkv_post(stream, s.q, s.kraw, s.vraw, 1, 1, 1, 0, 0, 0, L.norm[1], L.norm[2], s.positions,
+                                       s.q, s.run_k, s.run_v, rows, m.q_heads, m.kv_heads, m.head_dim, m.head_dim, base,
+                                       scale, m.eps, local ? s.rope_local : s.rope_global, status));
+        GUFFIN_TRY(guffin_hip_prefill_attention(stream, s.q, L.ring_k, L.ring_v, s.run_k, s.run_v, s.a, rows, position,
+                                                local ? m.sliding_window : 0u, ring_mask, m.q_heads, m.kv_heads,
+                                                m.head_dim, attn_scale));
+        GUFFIN_TRY(guffin_hip_publish_run(stream, s.run_k, s.run_v, L.ring_k, L.ring_v, rows, position, ring_mask, KW));
+        GUFFIN_TRY(guffin_hip_prefill_pack(stream, s.a, s.image, rows, QW));
+        GUFFIN_TRY(guffin_hip_prefill_gemm(stream, L.dtype[3], L.tiles[3], s.image, s.o, rows, QW, H));
+        GUFFIN_TRY(guffin_hip_rms_norm_add_norm(stream, s.o, 1, 0, L.norm[3], s.x, s.x1, L.norm[4], s.u, nullptr, rows, H,
+                                                m.eps, status));
+        GUFFIN_TRY(guffin_hip_prefill_pack(stream, s.u, s.image, rows, H));
+        GUFFIN_TRY(guffin_hip_prefill_gemm(stream, L.dtype[4], L.tiles[4], s.image, s.gate, rows, H, F));
+        GUFFIN_TRY(guffin_hip_prefill_gemm(stream, L.dtype[5], L.tiles[5], s.image, s.up, rows, H, F));
+        GUFFIN_TRY(guffin_hip_geglu(stream, s.gate, s.up, 1, 0, s.h, nullptr, rows, F));
+        GUFFIN_TRY(guffin_hip_prefill_pack(stream, s.h, s.image, rows, F));
+        GUFFIN_TRY(guffin_hip_prefill_gemm(stream, L.dtype[6], L.tiles[6], s.image, s.o, rows, F, H));
+        const bool last = l + 1 == m.layer_count;
+        GUFFIN_TRY(guffin_hip_rms_norm_add_norm(stream, s.o, 1, 0, L.norm[5], s.x1, s.x,
+                                                last ? m.out_norm : m.layers[l + 1].norm[0], last ? out_hidden : s.u,
+                                                nullptr, rows, H, m.eps, status));
+    }
+    return GUFFIN_OK;
+}
+
 // ---- one H1 cycle ---------------------------------------------------------------------
 extern "C" uint64_t guffin_hip_h1_scratch_bytes(const guffin_h1_desc* d) {
     if (!d || validate_model(d->target) || validate_model(d->drafter)) return 0;

@@ -1,0 +1,468 @@
+// Chunked prefill on the matrix core (gfx950): M rows x quantised weights, and causal GQA
+// attention over the fp16 KV rings for a run of consecutive positions.
+//
+// Replaces the reference's prefill matrix path (src/tensor/backends/metal/metal_kernels.mm:
+// 1031-1199, dispatch rules metal_command_context.mm:384-401) and encode_f16_prefill_attention
+// (metal_command_context.hpp:185, kernels metal_kernels.mm:2593-2800).
+//
+// GEMM.  Same wave tiles and the same exact-operand idea as the packed GEMV: quants enter
+// v_mfma_f32_16x16x32_f16 as fp16 subnormals (B), activations as an fp16 hi/lo image (A).  With
+// many rows the 16 A rows are 8 activation rows x {hi, lo}, so nothing is replicated: after
+// one MFMA lane (j, g) holds, for column 16*cg + j, rows 2g and 2g+1 of the row group as
+// (hi, lo) pairs.  A wave owns 64 columns x 32 rows (4 row groups), a workgroup 4 such waves on
+// the same tile (128 rows), so a weight tile is fetched from HBM once per 128 rows.  Block
+// scales and the per-(row, 32-group) activation multipliers are applied to each MFMA result in
+// fp32; the offset terms use per-(row, 32-group) sums (Q6_K: per 16-group).
+//
+// Attention.  A workgroup serves 16 consecutive query rows of one KV head (all query heads of the
+// group) and walks the visible key range in tiles of 32 tokens through LDS with an online
+// softmax, fp32 math on fp16 keys/values: positions before the run come from the ring, the run's
+// own positions from its private rows, which are published to the ring afterwards.
+#include "common.hpp"
+
+namespace guffin {
+namespace {
+
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+
+constexpr uint32_t kCols = 64;       // columns per wave tile
+constexpr uint32_t kWaveRows = 32;   // rows per wave (4 row groups of 8)
+constexpr uint32_t kChunkRows = 128; // rows per workgroup
+
+__host__ __device__ constexpr uint32_t block_bytes(int dtype) {
+    return dtype == GUFFIN_Q8_0 ? 34u : dtype == GUFFIN_Q4_K ? 144u : 210u;
+}
+__host__ __device__ constexpr uint32_t block_elems(int dtype) { return dtype == GUFFIN_Q8_0 ? 32u : 256u; }
+
+// ---- activation image of M rows --------------------------------------------------------
+// image: half [K/32][Mpad/8][16][32]   A row 2*(row % 8) + {0 hi, 1 lo}; inside a group the halves
+//                                      of elements 8s..8s+7 sit at 8s + {0,2,1,3,4,6,5,7}
+// mult : float [K/32][Mpad]            2^(E+24) of (row, group)
+// s32  : float [K/32][Mpad]            sum of the group's 32 activations
+// s16  : float [K/16][Mpad]            sums of 16
+struct ImageLayout { size_t mult_off, s32_off, s16_off, bytes; uint32_t mpad; };
+
+__host__ __device__ inline ImageLayout image_layout(uint32_t M, uint32_t K) {
+    const uint32_t mpad = (M + kChunkRows - 1) / kChunkRows * kChunkRows;
+    ImageLayout L {};
+    L.mpad = mpad;
+    L.mult_off = size_t(K / 32) * mpad * 128;  // 16 A rows x 64 B per 8 rows = 128 B per row and group
+    L.s32_off = L.mult_off + size_t(K / 32) * mpad * 4;
+    L.s16_off = L.s32_off + size_t(K / 32) * mpad * 4;
+    L.bytes = L.s16_off + size_t(K / 16) * mpad * 4;
+    return L;
+}
+
+// one thread per (row, group, k-slice); four consecutive lanes share a group
+__global__ void __launch_bounds__(256)
+prefill_pack_kernel(const float* __restrict__ x, uint8_t* __restrict__ blob, uint32_t M, uint32_t K) {
+    const ImageLayout L = image_layout(M, K);
+    const uint32_t groups = K / 32;
+    const uint64_t t = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (t >= uint64_t(L.mpad) * groups * 4) return;
+    const uint32_t s = t & 3u, g = (t >> 2) % groups, row = static_cast<uint32_t>((t >> 2) / groups);
+    float v[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = row < M ? x[size_t(row) * K + g * 32 + s * 8 + i] : 0.f;
+    float sum = v[0], m = fabsf(v[0]);
+#pragma unroll
+    for (int i = 1; i < 8; ++i) { sum += v[i]; m = fmaxf(m, fabsf(v[i])); }
+    m = fmaxf(m, __shfl_xor(m, 1, kWave));
+    m = fmaxf(m, __shfl_xor(m, 2, kWave));
+    const float sum16 = sum + __shfl_xor(sum, 1, kWave);
+    const float sum32 = sum16 + __shfl_xor(sum16, 2, kWave);
+    uint32_t eb = __float_as_uint(m) >> 23;
+    eb = eb < 14u ? 14u : eb > 244u ? 244u : eb;
+    const float inv = __uint_as_float((268u - eb) << 23);
+    float* mult = reinterpret_cast<float*>(blob + L.mult_off);
+    float* s32 = reinterpret_cast<float*>(blob + L.s32_off);
+    float* s16 = reinterpret_cast<float*>(blob + L.s16_off);
+    if (s == 0) { mult[size_t(g) * L.mpad + row] = __uint_as_float((eb + 10u) << 23); s32[size_t(g) * L.mpad + row] = sum32; }
+    if ((s & 1u) == 0) s16[size_t(2 * g + (s >> 1)) * L.mpad + row] = sum16;
+    uint32_t hi[4], lo[4];
+    constexpr int order[8] = {0, 2, 1, 3, 4, 6, 5, 7};
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+        uint32_t hw = 0, lw = 0;
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+            const float xv = v[order[2 * p + q]] * inv;
+            const _Float16 h = static_cast<_Float16>(xv);
+            const _Float16 l = static_cast<_Float16>(xv - static_cast<float>(h));
+            hw |= uint32_t(__builtin_bit_cast(uint16_t, h)) << (16 * q);
+            lw |= uint32_t(__builtin_bit_cast(uint16_t, l)) << (16 * q);
+        }
+        hi[p] = hw; lo[p] = lw;
+    }
+    uint8_t* base = blob + ((size_t(g) * (L.mpad / 8) + row / 8) * 16 + 2 * (row % 8)) * 64 + s * 16;
+    *reinterpret_cast<uint4*>(base) = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+    *reinterpret_cast<uint4*>(base + 64) = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+}
+
+__device__ __forceinline__ half8_t as_half8(uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
+    return __builtin_bit_cast(half8_t, make_uint4(a, b, c, d));
+}
+__device__ __forceinline__ uint32_t even_bytes(uint32_t v) { return __builtin_amdgcn_perm(0u, v, 0x0c020c00u); }
+__device__ __forceinline__ uint32_t odd_bytes(uint32_t v) { return __builtin_amdgcn_perm(0u, v, 0x0c030c01u); }
+__device__ __forceinline__ float sbyte(uint32_t w, int i) {
+    return i == 0 ? sb0(w) : i == 1 ? sb1(w) : i == 2 ? sb2(w) : sb3(w);
+}
+__device__ __forceinline__ float ubyte(uint32_t w, int i) {
+    return i == 0 ? ub0(w) : i == 1 ? ub1(w) : i == 2 ? ub2(w) : ub3(w);
+}
+
+// what a wave needs of the image for one 32-group: the A operands of its 4 row groups and the
+// multipliers / sums of the lane's two rows per row group
+struct GroupOperands {
+    half8_t a[4];
+    float2 mult[4];
+};
+
+struct WaveCtx {
+    const uint8_t* image;   // + lane offset inside a (group, row group) record
+    const float* mult; const float* s32; const float* s16;
+    uint32_t mpad, rg0, row0;  // first row group / first of the lane's rows of row group 0
+};
+
+__device__ __forceinline__ void load_group(const WaveCtx& c, uint32_t g, GroupOperands& o) {
+#pragma unroll
+    for (int rg = 0; rg < 4; ++rg) {
+        o.a[rg] = __builtin_bit_cast(half8_t, *reinterpret_cast<const uint4*>(
+            c.image + (size_t(g) * (c.mpad / 8) + c.rg0 + rg) * 1024));
+        o.mult[rg] = *reinterpret_cast<const float2*>(c.mult + size_t(g) * c.mpad + c.row0 + 8 * rg);
+    }
+}
+
+// acc[rg][2] += f * mult * (hi + lo sums) for the lane's two rows of every row group
+__device__ __forceinline__ void mfma_scale(const GroupOperands& o, half8_t b, float f, float (&acc)[4][2]) {
+    const float4_t zero = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int rg = 0; rg < 4; ++rg) {
+        const float4_t d = __builtin_amdgcn_mfma_f32_16x16x32_f16(o.a[rg], b, zero, 0, 0, 0);
+        acc[rg][0] = fmaf(f * o.mult[rg].x, d[0] + d[1], acc[rg][0]);
+        acc[rg][1] = fmaf(f * o.mult[rg].y, d[2] + d[3], acc[rg][1]);
+    }
+}
+
+__device__ __forceinline__ void add_offset(const float* sums, const WaveCtx& c, uint32_t index, float f, float (&acc)[4][2]) {
+#pragma unroll
+    for (int rg = 0; rg < 4; ++rg) {
+        const float2 s = *reinterpret_cast<const float2*>(sums + size_t(index) * c.mpad + c.row0 + 8 * rg);
+        acc[rg][0] = fmaf(f, s.x, acc[rg][0]);
+        acc[rg][1] = fmaf(f, s.y, acc[rg][1]);
+    }
+}
+
+// grid (N/64, Mpad/128), 256 threads.  y[M][N] fp32.
+template <int DTYPE>
+__global__ void __launch_bounds__(256)
+prefill_gemm_kernel(const uint8_t* __restrict__ tiles, const uint8_t* __restrict__ blob, float* __restrict__ y,
+                    uint32_t M, uint32_t K, uint32_t N) {
+    constexpr uint32_t TB = kCols * block_bytes(DTYPE);
+    const ImageLayout L = image_layout(M, K);
+    const uint32_t lane = threadIdx.x & 63, wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t j = lane & 15, lg = lane >> 4;
+    const uint32_t nblk = K / block_elems(DTYPE);
+    WaveCtx c;
+    c.mpad = L.mpad;
+    c.rg0 = (blockIdx.y * kChunkRows + wv * kWaveRows) / 8;
+    c.row0 = blockIdx.y * kChunkRows + wv * kWaveRows + 2 * lg;
+    c.image = blob + (lane & 15u) * 64 + (lane >> 4) * 16;  // A lane (i = lane % 16, s = lane / 16): row i, k-slice s
+    c.mult = reinterpret_cast<const float*>(blob + L.mult_off);
+    c.s32 = reinterpret_cast<const float*>(blob + L.s32_off);
+    c.s16 = reinterpret_cast<const float*>(blob + L.s16_off);
+    if (blockIdx.y * kChunkRows + wv * kWaveRows >= M) return;  // a wave of padding rows only
+    float acc[4][4][2];  // [column group][row group][row of the lane]
+#pragma unroll
+    for (int cg = 0; cg < 4; ++cg)
+#pragma unroll
+        for (int rg = 0; rg < 4; ++rg) { acc[cg][rg][0] = 0.f; acc[cg][rg][1] = 0.f; }
+    const uint8_t* tp = tiles + size_t(blockIdx.x) * nblk * TB;
+    for (uint32_t b = 0; b < nblk; ++b, tp += TB) {
+        if constexpr (DTYPE == GUFFIN_Q4_K) {
+            uint4 q[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) q[i] = *reinterpret_cast<const uint4*>(tp + 1024 * i + lane * 16);
+#pragma unroll
+            for (int ch = 0; ch < 4; ++ch) {
+                GroupOperands lo, hi;
+                load_group(c, b * 8 + 2 * ch, lo);
+                load_group(c, b * 8 + 2 * ch + 1, hi);
+#pragma unroll
+                for (int cg = 0; cg < 4; ++cg) {
+                    const uint4 hdr = *reinterpret_cast<const uint4*>(tp + 8192 + (16 * cg + j) * 16);
+                    const float d = h2f(hdr.x & 0xFFFFu), dmin = h2f(hdr.x >> 16);
+                    const uint32_t sc_a = hdr.y & 0x3F3F3F3Fu, mn_a = hdr.z & 0x3F3F3F3Fu;
+                    const uint32_t sc_b = (hdr.w & 0x0F0F0F0Fu) | ((hdr.y >> 2) & 0x30303030u);
+                    const uint32_t mn_b = ((hdr.w >> 4) & 0x0F0F0F0Fu) | ((hdr.z >> 2) & 0x30303030u);
+                    const uint32_t scw = ch < 2 ? sc_a : sc_b, mnw = ch < 2 ? mn_a : mn_b;
+                    const float sc_lo = ubyte(scw, 2 * (ch & 1)), sc_hi = ubyte(scw, 2 * (ch & 1) + 1);
+                    const float mn_lo = ubyte(mnw, 2 * (ch & 1)), mn_hi = ubyte(mnw, 2 * (ch & 1) + 1);
+                    const uint4 piece = q[2 * cg + (ch >> 1)];
+                    const uint32_t w0 = (ch & 1) ? piece.z : piece.x, w1 = (ch & 1) ? piece.w : piece.y;
+                    const uint32_t v0 = w0 >> 8, v1 = w1 >> 8;
+                    mfma_scale(lo, as_half8(w0 & 0x000F000Fu, v0 & 0x000F000Fu, w1 & 0x000F000Fu, v1 & 0x000F000Fu),
+                               d * sc_lo, acc[cg]);
+                    mfma_scale(hi, as_half8(w0 & 0x00F000F0u, v0 & 0x00F000F0u, w1 & 0x00F000F0u, v1 & 0x00F000F0u),
+                               d * 0.0625f * sc_hi, acc[cg]);
+                    add_offset(c.s32, c, b * 8 + 2 * ch, -dmin * mn_lo, acc[cg]);
+                    add_offset(c.s32, c, b * 8 + 2 * ch + 1, -dmin * mn_hi, acc[cg]);
+                }
+            }
+        } else if constexpr (DTYPE == GUFFIN_Q6_K) {
+            uint4 ql[8], qh[4];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) ql[i] = *reinterpret_cast<const uint4*>(tp + 1024 * i + lane * 16);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) qh[i] = *reinterpret_cast<const uint4*>(tp + 8192 + 1024 * i + lane * 16);
+            // a scale covers 16 elements: the two halves of a 32-group go through separate MFMAs with
+            // the other half's lanes (k-slices) zeroed
+            const uint32_t keep_first = lane < 32 ? 0xFFFFFFFFu : 0u;
+#pragma unroll
+            for (int g = 0; g < 8; ++g) {
+                const int n = g >> 2, qd = g & 3;
+                GroupOperands o;
+                load_group(c, b * 8 + g, o);
+#pragma unroll
+                for (int cg = 0; cg < 4; ++cg) {
+                    const uint4 scv = *reinterpret_cast<const uint4*>(tp + 12288 + (16 * cg + j) * 16);
+                    const float d = h2f(*reinterpret_cast<const uint16_t*>(tp + 13312 + (16 * cg + j) * 2));
+                    const int word = g >> 1;
+                    const uint32_t sw = word == 0 ? scv.x : word == 1 ? scv.y : word == 2 ? scv.z : scv.w;
+                    const float s_first = sbyte(sw, 2 * (g & 1)), s_second = sbyte(sw, 2 * (g & 1) + 1);
+                    const uint4 lq = ql[2 * cg + n], hq = qh[cg];
+                    const uint32_t w0 = (qd & 1) ? lq.z : lq.x, w1 = (qd & 1) ? lq.w : lq.y;
+                    const uint32_t h0 = n ? hq.z : hq.x, h1 = n ? hq.w : hq.y;
+                    const int ls = qd >= 2 ? 4 : 0;
+                    uint32_t bq[4];
+#pragma unroll
+                    for (int k = 0; k < 2; ++k) {
+                        const uint32_t w = k ? w1 : w0, h = k ? h1 : h0;
+                        const uint32_t lo0 = (w >> ls) & 0x000F000Fu, lo1 = (w >> (ls + 8)) & 0x000F000Fu;
+                        const uint32_t hs0 = qd == 0 ? h << 4 : qd == 1 ? h << 2 : qd == 2 ? h : h >> 2;
+                        const uint32_t hs1 = h >> (4 + 2 * qd);
+                        bq[2 * k] = (hs0 & 0x00300030u) | lo0;
+                        bq[2 * k + 1] = (hs1 & 0x00300030u) | lo1;
+                    }
+                    mfma_scale(o, as_half8(bq[0] & keep_first, bq[1] & keep_first, bq[2] & keep_first, bq[3] & keep_first),
+                               d * s_first, acc[cg]);
+                    mfma_scale(o, as_half8(bq[0] & ~keep_first, bq[1] & ~keep_first, bq[2] & ~keep_first, bq[3] & ~keep_first),
+                               d * s_second, acc[cg]);
+                    add_offset(c.s16, c, (b * 8 + g) * 2, -32.0f * d * s_first, acc[cg]);
+                    add_offset(c.s16, c, (b * 8 + g) * 2 + 1, -32.0f * d * s_second, acc[cg]);
+                }
+            }
+        } else {
+            const uint4 q0 = *reinterpret_cast<const uint4*>(tp + lane * 16);
+            const uint4 q1 = *reinterpret_cast<const uint4*>(tp + 1024 + lane * 16);
+            GroupOperands o;
+            load_group(c, b, o);
+#pragma unroll
+            for (int cg = 0; cg < 4; ++cg) {
+                const float d = h2f(*reinterpret_cast<const uint16_t*>(tp + 2048 + (16 * cg + j) * 2));
+                const uint4 piece = cg < 2 ? q0 : q1;
+                const uint32_t w0 = ((cg & 1) ? piece.z : piece.x) ^ 0x80808080u, w1 = ((cg & 1) ? piece.w : piece.y) ^ 0x80808080u;
+                mfma_scale(o, as_half8(even_bytes(w0), odd_bytes(w0), even_bytes(w1), odd_bytes(w1)), d, acc[cg]);
+                add_offset(c.s32, c, b, -128.0f * d, acc[cg]);
+            }
+        }
+    }
+#pragma unroll
+    for (int cg = 0; cg < 4; ++cg)
+#pragma unroll
+        for (int rg = 0; rg < 4; ++rg)
+#pragma unroll
+            for (int r = 0; r < 2; ++r) {
+                const uint32_t row = c.row0 + 8 * rg + r;
+                if (row < M) y[size_t(row) * N + blockIdx.x * kCols + 16 * cg + j] = acc[cg][rg][r];
+            }
+}
+
+// ---- causal attention for a run of rows ------------------------------------------------
+// grid (ceil(rows / 16), kv_heads), 256 threads: thread = (query slot of 16 rows x GROUP heads, one of
+// 256/(16*GROUP) interleaved dim slices).  Keys/values of positions below `position` come from the
+// ring, those of the run itself from its private fp16 rows [rows][kv_heads*256].
+template <int GROUP>
+__global__ void __launch_bounds__(256)
+prefill_attention_kernel(const float* __restrict__ q, const uint16_t* __restrict__ ring_k,
+                         const uint16_t* __restrict__ ring_v, const uint16_t* __restrict__ run_k,
+                         const uint16_t* __restrict__ run_v, float* __restrict__ out, uint32_t rows,
+                         uint32_t position, uint32_t window, uint32_t ring_mask, uint32_t q_heads,
+                         uint32_t kv_heads, float scale) {
+    constexpr int HD = 256, QT = 16, NQ = QT * GROUP, KT = 32;
+    constexpr int TPQ = 256 / NQ;        // threads per query: 16, 8 or 4
+    constexpr int DPT = HD / TPQ;        // dims per thread, interleaved: dim = part + TPQ * i
+    __shared__ _Float16 ks[KT][HD + 2];
+    __shared__ _Float16 vs[KT][HD + 2];
+    __shared__ float sc[NQ][KT];
+    const uint32_t kvh = blockIdx.y, r0 = blockIdx.x * QT;
+    const uint32_t qi = threadIdx.x / TPQ, part = threadIdx.x % TPQ;
+    const uint32_t row = r0 + qi / GROUP, head = kvh * GROUP + qi % GROUP;
+    const bool live = row < rows;
+    const uint32_t pos = position + row;
+    float qv[DPT], acc[DPT];
+#pragma unroll
+    for (int i = 0; i < DPT; ++i) {
+        qv[i] = live ? q[(size_t(row) * q_heads + head) * HD + part + TPQ * i] * scale : 0.f;
+        acc[i] = 0.f;
+    }
+    float mx = -INFINITY, den = 0.f;
+    const uint32_t last_row = min(r0 + QT, rows) - 1;
+    const uint32_t hi_pos = position + last_row;
+    const uint32_t lo_first = (window && position + r0 + 1 > window) ? position + r0 + 1 - window : 0;
+    const uint32_t my_first = (window && pos + 1 > window) ? pos + 1 - window : 0;
+    const size_t row_stride = size_t(kv_heads) * HD;
+    for (uint32_t t0 = lo_first; t0 <= hi_pos; t0 += KT) {
+        __syncthreads();
+        for (uint32_t i = threadIdx.x; i < KT * HD / 2; i += 256) {
+            const uint32_t t = i / (HD / 2), d2 = i % (HD / 2);
+            uint32_t kk = 0, vv = 0;
+            const uint32_t kp = t0 + t;
+            if (kp <= hi_pos) {
+                const bool own = kp >= position;
+                const size_t off = (own ? size_t(kp - position) : size_t(kp & ring_mask)) * row_stride + kvh * HD + 2 * d2;
+                kk = *reinterpret_cast<const uint32_t*>((own ? run_k : ring_k) + off);
+                vv = *reinterpret_cast<const uint32_t*>((own ? run_v : ring_v) + off);
+            }
+            *reinterpret_cast<uint32_t*>(&ks[t][2 * d2]) = kk;
+            *reinterpret_cast<uint32_t*>(&vs[t][2 * d2]) = vv;
+        }
+        __syncthreads();
+        float tile_max = -INFINITY;
+        float s_loc[KT / TPQ];
+        for (int t = 0; t < KT; ++t) {
+            float s = 0.f;
+#pragma unroll
+            for (int i = 0; i < DPT; ++i) s = fmaf(qv[i], static_cast<float>(ks[t][part + TPQ * i]), s);
+#pragma unroll
+            for (int o = TPQ / 2; o > 0; o >>= 1) s += __shfl_xor(s, o, kWave);
+            const uint32_t kp = t0 + t;
+            const bool visible = live && kp <= pos && kp >= my_first;
+            s = visible ? s : -INFINITY;
+            if (uint32_t(t) % TPQ == part) s_loc[t / TPQ] = s;
+            tile_max = fmaxf(tile_max, s);
+        }
+        const float new_max = fmaxf(mx, tile_max);
+        const float rescale = new_max == -INFINITY ? 1.f : expf(mx - new_max);
+        den *= rescale;
+#pragma unroll
+        for (int i = 0; i < DPT; ++i) acc[i] *= rescale;
+        float add = 0.f;
+#pragma unroll
+        for (int u = 0; u < KT / TPQ; ++u) {
+            const float p = s_loc[u] == -INFINITY ? 0.f : expf(s_loc[u] - new_max);
+            sc[qi][u * TPQ + part] = p;
+            add += p;
+        }
+#pragma unroll
+        for (int o = TPQ / 2; o > 0; o >>= 1) add += __shfl_xor(add, o, kWave);
+        den += add;
+        mx = new_max;
+        // the TPQ lanes of a query sit in one wave: their sc[] entries are visible after a wave barrier
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        for (int t = 0; t < KT; ++t) {
+            const float p = sc[qi][t];
+#pragma unroll
+            for (int i = 0; i < DPT; ++i) acc[i] = fmaf(p, static_cast<float>(vs[t][part + TPQ * i]), acc[i]);
+        }
+    }
+    if (live) {
+#pragma unroll
+        for (int i = 0; i < DPT; ++i) out[(size_t(row) * q_heads + head) * HD + part + TPQ * i] = acc[i] / den;
+    }
+}
+
+// ring[(position + row) & mask] = run[row] for the rows that survive in a ring of this capacity
+__global__ void publish_run_kernel(const uint4* __restrict__ run_k, const uint4* __restrict__ run_v,
+                                   uint4* __restrict__ ring_k, uint4* __restrict__ ring_v, uint32_t rows,
+                                   uint32_t first_row, uint32_t position, uint32_t ring_mask, uint32_t row_vec) {
+    const uint64_t i = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i >= uint64_t(rows - first_row) * row_vec) return;
+    const uint32_t row = first_row + static_cast<uint32_t>(i / row_vec), c = static_cast<uint32_t>(i % row_vec);
+    const size_t dst = size_t((position + row) & ring_mask) * row_vec + c;
+    ring_k[dst] = run_k[size_t(row) * row_vec + c];
+    ring_v[dst] = run_v[size_t(row) * row_vec + c];
+}
+
+}  // namespace
+}  // namespace guffin
+
+using namespace guffin;
+
+extern "C" int guffin_hip_publish_run(void* stream, const void* run_k, const void* run_v, void* ring_k, void* ring_v,
+                                      uint32_t rows, uint32_t position, uint32_t ring_mask, uint32_t row_width) {
+    if (!run_k || !run_v || !ring_k || !ring_v) return fail(GUFFIN_E_ARG, "publish_run: null pointer");
+    if (rows == 0 || row_width == 0 || row_width % 8 != 0) return fail(GUFFIN_E_SHAPE, "publish_run: row width must be a multiple of 8 halves");
+    if ((ring_mask & (ring_mask + 1)) != 0) return fail(GUFFIN_E_ARG, "publish_run: ring capacity must be a power of two");
+    const uint32_t first = rows > ring_mask + 1 ? rows - (ring_mask + 1) : 0;  // older rows would be overwritten anyway
+    const uint64_t n = uint64_t(rows - first) * (row_width / 8);
+    hipLaunchKernelGGL(publish_run_kernel, dim3(static_cast<uint32_t>((n + 255) / 256)), dim3(256), 0, as_stream(stream),
+                       static_cast<const uint4*>(run_k), static_cast<const uint4*>(run_v), static_cast<uint4*>(ring_k),
+                       static_cast<uint4*>(ring_v), rows, first, position, ring_mask, row_width / 8);
+    return check_launch("publish_run");
+}
+
+extern "C" uint64_t guffin_hip_prefill_image_bytes(uint32_t M, uint32_t K) {
+    if (M == 0 || K == 0 || K % 32 != 0) return 0;
+    return image_layout(M, K).bytes;
+}
+
+extern "C" int guffin_hip_prefill_pack(void* stream, const float* x, void* image, uint32_t M, uint32_t K) {
+    if (!x || !image) return fail(GUFFIN_E_ARG, "prefill_pack: null pointer");
+    if (M == 0 || K == 0 || K % 32 != 0) return fail(GUFFIN_E_SHAPE, "prefill_pack: K must be a positive multiple of 32");
+    if (reinterpret_cast<uintptr_t>(image) & 255u) return fail(GUFFIN_E_ALIGN, "prefill_pack: the image must be 256-byte aligned");
+    const ImageLayout L = image_layout(M, K);
+    const uint64_t threads = uint64_t(L.mpad) * (K / 32) * 4;
+    hipLaunchKernelGGL(prefill_pack_kernel, dim3(static_cast<uint32_t>((threads + 255) / 256)), dim3(256), 0,
+                       as_stream(stream), x, static_cast<uint8_t*>(image), M, K);
+    return check_launch("prefill_pack");
+}
+
+extern "C" int guffin_hip_prefill_gemm(void* stream, int dtype, const void* tiles, const void* image, float* y,
+                                       uint32_t M, uint32_t K, uint32_t N) {
+    if (!tiles || !image || !y) return fail(GUFFIN_E_ARG, "prefill_gemm: null pointer");
+    if (dtype < GUFFIN_Q8_0 || dtype > GUFFIN_Q6_K) return fail(GUFFIN_E_ARG, "prefill_gemm: unknown dtype");
+    if (M == 0 || K == 0 || N == 0 || K % block_elems(dtype) != 0 || N % kCols != 0)
+        return fail(GUFFIN_E_SHAPE, "prefill_gemm: need K % block == 0 and N % 64 == 0");
+    if ((reinterpret_cast<uintptr_t>(tiles) & 15u) || (reinterpret_cast<uintptr_t>(image) & 255u))
+        return fail(GUFFIN_E_ALIGN, "prefill_gemm: tiles need 16-byte, the image 256-byte alignment");
+    const ImageLayout L = image_layout(M, K);
+    const dim3 grid(N / kCols, L.mpad / kChunkRows), block(256);
+    hipStream_t s = as_stream(stream);
+    const uint8_t* t = static_cast<const uint8_t*>(tiles);
+    const uint8_t* im = static_cast<const uint8_t*>(image);
+    if (dtype == GUFFIN_Q4_K) hipLaunchKernelGGL(prefill_gemm_kernel<GUFFIN_Q4_K>, grid, block, 0, s, t, im, y, M, K, N);
+    else if (dtype == GUFFIN_Q6_K) hipLaunchKernelGGL(prefill_gemm_kernel<GUFFIN_Q6_K>, grid, block, 0, s, t, im, y, M, K, N);
+    else hipLaunchKernelGGL(prefill_gemm_kernel<GUFFIN_Q8_0>, grid, block, 0, s, t, im, y, M, K, N);
+    return check_launch("prefill_gemm");
+}
+
+extern "C" int guffin_hip_prefill_attention(void* stream, const float* q, const void* ring_k, const void* ring_v,
+                                            const void* run_k, const void* run_v, float* out, uint32_t rows,
+                                            uint32_t position, uint32_t window, uint32_t ring_mask,
+                                            uint32_t q_heads, uint32_t kv_heads, uint32_t head_dim, float scale) {
+    if (!q || !ring_k || !ring_v || !run_k || !run_v || !out) return fail(GUFFIN_E_ARG, "prefill_attention: null pointer");
+    if (rows == 0 || head_dim != 256 || kv_heads == 0 || q_heads % kv_heads != 0)
+        return fail(GUFFIN_E_SHAPE, "prefill_attention: head_dim must be 256 and q_heads a multiple of kv_heads");
+    if ((ring_mask & (ring_mask + 1)) != 0) return fail(GUFFIN_E_ARG, "prefill_attention: ring capacity must be a power of two");
+    const uint32_t past = window ? (window - 1 < position ? window - 1 : position) : position;  // ring tokens a row can see
+    if (past > ring_mask + 1) return fail(GUFFIN_E_CAPACITY, "prefill_attention: the ring does not hold the visible past");
+    if (!(scale > 0.f)) return fail(GUFFIN_E_ARG, "prefill_attention: scale must be positive");
+    const uint32_t group = q_heads / kv_heads;
+    const dim3 grid((rows + 15) / 16, kv_heads), block(256);
+    hipStream_t s = as_stream(stream);
+    const uint16_t* rk = static_cast<const uint16_t*>(ring_k);
+    const uint16_t* rv = static_cast<const uint16_t*>(ring_v);
+    const uint16_t* uk = static_cast<const uint16_t*>(run_k);
+    const uint16_t* uv = static_cast<const uint16_t*>(run_v);
+#define GUFFIN_PA(G_) hipLaunchKernelGGL(prefill_attention_kernel<G_>, grid, block, 0, s, q, rk, rv, uk, uv, out, rows, \
+                                         position, window, ring_mask, q_heads, kv_heads, scale)
+    if (group == 1) GUFFIN_PA(1); else if (group == 2) GUFFIN_PA(2); else if (group == 4) GUFFIN_PA(4);
+    else return fail(GUFFIN_E_SHAPE, "prefill_attention: q_heads / kv_heads must be 1, 2 or 4");
+#undef GUFFIN_PA
+    return check_launch("prefill_attention");
+}

@@ -362,3 +362,36 @@ def step_draws(seed, step):
     out = _np.zeros(1, draws_dtype)
     check(lib().guffin_hip_step_draws(C.c_uint64(seed), C.c_uint64(step), out.ctypes.data_as(C.c_void_p)))
     return out[0]
+
+
+def prefill_pack(x):
+    """Matrix-core operand (image, multipliers, sums) of the M rows of x."""
+    M, K = x.shape
+    lib().guffin_hip_prefill_image_bytes.restype = C.c_uint64
+    n = lib().guffin_hip_prefill_image_bytes(M, K)
+    if n == 0:
+        raise GuffinError(-2, "prefill_pack: K must be a positive multiple of 32")
+    image = torch.empty(n, dtype=torch.uint8, device=x.device)
+    check(lib().guffin_hip_prefill_pack(_stream(), _p(x), _p(image), M, K))
+    return image
+
+
+def prefill_gemm(dtype, tiles, image, M, K, N):
+    y = torch.empty((M, N), dtype=torch.float32, device=tiles.device)
+    check(lib().guffin_hip_prefill_gemm(_stream(), dtype, _p(tiles), _p(image), _p(y), M, K, N))
+    return y
+
+
+def prefill_attention(q, ring_k, ring_v, run_k, run_v, position, window, ring_mask, q_heads, kv_heads, head_dim, scale):
+    rows = q.shape[0]
+    out = torch.empty_like(q)
+    check(lib().guffin_hip_prefill_attention(_stream(), _p(q), _p(ring_k), _p(ring_v), _p(run_k), _p(run_v), _p(out),
+                                             rows, position, window, ring_mask, q_heads, kv_heads, head_dim,
+                                             C.c_float(scale)))
+    return out
+
+
+def publish_run(run_k, run_v, ring_k, ring_v, position, ring_mask):
+    rows, width = run_k.shape
+    check(lib().guffin_hip_publish_run(_stream(), _p(run_k), _p(run_v), _p(ring_k), _p(ring_v), rows, position,
+                                       ring_mask, width))

@@ -275,6 +275,24 @@ class DeviceModel:
         return hidden, sums, pk, pv, status
 
 
+    def prefill(self, tokens, position, status=None):
+        """Ingests len(tokens) rows at `position` (rings are updated); returns the output-normed rows."""
+        sh = self.shape
+        rows = tokens.numel()
+        lib = hip.lib()
+        lib.guffin_hip_prefill_scratch_bytes.restype = C.c_uint64
+        nbytes = lib.guffin_hip_prefill_scratch_bytes(C.byref(self.desc), rows)
+        if nbytes == 0:
+            raise hip.GuffinError(-1, lib.guffin_hip_last_error().decode())
+        scratch = torch.zeros(nbytes, dtype=torch.uint8, device="cuda")
+        hidden = torch.zeros((rows, sh.hidden), dtype=torch.float32, device="cuda")
+        if status is None:
+            status = hip.new_status()
+        hip.check(lib.guffin_hip_prefill_rows(hip._stream(), C.byref(self.desc), hip._p(tokens), rows, position,
+                                              hip._p(scratch), C.c_uint64(nbytes), hip._p(hidden), hip._p(status)))
+        return hidden, status
+
+
 class H1Plan:
     """One speculative cycle: buffers, descriptor and the call into guffin_hip_h1_step."""
 

@@ -288,6 +288,39 @@ int guffin_hip_commit_rows(void* stream, const guffin_model_desc* model, const v
                            const void* priv_v, void* const* ring_k_table, void* const* ring_v_table,
                            const uint32_t* accepted, uint32_t position, uint32_t rows);
 
+/* ---- chunked prefill ------------------------------------------------------------------------
+ * Replaces the reference's prefill matrix path (encode_verifier_matmul with allow_prefill_matrix,
+ * src/tensor/backends/metal/metal_command_context.mm:384-401, kernels metal_kernels.mm:1031-1199)
+ * and encode_f16_prefill_attention (metal_command_context.hpp:185, metal_kernels.mm:2593-2800).
+ *
+ * guffin_hip_prefill_pack turns x [M][K] fp32 into the matrix-core operand of M rows (fp16 hi/lo
+ * image, per-(row, 32-group) multipliers and sums; guffin_hip_prefill_image_bytes bytes, 256-byte
+ * aligned); guffin_hip_prefill_gemm multiplies it with a repacked weight matrix, y [M][N] fp32,
+ * exact products and fp32 sums like the packed GEMV. */
+uint64_t guffin_hip_prefill_image_bytes(uint32_t M, uint32_t K);
+int guffin_hip_prefill_pack(void* stream, const float* x, void* image, uint32_t M, uint32_t K);
+int guffin_hip_prefill_gemm(void* stream, int dtype, const void* tiles, const void* image, float* y,
+                            uint32_t M, uint32_t K, uint32_t N);
+/* Causal GQA attention of `rows` consecutive positions starting at `position`: row r sees the
+ * ring for positions below `position` and rows 0..r of the run's own fp16 K/V rows
+ * run_k / run_v [rows][kv_heads*head_dim]; window = 0 for global layers, else the sliding
+ * window (the last `window` positions including the row's own).  q, out: [rows][q_heads*256]. */
+int guffin_hip_prefill_attention(void* stream, const float* q, const void* ring_k, const void* ring_v,
+                                 const void* run_k, const void* run_v, float* out, uint32_t rows,
+                                 uint32_t position, uint32_t window, uint32_t ring_mask,
+                                 uint32_t q_heads, uint32_t kv_heads, uint32_t head_dim, float scale);
+/* ring[(position + row) & ring_mask] = run[row] for every row of the run that a ring of this
+ * capacity keeps (encode_gemma2_kv_cache_copy, metal_command_context.hpp:170). */
+int guffin_hip_publish_run(void* stream, const void* run_k, const void* run_v, void* ring_k, void* ring_v,
+                           uint32_t rows, uint32_t position, uint32_t ring_mask, uint32_t row_width);
+/* The block graph of guffin_hip_forward_rows for any number of rows (prompt ingestion): same
+ * operator order, matrix-core GEMMs, the run's K/V published to the rings layer by layer.
+ * out_hidden [rows][hidden] holds the output-normed rows. */
+uint64_t guffin_hip_prefill_scratch_bytes(const guffin_model_desc* model, uint32_t rows);
+int guffin_hip_prefill_rows(void* stream, const guffin_model_desc* model, const uint32_t* tokens,
+                            uint32_t rows, uint32_t position, void* scratch, uint64_t scratch_bytes,
+                            float* out_hidden, uint32_t* status);
+
 /* One H1 cycle (src/engine/standalone_chat.cpp:508-615, src/engine/chain_chat.mm:245-543):
  * the drafter ingests the pending root at drafter_position, projects through its tied head,
  * builds its proposal law and picks x with the step's word; the target evaluates rows

@@ -1,0 +1,119 @@
+"""GPU parity of the chunked-prefill path: matrix-core GEMM, causal attention, whole block graph.
+
+Bars: GEMM rows within 1e-3 relative of the oracle's sequential fp32 row dots and within fp32
+rounding of the packed GEMV on the same rows; attention within 2e-6 of a double softmax;
+the ingested run's hidden rows within 1e-3 (relative to the row RMS) of the oracle's forward of
+the same rows, and the published ring rows equal to the oracle's fp16 K/V up to rare rounding ties.
+"""
+import numpy as np
+import pytest
+
+from guffin_amd import synth
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def hip():
+    from guffin_amd import hip as module
+    module.init(0)
+    return module
+
+
+def dev(a):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+@pytest.mark.parametrize("dtype,K,N", [(1, 3840, 256), (2, 3840, 128), (0, 640, 256), (1, 256, 64), (2, 512, 192)])
+@pytest.mark.parametrize("M", [1, 7, 33, 130])
+def test_prefill_gemm_parity(hip, gfo, dtype, K, N, M):
+    w = synth.make_weight(dtype, K, N, seed=70 + dtype)
+    x = synth.make_activation(M, K, seed=71)
+    x[M // 2] *= 300.0          # rows of very different magnitude share nothing
+    x[0, ::7] *= 1e-3
+    tiles = hip.repack(dtype, dev(w), K, N)
+    xd = dev(x)
+    y = hip.prefill_gemm(dtype, tiles, hip.prefill_pack(xd), M, K, N).cpu().numpy()
+    ref = gfo.gemv(dtype, w, x, N, threads=8)
+    scale = np.sqrt((ref.astype(np.float64) ** 2).mean(axis=1, keepdims=True))
+    assert np.all(np.abs(y.astype(np.float64) - ref) <= 1e-3 * scale)
+    # the decode GEMV on the same rows computes the same exact products
+    for r in (0, M - 1):
+        xr = xd[r:r + 1].contiguous()
+        one = hip.gemv_packed(dtype, tiles, xr, hip.group_sums(xr), N).cpu().numpy()[0]
+        assert np.all(np.abs(one.astype(np.float64) - y[r]) <= 2e-5 * scale[r])
+
+
+@pytest.mark.parametrize("q_heads,kv_heads,rows,position,window,cap", [
+    (16, 8, 40, 100, 0, 256), (16, 8, 21, 300, 64, 128), (4, 1, 33, 0, 0, 64), (4, 1, 50, 17, 32, 64), (2, 2, 5, 3, 0, 16)])
+def test_prefill_attention_matches_double_softmax(hip, q_heads, kv_heads, rows, position, window, cap):
+    import torch
+    rng = np.random.default_rng(5)
+    hd = 256
+    q = rng.normal(0, 1, (rows, q_heads * hd)).astype(np.float32)
+    ring_k = rng.normal(0, 1, (cap, kv_heads * hd)).astype(np.float16)
+    ring_v = rng.normal(0, 1, (cap, kv_heads * hd)).astype(np.float16)
+    run_k = rng.normal(0, 1, (rows, kv_heads * hd)).astype(np.float16)
+    run_v = rng.normal(0, 1, (rows, kv_heads * hd)).astype(np.float16)
+    out = hip.prefill_attention(dev(q), dev(ring_k), dev(ring_v), dev(run_k), dev(run_v), position, window, cap - 1,
+                                q_heads, kv_heads, hd, 0.0625).cpu().numpy()
+    group = q_heads // kv_heads
+    want = np.zeros_like(out, dtype=np.float64)
+    for r in range(rows):
+        pos = position + r
+        first = max(0, pos + 1 - window) if window else 0
+        ks, vs = [], []
+        for p in range(first, pos + 1):
+            src_k, src_v, i = (run_k, run_v, p - position) if p >= position else (ring_k, ring_v, p & (cap - 1))
+            ks.append(src_k[i]); vs.append(src_v[i])
+        ks = np.array(ks, np.float64).reshape(len(ks), kv_heads, hd)
+        vs = np.array(vs, np.float64).reshape(len(vs), kv_heads, hd)
+        for h in range(q_heads):
+            s = ks[:, h // group] @ q[r, h * hd:(h + 1) * hd].astype(np.float64) * 0.0625
+            p = np.exp(s - s.max()); p /= p.sum()
+            want[r, h * hd:(h + 1) * hd] = p @ vs[:, h // group]
+    assert np.max(np.abs(out - want)) <= 2e-6 * max(1.0, np.abs(want).max())
+
+
+def test_publish_run_keeps_the_newest_rows(hip):
+    import torch
+    rows, width, cap, position = 40, 256, 16, 9
+    rk = torch.arange(rows * width, dtype=torch.float32, device="cuda").reshape(rows, width).to(torch.float16)
+    rv = -rk
+    ring_k = torch.zeros((cap, width), dtype=torch.float16, device="cuda")
+    ring_v = torch.zeros_like(ring_k)
+    hip.publish_run(rk, rv, ring_k, ring_v, position, cap - 1)
+    for row in range(rows - cap, rows):
+        slot = (position + row) & (cap - 1)
+        assert torch.equal(ring_k[slot], rk[row]) and torch.equal(ring_v[slot], rv[row])
+
+
+@pytest.mark.parametrize("kind,rows,position", [("target", 37, 20), ("drafter", 70, 0)])
+def test_prefill_rows_match_oracle_forward(hip, gfo, kind, rows, position):
+    import torch
+    from dataclasses import replace
+    from guffin_amd import model
+    if kind == "drafter":
+        shape = replace(model.GEMMA3_270M, layers=6, vocab=4096, ring_global=256, ring_local=128, sliding_window=48)
+    else:
+        shape = replace(model.GEMMA3_12B, layers=6, vocab=2048, ring_global=256, ring_local=128, sliding_window=32)
+    host = model.HostModel(shape, seed=4, position=position)
+    devm = model.DeviceModel.from_host(host)
+    tokens = np.random.default_rng(9).integers(0, shape.vocab, rows).astype(np.uint32)
+    want, wk, wv = host.oracle_forward(gfo, tokens, position, threads=8)
+    hidden, status = devm.prefill(dev(tokens), position)
+    assert int(status.item()) == 0
+    got = hidden.cpu().numpy().astype(np.float64)
+    scale = np.sqrt((want.astype(np.float64) ** 2).mean(axis=-1, keepdims=True)) + 1e-30
+    assert np.max(np.abs(got - want) / scale) <= 1e-3
+    # the rings now hold the run: compare the last layer's published rows with the oracle's K/V
+    for l in (0, shape.layers - 1):
+        cap = shape.ring_local if shape.is_local(l) else shape.ring_global
+        rk = devm.ring_k[l].view(torch.int16).cpu().numpy().view(np.uint16)
+        for row in range(max(0, rows - cap), rows):
+            g = rk[(position + row) & (cap - 1)]
+            w = wk[l, row]
+            assert np.mean(g == w) >= 0.95
+            d = np.abs(g.view(np.float16).astype(np.float32) - w.view(np.float16).astype(np.float32))
+            assert d.max() <= 2.0 ** -9 * np.abs(w.view(np.float16).astype(np.float32)).max() + 1e-6
