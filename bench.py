@@ -84,6 +84,25 @@ def cpu_baseline(T, D, budget_s=20.0):
     }
 
 
+def prefill_figure(target, T, tokens=2048):
+    """Config 4's second half: a 2048-token prompt through the 48 blocks on the matrix core."""
+    import torch
+    ids = torch.randint(0, T.vocab, (tokens,), dtype=torch.int32, device="cuda")
+    target.prefill(ids, 0)                      # warm-up (also sizes the scratch arena)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    _, status = target.prefill(ids, 0)
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3
+    macs = tokens * T.layers * sum(K * N for K, N in T.proj_shapes())
+    # every MAC is issued twice (fp16 hi and lo halves of the activation) on the f16 matrix pipe
+    issued_flops = 2 * 2 * macs
+    return {"tokens": tokens, "ms": round(ms, 2), "tokens_per_s": round(tokens / ms * 1e3, 1),
+            "model_tflops": round(2 * macs / ms / 1e9, 1), "bound": "mfma",
+            "mfma_frac": round(issued_flops / (ms * 1e-3) / 2.5e15, 4), "peak": "2.5 PFLOP/s f16 dense",
+            "status": int(status.item())}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -91,6 +110,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--layers", type=int, default=0, help="debug: truncate the target to this many blocks")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-prefill", action="store_true", help="skip the 2048-token prefill figure")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs the H1 step on ONE GPU; --gpus %d is not supported "
@@ -194,6 +214,8 @@ def main():
             "bytes_per_launch": kernel_bytes, "launch_us": round(launch_us, 3),
         },
     }
+    if not args.no_prefill:
+        line["prefill"] = prefill_figure(target, T)
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(T, D)
     print(json.dumps(line))

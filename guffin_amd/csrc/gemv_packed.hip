@@ -272,7 +272,8 @@ __device__ __forceinline__ void compute_tile(const Q6Tile& t, const uint8_t* __r
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             const float m = mult[r * per_mult + g];
-            const float s16 = khalf ? xs16[r * per_row + 2 * g + 1] : xs16[r * per_row + 2 * g];
+            const float s16_first = xs16[r * per_row + 2 * g], s16_second = xs16[r * per_row + 2 * g + 1];
+            const float s16 = khalf ? s16_second : s16_first;
             part[0][r] = fmaf(sc[0] * m, da[2 * r] + da[2 * r + 1], part[0][r]);
             part[1][r] = fmaf(sc[1] * m, db[2 * r] + db[2 * r + 1], part[1][r]);
             off[0][r] = fmaf(sc[0], s16, off[0][r]);
@@ -374,10 +375,12 @@ __device__ __forceinline__ void run_blocks(const uint8_t* __restrict__ wt, const
         for (int c = 0; c < 2; ++c)
 #pragma unroll
             for (int r = 0; r < R; ++r) acc2[c][r] = 0.f;
-        Q6Tile cur;
+        Q6Tile cur, nxt;
+        if (b0 < b1) load_tile(cur, tp, lane);
         for (uint32_t b = b0; b < b1; ++b) {
-            load_tile(cur, tp + size_t(b - b0) * TB, lane);
+            if (b + 1 < b1) load_tile(nxt, tp + size_t(b + 1 - b0) * TB, lane);
             compute_tile<R>(cur, image + size_t(b) * 2048u, keep, mult + b * 8u, K / 32, xs + b * 16u, per_row, lane, acc2);
+            cur = nxt;
         }
         q6_gather<R>(acc2, lane, acc);
     } else {
