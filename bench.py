@@ -8,10 +8,11 @@ seeded random weights drawn on the device.  A step is one whole cycle replayed a
 graph; `value` is the mean step latency in microseconds with every input resident in HBM.
 
 Extra objects on the JSON line:
-  roofline      the dominant kernel (2-row Q4_K gate+up GEMV of one block, 66.4 MB of weights
+  roofline      the dominant kernel (2-row Q4_K gate+up GEMV fused with GeGLU, 66.4 MB of weights
                 per launch): algorithmic bytes / mean launch duration, measured with HIP events
                 around a graph of 48 back-to-back launches over the 48 blocks' own weights
                 (3.2 GB, far beyond the caches) on the launch stream.
+  prefill       config 4's second half: a 2048-token prompt through the same stack.
   cpu_baseline  the reference's own CPU row dot (oracle/_ref) or the oracle port timed on the
                 host cores on a bounded sample (one block's seven GEMVs at 2 rows, a column
                 subset), extrapolated to a whole step by weight count.  Reported, not a target.
@@ -153,25 +154,19 @@ def main():
     if (replayed["accepted"], replayed["token"], replayed["next_root"]) != (first["accepted"], first["token"], first["next_root"]):
         raise RuntimeError("graph replay changed the step's decision")
 
-    # ---- roofline of the dominant kernel: 2-row Q4_K gate+up GEMV, one launch per block -----
-    import ctypes as C
+    # ---- roofline of the dominant kernel: fused 2-row Q4_K gate+up GEMV + GeGLU, one launch per block -----
     H, F = T.hidden, T.ffn
     x = torch.randn(2, H, device="cuda")
     xs = hip.group_sums(x)
+    h_out = torch.empty(2, F, device="cuda")
+    h_sums = hip._receipt(2, F, "cuda")
     lib = hip.lib()
-    lib.guffin_hip_gemv_packed_multi_slices.restype = C.c_uint32
-    S = lib.guffin_hip_gemv_packed_multi_slices(2, (C.c_int * 2)(T.dtypes[4], T.dtypes[5]), (C.c_uint32 * 2)(F, F), H)
-    pg = torch.empty(S, 2, F, device="cuda")
-    pu = torch.empty(S, 2, F, device="cuda")
 
     def launch_all():
         for l in range(T.layers):
             L = target.layers[l]
-            dt = (C.c_int * 2)(L.dtype[4], L.dtype[5])
-            tiles = (C.c_void_p * 2)(L.tiles[4], L.tiles[5])
-            n = (C.c_uint32 * 2)(F, F)
-            parts = (C.c_void_p * 2)(pg.data_ptr(), pu.data_ptr())
-            hip.check(lib.guffin_hip_gemv_packed_multi(hip._stream(), 2, dt, tiles, n, parts, hip._p(x), hip._p(xs), 2, H))
+            hip.check(lib.guffin_hip_gateup_geglu(hip._stream(), L.dtype[4], L.tiles[4], L.tiles[5], hip._p(x), hip._p(xs),
+                                                  hip._p(h_out), hip._p(h_sums), 2, H, F))
 
     launch_all()
     torch.cuda.synchronize()
@@ -190,7 +185,8 @@ def main():
     torch.cuda.synchronize()
     launch_us = e0.elapsed_time(e1) * 1e3 / (reps * T.layers)
     from guffin_amd import synth
-    kernel_bytes = 2 * synth.weight_bytes(T.dtypes[4], H, F) + 2 * (H + H // 16 + H // 32) * 4 + 2 * S * 2 * F * 4
+    # weights once, activation rows in (fp32 rows are the operator's input; the kernel reads their receipt), h out
+    kernel_bytes = 2 * synth.weight_bytes(T.dtypes[4], H, F) + 2 * H * 4 + 2 * F * 4
     achieved = kernel_bytes / launch_us / 1e3  # GB/s
 
     total_bytes = step_bytes(T, D, t_pos, d_pos)
@@ -208,7 +204,7 @@ def main():
             "accepted": int(first["accepted"]),
         },
         "roofline": {
-            "kernel": "gemv_packed_multi_kernel<2, 2> (Q4_K gate+up, 2 rows, K=3840, N=2x15360)",
+            "kernel": "gateup_geglu_kernel<Q4_K, 2> (Q4_K gate+up GEMV + GeGLU, 2 rows, K=3840, N=2x15360)",
             "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
             "bytes_per_launch": kernel_bytes, "launch_us": round(launch_us, 3),

@@ -464,6 +464,40 @@ gemv_packed_multi_kernel(const uint8_t* __restrict__ t0, const uint8_t* __restri
     finish_tile<R>(acc, part, N, ct, blockIdx.y, c.W);
 }
 
+// gate and up projections of one column tile in one workgroup (waves [0, W) gate, [W, 2W) up,
+// k-slices combined in wave order), then h = gelu_tanh(gate) * up for the 64 columns and the two
+// 32-groups of h's activation receipt: no partial planes and no separate GeGLU launch.
+template <int DTYPE, int R>
+__global__ void __launch_bounds__(1024)
+gateup_geglu_kernel(const uint8_t* __restrict__ gate_tiles, const uint8_t* __restrict__ up_tiles,
+                    const float* __restrict__ x, const float* __restrict__ xsums, float* __restrict__ h,
+                    void* __restrict__ h_receipt, uint32_t F, PackedCfg c) {
+    __shared__ float red[16 * 2 * 64];
+    __shared__ float vals[2 * 64];
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    const bool is_up = wave >= c.W;
+    const uint32_t slice = is_up ? wave - c.W : wave;
+    const uint32_t b0 = min(slice * c.bps, c.nblk), b1 = min(b0 + c.bps, c.nblk);
+    float acc[R];
+    run_blocks<DTYPE, R>(is_up ? up_tiles : gate_tiles, x, xsums, c.K, c.nblk, blockIdx.x, b0, b1, acc);
+#pragma unroll
+    for (int r = 0; r < R; ++r) red[(wave * R + r) * 64 + lane] = acc[r];
+    __syncthreads();
+    if (threadIdx.x < R * 64) {
+        const uint32_t r = threadIdx.x >> 6;
+        float g = red[r * 64 + lane], u = red[(c.W * R + r) * 64 + lane];
+        for (uint32_t w = 1; w < c.W; ++w) { g += red[(w * R + r) * 64 + lane]; u += red[((c.W + w) * R + r) * 64 + lane]; }
+        const float v = geglu_value(g, u);
+        h[size_t(r) * F + blockIdx.x * kTileCols + lane] = v;
+        vals[r * 64 + lane] = v;
+    }
+    __syncthreads();
+    if (h_receipt) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) emit_receipt(vals + r * 64, blockIdx.x * kTileCols, kTileCols, r, R, F, h_receipt);
+    }
+}
+
 int g_cus = 256;
 
 // Work split of a launch over `tiles` column tiles of `nblk` blocks each: blocks per wave so
@@ -623,6 +657,34 @@ extern "C" int guffin_hip_gemv_packed_multi(void* stream, uint32_t count, const 
 #undef GUFFIN_MULTI_MODE
 #undef GUFFIN_MULTI
     return check_launch("gemv_packed_multi");
+}
+
+extern "C" int guffin_hip_gateup_geglu(void* stream, int dtype, const void* gate_tiles, const void* up_tiles,
+                                       const float* x, const float* xsums, float* h, float* h_sums,
+                                       uint32_t rows, uint32_t K, uint32_t F) {
+    if (!gate_tiles || !up_tiles || !x || !xsums || !h) return fail(GUFFIN_E_ARG, "gateup_geglu: null pointer");
+    if (dtype != GUFFIN_Q4_K && dtype != GUFFIN_Q8_0) return fail(GUFFIN_E_SHAPE, "gateup_geglu: Q4_K or Q8_0 pairs only");
+    if (rows == 0 || rows > 2) return fail(GUFFIN_E_SHAPE, "gateup_geglu: rows must be 1 or 2");
+    if (int rc = check_packed_shape("gateup_geglu: need K % block == 0 and F % 64 == 0", dtype, K, F)) return rc;
+    if ((reinterpret_cast<uintptr_t>(gate_tiles) & 15u) || (reinterpret_cast<uintptr_t>(up_tiles) & 15u))
+        return fail(GUFFIN_E_ALIGN, "gateup_geglu: tiles must be 16-byte aligned");
+    if (reinterpret_cast<uintptr_t>(h_sums) & 255u) return fail(GUFFIN_E_ALIGN, "gateup_geglu: the receipt must be 256-byte aligned");
+    const uint32_t nblk = K / block_elems(dtype), tiles = F / kTileCols;
+    Split sp = choose_split(nblk, 2 * tiles, 8);
+    if (sp.planes > 1) {  // all k-slices of a tile must sit in one workgroup: at most 8 per matrix
+        sp.bps = (nblk + 7) / 8;
+        sp.W = (nblk + sp.bps - 1) / sp.bps;
+    }
+    const PackedCfg c {K, nblk, sp.bps, sp.W};
+    const dim3 grid(tiles), block(2 * sp.W * 64);
+    hipStream_t s = as_stream(stream);
+    const uint8_t* g = static_cast<const uint8_t*>(gate_tiles);
+    const uint8_t* u = static_cast<const uint8_t*>(up_tiles);
+#define GUFFIN_GU(D_, R_) hipLaunchKernelGGL((gateup_geglu_kernel<D_, R_>), grid, block, 0, s, g, u, x, xsums, h, h_sums, F, c)
+    if (dtype == GUFFIN_Q4_K) { if (rows == 2) GUFFIN_GU(GUFFIN_Q4_K, 2); else GUFFIN_GU(GUFFIN_Q4_K, 1); }
+    else { if (rows == 2) GUFFIN_GU(GUFFIN_Q8_0, 2); else GUFFIN_GU(GUFFIN_Q8_0, 1); }
+#undef GUFFIN_GU
+    return check_launch("gateup_geglu");
 }
 
 extern "C" int guffin_hip_gemv_packed(void* stream, int dtype, const void* tiles, const float* x, const float* xsums,

@@ -299,13 +299,6 @@ __global__ void __launch_bounds__(64) qkv_post_kernel(QkvArgs a) {
 
 // out = gelu_tanh(gate) * up, element-wise; gate/up may be partial planes.  One workgroup
 // per row when sums are requested (row image in LDS), grid-stride otherwise.
-__device__ __forceinline__ float geglu_value(float g, float u) {
-    constexpr float k0 = 0.7978845608028654f, k1 = 0.044715f;
-    const float inner = __fmul_rn(k0, __fadd_rn(g, __fmul_rn(__fmul_rn(__fmul_rn(k1, g), g), g)));
-    const float t = tanhf(inner);
-    return __fmul_rn(__fmul_rn(__fmul_rn(0.5f, g), __fadd_rn(1.0f, t)), u);
-}
-
 __global__ void __launch_bounds__(256)
 geglu_kernel(const float* __restrict__ gate, const float* __restrict__ up, uint32_t planes, size_t plane_stride,
              float* __restrict__ out, float* __restrict__ out_sums, uint32_t width) {

@@ -178,7 +178,9 @@ int forward_rows(hipStream_t stream, const guffin_model_desc& m, const uint32_t*
         // x1 = x + rms(o, post_attention_norm); u = rms(x1, ffn_norm)
         GUFFIN_TRY(guffin_hip_rms_norm_add_norm(st, s.part_a, slices(L.dtype[3], QW, H), uint64_t(rows) * H, L.norm[3],
                                                 s.x, s.x1, L.norm[4], s.u, s.us, rows, H, m.eps, status));
-        {
+        if (L.dtype[4] == L.dtype[5] && L.dtype[4] != GUFFIN_Q6_K) {
+            GUFFIN_TRY(guffin_hip_gateup_geglu(st, L.dtype[4], L.tiles[4], L.tiles[5], s.u, s.us, s.h, s.hs, rows, H, F));
+        } else {
             const int dt[2] = {L.dtype[4], L.dtype[5]};
             const void* tl[2] = {L.tiles[4], L.tiles[5]};
             const uint32_t n[2] = {F, F};

@@ -15,6 +15,14 @@
 
 namespace guffin {
 
+// gelu_tanh(g) * u with the reference's operation order (src/tensor/ops/elementwise.cpp:79-94, 50-63)
+__device__ __forceinline__ float geglu_value(float g, float u) {
+    constexpr float k0 = 0.7978845608028654f, k1 = 0.044715f;
+    const float inner = __fmul_rn(k0, __fadd_rn(g, __fmul_rn(__fmul_rn(__fmul_rn(k1, g), g), g)));
+    const float t = tanhf(inner);
+    return __fmul_rn(__fmul_rn(__fmul_rn(0.5f, g), __fadd_rn(1.0f, t)), u);
+}
+
 struct ReceiptLayout { size_t mult_off, image_off, bytes; };
 
 __host__ __device__ inline ReceiptLayout receipt_layout(uint32_t rows, uint32_t K) {

@@ -364,6 +364,15 @@ def step_draws(seed, step):
     return out[0]
 
 
+def gateup_geglu(dtype, gate_tiles, up_tiles, x, xsums, F, want_sums=True):
+    rows, K = x.shape
+    h = torch.empty((rows, F), dtype=torch.float32, device=x.device)
+    sums = _receipt(rows, F, x.device) if want_sums else None
+    check(lib().guffin_hip_gateup_geglu(_stream(), dtype, _p(gate_tiles), _p(up_tiles), _p(x), _p(xsums), _p(h),
+                                        _p(sums), rows, K, F))
+    return (h, sums) if want_sums else h
+
+
 def prefill_pack(x):
     """Matrix-core operand (image, multipliers, sums) of the M rows of x."""
     M, K = x.shape

@@ -114,6 +114,14 @@ int guffin_hip_gemv_packed_multi(void* stream, uint32_t count, const int* dtypes
                                  const uint32_t* N, float* const* partials, const float* x,
                                  const float* xsums, uint32_t rows, uint32_t K);
 
+/* h = gelu_tanh(x W_gate) * (x W_up) with its activation receipt in one launch (gate and up of
+ * the same dtype, Q4_K or Q8_0): guffin_hip_gemv_packed_multi + guffin_hip_geglu without the
+ * partial planes in between (reference: two encode_verifier_matmul and encode_gelu_tanh_multiply,
+ * src/engine/gemma_target_runtime.cpp:176-199).  h [rows][F]; h_sums may be NULL. */
+int guffin_hip_gateup_geglu(void* stream, int dtype, const void* gate_tiles, const void* up_tiles,
+                            const float* x, const float* xsums, float* h, float* h_sums,
+                            uint32_t rows, uint32_t K, uint32_t F);
+
 /* ---- per-layer operators -----------------------------------------------------------------
  * Inputs produced by a packed GEMV may be given as `planes` k-slice partial planes
  * (`plane_stride` floats apart) that the operator sums in slice order while loading; plain

@@ -181,6 +181,31 @@ def test_packed_multi_rejects_mixed_block_lengths(hip):
         hip.gemv_packed_multi((1, 0), [t, t], x, xs, (64, 64))
 
 
+@pytest.mark.parametrize("dtype,K,F,rows,bit_equal", [(1, 3840, 15360, 2, True), (1, 3840, 15360, 1, True),
+                                                     (0, 640, 2048, 1, False), (1, 512, 128, 2, False)])
+def test_fused_gate_up_geglu_equals_the_three_launches(hip, dtype, K, F, rows, bit_equal):
+    import torch
+    x = synth.make_activation(rows, K, seed=80)
+    xd = dev(x)
+    xs = hip.group_sums(xd)
+    gate = hip.repack(dtype, dev(synth.make_weight(dtype, K, F, seed=81)), K, F)
+    up = hip.repack(dtype, dev(synth.make_weight(dtype, K, F, seed=82)), K, F)
+    pg, pu = hip.gemv_packed_multi((dtype, dtype), [gate, up], xd, xs, (F, F))
+    want, want_sums = hip.geglu(pg, pu, planes=pg.shape[0], want_sums=True)
+    h, sums = hip.gateup_geglu(dtype, gate, up, xd, xs, F)
+    if bit_equal:   # same k-split as the unfused launch: identical arithmetic
+        assert torch.equal(h.view(torch.int32), want.view(torch.int32))
+    scale = float(want.abs().max())
+    assert float((h - want).abs().max()) <= 3e-6 * scale
+    assert float((sums - want_sums).abs().max()) <= 1e-4 * scale
+    mult, image = hip.receipt_parts(sums, rows, F)
+    mult_w, image_w = hip.receipt_parts(want_sums, rows, F)
+    if bit_equal:
+        assert torch.equal(mult, mult_w) and torch.equal(image.view(torch.int16), image_w.view(torch.int16))
+    with pytest.raises(hip.GuffinError):
+        hip.gateup_geglu(2, gate, up, xd, xs, F)
+
+
 def test_packed_rejects_bad_arguments(hip):
     import torch
     w = torch.zeros(144 * 64, dtype=torch.uint8, device="cuda")
