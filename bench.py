@@ -155,6 +155,7 @@ def main():
         raise RuntimeError("graph replay changed the step's decision")
 
     # ---- roofline of the dominant kernel: fused 2-row Q4_K gate+up GEMV + GeGLU, one launch per block -----
+    import ctypes as C
     H, F = T.hidden, T.ffn
     x = torch.randn(2, H, device="cuda")
     xs = hip.group_sums(x)
@@ -165,8 +166,9 @@ def main():
     def launch_all():
         for l in range(T.layers):
             L = target.layers[l]
-            hip.check(lib.guffin_hip_gateup_geglu(hip._stream(), L.dtype[4], L.tiles[4], L.tiles[5], hip._p(x), hip._p(xs),
-                                                  hip._p(h_out), hip._p(h_sums), 2, H, F))
+            # (ctypes passes a bare Python int as a 32-bit C int: pointers must be wrapped)
+            hip.check(lib.guffin_hip_gateup_geglu(hip._stream(), int(L.dtype[4]), C.c_void_p(L.tiles[4]), C.c_void_p(L.tiles[5]),
+                                                  hip._p(x), hip._p(xs), hip._p(h_out), hip._p(h_sums), 2, H, F))
 
     launch_all()
     torch.cuda.synchronize()
