@@ -191,6 +191,13 @@ def main():
     kernel_bytes = 2 * synth.weight_bytes(T.dtypes[4], H, F) + 2 * H * 4 + 2 * F * 4
     achieved = kernel_bytes / launch_us / 1e3  # GB/s
 
+    # a plain 256 MiB device copy: the reference reading for FETCH_SIZE / WRITE_SIZE counter runs
+    cal_src = torch.empty(64 << 20, dtype=torch.float32, device="cuda").fill_(1.0)
+    cal_dst = torch.empty_like(cal_src)
+    cal_dst.copy_(cal_src)
+    torch.cuda.synchronize()
+    del cal_src, cal_dst
+
     total_bytes = step_bytes(T, D, t_pos, d_pos)
     line = {
         "metric": "h1_step_latency_us", "value": round(ms_per_step * 1e3, 1), "unit": "us",
@@ -208,7 +215,10 @@ def main():
         "roofline": {
             "kernel": "gateup_geglu_kernel<Q4_K, 2> (Q4_K gate+up GEMV + GeGLU, 2 rows, K=3840, N=2x15360)",
             "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+            "frac": round(achieved / HBM_PEAK_GBS, 4),
+            # HBM bytes per launch from the FETCH_SIZE / WRITE_SIZE counter runs recorded in
+            # profiles/gateup_geglu_q4k_hbm_traffic.txt (copy-calibrated: fetch x 1.9997, write x 1)
+            "traffic": 67046400,
             "bytes_per_launch": kernel_bytes, "launch_us": round(launch_us, 3),
         },
     }
