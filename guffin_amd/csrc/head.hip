@@ -103,7 +103,7 @@ topk_merge_kernel(const float* __restrict__ logits, const uint64_t* __restrict__
     __shared__ uint32_t hist[256];
     __shared__ uint64_t sel[512];
     __shared__ uint64_t keys[512];  // selected keys in candidate order
-    __shared__ uint32_t s_bin, s_above, s_count;
+    __shared__ uint32_t s_bin, s_above, s_count, s_in_bin;
     const uint32_t row = blockIdx.x, lane = threadIdx.x & 63;
     const uint64_t* src = survivors + size_t(row) * n_survivors;
     // up to 8 keys per thread stay in registers; longer survivor lists are re-read from memory
@@ -152,7 +152,7 @@ topk_merge_kernel(const float* __restrict__ logits, const uint64_t* __restrict__
             if (above < remaining && remaining <= incl) {
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    if (remaining <= above + c[j]) { s_bin = 255 - 4 * lane - j; s_above = above; break; }
+                    if (remaining <= above + c[j]) { s_bin = 255 - 4 * lane - j; s_above = above; s_in_bin = c[j]; break; }
                     above += c[j];
                 }
             }
@@ -160,6 +160,9 @@ topk_merge_kernel(const float* __restrict__ logits, const uint64_t* __restrict__
         __syncthreads();
         prefix = (prefix << 8) | s_bin;
         remaining -= s_above;
+        // the upper 32 bits are the logit: if every key that shares the threshold logit is wanted
+        // (no tie across the cut), the token bits need no passes
+        if (pass == 3 && s_in_bin == remaining) { prefix <<= 32; remaining = 0; break; }
     }
     // `prefix` is the retain-th largest key; keys above it are taken, then `remaining` copies of it
     // (more than one only for the zero padding of a short last tile)
