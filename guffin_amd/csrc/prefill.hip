@@ -10,9 +10,11 @@
 // many rows the 16 A rows are 8 activation rows x {hi, lo}, so nothing is replicated: after
 // one MFMA lane (j, g) holds, for column 16*cg + j, rows 2g and 2g+1 of the row group as
 // (hi, lo) pairs.  A wave owns 64 columns x 32 rows (4 row groups), a workgroup 4 such waves on
-// the same tile (128 rows), so a weight tile is fetched from HBM once per 128 rows.  Block
-// scales and the per-(row, 32-group) activation multipliers are applied to each MFMA result in
-// fp32; the offset terms use per-(row, 32-group) sums (Q6_K: per 16-group).
+// the same tile (128 rows), so a weight tile is fetched from HBM once per 128 rows.  Q4_K folds
+// its 6-bit scales into B (sc * q <= 945 is still an exact subnormal) and accumulates a whole
+// 256-element block inside the MFMA chain; Q6_K and Q8_0 apply the block scale and the activation
+// multiplier to each MFMA result in fp32.  The offset terms use per-(row, 32-group) sums (Q6_K:
+// per 16-group).
 //
 // Attention.  A workgroup serves 16 consecutive query rows of one KV head (all query heads of the
 // group) and walks the visible key range in tiles of 32 tokens through LDS with an online
@@ -39,7 +41,8 @@ __host__ __device__ constexpr uint32_t block_elems(int dtype) { return dtype == 
 // ---- activation image of M rows --------------------------------------------------------
 // image: half [K/32][Mpad/8][16][32]   A row 2*(row % 8) + {0 hi, 1 lo}; inside a group the halves
 //                                      of elements 8s..8s+7 sit at 8s + {0,2,1,3,4,6,5,7}
-// mult : float [K/32][Mpad]            2^(E+24) of (row, group)
+// mult : float [K/32][Mpad]            2^(E+24) of (row, group); E is shared by the 8 groups of a
+//                                      256-element block when K is a multiple of 256
 // s32  : float [K/32][Mpad]            sum of the group's 32 activations
 // s16  : float [K/16][Mpad]            sums of 16
 struct ImageLayout { size_t mult_off, s32_off, s16_off, bytes; uint32_t mpad; };
@@ -71,6 +74,11 @@ prefill_pack_kernel(const float* __restrict__ x, uint8_t* __restrict__ blob, uin
     for (int i = 1; i < 8; ++i) { sum += v[i]; m = fmaxf(m, fabsf(v[i])); }
     m = fmaxf(m, __shfl_xor(m, 1, kWave));
     m = fmaxf(m, __shfl_xor(m, 2, kWave));
+    if (K % 256 == 0) {  // one exponent per 256 elements (32 consecutive threads): K-quant blocks
+        m = fmaxf(m, __shfl_xor(m, 4, kWave));
+        m = fmaxf(m, __shfl_xor(m, 8, kWave));
+        m = fmaxf(m, __shfl_xor(m, 16, kWave));
+    }
     const float sum16 = sum + __shfl_xor(sum, 1, kWave);
     const float sum32 = sum16 + __shfl_xor(sum16, 2, kWave);
     uint32_t eb = __float_as_uint(m) >> 23;
@@ -106,6 +114,11 @@ __device__ __forceinline__ half8_t as_half8(uint32_t a, uint32_t b, uint32_t c, 
 }
 __device__ __forceinline__ uint32_t even_bytes(uint32_t v) { return __builtin_amdgcn_perm(0u, v, 0x0c020c00u); }
 __device__ __forceinline__ uint32_t odd_bytes(uint32_t v) { return __builtin_amdgcn_perm(0u, v, 0x0c030c01u); }
+typedef unsigned short ushort2_t __attribute__((ext_vector_type(2)));
+// products of the two 16-bit fields of a and b (v_pk_mul_lo_u16)
+__device__ __forceinline__ uint32_t pk_mul(uint32_t a, uint32_t b) {
+    return __builtin_bit_cast(uint32_t, __builtin_bit_cast(ushort2_t, a) * __builtin_bit_cast(ushort2_t, b));
+}
 __device__ __forceinline__ float sbyte(uint32_t w, int i) {
     return i == 0 ? sb0(w) : i == 1 ? sb1(w) : i == 2 ? sb2(w) : sb3(w);
 }
@@ -182,9 +195,27 @@ prefill_gemm_kernel(const uint8_t* __restrict__ tiles, const uint8_t* __restrict
     const uint8_t* tp = tiles + size_t(blockIdx.x) * nblk * TB;
     for (uint32_t b = 0; b < nblk; ++b, tp += TB) {
         if constexpr (DTYPE == GUFFIN_Q4_K) {
+            // sc * q <= 945 is still an exact fp16 subnormal, so the 6-bit scales are folded into B
+            // and a whole 256-element block accumulates inside the MFMA chain; d and the block's
+            // activation multiplier are applied once per block
             uint4 q[8];
 #pragma unroll
             for (int i = 0; i < 8; ++i) q[i] = *reinterpret_cast<const uint4*>(tp + 1024 * i + lane * 16);
+            float d[4], dmin[4];
+            uint32_t sc_a[4], sc_b[4], mn_a[4], mn_b[4];
+#pragma unroll
+            for (int cg = 0; cg < 4; ++cg) {
+                const uint4 hdr = *reinterpret_cast<const uint4*>(tp + 8192 + (16 * cg + j) * 16);
+                d[cg] = h2f(hdr.x & 0xFFFFu); dmin[cg] = h2f(hdr.x >> 16);
+                sc_a[cg] = hdr.y & 0x3F3F3F3Fu; mn_a[cg] = hdr.z & 0x3F3F3F3Fu;
+                sc_b[cg] = (hdr.w & 0x0F0F0F0Fu) | ((hdr.y >> 2) & 0x30303030u);
+                mn_b[cg] = ((hdr.w >> 4) & 0x0F0F0F0Fu) | ((hdr.z >> 2) & 0x30303030u);
+            }
+            float4_t D[4][4];
+#pragma unroll
+            for (int cg = 0; cg < 4; ++cg)
+#pragma unroll
+                for (int rg = 0; rg < 4; ++rg) D[cg][rg] = float4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int ch = 0; ch < 4; ++ch) {
                 GroupOperands lo, hi;
@@ -192,25 +223,36 @@ prefill_gemm_kernel(const uint8_t* __restrict__ tiles, const uint8_t* __restrict
                 load_group(c, b * 8 + 2 * ch + 1, hi);
 #pragma unroll
                 for (int cg = 0; cg < 4; ++cg) {
-                    const uint4 hdr = *reinterpret_cast<const uint4*>(tp + 8192 + (16 * cg + j) * 16);
-                    const float d = h2f(hdr.x & 0xFFFFu), dmin = h2f(hdr.x >> 16);
-                    const uint32_t sc_a = hdr.y & 0x3F3F3F3Fu, mn_a = hdr.z & 0x3F3F3F3Fu;
-                    const uint32_t sc_b = (hdr.w & 0x0F0F0F0Fu) | ((hdr.y >> 2) & 0x30303030u);
-                    const uint32_t mn_b = ((hdr.w >> 4) & 0x0F0F0F0Fu) | ((hdr.z >> 2) & 0x30303030u);
-                    const uint32_t scw = ch < 2 ? sc_a : sc_b, mnw = ch < 2 ? mn_a : mn_b;
-                    const float sc_lo = ubyte(scw, 2 * (ch & 1)), sc_hi = ubyte(scw, 2 * (ch & 1) + 1);
-                    const float mn_lo = ubyte(mnw, 2 * (ch & 1)), mn_hi = ubyte(mnw, 2 * (ch & 1) + 1);
+                    const uint32_t scw = ch < 2 ? sc_a[cg] : sc_b[cg], mnw = ch < 2 ? mn_a[cg] : mn_b[cg];
+                    // the scale byte in both 16-bit fields
+                    const uint32_t pair_lo = __builtin_amdgcn_perm(0u, scw, (ch & 1) ? 0x0c020c02u : 0x0c000c00u);
+                    const uint32_t pair_hi = __builtin_amdgcn_perm(0u, scw, (ch & 1) ? 0x0c030c03u : 0x0c010c01u);
                     const uint4 piece = q[2 * cg + (ch >> 1)];
                     const uint32_t w0 = (ch & 1) ? piece.z : piece.x, w1 = (ch & 1) ? piece.w : piece.y;
-                    const uint32_t v0 = w0 >> 8, v1 = w1 >> 8;
-                    mfma_scale(lo, as_half8(w0 & 0x000F000Fu, v0 & 0x000F000Fu, w1 & 0x000F000Fu, v1 & 0x000F000Fu),
-                               d * sc_lo, acc[cg]);
-                    mfma_scale(hi, as_half8(w0 & 0x00F000F0u, v0 & 0x00F000F0u, w1 & 0x00F000F0u, v1 & 0x00F000F0u),
-                               d * 0.0625f * sc_hi, acc[cg]);
-                    add_offset(c.s32, c, b * 8 + 2 * ch, -dmin * mn_lo, acc[cg]);
-                    add_offset(c.s32, c, b * 8 + 2 * ch + 1, -dmin * mn_hi, acc[cg]);
+                    constexpr uint32_t M = 0x000F000Fu;
+                    const half8_t blo = as_half8(pk_mul(w0 & M, pair_lo), pk_mul((w0 >> 8) & M, pair_lo),
+                                                 pk_mul(w1 & M, pair_lo), pk_mul((w1 >> 8) & M, pair_lo));
+                    const half8_t bhi = as_half8(pk_mul((w0 >> 4) & M, pair_hi), pk_mul((w0 >> 12) & M, pair_hi),
+                                                 pk_mul((w1 >> 4) & M, pair_hi), pk_mul((w1 >> 12) & M, pair_hi));
+#pragma unroll
+                    for (int rg = 0; rg < 4; ++rg) {
+                        D[cg][rg] = __builtin_amdgcn_mfma_f32_16x16x32_f16(lo.a[rg], blo, D[cg][rg], 0, 0, 0);
+                        D[cg][rg] = __builtin_amdgcn_mfma_f32_16x16x32_f16(hi.a[rg], bhi, D[cg][rg], 0, 0, 0);
+                    }
+                    const float mn_lo = ubyte(mnw, 2 * (ch & 1)), mn_hi = ubyte(mnw, 2 * (ch & 1) + 1);
+                    add_offset(c.s32, c, b * 8 + 2 * ch, -dmin[cg] * mn_lo, acc[cg]);
+                    add_offset(c.s32, c, b * 8 + 2 * ch + 1, -dmin[cg] * mn_hi, acc[cg]);
                 }
             }
+            GroupOperands blk;
+            load_group(c, b * 8, blk);  // the block's multipliers (shared by its 8 groups)
+#pragma unroll
+            for (int cg = 0; cg < 4; ++cg)
+#pragma unroll
+                for (int rg = 0; rg < 4; ++rg) {
+                    acc[cg][rg][0] = fmaf(d[cg] * blk.mult[rg].x, D[cg][rg][0] + D[cg][rg][1], acc[cg][rg][0]);
+                    acc[cg][rg][1] = fmaf(d[cg] * blk.mult[rg].y, D[cg][rg][2] + D[cg][rg][3], acc[cg][rg][1]);
+                }
         } else if constexpr (DTYPE == GUFFIN_Q6_K) {
             uint4 ql[8], qh[4];
 #pragma unroll
