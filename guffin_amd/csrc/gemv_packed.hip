@@ -129,12 +129,20 @@ __device__ __forceinline__ uint32_t odd_bytes(uint32_t v) { return __builtin_amd
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef float float4_t __attribute__((ext_vector_type(4)));
 
+// Weight bytes are used once: streaming (non-temporal) loads keep the caches for the activation
+// image, which every wave re-reads.
+typedef uint32_t uint4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ uint4 stream_load(const uint8_t* p) {
+    const uint4_t v = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(p));
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
+
 struct Q4Tile { uint4 q[8]; uint4 hdr; };
 
 __device__ __forceinline__ void load_tile(Q4Tile& t, const uint8_t* p) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) t.q[i] = *reinterpret_cast<const uint4*>(p + 1024 * i);
-    t.hdr = *reinterpret_cast<const uint4*>(p + 8192);
+    for (int i = 0; i < 8; ++i) t.q[i] = stream_load(p + 1024 * i);
+    t.hdr = stream_load(p + 8192);
 }
 
 __device__ __forceinline__ half8_t as_half8(uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
@@ -204,9 +212,9 @@ struct Q6Tile { uint4 ql[8]; uint4 qh[4]; uint4 sc[2]; uint32_t d[2]; };
 
 __device__ __forceinline__ void load_tile(Q6Tile& t, const uint8_t* p, uint32_t lane) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) t.ql[i] = *reinterpret_cast<const uint4*>(p + 1024 * i);
+    for (int i = 0; i < 8; ++i) t.ql[i] = stream_load(p + 1024 * i);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) t.qh[i] = *reinterpret_cast<const uint4*>(p + 8192 + 1024 * i);
+    for (int i = 0; i < 4; ++i) t.qh[i] = stream_load(p + 8192 + 1024 * i);
     const uint8_t* base = p - lane * 16;
     const uint32_t col = 32u * (lane >> 5) + (lane & 15u);
 #pragma unroll
@@ -309,8 +317,8 @@ __device__ __forceinline__ void q6_gather(const float (&acc2)[2][R], uint32_t la
 struct Q8Tile { uint4 q[2]; uint32_t d; };
 
 __device__ __forceinline__ void load_tile(Q8Tile& t, const uint8_t* p, uint32_t lane) {
-    t.q[0] = *reinterpret_cast<const uint4*>(p);
-    t.q[1] = *reinterpret_cast<const uint4*>(p + 1024);
+    t.q[0] = stream_load(p);
+    t.q[1] = stream_load(p + 1024);
     t.d = *reinterpret_cast<const uint16_t*>(p - lane * 16 + 2048 + lane * 2);
 }
 
