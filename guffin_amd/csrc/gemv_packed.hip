@@ -520,6 +520,7 @@ Split choose_split(uint32_t nblk, uint32_t tiles, uint32_t max_w) {
     uint32_t planes = (wpt + max_w - 1) / max_w;
     if (tiles * planes * 4 < uint32_t(g_cus) * 3) {  // fewer workgroups than 3/4 of the CUs: split further
         uint32_t want = (g_cus + tiles - 1) / tiles;
+        if (want > 4) want = 4;  // small matrices are latency-bound: more planes only slow their consumers
         if (want > wpt) want = wpt;
         if (want > planes) planes = want;
     }
