@@ -102,4 +102,15 @@ __device__ __forceinline__ constexpr int reduce_multi_shift() {
     return s;
 }
 
+// cos and sin of the NeoX rotation of (position, pair)
+__device__ __forceinline__ void rope_sincos(uint32_t position, uint32_t pair, uint32_t rope_dim, float base,
+                                            float scale, float& c, float& s) {
+    // angle in double, as the CPU operator forms it (rope.cpp:109-117), times the layer's frequency scale
+    const double exponent = static_cast<double>(2u * pair) / static_cast<double>(rope_dim);
+    const double angle = static_cast<double>(position) / pow(static_cast<double>(base), exponent)
+        * static_cast<double>(scale);
+    c = static_cast<float>(cos(angle));
+    s = static_cast<float>(sin(angle));
+}
+
 }  // namespace guffin

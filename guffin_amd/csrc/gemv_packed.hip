@@ -707,11 +707,12 @@ extern "C" int guffin_hip_gemv_packed(void* stream, int dtype, const void* tiles
     const uint32_t S = choose_split(K / block_elems(dtype), N / kTileCols, max_waves(dtype)).planes;
     const uint8_t* w = static_cast<const uint8_t*>(tiles);
     hipStream_t s = as_stream(stream);
+    float* out = (y && S == 1) ? y : partials;  // a single plane is the result: no second launch
     int rc;
-    if (dtype == GUFFIN_Q4_K) rc = launch_packed<GUFFIN_Q4_K>(s, w, x, xsums, partials, rows, K, N);
-    else if (dtype == GUFFIN_Q6_K) rc = launch_packed<GUFFIN_Q6_K>(s, w, x, xsums, partials, rows, K, N);
-    else rc = launch_packed<GUFFIN_Q8_0>(s, w, x, xsums, partials, rows, K, N);
-    if (rc || !y) return rc;
+    if (dtype == GUFFIN_Q4_K) rc = launch_packed<GUFFIN_Q4_K>(s, w, x, xsums, out, rows, K, N);
+    else if (dtype == GUFFIN_Q6_K) rc = launch_packed<GUFFIN_Q6_K>(s, w, x, xsums, out, rows, K, N);
+    else rc = launch_packed<GUFFIN_Q8_0>(s, w, x, xsums, out, rows, K, N);
+    if (rc || !y || S == 1) return rc;
     const uint32_t count = rows * N;
     hipLaunchKernelGGL(reduce_partials_kernel, dim3((count + 255) / 256), dim3(256), 0, s, partials, y, S, count);
     return check_launch("reduce_partials");

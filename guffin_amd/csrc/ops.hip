@@ -201,16 +201,6 @@ head_rms_norm_kernel(const float* __restrict__ x, const float* __restrict__ gamm
     for (uint32_t c = threadIdx.x; c < head_dim; c += 64) y[base + c] = x[base + c] * inv * gamma[c];
 }
 
-__device__ __forceinline__ void rope_sincos(uint32_t position, uint32_t pair, uint32_t rope_dim, float base,
-                                            float scale, float& c, float& s) {
-    // angle in double, as the CPU operator forms it (rope.cpp:109-117), times the layer's frequency scale
-    const double exponent = static_cast<double>(2u * pair) / static_cast<double>(rope_dim);
-    const double angle = static_cast<double>(position) / pow(static_cast<double>(base), exponent)
-        * static_cast<double>(scale);
-    c = static_cast<float>(cos(angle));
-    s = static_cast<float>(sin(angle));
-}
-
 // Fused q/k head norm + NeoX RoPE + fp16 KV narrowing for `rows` new tokens:
 //   q_out = rope(headnorm(q_raw)) fp32;  k_out = f16(rope(headnorm(k_raw)));  v_out = f16(v_raw)
 // One wave per (row, head); q heads first, then k heads, then v heads.  Any of the three

@@ -108,10 +108,23 @@ Scratch layout(const guffin_model_desc& m, uint32_t rows, uint32_t position, uin
     return s;
 }
 
-// positions, ancestors and the per-layer attention schedule of `rows` contiguous rows
+// positions, ancestors, the per-layer attention schedule of `rows` contiguous rows and the two
+// rotation tables (local and global frequency base) of the pass
 __global__ void stage_rows_kernel(uint32_t* positions, uint32_t* ancestors, uint32_t* schedule, uint32_t rows,
-                                  uint32_t position, uint32_t layers, uint32_t window, uint32_t global_period) {
+                                  uint32_t position, uint32_t layers, uint32_t window, uint32_t global_period,
+                                  float2* rope_local, float2* rope_global, uint32_t rope_dim, float local_base,
+                                  float global_base, float global_scale) {
     const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    const uint32_t half = rope_dim / 2;
+    if (i < rows * half) {
+        float c, s;
+        if (global_period > 1) {  // a model without local blocks has no local base
+            rope_sincos(position + i / half, i % half, rope_dim, local_base, 1.0f, c, s);
+            rope_local[i] = make_float2(c, s);
+        }
+        rope_sincos(position + i / half, i % half, rope_dim, global_base, global_scale, c, s);
+        rope_global[i] = make_float2(c, s);
+    }
     if (i < rows) { positions[i] = position + i; ancestors[i] = i; }
     if (i >= layers * rows) return;
     const uint32_t layer = i / rows, row = i % rows, p = position + row;
@@ -126,6 +139,7 @@ __global__ void stage_rows_kernel(uint32_t* positions, uint32_t* ancestors, uint
 int validate_model(const guffin_model_desc* m) {
     if (!m || !m->layers || !m->embed_rows || !m->out_norm) return fail(GUFFIN_E_ARG, "forward: null model field");
     if (m->head_dim != 256) return fail(GUFFIN_E_SHAPE, "forward: head_dim must be 256");
+    if (m->layer_count == 0) return fail(GUFFIN_E_SHAPE, "forward: the model has no blocks");
     if (m->hidden % 64 || m->ffn % 64 || m->kv_heads == 0 || m->q_heads % m->kv_heads)
         return fail(GUFFIN_E_SHAPE, "forward: widths must be multiples of 64 and q_heads a multiple of kv_heads");
     if ((m->ring_local & (m->ring_local - 1)) || (m->ring_global & (m->ring_global - 1)) || !m->ring_local || !m->ring_global)
@@ -141,12 +155,12 @@ int forward_rows(hipStream_t stream, const guffin_model_desc& m, const uint32_t*
     void* st = stream;
     const uint32_t H = m.hidden, F = m.ffn, QW = m.q_heads * m.head_dim, KW = m.kv_heads * m.head_dim;
     const float attn_scale = 1.0f / std::sqrt(static_cast<float>(m.head_dim));
-    const uint32_t n_sched = m.layer_count * rows;
-    hipLaunchKernelGGL(stage_rows_kernel, dim3((n_sched + 63) / 64), dim3(64), 0, stream, s.positions, s.ancestors,
-                       s.schedule, rows, position, m.layer_count, m.sliding_window, m.global_period);
+    const uint32_t n_stage = std::max(m.layer_count * rows, rows * (m.head_dim / 2));
+    hipLaunchKernelGGL(stage_rows_kernel, dim3((n_stage + 63) / 64), dim3(64), 0, stream, s.positions, s.ancestors,
+                       s.schedule, rows, position, m.layer_count, m.sliding_window, m.global_period,
+                       reinterpret_cast<float2*>(s.rope_local), reinterpret_cast<float2*>(s.rope_global), m.head_dim,
+                       m.local_base, m.global_base, m.global_scale);
     GUFFIN_TRY(check_launch("stage_rows"));
-    GUFFIN_TRY(guffin_hip_rope_table(st, s.positions, s.rope_local, rows, m.head_dim, m.local_base, 1.0f));
-    GUFFIN_TRY(guffin_hip_rope_table(st, s.positions, s.rope_global, rows, m.head_dim, m.global_base, m.global_scale));
     GUFFIN_TRY(guffin_hip_embed(st, m.embed_dtype, m.embed_rows, tokens, s.x, rows, H,
                                 std::sqrt(static_cast<float>(H)), m.vocab, status));
     GUFFIN_TRY(guffin_hip_rms_norm(st, s.x, 1, 0, m.layers[0].norm[0], nullptr, s.u, s.us, rows, H, m.eps, status));

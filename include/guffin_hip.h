@@ -102,7 +102,8 @@ int guffin_hip_group_sums(void* stream, const float* x, float* xsums, uint32_t r
 uint32_t guffin_hip_gemv_packed_slices(int dtype, uint32_t K, uint32_t N);
 /* Same operator as guffin_hip_gemv on repacked weights.  rows in {1, 2}.  Slice partials are
  * written to partials[S][rows][N]; if y is non-null they are summed in slice order into
- * y[rows][N] by a second small launch, otherwise the consumer does that sum. */
+ * y[rows][N] by a second small launch (with S == 1 the kernel writes y directly and leaves
+ * partials untouched), otherwise the consumer does that sum. */
 int guffin_hip_gemv_packed(void* stream, int dtype, const void* tiles, const float* x, const float* xsums,
                            float* partials, float* y, uint32_t rows, uint32_t K, uint32_t N);
 
