@@ -216,3 +216,40 @@ def test_spec_accept_fails_closed(hip, gfo):
     bad_prop = torch.full((1,), 5000, dtype=torch.int32, device="cuda")   # not in q's support
     out = hip.spec_accept(res, law, bad_prop, opts(hip), status=status).cpu().numpy().view(hip.result_dtype)[0]
     assert out["status"] == 22 and int(status[0]) & 16
+
+
+def test_device_accept_replays_reference_golden_vectors(hip):
+    """tests/golden/accept.npz was written from the compiled reference sampling.cpp
+    (prepare_speculative_distribution + sample_speculative_token): the device kernel must take the
+    same decisions on the same candidate rows, proposal laws and injected draws."""
+    import os
+    import torch
+    g = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "accept.npz"))
+    o = hip.SamplerOptions(1.0, 64, 0.95, 0.0, 1.0)
+    n = g["proposal"].size
+    status = torch.zeros(1, dtype=torch.int32, device="cuda")
+    accepted = 0
+    for i in range(n):
+        cands = np.zeros(2, hip.candidates_dtype)
+        for r in range(2):
+            cands[r]["count"] = 64
+            cands[r]["values"]["token"][:64] = g["row_tokens"][i, r]
+            cands[r]["values"]["logit"][:64] = g["row_logits"][i, r]
+        law = np.zeros(1, hip.law_dtype)
+        cnt = int(g["law_count"][i])
+        law[0]["count"] = cnt
+        law[0]["ids"][:cnt] = g["law_ids"][i, :cnt]
+        law[0]["cdf"][:cnt + 1] = g["law_cdf"][i, :cnt + 1]
+        draws = np.zeros(1, hip.draws_dtype)
+        draws[0]["u_accept"], draws[0]["u_residual"], draws[0]["u_next"] = g["draws"][i]
+        out = hip.spec_accept(torch.from_numpy(cands.view(np.uint8)).cuda(), torch.from_numpy(law.view(np.uint8)).cuda(),
+                              torch.tensor([int(g["proposal"][i])], dtype=torch.int32, device="cuda"), o,
+                              draws=torch.from_numpy(draws.view(np.uint8)).cuda(), status=status)
+        got = out.cpu().numpy().view(hip.result_dtype)[0]
+        assert got["status"] == 0, i
+        assert (int(got["accepted"]), int(got["token"]), int(got["next_root"])) == \
+            (int(g["accepted"][i]), int(g["token"][i]), int(g["next_root"][i])), i
+        assert abs(float(got["acceptance_probability"]) - float(g["acceptance"][i])) <= 1e-13
+        assert int(got["residual_count"]) == int(g["residual_count"][i])
+        accepted += int(got["accepted"])
+    assert int(status[0]) == 0 and 0 < accepted < n
