@@ -64,22 +64,25 @@ def cpu_baseline(T, D, budget_s=20.0):
     layer_weights = sum(K * N for _, (K, N) in shapes)
     frac = min(1.0, budget_s / (per_weight * layer_weights * 1.3))
     done_weights, elapsed = 0, 0.0
-    for i, (dt, (K, N)) in enumerate(shapes):
-        n = max(64, int(N * frac) // 64 * 64)
-        w = synth.make_weight(dt, K, n, 10 + i)
-        x = synth.make_activation(2, K, 20 + i)
-        t0 = time.perf_counter()
-        gfo.gemv(dt, w, x, n, threads=cores, which=ref)
-        elapsed += time.perf_counter() - t0
-        done_weights += K * n
+    # whole blocks' worth of GEMVs (fresh weights each time) until about half the budget is spent
+    repeats = max(1, int(0.6 * budget_s / max(per_weight * layer_weights * frac, 1e-9)))
+    for rep in range(repeats):
+        for i, (dt, (K, N)) in enumerate(shapes):
+            n = max(64, int(N * frac) // 64 * 64)
+            w = synth.make_weight(dt, K, n, 10 + i + 100 * rep)
+            x = synth.make_activation(2, K, 20 + i + 100 * rep)
+            t0 = time.perf_counter()
+            gfo.gemv(dt, w, x, n, threads=cores, which=ref)
+            elapsed += time.perf_counter() - t0
+            done_weights += K * n
     step_weights = (T.layers * layer_weights + T.hidden * T.vocab
                     + 0.5 * (D.layers * sum(K * N for K, N in D.proj_shapes()) + D.hidden * D.vocab))  # drafter: 1 row
     value_us = elapsed / done_weights * step_weights * 1e6
     return {
         "value": round(value_us, 1), "unit": "us", "cores": cores, "kind": kind,
-        "sample": "one 12B block's 7 GEMVs at 2 rows, first %.1f%% of each matrix's columns (%.2f s of CPU work), "
+        "sample": "%d x one 12B block's 7 GEMVs at 2 rows, first %.1f%% of each matrix's columns (%.2f s of CPU work), "
                   "scaled to the step's weight count; %s" % (
-                      100 * frac, elapsed,
+                      repeats, 100 * frac, elapsed,
                       "reference dot_q4_k_row_f32 / dot_q6_k_row_f32 (src/tensor/quantization.cpp), single thread"
                       if ref is not None else "oracle gfo_gemv_mt on all host threads"),
     }
