@@ -370,23 +370,53 @@ extern "C" int guffin_hip_prefill_rows(void* stream, const guffin_model_desc* mo
 }
 
 // ---- one H1 cycle ---------------------------------------------------------------------
+namespace guffin {
+namespace {
+// the step's buffers inside the caller's scratch arena; scratch == nullptr only measures
+struct StepBuffers {
+    uint64_t d_bytes, t_bytes, bytes;
+    uint8_t *d_scratch, *t_scratch;
+    float *d_hidden, *t_hidden, *q_parts, *q_logits, *p_parts, *p_logits;
+    uint8_t *law_ws, *sel_ws, *law, *cands, *any_ws;
+    uint32_t* words;
+    uint64_t* full_cdf;
+};
+StepBuffers carve_step(const guffin_h1_desc* d, void* scratch) {
+    const guffin_model_desc& T = *d->target;
+    const guffin_model_desc& D = *d->drafter;
+    const uint64_t V = T.vocab;
+    Arena ar {static_cast<uint8_t*>(scratch), 0, 0};
+    StepBuffers b {};
+    b.d_bytes = guffin_hip_forward_scratch_bytes(&D, 1, d->drafter_position);
+    b.t_bytes = guffin_hip_forward_scratch_bytes(&T, 2, d->target_position);
+    b.d_scratch = ar.take<uint8_t>(b.d_bytes);
+    b.t_scratch = ar.take<uint8_t>(b.t_bytes);
+    b.d_hidden = ar.take<float>(hidden_with_receipt(1, D.hidden));
+    b.t_hidden = ar.take<float>(hidden_with_receipt(2, T.hidden));
+    b.q_parts = ar.take<float>(uint64_t(slices(D.head_dtype, D.hidden, D.vocab)) * D.vocab);
+    b.q_logits = ar.take<float>(D.vocab);
+    b.p_parts = ar.take<float>(uint64_t(slices(T.head_dtype, T.hidden, V)) * 2 * V);
+    b.p_logits = ar.take<float>(2 * V);
+    b.law_ws = ar.take<uint8_t>(guffin_hip_draft_law_workspace_bytes(D.vocab));
+    b.sel_ws = ar.take<uint8_t>(guffin_hip_select_workspace_bytes(2, V, d->top_k));
+    b.law = ar.take<uint8_t>(4096 + 2 * 3088);  // the compact law, then the two candidate rows
+    b.cands = b.law ? b.law + 4096 : nullptr;
+    b.words = ar.take<uint32_t>(16);
+    if (d->full_law) {
+        b.any_ws = ar.take<uint8_t>(guffin_hip_draft_law_any_workspace_bytes(D.vocab));
+        b.full_cdf = ar.take<uint64_t>(uint64_t(D.vocab) + 1);
+    }
+    b.bytes = (ar.used + 255) & ~uint64_t{255};
+    return b;
+}
+
+}  // namespace
+}  // namespace guffin
+using namespace guffin;
+
 extern "C" uint64_t guffin_hip_h1_scratch_bytes(const guffin_h1_desc* d) {
     if (!d || validate_model(d->target) || validate_model(d->drafter)) return 0;
-    Arena ar {nullptr, 0, 0};
-    const uint64_t V = d->target->vocab;
-    ar.take<uint8_t>(guffin_hip_forward_scratch_bytes(d->drafter, 1, d->drafter_position));
-    ar.take<uint8_t>(guffin_hip_forward_scratch_bytes(d->target, 2, d->target_position));
-    ar.take<float>(hidden_with_receipt(1, d->drafter->hidden));                 // drafter hidden + sums
-    ar.take<float>(hidden_with_receipt(2, d->target->hidden));             // target hidden + sums
-    ar.take<float>(uint64_t(slices(d->drafter->head_dtype, d->drafter->hidden, d->drafter->vocab)) * d->drafter->vocab);
-    ar.take<float>(d->drafter->vocab);                                                  // q logits
-    ar.take<float>(uint64_t(slices(d->target->head_dtype, d->target->hidden, V)) * 2 * V);
-    ar.take<float>(2 * V);                                                              // p logits
-    ar.take<uint8_t>(guffin_hip_draft_law_workspace_bytes(d->drafter->vocab));
-    ar.take<uint8_t>(guffin_hip_select_workspace_bytes(2, V, d->top_k));
-    ar.take<uint8_t>(4096 + 2 * 3088);                                                  // law, candidates
-    ar.take<uint32_t>(16);
-    return (ar.used + 255) & ~uint64_t{255};
+    return carve_step(d, nullptr).bytes;
 }
 
 extern "C" int guffin_hip_h1_step(void* stream, const guffin_h1_desc* d, const uint32_t* root_token, void* scratch,
@@ -398,29 +428,20 @@ extern "C" int guffin_hip_h1_step(void* stream, const guffin_h1_desc* d, const u
     if (!d->target->head_tiles || !d->drafter->head_tiles) return fail(GUFFIN_E_ARG, "h1_step: models need packed head weights");
     if (d->drafter->vocab != d->target->vocab) return fail(GUFFIN_E_SHAPE, "h1_step: drafter and target vocabularies must coincide");
     if (reinterpret_cast<uintptr_t>(scratch) & 255u) return fail(GUFFIN_E_ALIGN, "h1_step: scratch must be 256-byte aligned");
-    if (guffin_hip_h1_scratch_bytes(d) > scratch_bytes) return fail(GUFFIN_E_CAPACITY, "h1_step: scratch arena too small");
     const guffin_model_desc& T = *d->target;
     const guffin_model_desc& D = *d->drafter;
     const uint64_t V = T.vocab;
-    Arena ar {static_cast<uint8_t*>(scratch), 0, scratch_bytes};
-    const uint64_t d_bytes = guffin_hip_forward_scratch_bytes(&D, 1, d->drafter_position);
-    const uint64_t t_bytes = guffin_hip_forward_scratch_bytes(&T, 2, d->target_position);
-    uint8_t* d_scratch = ar.take<uint8_t>(d_bytes);
-    uint8_t* t_scratch = ar.take<uint8_t>(t_bytes);
-    float* d_hidden = ar.take<float>(hidden_with_receipt(1, D.hidden));
-    float* t_hidden = ar.take<float>(hidden_with_receipt(2, T.hidden));
-    float* q_parts = ar.take<float>(uint64_t(slices(D.head_dtype, D.hidden, D.vocab)) * D.vocab);
-    float* q_logits = ar.take<float>(D.vocab);
-    float* p_parts = ar.take<float>(uint64_t(slices(T.head_dtype, T.hidden, V)) * 2 * V);
-    float* p_logits = ar.take<float>(2 * V);
-    uint8_t* law_ws = ar.take<uint8_t>(guffin_hip_draft_law_workspace_bytes(D.vocab));
-    uint8_t* sel_ws = ar.take<uint8_t>(guffin_hip_select_workspace_bytes(2, V, d->top_k));
-    uint8_t* small = ar.take<uint8_t>(4096 + 2 * 3088);
-    uint32_t* words = ar.take<uint32_t>(16);
-    void* law = small;
-    void* cands = small + 4096;
-    uint32_t* tokens = words;          // [root, proposal]
-    uint32_t* sel_status = words + 4;  // per-row selection status
+    const StepBuffers B = carve_step(d, scratch);
+    if (B.bytes > scratch_bytes) return fail(GUFFIN_E_CAPACITY, "h1_step: scratch arena too small");
+    const uint64_t d_bytes = B.d_bytes, t_bytes = B.t_bytes;
+    uint8_t *d_scratch = B.d_scratch, *t_scratch = B.t_scratch, *law_ws = B.law_ws, *sel_ws = B.sel_ws, *any_ws = B.any_ws;
+    float *d_hidden = B.d_hidden, *t_hidden = B.t_hidden, *q_parts = B.q_parts, *q_logits = B.q_logits;
+    float *p_parts = B.p_parts, *p_logits = B.p_logits;
+    uint64_t* full_cdf = B.full_cdf;
+    void* law = B.law;
+    void* cands = B.cands;
+    uint32_t* tokens = B.words;          // [root, proposal]
+    uint32_t* sel_status = B.words + 4;  // per-row selection status
     hipStream_t s = as_stream(stream);
 
     struct { float temperature; uint32_t top_k; float top_p, min_p, repetition_penalty; } opt
@@ -433,8 +454,13 @@ extern "C" int guffin_hip_h1_step(void* stream, const guffin_h1_desc* d, const u
                                        drafter_priv_v, d_hidden, d_hidden + hidden_receipt_offset(1, D.hidden), status));
     GUFFIN_TRY(guffin_hip_gemv_packed(stream, D.head_dtype, D.head_tiles, d_hidden, d_hidden + hidden_receipt_offset(1, D.hidden), q_parts,
                                       q_logits, 1, D.hidden, D.vocab));
-    GUFFIN_TRY(guffin_hip_draft_law(stream, q_logits, D.vocab, &opt, d->seed, d->step, nullptr, law_ws, law,
-                                    tokens + 1, status));
+    if (d->full_law) {
+        GUFFIN_TRY(guffin_hip_draft_law_any(stream, q_logits, D.vocab, &opt, d->seed, d->step, nullptr, any_ws, law,
+                                            full_cdf, tokens + 1, status));
+    } else {
+        GUFFIN_TRY(guffin_hip_draft_law(stream, q_logits, D.vocab, &opt, d->seed, d->step, nullptr, law_ws, law,
+                                        tokens + 1, status));
+    }
     // 2. target: rows [root, x] together, head, candidates of both rows
     GUFFIN_TRY(guffin_hip_forward_rows(stream, &T, tokens, 2, d->target_position, t_scratch, t_bytes, target_priv_k,
                                        target_priv_v, t_hidden, t_hidden + hidden_receipt_offset(2, T.hidden), status));
@@ -442,7 +468,8 @@ extern "C" int guffin_hip_h1_step(void* stream, const guffin_h1_desc* d, const u
                                       p_logits, 2, T.hidden, V));
     GUFFIN_TRY(guffin_hip_select_candidates(stream, p_logits, 2, V, d->top_k, nullptr, nullptr, sel_ws, cands, sel_status));
     // 3. accept x or draw from the residual; on acceptance draw the next root from row 1
-    GUFFIN_TRY(guffin_hip_spec_accept(stream, cands, law, tokens + 1, &opt, d->seed, d->step, nullptr, result, status));
+    GUFFIN_TRY(guffin_hip_spec_accept_law(stream, cands, law, full_cdf, D.vocab, tokens + 1, &opt, d->seed, d->step,
+                                          nullptr, result, status));
     // 4. publish: the target keeps row 0, and row 1 if x was accepted; the drafter keeps the root
     if (d->target_ring_k && d->target_ring_v) {
         GUFFIN_TRY(guffin_hip_commit_rows(stream, &T, target_priv_k, target_priv_v, d->target_ring_k, d->target_ring_v,
@@ -462,28 +489,21 @@ extern "C" int guffin_hip_h1_buffers(const guffin_h1_desc* d, void* scratch, flo
     if (!d || !scratch) return fail(GUFFIN_E_ARG, "h1_buffers: null pointer");
     GUFFIN_TRY(validate_model(d->target));
     GUFFIN_TRY(validate_model(d->drafter));
-    const guffin_model_desc& T = *d->target;
-    const guffin_model_desc& D = *d->drafter;
-    const uint64_t V = T.vocab;
-    Arena ar {static_cast<uint8_t*>(scratch), 0, 0};
-    ar.take<uint8_t>(guffin_hip_forward_scratch_bytes(&D, 1, d->drafter_position));
-    ar.take<uint8_t>(guffin_hip_forward_scratch_bytes(&T, 2, d->target_position));
-    float* dh = ar.take<float>(hidden_with_receipt(1, D.hidden));
-    float* th = ar.take<float>(hidden_with_receipt(2, T.hidden));
-    ar.take<float>(uint64_t(slices(D.head_dtype, D.hidden, D.vocab)) * D.vocab);
-    float* ql = ar.take<float>(D.vocab);
-    ar.take<float>(uint64_t(slices(T.head_dtype, T.hidden, V)) * 2 * V);
-    float* pl = ar.take<float>(2 * V);
-    ar.take<uint8_t>(guffin_hip_draft_law_workspace_bytes(D.vocab));
-    ar.take<uint8_t>(guffin_hip_select_workspace_bytes(2, V, d->top_k));
-    uint8_t* small = ar.take<uint8_t>(4096 + 2 * 3088);
-    uint32_t* words = ar.take<uint32_t>(16);
-    if (drafter_hidden) *drafter_hidden = dh;
-    if (target_hidden) *target_hidden = th;
-    if (q_logits) *q_logits = ql;
-    if (p_logits) *p_logits = pl;
-    if (law) *law = small;
-    if (candidates) *candidates = small + 4096;
-    if (tokens) *tokens = words;
+    const StepBuffers B = carve_step(d, scratch);
+    if (drafter_hidden) *drafter_hidden = B.d_hidden;
+    if (target_hidden) *target_hidden = B.t_hidden;
+    if (q_logits) *q_logits = B.q_logits;
+    if (p_logits) *p_logits = B.p_logits;
+    if (law) *law = B.law;
+    if (candidates) *candidates = B.cands;
+    if (tokens) *tokens = B.words;
+    return GUFFIN_OK;
+}
+
+extern "C" int guffin_hip_h1_full_cdf(const guffin_h1_desc* d, void* scratch, uint64_t** full_cdf) {
+    if (!d || !scratch || !full_cdf) return fail(GUFFIN_E_ARG, "h1_full_cdf: null pointer");
+    GUFFIN_TRY(validate_model(d->target));
+    GUFFIN_TRY(validate_model(d->drafter));
+    *full_cdf = carve_step(d, scratch).full_cdf;
     return GUFFIN_OK;
 }

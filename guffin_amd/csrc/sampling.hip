@@ -19,6 +19,7 @@ namespace {
 
 constexpr uint32_t kMaxTopK = 256, kMaxCandidates = 384;
 constexpr uint64_t kMassTotal = uint64_t{1} << 32;
+constexpr uint32_t kLawFull = 0xFFFFFFFFu;  // DraftLaw::count of a law held as a full-vocabulary table
 
 struct Candidates { uint32_t count; uint32_t status; struct { uint32_t token; float logit; } values[384]; };
 struct DraftLaw { uint32_t count; uint32_t pad; uint32_t ids[256]; uint64_t cdf[257]; };
@@ -114,7 +115,9 @@ __device__ __forceinline__ uint64_t score_key(float score, uint32_t token) {
 __global__ void __launch_bounds__(256)
 draft_law_kernel(const Candidates* __restrict__ top, SamplerOptions opt, uint64_t seed, uint64_t step,
                  const StepDraws* __restrict__ injected, DraftLaw* __restrict__ law,
-                 uint32_t* __restrict__ proposal, uint32_t* __restrict__ status) {
+                 uint32_t* __restrict__ proposal, uint32_t* __restrict__ status, uint32_t* __restrict__ full_error) {
+    // full_error != nullptr: the full-vocabulary kernels follow, guarded by law->count; a support of
+    // more than 256 ties then hands over to them instead of failing
     __shared__ uint64_t keys[256];
     __shared__ float score[256], weight[256];
     __shared__ uint32_t s_n;
@@ -132,7 +135,9 @@ draft_law_kernel(const Candidates* __restrict__ top, SamplerOptions opt, uint64_
             if (n > 256) st = GUFFIN_STATUS_LAW_INVALID | 32u;  // support overflow: needs the full-vocabulary law
         }
         s_n = st ? 0 : n;
-        if (st) { atomicOr(status, st); law->count = 0; *proposal = 0xFFFFFFFFu; }
+        if (full_error) *full_error = 0;
+        if (st == (GUFFIN_STATUS_LAW_INVALID | 32u) && full_error) { law->count = kLawFull; *proposal = 0xFFFFFFFFu; }
+        else if (st) { atomicOr(status, st); law->count = 0; *proposal = 0xFFFFFFFFu; }
     }
     __syncthreads();
     const uint32_t n = s_n;
@@ -194,6 +199,210 @@ draft_law_kernel(const Candidates* __restrict__ top, SamplerOptions opt, uint64_
         if (st) { atomicOr(status, st); chosen = 0xFFFFFFFFu; }
         *proposal = chosen;
     }
+}
+
+// =========================================================================================
+// Full-vocabulary proposal law: the drafter's law when the compact support does not apply
+// (top_k > 64, greedy drafting, or more than 256 tokens tied into the support).
+// src/engine/gemma3_draft.mm:295-395 (kernels), :1040-1166 (dispatch order).  Every f32 sum is
+// taken in the reference's order: sequentially inside a 256-token tile, then sequentially over
+// the tile totals.  A guard pointer makes every kernel a no-op unless the compact kernel handed
+// over (law->count == kLawFull), like the reference's compact-count guards.
+// =========================================================================================
+constexpr uint32_t kSortTile = 2048, kLawTile = 256;
+
+struct FullLawWs {
+    uint64_t* keys_a; uint64_t* keys_b;  // sort ping-pong, padded to a power of two
+    float* scores;                       // processed score by token id; -inf once filtered out
+    float* prefix;                       // running f32 sums inside each 256-tile
+    float* offsets;                      // [tiles + 1] running sums of the tile totals
+    float* best;                         // [0] maximum of the surviving scores, [1] argmax as bits
+    uint32_t* error;                     // law-local error word (also mirrored into status)
+};
+
+__device__ __forceinline__ bool guarded_off(const uint32_t* guard) { return guard && *guard != kLawFull; }
+__device__ __forceinline__ float key_score(uint64_t key) {
+    const uint32_t o = static_cast<uint32_t>(key >> 32);
+    return __uint_as_float((o & 0x80000000u) ? (o & 0x7FFFFFFFu) : ~o);
+}
+__device__ __forceinline__ uint32_t key_token(uint64_t key) { return 0xFFFFFFFFu - static_cast<uint32_t>(key); }
+__device__ __forceinline__ void law_fail(uint32_t* status, uint32_t* error, uint32_t bits) {
+    atomicOr(status, bits);
+    atomicOr(error, bits);
+}
+
+// unguarded entry: claims the law slot for the full table
+__global__ void law_begin_kernel(DraftLaw* law, uint32_t* proposal, uint32_t* error) {
+    law->count = kLawFull; law->pad = 0; *proposal = 0xFFFFFFFFu; *error = 0;
+}
+
+// score = logit / T (gd_process), then 2048-token tiles sorted by (score desc, token asc)
+__global__ void __launch_bounds__(1024)
+law_sort_tile_kernel(const float* __restrict__ logits, uint32_t vocab, float temperature, bool sort,
+                     const uint32_t* __restrict__ guard, FullLawWs ws, uint32_t* __restrict__ status) {
+    if (guarded_off(guard)) return;
+    __shared__ uint64_t keys[kSortTile];
+    for (uint32_t e = threadIdx.x; e < kSortTile; e += blockDim.x) {
+        const uint32_t token = blockIdx.x * kSortTile + e;
+        uint64_t key = 0;  // padding sorts behind every real entry
+        if (token < vocab) {
+            float score = logits[token];
+            if (!isfinite(score)) { law_fail(status, ws.error, GUFFIN_STATUS_LAW_INVALID | GUFFIN_STATUS_NONFINITE); score = 0.f; }
+            if (temperature > 0.f) score = __fdiv_rn(score, temperature);
+            if (!isfinite(score)) { law_fail(status, ws.error, GUFFIN_STATUS_LAW_INVALID | GUFFIN_STATUS_NONFINITE); score = 0.f; }
+            ws.scores[token] = score;
+            key = score_key(score, token);
+        }
+        keys[e] = key;
+    }
+    if (!sort) return;
+    bitonic(keys, kSortTile, true);
+    for (uint32_t e = threadIdx.x; e < kSortTile; e += blockDim.x) ws.keys_a[size_t(blockIdx.x) * kSortTile + e] = keys[e];
+}
+
+// one merge level of sorted runs of `width` keys (descending; keys are distinct except padding)
+__global__ void __launch_bounds__(256)
+law_merge_kernel(const uint64_t* __restrict__ in, uint64_t* __restrict__ out, uint32_t width, uint32_t padded,
+                 const uint32_t* __restrict__ guard) {
+    if (guarded_off(guard)) return;
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= padded) return;
+    const uint32_t rank = i % (2 * width);
+    const uint64_t* a = in + (i - rank);
+    const uint64_t* b = a + width;
+    uint32_t lo = rank > width ? rank - width : 0, hi = rank < width ? rank : width;
+    while (lo < hi) {  // how many of the first `rank` outputs come from run a
+        const uint32_t mid = (lo + hi) >> 1;
+        if (a[mid] >= b[rank - mid - 1]) lo = mid + 1; else hi = mid;
+    }
+    const uint32_t ai = lo, bi = rank - lo;
+    out[i] = (ai < width && (bi >= width || a[ai] >= b[bi])) ? a[ai] : b[bi];
+}
+
+// sequential offsets over the tile totals left in offsets[1..tiles] (gd_offsets); one thread
+__device__ void finish_offsets(float* offsets, uint32_t tiles) {
+    float s = 0.f;
+    offsets[0] = 0.f;
+    for (uint32_t g = 0; g < tiles; ++g) { s = __fadd_rn(s, offsets[g + 1]); offsets[g + 1] = s; }
+}
+
+// gd_filter_prefix + gd_offsets: weights of the sorted entries walked from the tail
+__global__ void __launch_bounds__(1024)
+law_filter_prefix_kernel(const uint64_t* __restrict__ sorted, uint32_t vocab, uint32_t top_k,
+                         const uint32_t* __restrict__ guard, FullLawWs ws) {
+    if (guarded_off(guard)) return;
+    const uint32_t tiles = vocab / kLawTile;
+    const float best = key_score(sorted[0]);
+    const float cutoff = key_score(sorted[(top_k < vocab ? top_k : vocab) - 1]);
+    for (uint32_t g = threadIdx.x; g < tiles; g += blockDim.x) {
+        float run = 0.f;
+        for (uint32_t j = 0; j < kLawTile; ++j) {
+            const float score = key_score(sorted[vocab - 1 - (g * kLawTile + j)]);
+            run = __fadd_rn(run, score >= cutoff ? law_exp(__fsub_rn(score, best)) : 0.f);
+            ws.prefix[g * kLawTile + j] = run;
+        }
+        ws.offsets[g + 1] = run;
+    }
+    __threadfence();
+    __syncthreads();
+    if (threadIdx.x == 0) finish_offsets(ws.offsets, tiles);
+}
+
+// gd_filter_apply: top-k cutoff (ties kept), ascending-tail top-p, min-p; the best entry always stays
+__global__ void __launch_bounds__(256)
+law_filter_apply_kernel(const uint64_t* __restrict__ sorted, uint32_t vocab, SamplerOptions opt,
+                        const uint32_t* __restrict__ guard, FullLawWs ws) {
+    if (guarded_off(guard)) return;
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= vocab) return;
+    const uint32_t tiles = vocab / kLawTile;
+    const uint64_t item = sorted[vocab - 1 - i];
+    const float score = key_score(item), best = key_score(sorted[0]);
+    const float cutoff = key_score(sorted[(opt.top_k < vocab ? opt.top_k : vocab) - 1]);
+    bool keep = score >= cutoff;
+    const float tail = __fdiv_rn(__fadd_rn(ws.offsets[i / kLawTile], ws.prefix[i]), ws.offsets[tiles]);
+    if (opt.top_p < 1.0f && tail <= __fsub_rn(1.0f, opt.top_p) && i != vocab - 1) keep = false;
+    if (opt.min_p > 0.0f && law_exp(__fsub_rn(score, best)) < opt.min_p && i != vocab - 1) keep = false;
+    if (!keep) ws.scores[key_token(item)] = -INFINITY;
+}
+
+// gd_max + gd_max_finish + gd_prefix + gd_offsets: maximum (lowest id on ties) of the surviving
+// scores, then the weights exp(score - max) summed in token order
+__global__ void __launch_bounds__(1024)
+law_weights_kernel(uint32_t vocab, bool greedy, const uint32_t* __restrict__ guard, FullLawWs ws,
+                   uint32_t* __restrict__ status) {
+    if (guarded_off(guard)) return;
+    __shared__ float s_max[1024];
+    __shared__ uint32_t s_arg[1024];
+    const uint32_t t = threadIdx.x, tiles = vocab / kLawTile;
+    float m = -INFINITY;
+    uint32_t arg = 0xFFFFFFFFu;
+    for (uint32_t i = t; i < vocab; i += blockDim.x) {
+        const float v = ws.scores[i];
+        if (v > m) { m = v; arg = i; }  // ids ascend within a thread: the first maximum is the lowest id
+    }
+    s_max[t] = m; s_arg[t] = arg;
+    __syncthreads();
+    for (uint32_t half = blockDim.x >> 1; half > 0; half >>= 1) {
+        if (t < half && (s_max[t + half] > s_max[t] || (s_max[t + half] == s_max[t] && s_arg[t + half] < s_arg[t]))) {
+            s_max[t] = s_max[t + half]; s_arg[t] = s_arg[t + half];
+        }
+        __syncthreads();
+    }
+    const float maximum = s_max[0];
+    if (t == 0) {
+        ws.best[0] = maximum;
+        ws.best[1] = __uint_as_float(s_arg[0]);
+        if (!isfinite(maximum)) law_fail(status, ws.error, GUFFIN_STATUS_LAW_INVALID);
+    }
+    if (greedy) return;
+    for (uint32_t g = t; g < tiles; g += blockDim.x) {
+        float run = 0.f;
+        for (uint32_t j = 0; j < kLawTile; ++j) {
+            const float score = ws.scores[g * kLawTile + j];
+            // the reference divides by a temperature of exactly 1 here: scores were tempered up front
+            run = __fadd_rn(run, score > -INFINITY ? law_exp(__fdiv_rn(__fsub_rn(score, maximum), 1.0f)) : 0.f);
+            ws.prefix[g * kLawTile + j] = run;
+        }
+        ws.offsets[g + 1] = run;
+    }
+    __threadfence();
+    __syncthreads();
+    if (t == 0) {
+        finish_offsets(ws.offsets, tiles);
+        const float total = ws.offsets[tiles];
+        if (!(total > 0.f) || !isfinite(total)) law_fail(status, ws.error, GUFFIN_STATUS_LAW_INVALID);
+    }
+}
+
+__device__ __forceinline__ uint64_t full_cdf_at(uint32_t i, uint32_t vocab, bool greedy, const FullLawWs& ws) {
+    if (greedy) return i <= __float_as_uint(ws.best[1]) ? 0 : kMassTotal;
+    if (i == 0) return 0;
+    if (i == vocab) return kMassTotal;
+    const uint32_t b = i / kLawTile;
+    const float sum = (i % kLawTile == 0) ? ws.offsets[b] : __fadd_rn(ws.offsets[b], ws.prefix[i - 1]);
+    float scaled = __fmul_rn(__fdiv_rn(sum, ws.offsets[vocab / kLawTile]), 4294967296.0f);
+    scaled = fminf(fmaxf(scaled, 0.0f), 4294967296.0f);
+    return static_cast<uint64_t>(scaled);
+}
+
+// gd_cdf + gd_select: the u64 table, its validation, and the token whose bin holds the step's word
+__global__ void __launch_bounds__(256)
+law_cdf_select_kernel(uint32_t vocab, bool greedy, uint64_t seed, uint64_t step, const StepDraws* __restrict__ injected,
+                      const uint32_t* __restrict__ guard, FullLawWs ws, uint64_t* __restrict__ cdf,
+                      uint32_t* __restrict__ proposal, uint32_t* __restrict__ status) {
+    if (guarded_off(guard)) return;
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i > vocab) return;
+    if (*ws.error != 0) { cdf[i] = 0; return; }  // raised by an earlier kernel: no law, no proposal
+    const uint64_t begin = full_cdf_at(i, vocab, greedy, ws);
+    cdf[i] = begin;
+    if (i == vocab) return;
+    const uint64_t end = full_cdf_at(i + 1, vocab, greedy, ws);
+    if (begin > end || end > kMassTotal) { atomicOr(status, GUFFIN_STATUS_LAW_INVALID); return; }
+    if (begin < end && !(ws.scores[i] > -INFINITY)) { atomicOr(status, GUFFIN_STATUS_LAW_INVALID); return; }
+    const uint64_t word = injected ? injected->word : step_draws(seed, step).word;
+    if (word >= begin && word < end) *proposal = i;
 }
 
 // =========================================================================================
@@ -325,7 +534,13 @@ __device__ uint32_t select_prepared(const Prepared& p, double draw) {
     return p.token[p.count - 1];
 }
 
-__device__ uint64_t law_mass(const DraftLaw* law, uint32_t token, uint64_t* begin) {
+__device__ uint64_t law_mass(const DraftLaw* law, const uint64_t* full_cdf, uint32_t vocab, uint32_t token,
+                             uint64_t* begin) {
+    if (law->count == kLawFull) {  // gather from the full table (src/engine/gemma3_draft.mm:1544-1545)
+        if (!full_cdf || token >= vocab) { if (begin) *begin = 0; return 0; }
+        if (begin) *begin = full_cdf[token];
+        return full_cdf[token + 1] - full_cdf[token];
+    }
     uint32_t lo = 0, hi = law->count;
     while (lo < hi) {
         const uint32_t mid = (lo + hi) >> 1;
@@ -338,7 +553,7 @@ __device__ uint64_t law_mass(const DraftLaw* law, uint32_t token, uint64_t* begi
 
 __global__ void __launch_bounds__(512)
 spec_accept_kernel(const Candidates* __restrict__ rows, const DraftLaw* __restrict__ law,
-                   const uint32_t* __restrict__ proposal_ptr, SamplerOptions opt, uint64_t seed, uint64_t step,
+                   const uint64_t* __restrict__ full_cdf, uint32_t vocab, const uint32_t* __restrict__ proposal_ptr, SamplerOptions opt, uint64_t seed, uint64_t step,
                    const StepDraws* __restrict__ injected, SpecResult* __restrict__ result,
                    uint32_t* __restrict__ status) {
     __shared__ Scratch sc;
@@ -355,7 +570,7 @@ spec_accept_kernel(const Candidates* __restrict__ rows, const DraftLaw* __restri
         result->proposal = proposal;
     }
     int rc = prepare_distribution(&rows[0], opt, nullptr, 0, sc, target);
-    if (!rc && t < target.count) q[t] = law_mass(law, target.token[t], nullptr);
+    if (!rc && t < target.count) q[t] = law_mass(law, full_cdf, vocab, target.token[t], nullptr);
     __syncthreads();
     if (t == 0) {
         int code = rc;
@@ -365,7 +580,7 @@ spec_accept_kernel(const Candidates* __restrict__ rows, const DraftLaw* __restri
         if (!code) { normalization = validated_total(target); if (normalization < 0.0) code = -21; }
         uint64_t begin = 0, proposal_mass = 0;
         if (!code) {
-            proposal_mass = law_mass(law, proposal, &begin);
+            proposal_mass = law_mass(law, full_cdf, vocab, proposal, &begin);
             if (proposal_mass == 0 || proposal_mass > kMassTotal || begin > kMassTotal - proposal_mass) code = -22;
         }
         bool in_target = false;
@@ -446,16 +661,39 @@ extern "C" uint64_t guffin_hip_draft_law_workspace_bytes(uint32_t vocab) {
     return tiles * 257 * 8 + sizeof(Candidates) + 16;
 }
 
-extern "C" int guffin_hip_draft_law(void* stream, const float* logits, uint32_t vocab, const void* options,
-                                    uint64_t seed, uint64_t step, const void* injected_draws, void* workspace,
-                                    void* law, uint32_t* proposal, uint32_t* status) {
-    if (!logits || !options || !workspace || !law || !proposal || !status) return fail(GUFFIN_E_ARG, "draft_law: null pointer");
-    if (vocab < 1) return fail(GUFFIN_E_SHAPE, "draft_law: empty vocabulary");
-    if (reinterpret_cast<uintptr_t>(workspace) & 7u) return fail(GUFFIN_E_ALIGN, "draft_law: workspace must be 8-byte aligned");
-    const SamplerOptions opt = *static_cast<const SamplerOptions*>(options);
-    if (!(opt.temperature > 0.f) || opt.top_k == 0 || opt.top_k > 64)
-        return fail(GUFFIN_E_ARG, "draft_law: the compact law needs temperature > 0 and top_k in [1, 64]");
-    hipStream_t s = as_stream(stream);
+namespace {
+
+uint32_t padded_vocab(uint32_t vocab) {
+    uint32_t p = kSortTile;
+    while (p < vocab) p <<= 1;
+    return p;
+}
+uint64_t align16(uint64_t v) { return (v + 15) & ~uint64_t{15}; }
+uint64_t compact_ws_bytes(uint32_t vocab) { return align16(guffin_hip_draft_law_workspace_bytes(vocab)); }
+
+FullLawWs carve_full_ws(uint8_t* base, uint32_t vocab) {
+    const uint64_t padded = padded_vocab(vocab), tiles = vocab / kLawTile;
+    FullLawWs ws;
+    uint64_t at = 0;
+    auto take = [&](uint64_t bytes) { uint8_t* p = base ? base + at : nullptr; at += align16(bytes); return p; };
+    ws.keys_a = reinterpret_cast<uint64_t*>(take(padded * 8));
+    ws.keys_b = reinterpret_cast<uint64_t*>(take(padded * 8));
+    ws.scores = reinterpret_cast<float*>(take(uint64_t(vocab) * 4));
+    ws.prefix = reinterpret_cast<float*>(take(uint64_t(vocab) * 4));
+    ws.offsets = reinterpret_cast<float*>(take((tiles + 1) * 4));
+    ws.best = reinterpret_cast<float*>(take(8));
+    ws.error = reinterpret_cast<uint32_t*>(take(4));
+    return ws;
+}
+uint64_t full_ws_bytes(uint32_t vocab) {
+    const uint64_t padded = padded_vocab(vocab), tiles = vocab / kLawTile;
+    return align16(padded * 8) * 2 + align16(uint64_t(vocab) * 4) * 2 + align16((tiles + 1) * 4) + 16 + 16;
+}
+bool compact_options(const SamplerOptions& o) { return o.temperature > 0.f && o.top_k >= 1 && o.top_k <= 64; }
+
+int launch_compact_law(hipStream_t s, const float* logits, uint32_t vocab, const SamplerOptions& opt, uint64_t seed,
+                       uint64_t step, const void* injected_draws, void* workspace, void* law, uint32_t* proposal,
+                       uint32_t* status, uint32_t* full_error) {
     const uint64_t tiles = (uint64_t(vocab) + 2047) / 2048;
     uint8_t* ws = static_cast<uint8_t*>(workspace);
     Candidates* top = reinterpret_cast<Candidates*>(ws + ((tiles * 257 * 8 + 15) & ~uint64_t{15}));
@@ -464,20 +702,102 @@ extern "C" int guffin_hip_draft_law(void* stream, const float* logits, uint32_t 
                                           nullptr, ws, top, status))
         return rc;
     hipLaunchKernelGGL(draft_law_kernel, dim3(1), dim3(256), 0, s, top, opt, seed, step,
-                       static_cast<const StepDraws*>(injected_draws), static_cast<DraftLaw*>(law), proposal, status);
+                       static_cast<const StepDraws*>(injected_draws), static_cast<DraftLaw*>(law), proposal, status,
+                       full_error);
     return check_launch("draft_law");
+}
+
+// the full-vocabulary kernels in the reference's dispatch order (src/engine/gemma3_draft.mm:1040-1166)
+int launch_full_law(hipStream_t s, const float* logits, uint32_t vocab, const SamplerOptions& opt, uint64_t seed,
+                    uint64_t step, const void* injected_draws, const uint32_t* guard, const FullLawWs& ws,
+                    uint64_t* cdf, uint32_t* proposal, uint32_t* status) {
+    const bool greedy = opt.temperature == 0.f;
+    const uint32_t padded = padded_vocab(vocab);
+    hipLaunchKernelGGL(law_sort_tile_kernel, dim3(padded / kSortTile), dim3(1024), 0, s, logits, vocab, opt.temperature,
+                       !greedy, guard, ws, status);
+    if (!greedy) {
+        const uint64_t* sorted = ws.keys_a;
+        uint64_t* other = ws.keys_b;
+        for (uint32_t width = kSortTile; width < padded; width <<= 1) {
+            hipLaunchKernelGGL(law_merge_kernel, dim3(padded / 256), dim3(256), 0, s, sorted, other, width, padded, guard);
+            const uint64_t* done = other;
+            other = const_cast<uint64_t*>(sorted);
+            sorted = done;
+        }
+        hipLaunchKernelGGL(law_filter_prefix_kernel, dim3(1), dim3(1024), 0, s, sorted, vocab, opt.top_k, guard, ws);
+        hipLaunchKernelGGL(law_filter_apply_kernel, dim3((vocab + 255) / 256), dim3(256), 0, s, sorted, vocab, opt, guard, ws);
+    }
+    hipLaunchKernelGGL(law_weights_kernel, dim3(1), dim3(1024), 0, s, vocab, greedy, guard, ws, status);
+    hipLaunchKernelGGL(law_cdf_select_kernel, dim3(vocab / 256 + 1), dim3(256), 0, s, vocab, greedy, seed, step,
+                       static_cast<const StepDraws*>(injected_draws), guard, ws, cdf, proposal, status);
+    return check_launch("draft_law_full");
+}
+
+}  // namespace
+
+extern "C" int guffin_hip_draft_law(void* stream, const float* logits, uint32_t vocab, const void* options,
+                                    uint64_t seed, uint64_t step, const void* injected_draws, void* workspace,
+                                    void* law, uint32_t* proposal, uint32_t* status) {
+    if (!logits || !options || !workspace || !law || !proposal || !status) return fail(GUFFIN_E_ARG, "draft_law: null pointer");
+    if (vocab < 1) return fail(GUFFIN_E_SHAPE, "draft_law: empty vocabulary");
+    if (reinterpret_cast<uintptr_t>(workspace) & 7u) return fail(GUFFIN_E_ALIGN, "draft_law: workspace must be 8-byte aligned");
+    const SamplerOptions opt = *static_cast<const SamplerOptions*>(options);
+    if (!compact_options(opt))
+        return fail(GUFFIN_E_ARG, "draft_law: the compact law needs temperature > 0 and top_k in [1, 64]");
+    return launch_compact_law(as_stream(stream), logits, vocab, opt, seed, step, injected_draws, workspace, law,
+                              proposal, status, nullptr);
+}
+
+extern "C" uint64_t guffin_hip_draft_law_any_workspace_bytes(uint32_t vocab) {
+    return compact_ws_bytes(vocab) + full_ws_bytes(vocab);
+}
+
+extern "C" int guffin_hip_draft_law_any(void* stream, const float* logits, uint32_t vocab, const void* options,
+                                        uint64_t seed, uint64_t step, const void* injected_draws, void* workspace,
+                                        void* law, uint64_t* full_cdf, uint32_t* proposal, uint32_t* status) {
+    if (!logits || !options || !workspace || !law || !full_cdf || !proposal || !status)
+        return fail(GUFFIN_E_ARG, "draft_law_any: null pointer");
+    if (vocab < kLawTile || vocab % kLawTile != 0)
+        return fail(GUFFIN_E_SHAPE, "draft_law_any: the vocabulary must be a positive multiple of 256");
+    if (reinterpret_cast<uintptr_t>(workspace) & 15u) return fail(GUFFIN_E_ALIGN, "draft_law_any: workspace must be 16-byte aligned");
+    if (reinterpret_cast<uintptr_t>(full_cdf) & 7u) return fail(GUFFIN_E_ALIGN, "draft_law_any: the table must be 8-byte aligned");
+    const SamplerOptions opt = *static_cast<const SamplerOptions*>(options);
+    if (!std::isfinite(opt.temperature) || opt.temperature < 0.f || opt.top_k < 1 || opt.top_k > kMaxTopK
+        || !(opt.top_p > 0.f) || opt.top_p > 1.f || !(opt.min_p >= 0.f) || opt.min_p > 1.f)
+        return fail(GUFFIN_E_ARG, "draft_law_any: sampler options out of range");
+    hipStream_t s = as_stream(stream);
+    uint8_t* base = static_cast<uint8_t*>(workspace);
+    const FullLawWs ws = carve_full_ws(base + compact_ws_bytes(vocab), vocab);
+    DraftLaw* slot = static_cast<DraftLaw*>(law);
+    if (compact_options(opt)) {
+        // the compact law; its kernel hands over to the guarded full-vocabulary kernels when more
+        // than 256 tokens tie into the support
+        if (int rc = launch_compact_law(s, logits, vocab, opt, seed, step, injected_draws, base, law, proposal, status, ws.error))
+            return rc;
+        return launch_full_law(s, logits, vocab, opt, seed, step, injected_draws, &slot->count, ws, full_cdf, proposal, status);
+    }
+    hipLaunchKernelGGL(law_begin_kernel, dim3(1), dim3(1), 0, s, slot, proposal, ws.error);
+    return launch_full_law(s, logits, vocab, opt, seed, step, injected_draws, nullptr, ws, full_cdf, proposal, status);
+}
+
+extern "C" int guffin_hip_spec_accept_law(void* stream, const void* target_candidates, const void* law,
+                                          const uint64_t* full_cdf, uint32_t vocab, const uint32_t* proposal,
+                                          const void* options, uint64_t seed, uint64_t step,
+                                          const void* injected_draws, void* result, uint32_t* status) {
+    if (!target_candidates || !law || !proposal || !options || !result) return fail(GUFFIN_E_ARG, "spec_accept: null pointer");
+    const SamplerOptions opt = *static_cast<const SamplerOptions*>(options);
+    hipLaunchKernelGGL(spec_accept_kernel, dim3(1), dim3(512), 0, as_stream(stream),
+                       static_cast<const Candidates*>(target_candidates), static_cast<const DraftLaw*>(law), full_cdf,
+                       vocab, proposal, opt, seed, step, static_cast<const StepDraws*>(injected_draws),
+                       static_cast<SpecResult*>(result), status);
+    return check_launch("spec_accept");
 }
 
 extern "C" int guffin_hip_spec_accept(void* stream, const void* target_candidates, const void* law,
                                       const uint32_t* proposal, const void* options, uint64_t seed, uint64_t step,
                                       const void* injected_draws, void* result, uint32_t* status) {
-    if (!target_candidates || !law || !proposal || !options || !result) return fail(GUFFIN_E_ARG, "spec_accept: null pointer");
-    const SamplerOptions opt = *static_cast<const SamplerOptions*>(options);
-    hipLaunchKernelGGL(spec_accept_kernel, dim3(1), dim3(512), 0, as_stream(stream),
-                       static_cast<const Candidates*>(target_candidates), static_cast<const DraftLaw*>(law), proposal,
-                       opt, seed, step, static_cast<const StepDraws*>(injected_draws),
-                       static_cast<SpecResult*>(result), status);
-    return check_launch("spec_accept");
+    return guffin_hip_spec_accept_law(stream, target_candidates, law, nullptr, 0, proposal, options, seed, step,
+                                      injected_draws, result, status);
 }
 
 extern "C" int guffin_hip_step_draws(uint64_t seed, uint64_t step, void* out_draws_host) {

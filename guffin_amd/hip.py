@@ -350,6 +350,32 @@ def draft_law(logits, options, seed=0, step=0, draws=None, law=None, proposal=No
     return law, proposal, status
 
 
+def draft_law_any(logits, options, seed=0, step=0, draws=None, status=None):
+    """The drafter's law by whichever path it needs: (law, full table, proposal, status)."""
+    vocab = logits.numel()
+    lib().guffin_hip_draft_law_any_workspace_bytes.restype = C.c_uint64
+    workspace = _bytes(lib().guffin_hip_draft_law_any_workspace_bytes(vocab))
+    law = _bytes(law_dtype.itemsize)
+    cdf = torch.zeros(vocab + 1, dtype=torch.int64, device=logits.device)
+    proposal = torch.zeros(1, dtype=torch.int32, device=logits.device)
+    if status is None:
+        status = torch.zeros(1, dtype=torch.int32, device=logits.device)
+    check(lib().guffin_hip_draft_law_any(_stream(), _p(logits), vocab, C.byref(options), C.c_uint64(seed),
+                                         C.c_uint64(step), _p(draws), _p(workspace), _p(law), _p(cdf),
+                                         _p(proposal), _p(status)))
+    return law, cdf, proposal, status
+
+
+def spec_accept_law(cands, law, cdf, proposal, options, seed=0, step=0, draws=None, result=None, status=None):
+    if result is None:
+        result = _bytes(result_dtype.itemsize)
+    vocab = 0 if cdf is None else cdf.numel() - 1
+    check(lib().guffin_hip_spec_accept_law(_stream(), _p(cands), _p(law), _p(cdf), vocab, _p(proposal),
+                                           C.byref(options), C.c_uint64(seed), C.c_uint64(step), _p(draws),
+                                           _p(result), _p(status)))
+    return result
+
+
 def spec_accept(cands, law, proposal, options, seed=0, step=0, draws=None, result=None, status=None):
     if result is None:
         result = _bytes(result_dtype.itemsize)

@@ -38,7 +38,7 @@ class H1Desc(C.Structure):
                 ("temperature", C.c_float), ("top_k", C.c_uint32), ("top_p", C.c_float), ("min_p", C.c_float),
                 ("seed", C.c_uint64), ("step", C.c_uint64),
                 ("target_ring_k", C.c_void_p), ("target_ring_v", C.c_void_p),
-                ("drafter_ring_k", C.c_void_p), ("drafter_ring_v", C.c_void_p)]
+                ("drafter_ring_k", C.c_void_p), ("drafter_ring_v", C.c_void_p), ("full_law", C.c_uint32)]
 
 
 @dataclass(frozen=True)
@@ -297,13 +297,14 @@ class H1Plan:
     """One speculative cycle: buffers, descriptor and the call into guffin_hip_h1_step."""
 
     def __init__(self, target, drafter, target_position, drafter_position, temperature=1.0, top_k=64,
-                 top_p=0.95, min_p=0.0, seed=0, publish=True):
+                 top_p=0.95, min_p=0.0, seed=0, publish=True, full_law=False):
         self.target, self.drafter = target, drafter
         d = self.desc = H1Desc()
         d.target, d.drafter = C.pointer(target.desc), C.pointer(drafter.desc)
         d.target_position, d.drafter_position = target_position, drafter_position
         d.temperature, d.top_k, d.top_p, d.min_p = temperature, top_k, top_p, min_p
         d.seed, d.step = seed, 0
+        d.full_law = 1 if full_law else 0
         if publish:
             d.target_ring_k, d.target_ring_v = target.ring_k_table.data_ptr(), target.ring_v_table.data_ptr()
             d.drafter_ring_k, d.drafter_ring_v = drafter.ring_k_table.data_ptr(), drafter.ring_v_table.data_ptr()
@@ -342,7 +343,10 @@ class H1Plan:
             off = ptr.value - base
             return self.scratch[off:off + count * torch.tensor([], dtype=dtype).element_size()].view(dtype)
 
+        full = C.c_void_p()
+        hip.check(hip.lib().guffin_hip_h1_full_cdf(C.byref(self.desc), hip._p(self.scratch), C.byref(full)))
         return {
+            "full_cdf": view(full, D.vocab + 1, torch.int64) if full.value else None,
             "drafter_hidden": view(ptrs[0], D.hidden, torch.float32),
             "target_hidden": view(ptrs[1], 2 * T.hidden, torch.float32).view(2, T.hidden),
             "q_logits": view(ptrs[2], D.vocab, torch.float32),

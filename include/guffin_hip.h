@@ -242,6 +242,18 @@ uint64_t guffin_hip_draft_law_workspace_bytes(uint32_t vocab);
 int guffin_hip_draft_law(void* stream, const float* logits, uint32_t vocab, const void* options,
                          uint64_t seed, uint64_t step, const void* injected_draws, void* workspace,
                          void* law, uint32_t* proposal, uint32_t* status);
+/* The drafter's law by whichever path the options and the logits need, as the reference's
+ * `sample` encodes it (src/engine/gemma3_draft.mm:995-1166): the compact law when temperature > 0
+ * and top_k <= 64, followed by the full-vocabulary kernels (:295-395), which run only when more
+ * than 256 tokens tie into the compact support; the full-vocabulary kernels alone otherwise
+ * (top_k > 64, or temperature == 0: all mass on the lowest-id argmax).  A law held as the full
+ * table is marked by law.count == 0xFFFFFFFF and lives in full_cdf: u64[vocab + 1], bin of token
+ * i = [full_cdf[i], full_cdf[i+1]), last entry 2^32.  vocab must be a multiple of 256 (the
+ * reference's tile of sequential f32 sums). */
+uint64_t guffin_hip_draft_law_any_workspace_bytes(uint32_t vocab);
+int guffin_hip_draft_law_any(void* stream, const float* logits, uint32_t vocab, const void* options,
+                             uint64_t seed, uint64_t step, const void* injected_draws, void* workspace,
+                             void* law, uint64_t* full_cdf, uint32_t* proposal, uint32_t* status);
 /* One accept / residual decision (src/engine/sampling.cpp:394-499, 561-656):
  * target law p from row 0 of target_candidates (two rows of the select result), q gathered
  * from `law` on p's support, accept iff u_accept < min(1, p(x)/q(x)), else inverse-CDF draw
@@ -253,6 +265,12 @@ int guffin_hip_draft_law(void* stream, const float* logits, uint32_t vocab, cons
 int guffin_hip_spec_accept(void* stream, const void* target_candidates, const void* law,
                            const uint32_t* proposal, const void* options, uint64_t seed, uint64_t step,
                            const void* injected_draws, void* result, uint32_t* status);
+/* The same decision when the law may be a full table (guffin_hip_draft_law_any): q is then
+ * gathered as full_cdf[token + 1] - full_cdf[token] (src/engine/gemma3_draft.mm:1528-1581). */
+int guffin_hip_spec_accept_law(void* stream, const void* target_candidates, const void* law,
+                               const uint64_t* full_cdf, uint32_t vocab, const uint32_t* proposal,
+                               const void* options, uint64_t seed, uint64_t step,
+                               const void* injected_draws, void* result, uint32_t* status);
 /* Host evaluation of the draw schedule above (out: the draws struct). */
 int guffin_hip_step_draws(uint64_t seed, uint64_t step, void* out_draws_host);
 
@@ -344,6 +362,7 @@ typedef struct guffin_h1_desc {
     uint64_t seed, step;
     void* const* target_ring_k; void* const* target_ring_v;
     void* const* drafter_ring_k; void* const* drafter_ring_v;
+    uint32_t full_law;  /* != 0: encode the full-vocabulary law too (overflow fallback, top_k > 64, greedy) */
 } guffin_h1_desc;
 uint64_t guffin_hip_h1_scratch_bytes(const guffin_h1_desc* desc);
 int guffin_hip_h1_step(void* stream, const guffin_h1_desc* desc, const uint32_t* root_token, void* scratch,
@@ -353,6 +372,8 @@ int guffin_hip_h1_step(void* stream, const guffin_h1_desc* desc, const uint32_t*
 int guffin_hip_h1_buffers(const guffin_h1_desc* desc, void* scratch, float** drafter_hidden,
                           float** target_hidden, float** q_logits, float** p_logits, void** law,
                           void** candidates, uint32_t** tokens);
+/* The full-vocabulary table of the last step (desc->full_law != 0), else NULL. */
+int guffin_hip_h1_full_cdf(const guffin_h1_desc* desc, void* scratch, uint64_t** full_cdf);
 
 #ifdef __cplusplus
 }

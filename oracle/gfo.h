@@ -151,6 +151,11 @@ int gfo_spec_accept(const gfo_token_logit* row0, uint32_t n0,
                     const gfo_sampler_options* opt,
                     double u_accept, double u_residual, double u_next,
                     gfo_spec_result* out);
+/* the same decision with q gathered from a full-vocabulary table (cdf: vocab+1 entries) */
+int gfo_spec_accept_full(const gfo_token_logit* row0, uint32_t n0, const gfo_token_logit* row1,
+                         uint32_t n1, const uint64_t* cdf, uint32_t vocab, uint32_t proposal,
+                         const gfo_sampler_options* opt, double u_accept, double u_residual,
+                         double u_next, gfo_spec_result* out);
 
 void gfo_philox4x32_10(const uint32_t counter[4], const uint32_t key[2], uint32_t out[4]);
 /* draws of one H1 step: word, u_accept, u_residual, u_next */

@@ -237,6 +237,24 @@ def spec_accept(row0, row1, law, proposal, opt, u_accept, u_residual, u_next, wh
     return rc, out
 
 
+def spec_accept_full(row0, row1, cdf, proposal, opt, u_accept, u_residual, u_next):
+    row0 = np.ascontiguousarray(row0, token_logit)
+    row1 = np.ascontiguousarray(row1, token_logit)
+    cdf = np.ascontiguousarray(cdf, np.uint64)
+    out = SpecResult()
+    rc = lib().gfo_spec_accept_full(_ptr(row0), row0.size, _ptr(row1), row1.size, _ptr(cdf),
+                                    C.c_uint32(cdf.size - 1), C.c_uint32(proposal), C.byref(opt),
+                                    C.c_double(u_accept), C.c_double(u_residual), C.c_double(u_next),
+                                    C.byref(out))
+    return rc, out
+
+
+def draft_select_full(cdf, word):
+    cdf = np.ascontiguousarray(cdf, np.uint64)
+    lib().gfo_draft_select_full.restype = C.c_uint32
+    return lib().gfo_draft_select_full(_ptr(cdf), C.c_uint32(cdf.size - 1), C.c_uint32(word))
+
+
 def philox(counter, key):
     c = (C.c_uint32 * 4)(*counter)
     k = (C.c_uint32 * 2)(*key)

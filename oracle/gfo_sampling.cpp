@@ -92,6 +92,15 @@ uint64_t law_mass(const gfo_draft_law& law, uint32_t token, uint64_t* begin) {
     return law.cdf[i + 1] - law.cdf[i];
 }
 
+// a law as the gather sees it: compact receipt or full table (gemma3_draft.mm:1538-1556)
+struct LawView { const gfo_draft_law* compact; const uint64_t* full; uint32_t vocab; };
+uint64_t law_mass(const LawView& law, uint32_t token, uint64_t* begin) {
+    if (law.compact) return law_mass(*law.compact, token, begin);
+    if (token >= law.vocab) { if (begin) *begin = 0; return 0; }
+    if (begin) *begin = law.full[token];
+    return law.full[token + 1] - law.full[token];
+}
+
 struct Scored { uint32_t token; float score; };
 inline bool better_scored(const Scored& a, const Scored& b) {
     return a.score > b.score || (a.score == b.score && a.token < b.token);
@@ -262,10 +271,21 @@ int gfo_draft_law_compact(const float* logits, uint32_t vocab, const gfo_sampler
 
 int gfo_draft_law_full(const float* logits, uint32_t vocab, const gfo_sampler_options* opt,
                        uint64_t* cdf) {
-    // Unfiltered full-vocabulary law (top_k = 0 equivalent is not expressible in the
-    // sampler options, so this path is entered only on compact-support overflow):
+    // Full-vocabulary law (gemma3_draft.mm:295-395 in the dispatch order of :1040-1166), entered
+    // when top_k > 64, when drafting greedily, or when the compact support overflows:
     // tiles of 256 tokens, f32 prefix inside a tile, f32 running offsets across tiles.
-    if (!options_valid(*opt) || opt->temperature <= 0.0f || vocab % 256 != 0) return -1;
+    if (!options_valid(*opt) || opt->temperature < 0.0f || vocab == 0 || vocab % 256 != 0) return -1;
+    if (opt->temperature == 0.0f) {
+        // greedy drafting: no transform, no filter; all mass on the lowest-id maximum
+        // (gd_max / gd_max_finish, then gd_cdf's step function, gemma3_draft.mm:338-379)
+        uint32_t best = 0;
+        for (uint32_t i = 0; i < vocab; ++i) {
+            if (!std::isfinite(logits[i])) return -10;
+            if (logits[i] > logits[best]) best = i;
+        }
+        for (uint32_t i = 0; i <= vocab; ++i) cdf[i] = i <= best ? 0 : kMassTotal;
+        return 0;
+    }
     std::vector<float> score(vocab);
     for (uint32_t i = 0; i < vocab; ++i) {
         if (!std::isfinite(logits[i])) return -10;
@@ -349,9 +369,11 @@ uint32_t gfo_draft_select_full(const uint64_t* cdf, uint32_t vocab, uint32_t wor
     return 0xFFFFFFFFu;
 }
 
-int gfo_spec_from_prepared(const gfo_prepared* target_in, const gfo_draft_law* law,
-                           uint32_t proposal, double u_accept, double u_residual,
-                           gfo_spec_result* out) {
+namespace {
+int spec_from_prepared(const gfo_prepared* target_in, const LawView& view,
+                       uint32_t proposal, double u_accept, double u_residual,
+                       gfo_spec_result* out) {
+    const LawView* law = &view;
     const gfo_prepared& target = *target_in;
     std::memset(out, 0, sizeof(*out));
     auto unit = [](double u) { return std::isfinite(u) && u >= 0.0 && u < 1.0; };
@@ -410,16 +432,15 @@ int gfo_spec_from_prepared(const gfo_prepared* target_in, const gfo_draft_law* l
     return 0;
 }
 
-int gfo_spec_accept(const gfo_token_logit* row0, uint32_t n0, const gfo_token_logit* row1,
-                    uint32_t n1, const gfo_draft_law* law, uint32_t proposal,
-                    const gfo_sampler_options* opt, double u_accept, double u_residual,
-                    double u_next, gfo_spec_result* out) {
+int spec_accept(const gfo_token_logit* row0, uint32_t n0, const gfo_token_logit* row1, uint32_t n1,
+                const LawView& law, uint32_t proposal, const gfo_sampler_options* opt, double u_accept,
+                double u_residual, double u_next, gfo_spec_result* out) {
     std::memset(out, 0, sizeof(*out));
     if (!(std::isfinite(u_next) && u_next >= 0.0 && u_next < 1.0)) return -20;
     gfo_prepared target;
     int rc = gfo_prepare_token_distribution(row0, n0, opt, nullptr, 0, &target);
     if (rc) return rc;
-    rc = gfo_spec_from_prepared(&target, law, proposal, u_accept, u_residual, out);
+    rc = spec_from_prepared(&target, law, proposal, u_accept, u_residual, out);
     if (rc || !out->accepted) return rc;
     // a fully accepted chain leaves row 1's candidates to seed the next root
     gfo_prepared next;
@@ -428,6 +449,26 @@ int gfo_spec_accept(const gfo_token_logit* row0, uint32_t n0, const gfo_token_lo
     out->next_root = opt->temperature == 0.0f
         ? next.token[0] : select_prepared(next, u_next * next.total_sampling_weight);
     return 0;
+}
+}  // namespace
+
+int gfo_spec_from_prepared(const gfo_prepared* target, const gfo_draft_law* law, uint32_t proposal,
+                           double u_accept, double u_residual, gfo_spec_result* out) {
+    return spec_from_prepared(target, LawView{law, nullptr, 0}, proposal, u_accept, u_residual, out);
+}
+
+int gfo_spec_accept(const gfo_token_logit* row0, uint32_t n0, const gfo_token_logit* row1,
+                    uint32_t n1, const gfo_draft_law* law, uint32_t proposal,
+                    const gfo_sampler_options* opt, double u_accept, double u_residual,
+                    double u_next, gfo_spec_result* out) {
+    return spec_accept(row0, n0, row1, n1, LawView{law, nullptr, 0}, proposal, opt, u_accept, u_residual, u_next, out);
+}
+
+int gfo_spec_accept_full(const gfo_token_logit* row0, uint32_t n0, const gfo_token_logit* row1,
+                         uint32_t n1, const uint64_t* cdf, uint32_t vocab, uint32_t proposal,
+                         const gfo_sampler_options* opt, double u_accept, double u_residual,
+                         double u_next, gfo_spec_result* out) {
+    return spec_accept(row0, n0, row1, n1, LawView{nullptr, cdf, vocab}, proposal, opt, u_accept, u_residual, u_next, out);
 }
 
 void gfo_philox4x32_10(const uint32_t counter[4], const uint32_t key[2], uint32_t out[4]) {

@@ -129,6 +129,50 @@ def test_h1_cycle_small_models(hip, gfo):
     run_h1(hip, gfo, t_shape, d_shape, 1300, 1300, steps=12, seed=5)
 
 
+def test_h1_cycle_with_the_full_vocabulary_law(hip, gfo):
+    """A step whose sampler options rule out the compact law (top_k > 64, then greedy drafting):
+    proposal and decision equal the oracle's on the step's own logits, q gathered from the table."""
+    import torch
+    from dataclasses import replace
+    from guffin_amd import model
+    t_shape = replace(model.GEMMA3_12B, layers=2, vocab=8192, ring_global=2048)
+    d_shape = replace(model.GEMMA3_270M, layers=2, vocab=8192, ring_global=2048)
+    target = model.DeviceModel.from_host(model.HostModel(t_shape, seed=31, position=900))
+    drafter = model.DeviceModel.from_host(model.HostModel(d_shape, seed=32, position=900))
+    for temperature, top_k in ((1.0, 128), (0.0, 1)):
+        plan = model.H1Plan(target, drafter, 900, 900, temperature=temperature, top_k=top_k, seed=4, publish=False,
+                            full_law=True)
+        opt_cpu = gfo.SamplerOptions(temperature, top_k, 0.95, 0.0, 1.0)
+        plan.root.fill_(55)
+        for step in range(6):
+            plan.step(step)
+            torch.cuda.synchronize()
+            bufs, res = plan.buffers(), plan.read_result()
+            assert int(plan.status.item()) == 0
+            rc, cdf = gfo.draft_law_full(bufs["q_logits"].cpu().numpy(), opt_cpu)
+            assert rc == 0
+            assert np.array_equal(bufs["full_cdf"].cpu().numpy().view(np.uint64), cdf)
+            word, ua, ur, un = gfo.step_draws(4, step)
+            proposal = gfo.draft_select_full(cdf, word)
+            p_logits = bufs["p_logits"].cpu().numpy()
+            rows = [gfo.select_candidates(p_logits[r], top_k) for r in range(2)]
+            rc, want = gfo.spec_accept_full(rows[0], rows[1], cdf, proposal, opt_cpu, ua, ur, un)
+            assert res["proposal"] == proposal
+            if rc != 0:
+                assert res["status"] == -rc
+                continue
+            assert res["status"] == 0
+            assert (res["accepted"], res["token"], res["next_root"]) == (want.accepted, want.token, want.next_root)
+    # the compact options with the fallback encoded take the same decisions as without it
+    a = model.H1Plan(target, drafter, 900, 900, seed=4, publish=False, full_law=True)
+    b = model.H1Plan(target, drafter, 900, 900, seed=4, publish=False)
+    for plan in (a, b):
+        plan.root.fill_(55)
+        plan.step(3)
+    torch.cuda.synchronize()
+    assert a.read_result().tobytes() == b.read_result().tobytes()
+
+
 def test_h1_commit_publishes_verified_rows(hip, gfo):
     import torch
     from dataclasses import replace

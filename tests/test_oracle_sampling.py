@@ -300,3 +300,51 @@ def test_full_law_uniform_and_nucleus(gfo):
     assert rc == 0
     d = np.diff(cdf.astype(np.int64))
     assert d[0] == 32768 and d[1] == 32768 and d[-1] == 0 and d[-2] == 0 and d.sum() == TOTAL
+
+
+def test_full_law_reference_cases(gfo):
+    """tests/engine/gemma3_draft_tests.cpp:304-307, 392-403 of the reference, on the oracle's table."""
+    vocab = 262144
+    logits = np.zeros(vocab, np.float32)
+    tiny = np.float32(1.401298464324817e-45)  # denorm_min: nothing but the best entry survives
+    rc, cdf = gfo.draft_law_full(logits, opts(gfo, t=1.0, k=1, p=float(tiny)))
+    assert rc == 0 and int(cdf[0]) == 0 and int(cdf[1]) == TOTAL
+    assert gfo.draft_select_full(cdf, 0) == 0 and gfo.draft_select_full(cdf, 0xFFFFFFFF) == 0
+    for count in (256, 257, 64):
+        logits = np.full(vocab, -100, np.float32)
+        logits[:count] = 0
+        rc, cdf = gfo.draft_law_full(logits, opts(gfo, t=1.0, k=1, p=1.0))
+        assert rc == 0
+        assert gfo.draft_select_full(cdf, 0xFFFFFFFF) == count - 1
+        assert int(cdf[count + 1]) - int(cdf[count]) == 0
+        assert abs((int(cdf[count]) - int(cdf[count - 1])) / TOTAL - 1.0 / count) < 1e-6
+
+
+def test_full_law_greedy_is_a_step_at_the_lowest_argmax(gfo):
+    rng = np.random.default_rng(5)
+    logits = rng.normal(0, 2, 1024).astype(np.float32)
+    logits[[300, 17, 900]] = 9.5
+    rc, cdf = gfo.draft_law_full(logits, opts(gfo, t=0.0, k=1, p=1.0))
+    assert rc == 0
+    assert np.all(cdf[:18] == 0) and np.all(cdf[18:] == TOTAL)
+    for word in (0, 12345, 0xFFFFFFFF):
+        assert gfo.draft_select_full(cdf, word) == 17
+
+
+def test_full_law_agrees_with_the_compact_law(gfo):
+    """Two independently written paths of the same law: the same support, masses within 1e-6
+    (the f32 sums associate differently, so the tables need not be bit-equal)."""
+    rng = np.random.default_rng(6)
+    for k, p, m in ((64, 0.9, 0.0), (8, 1.0, 0.05), (40, 0.87, 0.05), (1, 1.0, 0.0)):
+        logits = rng.normal(0, 2, 4096).astype(np.float32)
+        o = opts(gfo, t=0.8, k=k, p=p, m=m)
+        rc, law = gfo.draft_law_compact(logits, o)
+        assert rc == 0
+        rc, cdf = gfo.draft_law_full(logits, o)
+        assert rc == 0
+        mass = np.diff(cdf.astype(np.int64))
+        support = np.nonzero(mass)[0]
+        ids = np.array(law.ids[:law.count])
+        cm = np.diff(np.array(law.cdf[:law.count + 1], dtype=np.int64))
+        assert list(support) == list(ids[cm > 0])
+        assert np.max(np.abs(mass[ids] - cm)) / TOTAL < 1e-6
