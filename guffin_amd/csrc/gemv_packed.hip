@@ -513,7 +513,8 @@ int g_cus = 256;
 // at most max_w) and planes (k-slices left to the consumer), preferring one workgroup per CU.
 struct Split { uint32_t bps, W, planes; };
 Split choose_split(uint32_t nblk, uint32_t tiles, uint32_t max_w) {
-    const uint64_t units = uint64_t(tiles) * nblk, target_waves = uint64_t(g_cus) * 16;
+    // a kernel capped at 8 waves per workgroup is register-bound: a CU holds 8 of its waves, not 16
+    const uint64_t units = uint64_t(tiles) * nblk, target_waves = uint64_t(g_cus) * (max_w < 16 ? 8 : 16);
     uint32_t bps = static_cast<uint32_t>((units + target_waves - 1) / target_waves);
     if (bps < 1) bps = 1;
     const uint32_t wpt = (nblk + bps - 1) / bps;  // waves per tile
