@@ -512,9 +512,10 @@ int g_cus = 256;
 // that the chip holds about four waves per SIMD, waves per workgroup (k-slices reduced in LDS,
 // at most max_w) and planes (k-slices left to the consumer), preferring one workgroup per CU.
 struct Split { uint32_t bps, W, planes; };
-Split choose_split(uint32_t nblk, uint32_t tiles, uint32_t max_w) {
+Split choose_split(uint32_t nblk, uint32_t tiles, uint32_t max_w, uint32_t waves_per_cu = 0) {
     // a kernel capped at 8 waves per workgroup is register-bound: a CU holds 8 of its waves, not 16
-    const uint64_t units = uint64_t(tiles) * nblk, target_waves = uint64_t(g_cus) * (max_w < 16 ? 8 : 16);
+    if (waves_per_cu == 0) waves_per_cu = max_w < 16 ? 8 : 16;
+    const uint64_t units = uint64_t(tiles) * nblk, target_waves = uint64_t(g_cus) * waves_per_cu;
     uint32_t bps = static_cast<uint32_t>((units + target_waves - 1) / target_waves);
     if (bps < 1) bps = 1;
     const uint32_t wpt = (nblk + bps - 1) / bps;  // waves per tile
@@ -680,7 +681,7 @@ extern "C" int guffin_hip_gateup_geglu(void* stream, int dtype, const void* gate
         return fail(GUFFIN_E_ALIGN, "gateup_geglu: tiles must be 16-byte aligned");
     if (reinterpret_cast<uintptr_t>(h_sums) & 255u) return fail(GUFFIN_E_ALIGN, "gateup_geglu: the receipt must be 256-byte aligned");
     const uint32_t nblk = K / block_elems(dtype), tiles = F / kTileCols;
-    Split sp = choose_split(nblk, 2 * tiles, 8);
+    Split sp = choose_split(nblk, 2 * tiles, 8, 16);  // two matrices of up to 8 waves each in a workgroup
     if (sp.planes > 1) {  // all k-slices of a tile must sit in one workgroup: at most 8 per matrix
         sp.bps = (nblk + 7) / 8;
         sp.W = (nblk + sp.bps - 1) / sp.bps;

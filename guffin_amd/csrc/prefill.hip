@@ -170,7 +170,7 @@ __device__ __forceinline__ void add_offset(const float* sums, const WaveCtx& c, 
 
 // grid (N/64, Mpad/128), 256 threads.  y[M][N] fp32.
 template <int DTYPE>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(256, DTYPE == GUFFIN_Q6_K ? 1 : 2)
 prefill_gemm_kernel(const uint8_t* __restrict__ tiles, const uint8_t* __restrict__ blob, float* __restrict__ y,
                     uint32_t M, uint32_t K, uint32_t N) {
     constexpr uint32_t TB = kCols * block_bytes(DTYPE);
@@ -254,47 +254,76 @@ prefill_gemm_kernel(const uint8_t* __restrict__ tiles, const uint8_t* __restrict
                     acc[cg][rg][1] = fmaf(d[cg] * blk.mult[rg].y, D[cg][rg][2] + D[cg][rg][3], acc[cg][rg][1]);
                 }
         } else if constexpr (DTYPE == GUFFIN_Q6_K) {
-            uint4 ql[8], qh[4];
+            // q = lo + 16 hi2 (4 + 2 bits): |scale| * lo <= 1905 and |scale| * hi2 <= 381 are exact as
+            // fp16 bit patterns (n < 2048 reads as n * 2^-24) and carry the scale's sign in bit 15, so
+            // both parts accumulate over the whole block inside the MFMA chain.  A scale covers 16
+            // elements: lanes of k-slices 0-1 take the group's first scale, 2-3 the second.
+            const bool second = lane >= 32;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) ql[i] = *reinterpret_cast<const uint4*>(tp + 1024 * i + lane * 16);
+            for (int half = 0; half < 2; ++half) {  // two column groups at a time keep the wave within 256 registers
+                uint4 ql[4], qh[2];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) qh[i] = *reinterpret_cast<const uint4*>(tp + 8192 + 1024 * i + lane * 16);
-            // a scale covers 16 elements: the two halves of a 32-group go through separate MFMAs with
-            // the other half's lanes (k-slices) zeroed
-            const uint32_t keep_first = lane < 32 ? 0xFFFFFFFFu : 0u;
+                for (int i = 0; i < 4; ++i) ql[i] = *reinterpret_cast<const uint4*>(tp + 1024 * (4 * half + i) + lane * 16);
 #pragma unroll
-            for (int g = 0; g < 8; ++g) {
-                const int n = g >> 2, qd = g & 3;
-                GroupOperands o;
-                load_group(c, b * 8 + g, o);
+                for (int i = 0; i < 2; ++i) qh[i] = *reinterpret_cast<const uint4*>(tp + 8192 + 1024 * (2 * half + i) + lane * 16);
+                float4_t Dl[2][4], Dh[2][4];
+                uint4 scv[2];
+                float d[2];
 #pragma unroll
-                for (int cg = 0; cg < 4; ++cg) {
-                    const uint4 scv = *reinterpret_cast<const uint4*>(tp + 12288 + (16 * cg + j) * 16);
-                    const float d = h2f(*reinterpret_cast<const uint16_t*>(tp + 13312 + (16 * cg + j) * 2));
-                    const int word = g >> 1;
-                    const uint32_t sw = word == 0 ? scv.x : word == 1 ? scv.y : word == 2 ? scv.z : scv.w;
-                    const float s_first = sbyte(sw, 2 * (g & 1)), s_second = sbyte(sw, 2 * (g & 1) + 1);
-                    const uint4 lq = ql[2 * cg + n], hq = qh[cg];
-                    const uint32_t w0 = (qd & 1) ? lq.z : lq.x, w1 = (qd & 1) ? lq.w : lq.y;
-                    const uint32_t h0 = n ? hq.z : hq.x, h1 = n ? hq.w : hq.y;
-                    const int ls = qd >= 2 ? 4 : 0;
-                    uint32_t bq[4];
+                for (int cc = 0; cc < 2; ++cc) {
+                    const int cg = 2 * half + cc;
+                    scv[cc] = *reinterpret_cast<const uint4*>(tp + 12288 + (16 * cg + j) * 16);
+                    d[cc] = h2f(*reinterpret_cast<const uint16_t*>(tp + 13312 + (16 * cg + j) * 2));
 #pragma unroll
-                    for (int k = 0; k < 2; ++k) {
-                        const uint32_t w = k ? w1 : w0, h = k ? h1 : h0;
-                        const uint32_t lo0 = (w >> ls) & 0x000F000Fu, lo1 = (w >> (ls + 8)) & 0x000F000Fu;
-                        const uint32_t hs0 = qd == 0 ? h << 4 : qd == 1 ? h << 2 : qd == 2 ? h : h >> 2;
-                        const uint32_t hs1 = h >> (4 + 2 * qd);
-                        bq[2 * k] = (hs0 & 0x00300030u) | lo0;
-                        bq[2 * k + 1] = (hs1 & 0x00300030u) | lo1;
-                    }
-                    mfma_scale(o, as_half8(bq[0] & keep_first, bq[1] & keep_first, bq[2] & keep_first, bq[3] & keep_first),
-                               d * s_first, acc[cg]);
-                    mfma_scale(o, as_half8(bq[0] & ~keep_first, bq[1] & ~keep_first, bq[2] & ~keep_first, bq[3] & ~keep_first),
-                               d * s_second, acc[cg]);
-                    add_offset(c.s16, c, (b * 8 + g) * 2, -32.0f * d * s_first, acc[cg]);
-                    add_offset(c.s16, c, (b * 8 + g) * 2 + 1, -32.0f * d * s_second, acc[cg]);
+                    for (int rg = 0; rg < 4; ++rg) { Dl[cc][rg] = float4_t{0.f, 0.f, 0.f, 0.f}; Dh[cc][rg] = Dl[cc][rg]; }
                 }
+#pragma unroll
+                for (int g = 0; g < 8; ++g) {
+                    const int n = g >> 2, qd = g & 3;
+                    GroupOperands o;
+                    load_group(c, b * 8 + g, o);
+#pragma unroll
+                    for (int cc = 0; cc < 2; ++cc) {
+                        const int cg = 2 * half + cc, word = g >> 1;
+                        const uint32_t sw = word == 0 ? scv[cc].x : word == 1 ? scv[cc].y : word == 2 ? scv[cc].z : scv[cc].w;
+                        const float s_first = sbyte(sw, 2 * (g & 1)), s_second = sbyte(sw, 2 * (g & 1) + 1);
+                        const int sc = static_cast<int>(second ? s_second : s_first);
+                        const uint32_t mag = static_cast<uint32_t>(sc < 0 ? -sc : sc);
+                        const uint32_t pair = mag | (mag << 16), sign = sc < 0 ? 0x80008000u : 0u;
+                        const uint4 lq = ql[2 * cc + n], hq = qh[cc];
+                        const uint32_t w0 = (qd & 1) ? lq.z : lq.x, w1 = (qd & 1) ? lq.w : lq.y;
+                        const uint32_t h0 = n ? hq.z : hq.x, h1 = n ? hq.w : hq.y;
+                        const int ls = qd >= 2 ? 4 : 0;
+                        uint32_t bl[4], bh[4];
+#pragma unroll
+                        for (int k = 0; k < 2; ++k) {
+                            const uint32_t w = k ? w1 : w0, h = k ? h1 : h0;
+                            bl[2 * k] = pk_mul((w >> ls) & 0x000F000Fu, pair) | sign;
+                            bl[2 * k + 1] = pk_mul((w >> (ls + 8)) & 0x000F000Fu, pair) | sign;
+                            bh[2 * k] = pk_mul((h >> (2 * qd)) & 0x00030003u, pair) | sign;
+                            bh[2 * k + 1] = pk_mul((h >> (8 + 2 * qd)) & 0x00030003u, pair) | sign;
+                        }
+                        const half8_t blo = as_half8(bl[0], bl[1], bl[2], bl[3]), bhi = as_half8(bh[0], bh[1], bh[2], bh[3]);
+#pragma unroll
+                        for (int rg = 0; rg < 4; ++rg) {
+                            Dl[cc][rg] = __builtin_amdgcn_mfma_f32_16x16x32_f16(o.a[rg], blo, Dl[cc][rg], 0, 0, 0);
+                            Dh[cc][rg] = __builtin_amdgcn_mfma_f32_16x16x32_f16(o.a[rg], bhi, Dh[cc][rg], 0, 0, 0);
+                        }
+                        add_offset(c.s16, c, (b * 8 + g) * 2, -32.0f * d[cc] * s_first, acc[cg]);
+                        add_offset(c.s16, c, (b * 8 + g) * 2 + 1, -32.0f * d[cc] * s_second, acc[cg]);
+                    }
+                }
+                GroupOperands blk;
+                load_group(c, b * 8, blk);  // the block's multipliers (shared by its 8 groups)
+#pragma unroll
+                for (int cc = 0; cc < 2; ++cc)
+#pragma unroll
+                    for (int rg = 0; rg < 4; ++rg) {
+                        const int cg = 2 * half + cc;
+                        const float4_t lo4 = Dl[cc][rg], hi4 = Dh[cc][rg];
+                        acc[cg][rg][0] = fmaf(d[cc] * blk.mult[rg].x, (lo4[0] + lo4[1]) + 16.0f * (hi4[0] + hi4[1]), acc[cg][rg][0]);
+                        acc[cg][rg][1] = fmaf(d[cc] * blk.mult[rg].y, (lo4[2] + lo4[3]) + 16.0f * (hi4[2] + hi4[3]), acc[cg][rg][1]);
+                    }
             }
         } else {
             const uint4 q0 = *reinterpret_cast<const uint4*>(tp + lane * 16);
