@@ -41,7 +41,51 @@ struct AttnArgs {
     float* part_ml;              // [rows][q_heads][partitions][2]
     uint32_t rows, q_heads, kv_heads, hd, ring_mask, tp, partitions, private_rows;
     float scale;
+    // fused mode: q, k, v arrive as the projections' partial planes; every workgroup prepares
+    // the query heads it serves (head norm, rotation) and the partition that holds a private
+    // row prepares that row's key and value and publishes them as fp16
+    const float* q_raw; const float* k_raw; const float* v_raw;
+    uint32_t planes; size_t q_stride, k_stride, v_stride;
+    const float* q_norm; const float* k_norm; const float2* rope;   // rope: [rows][hd/2] (cos, sin)
+    uint16_t* priv_k_out; uint16_t* priv_v_out;
+    float eps; uint32_t* status;
 };
+
+// One head row (hd = 256) by one wave, in registers: lane l holds columns l, l+64, l+128, l+192.
+// load: sum of the partial planes plus gamma and the rotation pairs, all requested together;
+// finish: optional RMS norm with gamma and rotation of the pairs (i, i + 128) — the arithmetic of
+// qkv_post_kernel.  Several rows may be loaded before any is finished (one memory round trip).
+struct HeadRow { float v[4]; float gm[4]; float2 rp[2]; };
+
+__device__ __forceinline__ void load_head_row(HeadRow& h, const float* src, uint32_t planes, size_t stride,
+                                              const float* gamma, const float2* rope_row, uint32_t lane) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) h.gm[i] = gamma ? gamma[lane + 64 * i] : 1.f;
+    h.rp[0] = rope_row ? rope_row[lane] : make_float2(1.f, 0.f);
+    h.rp[1] = rope_row ? rope_row[lane + 64] : make_float2(1.f, 0.f);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) h.v[i] = load_planes(src + lane + 64 * i, planes, stride);
+}
+
+__device__ __forceinline__ void finish_head_row(HeadRow& h, bool norm, bool rotate, float eps) {
+    if (norm) {
+        float ss = 0.f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) ss = fmaf(h.v[i], h.v[i], ss);
+        ss = wave_sum(ss);
+        const float inv = 1.0f / sqrtf(ss / 256.0f + eps);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) h.v[i] = h.v[i] * inv * h.gm[i];
+    }
+    if (rotate) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const float first = h.v[i], second = h.v[i + 2];
+            h.v[i] = __fsub_rn(__fmul_rn(first, h.rp[i].x), __fmul_rn(second, h.rp[i].y));
+            h.v[i + 2] = __fadd_rn(__fmul_rn(first, h.rp[i].y), __fmul_rn(second, h.rp[i].x));
+        }
+    }
+}
 
 __device__ __forceinline__ float dot2(float acc, uint32_t packed_half2, float a, float b) {
     const half2_t h = __builtin_bit_cast(half2_t, packed_half2);
@@ -49,19 +93,37 @@ __device__ __forceinline__ float dot2(float acc, uint32_t packed_half2, float a,
     return fmaf(static_cast<float>(h.y), b, acc);
 }
 
-template <int ROWS, int GROUP, int HD>
+template <int ROWS, int GROUP, int HD, bool FUSED>
 __global__ void __launch_bounds__(256) attn_partial_kernel(AttnArgs a) {
     static_assert(HD == 256, "head dimension 256 (16 lanes x 16 dims)");
     constexpr int NQ = ROWS * GROUP;
     extern __shared__ float lds[];
     float* sc = lds;                          // [NQ][tp] scores, then probabilities
     float* merge = lds + NQ * a.tp;           // [4][NQ][HD]
+    float* q_s = merge + 4 * NQ * HD;         // fused: [NQ][HD] prepared queries
     __shared__ float s_max[NQ], s_sum[NQ];
+    __shared__ __attribute__((aligned(16))) uint16_t k_s[FUSED ? ROWS : 1][HD], v_s[FUSED ? ROWS : 1][HD];
 
     const uint32_t part = blockIdx.x, kvh = blockIdx.y;
     const uint32_t lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
     constexpr uint32_t group = GROUP;
     const uint32_t row_stride = a.kv_heads * HD;  // in halves
+
+    // fused: the query rows of this wave (w, w+4, ..) are requested first; their addresses need
+    // nothing but the launch arguments, so they travel together with the schedule below
+    constexpr int QI = (NQ + 3) / 4;
+    HeadRow qr[FUSED ? QI : 1];
+    if constexpr (FUSED) {
+#pragma unroll
+        for (int i = 0; i < QI; ++i) {
+            const uint32_t item = wv + 4 * i;
+            if (item < NQ) {
+                const uint32_t r = item / group, head = kvh * group + item % group;
+                load_head_row(qr[i], a.q_raw + (size_t(r) * a.q_heads + head) * HD, a.planes, a.q_stride, a.q_norm,
+                              a.rope + size_t(r) * (HD / 2), lane);
+            }
+        }
+    }
 
     // merged virtual token list
     uint32_t u_first = 0xFFFFFFFFu, u_end = 0;
@@ -80,40 +142,107 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(AttnArgs a) {
     const uint32_t n_ring = u_end - u_first, n_total = n_ring + a.private_rows;
     const uint32_t t0 = part * a.tp, t1 = min(t0 + a.tp, n_total);
 
+    // ---- keys: four rounds of loads are issued before their dot products so that a wave keeps
+    // 16 key rows (8 KB) in flight; in fused mode the first batch travels during the preparation
+    constexpr int U = 4;
+    const uint32_t slot = lane >> 4, seg = lane & 15;  // token slot in the wave, 16-dim segment
+    const uint32_t tb_first = t0 + wv * 4 + slot;
+    uint4 k0[U], k1[U];
+    auto load_keys = [&](uint32_t tb) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const uint32_t t = tb + 16 * u;
+            k0[u] = make_uint4(0, 0, 0, 0); k1[u] = k0[u];
+            if (t < t1) {
+                const bool is_priv = t >= n_ring;
+                if (FUSED && is_priv) continue;  // taken from LDS once prepared
+                const uint16_t* kp = is_priv ? a.priv_k + size_t(t - n_ring) * row_stride
+                                             : a.ring_k + size_t((u_first + t) & a.ring_mask) * row_stride;
+                kp += kvh * HD + seg * 16;
+                k0[u] = *reinterpret_cast<const uint4*>(kp); k1[u] = *reinterpret_cast<const uint4*>(kp + 8);
+            }
+        }
+    };
+    if constexpr (FUSED) load_keys(tb_first);
+    // ---- values: a half wave covers one value row (32 lanes x 8 dims, 16-byte loads), a wave two
+    // tokens per round, four rounds in flight; in fused mode the first batch is requested while
+    // the softmax runs
+    const uint32_t hsel = lane >> 5, dl = (lane & 31) * 8;
+    const uint32_t vb_first = t0 + wv * 2 + hsel;
+    uint4 vv[U];
+    auto load_values = [&](uint32_t tb) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const uint32_t t = tb + 8 * u;
+            vv[u] = make_uint4(0, 0, 0, 0);
+            if (t < t1) {
+                const bool is_priv = t >= n_ring;
+                if (FUSED && is_priv) continue;  // taken from LDS once prepared
+                const uint16_t* vp = is_priv ? a.priv_v + size_t(t - n_ring) * row_stride
+                                             : a.ring_v + size_t((u_first + t) & a.ring_mask) * row_stride;
+                vv[u] = *reinterpret_cast<const uint4*>(vp + kvh * HD + dl);
+            }
+        }
+    };
+
+    if constexpr (FUSED) {
+        // wave w prepares query rows w, w+4, .. and one of the private rows' key / value (row w/2,
+        // key for even w) when this partition holds it; every load is issued before any arithmetic
+        HeadRow kvr;
+        const uint32_t pr = wv >> 1, pt = n_ring + pr;
+        const bool is_key = (wv & 1u) == 0;
+        const bool mine = pr < ROWS && pr < a.private_rows && pt >= t0 && pt < t1;
+        const size_t kv_off = (size_t(pr) * a.kv_heads + kvh) * HD;
+        if (mine)
+            load_head_row(kvr, (is_key ? a.k_raw : a.v_raw) + kv_off, a.planes, is_key ? a.k_stride : a.v_stride,
+                          is_key ? a.k_norm : nullptr, is_key ? a.rope + size_t(pr) * (HD / 2) : nullptr, lane);
+#pragma unroll
+        for (int i = 0; i < QI; ++i) {
+            const uint32_t item = wv + 4 * i;
+            if (item < NQ) {
+                finish_head_row(qr[i], a.q_norm != nullptr, true, a.eps);
+#pragma unroll
+                for (int c = 0; c < 4; ++c) q_s[item * HD + lane + 64 * c] = qr[i].v[c];
+            }
+        }
+        if (mine) {
+            finish_head_row(kvr, is_key && a.k_norm != nullptr, is_key, a.eps);
+            bool bad = false;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const _Float16 hv = static_cast<_Float16>(kvr.v[c]);  // round-to-nearest-even, after rotation
+                bad |= !isfinite(static_cast<float>(hv));
+                const uint16_t bits = __builtin_bit_cast(uint16_t, hv);
+                (is_key ? k_s : v_s)[pr][lane + 64 * c] = bits;
+                (is_key ? a.priv_k_out : a.priv_v_out)[kv_off + lane + 64 * c] = bits;
+            }
+            if (bad && a.status) atomicOr(a.status, GUFFIN_STATUS_KV_NONFINITE);
+        }
+        __syncthreads();
+    }
     // ---- pass 1: scores ------------------------------------------------------------
     {
-        const uint32_t slot = lane >> 4, seg = lane & 15;  // token slot in the wave, 16-dim segment
         float qv[NQ][16];
 #pragma unroll
         for (int n = 0; n < NQ; ++n) {
             const uint32_t r = n / group, g = n % group;
-            const float* qp = a.q + (size_t(r) * a.q_heads + kvh * group + g) * HD + seg * 16;
+            const float* qp = FUSED ? q_s + n * HD + seg * 16
+                                    : a.q + (size_t(r) * a.q_heads + kvh * group + g) * HD + seg * 16;
 #pragma unroll
             for (int i = 0; i < 16; ++i) qv[n][i] = qp[i] * a.scale;
         }
-        // four rounds of loads are issued before their dot products so that a wave keeps
-        // 16 key rows (8 KB) in flight
-        constexpr int U = 4;
-        for (uint32_t tb = t0 + wv * 4 + slot; tb < t0 + a.tp; tb += 16 * U) {
-            uint4 k0[U], k1[U];
-#pragma unroll
-            for (int u = 0; u < U; ++u) {
-                const uint32_t t = tb + 16 * u;
-                k0[u] = make_uint4(0, 0, 0, 0); k1[u] = k0[u];
-                if (t < t1) {
-                    const bool is_priv = t >= n_ring;
-                    const uint16_t* kp = is_priv ? a.priv_k + size_t(t - n_ring) * row_stride
-                                                 : a.ring_k + size_t((u_first + t) & a.ring_mask) * row_stride;
-                    kp += kvh * HD + seg * 16;
-                    k0[u] = *reinterpret_cast<const uint4*>(kp); k1[u] = *reinterpret_cast<const uint4*>(kp + 8);
-                }
-            }
+        for (uint32_t tb = tb_first; tb < t0 + a.tp; tb += 16 * U) {
+            if (!FUSED || tb != tb_first) load_keys(tb);
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 const uint32_t t = tb + 16 * u;
                 if (t >= t0 + a.tp) break;
                 const bool in_range = t < t1, is_priv = t >= n_ring;
                 const uint32_t pos = u_first + t, prow = t - n_ring;
+                if (FUSED && in_range && is_priv) {
+                    const uint16_t* kp = &k_s[prow][seg * 16];
+                    k0[u] = *reinterpret_cast<const uint4*>(kp); k1[u] = *reinterpret_cast<const uint4*>(kp + 8);
+                }
                 const uint32_t kw[8] = {k0[u].x, k0[u].y, k0[u].z, k0[u].w, k1[u].x, k1[u].y, k1[u].z, k1[u].w};
                 float s[NQ];
 #pragma unroll
@@ -138,6 +267,7 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(AttnArgs a) {
             }
         }
     }
+    if constexpr (FUSED) load_values(vb_first);  // in flight during the softmax
     __syncthreads();
 
     // ---- softmax over the partition, one wave per query ----------------------------------
@@ -156,35 +286,20 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(AttnArgs a) {
         if (lane == 0) { s_max[n] = m; s_sum[n] = l; }
     }
     __syncthreads();
-
-    // ---- pass 2: values -------------------------------------------------------------------
-    // A half wave covers one value row (32 lanes x 8 dims, 16-byte loads), a wave two tokens
-    // per round, four rounds in flight; halves are combined by a lane exchange, waves via LDS.
+    // ---- pass 2: values; halves are combined by a lane exchange, waves via LDS ------------
     {
-        constexpr int U = 4;
-        const uint32_t hsel = lane >> 5, dl = (lane & 31) * 8;
         float acc[NQ][8];
 #pragma unroll
         for (int n = 0; n < NQ; ++n)
 #pragma unroll
             for (int i = 0; i < 8; ++i) acc[n][i] = 0.f;
-        for (uint32_t tb = t0 + wv * 2 + hsel; tb < t1; tb += 8 * U) {
-            uint4 vv[U];
-#pragma unroll
-            for (int u = 0; u < U; ++u) {
-                const uint32_t t = tb + 8 * u;
-                vv[u] = make_uint4(0, 0, 0, 0);
-                if (t < t1) {
-                    const bool is_priv = t >= n_ring;
-                    const uint16_t* vp = is_priv ? a.priv_v + size_t(t - n_ring) * row_stride
-                                                 : a.ring_v + size_t((u_first + t) & a.ring_mask) * row_stride;
-                    vv[u] = *reinterpret_cast<const uint4*>(vp + kvh * HD + dl);
-                }
-            }
+        for (uint32_t tb = vb_first; tb < t1; tb += 8 * U) {
+            if (!FUSED || tb != vb_first) load_values(tb);
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 const uint32_t t = tb + 8 * u;
                 if (t >= t1) break;
+                if (FUSED && t >= n_ring) vv[u] = *reinterpret_cast<const uint4*>(&v_s[t - n_ring][dl]);
                 const uint32_t w4[4] = {vv[u].x, vv[u].y, vv[u].z, vv[u].w};
 #pragma unroll
                 for (int n = 0; n < NQ; ++n) {
@@ -284,8 +399,12 @@ attn_merge_kernel(const float* __restrict__ part_out, const float* __restrict__ 
 template <int ROWS, int GROUP>
 int launch_partial(hipStream_t s, const AttnArgs& a) {
     constexpr int NQ = ROWS * GROUP;
-    const size_t lds = (size_t(NQ) * a.tp + size_t(4) * NQ * 256) * sizeof(float);
-    hipLaunchKernelGGL((attn_partial_kernel<ROWS, GROUP, 256>), dim3(a.partitions, a.kv_heads), dim3(256), lds, s, a);
+    const bool fused = a.q_raw != nullptr;
+    const size_t lds = (size_t(NQ) * a.tp + size_t(4) * NQ * 256 + (fused ? size_t(NQ) * 256 : 0)) * sizeof(float);
+    if (fused)
+        hipLaunchKernelGGL((attn_partial_kernel<ROWS, GROUP, 256, true>), dim3(a.partitions, a.kv_heads), dim3(256), lds, s, a);
+    else
+        hipLaunchKernelGGL((attn_partial_kernel<ROWS, GROUP, 256, false>), dim3(a.partitions, a.kv_heads), dim3(256), lds, s, a);
     return check_launch("attention_partial");
 }
 
@@ -302,14 +421,19 @@ extern "C" uint32_t guffin_hip_attention_partitions(uint32_t max_tokens, uint32_
     return (max_tokens + tp - 1) / tp;
 }
 
-extern "C" int guffin_hip_attention_decode(void* stream, const float* q, const void* ring_k, const void* ring_v,
-                                           const void* priv_k, const void* priv_v, const uint32_t* schedule,
-                                           const uint32_t* ancestors, float* out, float* out_sums,
-                                           float* partial_out, float* partial_ml, uint32_t rows,
-                                           uint32_t private_rows, uint32_t max_tokens, uint32_t ring_mask,
-                                           uint32_t q_heads, uint32_t kv_heads, uint32_t head_dim, float scale,
-                                           uint32_t* status) {
-    if (!q || !ring_k || !ring_v || !priv_k || !priv_v || !schedule || !ancestors || !out || !partial_out || !partial_ml)
+namespace {
+struct FusedInputs {
+    const float* q_raw; const float* k_raw; const float* v_raw;
+    uint32_t planes; uint64_t q_stride, k_stride, v_stride;
+    const float* q_norm; const float* k_norm; const float* rope; float eps;
+};
+
+int attention_decode(void* stream, const float* q, const FusedInputs* fused, const void* ring_k, const void* ring_v,
+                     void* priv_k, void* priv_v, const uint32_t* schedule, const uint32_t* ancestors, float* out,
+                     float* out_sums, float* partial_out, float* partial_ml, uint32_t rows, uint32_t private_rows,
+                     uint32_t max_tokens, uint32_t ring_mask, uint32_t q_heads, uint32_t kv_heads, uint32_t head_dim,
+                     float scale, uint32_t* status) {
+    if ((!q && !fused) || !ring_k || !ring_v || !priv_k || !priv_v || !schedule || !ancestors || !out || !partial_out || !partial_ml)
         return fail(GUFFIN_E_ARG, "attention_decode: null pointer");
     if (rows == 0 || rows > kMaxRows || private_rows > 32) return fail(GUFFIN_E_SHAPE, "attention_decode: rows must be 1 or 2, private rows <= 32");
     if (head_dim != 256) return fail(GUFFIN_E_SHAPE, "attention_decode: head_dim must be 256");
@@ -332,6 +456,19 @@ extern "C" int guffin_hip_attention_decode(void* stream, const float* q, const v
     a.tp = (max_tokens + a.partitions - 1) / a.partitions;
     a.tp = (a.tp + 15u) & ~15u;  // whole rounds of 16 tokens per workgroup
     a.private_rows = private_rows; a.scale = scale;
+    if (fused) {
+        if (!fused->q_raw || !fused->k_raw || !fused->v_raw || !fused->rope)
+            return fail(GUFFIN_E_ARG, "qkv_attention: null pointer");
+        if (fused->planes == 0 || private_rows != rows)
+            return fail(GUFFIN_E_SHAPE, "qkv_attention: planes >= 1 and one private row per query row");
+        if (!(fused->eps > 0.f)) return fail(GUFFIN_E_ARG, "qkv_attention: epsilon must be positive");
+        if (reinterpret_cast<uintptr_t>(fused->rope) & 7u) return fail(GUFFIN_E_ALIGN, "qkv_attention: rope table must be 8-byte aligned");
+        a.q_raw = fused->q_raw; a.k_raw = fused->k_raw; a.v_raw = fused->v_raw; a.planes = fused->planes;
+        a.q_stride = fused->q_stride; a.k_stride = fused->k_stride; a.v_stride = fused->v_stride;
+        a.q_norm = fused->q_norm; a.k_norm = fused->k_norm; a.rope = reinterpret_cast<const float2*>(fused->rope);
+        a.priv_k_out = static_cast<uint16_t*>(priv_k); a.priv_v_out = static_cast<uint16_t*>(priv_v);
+        a.eps = fused->eps; a.status = status;
+    }
     hipStream_t s = as_stream(stream);
     int rc;
     switch (group * 10 + rows) {
@@ -347,4 +484,34 @@ extern "C" int guffin_hip_attention_decode(void* stream, const float* q, const v
     hipLaunchKernelGGL(attn_merge_kernel, dim3(rows * q_heads), dim3(256), a.partitions * sizeof(float), s, partial_out, partial_ml, out,
                        out_sums, a.partitions, head_dim, q_heads, status);
     return check_launch("attention_merge");
+}
+}  // namespace
+
+extern "C" int guffin_hip_attention_decode(void* stream, const float* q, const void* ring_k, const void* ring_v,
+                                           const void* priv_k, const void* priv_v, const uint32_t* schedule,
+                                           const uint32_t* ancestors, float* out, float* out_sums,
+                                           float* partial_out, float* partial_ml, uint32_t rows,
+                                           uint32_t private_rows, uint32_t max_tokens, uint32_t ring_mask,
+                                           uint32_t q_heads, uint32_t kv_heads, uint32_t head_dim, float scale,
+                                           uint32_t* status) {
+    if (!q) return fail(GUFFIN_E_ARG, "attention_decode: null pointer");
+    return attention_decode(stream, q, nullptr, ring_k, ring_v, const_cast<void*>(priv_k), const_cast<void*>(priv_v),
+                            schedule, ancestors, out, out_sums, partial_out, partial_ml, rows, private_rows, max_tokens,
+                            ring_mask, q_heads, kv_heads, head_dim, scale, status);
+}
+
+extern "C" int guffin_hip_qkv_attention(void* stream, const float* q_raw, const float* k_raw, const float* v_raw,
+                                        uint32_t planes, uint64_t q_plane_stride, uint64_t k_plane_stride,
+                                        uint64_t v_plane_stride, const float* q_norm, const float* k_norm,
+                                        const float* rope_table, float eps, const void* ring_k, const void* ring_v,
+                                        void* priv_k, void* priv_v, const uint32_t* schedule,
+                                        const uint32_t* ancestors, float* out, float* out_sums, float* partial_out,
+                                        float* partial_ml, uint32_t rows, uint32_t max_tokens, uint32_t ring_mask,
+                                        uint32_t q_heads, uint32_t kv_heads, uint32_t head_dim, float scale,
+                                        uint32_t* status) {
+    const FusedInputs f {q_raw, k_raw, v_raw, planes, q_plane_stride, k_plane_stride, v_plane_stride, q_norm, k_norm,
+                         rope_table, eps};
+    return attention_decode(stream, nullptr, &f, ring_k, ring_v, priv_k, priv_v, schedule, ancestors, out, out_sums,
+                            partial_out, partial_ml, rows, rows, max_tokens, ring_mask, q_heads, kv_heads, head_dim,
+                            scale, status);
 }

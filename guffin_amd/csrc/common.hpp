@@ -71,6 +71,20 @@ __device__ __forceinline__ float wave_max(float v) {
     return v;
 }
 
+// Sum of `planes` partial planes in plane order; loads are issued four at a time so that the
+// adds, not the memory latency, form the dependent chain.
+__device__ __forceinline__ float load_planes(const float* p, uint32_t planes, size_t plane_stride) {
+    float v = p[0];
+    uint32_t s = 1;
+    for (; s + 4 <= planes; s += 4) {
+        const float a = p[s * plane_stride], b = p[(s + 1) * plane_stride], c = p[(s + 2) * plane_stride],
+                    d = p[(s + 3) * plane_stride];
+        v += a; v += b; v += c; v += d;
+    }
+    for (; s < planes; ++s) v += p[s * plane_stride];
+    return v;
+}
+
 // Reduces NV per-lane values across the 64 lanes with NV-1 + (6 - log2 NV) exchanges
 // instead of 6*NV: at each level the upper half-wave keeps one half of the values and
 // the lower half-wave the other.  Afterwards v[0] on lane l holds the wave total of

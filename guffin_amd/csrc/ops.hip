@@ -30,20 +30,6 @@ __device__ __forceinline__ float block_sum(float v, float* scratch) {
     return t;
 }
 
-// Sum of `planes` partial planes in plane order; loads are issued four at a time so that the
-// adds, not the memory latency, form the dependent chain.
-__device__ __forceinline__ float load_planes(const float* p, uint32_t planes, size_t plane_stride) {
-    float v = p[0];
-    uint32_t s = 1;
-    for (; s + 4 <= planes; s += 4) {
-        const float a = p[s * plane_stride], b = p[(s + 1) * plane_stride], c = p[(s + 2) * plane_stride],
-                    d = p[(s + 3) * plane_stride];
-        v += a; v += b; v += c; v += d;
-    }
-    for (; s < planes; ++s) v += p[s * plane_stride];
-    return v;
-}
-
 // Loads the row (summing partial planes) into LDS and returns this thread's share of the
 // squared sum.  Four columns per thread are in flight at a time, plane loads in batches of
 // four, so a row of a few thousand columns costs two or three memory round trips.

@@ -167,7 +167,6 @@ int forward_rows(hipStream_t stream, const guffin_model_desc& m, const uint32_t*
     for (uint32_t l = 0; l < m.layer_count; ++l) {
         const guffin_layer_desc& L = m.layers[l];
         const bool local = is_local(m, l);
-        const float base = local ? m.local_base : m.global_base, scale = local ? 1.0f : m.global_scale;
         const uint32_t ring_mask = (local ? m.ring_local : m.ring_global) - 1;
         uint16_t* pk = static_cast<uint16_t*>(priv_k) + size_t(l) * rows * KW;
         uint16_t* pv = static_cast<uint16_t*>(priv_v) + size_t(l) * rows * KW;
@@ -179,15 +178,14 @@ int forward_rows(hipStream_t stream, const guffin_model_desc& m, const uint32_t*
             GUFFIN_TRY(guffin_hip_gemv_packed_multi(st, 3, dt, tl, n, parts, s.u, s.us, rows, H));
             const uint32_t sq = qkv_slices(L, H, QW, KW);
             if (sq == 0) return fail(GUFFIN_E_SHAPE, "forward: q, k and v must share the block length");
-            GUFFIN_TRY(guffin_hip_qkv_post(st, s.part_a, s.part_b, s.part_c, sq, sq, sq, uint64_t(rows) * QW, uint64_t(rows) * KW,
-                                           uint64_t(rows) * KW, L.norm[1], L.norm[2], s.positions, s.q, pk, pv, rows,
-                                           m.q_heads, m.kv_heads, m.head_dim, m.head_dim, base, scale, m.eps,
-                                           local ? s.rope_local : s.rope_global, status));
+            // head norms, rotation, fp16 K/V rows and the attention itself in one pass over the planes
+            GUFFIN_TRY(guffin_hip_qkv_attention(st, s.part_a, s.part_b, s.part_c, sq, uint64_t(rows) * QW, uint64_t(rows) * KW,
+                                                uint64_t(rows) * KW, L.norm[1], L.norm[2],
+                                                local ? s.rope_local : s.rope_global, m.eps, L.ring_k, L.ring_v, pk, pv,
+                                                s.schedule + size_t(l) * rows * 4, s.ancestors, s.a, s.as, s.attn_out,
+                                                s.attn_ml, rows, max_tokens_for(m, l, position, rows), ring_mask,
+                                                m.q_heads, m.kv_heads, m.head_dim, attn_scale, status));
         }
-        GUFFIN_TRY(guffin_hip_attention_decode(st, s.q, L.ring_k, L.ring_v, pk, pv, s.schedule + size_t(l) * rows * 4,
-                                               s.ancestors, s.a, s.as, s.attn_out, s.attn_ml, rows, rows,
-                                               max_tokens_for(m, l, position, rows), ring_mask, m.q_heads, m.kv_heads,
-                                               m.head_dim, attn_scale, status));
         GUFFIN_TRY(guffin_hip_gemv_packed(st, L.dtype[3], L.tiles[3], s.a, s.as, s.part_a, nullptr, rows, QW, H));
         // x1 = x + rms(o, post_attention_norm); u = rms(x1, ffn_norm)
         GUFFIN_TRY(guffin_hip_rms_norm_add_norm(st, s.part_a, slices(L.dtype[3], QW, H), uint64_t(rows) * H, L.norm[3],

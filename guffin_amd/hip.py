@@ -284,6 +284,28 @@ def attention_decode(q, ring_k, ring_v, priv_k, priv_v, schedule, ancestors, max
     return (out, sums) if want_sums else out
 
 
+def qkv_attention(q_raw, k_raw, v_raw, q_norm, k_norm, table, ring_k, ring_v, schedule, ancestors, max_tokens,
+                  ring_mask, q_heads, kv_heads, head_dim, scale, eps=1e-6, status=None):
+    """Head norms, rotation, fp16 K/V rows and attention from the projections' planes [planes, rows, width].
+    Returns (out, receipt, priv_k, priv_v)."""
+    planes, rows = q_raw.shape[0], q_raw.shape[1]
+    P = attention_partitions(max_tokens, kv_heads)
+    out = torch.empty((rows, q_heads * head_dim), dtype=torch.float32, device=q_raw.device)
+    sums = _receipt(rows, q_heads * head_dim, q_raw.device)
+    pk = torch.empty((rows, kv_heads * head_dim), dtype=torch.float16, device=q_raw.device)
+    pv = torch.empty_like(pk)
+    part_out = _f32((rows * q_heads * P * head_dim,), q_raw)
+    part_ml = _f32((rows * q_heads * P * 2,), q_raw)
+    check(lib().guffin_hip_qkv_attention(_stream(), _p(q_raw), _p(k_raw), _p(v_raw), planes,
+                                         C.c_uint64(q_raw[0].numel()), C.c_uint64(k_raw[0].numel()),
+                                         C.c_uint64(v_raw[0].numel()), _p(q_norm), _p(k_norm), _p(table),
+                                         C.c_float(eps), _p(ring_k), _p(ring_v), _p(pk), _p(pv), _p(schedule),
+                                         _p(ancestors), _p(out), _p(sums), _p(part_out), _p(part_ml), rows,
+                                         max_tokens, ring_mask, q_heads, kv_heads, head_dim, C.c_float(scale),
+                                         _p(status)))
+    return out, sums, pk, pv
+
+
 # ---- head selection, proposal law, acceptance ------------------------------------------
 import numpy as _np
 

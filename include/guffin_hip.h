@@ -205,6 +205,22 @@ int guffin_hip_attention_decode(void* stream, const float* q, const void* ring_k
                                 uint32_t private_rows, uint32_t max_tokens, uint32_t ring_mask,
                                 uint32_t q_heads, uint32_t kv_heads, uint32_t head_dim, float scale,
                                 uint32_t* status);
+/* encode_head_rms_norm + encode_verifier_rope + encode_verifier_kv_store + encode_verifier_attention
+ * (metal_command_context.hpp:119, 239, 250, 267) in one pass over the projections' partial planes
+ * ([planes][rows][heads * head_dim], summed in plane order): every attention workgroup prepares the
+ * query heads it serves, and the partition that holds a private row prepares that row's key and
+ * value, uses them and writes them to priv_k / priv_v as fp16 (one private row per query row, full
+ * rotation from rope_table: [rows][head_dim / 2] (cos, sin) pairs, guffin_hip_rope_table).
+ * q_norm / k_norm may be NULL (no head norm). */
+int guffin_hip_qkv_attention(void* stream, const float* q_raw, const float* k_raw, const float* v_raw,
+                             uint32_t planes, uint64_t q_plane_stride, uint64_t k_plane_stride,
+                             uint64_t v_plane_stride, const float* q_norm, const float* k_norm,
+                             const float* rope_table, float eps, const void* ring_k, const void* ring_v,
+                             void* priv_k, void* priv_v, const uint32_t* schedule,
+                             const uint32_t* ancestors, float* out, float* out_sums, float* partial_out,
+                             float* partial_ml, uint32_t rows, uint32_t max_tokens, uint32_t ring_mask,
+                             uint32_t q_heads, uint32_t kv_heads, uint32_t head_dim, float scale,
+                             uint32_t* status);
 
 /* ---- output-head selection ---------------------------------------------------------------
  * Per row the best `retain` (= top_k + history count, the reference's base_candidate_count)

@@ -108,3 +108,43 @@ def test_attention_rejects_bad_shapes(hip):
         hip.attention_decode(z[:256].view(1, 256), h, h, h[:1], h[:1], s, s, 4, 3, 2, 2, 128, 0.1)
     with pytest.raises(hip.GuffinError):   # ring capacity not a power of two
         hip.attention_decode(z[:1024].view(1, 1024), h, h, h[:1], h[:1], s, s, 4, 2, 4, 2, 256, 0.1)
+
+
+@pytest.mark.parametrize("rows,q_heads,kv_heads,cap,position,window,planes", [
+    (2, 16, 8, 1024, 8190, 1024, 2),   # target local block: private rows straddle the last partition
+    (2, 16, 8, 8192, 8190, 0, 2),      # target global block
+    (1, 4, 1, 512, 4096, 512, 4),      # drafter local block
+    (1, 4, 1, 8192, 4095, 0, 1),       # drafter global block, a single plane
+    (2, 4, 2, 64, 31, 0, 3),           # private rows fall into two different partitions
+    (2, 2, 2, 64, 0, 0, 1),            # empty prefix
+])
+def test_attention_from_projection_planes_equals_the_separate_passes(hip, rows, q_heads, kv_heads, cap, position,
+                                                                     window, planes):
+    """One launch that prepares q, k, v itself gives bit for bit what qkv_post + attention give."""
+    import torch
+    hd = 256
+    rng = np.random.default_rng(position * 7 + rows)
+    ring_k = dev(rng.normal(0, 1, (cap, kv_heads * hd)).astype(np.float16))
+    ring_v = dev(rng.normal(0, 1, (cap, kv_heads * hd)).astype(np.float16))
+    q_raw = dev(rng.normal(0, 1, (planes, rows, q_heads * hd)).astype(np.float32))
+    k_raw = dev(rng.normal(0, 1, (planes, rows, kv_heads * hd)).astype(np.float32))
+    v_raw = dev(rng.normal(0, 1, (planes, rows, kv_heads * hd)).astype(np.float32))
+    q_norm = dev(rng.normal(1, 0.1, hd).astype(np.float32))
+    k_norm = dev(rng.normal(1, 0.1, hd).astype(np.float32))
+    positions = dev(np.arange(position, position + rows, dtype=np.uint32))
+    table = hip.rope_table(positions, hd, 10000.0)
+    sched = contiguous_schedule(position, rows, window)
+    anc = dev(np.arange(rows, dtype=np.uint32))
+    union = int(max(s[0] + s[1] for s in sched) - min(s[0] for s in sched if s[1]) if any(s[1] for s in sched) else 0)
+    status = torch.zeros(1, dtype=torch.int32, device="cuda")
+    q, pk, pv = hip.qkv_post(q_raw, k_raw, v_raw, q_norm, k_norm, positions, rows, q_heads, kv_heads, hd, hd, 10000.0,
+                             planes=planes, table=table)
+    want, want_sums = hip.attention_decode(q, ring_k, ring_v, pk, pv, dev(sched), anc, union + rows, cap - 1,
+                                           q_heads, kv_heads, hd, 0.0625, want_sums=True)
+    got, got_sums, gk, gv = hip.qkv_attention(q_raw, k_raw, v_raw, q_norm, k_norm, table, ring_k, ring_v, dev(sched),
+                                              anc, union + rows, cap - 1, q_heads, kv_heads, hd, 0.0625, status=status)
+    torch.cuda.synchronize()
+    assert int(status[0]) == 0
+    assert torch.equal(gk.view(torch.int16), pk.view(torch.int16)) and torch.equal(gv.view(torch.int16), pv.view(torch.int16))
+    assert torch.equal(got.view(torch.int32), want.view(torch.int32))
+    assert torch.equal(got_sums.view(torch.int32), want_sums.view(torch.int32))
