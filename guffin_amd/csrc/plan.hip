@@ -227,7 +227,11 @@ __global__ void commit_rows_kernel(const uint16_t* priv_k, const uint16_t* priv_
     }
 }
 
-__global__ void set_token_kernel(const uint32_t* src, uint32_t* dst) { *dst = *src; }
+// the step's token slots: [0] root, [1] proposal (written later), [8..] the drafter's input rows
+__global__ void set_step_tokens_kernel(const uint32_t* root, const uint32_t* pending, uint32_t* words) {
+    words[0] = *root;
+    if (pending) { words[8] = *pending; words[9] = *root; } else { words[8] = *root; }
+}
 
 }  // namespace
 }  // namespace guffin
@@ -379,20 +383,24 @@ struct StepBuffers {
     uint32_t* words;
     uint64_t* full_cdf;
 };
+// rows the drafter ingests: the root alone, or the accepted proposal it still owes and the root
+uint32_t drafter_rows(const guffin_h1_desc* d) { return d->drafter_rows == 2 ? 2u : 1u; }
+
 StepBuffers carve_step(const guffin_h1_desc* d, void* scratch) {
     const guffin_model_desc& T = *d->target;
     const guffin_model_desc& D = *d->drafter;
     const uint64_t V = T.vocab;
     Arena ar {static_cast<uint8_t*>(scratch), 0, 0};
     StepBuffers b {};
-    b.d_bytes = guffin_hip_forward_scratch_bytes(&D, 1, d->drafter_position);
+    const uint32_t dr = drafter_rows(d);
+    b.d_bytes = guffin_hip_forward_scratch_bytes(&D, dr, d->drafter_position);
     b.t_bytes = guffin_hip_forward_scratch_bytes(&T, 2, d->target_position);
     b.d_scratch = ar.take<uint8_t>(b.d_bytes);
     b.t_scratch = ar.take<uint8_t>(b.t_bytes);
-    b.d_hidden = ar.take<float>(hidden_with_receipt(1, D.hidden));
+    b.d_hidden = ar.take<float>(hidden_with_receipt(dr, D.hidden));
     b.t_hidden = ar.take<float>(hidden_with_receipt(2, T.hidden));
-    b.q_parts = ar.take<float>(uint64_t(slices(D.head_dtype, D.hidden, D.vocab)) * D.vocab);
-    b.q_logits = ar.take<float>(D.vocab);
+    b.q_parts = ar.take<float>(uint64_t(slices(D.head_dtype, D.hidden, D.vocab)) * dr * D.vocab);
+    b.q_logits = ar.take<float>(uint64_t(dr) * D.vocab);
     b.p_parts = ar.take<float>(uint64_t(slices(T.head_dtype, T.hidden, V)) * 2 * V);
     b.p_logits = ar.take<float>(2 * V);
     b.law_ws = ar.take<uint8_t>(guffin_hip_draft_law_workspace_bytes(D.vocab));
@@ -445,13 +453,16 @@ extern "C" int guffin_hip_h1_step(void* stream, const guffin_h1_desc* d, const u
     struct { float temperature; uint32_t top_k; float top_p, min_p, repetition_penalty; } opt
         = {d->temperature, d->top_k, d->top_p, d->min_p, 1.0f};
 
-    // 1. drafter: ingest the root, project, build the proposal law, pick x with the step's word
-    hipLaunchKernelGGL(set_token_kernel, dim3(1), dim3(1), 0, s, root_token, tokens);
-    GUFFIN_TRY(check_launch("set_token"));
-    GUFFIN_TRY(guffin_hip_forward_rows(stream, &D, tokens, 1, d->drafter_position, d_scratch, d_bytes, drafter_priv_k,
-                                       drafter_priv_v, d_hidden, d_hidden + hidden_receipt_offset(1, D.hidden), status));
-    GUFFIN_TRY(guffin_hip_gemv_packed(stream, D.head_dtype, D.head_tiles, d_hidden, d_hidden + hidden_receipt_offset(1, D.hidden), q_parts,
-                                      q_logits, 1, D.hidden, D.vocab));
+    // 1. drafter: ingest (the pending proposal and) the root, project, build the proposal law, pick x
+    const uint32_t dr = drafter_rows(d);
+    if (dr == 2 && !d->pending_token) return fail(GUFFIN_E_ARG, "h1_step: two drafter rows need the pending token");
+    hipLaunchKernelGGL(set_step_tokens_kernel, dim3(1), dim3(1), 0, s, root_token, dr == 2 ? d->pending_token : nullptr, tokens);
+    GUFFIN_TRY(check_launch("set_step_tokens"));
+    GUFFIN_TRY(guffin_hip_forward_rows(stream, &D, tokens + 8, dr, d->drafter_position, d_scratch, d_bytes, drafter_priv_k,
+                                       drafter_priv_v, d_hidden, d_hidden + hidden_receipt_offset(dr, D.hidden), status));
+    GUFFIN_TRY(guffin_hip_gemv_packed(stream, D.head_dtype, D.head_tiles, d_hidden, d_hidden + hidden_receipt_offset(dr, D.hidden), q_parts,
+                                      q_logits, dr, D.hidden, D.vocab));
+    q_logits += uint64_t(dr - 1) * D.vocab;  // the law comes from the last ingested row (the root)
     if (d->full_law) {
         GUFFIN_TRY(guffin_hip_draft_law_any(stream, q_logits, D.vocab, &opt, d->seed, d->step, nullptr, any_ws, law,
                                             full_cdf, tokens + 1, status));
@@ -475,7 +486,7 @@ extern "C" int guffin_hip_h1_step(void* stream, const guffin_h1_desc* d, const u
     }
     if (d->drafter_ring_k && d->drafter_ring_v) {
         GUFFIN_TRY(guffin_hip_commit_rows(stream, &D, drafter_priv_k, drafter_priv_v, d->drafter_ring_k,
-                                          d->drafter_ring_v, nullptr, d->drafter_position, 1));
+                                          d->drafter_ring_v, nullptr, d->drafter_position, dr));
     }
     return GUFFIN_OK;
 }
@@ -490,7 +501,7 @@ extern "C" int guffin_hip_h1_buffers(const guffin_h1_desc* d, void* scratch, flo
     const StepBuffers B = carve_step(d, scratch);
     if (drafter_hidden) *drafter_hidden = B.d_hidden;
     if (target_hidden) *target_hidden = B.t_hidden;
-    if (q_logits) *q_logits = B.q_logits;
+    if (q_logits) *q_logits = B.q_logits + uint64_t(drafter_rows(d) - 1) * d->drafter->vocab;
     if (p_logits) *p_logits = B.p_logits;
     if (law) *law = B.law;
     if (candidates) *candidates = B.cands;
@@ -503,5 +514,101 @@ extern "C" int guffin_hip_h1_full_cdf(const guffin_h1_desc* d, void* scratch, ui
     GUFFIN_TRY(validate_model(d->target));
     GUFFIN_TRY(validate_model(d->drafter));
     *full_cdf = carve_step(d, scratch).full_cdf;
+    return GUFFIN_OK;
+}
+
+// ---- consecutive cycles ---------------------------------------------------------------------
+// Host-side lifecycle around guffin_hip_h1_step: positions, the drafter's pending token and the
+// transaction state of the verify pass.  States follow VerifierTransactionState
+// (include/local_gguf_engine/engine/gemma2_metal_plan.hpp:208-215); the pending token follows
+// Gemma3DraftPlan (include/local_gguf_engine/engine/gemma3_draft.hpp:61-63,
+// src/engine/gemma3_draft.mm:1430-1486): the drafter's last emission is materialised together with
+// the next root, and only if the target accepted it.
+namespace guffin {
+namespace {
+struct StepResultHead { uint32_t accepted, token, next_root, status; };
+
+int session_ready(const guffin_h1_session* s, const char* what) {
+    if (!s || !s->scratch || !s->drafter_priv_k || !s->drafter_priv_v || !s->target_priv_k || !s->target_priv_v
+        || !s->tokens || !s->result || !s->status)
+        return fail(GUFFIN_E_ARG, what);
+    return GUFFIN_OK;
+}
+}  // namespace
+}  // namespace guffin
+
+extern "C" uint64_t guffin_hip_session_scratch_bytes(const guffin_h1_session* s, uint32_t last_target_position,
+                                                     uint32_t last_drafter_position) {
+    if (!s) return 0;
+    guffin_h1_desc d = s->desc;  // the largest arena any cycle up to the given positions needs
+    d.target_position = last_target_position;
+    d.drafter_position = last_drafter_position;
+    d.drafter_rows = 2;
+    return guffin_hip_h1_scratch_bytes(&d);
+}
+
+extern "C" int guffin_hip_session_start(guffin_h1_session* s, uint32_t root_token, uint32_t target_position,
+                                        uint32_t drafter_position) {
+    GUFFIN_TRY(session_ready(s, "session_start: null pointer"));
+    if (!s->desc.target_ring_k || !s->desc.target_ring_v || !s->desc.drafter_ring_k || !s->desc.drafter_ring_v)
+        return fail(GUFFIN_E_ARG, "session_start: a session publishes its rows: ring tables are required");
+    s->desc.target_position = target_position;
+    s->desc.drafter_position = drafter_position;
+    s->desc.step = 0;
+    s->root = root_token; s->pending = 0; s->has_pending = 0;
+    s->cycles = 0; s->accepted = 0;
+    s->state = GUFFIN_TXN_IDLE;
+    return GUFFIN_OK;
+}
+
+extern "C" int guffin_hip_session_submit(void* stream, guffin_h1_session* s) {
+    GUFFIN_TRY(session_ready(s, "session_submit: null pointer"));
+    if (s->state == GUFFIN_TXN_POISONED) return fail(GUFFIN_E_STATE, "session_submit: the session is poisoned");
+    if (s->state != GUFFIN_TXN_IDLE) return fail(GUFFIN_E_STATE, "session_submit: a cycle is already in flight");
+    hipStream_t hs = as_stream(stream);
+    const uint32_t words[2] = {s->root, s->pending}, zero = 0;
+    if (hipMemcpyAsync(s->tokens, words, sizeof(words), hipMemcpyHostToDevice, hs) != hipSuccess
+        || hipMemcpyAsync(s->status, &zero, sizeof(zero), hipMemcpyHostToDevice, hs) != hipSuccess)
+        return fail(GUFFIN_E_HIP, "session_submit: upload failed");
+    s->desc.drafter_rows = s->has_pending ? 2u : 1u;
+    s->desc.pending_token = s->tokens + 1;
+    if (int rc = guffin_hip_h1_step(stream, &s->desc, s->tokens, s->scratch, s->scratch_bytes, s->drafter_priv_k,
+                                    s->drafter_priv_v, s->target_priv_k, s->target_priv_v, s->result, s->status))
+        return rc;  // nothing was enqueued that changes the caches: still idle
+    s->state = GUFFIN_TXN_SUBMITTED;
+    return GUFFIN_OK;
+}
+
+extern "C" int guffin_hip_session_complete(void* stream, guffin_h1_session* s, uint32_t* emitted, uint32_t* emitted_count) {
+    GUFFIN_TRY(session_ready(s, "session_complete: null pointer"));
+    if (!emitted || !emitted_count) return fail(GUFFIN_E_ARG, "session_complete: null pointer");
+    if (s->state != GUFFIN_TXN_SUBMITTED) return fail(GUFFIN_E_STATE, "session_complete: no cycle in flight");
+    StepResultHead r {};
+    uint32_t status = 0;
+    if (hipStreamSynchronize(as_stream(stream)) != hipSuccess
+        || hipMemcpy(&r, s->result, sizeof(r), hipMemcpyDeviceToHost) != hipSuccess
+        || hipMemcpy(&status, s->status, sizeof(status), hipMemcpyDeviceToHost) != hipSuccess) {
+        s->state = GUFFIN_TXN_POISONED;
+        return fail(GUFFIN_E_HIP, "session_complete: read-back failed");
+    }
+    *emitted_count = 0;
+    if (status != 0 || r.status != 0) {
+        // a numerical fault or a refused law: the rows of this cycle may already be in the caches
+        s->state = GUFFIN_TXN_POISONED;
+        return fail(GUFFIN_E_STATE, "session_complete: device status raised, the session is poisoned");
+    }
+    // row 0 (the root) is published; row 1 (the proposal) too if it was accepted
+    const uint32_t proposal = r.accepted ? r.token : 0;
+    s->desc.target_position += 1 + (r.accepted ? 1u : 0u);
+    s->desc.drafter_position += s->desc.drafter_rows == 2 ? 2u : 1u;
+    s->desc.step += 1;
+    s->cycles += 1;
+    s->accepted += r.accepted ? 1u : 0u;
+    if (r.accepted) { emitted[0] = proposal; emitted[1] = r.next_root; *emitted_count = 2; }
+    else { emitted[0] = r.token; *emitted_count = 1; }
+    s->has_pending = r.accepted ? 1u : 0u;   // the drafter has not seen the accepted proposal yet
+    s->pending = proposal;
+    s->root = r.next_root;
+    s->state = GUFFIN_TXN_IDLE;
     return GUFFIN_OK;
 }

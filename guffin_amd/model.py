@@ -38,7 +38,17 @@ class H1Desc(C.Structure):
                 ("temperature", C.c_float), ("top_k", C.c_uint32), ("top_p", C.c_float), ("min_p", C.c_float),
                 ("seed", C.c_uint64), ("step", C.c_uint64),
                 ("target_ring_k", C.c_void_p), ("target_ring_v", C.c_void_p),
-                ("drafter_ring_k", C.c_void_p), ("drafter_ring_v", C.c_void_p), ("full_law", C.c_uint32)]
+                ("drafter_ring_k", C.c_void_p), ("drafter_ring_v", C.c_void_p), ("full_law", C.c_uint32),
+                ("drafter_rows", C.c_uint32), ("pending_token", C.c_void_p)]
+
+
+class H1Session(C.Structure):
+    _fields_ = [("desc", H1Desc), ("scratch", C.c_void_p), ("scratch_bytes", C.c_uint64),
+                ("drafter_priv_k", C.c_void_p), ("drafter_priv_v", C.c_void_p),
+                ("target_priv_k", C.c_void_p), ("target_priv_v", C.c_void_p),
+                ("tokens", C.c_void_p), ("result", C.c_void_p), ("status", C.c_void_p),
+                ("state", C.c_uint32), ("root", C.c_uint32), ("pending", C.c_uint32), ("has_pending", C.c_uint32),
+                ("cycles", C.c_uint64), ("accepted", C.c_uint64)]
 
 
 @dataclass(frozen=True)
@@ -138,6 +148,14 @@ class HostModel:
             arr[l].ring_k = self.ring_k[l].ctypes.data
             arr[l].ring_v = self.ring_v[l].ctypes.data
         return arr
+
+    def commit(self, pk, pv, position, rows):
+        """Publishes the first `rows` private rows of a pass at `position` into the rings, like the device."""
+        for l in range(self.shape.layers):
+            cap = self.shape.ring_local if self.shape.is_local(l) else self.shape.ring_global
+            for r in range(rows):
+                self.ring_k[l][(position + r) & (cap - 1)] = pk[l, r].view(np.float16)
+                self.ring_v[l][(position + r) & (cap - 1)] = pv[l, r].view(np.float16)
 
     def oracle_forward(self, gfo, tokens, position, threads=8):
         sh = self.shape
@@ -338,6 +356,7 @@ class H1Plan:
                                                   *[C.byref(p) for p in ptrs]))
         base = self.scratch.data_ptr()
         T, D = self.target.shape, self.drafter.shape
+        d_rows = 2 if self.desc.drafter_rows == 2 else 1
 
         def view(ptr, count, dtype):
             off = ptr.value - base
@@ -347,7 +366,8 @@ class H1Plan:
         hip.check(hip.lib().guffin_hip_h1_full_cdf(C.byref(self.desc), hip._p(self.scratch), C.byref(full)))
         return {
             "full_cdf": view(full, D.vocab + 1, torch.int64) if full.value else None,
-            "drafter_hidden": view(ptrs[0], D.hidden, torch.float32),
+            "drafter_hidden": view(ptrs[0], d_rows * D.hidden, torch.float32).view(d_rows, D.hidden)[d_rows - 1],
+            "drafter_hidden_rows": view(ptrs[0], d_rows * D.hidden, torch.float32).view(d_rows, D.hidden),
             "target_hidden": view(ptrs[1], 2 * T.hidden, torch.float32).view(2, T.hidden),
             "q_logits": view(ptrs[2], D.vocab, torch.float32),
             "p_logits": view(ptrs[3], 2 * T.vocab, torch.float32).view(2, T.vocab),
@@ -355,3 +375,54 @@ class H1Plan:
             "candidates": view(ptrs[5], 2 * hip.candidates_dtype.itemsize, torch.uint8),
             "tokens": view(ptrs[6], 2, torch.int32),
         }
+
+
+class Session:
+    """Consecutive H1 cycles through guffin_hip_session_*: the library keeps positions, the drafter's
+    pending token and the transaction state; this class owns the device memory it points at."""
+
+    def __init__(self, target, drafter, root, target_position, drafter_position, cycles, temperature=1.0, top_k=64,
+                 top_p=0.95, min_p=0.0, seed=0, full_law=False):
+        self.target, self.drafter = target, drafter
+        s = self.s = H1Session()
+        d = s.desc
+        d.target, d.drafter = C.pointer(target.desc), C.pointer(drafter.desc)
+        d.temperature, d.top_k, d.top_p, d.min_p = temperature, top_k, top_p, min_p
+        d.seed, d.full_law = seed, 1 if full_law else 0
+        d.target_ring_k, d.target_ring_v = target.ring_k_table.data_ptr(), target.ring_v_table.data_ptr()
+        d.drafter_ring_k, d.drafter_ring_v = drafter.ring_k_table.data_ptr(), drafter.ring_v_table.data_ptr()
+        lib = hip.lib()
+        lib.guffin_hip_session_scratch_bytes.restype = C.c_uint64
+        nbytes = lib.guffin_hip_session_scratch_bytes(C.byref(s), target_position + 2 * cycles,
+                                                      drafter_position + 2 * cycles)
+        if nbytes == 0:
+            raise hip.GuffinError(-1, lib.guffin_hip_last_error().decode())
+        self.scratch = torch.zeros(nbytes, dtype=torch.uint8, device="cuda")
+        self.d_pk, self.d_pv = drafter.private_rows(2)
+        self.t_pk, self.t_pv = target.private_rows(2)
+        self.tokens = torch.zeros(2, dtype=torch.int32, device="cuda")
+        self.result = torch.zeros(hip.result_dtype.itemsize, dtype=torch.uint8, device="cuda")
+        self.status = hip.new_status()
+        s.scratch, s.scratch_bytes = self.scratch.data_ptr(), nbytes
+        s.drafter_priv_k, s.drafter_priv_v = self.d_pk.data_ptr(), self.d_pv.data_ptr()
+        s.target_priv_k, s.target_priv_v = self.t_pk.data_ptr(), self.t_pv.data_ptr()
+        s.tokens, s.result, s.status = self.tokens.data_ptr(), self.result.data_ptr(), self.status.data_ptr()
+        hip.check(lib.guffin_hip_session_start(C.byref(s), root, target_position, drafter_position))
+
+    def submit(self):
+        hip.check(hip.lib().guffin_hip_session_submit(hip._stream(), C.byref(self.s)))
+
+    def complete(self):
+        out = (C.c_uint32 * 2)()
+        n = C.c_uint32()
+        self._cycle_desc = H1Desc.from_buffer_copy(self.s.desc)   # the arena layout of the cycle in flight
+        hip.check(hip.lib().guffin_hip_session_complete(hip._stream(), C.byref(self.s), out, C.byref(n)))
+        return [int(out[i]) for i in range(n.value)]
+
+    def buffers(self):
+        plan = H1Plan.__new__(H1Plan)
+        plan.desc, plan.scratch, plan.target, plan.drafter = self._cycle_desc, self.scratch, self.target, self.drafter
+        return H1Plan.buffers(plan)
+
+    def read_result(self):
+        return self.result.cpu().numpy().view(hip.result_dtype)[0]

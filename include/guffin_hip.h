@@ -33,6 +33,7 @@ extern "C" {
 #define GUFFIN_E_ALIGN (-3)     /* pointer alignment below what the block stream guarantees */
 #define GUFFIN_E_CAPACITY (-4)  /* exceeds a fixed capacity (LDS, candidate count ...) */
 #define GUFFIN_E_HIP (-5)       /* HIP runtime error, see guffin_hip_last_error() */
+#define GUFFIN_E_STATE (-6)     /* call out of order for the session's state, or the session is poisoned */
 
 /* reference: include/local_gguf_engine/tensor/dtype.hpp:9-15 (block layouts 34/144/210 B) */
 #define GUFFIN_Q8_0 0
@@ -379,6 +380,9 @@ typedef struct guffin_h1_desc {
     void* const* target_ring_k; void* const* target_ring_v;
     void* const* drafter_ring_k; void* const* drafter_ring_v;
     uint32_t full_law;  /* != 0: encode the full-vocabulary law too (overflow fallback, top_k > 64, greedy) */
+    uint32_t drafter_rows;          /* 2: the drafter first ingests *pending_token (the proposal the target
+                                       accepted last cycle, src/engine/gemma3_draft.mm:1430-1449), then the root */
+    const uint32_t* pending_token;  /* device; read only when drafter_rows == 2 */
 } guffin_h1_desc;
 uint64_t guffin_hip_h1_scratch_bytes(const guffin_h1_desc* desc);
 int guffin_hip_h1_step(void* stream, const guffin_h1_desc* desc, const uint32_t* root_token, void* scratch,
@@ -390,6 +394,43 @@ int guffin_hip_h1_buffers(const guffin_h1_desc* desc, void* scratch, float** dra
                           void** candidates, uint32_t** tokens);
 /* The full-vocabulary table of the last step (desc->full_law != 0), else NULL. */
 int guffin_hip_h1_full_cdf(const guffin_h1_desc* desc, void* scratch, uint64_t** full_cdf);
+
+/* ---- consecutive cycles ---------------------------------------------------------------------
+ * Host-side lifecycle around guffin_hip_h1_step for generation over many cycles.  It keeps what
+ * the reference keeps between cycles: the verify pass's transaction state (VerifierTransactionState,
+ * include/local_gguf_engine/engine/gemma2_metal_plan.hpp:208-215: idle -> submitted -> idle, or
+ * poisoned for good once the device status word is raised), the positions of both caches, and the
+ * drafter's pending token (include/local_gguf_engine/engine/gemma3_draft.hpp:61-63,
+ * src/engine/gemma3_draft.mm:1430-1486): the proposal of a cycle is not in the drafter's cache; if
+ * the target accepted it, the next cycle's drafter pass ingests it together with the new root.
+ *
+ * The caller fills desc (models, sampler, seed, the four ring tables, full_law) and every device
+ * pointer below, then calls start once and submit / complete per cycle.  complete blocks on the
+ * stream, reads 20 bytes back and reports the tokens the cycle confirmed: {proposal, next root} on
+ * acceptance, {residual token} on rejection; the last one is the next cycle's root. */
+#define GUFFIN_TXN_IDLE 0u
+#define GUFFIN_TXN_SUBMITTED 2u
+#define GUFFIN_TXN_POISONED 5u
+typedef struct guffin_h1_session {
+    guffin_h1_desc desc;
+    void* scratch; uint64_t scratch_bytes;   /* device arena, >= guffin_hip_session_scratch_bytes */
+    void* drafter_priv_k; void* drafter_priv_v;   /* device, [blocks][2][kv width] fp16 each */
+    void* target_priv_k; void* target_priv_v;
+    uint32_t* tokens;                        /* device u32[2]: root, pending */
+    void* result;                            /* device, one result record (guffin_hip_spec_accept) */
+    uint32_t* status;                        /* device status word */
+    uint32_t state;                          /* GUFFIN_TXN_* */
+    uint32_t root, pending, has_pending;
+    uint64_t cycles, accepted;
+} guffin_h1_session;
+/* Arena size that covers every cycle up to the given cache positions. */
+uint64_t guffin_hip_session_scratch_bytes(const guffin_h1_session* session, uint32_t last_target_position,
+                                          uint32_t last_drafter_position);
+int guffin_hip_session_start(guffin_h1_session* session, uint32_t root_token, uint32_t target_position,
+                             uint32_t drafter_position);
+int guffin_hip_session_submit(void* stream, guffin_h1_session* session);
+int guffin_hip_session_complete(void* stream, guffin_h1_session* session, uint32_t* emitted /* [2] */,
+                                uint32_t* emitted_count);
 
 #ifdef __cplusplus
 }
