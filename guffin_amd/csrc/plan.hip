@@ -279,6 +279,7 @@ struct PrefillScratch {
     float *x, *x1, *u, *q, *kraw, *vraw, *a, *gate, *up, *h, *o;
     float *rope_local, *rope_global;
     uint16_t *run_k, *run_v;
+    uint8_t* attn_ws;   // transposed values of the matrix-core attention
     uint8_t* image;
     uint32_t* positions;
     uint64_t bytes;
@@ -296,6 +297,8 @@ PrefillScratch prefill_layout(const guffin_model_desc& m, uint32_t rows, uint8_t
     s.rope_local = ar.take<float>(uint64_t(rows) * m.head_dim);
     s.rope_global = ar.take<float>(uint64_t(rows) * m.head_dim);
     s.run_k = ar.take<uint16_t>(rows * KW); s.run_v = ar.take<uint16_t>(rows * KW);
+    // V^T of every token a row may see: at most a full global ring plus the run, in whole 32-token tiles
+    s.attn_ws = ar.take<uint8_t>(uint64_t(m.kv_heads) * m.head_dim * 2 * ((uint64_t(m.ring_global) + rows + 63) & ~uint64_t{31}));
     const uint32_t widest = std::max({m.hidden, m.ffn, m.q_heads * m.head_dim});
     s.image = ar.take<uint8_t>(guffin_hip_prefill_image_bytes(rows, widest));
     s.positions = ar.take<uint32_t>(rows);
@@ -351,7 +354,7 @@ extern "C" int guffin_hip_prefill_rows(void* stream, const guffin_model_desc* mo
                                        scale, m.eps, local ? s.rope_local : s.rope_global, status));
         GUFFIN_TRY(guffin_hip_prefill_attention(stream, s.q, L.ring_k, L.ring_v, s.run_k, s.run_v, s.a, rows, position,
                                                 local ? m.sliding_window : 0u, ring_mask, m.q_heads, m.kv_heads,
-                                                m.head_dim, attn_scale));
+                                                m.head_dim, attn_scale, s.attn_ws));
         GUFFIN_TRY(guffin_hip_publish_run(stream, s.run_k, s.run_v, L.ring_k, L.ring_v, rows, position, ring_mask, KW));
         GUFFIN_TRY(guffin_hip_prefill_pack(stream, s.a, s.image, rows, QW));
         GUFFIN_TRY(guffin_hip_prefill_gemm(stream, L.dtype[3], L.tiles[3], s.image, s.o, rows, QW, H));

@@ -447,6 +447,247 @@ prefill_attention_kernel(const float* __restrict__ q, const uint16_t* __restrict
     }
 }
 
+// ---- the same attention on the matrix core ------------------------------------------------
+// Values are contracted over tokens, so the B operand needs 8 consecutive tokens of one output
+// dimension: a small pass first writes V^T, [kv_heads][256][T] fp16, for the virtual tokens
+// base32 .. base32 + T (T a multiple of 32; tokens outside [first_visible, end) are zero).
+__global__ void __launch_bounds__(256)
+transpose_values_kernel(const uint16_t* __restrict__ ring_v, const uint16_t* __restrict__ run_v,
+                        uint16_t* __restrict__ vt, uint32_t base32, uint32_t T, uint32_t first_visible,
+                        uint32_t position, uint32_t end_pos, uint32_t ring_mask, uint32_t kv_heads) {
+    constexpr int HD = 256, PITCH = HD + 8;
+    __shared__ __attribute__((aligned(16))) uint16_t tile[32][PITCH];
+    const uint32_t kvh = blockIdx.y, v0 = blockIdx.x * 32;
+    const size_t row_stride = size_t(kv_heads) * HD;
+    for (uint32_t c = threadIdx.x; c < 32 * (HD / 8); c += 256) {
+        const uint32_t token = c / (HD / 8), d8 = c % (HD / 8);
+        const uint32_t kp = base32 + v0 + token;
+        uint4 val = make_uint4(0, 0, 0, 0);
+        if (kp >= first_visible && kp < end_pos) {
+            const uint16_t* src = kp >= position ? run_v + size_t(kp - position) * row_stride
+                                                 : ring_v + size_t(kp & ring_mask) * row_stride;
+            val = *reinterpret_cast<const uint4*>(src + kvh * HD + 8 * d8);
+        }
+        *reinterpret_cast<uint4*>(&tile[token][8 * d8]) = val;
+    }
+    __syncthreads();
+    const uint32_t dim = threadIdx.x;
+    uint32_t w[16];
+#pragma unroll
+    for (int t = 0; t < 16; ++t) w[t] = uint32_t(tile[2 * t][dim]) | (uint32_t(tile[2 * t + 1][dim]) << 16);
+    uint4* dst = reinterpret_cast<uint4*>(vt + (size_t(kvh) * HD + dim) * T + v0);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) dst[i] = make_uint4(w[4 * i], w[4 * i + 1], w[4 * i + 2], w[4 * i + 3]);
+}
+
+__device__ __forceinline__ void split_half8(const float (&x)[8], uint4& hi, uint4& lo) {
+    uint32_t h[4], l[4];
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+        uint32_t hw = 0, lw = 0;
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+            const _Float16 a = static_cast<_Float16>(x[2 * p + q]);
+            const _Float16 b = static_cast<_Float16>(x[2 * p + q] - static_cast<float>(a));
+            hw |= uint32_t(__builtin_bit_cast(uint16_t, a)) << (16 * q);
+            lw |= uint32_t(__builtin_bit_cast(uint16_t, b)) << (16 * q);
+        }
+        h[p] = hw; l[p] = lw;
+    }
+    hi = make_uint4(h[0], h[1], h[2], h[3]);
+    lo = make_uint4(l[0], l[1], l[2], l[3]);
+}
+
+// grid (ceil(rows / 16), kv_heads), 4 waves.  A workgroup serves 16 query rows x GROUP heads of one
+// KV head.  Each wave walks its own 32-token tiles (tile index = wave mod 4) with its own online
+// softmax state and its own output accumulators; the four states are merged at the end.
+//   scores   S = Q K^T: queries (scaled, fp16 hi + lo, staged once in LDS in operand order) as A,
+//            keys straight from their fp16 rows as B (a lane reads 8 dims of one key per MFMA)
+//   values   O += P V: probabilities times 2^10 as fp16 hi + lo through a wave-private LDS
+//            transpose as A, V^T rows as B
+template <int GROUP>
+__global__ void __launch_bounds__(256)
+prefill_attention_mfma_kernel(const float* __restrict__ q, const uint16_t* __restrict__ ring_k,
+                              const uint16_t* __restrict__ run_k, const uint16_t* __restrict__ vt,
+                              float* __restrict__ out, uint32_t rows, uint32_t position, uint32_t window,
+                              uint32_t ring_mask, uint32_t q_heads, uint32_t kv_heads, float scale,
+                              uint32_t base32, uint32_t T) {
+    constexpr int HD = 256, QT = 16;
+    constexpr float kProbScale = 1024.0f;
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    // [GROUP][8 k-steps][hi, lo][64 lanes] 16-byte query operands, later the merge buffer
+    uint8_t* qa = lds;
+    const uint32_t lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t j = lane & 15, lg = lane >> 4;
+    float* pt = reinterpret_cast<float*>(lds + GROUP * 16384) + wave * (GROUP * QT * 32);  // [GROUP][16 rows][32 tokens]
+    float* ml = reinterpret_cast<float*>(lds + GROUP * 16384 + 4 * GROUP * QT * 32 * 4);     // [GROUP][16][2] for the merge
+    const uint32_t kvh = blockIdx.y, r0 = blockIdx.x * QT;
+    const size_t row_stride = size_t(kv_heads) * HD;
+
+    for (uint32_t idx = threadIdx.x; idx < GROUP * QT * 32; idx += 256) {
+        const uint32_t g = idx / (QT * 32), i = (idx / 32) % QT, c8 = idx % 32;
+        const uint32_t row = min(r0 + i, rows - 1);
+        const float* src = q + (size_t(row) * q_heads + kvh * GROUP + g) * HD + 8 * c8;
+        const float4 a = *reinterpret_cast<const float4*>(src), b = *reinterpret_cast<const float4*>(src + 4);
+        const float x[8] = {a.x * scale, a.y * scale, a.z * scale, a.w * scale, b.x * scale, b.y * scale, b.z * scale, b.w * scale};
+        uint4 hi, lo;
+        split_half8(x, hi, lo);
+        uint8_t* dst = qa + ((g * 8 + c8 / 4) * 2) * 1024 + (i + 16 * (c8 % 4)) * 16;
+        *reinterpret_cast<uint4*>(dst) = hi;
+        *reinterpret_cast<uint4*>(dst + 1024) = lo;
+    }
+    __syncthreads();
+
+    float m[GROUP][4], l[GROUP][4];
+    float4_t O[GROUP][16];
+#pragma unroll
+    for (int g = 0; g < GROUP; ++g) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) { m[g][r] = -INFINITY; l[g][r] = 0.f; }
+#pragma unroll
+        for (int dt = 0; dt < 16; ++dt) O[g][dt] = float4_t{0.f, 0.f, 0.f, 0.f};
+    }
+    const uint32_t last_row = min(r0 + QT, rows) - 1;
+    const uint32_t hi_pos = position + last_row;
+    const uint32_t lo_first = (window && position + r0 + 1 > window) ? position + r0 + 1 - window : 0;
+    uint32_t pos_r[4], first_r[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const uint32_t row = r0 + 4 * lg + r;
+        pos_r[r] = row < rows ? position + row : 0u;  // a padding row sees nothing: first > pos
+        first_r[r] = row < rows ? ((window && position + row + 1 > window) ? position + row + 1 - window : 0u) : 1u;
+    }
+    const uint32_t tile_lo = (lo_first - base32) / 32, tile_hi = (hi_pos - base32) / 32;
+    for (uint32_t ti = tile_lo + wave; ti <= tile_hi; ti += 4) {
+        const uint32_t t0 = base32 + 32 * ti;
+        float4_t S[GROUP][2];
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+            const uint32_t kp = min(t0 + 16 * c + j, hi_pos);
+            const uint16_t* krow = (kp >= position ? run_k + size_t(kp - position) * row_stride
+                                                   : ring_k + size_t(kp & ring_mask) * row_stride) + kvh * HD + 8 * lg;
+            uint4 kb[8];
+#pragma unroll
+            for (int ks = 0; ks < 8; ++ks) kb[ks] = *reinterpret_cast<const uint4*>(krow + 32 * ks);
+#pragma unroll
+            for (int g = 0; g < GROUP; ++g) {
+                float4_t acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int ks = 0; ks < 8; ++ks) {
+                    const uint8_t* ap = qa + ((g * 8 + ks) * 2) * 1024 + lane * 16;
+                    const half8_t kv = __builtin_bit_cast(half8_t, kb[ks]);
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, *reinterpret_cast<const uint4*>(ap)), kv, acc, 0, 0, 0);
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, *reinterpret_cast<const uint4*>(ap + 1024)), kv, acc, 0, 0, 0);
+                }
+                S[g][c] = acc;
+            }
+        }
+        // online softmax of the lane group's four rows; a row's 32 scores sit in 16 lanes x 2 tiles
+#pragma unroll
+        for (int g = 0; g < GROUP; ++g) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                float sv[2];
+#pragma unroll
+                for (int c = 0; c < 2; ++c) {
+                    const uint32_t kp = t0 + 16 * c + j;
+                    const bool visible = kp <= pos_r[r] && kp >= first_r[r] && kp <= hi_pos;
+                    sv[c] = visible ? S[g][c][r] : -INFINITY;
+                }
+                float tmax = fmaxf(sv[0], sv[1]);
+#pragma unroll
+                for (int o = 8; o > 0; o >>= 1) tmax = fmaxf(tmax, __shfl_xor(tmax, o, kWave));
+                const float new_m = fmaxf(m[g][r], tmax);
+                const float resc = new_m == -INFINITY ? 1.f : expf(m[g][r] - new_m);
+                const float p0 = sv[0] == -INFINITY ? 0.f : expf(sv[0] - new_m);
+                const float p1 = sv[1] == -INFINITY ? 0.f : expf(sv[1] - new_m);
+                float add = p0 + p1;
+#pragma unroll
+                for (int o = 8; o > 0; o >>= 1) add += __shfl_xor(add, o, kWave);
+                l[g][r] = l[g][r] * resc + add;
+                m[g][r] = new_m;
+#pragma unroll
+                for (int dt = 0; dt < 16; ++dt) O[g][dt][r] *= resc;
+                pt[(g * QT + 4 * lg + r) * 32 + j] = p0 * kProbScale;
+                pt[(g * QT + 4 * lg + r) * 32 + 16 + j] = p1 * kProbScale;
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        half8_t pa_hi[GROUP], pa_lo[GROUP];
+#pragma unroll
+        for (int g = 0; g < GROUP; ++g) {
+            const float* src = pt + (g * QT + j) * 32 + 8 * lg;  // A lane (row j, tokens 8 lg .. 8 lg + 7)
+            const float4 a = *reinterpret_cast<const float4*>(src), b = *reinterpret_cast<const float4*>(src + 4);
+            const float x[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+            uint4 hi, lo;
+            split_half8(x, hi, lo);
+            pa_hi[g] = __builtin_bit_cast(half8_t, hi);
+            pa_lo[g] = __builtin_bit_cast(half8_t, lo);
+        }
+        const uint16_t* vcol = vt + (size_t(kvh) * HD + j) * T + (t0 - base32) + 8 * lg;
+#pragma unroll
+        for (int dt = 0; dt < 16; ++dt) {
+            const half8_t vb = __builtin_bit_cast(half8_t, *reinterpret_cast<const uint4*>(vcol + size_t(16 * dt) * T));
+#pragma unroll
+            for (int g = 0; g < GROUP; ++g) {
+                O[g][dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa_hi[g], vb, O[g][dt], 0, 0, 0);
+                O[g][dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa_lo[g], vb, O[g][dt], 0, 0, 0);
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+    // merge the four waves' states in wave order through LDS (the query operands are dead now)
+    float* ob = reinterpret_cast<float*>(qa);  // [(g * 16 + dt) * 4 + r][lane]
+    for (uint32_t w = 0; w < 4; ++w) {
+        __syncthreads();
+        if (wave != w) continue;
+#pragma unroll
+        for (int g = 0; g < GROUP; ++g)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                float mine = 1.f, theirs = 0.f;
+                if (w > 0) {
+                    const float mo = ml[(g * QT + 4 * lg + r) * 2], lo_ = ml[(g * QT + 4 * lg + r) * 2 + 1];
+                    const float M = fmaxf(m[g][r], mo);
+                    mine = m[g][r] == -INFINITY ? 0.f : expf(m[g][r] - M);
+                    theirs = mo == -INFINITY ? 0.f : expf(mo - M);
+                    l[g][r] = l[g][r] * mine + lo_ * theirs;
+                    m[g][r] = M;
+                }
+#pragma unroll
+                for (int dt = 0; dt < 16; ++dt) {
+                    float* slot = ob + (((g * 16 + dt) * 4 + r) * 64 + lane);
+                    const float v = O[g][dt][r] * mine + (w > 0 ? *slot * theirs : 0.f);
+                    *slot = v;
+                }
+            }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        if (j == 0) {
+#pragma unroll
+            for (int g = 0; g < GROUP; ++g)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    ml[(g * QT + 4 * lg + r) * 2] = m[g][r];
+                    ml[(g * QT + 4 * lg + r) * 2 + 1] = l[g][r];
+                }
+        }
+    }
+    __syncthreads();
+    for (uint32_t idx = threadIdx.x; idx < GROUP * QT * HD; idx += 256) {
+        const uint32_t g = idx / (QT * HD), i = (idx / HD) % QT, d = idx % HD;
+        const uint32_t row = r0 + i;
+        if (row >= rows) continue;
+        const float v = ob[((g * 16 + d / 16) * 4 + (i & 3)) * 64 + (d & 15) + 16 * (i >> 2)];
+        out[(size_t(row) * q_heads + kvh * GROUP + g) * HD + d] = v / (ml[(g * QT + i) * 2 + 1] * kProbScale);
+    }
+}
+
 // ring[(position + row) & mask] = run[row] for the rows that survive in a ring of this capacity
 __global__ void publish_run_kernel(const uint4* __restrict__ run_k, const uint4* __restrict__ run_v,
                                    uint4* __restrict__ ring_k, uint4* __restrict__ ring_v, uint32_t rows,
@@ -512,10 +753,27 @@ extern "C" int guffin_hip_prefill_gemm(void* stream, int dtype, const void* tile
     return check_launch("prefill_gemm");
 }
 
+namespace {
+struct ValueSpan { uint32_t first_visible, base32, T; };
+// virtual tokens whose values a run of `rows` rows at `position` can see, padded to whole 32-token tiles
+ValueSpan value_span(uint32_t rows, uint32_t position, uint32_t window) {
+    const uint32_t first = (window && position + 1 > window) ? position + 1 - window : 0;
+    const uint32_t base32 = first & ~31u;
+    return {first, base32, (position + rows - base32 + 31u) & ~31u};
+}
+}  // namespace
+
+extern "C" uint64_t guffin_hip_prefill_attention_workspace_bytes(uint32_t rows, uint32_t position, uint32_t window,
+                                                                 uint32_t kv_heads, uint32_t head_dim) {
+    if (rows == 0 || kv_heads == 0 || head_dim != 256) return 0;
+    return uint64_t(kv_heads) * head_dim * value_span(rows, position, window).T * 2;
+}
+
 extern "C" int guffin_hip_prefill_attention(void* stream, const float* q, const void* ring_k, const void* ring_v,
                                             const void* run_k, const void* run_v, float* out, uint32_t rows,
                                             uint32_t position, uint32_t window, uint32_t ring_mask,
-                                            uint32_t q_heads, uint32_t kv_heads, uint32_t head_dim, float scale) {
+                                            uint32_t q_heads, uint32_t kv_heads, uint32_t head_dim, float scale,
+                                            void* workspace) {
     if (!q || !ring_k || !ring_v || !run_k || !run_v || !out) return fail(GUFFIN_E_ARG, "prefill_attention: null pointer");
     if (rows == 0 || head_dim != 256 || kv_heads == 0 || q_heads % kv_heads != 0)
         return fail(GUFFIN_E_SHAPE, "prefill_attention: head_dim must be 256 and q_heads a multiple of kv_heads");
@@ -523,6 +781,7 @@ extern "C" int guffin_hip_prefill_attention(void* stream, const float* q, const 
     const uint32_t past = window ? (window - 1 < position ? window - 1 : position) : position;  // ring tokens a row can see
     if (past > ring_mask + 1) return fail(GUFFIN_E_CAPACITY, "prefill_attention: the ring does not hold the visible past");
     if (!(scale > 0.f)) return fail(GUFFIN_E_ARG, "prefill_attention: scale must be positive");
+    if (reinterpret_cast<uintptr_t>(workspace) & 15u) return fail(GUFFIN_E_ALIGN, "prefill_attention: workspace must be 16-byte aligned");
     const uint32_t group = q_heads / kv_heads;
     const dim3 grid((rows + 15) / 16, kv_heads), block(256);
     hipStream_t s = as_stream(stream);
@@ -530,6 +789,24 @@ extern "C" int guffin_hip_prefill_attention(void* stream, const float* q, const 
     const uint16_t* rv = static_cast<const uint16_t*>(ring_v);
     const uint16_t* uk = static_cast<const uint16_t*>(run_k);
     const uint16_t* uv = static_cast<const uint16_t*>(run_v);
+    if (workspace && group <= 2 && (reinterpret_cast<uintptr_t>(q) & 15u) == 0
+        && ((reinterpret_cast<uintptr_t>(ring_k) | reinterpret_cast<uintptr_t>(run_k) | reinterpret_cast<uintptr_t>(ring_v)
+             | reinterpret_cast<uintptr_t>(run_v)) & 15u) == 0) {
+        // matrix-core path: V^T first, then scores and values as MFMA chains
+        const ValueSpan vs = value_span(rows, position, window);
+        uint16_t* vt = static_cast<uint16_t*>(workspace);
+        hipLaunchKernelGGL(transpose_values_kernel, dim3(vs.T / 32, kv_heads), dim3(256), 0, s, rv, uv, vt, vs.base32, vs.T,
+                           vs.first_visible, position, position + rows, ring_mask, kv_heads);
+        if (int rc = check_launch("transpose_values")) return rc;
+        const size_t lds = size_t(group) * 16384 + size_t(4) * group * 16 * 32 * 4 + size_t(group) * 16 * 2 * 4;
+        if (group == 1)
+            hipLaunchKernelGGL(prefill_attention_mfma_kernel<1>, grid, block, lds, s, q, rk, uk, vt, out, rows, position, window,
+                               ring_mask, q_heads, kv_heads, scale, vs.base32, vs.T);
+        else
+            hipLaunchKernelGGL(prefill_attention_mfma_kernel<2>, grid, block, lds, s, q, rk, uk, vt, out, rows, position, window,
+                               ring_mask, q_heads, kv_heads, scale, vs.base32, vs.T);
+        return check_launch("prefill_attention_mfma");
+    }
 #define GUFFIN_PA(G_) hipLaunchKernelGGL(prefill_attention_kernel<G_>, grid, block, 0, s, q, rk, rv, uk, uv, out, rows, \
                                          position, window, ring_mask, q_heads, kv_heads, scale)
     if (group == 1) GUFFIN_PA(1); else if (group == 2) GUFFIN_PA(2); else if (group == 4) GUFFIN_PA(4);

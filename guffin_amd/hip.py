@@ -439,12 +439,17 @@ def prefill_gemm(dtype, tiles, image, M, K, N):
     return y
 
 
-def prefill_attention(q, ring_k, ring_v, run_k, run_v, position, window, ring_mask, q_heads, kv_heads, head_dim, scale):
+def prefill_attention(q, ring_k, ring_v, run_k, run_v, position, window, ring_mask, q_heads, kv_heads, head_dim, scale,
+                      matrix_core=True):
     rows = q.shape[0]
     out = torch.empty_like(q)
+    ws = None
+    if matrix_core:
+        lib().guffin_hip_prefill_attention_workspace_bytes.restype = C.c_uint64
+        ws = _bytes(max(16, lib().guffin_hip_prefill_attention_workspace_bytes(rows, position, window, kv_heads, head_dim)))
     check(lib().guffin_hip_prefill_attention(_stream(), _p(q), _p(ring_k), _p(ring_v), _p(run_k), _p(run_v), _p(out),
                                              rows, position, window, ring_mask, q_heads, kv_heads, head_dim,
-                                             C.c_float(scale)))
+                                             C.c_float(scale), _p(ws)))
     return out
 
 

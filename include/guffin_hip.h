@@ -348,11 +348,17 @@ int guffin_hip_prefill_gemm(void* stream, int dtype, const void* tiles, const vo
 /* Causal GQA attention of `rows` consecutive positions starting at `position`: row r sees the
  * ring for positions below `position` and rows 0..r of the run's own fp16 K/V rows
  * run_k / run_v [rows][kv_heads*head_dim]; window = 0 for global layers, else the sliding
- * window (the last `window` positions including the row's own).  q, out: [rows][q_heads*256]. */
+ * window (the last `window` positions including the row's own).  q, out: [rows][q_heads*256].
+ * workspace: guffin_hip_prefill_attention_workspace_bytes bytes (16-byte aligned) for the
+ * transposed values of the matrix-core path (q_heads / kv_heads <= 2); NULL selects the
+ * vector-unit kernel, which needs none. */
+uint64_t guffin_hip_prefill_attention_workspace_bytes(uint32_t rows, uint32_t position, uint32_t window,
+                                                      uint32_t kv_heads, uint32_t head_dim);
 int guffin_hip_prefill_attention(void* stream, const float* q, const void* ring_k, const void* ring_v,
                                  const void* run_k, const void* run_v, float* out, uint32_t rows,
                                  uint32_t position, uint32_t window, uint32_t ring_mask,
-                                 uint32_t q_heads, uint32_t kv_heads, uint32_t head_dim, float scale);
+                                 uint32_t q_heads, uint32_t kv_heads, uint32_t head_dim, float scale,
+                                 void* workspace);
 /* ring[(position + row) & ring_mask] = run[row] for every row of the run that a ring of this
  * capacity keeps (encode_gemma2_kv_cache_copy, metal_command_context.hpp:170). */
 int guffin_hip_publish_run(void* stream, const void* run_k, const void* run_v, void* ring_k, void* ring_v,

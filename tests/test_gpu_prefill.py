@@ -45,9 +45,11 @@ def test_prefill_gemm_parity(hip, gfo, dtype, K, N, M):
         assert np.all(np.abs(one.astype(np.float64) - y[r]) <= 2e-5 * scale[r])
 
 
+@pytest.mark.parametrize("matrix_core", [True, False])
 @pytest.mark.parametrize("q_heads,kv_heads,rows,position,window,cap", [
-    (16, 8, 40, 100, 0, 256), (16, 8, 21, 300, 64, 128), (4, 1, 33, 0, 0, 64), (4, 1, 50, 17, 32, 64), (2, 2, 5, 3, 0, 16)])
-def test_prefill_attention_matches_double_softmax(hip, q_heads, kv_heads, rows, position, window, cap):
+    (16, 8, 40, 100, 0, 256), (16, 8, 21, 300, 64, 128), (4, 1, 33, 0, 0, 64), (4, 1, 50, 17, 32, 64), (2, 2, 5, 3, 0, 16),
+    (16, 8, 200, 1000, 1024, 1024), (4, 2, 130, 0, 0, 16), (2, 2, 64, 95, 48, 64)])
+def test_prefill_attention_matches_double_softmax(hip, q_heads, kv_heads, rows, position, window, cap, matrix_core):
     import torch
     rng = np.random.default_rng(5)
     hd = 256
@@ -57,7 +59,7 @@ def test_prefill_attention_matches_double_softmax(hip, q_heads, kv_heads, rows, 
     run_k = rng.normal(0, 1, (rows, kv_heads * hd)).astype(np.float16)
     run_v = rng.normal(0, 1, (rows, kv_heads * hd)).astype(np.float16)
     out = hip.prefill_attention(dev(q), dev(ring_k), dev(ring_v), dev(run_k), dev(run_v), position, window, cap - 1,
-                                q_heads, kv_heads, hd, 0.0625).cpu().numpy()
+                                q_heads, kv_heads, hd, 0.0625, matrix_core=matrix_core).cpu().numpy()
     group = q_heads // kv_heads
     want = np.zeros_like(out, dtype=np.float64)
     for r in range(rows):
