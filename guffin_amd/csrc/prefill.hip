@@ -45,7 +45,10 @@ __host__ __device__ constexpr uint32_t block_elems(int dtype) { return dtype == 
 //                                      256-element block when K is a multiple of 256
 // s32  : float [K/32][Mpad]            sum of the group's 32 activations
 // s16  : float [K/16][Mpad]            sums of 16
-struct ImageLayout { size_t mult_off, s32_off, s16_off, bytes; uint32_t mpad; };
+// sumi : half  [K/256][Mpad/8][16][8]   (K % 256 == 0) the 8 group sums of a block as an A operand:
+//                                      same A rows, halves of groups t at {0,2,1,3,4,6,5,7}[t]
+// smul : float [K/256][Mpad]           2^(Es+24) of (row, block) for sumi
+struct ImageLayout { size_t mult_off, s32_off, s16_off, sumi_off, smul_off, bytes; uint32_t mpad; };
 
 __host__ __device__ inline ImageLayout image_layout(uint32_t M, uint32_t K) {
     const uint32_t mpad = (M + kChunkRows - 1) / kChunkRows * kChunkRows;
@@ -54,7 +57,9 @@ __host__ __device__ inline ImageLayout image_layout(uint32_t M, uint32_t K) {
     L.mult_off = size_t(K / 32) * mpad * 128;  // 16 A rows x 64 B per 8 rows = 128 B per row and group
     L.s32_off = L.mult_off + size_t(K / 32) * mpad * 4;
     L.s16_off = L.s32_off + size_t(K / 32) * mpad * 4;
-    L.bytes = L.s16_off + size_t(K / 16) * mpad * 4;
+    L.sumi_off = L.s16_off + size_t(K / 16) * mpad * 4;
+    L.smul_off = L.sumi_off + size_t(K / 256) * mpad * 32;   // 16 A rows x 16 B per 8 rows
+    L.bytes = L.smul_off + size_t(K / 256) * mpad * 4;
     return L;
 }
 
@@ -89,8 +94,26 @@ prefill_pack_kernel(const float* __restrict__ x, uint8_t* __restrict__ blob, uin
     float* s16 = reinterpret_cast<float*>(blob + L.s16_off);
     if (s == 0) { mult[size_t(g) * L.mpad + row] = __uint_as_float((eb + 10u) << 23); s32[size_t(g) * L.mpad + row] = sum32; }
     if ((s & 1u) == 0) s16[size_t(2 * g + (s >> 1)) * L.mpad + row] = sum16;
-    uint32_t hi[4], lo[4];
     constexpr int order[8] = {0, 2, 1, 3, 4, 6, 5, 7};
+    if (K % 256 == 0) {  // the block's 8 group sums as a second small A operand (hi/lo, own exponent)
+        float sm = fabsf(sum32);
+        sm = fmaxf(sm, __shfl_xor(sm, 4, kWave));
+        sm = fmaxf(sm, __shfl_xor(sm, 8, kWave));
+        sm = fmaxf(sm, __shfl_xor(sm, 16, kWave));
+        uint32_t es = __float_as_uint(sm) >> 23;
+        es = es < 14u ? 14u : es > 244u ? 244u : es;
+        if (s == 0) {
+            const float sv = sum32 * __uint_as_float((268u - es) << 23);
+            const _Float16 h = static_cast<_Float16>(sv);
+            const _Float16 l = static_cast<_Float16>(sv - static_cast<float>(h));
+            const uint32_t blk = g >> 3, t8 = g & 7u;
+            uint8_t* rec = blob + L.sumi_off + ((size_t(blk) * (L.mpad / 8) + row / 8) * 16 + 2 * (row % 8)) * 16 + order[t8] * 2;
+            *reinterpret_cast<uint16_t*>(rec) = __builtin_bit_cast(uint16_t, h);
+            *reinterpret_cast<uint16_t*>(rec + 16) = __builtin_bit_cast(uint16_t, l);
+            if (t8 == 0) reinterpret_cast<float*>(blob + L.smul_off)[size_t(blk) * L.mpad + row] = __uint_as_float((es + 10u) << 23);
+        }
+    }
+    uint32_t hi[4], lo[4];
 #pragma unroll
     for (int p = 0; p < 4; ++p) {
         uint32_t hw = 0, lw = 0;
@@ -121,9 +144,6 @@ __device__ __forceinline__ uint32_t pk_mul(uint32_t a, uint32_t b) {
 }
 __device__ __forceinline__ float sbyte(uint32_t w, int i) {
     return i == 0 ? sb0(w) : i == 1 ? sb1(w) : i == 2 ? sb2(w) : sb3(w);
-}
-__device__ __forceinline__ float ubyte(uint32_t w, int i) {
-    return i == 0 ? ub0(w) : i == 1 ? ub1(w) : i == 2 ? ub2(w) : ub3(w);
 }
 
 // what a wave needs of the image for one 32-group: the A operands of its 4 row groups and the
@@ -223,7 +243,7 @@ prefill_gemm_kernel(const uint8_t* __restrict__ tiles, const uint8_t* __restrict
                 load_group(c, b * 8 + 2 * ch + 1, hi);
 #pragma unroll
                 for (int cg = 0; cg < 4; ++cg) {
-                    const uint32_t scw = ch < 2 ? sc_a[cg] : sc_b[cg], mnw = ch < 2 ? mn_a[cg] : mn_b[cg];
+                    const uint32_t scw = ch < 2 ? sc_a[cg] : sc_b[cg];
                     // the scale byte in both 16-bit fields
                     const uint32_t pair_lo = __builtin_amdgcn_perm(0u, scw, (ch & 1) ? 0x0c020c02u : 0x0c000c00u);
                     const uint32_t pair_hi = __builtin_amdgcn_perm(0u, scw, (ch & 1) ? 0x0c030c03u : 0x0c010c01u);
@@ -235,24 +255,37 @@ prefill_gemm_kernel(const uint8_t* __restrict__ tiles, const uint8_t* __restrict
                     const half8_t bhi = as_half8(pk_mul((w0 >> 4) & M, pair_hi), pk_mul((w0 >> 12) & M, pair_hi),
                                                  pk_mul((w1 >> 4) & M, pair_hi), pk_mul((w1 >> 12) & M, pair_hi));
 #pragma unroll
-                    for (int rg = 0; rg < 4; ++rg) {
-                        D[cg][rg] = __builtin_amdgcn_mfma_f32_16x16x32_f16(lo.a[rg], blo, D[cg][rg], 0, 0, 0);
-                        D[cg][rg] = __builtin_amdgcn_mfma_f32_16x16x32_f16(hi.a[rg], bhi, D[cg][rg], 0, 0, 0);
-                    }
-                    const float mn_lo = ubyte(mnw, 2 * (ch & 1)), mn_hi = ubyte(mnw, 2 * (ch & 1) + 1);
-                    add_offset(c.s32, c, b * 8 + 2 * ch, -dmin[cg] * mn_lo, acc[cg]);
-                    add_offset(c.s32, c, b * 8 + 2 * ch + 1, -dmin[cg] * mn_hi, acc[cg]);
+                    for (int rg = 0; rg < 4; ++rg) D[cg][rg] = __builtin_amdgcn_mfma_f32_16x16x32_f16(lo.a[rg], blo, D[cg][rg], 0, 0, 0);
+#pragma unroll
+                    for (int rg = 0; rg < 4; ++rg) D[cg][rg] = __builtin_amdgcn_mfma_f32_16x16x32_f16(hi.a[rg], bhi, D[cg][rg], 0, 0, 0);
                 }
             }
+            // block done: -dmin * sum_g m_g * (sum of group g) as one more MFMA per tile on the sums
+            // image (its 8 halves are k-slice 0; the other k-slices are zero), then one scale step
             GroupOperands blk;
             load_group(c, b * 8, blk);  // the block's multipliers (shared by its 8 groups)
+            const float* smul = reinterpret_cast<const float*>(blob + L.smul_off);
+            half8_t as[4];
+            float2 ms[4];
 #pragma unroll
-            for (int cg = 0; cg < 4; ++cg)
+            for (int rg = 0; rg < 4; ++rg) {
+                uint4 v = *reinterpret_cast<const uint4*>(blob + L.sumi_off + (size_t(b) * (L.mpad / 8) + c.rg0 + rg) * 256 + (lane & 15u) * 16);
+                if (lane >= 16) v = make_uint4(0, 0, 0, 0);
+                as[rg] = __builtin_bit_cast(half8_t, v);
+                ms[rg] = *reinterpret_cast<const float2*>(smul + size_t(b) * L.mpad + c.row0 + 8 * rg);
+            }
+#pragma unroll
+            for (int cg = 0; cg < 4; ++cg) {
+                half8_t bm = as_half8(even_bytes(mn_a[cg]), odd_bytes(mn_a[cg]), even_bytes(mn_b[cg]), odd_bytes(mn_b[cg]));
+                if (lane >= 16) bm = as_half8(0, 0, 0, 0);
 #pragma unroll
                 for (int rg = 0; rg < 4; ++rg) {
-                    acc[cg][rg][0] = fmaf(d[cg] * blk.mult[rg].x, D[cg][rg][0] + D[cg][rg][1], acc[cg][rg][0]);
-                    acc[cg][rg][1] = fmaf(d[cg] * blk.mult[rg].y, D[cg][rg][2] + D[cg][rg][3], acc[cg][rg][1]);
+                    const float4_t dm = __builtin_amdgcn_mfma_f32_16x16x32_f16(as[rg], bm, float4_t{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+                    const float4_t dv = D[cg][rg];
+                    acc[cg][rg][0] = fmaf(d[cg] * blk.mult[rg].x, dv[0] + dv[1], fmaf(-dmin[cg] * ms[rg].x, dm[0] + dm[1], acc[cg][rg][0]));
+                    acc[cg][rg][1] = fmaf(d[cg] * blk.mult[rg].y, dv[2] + dv[3], fmaf(-dmin[cg] * ms[rg].y, dm[2] + dm[3], acc[cg][rg][1]));
                 }
+            }
         } else if constexpr (DTYPE == GUFFIN_Q6_K) {
             // q = lo + 16 hi2 (4 + 2 bits): |scale| * lo <= 1905 and |scale| * hi2 <= 381 are exact as
             // fp16 bit patterns (n < 2048 reads as n * 2^-24) and carry the scale's sign in bit 15, so
