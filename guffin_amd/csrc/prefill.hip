@@ -213,19 +213,36 @@ prefill_gemm_kernel(const uint8_t* __restrict__ tiles, const uint8_t* __restrict
 #pragma unroll
         for (int rg = 0; rg < 4; ++rg) { acc[cg][rg][0] = 0.f; acc[cg][rg][1] = 0.f; }
     const uint8_t* tp = tiles + size_t(blockIdx.x) * nblk * TB;
+    [[maybe_unused]] uint4 qn[8], hn[4];
     for (uint32_t b = 0; b < nblk; ++b, tp += TB) {
         if constexpr (DTYPE == GUFFIN_Q4_K) {
             // sc * q <= 945 is still an exact fp16 subnormal, so the 6-bit scales are folded into B
             // and a whole 256-element block accumulates inside the MFMA chain; d and the block's
             // activation multiplier are applied once per block
-            uint4 q[8];
+            // the next block's quants and headers travel while this block is multiplied
+            uint4 q[8], hd[4];
+            if (b == 0) {
 #pragma unroll
-            for (int i = 0; i < 8; ++i) q[i] = *reinterpret_cast<const uint4*>(tp + 1024 * i + lane * 16);
+                for (int i = 0; i < 8; ++i) q[i] = *reinterpret_cast<const uint4*>(tp + 1024 * i + lane * 16);
+#pragma unroll
+                for (int cg = 0; cg < 4; ++cg) hd[cg] = *reinterpret_cast<const uint4*>(tp + 8192 + (16 * cg + j) * 16);
+            } else {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) q[i] = qn[i];
+#pragma unroll
+                for (int cg = 0; cg < 4; ++cg) hd[cg] = hn[cg];
+            }
+            if (b + 1 < nblk) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) qn[i] = *reinterpret_cast<const uint4*>(tp + TB + 1024 * i + lane * 16);
+#pragma unroll
+                for (int cg = 0; cg < 4; ++cg) hn[cg] = *reinterpret_cast<const uint4*>(tp + TB + 8192 + (16 * cg + j) * 16);
+            }
             float d[4], dmin[4];
             uint32_t sc_a[4], sc_b[4], mn_a[4], mn_b[4];
 #pragma unroll
             for (int cg = 0; cg < 4; ++cg) {
-                const uint4 hdr = *reinterpret_cast<const uint4*>(tp + 8192 + (16 * cg + j) * 16);
+                const uint4 hdr = hd[cg];
                 d[cg] = h2f(hdr.x & 0xFFFFu); dmin[cg] = h2f(hdr.x >> 16);
                 sc_a[cg] = hdr.y & 0x3F3F3F3Fu; mn_a[cg] = hdr.z & 0x3F3F3F3Fu;
                 sc_b[cg] = (hdr.w & 0x0F0F0F0Fu) | ((hdr.y >> 2) & 0x30303030u);
