@@ -11,6 +11,7 @@
 // Like the reference's command context it allocates nothing: weights, KV rings and the
 // scratch arena are the caller's; everything is enqueued in order on one HIP stream, so a
 // caller can capture a whole step into a HIP graph.
+#include <cstddef>
 #include "common.hpp"
 #include "receipt.hpp"
 
@@ -569,9 +570,12 @@ extern "C" int guffin_hip_session_submit(void* stream, guffin_h1_session* s) {
     if (s->state == GUFFIN_TXN_POISONED) return fail(GUFFIN_E_STATE, "session_submit: the session is poisoned");
     if (s->state != GUFFIN_TXN_IDLE) return fail(GUFFIN_E_STATE, "session_submit: a cycle is already in flight");
     hipStream_t hs = as_stream(stream);
-    const uint32_t words[2] = {s->root, s->pending}, zero = 0;
-    if (hipMemcpyAsync(s->tokens, words, sizeof(words), hipMemcpyHostToDevice, hs) != hipSuccess
-        || hipMemcpyAsync(s->status, &zero, sizeof(zero), hipMemcpyHostToDevice, hs) != hipSuccess)
+    // sources that outlive the call: root and pending are adjacent fields of the session
+    static const uint32_t kZero = 0;
+    static_assert(offsetof(guffin_h1_session, pending) == offsetof(guffin_h1_session, root) + sizeof(uint32_t),
+                  "root and pending are uploaded as one pair");
+    if (hipMemcpyAsync(s->tokens, &s->root, 2 * sizeof(uint32_t), hipMemcpyHostToDevice, hs) != hipSuccess
+        || hipMemcpyAsync(s->status, &kZero, sizeof(kZero), hipMemcpyHostToDevice, hs) != hipSuccess)
         return fail(GUFFIN_E_HIP, "session_submit: upload failed");
     s->desc.drafter_rows = s->has_pending ? 2u : 1u;
     s->desc.pending_token = s->tokens + 1;
