@@ -17,7 +17,7 @@ FLAGS = [
 
 
 def _compile(src):
-    obj = os.path.join(OBJ, os.path.basename(src).replace(".hip", ".o"))
+    obj = os.path.join(OBJ, os.path.splitext(os.path.basename(src))[0] + ".o")
     cmd = [HIPCC, *FLAGS, "-c", src, "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
@@ -27,7 +27,7 @@ def _compile(src):
 
 def build(verbose=False):
     os.makedirs(OBJ, exist_ok=True)
-    sources = sorted(glob.glob(os.path.join(CSRC, "*.hip")))
+    sources = sorted(glob.glob(os.path.join(CSRC, "*.hip")) + glob.glob(os.path.join(CSRC, "*.cpp")))  # .cpp: host only
     with concurrent.futures.ThreadPoolExecutor(max_workers=8) as pool:
         results = list(pool.map(_compile, sources))
     objs = [o for o, _ in results]

@@ -223,6 +223,85 @@ class DeviceModel:
         torch.cuda.synchronize()
         return self._finish(embed, head, torch.from_numpy(host.out_norm).cuda())
 
+    # GGUF tensor names of a Gemma block in the order of LayerDesc.tiles / LayerDesc.norm
+    # (src/engine/gemma_model.cpp:36-72 of the reference)
+    GGUF_MATRICES = ("attn_q", "attn_k", "attn_v", "attn_output", "ffn_gate", "ffn_up", "ffn_down")
+    GGUF_NORMS = ("attn_norm", "attn_q_norm", "attn_k_norm", "post_attention_norm", "ffn_norm", "post_ffw_norm")
+    GGUF_TYPES = {8: Q8_0, 12: Q4_K, 14: Q6_K}
+
+    @classmethod
+    def from_gguf(cls, reader, ring_local=None, ring_global=8192, arch="gemma3"):
+        """Binds a parsed GGUF file (guffin_amd.gguf.Reader): shape from the `<arch>.*` metadata keys
+        (src/engine/model.cpp:330-390), matrices uploaded as they lie in the file ([input, output] with
+        the input dimension contiguous, i.e. blocks per output column) and repacked on the device, tied
+        head when there is no output.weight.  Rings start empty."""
+        md = reader.metadata()
+        key = lambda k: md[arch + "." + k]
+        scale = 1.0
+        if md.get(arch + ".rope.scaling.type", "none") == "linear":
+            scale = 1.0 / float(key("rope.scaling.factor"))
+        embed_info = reader.tensor("token_embd.weight")
+        hidden, vocab = embed_info["dims"]
+        if hidden != key("embedding_length"):
+            raise ValueError("token_embd.weight does not match " + arch + ".embedding_length")
+        layers = int(key("block_count"))
+
+        def matrix_type(name):
+            t = reader.tensor(name)["type_id"]
+            if t not in cls.GGUF_TYPES:
+                raise ValueError("%s: tensor type %d is not a supported block format" % (name, t))
+            return cls.GGUF_TYPES[t]
+
+        window = int(key("attention.sliding_window"))
+        shape = Shape(hidden=hidden, ffn=int(key("feed_forward_length")), q_heads=int(key("attention.head_count")),
+                      kv_heads=int(key("attention.head_count_kv")), head_dim=int(key("attention.key_length")),
+                      layers=layers, vocab=vocab, sliding_window=window,
+                      global_period=int(md.get(arch + ".attention.sliding_window_pattern", 6)),
+                      local_base=float(md.get(arch + ".rope.freq_base_swa", 10000.0)),
+                      global_base=float(key("rope.freq_base")), global_scale=scale,
+                      ring_local=ring_local or 1 << (window - 1).bit_length(), ring_global=ring_global,
+                      dtypes=tuple(matrix_type("blk.0.%s.weight" % m) for m in cls.GGUF_MATRICES),
+                      embed_dtype=matrix_type("token_embd.weight"),
+                      eps=float(key("attention.layer_norm_rms_epsilon")))
+        self = cls(shape)
+
+        def upload(name):
+            return torch.from_numpy(np.array(reader.payload(name))).cuda()   # staged through a writable copy
+
+        def norm(name, width):
+            t = reader.tensor(name)
+            if t["type_id"] != 0 or t["dims"] != [width]:
+                raise ValueError("%s: expected an F32 norm of width %d" % (name, width))
+            return upload(name).view(torch.float32)
+
+        widths = [hidden, shape.head_dim, shape.head_dim, hidden, hidden, hidden]
+        for l in range(layers):
+            for i, (m, (K, N)) in enumerate(zip(cls.GGUF_MATRICES, shape.proj_shapes())):
+                name = "blk.%d.%s.weight" % (l, m)
+                t = reader.tensor(name)
+                if t["dims"] != [K, N] or matrix_type(name) != shape.dtypes[i]:
+                    raise ValueError("%s: expected a [%d, %d] matrix of the block format of block 0" % (name, K, N))
+                tiles = hip.repack(shape.dtypes[i], upload(name), K, N)
+                self.keep.append(tiles)
+                self.layers[l].dtype[i] = shape.dtypes[i]
+                self.layers[l].tiles[i] = tiles.data_ptr()
+            for i, (n, w) in enumerate(zip(cls.GGUF_NORMS, widths)):
+                g = norm("blk.%d.%s.weight" % (l, n), w)
+                self.keep.append(g)
+                self.layers[l].norm[i] = g.data_ptr()
+            cap = shape.ring_local if shape.is_local(l) else shape.ring_global
+            rk = torch.zeros((cap, shape.kv_width), dtype=torch.float16, device="cuda")
+            rv = torch.zeros_like(rk)
+            self.ring_k.append(rk)
+            self.ring_v.append(rv)
+            self.layers[l].ring_k, self.layers[l].ring_v = rk.data_ptr(), rv.data_ptr()
+        embed = upload("token_embd.weight")
+        head_name = "output.weight" if any(t["name"] == "output.weight" for t in reader.tensors()) else "token_embd.weight"
+        head = hip.repack(matrix_type(head_name), embed if head_name == "token_embd.weight" else upload(head_name),
+                          hidden, vocab)
+        torch.cuda.synchronize()
+        return self._finish(embed, head, norm("output_norm.weight", hidden))
+
     @classmethod
     def random(cls, shape, seed, position):
         """Weights drawn on the device (full-size benchmark: no host copy of the 7 GB)."""

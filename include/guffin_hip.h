@@ -401,6 +401,67 @@ int guffin_hip_h1_buffers(const guffin_h1_desc* desc, void* scratch, float** dra
 /* The full-vocabulary table of the last step (desc->full_law != 0), else NULL. */
 int guffin_hip_h1_full_cdf(const guffin_h1_desc* desc, void* scratch, uint64_t** full_cdf);
 
+/* ---- GGUF container reader (host only) ---------------------------------------------------
+ * The validating reader of src/model_format/gguf_reader.cpp (types in
+ * include/local_gguf_engine/model_format/gguf_{header,metadata,tensor,reader}.hpp): one pass over
+ * the caller's bytes up to `stage` — the depths the reference exposes as read_gguf_header,
+ * read_gguf_metadata_section, read_gguf_tensor_directory and read_gguf_model_view.  The handle
+ * keeps keys, names and scalar values; tensor payloads are (file_offset, byte_count) views into
+ * the caller's bytes, which must outlive the handle.  guffin_gguf_open returns 0, a GUFFIN_E_*
+ * argument error, or one of the reader's error codes below (GGUFReadErrorCode, same order), with
+ * the reference's expected / actual counts and the offending magic from guffin_gguf_last_failure
+ * (per thread).  Tensor types: 0 F32, 1 F16, 8 Q8_0, 12 Q4_K, 14 Q6_K; names up to 64 bytes, up to
+ * 4 dimensions, general.alignment a non-zero uint32 multiple of 8 (default 32), zero padding. */
+#define GUFFIN_GGUF_TRUNCATED_HEADER (-100)
+#define GUFFIN_GGUF_INVALID_MAGIC (-101)
+#define GUFFIN_GGUF_TRUNCATED_METADATA (-102)
+#define GUFFIN_GGUF_INVALID_METADATA_VALUE_TYPE (-103)
+#define GUFFIN_GGUF_INVALID_METADATA_VALUE (-104)
+#define GUFFIN_GGUF_UNSUPPORTED_METADATA_VALUE_TYPE (-105)
+#define GUFFIN_GGUF_TRUNCATED_TENSOR_DIRECTORY (-106)
+#define GUFFIN_GGUF_INVALID_TENSOR_DIMENSION_COUNT (-107)
+#define GUFFIN_GGUF_INVALID_TENSOR_NAME (-108)
+#define GUFFIN_GGUF_INVALID_ALIGNMENT (-109)
+#define GUFFIN_GGUF_INVALID_TENSOR_OFFSET (-110)
+#define GUFFIN_GGUF_INVALID_TENSOR_PADDING (-111)
+#define GUFFIN_GGUF_TRUNCATED_TENSOR_PAYLOAD (-112)
+#define GUFFIN_GGUF_UNSUPPORTED_TENSOR_TYPE (-113)
+#define GUFFIN_GGUF_INVALID_TENSOR_SIZE (-114)
+#define GUFFIN_GGUF_STAGE_HEADER 0
+#define GUFFIN_GGUF_STAGE_METADATA 1
+#define GUFFIN_GGUF_STAGE_DIRECTORY 2
+#define GUFFIN_GGUF_STAGE_MODEL 3
+typedef struct guffin_gguf guffin_gguf;
+typedef struct guffin_gguf_info {
+    uint32_t version, alignment;
+    uint64_t tensor_count, metadata_kv_count;   /* as the header states them */
+    uint64_t metadata_end_offset, tensor_infos_end_offset, padding_byte_count, tensor_data_start_offset;
+    uint64_t parsed_entries, parsed_tensors;    /* what this handle holds for its stage */
+} guffin_gguf_info;
+typedef struct guffin_gguf_entry_info {
+    const char* key;
+    uint32_t type, element_type;   /* GGUFMetadataValueType; element_type for arrays (type 9) */
+    uint64_t bits;                 /* scalars: the little-endian value (floats by bit pattern, bool 0 / 1) */
+    const char* text; uint64_t text_bytes;   /* strings (type 8) */
+    uint64_t count;                /* arrays: number of elements */
+} guffin_gguf_entry_info;
+typedef struct guffin_gguf_tensor_info {
+    const char* name;
+    uint32_t n_dims, type_id;
+    uint64_t dims[4];
+    uint64_t offset, file_offset, byte_count;   /* byte_count is set from GUFFIN_GGUF_STAGE_MODEL on */
+} guffin_gguf_tensor_info;
+int guffin_gguf_open(const void* bytes, uint64_t size, int stage, guffin_gguf** out);
+void guffin_gguf_close(guffin_gguf* gguf);
+void guffin_gguf_last_failure(uint64_t* expected, uint64_t* actual, uint8_t magic[4]);
+int guffin_gguf_summary(const guffin_gguf* gguf, guffin_gguf_info* out);
+int guffin_gguf_entry(const guffin_gguf* gguf, uint64_t index, guffin_gguf_entry_info* out);
+int guffin_gguf_entry_element(const guffin_gguf* gguf, uint64_t index, uint64_t element, uint64_t* bits,
+                              const char** text, uint64_t* text_bytes);
+int guffin_gguf_find_entry(const guffin_gguf* gguf, const char* key, uint64_t* index);
+int guffin_gguf_tensor(const guffin_gguf* gguf, uint64_t index, guffin_gguf_tensor_info* out);
+int guffin_gguf_find_tensor(const guffin_gguf* gguf, const char* name, uint64_t* index);
+
 /* ---- consecutive cycles ---------------------------------------------------------------------
  * Host-side lifecycle around guffin_hip_h1_step for generation over many cycles.  It keeps what
  * the reference keeps between cycles: the verify pass's transaction state (VerifierTransactionState,
