@@ -142,6 +142,12 @@ typedef unsigned short ushort2_t __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ uint32_t pk_mul(uint32_t a, uint32_t b) {
     return __builtin_bit_cast(uint32_t, __builtin_bit_cast(ushort2_t, a) * __builtin_bit_cast(ushort2_t, b));
 }
+// a * b + c on both 16-bit fields
+__device__ __forceinline__ uint32_t pk_mad(uint32_t a, uint32_t b, uint32_t c) {
+    uint32_t r;
+    asm("v_pk_mad_u16 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
 __device__ __forceinline__ float sbyte(uint32_t w, int i) {
     return i == 0 ? sb0(w) : i == 1 ? sb1(w) : i == 2 ? sb2(w) : sb3(w);
 }
@@ -348,10 +354,11 @@ prefill_gemm_kernel(const uint8_t* __restrict__ tiles, const uint8_t* __restrict
 #pragma unroll
                         for (int k = 0; k < 2; ++k) {
                             const uint32_t w = k ? w1 : w0, h = k ? h1 : h0;
-                            bl[2 * k] = pk_mul((w >> ls) & 0x000F000Fu, pair) | sign;
-                            bl[2 * k + 1] = pk_mul((w >> (ls + 8)) & 0x000F000Fu, pair) | sign;
-                            bh[2 * k] = pk_mul((h >> (2 * qd)) & 0x00030003u, pair) | sign;
-                            bh[2 * k + 1] = pk_mul((h >> (8 + 2 * qd)) & 0x00030003u, pair) | sign;
+                            // the products stay below 2^11, so adding the sign bit sets it
+                            bl[2 * k] = pk_mad((w >> ls) & 0x000F000Fu, pair, sign);
+                            bl[2 * k + 1] = pk_mad((w >> (ls + 8)) & 0x000F000Fu, pair, sign);
+                            bh[2 * k] = pk_mad((h >> (2 * qd)) & 0x00030003u, pair, sign);
+                            bh[2 * k + 1] = pk_mad((h >> (8 + 2 * qd)) & 0x00030003u, pair, sign);
                         }
                         const half8_t blo = as_half8(bl[0], bl[1], bl[2], bl[3]), bhi = as_half8(bh[0], bh[1], bh[2], bh[3]);
 #pragma unroll
