@@ -22,6 +22,9 @@
 namespace guffin {
 namespace {
 
+// history window of the reference's sampler (token_sampler history, 64 tokens)
+constexpr uint32_t kHistoryWindow = 64;
+
 struct Arena {
     uint8_t* base; uint64_t used, capacity;
     template <typename T> T* take(uint64_t count) {
@@ -228,6 +231,17 @@ __global__ void commit_rows_kernel(const uint16_t* priv_k, const uint16_t* priv_
     }
 }
 
+// row 0 keeps the caller's history, row 1 the same plus the proposal (oldest dropped at 64)
+__global__ void build_history_kernel(const uint32_t* history, uint32_t count, const uint32_t* proposal, uint32_t* out) {
+    const uint32_t t = threadIdx.x;
+    const uint32_t drop = count == kHistoryWindow ? 1u : 0u, count1 = count + 1 - drop;
+    if (t < kHistoryWindow) {
+        out[t] = t < count ? history[t] : 0u;
+        out[kHistoryWindow + t] = t + 1 < count1 ? history[t + drop] : (t + 1 == count1 ? *proposal : 0u);
+    }
+    if (t == 0) { out[2 * kHistoryWindow] = count; out[2 * kHistoryWindow + 1] = count1; }
+}
+
 // the step's token slots: [0] root, [1] proposal (written later), [8..] the drafter's input rows
 __global__ void set_step_tokens_kernel(const uint32_t* root, const uint32_t* pending, uint32_t* words) {
     words[0] = *root;
@@ -385,6 +399,7 @@ struct StepBuffers {
     float *d_hidden, *t_hidden, *q_parts, *q_logits, *p_parts, *p_logits;
     uint8_t *law_ws, *sel_ws, *law, *cands, *any_ws;
     uint32_t* words;
+    uint32_t* hist;      // [2][64] sampler history of the two verify rows, then their two counts
     uint64_t* full_cdf;
 };
 // rows the drafter ingests: the root alone, or the accepted proposal it still owes and the root
@@ -408,10 +423,11 @@ StepBuffers carve_step(const guffin_h1_desc* d, void* scratch) {
     b.p_parts = ar.take<float>(uint64_t(slices(T.head_dtype, T.hidden, V)) * 2 * V);
     b.p_logits = ar.take<float>(2 * V);
     b.law_ws = ar.take<uint8_t>(guffin_hip_draft_law_workspace_bytes(D.vocab));
-    b.sel_ws = ar.take<uint8_t>(guffin_hip_select_workspace_bytes(2, V, d->top_k));
+    b.sel_ws = ar.take<uint8_t>(guffin_hip_select_workspace_bytes(2, V, d->top_k + kHistoryWindow));
     b.law = ar.take<uint8_t>(4096 + 2 * 3088);  // the compact law, then the two candidate rows
     b.cands = b.law ? b.law + 4096 : nullptr;
     b.words = ar.take<uint32_t>(16);
+    b.hist = ar.take<uint32_t>(2 * 64 + 2);
     if (d->full_law) {
         b.any_ws = ar.take<uint8_t>(guffin_hip_draft_law_any_workspace_bytes(D.vocab));
         b.full_cdf = ar.take<uint64_t>(uint64_t(D.vocab) + 1);
@@ -454,8 +470,11 @@ extern "C" int guffin_hip_h1_step(void* stream, const guffin_h1_desc* d, const u
     uint32_t* sel_status = B.words + 4;  // per-row selection status
     hipStream_t s = as_stream(stream);
 
+    const bool with_history = d->history != nullptr && d->history_count > 0;
+    if (d->history_count > kHistoryWindow) return fail(GUFFIN_E_CAPACITY, "h1_step: at most 64 history tokens");
+    if (with_history && !(d->repetition_penalty > 0.f)) return fail(GUFFIN_E_ARG, "h1_step: the repetition penalty must be positive");
     struct { float temperature; uint32_t top_k; float top_p, min_p, repetition_penalty; } opt
-        = {d->temperature, d->top_k, d->top_p, d->min_p, 1.0f};
+        = {d->temperature, d->top_k, d->top_p, d->min_p, with_history ? d->repetition_penalty : 1.0f};
 
     // 1. drafter: ingest (the pending proposal and) the root, project, build the proposal law, pick x
     const uint32_t dr = drafter_rows(d);
@@ -479,10 +498,22 @@ extern "C" int guffin_hip_h1_step(void* stream, const guffin_h1_desc* d, const u
                                        target_priv_v, t_hidden, t_hidden + hidden_receipt_offset(2, T.hidden), status));
     GUFFIN_TRY(guffin_hip_gemv_packed(stream, T.head_dtype, T.head_tiles, t_hidden, t_hidden + hidden_receipt_offset(2, T.hidden), p_parts,
                                       p_logits, 2, T.hidden, V));
-    GUFFIN_TRY(guffin_hip_select_candidates(stream, p_logits, 2, V, d->top_k, nullptr, nullptr, sel_ws, cands, sel_status));
+    // candidates: the top_k best plus one per history token (a penalised token can fall out of the
+    // top_k, src/engine/sampling.cpp:430-446), then the history tokens' own logits
+    uint32_t retain = d->top_k;
+    const uint32_t* hist = nullptr;
+    if (with_history) {
+        hipLaunchKernelGGL(build_history_kernel, dim3(1), dim3(64), 0, s, d->history, d->history_count, tokens + 1, B.hist);
+        GUFFIN_TRY(check_launch("build_history"));
+        hist = B.hist;
+        retain = std::min<uint64_t>(V, uint64_t(d->top_k) + std::min(d->history_count + 1, kHistoryWindow));
+    }
+    GUFFIN_TRY(guffin_hip_select_candidates(stream, p_logits, 2, V, retain, hist, hist ? hist + 2 * kHistoryWindow : nullptr,
+                                            sel_ws, cands, sel_status));
     // 3. accept x or draw from the residual; on acceptance draw the next root from row 1
-    GUFFIN_TRY(guffin_hip_spec_accept_law(stream, cands, law, full_cdf, D.vocab, tokens + 1, &opt, d->seed, d->step,
-                                          nullptr, result, status));
+    GUFFIN_TRY(guffin_hip_spec_accept_history(stream, cands, law, full_cdf, D.vocab, hist,
+                                              hist ? hist + 2 * kHistoryWindow : nullptr, tokens + 1, &opt, d->seed, d->step,
+                                              nullptr, result, status));
     // 4. publish: the target keeps row 0, and row 1 if x was accepted; the drafter keeps the root
     if (d->target_ring_k && d->target_ring_v) {
         GUFFIN_TRY(guffin_hip_commit_rows(stream, &T, target_priv_k, target_priv_v, d->target_ring_k, d->target_ring_v,

@@ -553,7 +553,8 @@ __device__ uint64_t law_mass(const DraftLaw* law, const uint64_t* full_cdf, uint
 
 __global__ void __launch_bounds__(512)
 spec_accept_kernel(const Candidates* __restrict__ rows, const DraftLaw* __restrict__ law,
-                   const uint64_t* __restrict__ full_cdf, uint32_t vocab, const uint32_t* __restrict__ proposal_ptr, SamplerOptions opt, uint64_t seed, uint64_t step,
+                   const uint64_t* __restrict__ full_cdf, uint32_t vocab, const uint32_t* __restrict__ history,
+                   const uint32_t* __restrict__ history_count, const uint32_t* __restrict__ proposal_ptr, SamplerOptions opt, uint64_t seed, uint64_t step,
                    const StepDraws* __restrict__ injected, SpecResult* __restrict__ result,
                    uint32_t* __restrict__ status) {
     __shared__ Scratch sc;
@@ -569,7 +570,8 @@ spec_accept_kernel(const Candidates* __restrict__ rows, const DraftLaw* __restri
         result->acceptance_probability = 0.0; result->residual_total = 0.0; result->residual_count = 0;
         result->proposal = proposal;
     }
-    int rc = prepare_distribution(&rows[0], opt, nullptr, 0, sc, target);
+    // history: [2][64] token ids and their counts per row (null: no repetition history)
+    int rc = prepare_distribution(&rows[0], opt, history, history ? history_count[0] : 0u, sc, target);
     if (!rc && t < target.count) q[t] = law_mass(law, full_cdf, vocab, target.token[t], nullptr);
     __syncthreads();
     if (t == 0) {
@@ -630,7 +632,7 @@ spec_accept_kernel(const Candidates* __restrict__ rows, const DraftLaw* __restri
     __syncthreads();
     if (s_code == 0 && s_accepted) {
         // a fully accepted chain leaves row 1's candidates to seed the next root
-        rc = prepare_distribution(&rows[1], opt, nullptr, 0, sc, target);
+        rc = prepare_distribution(&rows[1], opt, history ? history + 64 : nullptr, history ? history_count[1] : 0u, sc, target);
         if (t == 0) {
             if (rc) s_code = rc - 100;
             else result->next_root = opt.temperature == 0.f ? target.token[0]
@@ -780,17 +782,27 @@ extern "C" int guffin_hip_draft_law_any(void* stream, const float* logits, uint3
     return launch_full_law(s, logits, vocab, opt, seed, step, injected_draws, nullptr, ws, full_cdf, proposal, status);
 }
 
+extern "C" int guffin_hip_spec_accept_history(void* stream, const void* target_candidates, const void* law,
+                                              const uint64_t* full_cdf, uint32_t vocab, const uint32_t* history,
+                                              const uint32_t* history_count, const uint32_t* proposal,
+                                              const void* options, uint64_t seed, uint64_t step,
+                                              const void* injected_draws, void* result, uint32_t* status) {
+    if (!target_candidates || !law || !proposal || !options || !result) return fail(GUFFIN_E_ARG, "spec_accept: null pointer");
+    if ((history == nullptr) != (history_count == nullptr)) return fail(GUFFIN_E_ARG, "spec_accept: history needs its counts");
+    const SamplerOptions opt = *static_cast<const SamplerOptions*>(options);
+    hipLaunchKernelGGL(spec_accept_kernel, dim3(1), dim3(512), 0, as_stream(stream),
+                       static_cast<const Candidates*>(target_candidates), static_cast<const DraftLaw*>(law), full_cdf,
+                       vocab, history, history_count, proposal, opt, seed, step,
+                       static_cast<const StepDraws*>(injected_draws), static_cast<SpecResult*>(result), status);
+    return check_launch("spec_accept");
+}
+
 extern "C" int guffin_hip_spec_accept_law(void* stream, const void* target_candidates, const void* law,
                                           const uint64_t* full_cdf, uint32_t vocab, const uint32_t* proposal,
                                           const void* options, uint64_t seed, uint64_t step,
                                           const void* injected_draws, void* result, uint32_t* status) {
-    if (!target_candidates || !law || !proposal || !options || !result) return fail(GUFFIN_E_ARG, "spec_accept: null pointer");
-    const SamplerOptions opt = *static_cast<const SamplerOptions*>(options);
-    hipLaunchKernelGGL(spec_accept_kernel, dim3(1), dim3(512), 0, as_stream(stream),
-                       static_cast<const Candidates*>(target_candidates), static_cast<const DraftLaw*>(law), full_cdf,
-                       vocab, proposal, opt, seed, step, static_cast<const StepDraws*>(injected_draws),
-                       static_cast<SpecResult*>(result), status);
-    return check_launch("spec_accept");
+    return guffin_hip_spec_accept_history(stream, target_candidates, law, full_cdf, vocab, nullptr, nullptr, proposal,
+                                          options, seed, step, injected_draws, result, status);
 }
 
 extern "C" int guffin_hip_spec_accept(void* stream, const void* target_candidates, const void* law,

@@ -398,6 +398,15 @@ def spec_accept_law(cands, law, cdf, proposal, options, seed=0, step=0, draws=No
     return result
 
 
+def spec_accept_history(cands, law, history, history_count, proposal, options, seed=0, step=0, draws=None, status=None):
+    """history: int32 [2, 64] token ids, history_count: int32 [2] (device tensors)."""
+    result = _bytes(result_dtype.itemsize)
+    check(lib().guffin_hip_spec_accept_history(_stream(), _p(cands), _p(law), None, 0, _p(history), _p(history_count),
+                                               _p(proposal), C.byref(options), C.c_uint64(seed), C.c_uint64(step),
+                                               _p(draws), _p(result), _p(status)))
+    return result
+
+
 def spec_accept(cands, law, proposal, options, seed=0, step=0, draws=None, result=None, status=None):
     if result is None:
         result = _bytes(result_dtype.itemsize)

@@ -39,7 +39,8 @@ class H1Desc(C.Structure):
                 ("seed", C.c_uint64), ("step", C.c_uint64),
                 ("target_ring_k", C.c_void_p), ("target_ring_v", C.c_void_p),
                 ("drafter_ring_k", C.c_void_p), ("drafter_ring_v", C.c_void_p), ("full_law", C.c_uint32),
-                ("drafter_rows", C.c_uint32), ("pending_token", C.c_void_p)]
+                ("drafter_rows", C.c_uint32), ("pending_token", C.c_void_p),
+                ("history", C.c_void_p), ("history_count", C.c_uint32), ("repetition_penalty", C.c_float)]
 
 
 class H1Session(C.Structure):
@@ -394,7 +395,7 @@ class H1Plan:
     """One speculative cycle: buffers, descriptor and the call into guffin_hip_h1_step."""
 
     def __init__(self, target, drafter, target_position, drafter_position, temperature=1.0, top_k=64,
-                 top_p=0.95, min_p=0.0, seed=0, publish=True, full_law=False):
+                 top_p=0.95, min_p=0.0, seed=0, publish=True, full_law=False, history=None, repetition_penalty=1.0):
         self.target, self.drafter = target, drafter
         d = self.desc = H1Desc()
         d.target, d.drafter = C.pointer(target.desc), C.pointer(drafter.desc)
@@ -402,6 +403,9 @@ class H1Plan:
         d.temperature, d.top_k, d.top_p, d.min_p = temperature, top_k, top_p, min_p
         d.seed, d.step = seed, 0
         d.full_law = 1 if full_law else 0
+        if history is not None:
+            self.history = torch.tensor(list(history), dtype=torch.int32, device="cuda")
+            d.history, d.history_count, d.repetition_penalty = self.history.data_ptr(), len(history), repetition_penalty
         if publish:
             d.target_ring_k, d.target_ring_v = target.ring_k_table.data_ptr(), target.ring_v_table.data_ptr()
             d.drafter_ring_k, d.drafter_ring_v = drafter.ring_k_table.data_ptr(), drafter.ring_v_table.data_ptr()

@@ -288,6 +288,15 @@ int guffin_hip_spec_accept_law(void* stream, const void* target_candidates, cons
                                const uint64_t* full_cdf, uint32_t vocab, const uint32_t* proposal,
                                const void* options, uint64_t seed, uint64_t step,
                                const void* injected_draws, void* result, uint32_t* status);
+/* The same decision with the sampler history of each row (SamplerHistorySnapshot of the reference:
+ * the tokens the repetition penalty of `options` applies to, src/engine/sampling.cpp:430-446):
+ * history [2][64] token ids, history_count [2], both on the device; the candidate rows must carry
+ * the history tokens' logits (guffin_hip_select_candidates with the same history). */
+int guffin_hip_spec_accept_history(void* stream, const void* target_candidates, const void* law,
+                                   const uint64_t* full_cdf, uint32_t vocab, const uint32_t* history,
+                                   const uint32_t* history_count, const uint32_t* proposal,
+                                   const void* options, uint64_t seed, uint64_t step,
+                                   const void* injected_draws, void* result, uint32_t* status);
 /* Host evaluation of the draw schedule above (out: the draws struct). */
 int guffin_hip_step_draws(uint64_t seed, uint64_t step, void* out_draws_host);
 
@@ -389,6 +398,10 @@ typedef struct guffin_h1_desc {
     uint32_t drafter_rows;          /* 2: the drafter first ingests *pending_token (the proposal the target
                                        accepted last cycle, src/engine/gemma3_draft.mm:1430-1449), then the root */
     const uint32_t* pending_token;  /* device; read only when drafter_rows == 2 */
+    /* sampler history of the verify pass: the last <= 64 confirmed tokens, the root last (device).
+     * Row 0 is sampled with the repetition penalty on these, row 1 on these plus the proposal
+     * (src/engine/sampling.cpp:430-446).  NULL / 0: no penalty.  The drafter's law is not penalised. */
+    const uint32_t* history; uint32_t history_count; float repetition_penalty;
 } guffin_h1_desc;
 uint64_t guffin_hip_h1_scratch_bytes(const guffin_h1_desc* desc);
 int guffin_hip_h1_step(void* stream, const guffin_h1_desc* desc, const uint32_t* root_token, void* scratch,

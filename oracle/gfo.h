@@ -151,6 +151,11 @@ int gfo_spec_accept(const gfo_token_logit* row0, uint32_t n0,
                     const gfo_sampler_options* opt,
                     double u_accept, double u_residual, double u_next,
                     gfo_spec_result* out);
+/* the same decision with a sampler history per row (repetition penalty on those tokens) */
+int gfo_spec_accept_history(const gfo_token_logit* row0, uint32_t n0, const uint32_t* history0, uint32_t count0,
+                            const gfo_token_logit* row1, uint32_t n1, const uint32_t* history1, uint32_t count1,
+                            const gfo_draft_law* law, uint32_t proposal, const gfo_sampler_options* opt,
+                            double u_accept, double u_residual, double u_next, gfo_spec_result* out);
 /* the same decision with q gathered from a full-vocabulary table (cdf: vocab+1 entries) */
 int gfo_spec_accept_full(const gfo_token_logit* row0, uint32_t n0, const gfo_token_logit* row1,
                          uint32_t n1, const uint64_t* cdf, uint32_t vocab, uint32_t proposal,

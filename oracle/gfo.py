@@ -237,6 +237,19 @@ def spec_accept(row0, row1, law, proposal, opt, u_accept, u_residual, u_next, wh
     return rc, out
 
 
+def spec_accept_history(row0, hist0, row1, hist1, law, proposal, opt, u_accept, u_residual, u_next):
+    row0 = np.ascontiguousarray(row0, token_logit)
+    row1 = np.ascontiguousarray(row1, token_logit)
+    hist0 = np.ascontiguousarray(hist0, np.uint32)
+    hist1 = np.ascontiguousarray(hist1, np.uint32)
+    out = SpecResult()
+    rc = lib().gfo_spec_accept_history(_ptr(row0), row0.size, _ptr(hist0), hist0.size, _ptr(row1), row1.size,
+                                       _ptr(hist1), hist1.size, C.byref(law), C.c_uint32(proposal), C.byref(opt),
+                                       C.c_double(u_accept), C.c_double(u_residual), C.c_double(u_next),
+                                       C.byref(out))
+    return rc, out
+
+
 def spec_accept_full(row0, row1, cdf, proposal, opt, u_accept, u_residual, u_next):
     row0 = np.ascontiguousarray(row0, token_logit)
     row1 = np.ascontiguousarray(row1, token_logit)

@@ -432,19 +432,23 @@ int spec_from_prepared(const gfo_prepared* target_in, const LawView& view,
     return 0;
 }
 
+// per-row sampler history (the reference's SamplerHistorySnapshot: the tokens a repetition
+// penalty applies to, src/engine/sampling.cpp:430-446); null for none
+struct RowHistory { const uint32_t* tokens[2]; uint32_t count[2]; };
+
 int spec_accept(const gfo_token_logit* row0, uint32_t n0, const gfo_token_logit* row1, uint32_t n1,
                 const LawView& law, uint32_t proposal, const gfo_sampler_options* opt, double u_accept,
-                double u_residual, double u_next, gfo_spec_result* out) {
+                double u_residual, double u_next, gfo_spec_result* out, const RowHistory& hist = RowHistory{}) {
     std::memset(out, 0, sizeof(*out));
     if (!(std::isfinite(u_next) && u_next >= 0.0 && u_next < 1.0)) return -20;
     gfo_prepared target;
-    int rc = gfo_prepare_token_distribution(row0, n0, opt, nullptr, 0, &target);
+    int rc = gfo_prepare_token_distribution(row0, n0, opt, hist.tokens[0], hist.count[0], &target);
     if (rc) return rc;
     rc = spec_from_prepared(&target, law, proposal, u_accept, u_residual, out);
     if (rc || !out->accepted) return rc;
     // a fully accepted chain leaves row 1's candidates to seed the next root
     gfo_prepared next;
-    rc = gfo_prepare_token_distribution(row1, n1, opt, nullptr, 0, &next);
+    rc = gfo_prepare_token_distribution(row1, n1, opt, hist.tokens[1], hist.count[1], &next);
     if (rc) return rc - 100;
     out->next_root = opt->temperature == 0.0f
         ? next.token[0] : select_prepared(next, u_next * next.total_sampling_weight);
@@ -462,6 +466,14 @@ int gfo_spec_accept(const gfo_token_logit* row0, uint32_t n0, const gfo_token_lo
                     const gfo_sampler_options* opt, double u_accept, double u_residual,
                     double u_next, gfo_spec_result* out) {
     return spec_accept(row0, n0, row1, n1, LawView{law, nullptr, 0}, proposal, opt, u_accept, u_residual, u_next, out);
+}
+
+int gfo_spec_accept_history(const gfo_token_logit* row0, uint32_t n0, const uint32_t* history0, uint32_t count0,
+                            const gfo_token_logit* row1, uint32_t n1, const uint32_t* history1, uint32_t count1,
+                            const gfo_draft_law* law, uint32_t proposal, const gfo_sampler_options* opt,
+                            double u_accept, double u_residual, double u_next, gfo_spec_result* out) {
+    const RowHistory h {{history0, history1}, {count0, count1}};
+    return spec_accept(row0, n0, row1, n1, LawView{law, nullptr, 0}, proposal, opt, u_accept, u_residual, u_next, out, h);
 }
 
 int gfo_spec_accept_full(const gfo_token_logit* row0, uint32_t n0, const gfo_token_logit* row1,

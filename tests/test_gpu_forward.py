@@ -173,6 +173,60 @@ def test_h1_cycle_with_the_full_vocabulary_law(hip, gfo):
     assert a.read_result().tobytes() == b.read_result().tobytes()
 
 
+def test_h1_cycle_with_sampler_history(hip, gfo):
+    """The verify pass's sampler sees the generated tokens so far, and row 1 also the proposal
+    (src/engine/sampling.cpp:430-446): decisions equal the oracle's with both rows' histories, for a
+    short history and for a full window where the oldest token leaves row 1's history."""
+    import torch
+    from dataclasses import replace
+    from guffin_amd import model
+    t_shape = replace(model.GEMMA3_12B, layers=2, vocab=8192, ring_global=2048)
+    d_shape = replace(model.GEMMA3_270M, layers=2, vocab=8192, ring_global=2048)
+    t_host, d_host = model.HostModel(t_shape, seed=41, position=600), model.HostModel(d_shape, seed=42, position=600)
+    # these random models' logits reach 9e4 (target) and 1e3 (drafter): bring them to a sampler's range
+    t_host.out_norm *= np.float32(1e-4)
+    d_host.out_norm *= np.float32(1e-2)
+    target, drafter = model.DeviceModel.from_host(t_host), model.DeviceModel.from_host(d_host)
+    # where the target's mass sits for this root, so that the penalty moves decisions
+    probe = model.H1Plan(target, drafter, 600, 600, seed=9, publish=False)
+    probe.root.fill_(77)
+    probe.step(0)
+    torch.cuda.synchronize()
+    best = np.argsort(-probe.buffers()["p_logits"].cpu().numpy()[0])[:6].astype(np.uint32)
+    rng = np.random.default_rng(5)
+    differs = 0
+    for count in (9, 64):
+        history = np.concatenate([rng.integers(0, 8192, count - best.size).astype(np.uint32), best])
+        plan = model.H1Plan(target, drafter, 600, 600, temperature=1.0, top_k=32, seed=9, publish=False,
+                            history=history.tolist(), repetition_penalty=1.9)
+        opt_cpu = gfo.SamplerOptions(1.0, 32, 0.95, 0.0, 1.9)
+        plan.root.fill_(77)
+        for step in range(8):
+            plan.step(step)
+            torch.cuda.synchronize()
+            bufs, res = plan.buffers(), plan.read_result()
+            assert int(plan.status.item()) == 0 and res["status"] == 0
+            rc, law = gfo.draft_law_compact(bufs["q_logits"].cpu().numpy(), opt_cpu)
+            assert rc == 0
+            word, ua, ur, un = gfo.step_draws(9, step)
+            proposal = gfo.lib().gfo_draft_select(C.byref(law), C.c_uint32(word))
+            assert res["proposal"] == proposal
+            hist1 = np.concatenate([history, [proposal]]).astype(np.uint32)[-64:]
+            retain = 32 + min(count + 1, 64)
+            p_logits = bufs["p_logits"].cpu().numpy()
+            r0 = gfo.select_candidates(p_logits[0], retain, history)
+            r1 = gfo.select_candidates(p_logits[1], retain, hist1)
+            rc, want = gfo.spec_accept_history(r0, history, r1, hist1, law, proposal, opt_cpu, ua, ur, un)
+            assert rc == 0
+            assert (res["accepted"], res["token"], res["next_root"]) == (want.accepted, want.token, want.next_root)
+            assert abs(res["acceptance_probability"] - want.acceptance_probability) <= 1e-13
+            rc, plain = gfo.spec_accept(gfo.select_candidates(p_logits[0], 32), gfo.select_candidates(p_logits[1], 32),
+                                        law, proposal, opt_cpu, ua, ur, un)
+            differs += int(rc != 0 or plain.acceptance_probability != want.acceptance_probability
+                           or plain.token != want.token)
+    assert differs > 0   # the history is not a no-op on these steps
+
+
 def test_h1_commit_publishes_verified_rows(hip, gfo):
     import torch
     from dataclasses import replace

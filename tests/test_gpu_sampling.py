@@ -253,3 +253,39 @@ def test_device_accept_replays_reference_golden_vectors(hip):
         assert int(got["residual_count"]) == int(g["residual_count"][i])
         accepted += int(got["accepted"])
     assert int(status[0]) == 0 and 0 < accepted < n
+
+
+def test_accept_applies_the_repetition_penalty_to_each_rows_history(hip, gfo):
+    """src/engine/sampling.cpp:430-446: history tokens are penalised before the sort, so the candidate
+    rows carry top_k + |history| entries plus the history tokens' own logits; decisions equal the oracle's."""
+    import torch
+    rng = np.random.default_rng(77)
+    vocab, k = 8192, 40
+    o_gpu, o_cpu = hip.SamplerOptions(0.9, k, 0.95, 0.0, 1.7), gfo.SamplerOptions(0.9, k, 0.95, 0.0, 1.7)
+    accepted = rejected = 0
+    for trial in range(40):
+        p_logits = rng.normal(0, 3, (2, vocab)).astype(np.float32)
+        q_logits = (p_logits[0] + rng.normal(0, 1.0, vocab)).astype(np.float32)
+        top = np.argsort(-p_logits[0])[:8]                      # penalise some of the very best tokens
+        hist0 = np.concatenate([top[:5], rng.integers(0, vocab, 20)]).astype(np.uint32)
+        hist1 = np.concatenate([hist0, top[5:6]]).astype(np.uint32)
+        hist = np.zeros((2, 64), np.uint32)
+        hist[0, :hist0.size], hist[1, :hist1.size] = hist0, hist1
+        counts = np.array([hist0.size, hist1.size], np.uint32)
+        retain = k + hist1.size
+        res, status = hip.select_candidates(dev(p_logits), retain, history=dev(hist), history_count=dev(counts))
+        assert int(status.abs().sum()) == 0
+        law, proposal, st = hip.draft_law(dev(q_logits), hip.SamplerOptions(0.9, k, 0.95, 0.0, 1.0), seed=3, step=trial)
+        out = hip.spec_accept_history(res, law, dev(hist), dev(counts), proposal, o_gpu, seed=3, step=trial, status=st)
+        got = out.cpu().numpy().view(hip.result_dtype)[0]
+        rc, law_cpu = gfo.draft_law_compact(q_logits, gfo.SamplerOptions(0.9, k, 0.95, 0.0, 1.0))
+        word, ua, ur, un = gfo.step_draws(3, trial)
+        prop = gfo.lib().gfo_draft_select(C.byref(law_cpu), C.c_uint32(word))
+        rows = [gfo.select_candidates(p_logits[0], retain, hist0), gfo.select_candidates(p_logits[1], retain, hist1)]
+        rc, want = gfo.spec_accept_history(rows[0], hist0, rows[1], hist1, law_cpu, prop, o_cpu, ua, ur, un)
+        assert int(st[0]) == 0 and rc == 0 and got["status"] == 0 and got["proposal"] == prop
+        assert (got["accepted"], got["token"], got["next_root"]) == (want.accepted, want.token, want.next_root), trial
+        # the penalty matters: without it the decision inputs differ for at least the penalised best token
+        accepted += want.accepted
+        rejected += 1 - want.accepted
+    assert accepted > 0 and rejected > 0
