@@ -175,6 +175,79 @@ rms_norm_add_norm_kernel(const float* __restrict__ x, uint32_t planes, size_t pl
     }
 }
 
+// The same for the common shape (at most four planes, 16-byte aligned rows, width a multiple of 8
+// and at most 8 x 1024): a thread owns 8 consecutive columns from the operands to the receipt, so
+// every operand is requested at once (one trip to memory instead of one per plane batch) and
+// nothing is staged in LDS but the per-wave sums.
+constexpr int kFastPlanes = 4;
+__device__ __forceinline__ float4 ld4(const float* p, bool on) {
+    return on ? *reinterpret_cast<const float4*>(p) : make_float4(0.f, 0.f, 0.f, 0.f);
+}
+__device__ __forceinline__ void unpack4(const float4& a, float* o) { o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w; }
+
+__global__ void __launch_bounds__(1024)
+rms_norm_add_norm_regs_kernel(const float* __restrict__ x, uint32_t planes, size_t plane_stride,
+                              const float* __restrict__ gamma_post, const float* __restrict__ residual,
+                              float* __restrict__ out_residual, const float* __restrict__ gamma_next,
+                              float* __restrict__ out_norm, float* __restrict__ out_sums, uint32_t width,
+                              float eps, uint32_t* __restrict__ status) {
+    __shared__ float scratch[16];
+    const uint32_t r = blockIdx.x, item = threadIdx.x;
+    const bool active = item < width / 8;
+    const size_t col = active ? item * 8u : 0u, at = size_t(r) * width + col;
+    float4 p[kFastPlanes][2], res4[2], gp4[2], gn4[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        gp4[h] = ld4(gamma_post + col + 4 * h, active);
+        gn4[h] = ld4(gamma_next + col + 4 * h, active);
+        res4[h] = ld4(residual + at + 4 * h, active);
+#pragma unroll
+        for (int s = 0; s < kFastPlanes; ++s) p[s][h] = ld4(x + s * plane_stride + at + 4 * h, active && uint32_t(s) < planes);
+    }
+    float v[8], a[8], gp[8], gn[8], res[8];
+    unpack4(p[0][0], v); unpack4(p[0][1], v + 4);
+#pragma unroll
+    for (int s = 1; s < kFastPlanes; ++s) {  // plane order
+        if (uint32_t(s) < planes) {
+            unpack4(p[s][0], a); unpack4(p[s][1], a + 4);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[i] += a[i];
+        }
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) ss = fmaf(v[i], v[i], ss);
+    float total = block_sum(ss, scratch);
+    float inv = 1.0f / sqrtf(total / static_cast<float>(width) + eps);
+    unpack4(gp4[0], gp); unpack4(gp4[1], gp + 4);
+    unpack4(gn4[0], gn); unpack4(gn4[1], gn + 4);
+    unpack4(res4[0], res); unpack4(res4[1], res + 4);
+    bool bad = false;
+    ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const float t = active ? v[i] * inv * gp[i] + res[i] : 0.f;
+        bad |= !isfinite(t);
+        v[i] = t;
+        ss = fmaf(t, t, ss);
+    }
+    if (active) {
+        *reinterpret_cast<float4*>(out_residual + at) = make_float4(v[0], v[1], v[2], v[3]);
+        *reinterpret_cast<float4*>(out_residual + at + 4) = make_float4(v[4], v[5], v[6], v[7]);
+    }
+    total = block_sum(ss, scratch);
+    inv = 1.0f / sqrtf(total / static_cast<float>(width) + eps);
+    float y[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) y[i] = v[i] * inv * gn[i];
+    if (active) {
+        *reinterpret_cast<float4*>(out_norm + at) = make_float4(y[0], y[1], y[2], y[3]);
+        *reinterpret_cast<float4*>(out_norm + at + 4) = make_float4(y[4], y[5], y[6], y[7]);
+        if (out_sums) emit_receipt_values(y, 0, item, r, gridDim.x, width, out_sums);
+    }
+    if (bad && status) atomicOr(status, GUFFIN_STATUS_NONFINITE);
+}
+
 // Per-head RMS norm over head_dim (one wave per (row, head)); in place allowed.
 __global__ void __launch_bounds__(64)
 head_rms_norm_kernel(const float* __restrict__ x, const float* __restrict__ gamma, float* __restrict__ y,
@@ -408,6 +481,15 @@ extern "C" int guffin_hip_rms_norm_add_norm(void* stream, const float* x, uint32
     if (out_sums && (width % 32 != 0 || rows > 2)) return fail(GUFFIN_E_SHAPE, "rms_norm_add_norm: a receipt needs width % 32 == 0 and rows <= 2");
     if (reinterpret_cast<uintptr_t>(out_sums) & 255u) return fail(GUFFIN_E_ALIGN, "rms_norm_add_norm: the receipt must be 256-byte aligned");
     if (!(eps > 0.f)) return fail(GUFFIN_E_ARG, "rms_norm_add_norm: epsilon must be positive");
+    auto a16 = [](const void* q) { return (reinterpret_cast<uintptr_t>(q) & 15u) == 0; };
+    if (planes <= uint32_t(kFastPlanes) && width % 8 == 0 && width / 8 <= 1024 && (!out_sums || width % 32 == 0)
+        && plane_stride % 4 == 0 && a16(x) && a16(gamma_post) && a16(residual) && a16(out_residual) && a16(gamma_next) && a16(out_norm)) {
+        const uint32_t threads = (width / 8 + 63) / 64 * 64;
+        hipLaunchKernelGGL(rms_norm_add_norm_regs_kernel, dim3(rows), dim3(threads), 0, as_stream(stream), x, planes,
+                           static_cast<size_t>(plane_stride), gamma_post, residual, out_residual, gamma_next, out_norm,
+                           out_sums, width, eps, status);
+        return check_launch("rms_norm_add_norm");
+    }
     const size_t lds = (size_t(width) + 16) * 4;
     if (lds > 160 * 1024) return fail(GUFFIN_E_CAPACITY, "rms_norm_add_norm: row does not fit in LDS");
     hipLaunchKernelGGL(rms_norm_add_norm_kernel, dim3(rows), dim3(norm_threads(width)), lds, as_stream(stream), x, planes,

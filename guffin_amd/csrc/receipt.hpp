@@ -32,21 +32,17 @@ __host__ __device__ inline ReceiptLayout receipt_layout(uint32_t rows, uint32_t 
     return {mult, image, image + size_t(K / 32) * 256};
 }
 
-// Writes the part of row r's receipt that covers elements k0 .. k0+count (both multiples of 32)
-// from vals[0 .. count) (LDS or global).  Called by every thread of a workgroup whose size is a
-// multiple of 64; four consecutive lanes share a group.
-__device__ __forceinline__ void emit_receipt(const float* vals, uint32_t k0, uint32_t count, uint32_t r, uint32_t rows,
-                                             uint32_t K, void* blob) {
+// One item: the 8 consecutive activations v[] of row r, elements k0 + 8t .. k0 + 8t + 7.  The four
+// lanes of a 32-group (t % 4 = 0..3 in consecutive lanes) must run it together.
+__device__ __forceinline__ void emit_receipt_values(const float (&v)[8], uint32_t k0, uint32_t t, uint32_t r, uint32_t rows,
+                                                    uint32_t K, void* blob) {
     const ReceiptLayout L = receipt_layout(rows, K);
     const uint32_t n16 = K / 16;
     float* sums = static_cast<float*>(blob) + size_t(r) * (n16 + K / 32);
     float* mult = reinterpret_cast<float*>(static_cast<uint8_t*>(blob) + L.mult_off) + size_t(r) * (K / 32);
     uint8_t* image = static_cast<uint8_t*>(blob) + L.image_off;
-    for (uint32_t t = threadIdx.x; t < count / 8; t += blockDim.x) {
+    {
         const uint32_t g = (k0 >> 5) + (t >> 2), s = t & 3;
-        float v[8];
-#pragma unroll
-        for (int i = 0; i < 8; ++i) v[i] = vals[t * 8 + i];
         float sum = v[0], m = fabsf(v[0]);
 #pragma unroll
         for (int i = 1; i < 8; ++i) { sum += v[i]; m = fmaxf(m, fabsf(v[i])); }
@@ -82,6 +78,19 @@ __device__ __forceinline__ void emit_receipt(const float* vals, uint32_t k0, uin
             *reinterpret_cast<uint4*>(base + 128) = make_uint4(0, 0, 0, 0);
             *reinterpret_cast<uint4*>(base + 192) = make_uint4(0, 0, 0, 0);
         }
+    }
+}
+
+// Writes the part of row r's receipt that covers elements k0 .. k0+count (both multiples of 32)
+// from vals[0 .. count) (LDS or global).  Called by every thread of a workgroup whose size is a
+// multiple of 64; four consecutive lanes share a group.
+__device__ __forceinline__ void emit_receipt(const float* vals, uint32_t k0, uint32_t count, uint32_t r, uint32_t rows,
+                                             uint32_t K, void* blob) {
+    for (uint32_t t = threadIdx.x; t < count / 8; t += blockDim.x) {
+        float v[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = vals[t * 8 + i];
+        emit_receipt_values(v, k0, t, r, rows, K, blob);
     }
 }
 

@@ -94,6 +94,42 @@ def test_rms_norm_add_norm_joint(hip, gfo):
     assert np.allclose(sums.cpu().numpy(), group_sums_ref(out_norm.cpu().numpy()), rtol=0, atol=1e-4)
 
 
+@pytest.mark.parametrize("rows,width,planes", [(2, 3840, 4), (1, 3840, 1), (2, 640, 2), (1, 8192, 3), (2, 3840, 5), (2, 96, 4)])
+def test_rms_norm_add_norm_over_planes(hip, gfo, rows, width, planes):
+    """Both kernels behind the entry point (registers for up to four planes, staged rows beyond) against the
+    oracle on the plane sum taken in plane order; image and multipliers of the receipt rebuild the normed rows."""
+    rng = np.random.default_rng(31)
+    parts = rng.normal(0, 10, (planes, rows, width)).astype(np.float32)
+    res = rng.normal(0, 2, (rows, width)).astype(np.float32)
+    g1 = rng.normal(1, 0.1, width).astype(np.float32)
+    g2 = rng.normal(1, 0.1, width).astype(np.float32)
+    total = parts[0].copy()
+    for s in range(1, planes):
+        total = total + parts[s]
+    want_res = gfo.rms_norm(total, g1, 1e-6, residual=res)
+    want_norm = gfo.rms_norm(want_res, g2, 1e-6)
+    status = hip.new_status()
+    out_res, out_norm, sums = hip.rms_norm_add_norm(dev(parts), dev(g1), dev(res), dev(g2), planes=planes, want_sums=True,
+                                                    status=status)
+    y = out_norm.cpu().numpy()
+    assert int(status[0]) == 0
+    assert np.max(np.abs(out_res.cpu().numpy() - want_res)) <= 2e-5 * np.abs(want_res).max()
+    assert np.max(np.abs(y - want_norm)) <= 4e-5 * np.abs(want_norm).max()
+    assert np.allclose(sums.cpu().numpy(), group_sums_ref(y), rtol=0, atol=1e-4)
+    mult, image = hip.receipt_parts(sums, rows, width)
+    m, img = mult.cpu().numpy().astype(np.float64), image.cpu().numpy().astype(np.float64)
+    order = [0, 2, 1, 3, 4, 6, 5, 7]
+    img = img.reshape(width // 32, 4, 4, 8)
+    for r in range(rows):
+        back = np.empty((width // 32, 4, 8))
+        back[:, :, order] = img[:, 2 * r] + img[:, 2 * r + 1]
+        back = back.reshape(width // 32, 32) * (m[r][:, None] / 2.0 ** 24)
+        assert np.max(np.abs(back.reshape(-1) - y[r])) <= 2.0 ** -21 * np.abs(y[r]).max()
+    parts[0, rows - 1, width - 1] = np.inf
+    hip.rms_norm_add_norm(dev(parts), dev(g1), dev(res), dev(g2), planes=planes, status=status)
+    assert int(status[0]) == 2
+
+
 def test_head_rms_norm(hip, gfo):
     rng = np.random.default_rng(4)
     x = rng.normal(0, 4, (2, 16 * 256)).astype(np.float32)
