@@ -21,6 +21,8 @@
 //           halves are combined by one lane exchange, the four waves through LDS.
 // Partitions emit (max, denominator, unnormalised output); a second kernel merges them in
 // partition order.  fp32 throughout, keys/values stay fp16 in memory.
+#include <algorithm>
+
 #include "common.hpp"
 #include "receipt.hpp"
 
@@ -337,45 +339,55 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(AttnArgs a) {
 }
 
 // out[row][head][:] = sum_p e^(m_p - M) acc_p / sum_p e^(m_p - M) l_p, partitions in order.
-// The partition weights are formed once, in parallel, in LDS; each thread then owns one
-// output dimension and walks the partitions with independent loads.
+// Each thread owns one output dimension.  The outputs of the first 64 partitions are requested at
+// once, before the weights exist (indices beyond the last partition read the last one again and
+// meet a zero weight), so up to 64 partitions cost one trip to memory; weights and denominators
+// terms are formed once, in parallel, in LDS.
+constexpr int kMergeAhead = 64;
 __global__ void __launch_bounds__(256)
 attn_merge_kernel(const float* __restrict__ part_out, const float* __restrict__ part_ml, float* __restrict__ out,
                   float* __restrict__ out_sums, uint32_t partitions, uint32_t hd, uint32_t q_heads,
                   uint32_t* __restrict__ status) {
-    extern __shared__ float wgt[];  // [partitions]
+    extern __shared__ float wgt[];  // [max(partitions, 64)] weights, then as many partition sums l_p
     __shared__ float red[4];
     __shared__ float rowbuf[1024];
     const uint32_t rh = blockIdx.x;  // row * q_heads + head
     const uint32_t lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const uint32_t slots = partitions > uint32_t(kMergeAhead) ? partitions : uint32_t(kMergeAhead);
+    float* lsum = wgt + slots;
     const float* ml = part_ml + size_t(rh) * partitions * 2;
     const float* po = part_out + size_t(rh) * partitions * hd;
-    // the first partitions' outputs are requested before the weights exist
-    constexpr int PF = 16;
     const uint32_t d0 = threadIdx.x;
-    float pre[PF];
+    float pre[kMergeAhead];
 #pragma unroll
-    for (int p = 0; p < PF; ++p) pre[p] = (uint32_t(p) < partitions && d0 < hd) ? po[size_t(p) * hd + d0] : 0.f;
+    for (int p = 0; p < kMergeAhead; ++p) {
+        const uint32_t q = uint32_t(p) < partitions ? uint32_t(p) : partitions - 1;
+        pre[p] = d0 < hd ? po[size_t(q) * hd + d0] : 0.f;
+    }
     float m = -INFINITY;
     for (uint32_t p = threadIdx.x; p < partitions; p += 256) if (ml[2 * p + 1] > 0.f) m = fmaxf(m, ml[2 * p]);
     m = wave_max(m);
     if (lane == 0) red[wv] = m;
     __syncthreads();
     const float M = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
-    for (uint32_t p = threadIdx.x; p < partitions; p += 256)
-        wgt[p] = ml[2 * p + 1] > 0.f ? expf(ml[2 * p] - M) : 0.f;
+    for (uint32_t p = threadIdx.x; p < slots; p += 256) {
+        const float l = p < partitions ? ml[2 * p + 1] : 0.f;
+        wgt[p] = l > 0.f ? expf(ml[2 * p] - M) : 0.f;
+        lsum[p] = l;
+    }
     __syncthreads();
-    float denom = 0.f;
-    for (uint32_t p = 0; p < partitions; ++p) denom = fmaf(wgt[p], ml[2 * p + 1], denom);
+    float denom = 0.f, acc0 = 0.f;
+#pragma unroll
+    for (int q = 0; q < kMergeAhead; ++q) {
+        denom = fmaf(wgt[q], lsum[q], denom);
+        acc0 = fmaf(wgt[q], pre[q], acc0);
+    }
+    for (uint32_t p = kMergeAhead; p < partitions; ++p) denom = fmaf(wgt[p], lsum[p], denom);
     bool bad = false;
     for (uint32_t d = threadIdx.x; d < hd; d += blockDim.x) {
         float acc = 0.f;
         uint32_t p = 0;
-        if (d == d0) {
-#pragma unroll
-            for (int q = 0; q < PF; ++q) if (uint32_t(q) < partitions) acc = fmaf(wgt[q], pre[q], acc);
-            p = partitions < PF ? partitions : PF;
-        }
+        if (d == d0) { acc = acc0; p = partitions < uint32_t(kMergeAhead) ? partitions : uint32_t(kMergeAhead); }
         for (; p + 4 <= partitions; p += 4) {
             const float v0 = po[size_t(p) * hd + d], v1 = po[size_t(p + 1) * hd + d], v2 = po[size_t(p + 2) * hd + d],
                         v3 = po[size_t(p + 3) * hd + d];
@@ -481,7 +493,7 @@ int attention_decode(void* stream, const float* q, const FusedInputs* fused, con
         default: return fail(GUFFIN_E_SHAPE, "attention_decode: q_heads / kv_heads must be 1, 2 or 4");
     }
     if (rc) return rc;
-    hipLaunchKernelGGL(attn_merge_kernel, dim3(rows * q_heads), dim3(256), a.partitions * sizeof(float), s, partial_out, partial_ml, out,
+    hipLaunchKernelGGL(attn_merge_kernel, dim3(rows * q_heads), dim3(256), 2 * std::max<uint32_t>(a.partitions, kMergeAhead) * sizeof(float), s, partial_out, partial_ml, out,
                        out_sums, a.partitions, head_dim, q_heads, status);
     return check_launch("attention_merge");
 }
