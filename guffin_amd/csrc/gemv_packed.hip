@@ -151,11 +151,18 @@ __device__ __forceinline__ half8_t as_half8(uint32_t a, uint32_t b, uint32_t c, 
 
 // image: this block's 8 groups of the activation image, already offset for this lane;
 // mult / xs32: this block's 8 multipliers / 32-sums of row 0 (rows `per_mult` / `per_row` apart)
+struct Q4Operand { half8_t a[8]; };
+__device__ __forceinline__ void load_operand(Q4Operand& o, const uint8_t* __restrict__ image) {
+#pragma unroll
+    for (int g = 0; g < 8; ++g) o.a[g] = __builtin_bit_cast(half8_t, *reinterpret_cast<const uint4*>(image + 256 * g));
+}
+
 template <int R>
-__device__ __forceinline__ void compute_tile(const Q4Tile& t, const uint8_t* __restrict__ image,
+__device__ __forceinline__ void compute_tile(const Q4Tile& t, const Q4Operand& op,
                                              const float* __restrict__ mult, uint32_t per_mult,
                                              const float* __restrict__ xs32, uint32_t per_row,
                                              uint32_t lane_group, float (&acc)[R]) {
+    const half8_t (&a)[8] = op.a;
     const float d = h2f(t.hdr.x & 0xFFFFu), dmin = h2f(t.hdr.x >> 16);
     const uint32_t s0 = t.hdr.y, s1 = t.hdr.z, s2 = t.hdr.w;
     const uint32_t sc_a = s0 & 0x3F3F3F3Fu, mn_a = s1 & 0x3F3F3F3Fu;
@@ -165,9 +172,6 @@ __device__ __forceinline__ void compute_tile(const Q4Tile& t, const uint8_t* __r
     float mt[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) mt[r] = 0.f;
-    half8_t a[8];
-#pragma unroll
-    for (int g = 0; g < 8; ++g) a[g] = __builtin_bit_cast(half8_t, *reinterpret_cast<const uint4*>(image + 256 * g));
     const float4_t zero = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int ch = 0; ch < 4; ++ch) {  // 32-byte chunk: sub-blocks 2ch (low nibbles) and 2ch+1 (high)
@@ -368,11 +372,15 @@ __device__ __forceinline__ void run_blocks(const uint8_t* __restrict__ wt, const
     // lane (i = lane % 16, s = lane / 16) of the A operand: variant i % 4, k-slice s
     const uint8_t* image = blob + L.image_off + (lane & 3u) * 64u + (lane >> 4) * 16u;
     if constexpr (DTYPE == GUFFIN_Q4_K) {
+        // the first block's operand (a hit in the caches) is requested ahead of the weight tiles, which
+        // come from HBM: behind them it would cost every wave a second trip before its first product
         Q4Tile cur, nxt;
-        if (b0 < b1) load_tile(cur, tp);
+        Q4Operand op;
+        if (b0 < b1) { load_operand(op, image + size_t(b0) * 2048u); load_tile(cur, tp); }
         for (uint32_t b = b0; b < b1; ++b) {
             if (b + 1 < b1) load_tile(nxt, tp + size_t(b + 1 - b0) * TB);
-            compute_tile<R>(cur, image + size_t(b) * 2048u, mult + b * 8u, K / 32, xs + b * 8u, per_row, lane >> 4, acc);
+            if (b != b0) load_operand(op, image + size_t(b) * 2048u);
+            compute_tile<R>(cur, op, mult + b * 8u, K / 32, xs + b * 8u, per_row, lane >> 4, acc);
             cur = nxt;
         }
     } else if constexpr (DTYPE == GUFFIN_Q6_K) {
