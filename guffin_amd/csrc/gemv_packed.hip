@@ -327,11 +327,10 @@ __device__ __forceinline__ void load_tile(Q8Tile& t, const uint8_t* p, uint32_t 
 }
 
 template <int R>
-__device__ __forceinline__ void compute_tile(const Q8Tile& t, const uint8_t* __restrict__ image,
+__device__ __forceinline__ void compute_tile(const Q8Tile& t, const half8_t a,
                                              const float* __restrict__ mult, uint32_t per_mult,
                                              const float* __restrict__ xs32, uint32_t per_row,
                                              uint32_t lane_group, float (&acc)[R]) {
-    const half8_t a = __builtin_bit_cast(half8_t, *reinterpret_cast<const uint4*>(image));
     const float4_t zero = {0.f, 0.f, 0.f, 0.f};
     float4_t own = zero;
 #pragma unroll
@@ -391,6 +390,7 @@ __device__ __forceinline__ void run_blocks(const uint8_t* __restrict__ wt, const
         for (int c = 0; c < 2; ++c)
 #pragma unroll
             for (int r = 0; r < R; ++r) acc2[c][r] = 0.f;
+        // (this tile and its operand together do not fit the registers: the operand is read group by group)
         Q6Tile cur, nxt;
         if (b0 < b1) load_tile(cur, tp, lane);
         for (uint32_t b = b0; b < b1; ++b) {
@@ -401,11 +401,14 @@ __device__ __forceinline__ void run_blocks(const uint8_t* __restrict__ wt, const
         q6_gather<R>(acc2, lane, acc);
     } else {
         Q8Tile cur, nxt;
-        if (b0 < b1) load_tile(cur, tp, lane);
+        auto operand = [&](uint32_t b) { return __builtin_bit_cast(half8_t, *reinterpret_cast<const uint4*>(image + size_t(b) * 256u)); };
+        half8_t a = {}, an = {};
+        if (b0 < b1) { a = operand(b0); load_tile(cur, tp, lane); }
         for (uint32_t b = b0; b < b1; ++b) {
-            if (b + 1 < b1) load_tile(nxt, tp + size_t(b + 1 - b0) * TB, lane);
-            compute_tile<R>(cur, image + size_t(b) * 256u, mult + b, K / 32, xs + b, per_row, lane >> 4, acc);
+            if (b + 1 < b1) { an = operand(b + 1); load_tile(nxt, tp + size_t(b + 1 - b0) * TB, lane); }
+            compute_tile<R>(cur, a, mult + b, K / 32, xs + b, per_row, lane >> 4, acc);
             cur = nxt;
+            a = an;
         }
     }
 }
