@@ -95,6 +95,7 @@ __device__ __forceinline__ void hist_add(uint32_t* hist, bool valid, uint32_t bi
 // Stage 2: exact selection of the best `retain` of n unique keys by an 8-pass radix select
 // (one byte per pass, most significant first: a 256-bin histogram in LDS, then the bin that
 // holds the retain-th largest key), followed by a rank sort of the selected keys.
+template <int kMine>
 __global__ void __launch_bounds__(1024)
 topk_merge_kernel(const float* __restrict__ logits, const uint64_t* __restrict__ survivors, uint32_t n_survivors,
                   uint32_t vocab, uint32_t retain, float divisor, const uint32_t* __restrict__ history,
@@ -106,8 +107,8 @@ topk_merge_kernel(const float* __restrict__ logits, const uint64_t* __restrict__
     __shared__ uint32_t s_bin, s_above, s_count, s_in_bin;
     const uint32_t row = blockIdx.x, lane = threadIdx.x & 63;
     const uint64_t* src = survivors + size_t(row) * n_survivors;
-    // up to 8 keys per thread stay in registers; longer survivor lists are re-read from memory
-    constexpr int kMine = 8;
+    // up to kMine keys per thread stay in registers (8 for the verify pass's lists, 34 for the 257 per
+    // tile that the proposal law asks for); longer survivor lists are re-read from memory in every pass
     const bool cached = n_survivors <= kMine * blockDim.x;
     uint64_t mine[kMine];
 #pragma unroll
@@ -314,8 +315,12 @@ int guffin::select_candidates_scaled(hipStream_t s, const float* logits, uint32_
     uint64_t* surv = static_cast<uint64_t*>(workspace);
     hipLaunchKernelGGL(topk_tile_kernel, dim3(tiles, rows), dim3(1024), 0, s, logits, surv, vocab, keep, divisor, status);
     if (int rc = check_launch("select_candidates(tile)")) return rc;
-    hipLaunchKernelGGL(topk_merge_kernel, dim3(rows), dim3(1024), 0, s, logits, surv, tiles * keep, vocab,
-                       keep, divisor, history, history_count, static_cast<Candidates*>(result), status);
+    if (tiles * keep <= 8 * 1024)
+        hipLaunchKernelGGL(topk_merge_kernel<8>, dim3(rows), dim3(1024), 0, s, logits, surv, tiles * keep, vocab,
+                           keep, divisor, history, history_count, static_cast<Candidates*>(result), status);
+    else
+        hipLaunchKernelGGL(topk_merge_kernel<34>, dim3(rows), dim3(1024), 0, s, logits, surv, tiles * keep, vocab,
+                           keep, divisor, history, history_count, static_cast<Candidates*>(result), status);
     return check_launch("select_candidates(merge)");
 }
 
