@@ -757,10 +757,40 @@ __global__ void publish_run_kernel(const uint4* __restrict__ run_k, const uint4*
     ring_v[dst] = run_v[size_t(row) * row_vec + c];
 }
 
+// dst[(position + t) & dst_mask] = src[(position + t) & src_mask], keys and values
+__global__ void kv_cache_copy_kernel(const uint4* __restrict__ src_k, const uint4* __restrict__ src_v,
+                                     uint4* __restrict__ dst_k, uint4* __restrict__ dst_v, uint32_t tokens,
+                                     uint32_t position, uint32_t src_mask, uint32_t dst_mask, uint32_t row_vec) {
+    const uint64_t i = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i >= uint64_t(tokens) * row_vec) return;
+    const uint32_t t = static_cast<uint32_t>(i / row_vec), c = static_cast<uint32_t>(i % row_vec);
+    const size_t from = size_t((position + t) & src_mask) * row_vec + c, to = size_t((position + t) & dst_mask) * row_vec + c;
+    dst_k[to] = src_k[from];
+    dst_v[to] = src_v[from];
+}
+
 }  // namespace
 }  // namespace guffin
 
 using namespace guffin;
+
+extern "C" int guffin_hip_kv_cache_copy(void* stream, const void* src_k, const void* src_v, void* dst_k, void* dst_v,
+                                        uint32_t position, uint32_t tokens, uint32_t src_mask, uint32_t dst_mask,
+                                        uint32_t row_width) {
+    if (!src_k || !src_v || !dst_k || !dst_v) return fail(GUFFIN_E_ARG, "kv_cache_copy: null pointer");
+    if (tokens == 0 || row_width == 0 || row_width % 8 != 0) return fail(GUFFIN_E_SHAPE, "kv_cache_copy: row width must be a multiple of 8 halves");
+    if ((src_mask & (src_mask + 1)) != 0 || (dst_mask & (dst_mask + 1)) != 0)
+        return fail(GUFFIN_E_ARG, "kv_cache_copy: row masks must be a power of two minus one");
+    if (tokens > src_mask + 1 || tokens > dst_mask + 1) return fail(GUFFIN_E_CAPACITY, "kv_cache_copy: more tokens than rows on one side");
+    if (((reinterpret_cast<uintptr_t>(src_k) | reinterpret_cast<uintptr_t>(src_v) | reinterpret_cast<uintptr_t>(dst_k)
+          | reinterpret_cast<uintptr_t>(dst_v)) & 15u) != 0)
+        return fail(GUFFIN_E_ALIGN, "kv_cache_copy: rows must be 16-byte aligned");
+    const uint64_t n = uint64_t(tokens) * (row_width / 8);
+    hipLaunchKernelGGL(kv_cache_copy_kernel, dim3(static_cast<uint32_t>((n + 255) / 256)), dim3(256), 0, as_stream(stream),
+                       static_cast<const uint4*>(src_k), static_cast<const uint4*>(src_v), static_cast<uint4*>(dst_k),
+                       static_cast<uint4*>(dst_v), tokens, position, src_mask, dst_mask, row_width / 8);
+    return check_launch("kv_cache_copy");
+}
 
 extern "C" int guffin_hip_publish_run(void* stream, const void* run_k, const void* run_v, void* ring_k, void* ring_v,
                                       uint32_t rows, uint32_t position, uint32_t ring_mask, uint32_t row_width) {

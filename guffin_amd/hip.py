@@ -462,6 +462,11 @@ def prefill_attention(q, ring_k, ring_v, run_k, run_v, position, window, ring_ma
     return out
 
 
+def kv_cache_copy(src_k, src_v, dst_k, dst_v, position, tokens, src_mask, dst_mask):
+    check(lib().guffin_hip_kv_cache_copy(_stream(), _p(src_k), _p(src_v), _p(dst_k), _p(dst_v), position, tokens,
+                                         src_mask, dst_mask, src_k.shape[-1]))
+
+
 def publish_run(run_k, run_v, ring_k, ring_v, position, ring_mask):
     rows, width = run_k.shape
     check(lib().guffin_hip_publish_run(_stream(), _p(run_k), _p(run_v), _p(ring_k), _p(ring_v), rows, position,

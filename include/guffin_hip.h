@@ -372,6 +372,16 @@ int guffin_hip_prefill_attention(void* stream, const float* q, const void* ring_
  * capacity keeps (encode_gemma2_kv_cache_copy, metal_command_context.hpp:170). */
 int guffin_hip_publish_run(void* stream, const void* run_k, const void* run_v, void* ring_k, void* ring_v,
                            uint32_t rows, uint32_t position, uint32_t ring_mask, uint32_t row_width);
+/* dst[(position + t) & dst_mask] = src[(position + t) & src_mask] for t < tokens, keys and values:
+ * encode_gemma2_kv_cache_copy (metal_command_context.hpp:170) with both row masks.  A mask is the
+ * side's row capacity minus one (a power of two minus one; 0 = a single row).  With it a host that
+ * keeps the reference's provisional protocol backs the ring rows of a verify pass up
+ * (src/engine/gemma_target_runtime.cpp:473-479) and restores a rejected suffix
+ * (src/engine/gemma2_runtime.cpp:756-765); guffin_hip_h1_step needs neither, it publishes after the
+ * decision. */
+int guffin_hip_kv_cache_copy(void* stream, const void* src_k, const void* src_v, void* dst_k, void* dst_v,
+                             uint32_t position, uint32_t tokens, uint32_t src_mask, uint32_t dst_mask,
+                             uint32_t row_width);
 /* The block graph of guffin_hip_forward_rows for any number of rows (prompt ingestion): same
  * operator order, matrix-core GEMMs, the run's K/V published to the rings layer by layer.
  * out_hidden [rows][hidden] holds the output-normed rows. */

@@ -263,3 +263,34 @@ def test_kv_scatter_publishes_selected_rows(hip):
     assert torch.equal(ring_k[7], pk[2]) and torch.equal(ring_k[0], pk[0])
     assert torch.equal(ring_v[7], pv[2]) and torch.equal(ring_v[0], pv[0])
     assert float(ring_k[1:7].abs().sum()) == 0.0
+
+
+def test_kv_cache_copy_backs_ring_rows_up_and_restores_them(hip):
+    """encode_gemma2_kv_cache_copy with both row masks (metal_command_context.hpp:170), used as the reference's
+    verify pass uses it (gemma_target_runtime.cpp:473-479, gemma2_runtime.cpp:756-765): the two rows a verify
+    pair will overwrite are saved from a ring that wraps, overwritten, and the rejected suffix is put back."""
+    import torch
+    rng = np.random.default_rng(10)
+    cap, width, position = 8, 2048, 7        # rows 7 and 8 -> ring slots 7 and 0
+    ring_k = dev(rng.normal(0, 1, (cap, width)).astype(np.float16))
+    ring_v = dev(rng.normal(0, 1, (cap, width)).astype(np.float16))
+    before_k, before_v = ring_k.clone(), ring_v.clone()
+    backup_k = torch.zeros((2, width), dtype=torch.float16, device="cuda")
+    backup_v = torch.zeros((2, width), dtype=torch.float16, device="cuda")
+    hip.kv_cache_copy(ring_k, ring_v, backup_k, backup_v, position, 2, cap - 1, 1)
+    # a backup of capacity 2 keeps row p in slot p & 1
+    assert torch.equal(backup_k[1], before_k[7]) and torch.equal(backup_k[0], before_k[0])
+    assert torch.equal(backup_v[1], before_v[7]) and torch.equal(backup_v[0], before_v[0])
+    new_k = dev(rng.normal(0, 1, (2, width)).astype(np.float16))
+    new_v = dev(rng.normal(0, 1, (2, width)).astype(np.float16))
+    hip.publish_run(new_k, new_v, ring_k, ring_v, position, cap - 1)
+    assert torch.equal(ring_k[7], new_k[0]) and torch.equal(ring_k[0], new_k[1])
+    # the proposal was rejected: row 0 stays, the suffix (row position + 1) returns
+    hip.kv_cache_copy(backup_k, backup_v, ring_k, ring_v, position + 1, 1, 1, cap - 1)
+    assert torch.equal(ring_k[0], before_k[0]) and torch.equal(ring_v[0], before_v[0])
+    assert torch.equal(ring_k[7], new_k[0]) and torch.equal(ring_v[7], new_v[0])
+    assert torch.equal(ring_k[1:7], before_k[1:7]) and torch.equal(ring_v[1:7], before_v[1:7])
+    with pytest.raises(hip.GuffinError):
+        hip.kv_cache_copy(ring_k, ring_v, backup_k, backup_v, position, 3, cap - 1, 1)   # three tokens, two rows
+    with pytest.raises(hip.GuffinError):
+        hip.kv_cache_copy(ring_k, ring_v, backup_k, backup_v, position, 2, 5, 1)         # not a row mask
