@@ -486,6 +486,12 @@ extern "C" int guffin_hip_h1_step(void* stream, const guffin_h1_desc* d, const u
     GUFFIN_TRY(guffin_hip_gemv_packed(stream, D.head_dtype, D.head_tiles, d_hidden, d_hidden + hidden_receipt_offset(dr, D.hidden), q_parts,
                                       q_logits, dr, D.hidden, D.vocab));
     q_logits += uint64_t(dr - 1) * D.vocab;  // the law comes from the last ingested row (the root)
+    if (with_history && d->repetition_penalty != 1.0f) {
+        // the proposal law sees the same history as the verify pass's first row (the head's partial
+        // planes are summed by now: their buffer takes the penalised scores)
+        GUFFIN_TRY(guffin_hip_draft_process(stream, q_logits, D.vocab, d->history, d->history_count, d->repetition_penalty, q_parts));
+        q_logits = q_parts;
+    }
     if (d->full_law) {
         GUFFIN_TRY(guffin_hip_draft_law_any(stream, q_logits, D.vocab, &opt, d->seed, d->step, nullptr, any_ws, law,
                                             full_cdf, tokens + 1, status));

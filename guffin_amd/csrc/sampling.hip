@@ -17,7 +17,7 @@
 namespace guffin {
 namespace {
 
-constexpr uint32_t kMaxTopK = 256, kMaxCandidates = 384;
+constexpr uint32_t kMaxTopK = 256, kMaxCandidates = 384, kHistoryCap = 64;
 constexpr uint64_t kMassTotal = uint64_t{1} << 32;
 constexpr uint32_t kLawFull = 0xFFFFFFFFu;  // DraftLaw::count of a law held as a full-vocabulary table
 
@@ -748,6 +748,40 @@ extern "C" int guffin_hip_draft_law(void* stream, const float* logits, uint32_t 
         return fail(GUFFIN_E_ARG, "draft_law: the compact law needs temperature > 0 and top_k in [1, 64]");
     return launch_compact_law(as_stream(stream), logits, vocab, opt, seed, step, injected_draws, workspace, law,
                               proposal, status, nullptr);
+}
+
+namespace guffin {
+namespace {
+// scores[i] = logits[i], divided by the penalty (multiplied when negative) for the tokens of the
+// sampler history: the first half of the drafter's gd_process (src/engine/gemma3_draft.mm:191-204;
+// the division by the temperature follows in the selection)
+__global__ void __launch_bounds__(256)
+draft_process_kernel(const float* __restrict__ logits, uint32_t vocab, const uint32_t* __restrict__ history,
+                     uint32_t count, float penalty, float* __restrict__ scores) {
+    __shared__ uint32_t seen[kHistoryCap];
+    if (threadIdx.x < count) seen[threadIdx.x] = history[threadIdx.x];
+    __syncthreads();
+    for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < vocab; i += gridDim.x * blockDim.x) {
+        float v = logits[i];
+        bool hit = false;
+        for (uint32_t j = 0; j < count; ++j) hit |= seen[j] == i;
+        if (hit) v = v < 0.f ? v * penalty : v / penalty;
+        scores[i] = v;
+    }
+}
+}  // namespace
+}  // namespace guffin
+
+extern "C" int guffin_hip_draft_process(void* stream, const float* logits, uint32_t vocab, const uint32_t* history,
+                                        uint32_t history_count, float repetition_penalty, float* scores) {
+    if (!logits || !scores || (history_count && !history)) return fail(GUFFIN_E_ARG, "draft_process: null pointer");
+    if (vocab == 0) return fail(GUFFIN_E_SHAPE, "draft_process: empty vocabulary");
+    if (history_count > kHistoryCap) return fail(GUFFIN_E_CAPACITY, "draft_process: at most 64 history tokens");
+    if (!std::isfinite(repetition_penalty) || !(repetition_penalty > 0.f)) return fail(GUFFIN_E_ARG, "draft_process: the penalty must be positive");
+    const uint32_t blocks = std::min<uint32_t>((vocab + 255) / 256, 1024);
+    hipLaunchKernelGGL(draft_process_kernel, dim3(blocks), dim3(256), 0, as_stream(stream), logits, vocab, history,
+                       history_count, repetition_penalty, scores);
+    return check_launch("draft_process");
 }
 
 extern "C" uint64_t guffin_hip_draft_law_any_workspace_bytes(uint32_t vocab) {

@@ -372,6 +372,14 @@ def draft_law(logits, options, seed=0, step=0, draws=None, law=None, proposal=No
     return law, proposal, status
 
 
+def draft_process(logits, history, repetition_penalty):
+    """Drafter scores: the logits with the repetition penalty on the history's tokens."""
+    scores = torch.empty_like(logits)
+    check(lib().guffin_hip_draft_process(_stream(), _p(logits), logits.numel(), _p(history), history.numel(),
+                                         C.c_float(repetition_penalty), _p(scores)))
+    return scores
+
+
 def draft_law_any(logits, options, seed=0, step=0, draws=None, status=None):
     """The drafter's law by whichever path it needs: (law, full table, proposal, status)."""
     vocab = logits.numel()

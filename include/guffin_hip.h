@@ -259,6 +259,13 @@ uint64_t guffin_hip_draft_law_workspace_bytes(uint32_t vocab);
 int guffin_hip_draft_law(void* stream, const float* logits, uint32_t vocab, const void* options,
                          uint64_t seed, uint64_t step, const void* injected_draws, void* workspace,
                          void* law, uint32_t* proposal, uint32_t* status);
+/* scores[i] = logits[i] with the repetition penalty on the tokens of the sampler history (divided
+ * when >= 0, multiplied when negative): what the drafter's gd_process does before its law is built
+ * (src/engine/gemma3_draft.mm:186-204); the law entry points then take `scores` for logits.
+ * history: at most 64 device words; scores may not alias logits. */
+int guffin_hip_draft_process(void* stream, const float* logits, uint32_t vocab, const uint32_t* history,
+                             uint32_t history_count, float repetition_penalty, float* scores);
+
 /* The drafter's law by whichever path the options and the logits need, as the reference's
  * `sample` encodes it (src/engine/gemma3_draft.mm:995-1166): the compact law when temperature > 0
  * and top_k <= 64, followed by the full-vocabulary kernels (:295-395), which run only when more

@@ -206,7 +206,13 @@ def test_h1_cycle_with_sampler_history(hip, gfo):
             torch.cuda.synchronize()
             bufs, res = plan.buffers(), plan.read_result()
             assert int(plan.status.item()) == 0 and res["status"] == 0
-            rc, law = gfo.draft_law_compact(bufs["q_logits"].cpu().numpy(), opt_cpu)
+            # the drafter penalises the same history before it builds its law (gemma3_draft.mm:186-204)
+            q_scores = bufs["q_logits"].cpu().numpy().copy()
+            hit = np.zeros(q_scores.size, bool)
+            hit[history] = True
+            r = np.float32(1.9)
+            q_scores[hit] = np.where(q_scores[hit] < 0, q_scores[hit] * r, q_scores[hit] / r)
+            rc, law = gfo.draft_law_compact(q_scores, opt_cpu)
             assert rc == 0
             word, ua, ur, un = gfo.step_draws(9, step)
             proposal = gfo.lib().gfo_draft_select(C.byref(law), C.c_uint32(word))

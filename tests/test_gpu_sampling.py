@@ -289,3 +289,35 @@ def test_accept_applies_the_repetition_penalty_to_each_rows_history(hip, gfo):
         accepted += want.accepted
         rejected += 1 - want.accepted
     assert accepted > 0 and rejected > 0
+
+
+def test_draft_side_repetition_penalty(hip, gfo):
+    """src/engine/gemma3_draft.mm:186-204: the drafter penalises the history's tokens before its law is built
+    (score < 0 ? score * r : score / r, then the temperature).  The scores equal the same float32 arithmetic in
+    numpy bit for bit, and the law built from them equals the oracle's law on those scores."""
+    import torch
+    rng = np.random.default_rng(123)
+    vocab = 16384
+    logits = rng.normal(0, 3, vocab).astype(np.float32)
+    best = np.argsort(-logits)[:6]
+    history = np.concatenate([best[:4], rng.integers(0, vocab, 40), np.argsort(logits)[:2]]).astype(np.uint32)
+    r = np.float32(1.6)
+    want = logits.copy()
+    hit = np.zeros(vocab, bool)
+    hit[history] = True
+    want[hit & (logits < 0)] = logits[hit & (logits < 0)] * r
+    want[hit & (logits >= 0)] = logits[hit & (logits >= 0)] / r
+    scores = hip.draft_process(dev(logits), dev(history), float(r))
+    assert np.array_equal(scores.cpu().numpy().view(np.uint32), want.view(np.uint32))
+    o_gpu, o_cpu = opts(hip, t=0.8, k=40), opts(gfo, t=0.8, k=40)
+    for step in range(4):
+        word = gfo.step_draws(11, step)[0]
+        check_law(hip, gfo, want, o_gpu, o_cpu, word)
+        law, proposal, st = hip.draft_law(scores, o_gpu, seed=11, step=step)
+        rc, law_cpu = gfo.draft_law_compact(want, o_cpu)
+        assert rc == 0 and int(st[0]) == 0
+        assert int(proposal[0]) == gfo.lib().gfo_draft_select(C.byref(law_cpu), C.c_uint32(word))
+    plain = gfo.draft_law_compact(logits, o_cpu)[1]
+    assert bytes(plain) != bytes(law_cpu)   # the penalty moved the law
+    with pytest.raises(hip.GuffinError):
+        hip.draft_process(dev(logits), dev(np.zeros(65, np.uint32)), 1.5)
