@@ -51,7 +51,7 @@ __device__ __forceinline__ void bitonic_desc(uint64_t* keys, uint32_t n) {
 
 __global__ void __launch_bounds__(1024)
 topk_tile_kernel(const float* __restrict__ logits, uint64_t* __restrict__ survivors, uint32_t vocab,
-                 uint32_t keep, float divisor, uint32_t* __restrict__ status) {
+                 uint32_t keep, float divisor, uint32_t* __restrict__ status, bool suppressed_ok) {
     __shared__ uint64_t keys[kTile];
     const uint32_t tile = blockIdx.x, row = blockIdx.y;
     const float* lr = logits + size_t(row) * vocab;
@@ -61,7 +61,8 @@ topk_tile_kernel(const float* __restrict__ logits, uint64_t* __restrict__ surviv
         uint64_t k = 0;  // below every real key
         if (t < vocab) {
             const float v = lr[t] / divisor;  // IEEE division: the drafter's score = logit / T
-            bad |= !isfinite(v) || !isfinite(lr[t]);
+            // -inf marks a score that its producer suppressed (a draft token without a target token)
+            bad |= (!isfinite(v) || !isfinite(lr[t])) && !(suppressed_ok && lr[t] == -INFINITY);
             k = make_key(v, t);
         }
         keys[i] = k;
@@ -292,7 +293,7 @@ extern "C" uint64_t guffin_hip_select_workspace_bytes(uint32_t rows, uint32_t vo
 namespace guffin {
 int select_candidates_scaled(hipStream_t s, const float* logits, uint32_t rows, uint32_t vocab, uint32_t retain,
                              float divisor, const uint32_t* history, const uint32_t* history_count,
-                             void* workspace, void* result, uint32_t* status);
+                             void* workspace, void* result, uint32_t* status, bool suppressed_ok = false);
 }
 
 extern "C" int guffin_hip_select_candidates(void* stream, const float* logits, uint32_t rows, uint32_t vocab,
@@ -304,7 +305,8 @@ extern "C" int guffin_hip_select_candidates(void* stream, const float* logits, u
 
 int guffin::select_candidates_scaled(hipStream_t s, const float* logits, uint32_t rows, uint32_t vocab,
                                      uint32_t retain, float divisor, const uint32_t* history,
-                                     const uint32_t* history_count, void* workspace, void* result, uint32_t* status) {
+                                     const uint32_t* history_count, void* workspace, void* result, uint32_t* status,
+                                     bool suppressed_ok) {
     if (!logits || !workspace || !result) return fail(GUFFIN_E_ARG, "select_candidates: null pointer");
     if (rows == 0 || vocab == 0) return fail(GUFFIN_E_SHAPE, "select_candidates: empty shape");
     if (retain == 0 || retain > 320) return fail(GUFFIN_E_CAPACITY, "select_candidates: retain must be in [1, 320] (top_k <= 256 plus 64 history tokens)");
@@ -313,7 +315,7 @@ int guffin::select_candidates_scaled(hipStream_t s, const float* logits, uint32_
     const uint32_t keep = retain < vocab ? retain : vocab;
     const uint32_t tiles = (vocab + kTile - 1) / kTile;
     uint64_t* surv = static_cast<uint64_t*>(workspace);
-    hipLaunchKernelGGL(topk_tile_kernel, dim3(tiles, rows), dim3(1024), 0, s, logits, surv, vocab, keep, divisor, status);
+    hipLaunchKernelGGL(topk_tile_kernel, dim3(tiles, rows), dim3(1024), 0, s, logits, surv, vocab, keep, divisor, status, suppressed_ok);
     if (int rc = check_launch("select_candidates(tile)")) return rc;
     if (tiles * keep <= 8 * 1024)
         hipLaunchKernelGGL(topk_merge_kernel<8>, dim3(rows), dim3(1024), 0, s, logits, surv, tiles * keep, vocab,

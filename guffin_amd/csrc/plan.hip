@@ -231,6 +231,16 @@ __global__ void commit_rows_kernel(const uint16_t* priv_k, const uint16_t* priv_
     }
 }
 
+// the caller's history (target ids) in the drafter's ids; a token without a draft id matches nothing
+__global__ void draft_history_kernel(const uint32_t* history, uint32_t count, const int32_t* target_to_draft, uint32_t vocab,
+                                     uint32_t* out) {
+    const uint32_t t = threadIdx.x;
+    if (t >= count) return;
+    const uint32_t token = history[t];
+    const int32_t d = token < vocab ? target_to_draft[token] : -1;
+    out[t] = d < 0 ? 0xFFFFFFFFu : static_cast<uint32_t>(d);
+}
+
 // row 0 keeps the caller's history, row 1 the same plus the proposal (oldest dropped at 64)
 __global__ void build_history_kernel(const uint32_t* history, uint32_t count, const uint32_t* proposal, uint32_t* out) {
     const uint32_t t = threadIdx.x;
@@ -243,9 +253,18 @@ __global__ void build_history_kernel(const uint32_t* history, uint32_t count, co
 }
 
 // the step's token slots: [0] root, [1] proposal (written later), [8..] the drafter's input rows
-__global__ void set_step_tokens_kernel(const uint32_t* root, const uint32_t* pending, uint32_t* words) {
+// With a vocabulary map the drafter's rows are the same tokens in its own ids; a token it does not
+// have raises GUFFIN_STATUS_BAD_TOKEN (the reference refuses such a root on the host).
+__global__ void set_step_tokens_kernel(const uint32_t* root, const uint32_t* pending, uint32_t* words,
+                                       const int32_t* target_to_draft, uint32_t target_vocab, uint32_t* status) {
+    auto drafter_id = [&](uint32_t token) {
+        if (!target_to_draft) return token;
+        const int32_t d = token < target_vocab ? target_to_draft[token] : -1;
+        if (d < 0) { atomicOr(status, GUFFIN_STATUS_BAD_TOKEN); return 0u; }
+        return static_cast<uint32_t>(d);
+    };
     words[0] = *root;
-    if (pending) { words[8] = *pending; words[9] = *root; } else { words[8] = *root; }
+    if (pending) { words[8] = drafter_id(*pending); words[9] = drafter_id(*root); } else { words[8] = drafter_id(*root); }
 }
 
 }  // namespace
@@ -427,7 +446,7 @@ StepBuffers carve_step(const guffin_h1_desc* d, void* scratch) {
     b.law = ar.take<uint8_t>(4096 + 2 * 3088);  // the compact law, then the two candidate rows
     b.cands = b.law ? b.law + 4096 : nullptr;
     b.words = ar.take<uint32_t>(16);
-    b.hist = ar.take<uint32_t>(2 * 64 + 2);
+    b.hist = ar.take<uint32_t>(3 * 64 + 2);  // then the same history in the drafter's ids (with a vocabulary map)
     if (d->full_law) {
         b.any_ws = ar.take<uint8_t>(guffin_hip_draft_law_any_workspace_bytes(D.vocab));
         b.full_cdf = ar.take<uint64_t>(uint64_t(D.vocab) + 1);
@@ -479,20 +498,39 @@ extern "C" int guffin_hip_h1_step(void* stream, const guffin_h1_desc* d, const u
     // 1. drafter: ingest (the pending proposal and) the root, project, build the proposal law, pick x
     const uint32_t dr = drafter_rows(d);
     if (dr == 2 && !d->pending_token) return fail(GUFFIN_E_ARG, "h1_step: two drafter rows need the pending token");
-    hipLaunchKernelGGL(set_step_tokens_kernel, dim3(1), dim3(1), 0, s, root_token, dr == 2 ? d->pending_token : nullptr, tokens);
+    const bool mapped = d->draft_to_target != nullptr;
+    if (mapped != (d->target_to_draft != nullptr)) return fail(GUFFIN_E_ARG, "h1_step: the vocabulary map needs its inverse");
+    if (mapped && d->full_law) return fail(GUFFIN_E_ARG, "h1_step: the vocabulary map goes with the compact law only");
+    hipLaunchKernelGGL(set_step_tokens_kernel, dim3(1), dim3(1), 0, s, root_token, dr == 2 ? d->pending_token : nullptr, tokens,
+                       d->target_to_draft, T.vocab, status);
     GUFFIN_TRY(check_launch("set_step_tokens"));
     GUFFIN_TRY(guffin_hip_forward_rows(stream, &D, tokens + 8, dr, d->drafter_position, d_scratch, d_bytes, drafter_priv_k,
                                        drafter_priv_v, d_hidden, d_hidden + hidden_receipt_offset(dr, D.hidden), status));
     GUFFIN_TRY(guffin_hip_gemv_packed(stream, D.head_dtype, D.head_tiles, d_hidden, d_hidden + hidden_receipt_offset(dr, D.hidden), q_parts,
                                       q_logits, dr, D.hidden, D.vocab));
     q_logits += uint64_t(dr - 1) * D.vocab;  // the law comes from the last ingested row (the root)
-    if (with_history && d->repetition_penalty != 1.0f) {
+    if (mapped) {
+        // gd_process -> compact law -> proposal, through the map: tokens[2] keeps the proposal in the
+        // drafter's ids, tokens[1] carries it to the verify pass in the target's
+        const uint32_t* draft_hist = nullptr;
+        if (with_history) {
+            hipLaunchKernelGGL(draft_history_kernel, dim3(1), dim3(64), 0, s, d->history, d->history_count, d->target_to_draft,
+                               T.vocab, B.hist + 2 * kHistoryWindow + 2);
+            GUFFIN_TRY(check_launch("draft_history"));
+            draft_hist = B.hist + 2 * kHistoryWindow + 2;
+        }
+        GUFFIN_TRY(guffin_hip_draft_law_mapped(stream, q_logits, D.vocab, d->draft_to_target, draft_hist,
+                                               with_history ? d->history_count : 0u, &opt, d->seed, d->step, nullptr, law_ws,
+                                               q_parts, law, tokens + 2, tokens + 1, status));
+    } else if (with_history && d->repetition_penalty != 1.0f) {
         // the proposal law sees the same history as the verify pass's first row (the head's partial
         // planes are summed by now: their buffer takes the penalised scores)
         GUFFIN_TRY(guffin_hip_draft_process(stream, q_logits, D.vocab, d->history, d->history_count, d->repetition_penalty, q_parts));
         q_logits = q_parts;
     }
-    if (d->full_law) {
+    if (mapped) {
+        // built above
+    } else if (d->full_law) {
         GUFFIN_TRY(guffin_hip_draft_law_any(stream, q_logits, D.vocab, &opt, d->seed, d->step, nullptr, any_ws, law,
                                             full_cdf, tokens + 1, status));
     } else {
@@ -517,9 +555,9 @@ extern "C" int guffin_hip_h1_step(void* stream, const guffin_h1_desc* d, const u
     GUFFIN_TRY(guffin_hip_select_candidates(stream, p_logits, 2, V, retain, hist, hist ? hist + 2 * kHistoryWindow : nullptr,
                                             sel_ws, cands, sel_status));
     // 3. accept x or draw from the residual; on acceptance draw the next root from row 1
-    GUFFIN_TRY(guffin_hip_spec_accept_history(stream, cands, law, full_cdf, D.vocab, hist,
-                                              hist ? hist + 2 * kHistoryWindow : nullptr, tokens + 1, &opt, d->seed, d->step,
-                                              nullptr, result, status));
+    GUFFIN_TRY(guffin_hip_spec_accept_mapped(stream, cands, law, full_cdf, D.vocab, d->target_to_draft, hist,
+                                             hist ? hist + 2 * kHistoryWindow : nullptr, tokens + 1, &opt, d->seed, d->step,
+                                             nullptr, result, status));
     // 4. publish: the target keeps row 0, and row 1 if x was accepted; the drafter keeps the root
     if (d->target_ring_k && d->target_ring_v) {
         GUFFIN_TRY(guffin_hip_commit_rows(stream, &T, target_priv_k, target_priv_v, d->target_ring_k, d->target_ring_v,

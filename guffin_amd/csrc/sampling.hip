@@ -131,7 +131,8 @@ draft_law_kernel(const Candidates* __restrict__ top, SamplerOptions opt, uint64_
             const uint32_t k = opt.top_k < avail ? opt.top_k : avail;
             const float cutoff = top->values[k - 1].logit;
             // entries are sorted by (score desc, token asc): the support is a prefix
-            while (n < avail && !(top->values[n].logit < cutoff)) ++n;
+            while (n < avail && !(top->values[n].logit < cutoff) && top->values[n].logit != -INFINITY) ++n;
+            if (n == 0) st = GUFFIN_STATUS_LAW_INVALID;  // nothing eligible
             if (n > 256) st = GUFFIN_STATUS_LAW_INVALID | 32u;  // support overflow: needs the full-vocabulary law
         }
         s_n = st ? 0 : n;
@@ -534,8 +535,16 @@ __device__ uint32_t select_prepared(const Prepared& p, double draw) {
     return p.token[p.count - 1];
 }
 
+// target_to_draft: null when both sides share one vocabulary; else the law lives in draft ids and a
+// target token's mass is that of the draft token mapped to it, if any (Gemma3DraftPlan::gather,
+// src/engine/gemma3_draft.mm:1570-1578)
 __device__ uint64_t law_mass(const DraftLaw* law, const uint64_t* full_cdf, uint32_t vocab, uint32_t token,
-                             uint64_t* begin) {
+                             uint64_t* begin, const int32_t* target_to_draft = nullptr) {
+    if (target_to_draft) {
+        const int32_t draft = target_to_draft[token];
+        if (draft < 0) { if (begin) *begin = 0; return 0; }
+        token = static_cast<uint32_t>(draft);
+    }
     if (law->count == kLawFull) {  // gather from the full table (src/engine/gemma3_draft.mm:1544-1545)
         if (!full_cdf || token >= vocab) { if (begin) *begin = 0; return 0; }
         if (begin) *begin = full_cdf[token];
@@ -556,7 +565,7 @@ spec_accept_kernel(const Candidates* __restrict__ rows, const DraftLaw* __restri
                    const uint64_t* __restrict__ full_cdf, uint32_t vocab, const uint32_t* __restrict__ history,
                    const uint32_t* __restrict__ history_count, const uint32_t* __restrict__ proposal_ptr, SamplerOptions opt, uint64_t seed, uint64_t step,
                    const StepDraws* __restrict__ injected, SpecResult* __restrict__ result,
-                   uint32_t* __restrict__ status) {
+                   uint32_t* __restrict__ status, const int32_t* __restrict__ target_to_draft) {
     __shared__ Scratch sc;
     __shared__ Prepared target, residual;
     __shared__ uint64_t q[kMaxTopK];
@@ -572,7 +581,7 @@ spec_accept_kernel(const Candidates* __restrict__ rows, const DraftLaw* __restri
     }
     // history: [2][64] token ids and their counts per row (null: no repetition history)
     int rc = prepare_distribution(&rows[0], opt, history, history ? history_count[0] : 0u, sc, target);
-    if (!rc && t < target.count) q[t] = law_mass(law, full_cdf, vocab, target.token[t], nullptr);
+    if (!rc && t < target.count) q[t] = law_mass(law, full_cdf, vocab, target.token[t], nullptr, target_to_draft);
     __syncthreads();
     if (t == 0) {
         int code = rc;
@@ -582,7 +591,7 @@ spec_accept_kernel(const Candidates* __restrict__ rows, const DraftLaw* __restri
         if (!code) { normalization = validated_total(target); if (normalization < 0.0) code = -21; }
         uint64_t begin = 0, proposal_mass = 0;
         if (!code) {
-            proposal_mass = law_mass(law, full_cdf, vocab, proposal, &begin);
+            proposal_mass = law_mass(law, full_cdf, vocab, proposal, &begin, target_to_draft);
             if (proposal_mass == 0 || proposal_mass > kMassTotal || begin > kMassTotal - proposal_mass) code = -22;
         }
         bool in_target = false;
@@ -651,7 +660,7 @@ spec_accept_kernel(const Candidates* __restrict__ rows, const DraftLaw* __restri
 
 int select_candidates_scaled(hipStream_t s, const float* logits, uint32_t rows, uint32_t vocab, uint32_t retain,
                              float divisor, const uint32_t* history, const uint32_t* history_count,
-                             void* workspace, void* result, uint32_t* status);
+                             void* workspace, void* result, uint32_t* status, bool suppressed_ok = false);
 
 }  // namespace guffin
 
@@ -695,13 +704,13 @@ bool compact_options(const SamplerOptions& o) { return o.temperature > 0.f && o.
 
 int launch_compact_law(hipStream_t s, const float* logits, uint32_t vocab, const SamplerOptions& opt, uint64_t seed,
                        uint64_t step, const void* injected_draws, void* workspace, void* law, uint32_t* proposal,
-                       uint32_t* status, uint32_t* full_error) {
+                       uint32_t* status, uint32_t* full_error, bool suppressed_ok = false) {
     const uint64_t tiles = (uint64_t(vocab) + 2047) / 2048;
     uint8_t* ws = static_cast<uint8_t*>(workspace);
     Candidates* top = reinterpret_cast<Candidates*>(ws + ((tiles * 257 * 8 + 15) & ~uint64_t{15}));
     // the k-th best score and every tie with it: the best 257 scores decide both
     if (int rc = select_candidates_scaled(s, logits, 1, vocab, vocab < 257 ? vocab : 257, opt.temperature, nullptr,
-                                          nullptr, ws, top, status))
+                                          nullptr, ws, top, status, suppressed_ok))
         return rc;
     hipLaunchKernelGGL(draft_law_kernel, dim3(1), dim3(256), 0, s, top, opt, seed, step,
                        static_cast<const StepDraws*>(injected_draws), static_cast<DraftLaw*>(law), proposal, status,
@@ -753,21 +762,35 @@ extern "C" int guffin_hip_draft_law(void* stream, const float* logits, uint32_t 
 namespace guffin {
 namespace {
 // scores[i] = logits[i], divided by the penalty (multiplied when negative) for the tokens of the
-// sampler history: the first half of the drafter's gd_process (src/engine/gemma3_draft.mm:191-204;
-// the division by the temperature follows in the selection)
+// sampler history, and -inf for a draft token that the vocabulary map gives no target token: the
+// drafter's gd_process without its division by the temperature, which follows in the selection
+// (src/engine/gemma3_draft.mm:191-204).  With a map the raw logits are validated here, the
+// suppressed ones included.
 __global__ void __launch_bounds__(256)
 draft_process_kernel(const float* __restrict__ logits, uint32_t vocab, const uint32_t* __restrict__ history,
-                     uint32_t count, float penalty, float* __restrict__ scores) {
+                     uint32_t count, float penalty, const int32_t* __restrict__ draft_to_target,
+                     float* __restrict__ scores, uint32_t* __restrict__ status) {
     __shared__ uint32_t seen[kHistoryCap];
     if (threadIdx.x < count) seen[threadIdx.x] = history[threadIdx.x];
     __syncthreads();
+    bool bad = false;
     for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < vocab; i += gridDim.x * blockDim.x) {
         float v = logits[i];
+        bad |= !isfinite(v);
         bool hit = false;
         for (uint32_t j = 0; j < count; ++j) hit |= seen[j] == i;
-        if (hit) v = v < 0.f ? v * penalty : v / penalty;
+        if (hit && penalty != 1.0f) v = v < 0.f ? v * penalty : v / penalty;
+        if (draft_to_target && draft_to_target[i] < 0) v = -INFINITY;
         scores[i] = v;
     }
+    if (bad && draft_to_target && status) atomicOr(status, GUFFIN_STATUS_NONFINITE);
+}
+
+// proposal in draft ids -> the target's id for it
+__global__ void map_proposal_kernel(const int32_t* __restrict__ draft_to_target, uint32_t vocab,
+                                    const uint32_t* __restrict__ draft_proposal, uint32_t* __restrict__ target_proposal) {
+    const uint32_t d = *draft_proposal;
+    *target_proposal = d < vocab && draft_to_target[d] >= 0 ? static_cast<uint32_t>(draft_to_target[d]) : 0xFFFFFFFFu;
 }
 }  // namespace
 }  // namespace guffin
@@ -780,8 +803,36 @@ extern "C" int guffin_hip_draft_process(void* stream, const float* logits, uint3
     if (!std::isfinite(repetition_penalty) || !(repetition_penalty > 0.f)) return fail(GUFFIN_E_ARG, "draft_process: the penalty must be positive");
     const uint32_t blocks = std::min<uint32_t>((vocab + 255) / 256, 1024);
     hipLaunchKernelGGL(draft_process_kernel, dim3(blocks), dim3(256), 0, as_stream(stream), logits, vocab, history,
-                       history_count, repetition_penalty, scores);
+                       history_count, repetition_penalty, static_cast<const int32_t*>(nullptr), scores,
+                       static_cast<uint32_t*>(nullptr));
     return check_launch("draft_process");
+}
+
+extern "C" int guffin_hip_draft_law_mapped(void* stream, const float* logits, uint32_t vocab, const int32_t* draft_to_target,
+                                           const uint32_t* history, uint32_t history_count, const void* options,
+                                           uint64_t seed, uint64_t step, const void* injected_draws, void* workspace,
+                                           float* scores, void* law, uint32_t* draft_proposal, uint32_t* target_proposal,
+                                           uint32_t* status) {
+    if (!logits || !draft_to_target || !options || !workspace || !scores || !law || !draft_proposal || !target_proposal || !status
+        || (history_count && !history))
+        return fail(GUFFIN_E_ARG, "draft_law_mapped: null pointer");
+    if (vocab == 0) return fail(GUFFIN_E_SHAPE, "draft_law_mapped: empty vocabulary");
+    if (history_count > kHistoryCap) return fail(GUFFIN_E_CAPACITY, "draft_law_mapped: at most 64 history tokens");
+    if (reinterpret_cast<uintptr_t>(workspace) & 15u) return fail(GUFFIN_E_ALIGN, "draft_law_mapped: workspace must be 16-byte aligned");
+    const SamplerOptions opt = *static_cast<const SamplerOptions*>(options);
+    if (!compact_options(opt))
+        return fail(GUFFIN_E_ARG, "draft_law_mapped: the compact law needs temperature > 0 and top_k in [1, 64]");
+    if (!std::isfinite(opt.repetition_penalty) || !(opt.repetition_penalty > 0.f)) return fail(GUFFIN_E_ARG, "draft_law_mapped: the penalty must be positive");
+    hipStream_t s = as_stream(stream);
+    const uint32_t blocks = std::min<uint32_t>((vocab + 255) / 256, 1024);
+    hipLaunchKernelGGL(draft_process_kernel, dim3(blocks), dim3(256), 0, s, logits, vocab, history, history_count,
+                       opt.repetition_penalty, draft_to_target, scores, status);
+    if (int rc = check_launch("draft_process")) return rc;
+    if (int rc = launch_compact_law(s, scores, vocab, opt, seed, step, injected_draws, workspace, law, draft_proposal, status,
+                                    nullptr, true))
+        return rc;
+    hipLaunchKernelGGL(map_proposal_kernel, dim3(1), dim3(1), 0, s, draft_to_target, vocab, draft_proposal, target_proposal);
+    return check_launch("map_proposal");
 }
 
 extern "C" uint64_t guffin_hip_draft_law_any_workspace_bytes(uint32_t vocab) {
@@ -816,19 +867,29 @@ extern "C" int guffin_hip_draft_law_any(void* stream, const float* logits, uint3
     return launch_full_law(s, logits, vocab, opt, seed, step, injected_draws, nullptr, ws, full_cdf, proposal, status);
 }
 
-extern "C" int guffin_hip_spec_accept_history(void* stream, const void* target_candidates, const void* law,
-                                              const uint64_t* full_cdf, uint32_t vocab, const uint32_t* history,
-                                              const uint32_t* history_count, const uint32_t* proposal,
-                                              const void* options, uint64_t seed, uint64_t step,
-                                              const void* injected_draws, void* result, uint32_t* status) {
+extern "C" int guffin_hip_spec_accept_mapped(void* stream, const void* target_candidates, const void* law,
+                                             const uint64_t* full_cdf, uint32_t vocab, const int32_t* target_to_draft,
+                                             const uint32_t* history, const uint32_t* history_count,
+                                             const uint32_t* proposal, const void* options, uint64_t seed, uint64_t step,
+                                             const void* injected_draws, void* result, uint32_t* status) {
     if (!target_candidates || !law || !proposal || !options || !result) return fail(GUFFIN_E_ARG, "spec_accept: null pointer");
     if ((history == nullptr) != (history_count == nullptr)) return fail(GUFFIN_E_ARG, "spec_accept: history needs its counts");
     const SamplerOptions opt = *static_cast<const SamplerOptions*>(options);
     hipLaunchKernelGGL(spec_accept_kernel, dim3(1), dim3(512), 0, as_stream(stream),
                        static_cast<const Candidates*>(target_candidates), static_cast<const DraftLaw*>(law), full_cdf,
                        vocab, history, history_count, proposal, opt, seed, step,
-                       static_cast<const StepDraws*>(injected_draws), static_cast<SpecResult*>(result), status);
+                       static_cast<const StepDraws*>(injected_draws), static_cast<SpecResult*>(result), status,
+                       target_to_draft);
     return check_launch("spec_accept");
+}
+
+extern "C" int guffin_hip_spec_accept_history(void* stream, const void* target_candidates, const void* law,
+                                              const uint64_t* full_cdf, uint32_t vocab, const uint32_t* history,
+                                              const uint32_t* history_count, const uint32_t* proposal,
+                                              const void* options, uint64_t seed, uint64_t step,
+                                              const void* injected_draws, void* result, uint32_t* status) {
+    return guffin_hip_spec_accept_mapped(stream, target_candidates, law, full_cdf, vocab, nullptr, history, history_count,
+                                         proposal, options, seed, step, injected_draws, result, status);
 }
 
 extern "C" int guffin_hip_spec_accept_law(void* stream, const void* target_candidates, const void* law,

@@ -380,6 +380,33 @@ def draft_process(logits, history, repetition_penalty):
     return scores
 
 
+def draft_law_mapped(logits, draft_to_target, options, history=None, seed=0, step=0, draws=None, status=None):
+    """(law in draft ids, draft proposal, target proposal, status) with the drafter's vocabulary map."""
+    vocab = logits.numel()
+    lib().guffin_hip_draft_law_workspace_bytes.restype = C.c_uint64
+    workspace = _bytes(lib().guffin_hip_draft_law_workspace_bytes(vocab))
+    scores = torch.empty_like(logits)
+    law = _bytes(law_dtype.itemsize)
+    draft = torch.zeros(1, dtype=torch.int32, device=logits.device)
+    target = torch.zeros(1, dtype=torch.int32, device=logits.device)
+    if status is None:
+        status = torch.zeros(1, dtype=torch.int32, device=logits.device)
+    check(lib().guffin_hip_draft_law_mapped(_stream(), _p(logits), vocab, _p(draft_to_target), _p(history),
+                                            0 if history is None else history.numel(), C.byref(options),
+                                            C.c_uint64(seed), C.c_uint64(step), _p(draws), _p(workspace), _p(scores),
+                                            _p(law), _p(draft), _p(target), _p(status)))
+    return law, draft, target, status
+
+
+def spec_accept_mapped(cands, law, target_to_draft, proposal, options, history=None, history_count=None, seed=0,
+                       step=0, draws=None, status=None):
+    result = _bytes(result_dtype.itemsize)
+    check(lib().guffin_hip_spec_accept_mapped(_stream(), _p(cands), _p(law), None, 0, _p(target_to_draft), _p(history),
+                                              _p(history_count), _p(proposal), C.byref(options), C.c_uint64(seed),
+                                              C.c_uint64(step), _p(draws), _p(result), _p(status)))
+    return result
+
+
 def draft_law_any(logits, options, seed=0, step=0, draws=None, status=None):
     """The drafter's law by whichever path it needs: (law, full table, proposal, status)."""
     vocab = logits.numel()

@@ -40,7 +40,8 @@ class H1Desc(C.Structure):
                 ("target_ring_k", C.c_void_p), ("target_ring_v", C.c_void_p),
                 ("drafter_ring_k", C.c_void_p), ("drafter_ring_v", C.c_void_p), ("full_law", C.c_uint32),
                 ("drafter_rows", C.c_uint32), ("pending_token", C.c_void_p),
-                ("history", C.c_void_p), ("history_count", C.c_uint32), ("repetition_penalty", C.c_float)]
+                ("history", C.c_void_p), ("history_count", C.c_uint32), ("repetition_penalty", C.c_float),
+                ("draft_to_target", C.c_void_p), ("target_to_draft", C.c_void_p)]
 
 
 class H1Session(C.Structure):
@@ -395,7 +396,8 @@ class H1Plan:
     """One speculative cycle: buffers, descriptor and the call into guffin_hip_h1_step."""
 
     def __init__(self, target, drafter, target_position, drafter_position, temperature=1.0, top_k=64,
-                 top_p=0.95, min_p=0.0, seed=0, publish=True, full_law=False, history=None, repetition_penalty=1.0):
+                 top_p=0.95, min_p=0.0, seed=0, publish=True, full_law=False, history=None, repetition_penalty=1.0,
+                 draft_to_target=None, target_to_draft=None):
         self.target, self.drafter = target, drafter
         d = self.desc = H1Desc()
         d.target, d.drafter = C.pointer(target.desc), C.pointer(drafter.desc)
@@ -406,6 +408,10 @@ class H1Plan:
         if history is not None:
             self.history = torch.tensor(list(history), dtype=torch.int32, device="cuda")
             d.history, d.history_count, d.repetition_penalty = self.history.data_ptr(), len(history), repetition_penalty
+        if draft_to_target is not None:
+            self.draft_to_target = torch.as_tensor(draft_to_target, dtype=torch.int32).cuda()
+            self.target_to_draft = torch.as_tensor(target_to_draft, dtype=torch.int32).cuda()
+            d.draft_to_target, d.target_to_draft = self.draft_to_target.data_ptr(), self.target_to_draft.data_ptr()
         if publish:
             d.target_ring_k, d.target_ring_v = target.ring_k_table.data_ptr(), target.ring_v_table.data_ptr()
             d.drafter_ring_k, d.drafter_ring_v = drafter.ring_k_table.data_ptr(), drafter.ring_v_table.data_ptr()
@@ -456,7 +462,7 @@ class H1Plan:
             "p_logits": view(ptrs[3], 2 * T.vocab, torch.float32).view(2, T.vocab),
             "law": view(ptrs[4], hip.law_dtype.itemsize, torch.uint8),
             "candidates": view(ptrs[5], 2 * hip.candidates_dtype.itemsize, torch.uint8),
-            "tokens": view(ptrs[6], 2, torch.int32),
+            "tokens": view(ptrs[6], 10, torch.int32),
         }
 
 

@@ -304,6 +304,27 @@ int guffin_hip_spec_accept_history(void* stream, const void* target_candidates, 
                                    const uint32_t* history_count, const uint32_t* proposal,
                                    const void* options, uint64_t seed, uint64_t step,
                                    const void* injected_draws, void* result, uint32_t* status);
+
+/* The drafter's vocabulary map (the reference's TLI map, src/engine/gemma3_draft.mm:648-675):
+ * draft_to_target[d] = the target's id of draft token d, or -1 for a draft token the target does not
+ * have; injective.  target_to_draft is its inverse over the target's vocabulary (-1 where no draft
+ * token maps).  guffin_hip_draft_law_mapped is gd_process -> compact law -> gd_compact_sample with the
+ * map: scores (scratch, [vocab] floats) = logits with the repetition penalty of `options` on the
+ * history's tokens and -inf for unmapped draft tokens (their raw logits are validated all the same:
+ * GUFFIN_STATUS_NONFINITE), the law in draft ids, the proposal in both id spaces.  workspace as for
+ * guffin_hip_draft_law.  guffin_hip_spec_accept_mapped is guffin_hip_spec_accept_history with the
+ * candidates and the proposal in target ids and masses gathered through target_to_draft
+ * (Gemma3DraftPlan::gather, :1528-1581); NULL maps mean one shared vocabulary. */
+int guffin_hip_draft_law_mapped(void* stream, const float* logits, uint32_t vocab, const int32_t* draft_to_target,
+                                const uint32_t* history, uint32_t history_count, const void* options,
+                                uint64_t seed, uint64_t step, const void* injected_draws, void* workspace,
+                                float* scores, void* law, uint32_t* draft_proposal, uint32_t* target_proposal,
+                                uint32_t* status);
+int guffin_hip_spec_accept_mapped(void* stream, const void* target_candidates, const void* law,
+                                  const uint64_t* full_cdf, uint32_t vocab, const int32_t* target_to_draft,
+                                  const uint32_t* history, const uint32_t* history_count,
+                                  const uint32_t* proposal, const void* options, uint64_t seed, uint64_t step,
+                                  const void* injected_draws, void* result, uint32_t* status);
 /* Host evaluation of the draw schedule above (out: the draws struct). */
 int guffin_hip_step_draws(uint64_t seed, uint64_t step, void* out_draws_host);
 
@@ -417,8 +438,14 @@ typedef struct guffin_h1_desc {
     const uint32_t* pending_token;  /* device; read only when drafter_rows == 2 */
     /* sampler history of the verify pass: the last <= 64 confirmed tokens, the root last (device).
      * Row 0 is sampled with the repetition penalty on these, row 1 on these plus the proposal
-     * (src/engine/sampling.cpp:430-446).  NULL / 0: no penalty.  The drafter's law is not penalised. */
+     * (src/engine/sampling.cpp:430-446).  NULL / 0: no penalty.  The drafter penalises the same tokens
+     * before it builds its law (src/engine/gemma3_draft.mm:186-204). */
     const uint32_t* history; uint32_t history_count; float repetition_penalty;
+    /* The drafter's vocabulary map and its inverse (device; see guffin_hip_draft_law_mapped): both or
+     * neither.  With them the root, the pending token and the history reach the drafter in its own ids,
+     * its law lives in its ids, and the proposal enters the verify pass in the target's.  Only with the
+     * compact law (full_law == 0). */
+    const int32_t* draft_to_target; const int32_t* target_to_draft;
 } guffin_h1_desc;
 uint64_t guffin_hip_h1_scratch_bytes(const guffin_h1_desc* desc);
 int guffin_hip_h1_step(void* stream, const guffin_h1_desc* desc, const uint32_t* root_token, void* scratch,

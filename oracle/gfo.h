@@ -129,6 +129,8 @@ typedef struct {
  * negative on invalid input. */
 int gfo_draft_law_compact(const float* logits, uint32_t vocab, const gfo_sampler_options* opt,
                           gfo_draft_law* out);
+int gfo_draft_law_compact_mapped(const float* logits, uint32_t vocab, const gfo_sampler_options* opt,
+                                 const int32_t* draft_to_target, gfo_draft_law* out);
 /* full-vocabulary law: cdf has vocab+1 entries */
 int gfo_draft_law_full(const float* logits, uint32_t vocab, const gfo_sampler_options* opt,
                        uint64_t* cdf);
@@ -157,6 +159,14 @@ int gfo_spec_accept_history(const gfo_token_logit* row0, uint32_t n0, const uint
                             const gfo_draft_law* law, uint32_t proposal, const gfo_sampler_options* opt,
                             double u_accept, double u_residual, double u_next, gfo_spec_result* out);
 /* the same decision with q gathered from a full-vocabulary table (cdf: vocab+1 entries) */
+/* the same with the drafter's vocabulary map: `law` is in draft ids, `proposal` and the rows in target
+ * ids, target_to_draft[t] = the draft id of target token t or -1 (gemma3_draft.mm:659-671, 1570-1578) */
+uint64_t gfo_law_mass_mapped(const gfo_draft_law* law, const int32_t* target_to_draft, uint32_t token, uint64_t* begin);
+int gfo_spec_accept_mapped(const gfo_token_logit* row0, uint32_t n0, const uint32_t* history0, uint32_t count0,
+                           const gfo_token_logit* row1, uint32_t n1, const uint32_t* history1, uint32_t count1,
+                           const gfo_draft_law* law, const int32_t* target_to_draft, uint32_t proposal,
+                           const gfo_sampler_options* opt, double u_accept, double u_residual, double u_next,
+                           gfo_spec_result* out);
 int gfo_spec_accept_full(const gfo_token_logit* row0, uint32_t n0, const gfo_token_logit* row1,
                          uint32_t n1, const uint64_t* cdf, uint32_t vocab, uint32_t proposal,
                          const gfo_sampler_options* opt, double u_accept, double u_residual,

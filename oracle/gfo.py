@@ -219,6 +219,14 @@ def draft_law_compact(logits, opt):
     return rc, law
 
 
+def draft_law_compact_mapped(logits, opt, draft_to_target):
+    logits = np.ascontiguousarray(logits, np.float32)
+    d2t = np.ascontiguousarray(draft_to_target, np.int32)
+    law = DraftLaw()
+    rc = lib().gfo_draft_law_compact_mapped(_ptr(logits), logits.size, C.byref(opt), _ptr(d2t), C.byref(law))
+    return rc, law
+
+
 def draft_law_full(logits, opt):
     logits = np.ascontiguousarray(logits, np.float32)
     cdf = np.zeros(logits.size + 1, np.uint64)
@@ -247,6 +255,20 @@ def spec_accept_history(row0, hist0, row1, hist1, law, proposal, opt, u_accept, 
                                        _ptr(hist1), hist1.size, C.byref(law), C.c_uint32(proposal), C.byref(opt),
                                        C.c_double(u_accept), C.c_double(u_residual), C.c_double(u_next),
                                        C.byref(out))
+    return rc, out
+
+
+def spec_accept_mapped(row0, hist0, row1, hist1, law, target_to_draft, proposal, opt, u_accept, u_residual, u_next):
+    row0 = np.ascontiguousarray(row0, token_logit)
+    row1 = np.ascontiguousarray(row1, token_logit)
+    hist0 = np.ascontiguousarray(hist0, np.uint32)
+    hist1 = np.ascontiguousarray(hist1, np.uint32)
+    t2d = np.ascontiguousarray(target_to_draft, np.int32)
+    out = SpecResult()
+    rc = lib().gfo_spec_accept_mapped(_ptr(row0), row0.size, _ptr(hist0), hist0.size, _ptr(row1), row1.size,
+                                      _ptr(hist1), hist1.size, C.byref(law), _ptr(t2d), C.c_uint32(proposal),
+                                      C.byref(opt), C.c_double(u_accept), C.c_double(u_residual), C.c_double(u_next),
+                                      C.byref(out))
     return rc, out
 
 

@@ -93,8 +93,16 @@ uint64_t law_mass(const gfo_draft_law& law, uint32_t token, uint64_t* begin) {
 }
 
 // a law as the gather sees it: compact receipt or full table (gemma3_draft.mm:1538-1556)
-struct LawView { const gfo_draft_law* compact; const uint64_t* full; uint32_t vocab; };
+// target_to_draft: the inverse of the drafter's vocabulary map (src/engine/gemma3_draft.mm:659-671), -1
+// for a target token no draft token maps to; null when both sides share one vocabulary.  The law lives in
+// draft ids; masses are looked up by target id (Gemma3DraftPlan::gather, :1570-1578).
+struct LawView { const gfo_draft_law* compact; const uint64_t* full; uint32_t vocab; const int32_t* target_to_draft = nullptr; };
 uint64_t law_mass(const LawView& law, uint32_t token, uint64_t* begin) {
+    if (law.target_to_draft) {
+        const int32_t draft = law.target_to_draft[token];
+        if (draft < 0) { if (begin) *begin = 0; return 0; }
+        token = static_cast<uint32_t>(draft);
+    }
     if (law.compact) return law_mass(*law.compact, token, begin);
     if (token >= law.vocab) { if (begin) *begin = 0; return 0; }
     if (begin) *begin = law.full[token];
@@ -204,14 +212,30 @@ int gfo_prepare_token_distribution(const gfo_token_logit* cands, uint32_t n,
     return 0;
 }
 
+static int compact_law(const float* logits, uint32_t vocab, const gfo_sampler_options* opt,
+                       const int32_t* draft_to_target, gfo_draft_law* out);
+
 int gfo_draft_law_compact(const float* logits, uint32_t vocab, const gfo_sampler_options* opt,
                           gfo_draft_law* out) {
+    return compact_law(logits, vocab, opt, nullptr, out);
+}
+
+// with the drafter's vocabulary map: a draft token without a target token (map < 0) is suppressed, its
+// raw logit is still validated (gd_process, gd_compact_collect: src/engine/gemma3_draft.mm:191-204, 237-243)
+int gfo_draft_law_compact_mapped(const float* logits, uint32_t vocab, const gfo_sampler_options* opt,
+                                 const int32_t* draft_to_target, gfo_draft_law* out) {
+    return compact_law(logits, vocab, opt, draft_to_target, out);
+}
+
+static int compact_law(const float* logits, uint32_t vocab, const gfo_sampler_options* opt,
+                       const int32_t* draft_to_target, gfo_draft_law* out) {
     if (!options_valid(*opt) || opt->temperature <= 0.0f || opt->top_k > 64) return -1;
     std::memset(out, 0, sizeof(*out));
     // gd_process: validate, score = logit / T (repetition penalty handled by the caller's logits)
     std::vector<float> score(vocab);
     for (uint32_t i = 0; i < vocab; ++i) {
         if (!std::isfinite(logits[i])) return -10;
+        if (draft_to_target && draft_to_target[i] < 0) { score[i] = -std::numeric_limits<float>::infinity(); continue; }
         float s = logits[i];
         s /= opt->temperature;
         if (!std::isfinite(s)) return -11;
@@ -226,7 +250,8 @@ int gfo_draft_law_compact(const float* logits, uint32_t vocab, const gfo_sampler
     // gd_compact_collect: every token whose score >= the k-th best (ties included)
     std::vector<Scored> v;
     for (uint32_t i = 0; i < vocab; ++i)
-        if (!(score[i] < cutoff)) v.push_back({i, score[i]});
+        if (!(draft_to_target && draft_to_target[i] < 0) && !(score[i] < cutoff)) v.push_back({i, score[i]});
+    if (v.empty()) return -12;
     if (v.size() > 256) return 1;
     const uint32_t n = static_cast<uint32_t>(v.size());
     std::sort(v.begin(), v.end(), better_scored);
@@ -474,6 +499,22 @@ int gfo_spec_accept_history(const gfo_token_logit* row0, uint32_t n0, const uint
                             double u_accept, double u_residual, double u_next, gfo_spec_result* out) {
     const RowHistory h {{history0, history1}, {count0, count1}};
     return spec_accept(row0, n0, row1, n1, LawView{law, nullptr, 0}, proposal, opt, u_accept, u_residual, u_next, out, h);
+}
+
+// Gemma3DraftPlan::gather for one target token (src/engine/gemma3_draft.mm:1570-1578): its mass under a
+// compact law in draft ids and the start of its interval; target_to_draft may be null (shared vocabulary)
+uint64_t gfo_law_mass_mapped(const gfo_draft_law* law, const int32_t* target_to_draft, uint32_t token, uint64_t* begin) {
+    return law_mass(LawView{law, nullptr, 0, target_to_draft}, token, begin);
+}
+
+int gfo_spec_accept_mapped(const gfo_token_logit* row0, uint32_t n0, const uint32_t* history0, uint32_t count0,
+                           const gfo_token_logit* row1, uint32_t n1, const uint32_t* history1, uint32_t count1,
+                           const gfo_draft_law* law, const int32_t* target_to_draft, uint32_t proposal,
+                           const gfo_sampler_options* opt, double u_accept, double u_residual, double u_next,
+                           gfo_spec_result* out) {
+    const RowHistory h {{history0, history1}, {count0, count1}};
+    return spec_accept(row0, n0, row1, n1, LawView{law, nullptr, 0, target_to_draft}, proposal, opt, u_accept, u_residual,
+                       u_next, out, h);
 }
 
 int gfo_spec_accept_full(const gfo_token_logit* row0, uint32_t n0, const gfo_token_logit* row1,

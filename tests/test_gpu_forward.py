@@ -110,7 +110,7 @@ def run_h1(hip, gfo, t_shape, d_shape, t_pos, d_pos, steps, seed, threads=8):
             assert rel_rms(bufs["drafter_hidden"].cpu().numpy()[None, :], dh) <= 1e-3
             ql = gfo.gemv(d_shape.embed_dtype, d_host.embed, dh, d_shape.vocab, threads=threads)
             assert rel_rms(bufs["q_logits"].cpu().numpy()[None, :], ql) <= 1e-3
-            toks = bufs["tokens"].cpu().numpy().view(np.uint32)
+            toks = bufs["tokens"].cpu().numpy().view(np.uint32)[:2]   # the verify pair: root, proposal
             assert toks[0] == root and toks[1] == proposal
             th, wk, wv = t_host.oracle_forward(gfo, toks, t_pos, threads=threads)
             assert rel_rms(bufs["target_hidden"].cpu().numpy(), th) <= 1e-3
@@ -268,3 +268,67 @@ def test_h1_cycle_full_size_models(hip, gfo):
     """Config 4 shapes: the 48-block 12B target at an 8192-token context with the 18-block drafter."""
     from guffin_amd import model
     accepted, plan, *_ = run_h1(hip, gfo, model.GEMMA3_12B, model.GEMMA3_270M, 8190, 4096, steps=2, seed=1, threads=16)
+
+
+def test_h1_cycle_with_a_vocabulary_map(hip, gfo):
+    """The drafter's vocabulary is a shuffled, partly unmapped view of the target's (the reference's TLI map,
+    src/engine/gemma3_draft.mm:648-675): the root reaches the drafter in its own id, the law lives in draft ids
+    without unmapped tokens, the proposal enters the verify pass in the target's id, and the decision equals the
+    oracle's with the same maps on the step's own logits."""
+    import torch
+    from dataclasses import replace
+    from guffin_amd import model
+    vocab = 8192
+    t_shape = replace(model.GEMMA3_12B, layers=2, vocab=vocab, ring_global=2048)
+    d_shape = replace(model.GEMMA3_270M, layers=2, vocab=vocab, ring_global=2048)
+    t_host, d_host = model.HostModel(t_shape, seed=51, position=300), model.HostModel(d_shape, seed=52, position=300)
+    t_host.out_norm *= np.float32(1e-4)   # bring these random models' logits to a sampler's range
+    d_host.out_norm *= np.float32(1e-2)
+    target, drafter = model.DeviceModel.from_host(t_host), model.DeviceModel.from_host(d_host)
+    rng = np.random.default_rng(8)
+    d2t = rng.permutation(vocab).astype(np.int32)
+    root = 77
+    unmapped = rng.choice(vocab, 500, replace=False)
+    unmapped = unmapped[d2t[unmapped] != root]        # the root stays known to the drafter
+    d2t[unmapped] = -1
+    t2d = np.full(vocab, -1, np.int32)
+    t2d[d2t[d2t >= 0]] = np.nonzero(d2t >= 0)[0].astype(np.int32)
+    history = np.array([5, 6, root], np.uint32)
+    plan = model.H1Plan(target, drafter, 300, 300, temperature=1.0, top_k=32, seed=3, publish=False,
+                        history=history.tolist(), repetition_penalty=1.5, draft_to_target=d2t, target_to_draft=t2d)
+    opt_cpu = gfo.SamplerOptions(1.0, 32, 0.95, 0.0, 1.5)
+    plan.root.fill_(root)
+    for step in range(6):
+        plan.step(step)
+        torch.cuda.synchronize()
+        bufs, res = plan.buffers(), plan.read_result()
+        assert int(plan.status.item()) == 0 and res["status"] == 0
+        toks = bufs["tokens"].cpu().numpy().view(np.uint32)
+        assert toks[8] == t2d[root]                                        # the drafter's input row, in its ids
+        if step == 0:   # the drafter really ran on that id
+            dh, _, _ = d_host.oracle_forward(gfo, [int(t2d[root])], 300, threads=8)
+            assert rel_rms(bufs["drafter_hidden"].cpu().numpy()[None, :], dh) <= 1e-3
+        scores = bufs["q_logits"].cpu().numpy().copy()
+        hist_draft = t2d[history]
+        r = np.float32(1.5)
+        for dtok in hist_draft[hist_draft >= 0]:
+            scores[dtok] = scores[dtok] * r if scores[dtok] < 0 else scores[dtok] / r
+        rc, law = gfo.draft_law_compact_mapped(scores, opt_cpu, d2t)
+        assert rc == 0
+        word, ua, ur, un = gfo.step_draws(3, step)
+        draft = gfo.lib().gfo_draft_select(C.byref(law), C.c_uint32(word))
+        assert toks[2] == draft and toks[1] == d2t[draft] and res["proposal"] == d2t[draft]
+        hist1 = np.concatenate([history, [d2t[draft]]]).astype(np.uint32)
+        retain = 32 + history.size + 1
+        p_logits = bufs["p_logits"].cpu().numpy()
+        r0 = gfo.select_candidates(p_logits[0], retain, history)
+        r1 = gfo.select_candidates(p_logits[1], retain, hist1)
+        rc, want = gfo.spec_accept_mapped(r0, history, r1, hist1, law, t2d, int(d2t[draft]), opt_cpu, ua, ur, un)
+        assert rc == 0
+        assert (res["accepted"], res["token"], res["next_root"]) == (want.accepted, want.token, want.next_root)
+    # a root the drafter does not have raises the bad-token bit instead of reading outside its table
+    orphan = int(np.nonzero(t2d < 0)[0][0])
+    plan.root.fill_(orphan)
+    plan.step(9)
+    torch.cuda.synchronize()
+    assert int(plan.status.item()) & 1

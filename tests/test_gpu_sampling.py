@@ -321,3 +321,81 @@ def test_draft_side_repetition_penalty(hip, gfo):
     assert bytes(plain) != bytes(law_cpu)   # the penalty moved the law
     with pytest.raises(hip.GuffinError):
         hip.draft_process(dev(logits), dev(np.zeros(65, np.uint32)), 1.5)
+
+
+def _reverse_map(draft_to_target, target_vocab):
+    t2d = np.full(target_vocab, -1, np.int32)
+    ok = draft_to_target >= 0
+    t2d[draft_to_target[ok]] = np.nonzero(ok)[0].astype(np.int32)
+    return t2d
+
+
+def test_mapped_law_reference_case_on_the_device(hip, gfo):
+    """tests/engine/gemma3_draft_tests.cpp:404-425 on the device path: law in draft ids {12, 511} with half the
+    mass each, proposals 50000 / 511 in target ids, and a NaN in an excluded raw logit still refuses."""
+    vocab = 262144
+    d2t = np.arange(vocab, dtype=np.int32)
+    d2t[12], d2t[50000] = d2t[50000], d2t[12]
+    d2t[0] = -1
+    logits = np.full(vocab, -100, np.float32)
+    logits[0], logits[12], logits[511] = 100, 0, 0
+    o = hip.SamplerOptions(1.0, 1, 1.0, 0.0, 1.0)
+    half = 1 << 31
+    for word, draft_want, target_want in ((0, 12, 50000), (0xFFFFFFFF, 511, 511)):
+        draws = np.zeros(1, hip.draws_dtype)
+        draws["word"] = word
+        draws["u_accept"], draws["u_residual"], draws["u_next"] = 0.5, 0.5, 0.5
+        law, draft, target, status = hip.draft_law_mapped(dev(logits), dev(d2t), o, draws=dev(draws.view(np.uint8)))
+        got = law_np(hip, law)
+        assert int(status[0]) == 0 and got["count"] == 2
+        assert list(got["ids"][:2]) == [12, 511] and list(got["cdf"][:3]) == [0, half, 2 * half]
+        assert int(draft[0]) == draft_want and int(target[0]) == target_want
+    logits[0] = np.nan
+    status = hip.draft_law_mapped(dev(logits), dev(d2t), o)[3]
+    assert int(status[0]) & 2
+
+
+def test_mapped_law_and_accept_against_the_oracle(hip, gfo):
+    """A drafter vocabulary that is a shuffled, partly unmapped view of the target's: the law (draft ids), the
+    proposal in both id spaces and every accept / residual decision equal the oracle's with the same maps."""
+    import torch
+    rng = np.random.default_rng(321)
+    vocab, k = 8192, 24
+    perm = rng.permutation(vocab).astype(np.int32)
+    d2t = perm.copy()
+    d2t[rng.choice(vocab, 700, replace=False)] = -1            # draft tokens the target does not have
+    t2d = _reverse_map(d2t, vocab)
+    o_gpu, o_cpu = hip.SamplerOptions(0.9, k, 0.95, 0.0, 1.3), gfo.SamplerOptions(0.9, k, 0.95, 0.0, 1.3)
+    accepted = rejected = unmapped_best = 0
+    for trial in range(30):
+        p_logits = rng.normal(0, 3, (2, vocab)).astype(np.float32)
+        # the drafter sees the target's row 0 through the map, plus noise
+        q_logits = np.where(d2t >= 0, p_logits[0][np.maximum(d2t, 0)], 0).astype(np.float32) + rng.normal(0, 1, vocab).astype(np.float32)
+        unmapped_best += int(d2t[int(np.argmax(q_logits))] < 0)
+        hist_draft = rng.integers(0, vocab, 12).astype(np.uint32)           # draft-side history, draft ids
+        law, draft, target, st = hip.draft_law_mapped(dev(q_logits), dev(d2t), o_gpu, history=dev(hist_draft), seed=5, step=trial)
+        r = np.float32(1.3)
+        scores = q_logits.copy()
+        hit = np.zeros(vocab, bool)
+        hit[hist_draft] = True
+        scores[hit] = np.where(scores[hit] < 0, scores[hit] * r, scores[hit] / r)
+        rc, law_cpu = gfo.draft_law_compact_mapped(scores, o_cpu, d2t)
+        word, ua, ur, un = gfo.step_draws(5, trial)
+        d_want = gfo.lib().gfo_draft_select(C.byref(law_cpu), C.c_uint32(word))
+        got = law_np(hip, law)
+        assert rc == 0 and int(st[0]) == 0 and got["count"] == law_cpu.count
+        assert list(got["ids"][:law_cpu.count]) == [law_cpu.ids[i] for i in range(law_cpu.count)]
+        assert list(got["cdf"][:law_cpu.count + 1]) == [law_cpu.cdf[i] for i in range(law_cpu.count + 1)]
+        assert all(d2t[i] >= 0 for i in got["ids"][:law_cpu.count])
+        assert int(draft[0]) == d_want and int(target[0]) == d2t[d_want]
+        res, status = hip.select_candidates(dev(p_logits), k)
+        out = hip.spec_accept_mapped(res, law, dev(t2d), target, o_gpu, seed=5, step=trial, status=st)
+        g = out.cpu().numpy().view(hip.result_dtype)[0]
+        rows = [gfo.select_candidates(p_logits[i], k) for i in range(2)]
+        rc, want = gfo.spec_accept_mapped(rows[0], (), rows[1], (), law_cpu, t2d, int(d2t[d_want]), o_cpu, ua, ur, un)
+        assert rc == 0 and g["status"] == 0 and int(st[0]) == 0
+        assert (g["accepted"], g["token"], g["next_root"]) == (want.accepted, want.token, want.next_root), trial
+        assert abs(g["acceptance_probability"] - want.acceptance_probability) <= 1e-14
+        accepted += want.accepted
+        rejected += 1 - want.accepted
+    assert accepted > 0 and rejected > 0

@@ -348,3 +348,43 @@ def test_full_law_agrees_with_the_compact_law(gfo):
         cm = np.diff(np.array(law.cdf[:law.count + 1], dtype=np.int64))
         assert list(support) == list(ids[cm > 0])
         assert np.max(np.abs(mass[ids] - cm)) / TOTAL < 1e-6
+
+
+def reverse_map(draft_to_target, target_vocab):
+    t2d = np.full(target_vocab, -1, np.int32)
+    for d, t in enumerate(draft_to_target):
+        if t >= 0:
+            assert t2d[t] < 0   # injective
+            t2d[t] = d
+    return t2d
+
+
+def test_mapped_law_reference_case(gfo):
+    """tests/engine/gemma3_draft_tests.cpp:404-425: a compact receipt lives in draft-id order; masses are looked up
+    by target id through the map, an excluded control token gets no mass, and a NaN in an excluded raw logit
+    still refuses."""
+    vocab = 262144
+    d2t = np.arange(vocab, dtype=np.int32)
+    d2t[12], d2t[50000] = d2t[50000], d2t[12]
+    d2t[0] = -1
+    t2d = reverse_map(d2t, vocab)
+    logits = np.full(vocab, -100, np.float32)
+    logits[0], logits[12], logits[511] = 100, 0, 0
+    opt = gfo.SamplerOptions(1.0, 1, 1.0, 0.0, 1.0)
+    rc, law = gfo.draft_law_compact_mapped(logits, opt, d2t)
+    half = 1 << 31
+    assert rc == 0 and law.count == 2 and [law.ids[0], law.ids[1]] == [12, 511]
+    assert [law.cdf[i] for i in range(3)] == [0, half, 2 * half]
+    lib = gfo.lib()
+    lib.gfo_law_mass_mapped.restype = C.c_uint64
+    def mass(token):
+        begin = C.c_uint64(0)
+        m = lib.gfo_law_mass_mapped(C.byref(law), t2d.ctypes.data_as(C.c_void_p), C.c_uint32(token), C.byref(begin))
+        return m, begin.value
+    left = lib.gfo_draft_select(C.byref(law), C.c_uint32(0))
+    assert left == 12 and d2t[left] == 50000 and mass(50000) == (half, 0)
+    assert mass(0)[0] == 0 and mass(12)[0] == 0 and mass(511) == (half, half)
+    right = lib.gfo_draft_select(C.byref(law), C.c_uint32(0xFFFFFFFF))
+    assert right == 511 and d2t[right] == 511
+    logits[0] = np.nan
+    assert gfo.draft_law_compact_mapped(logits, opt, d2t)[0] == -10
