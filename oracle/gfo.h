@@ -30,6 +30,11 @@
  *                            file defines the CPU law following gemma3_draft.mm:247-294
  *                            and pins it by invariants (sum 2^32, monotone, uniform ->
  *                            equal bins, top-p 0.5 case, 1e-6 vs double softmax).
+ *   vocabulary map (mapped law, mass gather, mapped accept):
+ *                            pinned: the reference's mapped case as data (gemma3_draft_tests.cpp:
+ *                            404-425: support {12, 511}, half the mass each, proposals 50000 / 511,
+ *                            zero mass for the excluded and the unmapped token, NaN refusal); the
+ *                            law's edges share the compact law's note above
  *   philox4x32-10            pinned: Random123 known-answer vectors
  */
 #pragma once
