@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the H1 speculative decode step on one MI355X.
 
-Workload (BASELINE.json config 4): one H1 cycle of the Gemma-3-12B-shaped Q4_K_M target
+Workload (configuration 4 of the benchmark): one H1 cycle of the Gemma-3-12B-shaped Q4_K_M target
 (48 blocks, 2-row verify at an 8192-token fp16 KV context, tied Q6_K 262144 head, top-64
 selection, lossless accept) with the 270M-shaped Q8_0 drafter (1 row, 4096-token context),
 seeded random weights drawn on the device.  A step is one whole cycle replayed as a HIP

@@ -1,6 +1,6 @@
 """Synthetic Gemma-3 shaped models for the H1 step: descriptors, seeded weights, KV rings.
 
-Shapes follow BASELINE's configurations: the 12B target (48 blocks, hidden 3840, FFN 15360,
+Shapes of the benchmark configurations: the 12B target (48 blocks, hidden 3840, FFN 15360,
 16 query / 8 KV heads of 256, sliding window 1024 on 5 of every 6 blocks, Q4_K projections
 with Q6_K v_proj / down_proj and a tied Q6_K head) and the 270M drafter (18 blocks, hidden 640,
 FFN 2048, 4 query / 1 KV head, window 512, Q8_0 everywhere).  Layer policy and RoPE bases:
