@@ -189,6 +189,18 @@ def main():
     e1.record(stream)
     torch.cuda.synchronize()
     launch_us = e0.elapsed_time(e1) * 1e3 / (reps * T.layers)
+    # the same kernel dispatched alone (one launch, then a wait): the reference's benchmark reports both an
+    # isolated and a sustained mode (include/local_gguf_engine/benchmarks/quick_benchmark.hpp:13-17)
+    isolated = []
+    for rep in range(3 * T.layers):
+        L = target.layers[rep % T.layers]
+        e0.record(stream)
+        hip.check(lib.guffin_hip_gateup_geglu(hip._stream(), int(L.dtype[4]), C.c_void_p(L.tiles[4]), C.c_void_p(L.tiles[5]),
+                                              hip._p(x), hip._p(xs), hip._p(h_out), hip._p(h_sums), 2, H, F))
+        e1.record(stream)
+        torch.cuda.synchronize()
+        isolated.append(e0.elapsed_time(e1) * 1e3)
+    isolated_us = sorted(isolated)[len(isolated) // 2]
     from guffin_amd import synth
     # weights once, activation rows in (fp32 rows are the operator's input; the kernel reads their receipt), h out
     kernel_bytes = 2 * synth.weight_bytes(T.dtypes[4], H, F) + 2 * H * 4 + 2 * F * 4
@@ -223,6 +235,7 @@ def main():
             # profiles/gateup_geglu_q4k_hbm_traffic.txt (copy-calibrated: fetch x 1.9997, write x 1)
             "traffic": 67046400,
             "bytes_per_launch": kernel_bytes, "launch_us": round(launch_us, 3),
+            "sustained_dispatches": T.layers, "isolated_launch_us": round(isolated_us, 3),
         },
     }
     if not args.no_prefill:
