@@ -353,7 +353,7 @@ __device__ __forceinline__ void compute_tile(const Q8Tile& t, const half8_t a,
 // The streaming kernel: one wave = one (column tile, k-slice)
 // =======================================================================================
 // One wave: blocks [b0, b1) of column tile `ct`; returns the per-lane column sums.
-template <int DTYPE, int R>
+template <int DTYPE, int R, bool SINGLE = false>
 __device__ __forceinline__ void run_blocks(const uint8_t* __restrict__ wt, const float* __restrict__ x,
                                            const float* __restrict__ xsums, uint32_t K, uint32_t nblk,
                                            uint32_t ct, uint32_t b0, uint32_t b1, float (&acc)[R]) {
@@ -391,12 +391,20 @@ __device__ __forceinline__ void run_blocks(const uint8_t* __restrict__ wt, const
 #pragma unroll
             for (int r = 0; r < R; ++r) acc2[c][r] = 0.f;
         // (this tile and its operand together do not fit the registers: the operand is read group by group)
-        Q6Tile cur, nxt;
-        if (b0 < b1) load_tile(cur, tp, lane);
-        for (uint32_t b = b0; b < b1; ++b) {
-            if (b + 1 < b1) load_tile(nxt, tp + size_t(b + 1 - b0) * TB, lane);
-            compute_tile<R>(cur, image + size_t(b) * 2048u, keep, mult + b * 8u, K / 32, xs + b * 16u, per_row, lane, acc2);
-            cur = nxt;
+        if constexpr (SINGLE) {  // at most one block per wave: no second tile in registers, 16 waves fit a workgroup
+            Q6Tile cur;
+            if (b0 < b1) {
+                load_tile(cur, tp, lane);
+                compute_tile<R>(cur, image + size_t(b0) * 2048u, keep, mult + b0 * 8u, K / 32, xs + b0 * 16u, per_row, lane, acc2);
+            }
+        } else {
+            Q6Tile cur, nxt;
+            if (b0 < b1) load_tile(cur, tp, lane);
+            for (uint32_t b = b0; b < b1; ++b) {
+                if (b + 1 < b1) load_tile(nxt, tp + size_t(b + 1 - b0) * TB, lane);
+                compute_tile<R>(cur, image + size_t(b) * 2048u, keep, mult + b * 8u, K / 32, xs + b * 16u, per_row, lane, acc2);
+                cur = nxt;
+            }
         }
         q6_gather<R>(acc2, lane, acc);
     } else {
@@ -450,6 +458,18 @@ gemv_packed_kernel(const uint8_t* __restrict__ wt, const float* __restrict__ x, 
     const uint32_t b0 = min(slice * c.bps, c.nblk), b1 = min(b0 + c.bps, c.nblk);
     float acc[R];
     run_blocks<DTYPE, R>(wt, x, xsums, c.K, c.nblk, blockIdx.x, b0, b1, acc);
+    finish_tile<R>(acc, part, N, blockIdx.x, blockIdx.y, c.W);
+}
+
+// Q6_K with one block per wave and 16 waves per workgroup (shapes whose split leaves every wave a single block)
+template <int R>
+__global__ void __launch_bounds__(1024)
+gemv_q6k_single_kernel(const uint8_t* __restrict__ wt, const float* __restrict__ x, const float* __restrict__ xsums,
+                       float* __restrict__ part, uint32_t N, PackedCfg c) {
+    const uint32_t slice = blockIdx.y * c.W + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t b0 = min(slice, c.nblk), b1 = min(b0 + 1u, c.nblk);
+    float acc[R];
+    run_blocks<GUFFIN_Q6_K, R, true>(wt, x, xsums, c.K, c.nblk, blockIdx.x, b0, b1, acc);
     finish_tile<R>(acc, part, N, blockIdx.x, blockIdx.y, c.W);
 }
 
@@ -542,13 +562,32 @@ Split choose_split(uint32_t nblk, uint32_t tiles, uint32_t max_w, uint32_t waves
     return {bps, W, planes};
 }
 
+// The split of a single-matrix launch.  A Q6_K shape whose finest split leaves every wave one block runs
+// the single-block kernel: without a second tile in registers 16 waves fit a workgroup.
+struct PackedPlan { Split sp; bool single; };
+PackedPlan packed_plan(int dtype, uint32_t nblk, uint32_t tiles) {
+    if (dtype == GUFFIN_Q6_K) {
+        const Split wide = choose_split(nblk, tiles, 16, 16);
+        if (wide.bps == 1) return {wide, true};
+    }
+    return {choose_split(nblk, tiles, max_waves(dtype)), false};
+}
+
 template <int DTYPE>
 int launch_packed(hipStream_t s, const uint8_t* w, const float* x, const float* xsums, float* part,
                   uint32_t rows, uint32_t K, uint32_t N) {
     const uint32_t nblk = K / block_elems(DTYPE);
-    const Split sp = choose_split(nblk, N / kTileCols, max_waves(DTYPE));
+    const PackedPlan plan = packed_plan(DTYPE, nblk, N / kTileCols);
+    const Split sp = plan.sp;
     const PackedCfg c {K, nblk, sp.bps, sp.W};
     const dim3 grid(N / kTileCols, sp.planes), block(sp.W * 64);
+    if constexpr (DTYPE == GUFFIN_Q6_K) {
+        if (plan.single) {
+            if (rows == 2) hipLaunchKernelGGL((gemv_q6k_single_kernel<2>), grid, block, 0, s, w, x, xsums, part, N, c);
+            else hipLaunchKernelGGL((gemv_q6k_single_kernel<1>), grid, block, 0, s, w, x, xsums, part, N, c);
+            return check_launch("gemv_packed");
+        }
+    }
     if (rows == 2) hipLaunchKernelGGL((gemv_packed_kernel<DTYPE, 2>), grid, block, 0, s, w, x, xsums, part, N, c);
     else hipLaunchKernelGGL((gemv_packed_kernel<DTYPE, 1>), grid, block, 0, s, w, x, xsums, part, N, c);
     return check_launch("gemv_packed");
@@ -617,7 +656,7 @@ extern "C" uint64_t guffin_hip_receipt_bytes(uint32_t rows, uint32_t K) {
 
 extern "C" uint32_t guffin_hip_gemv_packed_slices(int dtype, uint32_t K, uint32_t N) {
     if (check_packed_shape("gemv_packed_slices: need K % block == 0 and N % 64 == 0", dtype, K, N)) return 0;
-    return choose_split(K / block_elems(dtype), N / kTileCols, max_waves(dtype)).planes;
+    return packed_plan(dtype, K / block_elems(dtype), N / kTileCols).sp.planes;
 }
 
 static int multi_split(const char* what, uint32_t count, const int* dtypes, const uint32_t* N, uint32_t K, Split* out, int* mode) {
@@ -717,7 +756,7 @@ extern "C" int guffin_hip_gemv_packed(void* stream, int dtype, const void* tiles
     if (reinterpret_cast<uintptr_t>(tiles) & 15u) return fail(GUFFIN_E_ALIGN, "gemv_packed: tiles must be 16-byte aligned");
     if ((reinterpret_cast<uintptr_t>(x) & 3u) || (reinterpret_cast<uintptr_t>(xsums) & 3u) || (reinterpret_cast<uintptr_t>(partials) & 3u))
         return fail(GUFFIN_E_ALIGN, "gemv_packed: fp32 pointers must be 4-byte aligned");
-    const uint32_t S = choose_split(K / block_elems(dtype), N / kTileCols, max_waves(dtype)).planes;
+    const uint32_t S = packed_plan(dtype, K / block_elems(dtype), N / kTileCols).sp.planes;
     const uint8_t* w = static_cast<const uint8_t*>(tiles);
     hipStream_t s = as_stream(stream);
     float* out = (y && S == 1) ? y : partials;  // a single plane is the result: no second launch
