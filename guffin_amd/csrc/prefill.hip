@@ -9,8 +9,10 @@
 // v_mfma_f32_16x16x32_f16 as fp16 subnormals (B), activations as an fp16 hi/lo image (A).  With
 // many rows the 16 A rows are 8 activation rows x {hi, lo}, so nothing is replicated: after
 // one MFMA lane (j, g) holds, for column 16*cg + j, rows 2g and 2g+1 of the row group as
-// (hi, lo) pairs.  A wave owns 64 columns x 32 rows (4 row groups), a workgroup 4 such waves on
-// the same tile (128 rows), so a weight tile is fetched from HBM once per 128 rows.  Q4_K folds
+// (hi, lo) pairs.  A wave owns 64 columns x 32 rows (4 row groups).  For Q6_K and Q8_0 a workgroup
+// is 4 such waves on the same tile (128 rows), each loading its own operands; for Q4_K it is 4
+// waves on 4 neighbouring tiles and the same 32 rows, which share the A operands through LDS
+// (the vector memory path, not the matrix core, bounds the kernel that does not).  Q4_K folds
 // its 6-bit scales into B (sc * q <= 945 is still an exact subnormal) and accumulates a whole
 // 256-element block inside the MFMA chain; Q6_K and Q8_0 apply the block scale and the activation
 // multiplier to each MFMA result in fp32.  The offset terms use per-(row, 32-group) sums (Q6_K:
@@ -194,7 +196,221 @@ __device__ __forceinline__ void add_offset(const float* sums, const WaveCtx& c, 
     }
 }
 
-// grid (N/64, Mpad/128), 256 threads.  y[M][N] fp32.
+// The image and the weight tile are read through buffer resources: an address is the resource
+// (scalar registers) + a wave-uniform byte offset (a scalar register) + the lane's 32-bit offset,
+// so a load costs one address register however many groups the loop walks.
+typedef uint32_t uint4_t __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_resource(const void* base, uint32_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, static_cast<int>(bytes), 0x00020000);
+}
+__device__ __forceinline__ uint4 ld16(__amdgpu_buffer_rsrc_t r, uint32_t lane_off, uint32_t uniform_off) {
+    const uint4_t v = __builtin_amdgcn_raw_buffer_load_b128(r, static_cast<int>(lane_off), static_cast<int>(uniform_off), 0);
+    return make_uint4(v[0], v[1], v[2], v[3]);
+}
+__device__ __forceinline__ float2 ld8(__amdgpu_buffer_rsrc_t r, uint32_t lane_off, uint32_t uniform_off) {
+    typedef uint32_t uint2_t __attribute__((ext_vector_type(2)));
+    const uint2_t v = __builtin_amdgcn_raw_buffer_load_b64(r, static_cast<int>(lane_off), static_cast<int>(uniform_off), 0);
+    return make_float2(__uint_as_float(v[0]), __uint_as_float(v[1]));
+}
+
+// the A operands of one 32-group for the wave's 4 row groups
+struct GroupA { half8_t a[4]; };
+
+
+// chunk CH (64 elements of K) of a Q4_K block: D[cg][rg] += A(lo group) * (sc * low nibbles) +
+// A(hi group) * (sc * high nibbles); scw holds the scale bytes of chunks 0-1 or 2-3
+template <int CH>
+__device__ __forceinline__ void q4_chunk(const GroupA& lo, const GroupA& hi, const uint4 (&q)[8], const uint32_t (&scw)[4],
+                                         float4_t (&D)[4][4]) {
+#pragma unroll
+    for (int cg = 0; cg < 4; ++cg) {
+        // the scale byte in both 16-bit fields
+        const uint32_t pair_lo = __builtin_amdgcn_perm(0u, scw[cg], (CH & 1) ? 0x0c020c02u : 0x0c000c00u);
+        const uint32_t pair_hi = __builtin_amdgcn_perm(0u, scw[cg], (CH & 1) ? 0x0c030c03u : 0x0c010c01u);
+        const uint4 piece = q[2 * cg + (CH >> 1)];
+        const uint32_t w0 = (CH & 1) ? piece.z : piece.x, w1 = (CH & 1) ? piece.w : piece.y;
+        constexpr uint32_t M = 0x000F000Fu;
+        const half8_t blo = as_half8(pk_mul(w0 & M, pair_lo), pk_mul((w0 >> 8) & M, pair_lo),
+                                     pk_mul(w1 & M, pair_lo), pk_mul((w1 >> 8) & M, pair_lo));
+        const half8_t bhi = as_half8(pk_mul((w0 >> 4) & M, pair_hi), pk_mul((w0 >> 12) & M, pair_hi),
+                                     pk_mul((w1 >> 4) & M, pair_hi), pk_mul((w1 >> 12) & M, pair_hi));
+#pragma unroll
+        for (int rg = 0; rg < 4; ++rg) D[cg][rg] = __builtin_amdgcn_mfma_f32_16x16x32_f16(lo.a[rg], blo, D[cg][rg], 0, 0, 0);
+#pragma unroll
+        for (int rg = 0; rg < 4; ++rg) D[cg][rg] = __builtin_amdgcn_mfma_f32_16x16x32_f16(hi.a[rg], bhi, D[cg][rg], 0, 0, 0);
+    }
+    // one MFMA occupies the matrix pipe for four issue slots: the next column group's operands
+    // are built in the other three
+#pragma unroll
+    for (int i = 0; i < 32; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);
+    }
+}
+
+// Q4_K with the activations shared through LDS.  The four waves of a workgroup own four
+// neighbouring column tiles and the SAME 32 rows: each wave fetches a quarter of a chunk's A
+// operands (64 elements of K: a low-nibble and a high-nibble group x 4 row groups = 8 records of
+// 1 KB) and all four read the whole chunk from LDS, which cuts the bytes that pass the vector
+// memory path per MFMA by more than half -- that path, not the matrix core, bounds the kernel
+// that loads every operand itself.  Three LDS buffers rotate: chunk c is read, c + 1 is complete,
+// c + 2 is written after the one barrier of the step.  grid (Mpad/32, ceil(N/256)), 256 threads;
+// consecutive workgroups walk the rows, so one XCD's L2 keeps an eighth of the image.
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+__global__ void __launch_bounds__(256, 2)
+prefill_gemm_q4k_kernel(const uint8_t* __restrict__ tiles, const uint8_t* __restrict__ blob, float* __restrict__ y,
+                        uint32_t M, uint32_t K, uint32_t N) {
+    constexpr uint32_t TB = kCols * block_bytes(GUFFIN_Q4_K);
+    constexpr uint32_t kStage = 8192;  // one chunk of A operands
+    __shared__ __attribute__((aligned(16))) uint8_t stage[3 * kStage];
+    const ImageLayout L = image_layout(M, K);
+    const uint32_t lane = threadIdx.x & 63, wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t j = lane & 15, lg = lane >> 4;
+    const uint32_t nblk = K / 256, nchunk = nblk * 4;
+    const uint32_t wave_row = blockIdx.x * kWaveRows;
+    if (wave_row >= M) return;  // padding rows only (the whole workgroup)
+    const uint32_t tile_index = blockIdx.y * 4 + wv;
+    const bool valid = tile_index < N / kCols;  // a wave past the last tile works on tile 0 and stores nothing
+    // addresses into the image: the resource, a wave-uniform byte offset and the lane's offset
+    struct { __amdgpu_buffer_rsrc_t blob; uint32_t image, mult, a_off, r_off, mpad, rg0, row0; } c;
+    c.mpad = L.mpad;
+    c.rg0 = wave_row / 8;
+    c.row0 = wave_row + 2 * lg;
+    c.a_off = j * 64 + lg * 16;  // A lane (i = lane % 16, s = lane / 16): row i, k-slice s
+    c.r_off = 8 * lg;            // the lane's first row inside a row group, in bytes of a float row
+    c.blob = make_resource(blob, static_cast<uint32_t>(L.bytes));
+    c.image = c.rg0 * 1024;      // the wave's first row group of group 0
+    c.mult = static_cast<uint32_t>(L.mult_off) + wave_row * 4;
+    const uint32_t smul = static_cast<uint32_t>(L.smul_off) + wave_row * 4;
+    const uint32_t sumi = static_cast<uint32_t>(L.sumi_off) + c.rg0 * 256;
+    // the sums image fills k-slice 0 only: the other lanes read past the resource's end, which a
+    // buffer load answers with zeros
+    const uint32_t sums_off = lane < 16 ? lane * 16 : 0x80000000u;
+    const __amdgpu_buffer_rsrc_t tile = make_resource(tiles + size_t(valid ? tile_index : 0) * nblk * TB, nblk * TB);
+    // this wave's share of chunk n: row group wv of its two groups
+    const uint32_t share = c.image + wv * 1024;
+    auto fetch = [&](uint32_t n, uint4& lo, uint4& hi) {
+        const uint32_t g = 2 * (n < nchunk ? n : nchunk - 1);  // past the end: the last chunk again, never read
+        lo = ld16(c.blob, c.a_off, share + g * c.mpad * 128);
+        hi = ld16(c.blob, c.a_off, share + (g + 1) * c.mpad * 128);
+    };
+    auto deposit = [&](uint32_t buffer, const uint4& lo, const uint4& hi) {
+        *reinterpret_cast<uint4*>(stage + buffer * kStage + wv * 1024 + lane * 16) = lo;
+        *reinterpret_cast<uint4*>(stage + buffer * kStage + 4096 + wv * 1024 + lane * 16) = hi;
+    };
+    float acc[4][4][2];  // [column group][row group][row of the lane]
+#pragma unroll
+    for (int cg = 0; cg < 4; ++cg)
+#pragma unroll
+        for (int rg = 0; rg < 4; ++rg) { acc[cg][rg][0] = 0.f; acc[cg][rg][1] = 0.f; }
+    uint4 q[8], hd[4], slo, shi;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) q[i] = ld16(tile, lane * 16, 1024 * i);
+#pragma unroll
+    for (int cg = 0; cg < 4; ++cg) hd[cg] = ld16(tile, j * 16, 8192 + 256 * cg);
+    fetch(0, slo, shi); deposit(0, slo, shi);
+    fetch(1, slo, shi); deposit(1, slo, shi);
+    fetch(2, slo, shi);
+    lds_barrier();  // chunks 0 and 1 are complete
+    uint32_t rd = 0, wr = 2;  // buffers of the chunk to read and of the chunk to deposit
+    float4_t D[4][4];
+    uint32_t sc_a[4], sc_b[4];
+    // one step: read chunk n's operands, barrier, deposit chunk n + 2, ask for chunk n + 3
+    auto step = [&](uint32_t n, GroupA& lo, GroupA& hi) {
+#pragma unroll
+        for (int rg = 0; rg < 4; ++rg) {
+            lo.a[rg] = __builtin_bit_cast(half8_t, *reinterpret_cast<const uint4*>(stage + rd * kStage + rg * 1024 + lane * 16));
+            hi.a[rg] = __builtin_bit_cast(half8_t, *reinterpret_cast<const uint4*>(stage + rd * kStage + 4096 + rg * 1024 + lane * 16));
+        }
+        lds_barrier();
+        deposit(wr, slo, shi);
+        fetch(n + 3, slo, shi);
+        rd = rd == 2 ? 0 : rd + 1;
+        wr = wr == 2 ? 0 : wr + 1;
+    };
+    for (uint32_t b = 0; b < nblk; ++b) {
+        const uint32_t bn = b + 1 < nblk ? b + 1 : b;   // the last block requests itself again
+        const uint32_t tn = bn * TB;
+        GroupA lo, hi;
+#pragma unroll
+        for (int cg = 0; cg < 4; ++cg) {
+            const uint4 hdr = hd[cg];
+            sc_a[cg] = hdr.y & 0x3F3F3F3Fu;
+            sc_b[cg] = (hdr.w & 0x0F0F0F0Fu) | ((hdr.y >> 2) & 0x30303030u);
+#pragma unroll
+            for (int rg = 0; rg < 4; ++rg) D[cg][rg] = float4_t{0.f, 0.f, 0.f, 0.f};
+        }
+        step(4 * b, lo, hi);
+        __builtin_amdgcn_sched_barrier(0);
+        q4_chunk<0>(lo, hi, q, sc_a, D);
+        __builtin_amdgcn_sched_barrier(0);
+        step(4 * b + 1, lo, hi);
+        __builtin_amdgcn_sched_barrier(0);
+        q4_chunk<1>(lo, hi, q, sc_a, D);
+        __builtin_amdgcn_sched_barrier(0);
+        step(4 * b + 2, lo, hi);
+        // the weights of the next block: after the A request that is awaited first
+#pragma unroll
+        for (int i = 0; i < 8; i += 2) q[i] = ld16(tile, lane * 16, tn + 1024 * i);
+#pragma unroll
+        for (int cg = 0; cg < 4; ++cg) hd[cg] = ld16(tile, j * 16, tn + 8192 + 256 * cg);
+        __builtin_amdgcn_sched_barrier(0);
+        q4_chunk<2>(lo, hi, q, sc_b, D);
+        __builtin_amdgcn_sched_barrier(0);
+        step(4 * b + 3, lo, hi);
+        // what the block's end needs travels during the last chunk: the sums image (its 8 halves
+        // are k-slice 0; the other k-slices are zero), the multipliers, and d, dmin and the minima,
+        // which are read again rather than held through the block
+        half8_t as[4];
+        float2 ms[4], mult[4];
+        uint4 hb[4];
+#pragma unroll
+        for (int rg = 0; rg < 4; ++rg) {
+            as[rg] = __builtin_bit_cast(half8_t, ld16(c.blob, sums_off + rg * 256, sumi + b * L.mpad * 32));
+            ms[rg] = ld8(c.blob, c.r_off + rg * 32, smul + b * L.mpad * 4);
+            mult[rg] = ld8(c.blob, c.r_off + rg * 32, c.mult + b * 8 * c.mpad * 4);  // shared by the block's 8 groups
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        q4_chunk<3>(lo, hi, q, sc_b, D);
+        __builtin_amdgcn_sched_barrier(0);
+        // the odd quants are consumed: the header again and the next block's quants take their registers
+#pragma unroll
+        for (int cg = 0; cg < 4; ++cg) hb[cg] = ld16(tile, j * 16, b * TB + 8192 + 256 * cg);
+#pragma unroll
+        for (int i = 1; i < 8; i += 2) q[i] = ld16(tile, lane * 16, tn + 1024 * i);
+        __builtin_amdgcn_sched_barrier(0);
+        // block done: -dmin * sum_g m_g * (sum of group g) as one more MFMA per tile, then one scale step
+#pragma unroll
+        for (int cg = 0; cg < 4; ++cg) {
+            const float d = h2f(hb[cg].x & 0xFFFFu), dmin = h2f(hb[cg].x >> 16);
+            const uint32_t mn_a = hb[cg].z & 0x3F3F3F3Fu;
+            const uint32_t mn_b = ((hb[cg].w >> 4) & 0x0F0F0F0Fu) | ((hb[cg].z >> 2) & 0x30303030u);
+            const half8_t bm = as_half8(even_bytes(mn_a), odd_bytes(mn_a), even_bytes(mn_b), odd_bytes(mn_b));
+#pragma unroll
+            for (int rg = 0; rg < 4; ++rg) {
+                const float4_t dm = __builtin_amdgcn_mfma_f32_16x16x32_f16(as[rg], bm, float4_t{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+                const float4_t dv = D[cg][rg];
+                acc[cg][rg][0] = fmaf(d * mult[rg].x, dv[0] + dv[1], fmaf(-dmin * ms[rg].x, dm[0] + dm[1], acc[cg][rg][0]));
+                acc[cg][rg][1] = fmaf(d * mult[rg].y, dv[2] + dv[3], fmaf(-dmin * ms[rg].y, dm[2] + dm[3], acc[cg][rg][1]));
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    if (!valid) return;
+#pragma unroll
+    for (int cg = 0; cg < 4; ++cg)
+#pragma unroll
+        for (int rg = 0; rg < 4; ++rg)
+#pragma unroll
+            for (int r = 0; r < 2; ++r) {
+                const uint32_t row = c.row0 + 8 * rg + r;
+                if (row < M) y[size_t(row) * N + tile_index * kCols + 16 * cg + j] = acc[cg][rg][r];
+            }
+}
+
+// Q6_K and Q8_0.  grid (N/64, Mpad/128), 256 threads.  y[M][N] fp32.
 template <int DTYPE>
 __global__ void __launch_bounds__(256, DTYPE == GUFFIN_Q6_K ? 1 : 2)
 prefill_gemm_kernel(const uint8_t* __restrict__ tiles, const uint8_t* __restrict__ blob, float* __restrict__ y,
@@ -219,97 +435,9 @@ prefill_gemm_kernel(const uint8_t* __restrict__ tiles, const uint8_t* __restrict
 #pragma unroll
         for (int rg = 0; rg < 4; ++rg) { acc[cg][rg][0] = 0.f; acc[cg][rg][1] = 0.f; }
     const uint8_t* tp = tiles + size_t(blockIdx.x) * nblk * TB;
-    [[maybe_unused]] uint4 qn[8], hn[4];
     for (uint32_t b = 0; b < nblk; ++b, tp += TB) {
-        if constexpr (DTYPE == GUFFIN_Q4_K) {
-            // sc * q <= 945 is still an exact fp16 subnormal, so the 6-bit scales are folded into B
-            // and a whole 256-element block accumulates inside the MFMA chain; d and the block's
-            // activation multiplier are applied once per block
-            // the next block's quants and headers travel while this block is multiplied
-            uint4 q[8], hd[4];
-            if (b == 0) {
-#pragma unroll
-                for (int i = 0; i < 8; ++i) q[i] = *reinterpret_cast<const uint4*>(tp + 1024 * i + lane * 16);
-#pragma unroll
-                for (int cg = 0; cg < 4; ++cg) hd[cg] = *reinterpret_cast<const uint4*>(tp + 8192 + (16 * cg + j) * 16);
-            } else {
-#pragma unroll
-                for (int i = 0; i < 8; ++i) q[i] = qn[i];
-#pragma unroll
-                for (int cg = 0; cg < 4; ++cg) hd[cg] = hn[cg];
-            }
-            if (b + 1 < nblk) {
-#pragma unroll
-                for (int i = 0; i < 8; ++i) qn[i] = *reinterpret_cast<const uint4*>(tp + TB + 1024 * i + lane * 16);
-#pragma unroll
-                for (int cg = 0; cg < 4; ++cg) hn[cg] = *reinterpret_cast<const uint4*>(tp + TB + 8192 + (16 * cg + j) * 16);
-            }
-            float d[4], dmin[4];
-            uint32_t sc_a[4], sc_b[4], mn_a[4], mn_b[4];
-#pragma unroll
-            for (int cg = 0; cg < 4; ++cg) {
-                const uint4 hdr = hd[cg];
-                d[cg] = h2f(hdr.x & 0xFFFFu); dmin[cg] = h2f(hdr.x >> 16);
-                sc_a[cg] = hdr.y & 0x3F3F3F3Fu; mn_a[cg] = hdr.z & 0x3F3F3F3Fu;
-                sc_b[cg] = (hdr.w & 0x0F0F0F0Fu) | ((hdr.y >> 2) & 0x30303030u);
-                mn_b[cg] = ((hdr.w >> 4) & 0x0F0F0F0Fu) | ((hdr.z >> 2) & 0x30303030u);
-            }
-            float4_t D[4][4];
-#pragma unroll
-            for (int cg = 0; cg < 4; ++cg)
-#pragma unroll
-                for (int rg = 0; rg < 4; ++rg) D[cg][rg] = float4_t{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int ch = 0; ch < 4; ++ch) {
-                GroupOperands lo, hi;
-                load_group(c, b * 8 + 2 * ch, lo);
-                load_group(c, b * 8 + 2 * ch + 1, hi);
-#pragma unroll
-                for (int cg = 0; cg < 4; ++cg) {
-                    const uint32_t scw = ch < 2 ? sc_a[cg] : sc_b[cg];
-                    // the scale byte in both 16-bit fields
-                    const uint32_t pair_lo = __builtin_amdgcn_perm(0u, scw, (ch & 1) ? 0x0c020c02u : 0x0c000c00u);
-                    const uint32_t pair_hi = __builtin_amdgcn_perm(0u, scw, (ch & 1) ? 0x0c030c03u : 0x0c010c01u);
-                    const uint4 piece = q[2 * cg + (ch >> 1)];
-                    const uint32_t w0 = (ch & 1) ? piece.z : piece.x, w1 = (ch & 1) ? piece.w : piece.y;
-                    constexpr uint32_t M = 0x000F000Fu;
-                    const half8_t blo = as_half8(pk_mul(w0 & M, pair_lo), pk_mul((w0 >> 8) & M, pair_lo),
-                                                 pk_mul(w1 & M, pair_lo), pk_mul((w1 >> 8) & M, pair_lo));
-                    const half8_t bhi = as_half8(pk_mul((w0 >> 4) & M, pair_hi), pk_mul((w0 >> 12) & M, pair_hi),
-                                                 pk_mul((w1 >> 4) & M, pair_hi), pk_mul((w1 >> 12) & M, pair_hi));
-#pragma unroll
-                    for (int rg = 0; rg < 4; ++rg) D[cg][rg] = __builtin_amdgcn_mfma_f32_16x16x32_f16(lo.a[rg], blo, D[cg][rg], 0, 0, 0);
-#pragma unroll
-                    for (int rg = 0; rg < 4; ++rg) D[cg][rg] = __builtin_amdgcn_mfma_f32_16x16x32_f16(hi.a[rg], bhi, D[cg][rg], 0, 0, 0);
-                }
-            }
-            // block done: -dmin * sum_g m_g * (sum of group g) as one more MFMA per tile on the sums
-            // image (its 8 halves are k-slice 0; the other k-slices are zero), then one scale step
-            GroupOperands blk;
-            load_group(c, b * 8, blk);  // the block's multipliers (shared by its 8 groups)
-            const float* smul = reinterpret_cast<const float*>(blob + L.smul_off);
-            half8_t as[4];
-            float2 ms[4];
-#pragma unroll
-            for (int rg = 0; rg < 4; ++rg) {
-                uint4 v = *reinterpret_cast<const uint4*>(blob + L.sumi_off + (size_t(b) * (L.mpad / 8) + c.rg0 + rg) * 256 + (lane & 15u) * 16);
-                if (lane >= 16) v = make_uint4(0, 0, 0, 0);
-                as[rg] = __builtin_bit_cast(half8_t, v);
-                ms[rg] = *reinterpret_cast<const float2*>(smul + size_t(b) * L.mpad + c.row0 + 8 * rg);
-            }
-#pragma unroll
-            for (int cg = 0; cg < 4; ++cg) {
-                half8_t bm = as_half8(even_bytes(mn_a[cg]), odd_bytes(mn_a[cg]), even_bytes(mn_b[cg]), odd_bytes(mn_b[cg]));
-                if (lane >= 16) bm = as_half8(0, 0, 0, 0);
-#pragma unroll
-                for (int rg = 0; rg < 4; ++rg) {
-                    const float4_t dm = __builtin_amdgcn_mfma_f32_16x16x32_f16(as[rg], bm, float4_t{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
-                    const float4_t dv = D[cg][rg];
-                    acc[cg][rg][0] = fmaf(d[cg] * blk.mult[rg].x, dv[0] + dv[1], fmaf(-dmin[cg] * ms[rg].x, dm[0] + dm[1], acc[cg][rg][0]));
-                    acc[cg][rg][1] = fmaf(d[cg] * blk.mult[rg].y, dv[2] + dv[3], fmaf(-dmin[cg] * ms[rg].y, dm[2] + dm[3], acc[cg][rg][1]));
-                }
-            }
-        } else if constexpr (DTYPE == GUFFIN_Q6_K) {
+        static_assert(DTYPE != GUFFIN_Q4_K, "Q4_K has its own kernel");
+        if constexpr (DTYPE == GUFFIN_Q6_K) {
             // q = lo + 16 hi2 (4 + 2 bits): |scale| * lo <= 1905 and |scale| * hi2 <= 381 are exact as
             // fp16 bit patterns (n < 2048 reads as n * 2^-24) and carry the scale's sign in bit 15, so
             // both parts accumulate over the whole block inside the MFMA chain.  A scale covers 16
@@ -830,11 +958,14 @@ extern "C" int guffin_hip_prefill_gemm(void* stream, int dtype, const void* tile
     if ((reinterpret_cast<uintptr_t>(tiles) & 15u) || (reinterpret_cast<uintptr_t>(image) & 255u))
         return fail(GUFFIN_E_ALIGN, "prefill_gemm: tiles need 16-byte, the image 256-byte alignment");
     const ImageLayout L = image_layout(M, K);
+    // the Q4_K kernel addresses the image with 32-bit offsets
+    if (L.bytes >= (size_t(1) << 31)) return fail(GUFFIN_E_SHAPE, "prefill_gemm: the image of M x K exceeds 2 GiB, split the rows");
     const dim3 grid(N / kCols, L.mpad / kChunkRows), block(256);
     hipStream_t s = as_stream(stream);
     const uint8_t* t = static_cast<const uint8_t*>(tiles);
     const uint8_t* im = static_cast<const uint8_t*>(image);
-    if (dtype == GUFFIN_Q4_K) hipLaunchKernelGGL(prefill_gemm_kernel<GUFFIN_Q4_K>, grid, block, 0, s, t, im, y, M, K, N);
+    if (dtype == GUFFIN_Q4_K)
+        hipLaunchKernelGGL(prefill_gemm_q4k_kernel, dim3(L.mpad / kWaveRows, (N / kCols + 3) / 4), block, 0, s, t, im, y, M, K, N);
     else if (dtype == GUFFIN_Q6_K) hipLaunchKernelGGL(prefill_gemm_kernel<GUFFIN_Q6_K>, grid, block, 0, s, t, im, y, M, K, N);
     else hipLaunchKernelGGL(prefill_gemm_kernel<GUFFIN_Q8_0>, grid, block, 0, s, t, im, y, M, K, N);
     return check_launch("prefill_gemm");
