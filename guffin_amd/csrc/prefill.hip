@@ -9,14 +9,16 @@
 // v_mfma_f32_16x16x32_f16 as fp16 subnormals (B), activations as an fp16 hi/lo image (A).  With
 // many rows the 16 A rows are 8 activation rows x {hi, lo}, so nothing is replicated: after
 // one MFMA lane (j, g) holds, for column 16*cg + j, rows 2g and 2g+1 of the row group as
-// (hi, lo) pairs.  A wave owns 64 columns x 32 rows (4 row groups).  For Q6_K and Q8_0 a workgroup
-// is 4 such waves on the same tile (128 rows), each loading its own operands; for Q4_K it is 4
-// waves on 4 neighbouring tiles and the same 32 rows, which share the A operands through LDS
-// (the vector memory path, not the matrix core, bounds the kernel that does not).  Q4_K folds
-// its 6-bit scales into B (sc * q <= 945 is still an exact subnormal) and accumulates a whole
-// 256-element block inside the MFMA chain; Q6_K and Q8_0 apply the block scale and the activation
-// multiplier to each MFMA result in fp32.  The offset terms use per-(row, 32-group) sums (Q6_K:
-// per 16-group).
+// (hi, lo) pairs.  A wave owns 32 rows (4 row groups) of 64 columns (Q4_K, Q8_0) or 32 columns
+// (Q6_K).  For Q8_0 a workgroup is 4 waves on the same tile (128 rows), each loading its own
+// operands; for Q4_K it is 4 waves on 4 neighbouring tiles and the same 32 rows, for Q6_K 4 waves
+// on the halves of 2 neighbouring tiles, which share the A operands through LDS (the vector
+// memory path, not the matrix core, bounds the kernel that does not).  The K-quants fold their
+// scales into B (Q4_K: sc * q <= 945; Q6_K: |scale| times the low four and the high two bits of q,
+// sign in bit 15 -- all still exact fp16 bit patterns) and accumulate a whole 256-element block
+// inside the MFMA chain; Q8_0 applies the block scale and the activation multiplier to each MFMA
+// result in fp32.  The offset terms (-dmin m, -32 d scale) are one more MFMA per block on an image
+// of the block's group sums (Q6_K: half-group sums); Q8_0 uses per-(row, 32-group) sums in fp32.
 //
 // Attention.  A workgroup serves 16 consecutive query rows of one KV head (all query heads of the
 // group) and walks the visible key range in tiles of 32 tokens through LDS with an online
@@ -46,11 +48,13 @@ __host__ __device__ constexpr uint32_t block_elems(int dtype) { return dtype == 
 // mult : float [K/32][Mpad]            2^(E+24) of (row, group); E is shared by the 8 groups of a
 //                                      256-element block when K is a multiple of 256
 // s32  : float [K/32][Mpad]            sum of the group's 32 activations
-// s16  : float [K/16][Mpad]            sums of 16
 // sumi : half  [K/256][Mpad/8][16][8]   (K % 256 == 0) the 8 group sums of a block as an A operand:
 //                                      same A rows, halves of groups t at {0,2,1,3,4,6,5,7}[t]
 // smul : float [K/256][Mpad]           2^(Es+24) of (row, block) for sumi
-struct ImageLayout { size_t mult_off, s32_off, s16_off, sumi_off, smul_off, bytes; uint32_t mpad; };
+// sumh : half  [K/256][Mpad/8][16][16]  (K % 256 == 0) the 16 half-group sums of a block as an A
+//                                      operand: same A rows, the sum of elements 16t..16t+15 at t
+// shml : float [K/256][Mpad]           2^(Eh+24) of (row, block) for sumh
+struct ImageLayout { size_t mult_off, s32_off, sumi_off, smul_off, sumh_off, shml_off, bytes; uint32_t mpad; };
 
 __host__ __device__ inline ImageLayout image_layout(uint32_t M, uint32_t K) {
     const uint32_t mpad = (M + kChunkRows - 1) / kChunkRows * kChunkRows;
@@ -58,10 +62,11 @@ __host__ __device__ inline ImageLayout image_layout(uint32_t M, uint32_t K) {
     L.mpad = mpad;
     L.mult_off = size_t(K / 32) * mpad * 128;  // 16 A rows x 64 B per 8 rows = 128 B per row and group
     L.s32_off = L.mult_off + size_t(K / 32) * mpad * 4;
-    L.s16_off = L.s32_off + size_t(K / 32) * mpad * 4;
-    L.sumi_off = L.s16_off + size_t(K / 16) * mpad * 4;
+    L.sumi_off = L.s32_off + size_t(K / 32) * mpad * 4;
     L.smul_off = L.sumi_off + size_t(K / 256) * mpad * 32;   // 16 A rows x 16 B per 8 rows
-    L.bytes = L.smul_off + size_t(K / 256) * mpad * 4;
+    L.sumh_off = L.smul_off + size_t(K / 256) * mpad * 4;
+    L.shml_off = L.sumh_off + size_t(K / 256) * mpad * 64;   // 16 A rows x 32 B per 8 rows
+    L.bytes = L.shml_off + size_t(K / 256) * mpad * 4;
     return L;
 }
 
@@ -93,9 +98,7 @@ prefill_pack_kernel(const float* __restrict__ x, uint8_t* __restrict__ blob, uin
     const float inv = __uint_as_float((268u - eb) << 23);
     float* mult = reinterpret_cast<float*>(blob + L.mult_off);
     float* s32 = reinterpret_cast<float*>(blob + L.s32_off);
-    float* s16 = reinterpret_cast<float*>(blob + L.s16_off);
     if (s == 0) { mult[size_t(g) * L.mpad + row] = __uint_as_float((eb + 10u) << 23); s32[size_t(g) * L.mpad + row] = sum32; }
-    if ((s & 1u) == 0) s16[size_t(2 * g + (s >> 1)) * L.mpad + row] = sum16;
     constexpr int order[8] = {0, 2, 1, 3, 4, 6, 5, 7};
     if (K % 256 == 0) {  // the block's 8 group sums as a second small A operand (hi/lo, own exponent)
         float sm = fabsf(sum32);
@@ -113,6 +116,24 @@ prefill_pack_kernel(const float* __restrict__ x, uint8_t* __restrict__ blob, uin
             *reinterpret_cast<uint16_t*>(rec) = __builtin_bit_cast(uint16_t, h);
             *reinterpret_cast<uint16_t*>(rec + 16) = __builtin_bit_cast(uint16_t, l);
             if (t8 == 0) reinterpret_cast<float*>(blob + L.smul_off)[size_t(blk) * L.mpad + row] = __uint_as_float((es + 10u) << 23);
+        }
+        // and its 16 half-group sums (Q6_K scales cover 16 elements); lanes s and s ^ 1 hold the same sum
+        float sh = fabsf(sum16);
+        sh = fmaxf(sh, __shfl_xor(sh, 2, kWave));
+        sh = fmaxf(sh, __shfl_xor(sh, 4, kWave));
+        sh = fmaxf(sh, __shfl_xor(sh, 8, kWave));
+        sh = fmaxf(sh, __shfl_xor(sh, 16, kWave));
+        uint32_t eh = __float_as_uint(sh) >> 23;
+        eh = eh < 14u ? 14u : eh > 244u ? 244u : eh;
+        if ((s & 1u) == 0) {
+            const float sv = sum16 * __uint_as_float((268u - eh) << 23);
+            const _Float16 h = static_cast<_Float16>(sv);
+            const _Float16 l = static_cast<_Float16>(sv - static_cast<float>(h));
+            const uint32_t blk = g >> 3, t16 = 2 * (g & 7u) + (s >> 1);
+            uint8_t* rec = blob + L.sumh_off + ((size_t(blk) * (L.mpad / 8) + row / 8) * 16 + 2 * (row % 8)) * 32 + t16 * 2;
+            *reinterpret_cast<uint16_t*>(rec) = __builtin_bit_cast(uint16_t, h);
+            *reinterpret_cast<uint16_t*>(rec + 32) = __builtin_bit_cast(uint16_t, l);
+            if (t16 == 0) reinterpret_cast<float*>(blob + L.shml_off)[size_t(blk) * L.mpad + row] = __uint_as_float((eh + 10u) << 23);
         }
     }
     uint32_t hi[4], lo[4];
@@ -146,12 +167,10 @@ __device__ __forceinline__ uint32_t pk_mul(uint32_t a, uint32_t b) {
 }
 // a * b + c on both 16-bit fields
 __device__ __forceinline__ uint32_t pk_mad(uint32_t a, uint32_t b, uint32_t c) {
-    uint32_t r;
-    asm("v_pk_mad_u16 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
-    return r;
-}
-__device__ __forceinline__ float sbyte(uint32_t w, int i) {
-    return i == 0 ? sb0(w) : i == 1 ? sb1(w) : i == 2 ? sb2(w) : sb3(w);
+    // vector arithmetic rather than inline assembly: the compiler's hazard handling around matrix
+    // instructions does not look into an asm statement
+    return __builtin_bit_cast(uint32_t, __builtin_bit_cast(ushort2_t, a) * __builtin_bit_cast(ushort2_t, b)
+                                            + __builtin_bit_cast(ushort2_t, c));
 }
 
 // what a wave needs of the image for one 32-group: the A operands of its 4 row groups and the
@@ -163,7 +182,7 @@ struct GroupOperands {
 
 struct WaveCtx {
     const uint8_t* image;   // + lane offset inside a (group, row group) record
-    const float* mult; const float* s32; const float* s16;
+    const float* mult; const float* s32;
     uint32_t mpad, rg0, row0;  // first row group / first of the lane's rows of row group 0
 };
 
@@ -410,9 +429,243 @@ prefill_gemm_q4k_kernel(const uint8_t* __restrict__ tiles, const uint8_t* __rest
             }
 }
 
-// Q6_K and Q8_0.  grid (N/64, Mpad/128), 256 threads.  y[M][N] fp32.
+// ---- Q6_K with the activations shared through LDS ------------------------------------------
+__device__ __forceinline__ uint32_t ld4(__amdgpu_buffer_rsrc_t r, uint32_t lane_off, uint32_t uniform_off) {
+    return __builtin_amdgcn_raw_buffer_load_b32(r, static_cast<int>(lane_off), static_cast<int>(uniform_off), 0);
+}
+
+typedef short short2_t __attribute__((ext_vector_type(2)));
+// two int8 scales (one per 16-bit field, as unsigned bytes) -> two fp16 bit patterns |s| with the
+// sign in bit 15: the half reads as s * 2^-24
+__device__ __forceinline__ uint32_t scale_patterns(uint32_t fields) {
+    const short2_t sv = __builtin_bit_cast(short2_t, fields ^ 0x00800080u) - short2_t{0x80, 0x80};
+    const uint32_t mag = __builtin_bit_cast(uint32_t, __builtin_elementwise_abs(sv));
+    return mag | (__builtin_bit_cast(uint32_t, sv) & 0x80008000u);
+}
+
+// group G (32 elements of K) of a Q6_K block for the wave's two column groups: q = lo + 16 hi2
+// (4 + 2 bits); |scale| * lo <= 1905 and |scale| * hi2 <= 381 are exact as fp16 bit patterns
+// (n < 2048 reads as n * 2^-24) and carry the scale's sign in bit 15, so both parts accumulate over
+// the whole block inside the MFMA chains Dl and Dh.  A scale covers 16 elements: lanes of k-slices
+// 0-1 take the group's first scale, 2-3 the second (sel picks that field of the pattern word).
+template <int G>
+__device__ __forceinline__ void q6_group(const GroupA& A, const uint4 (&ql)[4], const uint4 (&qh)[2], const uint32_t (&P)[2][8],
+                                         uint32_t sel, float4_t (&Dl)[2][4], float4_t (&Dh)[2][4]) {
+    constexpr int n = G >> 2, qd = G & 3, ls = qd >= 2 ? 4 : 0;
+#pragma unroll
+    for (int cc = 0; cc < 2; ++cc) {
+        const uint32_t ps = __builtin_amdgcn_perm(0u, P[cc][G], sel);
+        const uint32_t pair = ps & 0x7FFF7FFFu, sign = ps & 0x80008000u;
+        const uint4 lq = ql[2 * cc + n], hq = qh[cc];
+        const uint32_t w0 = (qd & 1) ? lq.z : lq.x, w1 = (qd & 1) ? lq.w : lq.y;
+        const uint32_t h0 = n ? hq.z : hq.x, h1 = n ? hq.w : hq.y;
+        uint32_t bl[4], bh[4];
+#pragma unroll
+        for (int k = 0; k < 2; ++k) {
+            const uint32_t w = k ? w1 : w0, h = k ? h1 : h0;
+            // the products stay below 2^11, so adding the sign bit sets it
+            bl[2 * k] = pk_mad((w >> ls) & 0x000F000Fu, pair, sign);
+            bl[2 * k + 1] = pk_mad((w >> (ls + 8)) & 0x000F000Fu, pair, sign);
+            bh[2 * k] = pk_mad((h >> (2 * qd)) & 0x00030003u, pair, sign);
+            bh[2 * k + 1] = pk_mad((h >> (8 + 2 * qd)) & 0x00030003u, pair, sign);
+        }
+        const half8_t blo = as_half8(bl[0], bl[1], bl[2], bl[3]), bhi = as_half8(bh[0], bh[1], bh[2], bh[3]);
+#pragma unroll
+        for (int rg = 0; rg < 4; ++rg) Dl[cc][rg] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A.a[rg], blo, Dl[cc][rg], 0, 0, 0);
+#pragma unroll
+        for (int rg = 0; rg < 4; ++rg) Dh[cc][rg] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A.a[rg], bhi, Dh[cc][rg], 0, 0, 0);
+    }
+}
+
+// The four waves of a workgroup own the two halves (two column groups each) of two neighbouring
+// column tiles and the SAME 32 rows, and share the A operands through LDS exactly as the Q4_K
+// kernel does (three rotating buffers of one 64-element chunk, one barrier per chunk).  The offset
+// term -32 d sum_t scale_t (sum of half-group t) is one more MFMA per block on the image of the 16
+// half-group sums.  grid (Mpad/32, ceil(N/128)), 256 threads.
+__global__ void __launch_bounds__(256, 2)
+prefill_gemm_q6k_kernel(const uint8_t* __restrict__ tiles, const uint8_t* __restrict__ blob, float* __restrict__ y,
+                        uint32_t M, uint32_t K, uint32_t N) {
+    constexpr uint32_t TB = kCols * block_bytes(GUFFIN_Q6_K);
+    constexpr uint32_t kStage = 8192;  // one chunk of A operands
+    __shared__ __attribute__((aligned(16))) uint8_t stage[3 * kStage];
+    const ImageLayout L = image_layout(M, K);
+    const uint32_t lane = threadIdx.x & 63, wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t j = lane & 15, lg = lane >> 4;
+    const uint32_t nblk = K / 256, nchunk = nblk * 4;
+    const uint32_t wave_row = blockIdx.x * kWaveRows;
+    if (wave_row >= M) return;  // padding rows only (the whole workgroup)
+    const uint32_t tile_index = blockIdx.y * 2 + (wv >> 1), half = wv & 1u;
+    const bool valid = tile_index < N / kCols;  // a wave past the last tile works on tile 0 and stores nothing
+    const uint32_t mpad = L.mpad, rg0 = wave_row / 8, row0 = wave_row + 2 * lg;
+    const uint32_t a_off = j * 64 + lg * 16;  // A lane (i = lane % 16, s = lane / 16): row i, k-slice s
+    const uint32_t r_off = 8 * lg;            // the lane's first row inside a row group, in bytes of a float row
+    const __amdgpu_buffer_rsrc_t img = make_resource(blob, static_cast<uint32_t>(L.bytes));
+    const uint32_t mult_off = static_cast<uint32_t>(L.mult_off) + wave_row * 4;
+    const uint32_t shml = static_cast<uint32_t>(L.shml_off) + wave_row * 4;
+    const uint32_t sumh = static_cast<uint32_t>(L.sumh_off) + rg0 * 512;
+    // the sums image fills k-slices 0 and 1 only: the other lanes read past the resource's end,
+    // which a buffer load answers with zeros
+    const uint32_t sums_off = lane < 32 ? j * 32 + lg * 16 : 0x80000000u;
+    const __amdgpu_buffer_rsrc_t tile = make_resource(tiles + size_t(valid ? tile_index : 0) * nblk * TB, nblk * TB);
+    const uint32_t sel = lane >= 32 ? 0x03020302u : 0x01000100u;
+    // this wave's share of chunk n: row group wv of its two groups
+    const uint32_t share = (rg0 + wv) * 1024;
+    uint4 slo, shi;
+    auto fetch = [&](uint32_t n) {
+        const uint32_t g = 2 * (n < nchunk ? n : nchunk - 1);  // past the end: the last chunk again, never read
+        slo = ld16(img, a_off, share + g * mpad * 128);
+        shi = ld16(img, a_off, share + (g + 1) * mpad * 128);
+    };
+    auto deposit = [&](uint32_t buffer) {
+        *reinterpret_cast<uint4*>(stage + buffer * kStage + wv * 1024 + lane * 16) = slo;
+        *reinterpret_cast<uint4*>(stage + buffer * kStage + 4096 + wv * 1024 + lane * 16) = shi;
+    };
+    float acc[2][4][2];  // [column group of the half][row group][row of the lane]
+#pragma unroll
+    for (int cc = 0; cc < 2; ++cc)
+#pragma unroll
+        for (int rg = 0; rg < 4; ++rg) { acc[cc][rg][0] = 0.f; acc[cc][rg][1] = 0.f; }
+    // the block's bytes of this wave's half tile: low nibbles (pieces 4 half .. 4 half + 3), high
+    // bit pairs (8 + 2 half, + 1), the 16 scales of the lane's column and the dword that holds its d
+    uint4 ql[4], qh[2], scv[2], qh_next[2], scv_next[2];
+    uint32_t dw[2], dw_next[2];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) ql[i] = ld16(tile, lane * 16, 1024 * (4 * half + i));
+#pragma unroll
+    for (int cc = 0; cc < 2; ++cc) {
+        qh[cc] = ld16(tile, lane * 16, 8192 + 1024 * (2 * half + cc));
+        scv[cc] = ld16(tile, j * 16, 12288 + 256 * (2 * half + cc));
+        dw[cc] = ld4(tile, (j >> 1) * 4, 13312 + 32 * (2 * half + cc));
+    }
+    fetch(0); deposit(0);
+    fetch(1); deposit(1);
+    fetch(2);
+    lds_barrier();  // chunks 0 and 1 are complete
+    uint32_t rd = 0, wr = 2;  // buffers of the chunk to read and of the chunk to deposit
+    // one step: read chunk n's operands, barrier, deposit chunk n + 2, ask for chunk n + 3
+    auto step = [&](uint32_t n, GroupA& lo, GroupA& hi) {
+#pragma unroll
+        for (int rg = 0; rg < 4; ++rg) {
+            lo.a[rg] = __builtin_bit_cast(half8_t, *reinterpret_cast<const uint4*>(stage + rd * kStage + rg * 1024 + lane * 16));
+            hi.a[rg] = __builtin_bit_cast(half8_t, *reinterpret_cast<const uint4*>(stage + rd * kStage + 4096 + rg * 1024 + lane * 16));
+        }
+        lds_barrier();
+        deposit(wr);
+        fetch(n + 3);
+        rd = rd == 2 ? 0 : rd + 1;
+        wr = wr == 2 ? 0 : wr + 1;
+    };
+    // one matrix instruction keeps its pipe for four issue slots: the next operands are built in the other three
+    auto interleave = [] {
+#pragma unroll
+        for (int i = 0; i < 32; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);
+        }
+    };
+    float4_t Dl[2][4], Dh[2][4];
+    uint32_t P[2][8];  // word m: the patterns of scales 2m and 2m + 1 of the lane's column
+    for (uint32_t b = 0; b < nblk; ++b) {
+        const uint32_t tn = (b + 1 < nblk ? b + 1 : b) * TB;   // the last block requests itself again
+        GroupA lo, hi;
+#pragma unroll
+        for (int cc = 0; cc < 2; ++cc) {
+            const uint32_t w[4] = {scv[cc].x, scv[cc].y, scv[cc].z, scv[cc].w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                P[cc][2 * i] = scale_patterns(__builtin_amdgcn_perm(0u, w[i], 0x0c010c00u));
+                P[cc][2 * i + 1] = scale_patterns(__builtin_amdgcn_perm(0u, w[i], 0x0c030c02u));
+            }
+#pragma unroll
+            for (int rg = 0; rg < 4; ++rg) { Dl[cc][rg] = float4_t{0.f, 0.f, 0.f, 0.f}; Dh[cc][rg] = Dl[cc][rg]; }
+        }
+        step(4 * b, lo, hi);
+        __builtin_amdgcn_sched_barrier(0);
+        q6_group<0>(lo, ql, qh, P, sel, Dl, Dh);
+        q6_group<1>(hi, ql, qh, P, sel, Dl, Dh);
+        interleave();
+        __builtin_amdgcn_sched_barrier(0);
+        step(4 * b + 1, lo, hi);
+        __builtin_amdgcn_sched_barrier(0);
+        q6_group<2>(lo, ql, qh, P, sel, Dl, Dh);
+        q6_group<3>(hi, ql, qh, P, sel, Dl, Dh);
+        interleave();
+        __builtin_amdgcn_sched_barrier(0);
+        step(4 * b + 2, lo, hi);
+        // the first 128 elements' nibbles are consumed: the next block's take their registers, and
+        // its bit pairs, scales and d are requested beside them
+        ql[0] = ld16(tile, lane * 16, tn + 1024 * (4 * half));
+        ql[2] = ld16(tile, lane * 16, tn + 1024 * (4 * half + 2));
+#pragma unroll
+        for (int cc = 0; cc < 2; ++cc) {
+            qh_next[cc] = ld16(tile, lane * 16, tn + 8192 + 1024 * (2 * half + cc));
+            scv_next[cc] = ld16(tile, j * 16, tn + 12288 + 256 * (2 * half + cc));
+            dw_next[cc] = ld4(tile, (j >> 1) * 4, tn + 13312 + 32 * (2 * half + cc));
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        q6_group<4>(lo, ql, qh, P, sel, Dl, Dh);
+        q6_group<5>(hi, ql, qh, P, sel, Dl, Dh);
+        interleave();
+        __builtin_amdgcn_sched_barrier(0);
+        step(4 * b + 3, lo, hi);
+        // what the block's end needs travels during the last chunk: the sums image and the multipliers
+        half8_t as[4];
+        float2 ms[4], mult[4];
+#pragma unroll
+        for (int rg = 0; rg < 4; ++rg) {
+            as[rg] = __builtin_bit_cast(half8_t, ld16(img, sums_off + rg * 512, sumh + b * mpad * 64));
+            ms[rg] = ld8(img, r_off + rg * 32, shml + b * mpad * 4);
+            mult[rg] = ld8(img, r_off + rg * 32, mult_off + b * 8 * mpad * 4);  // shared by the block's 8 groups
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        q6_group<6>(lo, ql, qh, P, sel, Dl, Dh);
+        q6_group<7>(hi, ql, qh, P, sel, Dl, Dh);
+        interleave();
+        __builtin_amdgcn_sched_barrier(0);
+        ql[1] = ld16(tile, lane * 16, tn + 1024 * (4 * half + 1));
+        ql[3] = ld16(tile, lane * 16, tn + 1024 * (4 * half + 3));
+        __builtin_amdgcn_sched_barrier(0);
+        // block done: the offset term as one more MFMA per column group, then one scale step
+#pragma unroll
+        for (int cc = 0; cc < 2; ++cc) {
+            const float d = h2f((dw[cc] >> (16 * (j & 1u))) & 0xFFFFu);
+            const bool upper = (lg & 1u) != 0;  // k-slice 1 holds half-groups 8..15
+            uint32_t bw[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const uint32_t first = P[cc][i], second = P[cc][4 + i];  // values, so that P stays in registers
+                bw[i] = upper ? second : first;
+            }
+            const half8_t bm = as_half8(bw[0], bw[1], bw[2], bw[3]);
+#pragma unroll
+            for (int rg = 0; rg < 4; ++rg) {
+                const float4_t dm = __builtin_amdgcn_mfma_f32_16x16x32_f16(as[rg], bm, float4_t{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+                const float4_t lo4 = Dl[cc][rg], hi4 = Dh[cc][rg];
+                acc[cc][rg][0] = fmaf(d * mult[rg].x, (lo4[0] + lo4[1]) + 16.0f * (hi4[0] + hi4[1]),
+                                      fmaf(-32.0f * d * ms[rg].x, dm[0] + dm[1], acc[cc][rg][0]));
+                acc[cc][rg][1] = fmaf(d * mult[rg].y, (lo4[2] + lo4[3]) + 16.0f * (hi4[2] + hi4[3]),
+                                      fmaf(-32.0f * d * ms[rg].y, dm[2] + dm[3], acc[cc][rg][1]));
+            }
+            qh[cc] = qh_next[cc]; scv[cc] = scv_next[cc]; dw[cc] = dw_next[cc];
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    if (!valid) return;
+#pragma unroll
+    for (int cc = 0; cc < 2; ++cc)
+#pragma unroll
+        for (int rg = 0; rg < 4; ++rg)
+#pragma unroll
+            for (int r = 0; r < 2; ++r) {
+                const uint32_t row = row0 + 8 * rg + r;
+                if (row < M) y[size_t(row) * N + tile_index * kCols + 16 * (2 * half + cc) + j] = acc[cc][rg][r];
+            }
+}
+
+// Q8_0.  grid (N/64, Mpad/128), 256 threads, four waves on the same tile (128 rows), each loading its
+// own operands.  y[M][N] fp32.
 template <int DTYPE>
-__global__ void __launch_bounds__(256, DTYPE == GUFFIN_Q6_K ? 1 : 2)
+__global__ void __launch_bounds__(256, 2)
 prefill_gemm_kernel(const uint8_t* __restrict__ tiles, const uint8_t* __restrict__ blob, float* __restrict__ y,
                     uint32_t M, uint32_t K, uint32_t N) {
     constexpr uint32_t TB = kCols * block_bytes(DTYPE);
@@ -427,7 +680,6 @@ prefill_gemm_kernel(const uint8_t* __restrict__ tiles, const uint8_t* __restrict
     c.image = blob + (lane & 15u) * 64 + (lane >> 4) * 16;  // A lane (i = lane % 16, s = lane / 16): row i, k-slice s
     c.mult = reinterpret_cast<const float*>(blob + L.mult_off);
     c.s32 = reinterpret_cast<const float*>(blob + L.s32_off);
-    c.s16 = reinterpret_cast<const float*>(blob + L.s16_off);
     if (blockIdx.y * kChunkRows + wv * kWaveRows >= M) return;  // a wave of padding rows only
     float acc[4][4][2];  // [column group][row group][row of the lane]
 #pragma unroll
@@ -436,93 +688,18 @@ prefill_gemm_kernel(const uint8_t* __restrict__ tiles, const uint8_t* __restrict
         for (int rg = 0; rg < 4; ++rg) { acc[cg][rg][0] = 0.f; acc[cg][rg][1] = 0.f; }
     const uint8_t* tp = tiles + size_t(blockIdx.x) * nblk * TB;
     for (uint32_t b = 0; b < nblk; ++b, tp += TB) {
-        static_assert(DTYPE != GUFFIN_Q4_K, "Q4_K has its own kernel");
-        if constexpr (DTYPE == GUFFIN_Q6_K) {
-            // q = lo + 16 hi2 (4 + 2 bits): |scale| * lo <= 1905 and |scale| * hi2 <= 381 are exact as
-            // fp16 bit patterns (n < 2048 reads as n * 2^-24) and carry the scale's sign in bit 15, so
-            // both parts accumulate over the whole block inside the MFMA chain.  A scale covers 16
-            // elements: lanes of k-slices 0-1 take the group's first scale, 2-3 the second.
-            const bool second = lane >= 32;
+        static_assert(DTYPE == GUFFIN_Q8_0, "Q4_K and Q6_K have their own kernels");
+        const uint4 q0 = *reinterpret_cast<const uint4*>(tp + lane * 16);
+        const uint4 q1 = *reinterpret_cast<const uint4*>(tp + 1024 + lane * 16);
+        GroupOperands o;
+        load_group(c, b, o);
 #pragma unroll
-            for (int half = 0; half < 2; ++half) {  // two column groups at a time keep the wave within 256 registers
-                uint4 ql[4], qh[2];
-#pragma unroll
-                for (int i = 0; i < 4; ++i) ql[i] = *reinterpret_cast<const uint4*>(tp + 1024 * (4 * half + i) + lane * 16);
-#pragma unroll
-                for (int i = 0; i < 2; ++i) qh[i] = *reinterpret_cast<const uint4*>(tp + 8192 + 1024 * (2 * half + i) + lane * 16);
-                float4_t Dl[2][4], Dh[2][4];
-                uint4 scv[2];
-                float d[2];
-#pragma unroll
-                for (int cc = 0; cc < 2; ++cc) {
-                    const int cg = 2 * half + cc;
-                    scv[cc] = *reinterpret_cast<const uint4*>(tp + 12288 + (16 * cg + j) * 16);
-                    d[cc] = h2f(*reinterpret_cast<const uint16_t*>(tp + 13312 + (16 * cg + j) * 2));
-#pragma unroll
-                    for (int rg = 0; rg < 4; ++rg) { Dl[cc][rg] = float4_t{0.f, 0.f, 0.f, 0.f}; Dh[cc][rg] = Dl[cc][rg]; }
-                }
-#pragma unroll
-                for (int g = 0; g < 8; ++g) {
-                    const int n = g >> 2, qd = g & 3;
-                    GroupOperands o;
-                    load_group(c, b * 8 + g, o);
-#pragma unroll
-                    for (int cc = 0; cc < 2; ++cc) {
-                        const int cg = 2 * half + cc, word = g >> 1;
-                        const uint32_t sw = word == 0 ? scv[cc].x : word == 1 ? scv[cc].y : word == 2 ? scv[cc].z : scv[cc].w;
-                        const float s_first = sbyte(sw, 2 * (g & 1)), s_second = sbyte(sw, 2 * (g & 1) + 1);
-                        const int sc = static_cast<int>(second ? s_second : s_first);
-                        const uint32_t mag = static_cast<uint32_t>(sc < 0 ? -sc : sc);
-                        const uint32_t pair = mag | (mag << 16), sign = sc < 0 ? 0x80008000u : 0u;
-                        const uint4 lq = ql[2 * cc + n], hq = qh[cc];
-                        const uint32_t w0 = (qd & 1) ? lq.z : lq.x, w1 = (qd & 1) ? lq.w : lq.y;
-                        const uint32_t h0 = n ? hq.z : hq.x, h1 = n ? hq.w : hq.y;
-                        const int ls = qd >= 2 ? 4 : 0;
-                        uint32_t bl[4], bh[4];
-#pragma unroll
-                        for (int k = 0; k < 2; ++k) {
-                            const uint32_t w = k ? w1 : w0, h = k ? h1 : h0;
-                            // the products stay below 2^11, so adding the sign bit sets it
-                            bl[2 * k] = pk_mad((w >> ls) & 0x000F000Fu, pair, sign);
-                            bl[2 * k + 1] = pk_mad((w >> (ls + 8)) & 0x000F000Fu, pair, sign);
-                            bh[2 * k] = pk_mad((h >> (2 * qd)) & 0x00030003u, pair, sign);
-                            bh[2 * k + 1] = pk_mad((h >> (8 + 2 * qd)) & 0x00030003u, pair, sign);
-                        }
-                        const half8_t blo = as_half8(bl[0], bl[1], bl[2], bl[3]), bhi = as_half8(bh[0], bh[1], bh[2], bh[3]);
-#pragma unroll
-                        for (int rg = 0; rg < 4; ++rg) {
-                            Dl[cc][rg] = __builtin_amdgcn_mfma_f32_16x16x32_f16(o.a[rg], blo, Dl[cc][rg], 0, 0, 0);
-                            Dh[cc][rg] = __builtin_amdgcn_mfma_f32_16x16x32_f16(o.a[rg], bhi, Dh[cc][rg], 0, 0, 0);
-                        }
-                        add_offset(c.s16, c, (b * 8 + g) * 2, -32.0f * d[cc] * s_first, acc[cg]);
-                        add_offset(c.s16, c, (b * 8 + g) * 2 + 1, -32.0f * d[cc] * s_second, acc[cg]);
-                    }
-                }
-                GroupOperands blk;
-                load_group(c, b * 8, blk);  // the block's multipliers (shared by its 8 groups)
-#pragma unroll
-                for (int cc = 0; cc < 2; ++cc)
-#pragma unroll
-                    for (int rg = 0; rg < 4; ++rg) {
-                        const int cg = 2 * half + cc;
-                        const float4_t lo4 = Dl[cc][rg], hi4 = Dh[cc][rg];
-                        acc[cg][rg][0] = fmaf(d[cc] * blk.mult[rg].x, (lo4[0] + lo4[1]) + 16.0f * (hi4[0] + hi4[1]), acc[cg][rg][0]);
-                        acc[cg][rg][1] = fmaf(d[cc] * blk.mult[rg].y, (lo4[2] + lo4[3]) + 16.0f * (hi4[2] + hi4[3]), acc[cg][rg][1]);
-                    }
-            }
-        } else {
-            const uint4 q0 = *reinterpret_cast<const uint4*>(tp + lane * 16);
-            const uint4 q1 = *reinterpret_cast<const uint4*>(tp + 1024 + lane * 16);
-            GroupOperands o;
-            load_group(c, b, o);
-#pragma unroll
-            for (int cg = 0; cg < 4; ++cg) {
-                const float d = h2f(*reinterpret_cast<const uint16_t*>(tp + 2048 + (16 * cg + j) * 2));
-                const uint4 piece = cg < 2 ? q0 : q1;
-                const uint32_t w0 = ((cg & 1) ? piece.z : piece.x) ^ 0x80808080u, w1 = ((cg & 1) ? piece.w : piece.y) ^ 0x80808080u;
-                mfma_scale(o, as_half8(even_bytes(w0), odd_bytes(w0), even_bytes(w1), odd_bytes(w1)), d, acc[cg]);
-                add_offset(c.s32, c, b, -128.0f * d, acc[cg]);
-            }
+        for (int cg = 0; cg < 4; ++cg) {
+            const float d = h2f(*reinterpret_cast<const uint16_t*>(tp + 2048 + (16 * cg + j) * 2));
+            const uint4 piece = cg < 2 ? q0 : q1;
+            const uint32_t w0 = ((cg & 1) ? piece.z : piece.x) ^ 0x80808080u, w1 = ((cg & 1) ? piece.w : piece.y) ^ 0x80808080u;
+            mfma_scale(o, as_half8(even_bytes(w0), odd_bytes(w0), even_bytes(w1), odd_bytes(w1)), d, acc[cg]);
+            add_offset(c.s32, c, b, -128.0f * d, acc[cg]);
         }
     }
 #pragma unroll
@@ -958,7 +1135,7 @@ extern "C" int guffin_hip_prefill_gemm(void* stream, int dtype, const void* tile
     if ((reinterpret_cast<uintptr_t>(tiles) & 15u) || (reinterpret_cast<uintptr_t>(image) & 255u))
         return fail(GUFFIN_E_ALIGN, "prefill_gemm: tiles need 16-byte, the image 256-byte alignment");
     const ImageLayout L = image_layout(M, K);
-    // the Q4_K kernel addresses the image with 32-bit offsets
+    // the Q4_K and Q6_K kernels address the image with 32-bit offsets
     if (L.bytes >= (size_t(1) << 31)) return fail(GUFFIN_E_SHAPE, "prefill_gemm: the image of M x K exceeds 2 GiB, split the rows");
     const dim3 grid(N / kCols, L.mpad / kChunkRows), block(256);
     hipStream_t s = as_stream(stream);
@@ -966,7 +1143,8 @@ extern "C" int guffin_hip_prefill_gemm(void* stream, int dtype, const void* tile
     const uint8_t* im = static_cast<const uint8_t*>(image);
     if (dtype == GUFFIN_Q4_K)
         hipLaunchKernelGGL(prefill_gemm_q4k_kernel, dim3(L.mpad / kWaveRows, (N / kCols + 3) / 4), block, 0, s, t, im, y, M, K, N);
-    else if (dtype == GUFFIN_Q6_K) hipLaunchKernelGGL(prefill_gemm_kernel<GUFFIN_Q6_K>, grid, block, 0, s, t, im, y, M, K, N);
+    else if (dtype == GUFFIN_Q6_K)
+        hipLaunchKernelGGL(prefill_gemm_q6k_kernel, dim3(L.mpad / kWaveRows, (N / kCols + 1) / 2), block, 0, s, t, im, y, M, K, N);
     else hipLaunchKernelGGL(prefill_gemm_kernel<GUFFIN_Q8_0>, grid, block, 0, s, t, im, y, M, K, N);
     return check_launch("prefill_gemm");
 }
