@@ -12,6 +12,10 @@ Extra objects on the JSON line:
                 per launch): algorithmic bytes / mean launch duration, measured with HIP events
                 around a graph of 48 back-to-back launches over the 48 blocks' own weights
                 (3.2 GB, far beyond the caches) on the launch stream.
+  configs       configs 0-3 on their own (one Q4_K GEMV at 1 row; one block's seven GEMVs at 2 rows;
+                the drafter's decode with head and argmax; the Q6_K head with selection and
+                acceptance): microseconds per unit as HIP graphs, algorithmic bytes, GB/s and the
+                fraction of the 8 TB/s HBM peak.
   prefill       config 4's second half: a 2048-token prompt through the same stack.
   cpu_baseline  the reference's own CPU row dot (oracle/_ref) or the oracle port timed on the
                 host cores on a bounded sample (one block's seven GEMVs at 2 rows, a column
@@ -29,19 +33,137 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0
 
 
+def model_bytes(sh, rows, pos):
+    """Algorithmic HBM bytes of one forward pass with its head: weights once per GEMV, activations in/out,
+    KV once per KV head."""
+    w = sh.layers * sh.layer_weight_bytes() + sh.head_bytes()
+    kv = 0
+    for l in range(sh.layers):
+        tokens = min(pos, sh.sliding_window) if sh.is_local(l) else pos
+        kv += tokens * sh.kv_width * 2 * 2
+    act = sh.layers * rows * 4 * (2 * sh.hidden * 4 + 2 * sh.q_width + 2 * sh.kv_width + 3 * sh.ffn)
+    logits = rows * sh.vocab * 4 * 2
+    norms = sh.layers * (4 * sh.hidden + 2 * sh.head_dim) * 4
+    return w + kv + act + logits + norms
+
+
 def step_bytes(T, D, t_pos, d_pos):
-    """Algorithmic HBM bytes of one cycle: weights once per GEMV, activations in/out, KV once per KV head."""
-    def model(sh, rows, pos):
-        w = sh.layers * sh.layer_weight_bytes() + sh.head_bytes()
-        kv = 0
-        for l in range(sh.layers):
-            tokens = min(pos, sh.sliding_window) if sh.is_local(l) else pos
-            kv += tokens * sh.kv_width * 2 * 2
-        act = sh.layers * rows * 4 * (2 * sh.hidden * 4 + 2 * sh.q_width + 2 * sh.kv_width + 3 * sh.ffn)
-        logits = rows * sh.vocab * 4 * 2
-        norms = sh.layers * (4 * sh.hidden + 2 * sh.head_dim) * 4
-        return w + kv + act + logits + norms
-    return model(T, 2, t_pos) + model(D, 1, d_pos)
+    """Algorithmic HBM bytes of one cycle."""
+    return model_bytes(T, 2, t_pos) + model_bytes(D, 1, d_pos)
+
+
+def timed_graph(fn, reps=10, warm=3):
+    """fn's launches captured as one HIP graph; microseconds per replay, from events on the launch stream."""
+    import torch
+    fn()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        fn()
+    for _ in range(warm):
+        graph.replay()
+    stream = torch.cuda.current_stream()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record(stream)
+    for _ in range(reps):
+        graph.replay()
+    e1.record(stream)
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e3 / reps
+
+
+def config_figures(target, drafter, T, D, d_pos):
+    """Configs 0-3 of the baseline on their own: microseconds, algorithmic bytes, GB/s and fraction of the
+    HBM peak.  Every GEMV graph walks the 48 blocks' own weights, so the bytes come from HBM."""
+    import ctypes as C
+    import torch
+    from guffin_amd import hip, synth
+    lib = hip.lib()
+    H, F, QW, KW = T.hidden, T.ffn, T.q_width, T.kv_width
+    dts = [int(d) for d in T.dtypes]
+
+    def figure(us, nbytes, what):
+        gbs = nbytes / us / 1e3
+        return {"what": what, "us": round(us, 2), "bytes": int(nbytes), "GB/s": round(gbs, 1),
+                "hbm_frac": round(gbs / HBM_PEAK_GBS, 4)}
+
+    def gemv(dtype, tiles, x, xs, parts, out, rows, K, N):
+        hip.check(lib.guffin_hip_gemv_packed(hip._stream(), dtype, C.c_void_p(tiles), hip._p(x), hip._p(xs), hip._p(parts),
+                                             hip._p(out), rows, K, N))
+
+    def buffers(rows, K, N, dtype):
+        x = torch.randn(rows, K, device="cuda")
+        return (x, hip.group_sums(x), torch.empty((hip.gemv_packed_slices(dtype, K, N), rows, N), device="cuda"),
+                torch.empty((rows, N), device="cuda"))
+
+    out = {}
+    print("bench: timing config 0", file=sys.stderr, flush=True)
+    # config 0: one Q4_K matvec, 1 row, 3840 -> 15360 (the gate matrices of the 48 blocks in turn)
+    x1, xs1, parts1, y1 = buffers(1, H, F, dts[4])
+    us = timed_graph(lambda: [gemv(dts[4], target.layers[l].tiles[4], x1, xs1, parts1, y1, 1, H, F)
+                              for l in range(T.layers)]) / T.layers
+    out["0"] = figure(us, synth.weight_bytes(dts[4], H, F) + H * 4 + F * 4,
+                      "one Q4_K GEMV, 1 row, 3840 -> 15360 (gemv_packed_kernel<Q4_K, 1>)")
+
+    print("bench: timing config 1", file=sys.stderr, flush=True)
+    # config 1: the seven GEMVs of one block at 2 rows, as the step launches them (q/k/v in one launch,
+    # o, gate+up fused with GeGLU, down)
+    x2, xs2, _, _ = buffers(2, H, F, dts[4])
+    qkv_n = (C.c_uint32 * 3)(QW, KW, KW)
+    qkv_dt = (C.c_int * 3)(dts[0], dts[1], dts[2])
+    lib.guffin_hip_gemv_packed_multi_slices.restype = C.c_uint32
+    S = lib.guffin_hip_gemv_packed_multi_slices(3, qkv_dt, qkv_n, H)
+    qkv_parts = [torch.empty((S, 2, n), device="cuda") for n in (QW, KW, KW)]
+    qkv_pp = (C.c_void_p * 3)(*[t.data_ptr() for t in qkv_parts])
+    xa, xas, parts_o, y_o = buffers(2, QW, H, dts[3])
+    xh, xhs, parts_d, y_d = buffers(2, F, H, dts[6])
+    h_out, h_sums = torch.empty(2, F, device="cuda"), hip._receipt(2, F, "cuda")
+
+    def block_gemvs():
+        for l in range(T.layers):
+            L = target.layers[l]
+            tl = (C.c_void_p * 3)(L.tiles[0], L.tiles[1], L.tiles[2])
+            hip.check(lib.guffin_hip_gemv_packed_multi(hip._stream(), 3, qkv_dt, tl, qkv_n, qkv_pp, hip._p(x2), hip._p(xs2), 2, H))
+            gemv(dts[3], L.tiles[3], xa, xas, parts_o, y_o, 2, QW, H)
+            hip.check(lib.guffin_hip_gateup_geglu(hip._stream(), dts[4], C.c_void_p(L.tiles[4]), C.c_void_p(L.tiles[5]),
+                                                  hip._p(x2), hip._p(xs2), hip._p(h_out), hip._p(h_sums), 2, H, F))
+            gemv(dts[6], L.tiles[6], xh, xhs, parts_d, y_d, 2, F, H)
+
+    us = timed_graph(block_gemvs) / T.layers
+    acts = 2 * 4 * (H + QW + 2 * KW + QW + H + H + F + F + H)   # rows x fp32 x (inputs and outputs of the four launches)
+    out["1"] = figure(us, T.layer_weight_bytes() + acts,
+                      "the 7 GEMVs of one 12B block at 2 rows: q/k/v (one launch), o, gate+up+GeGLU, down")
+
+    print("bench: timing config 2", file=sys.stderr, flush=True)
+    # config 2: drafter decode of one token at a 4096-token cache, tied Q8_0 head, greedy argmax
+    token = torch.full((1,), 2, dtype=torch.int32, device="cuda")
+    head_d = drafter.head_tiles
+    assert head_d.numel() == hip.packed_bytes(int(D.embed_dtype), D.hidden, D.vocab)
+
+    def draft_decode():
+        hidden, sums, _, _, _ = drafter.forward(token, d_pos)
+        hip.argmax(hip.gemv_packed(int(D.embed_dtype), head_d, hidden, sums, D.vocab))
+
+    out["2"] = figure(timed_graph(draft_decode), model_bytes(D, 1, d_pos),
+                      "270M Q8_0 drafter: 18 blocks at a %d-token cache, 262144 x 640 head, argmax" % d_pos)
+
+    print("bench: timing config 3", file=sys.stderr, flush=True)
+    # config 3: Q6_K head on 2 rows, top-64 selection, draft law of N(0, 4) logits, acceptance
+    xo, xos, _, _ = buffers(2, H, 64, dts[4])
+    q_logits = 2.0 * torch.randn(T.vocab, device="cuda")
+    options = hip.SamplerOptions(1.0, 64, 0.95, 0.0, 1.0)
+    head_t = target.head_tiles
+    assert head_t.numel() == hip.packed_bytes(int(T.embed_dtype), H, T.vocab)
+
+    def head_accept():
+        p = hip.gemv_packed(int(T.embed_dtype), head_t, xo, xos, T.vocab)
+        cands, _ = hip.select_candidates(p, 64)
+        law, proposal, status = hip.draft_law(q_logits, options, seed=0, step=0)
+        hip.spec_accept(cands, law, proposal, options, seed=0, step=0, status=status)
+
+    out["3"] = figure(timed_graph(head_accept), T.head_bytes() + 2 * 2 * T.vocab * 4 + T.vocab * 4,
+                      "262144 x 3840 Q6_K head on 2 rows, top-64 selection, draft law, accept / residual")
+    return out
 
 
 def cpu_baseline(T, D, budget_s=20.0):
@@ -238,6 +360,7 @@ def main():
             "sustained_dispatches": T.layers, "isolated_launch_us": round(isolated_us, 3),
         },
     }
+    line["configs"] = config_figures(target, drafter, T, D, d_pos)
     if not args.no_prefill:
         line["prefill"] = prefill_figure(target, T)
     if not args.no_cpu_baseline:

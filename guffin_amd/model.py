@@ -197,6 +197,7 @@ class DeviceModel:
         d.out_norm = out_norm.data_ptr()
         d.layers = C.cast(self.layers, C.POINTER(LayerDesc))
         self.keep += [embed_rows, head_tiles, out_norm]
+        self.head_tiles = head_tiles   # the packed head matrix (tied embedding)
         self.ring_k_table = torch.tensor([t.data_ptr() for t in self.ring_k], dtype=torch.int64, device="cuda")
         self.ring_v_table = torch.tensor([t.data_ptr() for t in self.ring_v], dtype=torch.int64, device="cuda")
         return self
