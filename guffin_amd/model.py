@@ -467,6 +467,78 @@ class H1Plan:
         }
 
 
+class VerifyTicketDesc(C.Structure):
+    _fields_ = [("target", C.POINTER(ModelDesc)), ("scratch", C.c_void_p), ("scratch_bytes", C.c_uint64),
+                ("priv_k", C.c_void_p), ("priv_v", C.c_void_p), ("backup_k", C.c_void_p), ("backup_v", C.c_void_p),
+                ("tokens", C.c_void_p), ("selected", C.c_void_p), ("candidates", C.c_void_p), ("status", C.c_void_p),
+                ("retain", C.c_uint32), ("state", C.c_uint32), ("rows", C.c_uint32), ("position", C.c_uint32),
+                ("provisional_count", C.c_uint32), ("provisional_path", C.c_uint32 * 2), ("row_tokens", C.c_uint32 * 2)]
+
+
+TXN_IDLE, TXN_ENCODED, TXN_SUBMITTED, TXN_COMPLETED, TXN_PROVISIONAL, TXN_POISONED = range(6)
+
+
+class VerifyTicket:
+    """The target's verify pass as a transaction (guffin_hip_ticket_*): buffers and the calls."""
+
+    def __init__(self, target, last_position, retain=64):
+        self.target = target
+        sh = target.shape
+        t = self.desc = VerifyTicketDesc()
+        t.target = C.pointer(target.desc)
+        t.retain = retain
+        lib = hip.lib()
+        lib.guffin_hip_ticket_scratch_bytes.restype = C.c_uint64
+        nbytes = lib.guffin_hip_ticket_scratch_bytes(C.byref(t), last_position)
+        if nbytes == 0:
+            raise hip.GuffinError(-1, "ticket: no arena size for this target")
+        self.scratch = torch.zeros(nbytes, dtype=torch.uint8, device="cuda")
+        self.priv_k, self.priv_v = target.private_rows(2)
+        self.backup_k, self.backup_v = target.private_rows(2)
+        self.tokens = torch.zeros(2, dtype=torch.int32, device="cuda")
+        self.selected = torch.zeros(2, dtype=torch.int32, device="cuda")
+        self.candidates = torch.zeros(2 * hip.candidates_dtype.itemsize, dtype=torch.uint8, device="cuda")
+        self.status = torch.zeros(3, dtype=torch.int32, device="cuda")
+        t.scratch, t.scratch_bytes = self.scratch.data_ptr(), nbytes
+        t.priv_k, t.priv_v = self.priv_k.data_ptr(), self.priv_v.data_ptr()
+        t.backup_k, t.backup_v = self.backup_k.data_ptr(), self.backup_v.data_ptr()
+        t.tokens, t.selected = self.tokens.data_ptr(), self.selected.data_ptr()
+        t.candidates, t.status = self.candidates.data_ptr(), self.status.data_ptr()
+        t.state = TXN_IDLE
+
+    @property
+    def state(self):
+        return int(self.desc.state)
+
+    def encode(self, row_tokens, position):
+        arr = (C.c_uint32 * len(row_tokens))(*row_tokens)
+        hip.check(hip.lib().guffin_hip_ticket_encode(C.byref(self.desc), arr, len(row_tokens), position))
+
+    def submit(self):
+        hip.check(hip.lib().guffin_hip_ticket_submit(hip._stream(), C.byref(self.desc)))
+
+    def complete(self):
+        raised = C.c_uint32(0)
+        hip.check(hip.lib().guffin_hip_ticket_complete(hip._stream(), C.byref(self.desc), C.byref(raised)))
+        return raised.value
+
+    def provisional_commit(self, path):
+        arr = (C.c_uint32 * max(1, len(path)))(*path)
+        hip.check(hip.lib().guffin_hip_ticket_provisional_commit(hip._stream(), C.byref(self.desc), arr, len(path)))
+
+    def finalize(self, retained):
+        hip.check(hip.lib().guffin_hip_ticket_finalize(hip._stream(), C.byref(self.desc), retained))
+
+    def discard(self):
+        hip.check(hip.lib().guffin_hip_ticket_discard(hip._stream(), C.byref(self.desc)))
+
+    def release(self):
+        hip.check(hip.lib().guffin_hip_ticket_release(hip._stream(), C.byref(self.desc)))
+
+    def read_candidates(self):
+        return self.candidates.cpu().numpy().view(hip.candidates_dtype)
+
+
 class Session:
     """Consecutive H1 cycles through guffin_hip_session_*: the library keeps positions, the drafter's
     pending token and the transaction state; this class owns the device memory it points at."""

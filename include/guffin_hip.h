@@ -34,6 +34,7 @@ extern "C" {
 #define GUFFIN_E_CAPACITY (-4)  /* exceeds a fixed capacity (LDS, candidate count ...) */
 #define GUFFIN_E_HIP (-5)       /* HIP runtime error, see guffin_hip_last_error() */
 #define GUFFIN_E_STATE (-6)     /* call out of order for the session's state, or the session is poisoned */
+#define GUFFIN_E_NUMERIC (-7)   /* a verify pass raised its device status word (guffin_hip_ticket_complete) */
 
 /* reference: include/local_gguf_engine/tensor/dtype.hpp:9-15 (block layouts 34/144/210 B) */
 #define GUFFIN_Q8_0 0
@@ -555,6 +556,61 @@ int guffin_hip_session_start(guffin_h1_session* session, uint32_t root_token, ui
 int guffin_hip_session_submit(void* stream, guffin_h1_session* session);
 int guffin_hip_session_complete(void* stream, guffin_h1_session* session, uint32_t* emitted /* [2] */,
                                 uint32_t* emitted_count);
+
+/* ---- the verify pass as a transaction ---------------------------------------------------------
+ * The reference's TargetVerificationTicket (include/local_gguf_engine/engine/target_verifier.hpp:
+ * 366-412) with its free functions (src/engine/target_verifier_runtime.cpp): encode :349-445,
+ * submit :447-463, complete :465-533, provisionally_commit :535-609, finalize :611-673, discard
+ * :675-688, and the destructor's rules :315-335 as release.  States are VerifierTransactionState
+ * (include/local_gguf_engine/engine/gemma2_metal_plan.hpp:208-215):
+ *
+ *   idle -encode-> encoded -submit-> submitted -complete-> completed -provisional_commit->
+ *   provisional -finalize-> idle;   discard: encoded / completed -> idle, provisional -> finalize(0)
+ *
+ * A pass runs 1 or 2 contiguous rows (row r's parent is row r - 1) through the target, its head and
+ * the candidate selection; its K/V stay in the private rows.  provisional_commit(path) backs the ring
+ * rows at position .. position + count - 1 of every layer up into the backup rows and publishes the
+ * selected private rows there; finalize(retained) keeps the first `retained` of them and restores
+ * the others.  The only causal paths of a chain are {0} and {0, 1}.  Errors follow the reference:
+ * a call out of order returns GUFFIN_E_STATE and changes nothing (std::logic_error there); a bad
+ * path or row count GUFFIN_E_ARG (std::invalid_argument); a raised device status word drops the
+ * transaction (idle again, the caches untouched) and returns GUFFIN_E_NUMERIC; a failed wait, or a
+ * failure after the first ring row was written, poisons the ticket for good.
+ *
+ * The caller fills the first block of fields once (state = GUFFIN_TXN_IDLE); the library keeps the
+ * second.  After complete, `candidates` holds one record per row (guffin_hip_select_candidates). */
+#define GUFFIN_TXN_ENCODED 1u
+#define GUFFIN_TXN_COMPLETED 3u
+#define GUFFIN_TXN_PROVISIONAL 4u
+#define GUFFIN_TICKET_MAX_ROWS 2u
+typedef struct guffin_verify_ticket {
+    const guffin_model_desc* target;         /* with head_tiles */
+    void* scratch; uint64_t scratch_bytes;   /* device arena, >= guffin_hip_ticket_scratch_bytes */
+    void* priv_k; void* priv_v;              /* device, [blocks][rows][kv width] fp16: the pass's own rows */
+    void* backup_k; void* backup_v;          /* device, [blocks][2][kv width] fp16: ring rows a commit overwrites */
+    uint32_t* tokens;                        /* device u32[2]: the rows' tokens */
+    uint32_t* selected;                      /* device u32[2]: the selected path */
+    void* candidates;                        /* device, 2 candidate records */
+    uint32_t* status;                        /* device u32[3]: the pass's status word, one selection status per row */
+    uint32_t retain;                         /* candidates kept per row (top_k), 1..384 */
+    uint32_t state;                          /* GUFFIN_TXN_* */
+    uint32_t rows, position, provisional_count;
+    uint32_t provisional_path[GUFFIN_TICKET_MAX_ROWS];
+    uint32_t row_tokens[GUFFIN_TICKET_MAX_ROWS];
+} guffin_verify_ticket;
+/* Arena size that covers every pass up to the given cache position. */
+uint64_t guffin_hip_ticket_scratch_bytes(const guffin_verify_ticket* ticket, uint32_t last_position);
+/* Host only: validates and records the pass (row tokens are host memory). */
+int guffin_hip_ticket_encode(guffin_verify_ticket* ticket, const uint32_t* row_tokens, uint32_t rows, uint32_t position);
+int guffin_hip_ticket_submit(void* stream, guffin_verify_ticket* ticket);
+/* Blocks on the stream.  device_status (may be NULL) receives the OR of the status words. */
+int guffin_hip_ticket_complete(void* stream, guffin_verify_ticket* ticket, uint32_t* device_status);
+int guffin_hip_ticket_provisional_commit(void* stream, guffin_verify_ticket* ticket, const uint32_t* path, uint32_t count);
+int guffin_hip_ticket_finalize(void* stream, guffin_verify_ticket* ticket, uint32_t retained);
+int guffin_hip_ticket_discard(void* stream, guffin_verify_ticket* ticket);
+/* What the reference's destructor does: encoded / completed are dropped, a provisional commit is
+ * rolled back, a submitted pass poisons the ticket.  Never fails. */
+int guffin_hip_ticket_release(void* stream, guffin_verify_ticket* ticket);
 
 #ifdef __cplusplus
 }
