@@ -124,10 +124,10 @@ def config_figures(target, drafter, T, D, d_pos):
             L = target.layers[l]
             tl = (C.c_void_p * 3)(L.tiles[0], L.tiles[1], L.tiles[2])
             hip.check(lib.guffin_hip_gemv_packed_multi(hip._stream(), 3, qkv_dt, tl, qkv_n, qkv_pp, hip._p(x2), hip._p(xs2), 2, H))
-            gemv(dts[3], L.tiles[3], xa, xas, parts_o, y_o, 2, QW, H)
+            gemv(dts[3], L.tiles[3], xa, xas, parts_o, None, 2, QW, H)   # partial planes out, as in the step
             hip.check(lib.guffin_hip_gateup_geglu(hip._stream(), dts[4], C.c_void_p(L.tiles[4]), C.c_void_p(L.tiles[5]),
                                                   hip._p(x2), hip._p(xs2), hip._p(h_out), hip._p(h_sums), 2, H, F))
-            gemv(dts[6], L.tiles[6], xh, xhs, parts_d, y_d, 2, F, H)
+            gemv(dts[6], L.tiles[6], xh, xhs, parts_d, None, 2, F, H)
 
     us = timed_graph(block_gemvs) / T.layers
     acts = 2 * 4 * (H + QW + 2 * KW + QW + H + H + F + F + H)   # rows x fp32 x (inputs and outputs of the four launches)
