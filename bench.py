@@ -19,7 +19,8 @@ Extra objects on the JSON line:
   prefill       config 4's second half: a 2048-token prompt through the same stack.
   cpu_baseline  the reference's own CPU row dot (oracle/_ref) or the oracle port timed on the
                 host cores on a bounded sample (one block's seven GEMVs at 2 rows, a column
-                subset), extrapolated to a whole step by weight count.  Reported, not a target.
+                subset), extrapolated to a whole step by weight count; `all_cores` is the oracle's
+                threaded row dot on the same GEMVs over the host's cores.  Reported, not a target.
 """
 import argparse
 import json
@@ -200,8 +201,23 @@ def cpu_baseline(T, D, budget_s=20.0):
     step_weights = (T.layers * layer_weights + T.hidden * T.vocab
                     + 0.5 * (D.layers * sum(K * N for K, N in D.proj_shapes()) + D.hidden * D.vocab))  # drafter: 1 row
     value_us = elapsed / done_weights * step_weights * 1e6
+    # the same rows spread over the host's cores (rows of W are independent; a row's arithmetic is
+    # unchanged): the oracle's threaded row dot on one block's GEMVs
+    many = min(os.cpu_count() or 1, 16)
+    par_weights, par_elapsed = 0, 0.0
+    for i, (dt, (K, N)) in enumerate(shapes):
+        n = max(64, int(N * min(1.0, 4.0 * frac)) // 64 * 64)
+        w = synth.make_weight(dt, K, n, 900 + i)
+        x = synth.make_activation(2, K, 920 + i)
+        t0 = time.perf_counter()
+        gfo.gemv(dt, w, x, n, threads=many)
+        par_elapsed += time.perf_counter() - t0
+        par_weights += K * n
     return {
         "value": round(value_us, 1), "unit": "us", "cores": cores, "kind": kind,
+        "all_cores": {"value": round(par_elapsed / par_weights * step_weights * 1e6, 1), "unit": "us", "cores": many,
+                      "kind": "port", "sample": "one 12B block's 7 GEMVs at 2 rows (%.2f s), oracle row dots on %d threads"
+                                                % (par_elapsed, many)},
         "sample": "%d x one 12B block's 7 GEMVs at 2 rows, first %.1f%% of each matrix's columns (%.2f s of CPU work), "
                   "scaled to the step's weight count; %s" % (
                       repeats, 100 * frac, elapsed,
