@@ -45,6 +45,25 @@ def test_prefill_gemm_parity(hip, gfo, dtype, K, N, M):
         assert np.all(np.abs(one.astype(np.float64) - y[r]) <= 2e-5 * scale[r])
 
 
+def test_prefill_gemm_down_projection_shape(hip, gfo):
+    """Q6_K at the down projection's K = 15360 (60 blocks per column, the longest chain of LDS
+    stages and weight prefetches) with an odd number of column tiles and rows in every row group."""
+    dtype, K, N, M = 2, 15360, 192, 37
+    w = synth.make_weight(dtype, K, N, seed=81)
+    x = synth.make_activation(M, K, seed=82)
+    x[5] *= 1e3
+    tiles = hip.repack(dtype, dev(w), K, N)
+    xd = dev(x)
+    y = hip.prefill_gemm(dtype, tiles, hip.prefill_pack(xd), M, K, N).cpu().numpy()
+    ref = gfo.gemv(dtype, w, x, N, threads=8)
+    scale = np.sqrt((ref.astype(np.float64) ** 2).mean(axis=1, keepdims=True))
+    assert np.all(np.abs(y.astype(np.float64) - ref) <= 1e-3 * scale)
+    for r in (0, 5, 24, M - 1):
+        xr = xd[r:r + 1].contiguous()
+        one = hip.gemv_packed(dtype, tiles, xr, hip.group_sums(xr), N).cpu().numpy()[0]
+        assert np.all(np.abs(one.astype(np.float64) - y[r]) <= 2e-5 * scale[r])
+
+
 @pytest.mark.parametrize("matrix_core", [True, False])
 @pytest.mark.parametrize("q_heads,kv_heads,rows,position,window,cap", [
     (16, 8, 40, 100, 0, 256), (16, 8, 21, 300, 64, 128), (4, 1, 33, 0, 0, 64), (4, 1, 50, 17, 32, 64), (2, 2, 5, 3, 0, 16),
