@@ -37,7 +37,7 @@ HBM_PEAK_GBS = 8000.0
 def model_bytes(sh, rows, pos):
     """Algorithmic HBM bytes of one forward pass with its head: weights once per GEMV, activations in/out,
     KV once per KV head."""
-    w = sh.layers * sh.layer_weight_bytes() + sh.head_bytes()
+    w = sh.body_weight_bytes() + sh.head_bytes()
     kv = 0
     for l in range(sh.layers):
         tokens = min(pos, sh.sliding_window) if sh.is_local(l) else pos

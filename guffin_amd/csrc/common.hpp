@@ -16,6 +16,12 @@ int check_launch(const char* what);
 
 inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
 
+// Layer policy of src/engine/model.cpp:607-610: with a period above one, every layer but the last of
+// each period uses the sliding window (local ring, local rotation base); otherwise every layer is global.
+__host__ __device__ inline bool layer_is_local(uint32_t global_period, uint32_t layer) {
+    return global_period > 1 && (layer % global_period) != global_period - 1;
+}
+
 // ---- typed loads at the alignment a GGUF block stream guarantees ------------
 struct __attribute__((packed, aligned(4))) U4a4 { uint32_t x, y, z, w; };
 struct __attribute__((packed, aligned(2))) U4a2 { uint32_t x, y, z, w; };

@@ -59,9 +59,7 @@ uint32_t ffn_slices(const guffin_layer_desc& L, uint32_t H, uint32_t F) {
     return guffin_hip_gemv_packed_multi_slices(2, L.dtype + 4, n, H);
 }
 
-bool is_local(const guffin_model_desc& m, uint32_t layer) {
-    return m.global_period > 1 && (layer % m.global_period) != m.global_period - 1;
-}
+bool is_local(const guffin_model_desc& m, uint32_t layer) { return layer_is_local(m.global_period, layer); }
 
 // longest token list an attention call of this model can see at `position` with `rows` rows
 uint32_t max_tokens_for(const guffin_model_desc& m, uint32_t layer, uint32_t position, uint32_t rows) {
@@ -132,7 +130,7 @@ __global__ void stage_rows_kernel(uint32_t* positions, uint32_t* ancestors, uint
     if (i < rows) { positions[i] = position + i; ancestors[i] = i; }
     if (i >= layers * rows) return;
     const uint32_t layer = i / rows, row = i % rows, p = position + row;
-    const bool local = global_period > 1 && (layer % global_period) != global_period - 1;
+    const bool local = layer_is_local(global_period, layer);
     const uint32_t window_start = (local && p >= window) ? p + 1 - window : 0;
     const uint32_t base_start = position < window_start ? position : window_start;
     const uint32_t private_start = window_start > position ? window_start - position : 0;
@@ -152,6 +150,15 @@ int validate_model(const guffin_model_desc* m) {
 }
 
 #define GUFFIN_TRY(expr) do { if (int rc_ = (expr)) return rc_; } while (0)
+
+// The rows of a pass at `position` must fit the rings they are published to and read from: global
+// layers address [0, position + rows) through the mask, so the global rings must hold all of it; a
+// local layer reads the window - 1 positions before a row from its ring.
+int check_ring_capacity(const guffin_model_desc& m, uint32_t position, uint32_t rows, const char* what) {
+    if (uint64_t(position) + rows > m.ring_global) return fail(GUFFIN_E_CAPACITY, what);
+    if (m.global_period > 1 && m.sliding_window > 0 && m.sliding_window - 1 > m.ring_local) return fail(GUFFIN_E_CAPACITY, what);
+    return GUFFIN_OK;
+}
 
 int forward_rows(hipStream_t stream, const guffin_model_desc& m, const uint32_t* tokens, uint32_t rows,
                  uint32_t position, const Scratch& s, void* priv_k, void* priv_v, float* out_hidden,
@@ -222,7 +229,7 @@ __global__ void commit_rows_kernel(const uint16_t* priv_k, const uint16_t* priv_
     const uint32_t layer = blockIdx.y, row = blockIdx.z;
     const uint32_t publish = accepted ? 1u + (*accepted != 0u) : rows;
     if (row >= publish || row >= rows) return;
-    const bool local = global_period > 1 && (layer % global_period) != global_period - 1;
+    const bool local = layer_is_local(global_period, layer);
     const uint32_t mask = local ? mask_local : mask_global;
     const size_t src = (size_t(layer) * rows + row) * row_width, dst = size_t((position + row) & mask) * row_width;
     for (uint32_t c = blockIdx.x * blockDim.x + threadIdx.x; c < row_width; c += gridDim.x * blockDim.x) {
@@ -284,6 +291,7 @@ extern "C" int guffin_hip_forward_rows(void* stream, const guffin_model_desc* mo
     GUFFIN_TRY(validate_model(model));
     if (!tokens || !scratch || !priv_k || !priv_v || !out_hidden || !status) return fail(GUFFIN_E_ARG, "forward_rows: null pointer");
     if (rows == 0 || rows > 2) return fail(GUFFIN_E_SHAPE, "forward_rows: rows must be 1 or 2");
+    GUFFIN_TRY(check_ring_capacity(*model, position, rows, "forward_rows: the rows do not fit the KV rings"));
     if (reinterpret_cast<uintptr_t>(scratch) & 255u) return fail(GUFFIN_E_ALIGN, "forward_rows: scratch must be 256-byte aligned");
     const Scratch s = layout(*model, rows, position, static_cast<uint8_t*>(scratch));
     if (s.bytes > scratch_bytes) return fail(GUFFIN_E_CAPACITY, "forward_rows: scratch arena too small");
@@ -360,6 +368,7 @@ extern "C" int guffin_hip_prefill_rows(void* stream, const guffin_model_desc* mo
     if (!tokens || !scratch || !out_hidden || !status) return fail(GUFFIN_E_ARG, "prefill_rows: null pointer");
     GUFFIN_TRY(validate_model(model));
     if (rows == 0) return fail(GUFFIN_E_SHAPE, "prefill_rows: no rows");
+    GUFFIN_TRY(check_ring_capacity(*model, position, rows, "prefill_rows: the rows do not fit the KV rings"));
     if (reinterpret_cast<uintptr_t>(scratch) & 255u) return fail(GUFFIN_E_ALIGN, "prefill_rows: scratch must be 256-byte aligned");
     const guffin_model_desc& m = *model;
     const PrefillScratch s = prefill_layout(m, rows, static_cast<uint8_t*>(scratch));
@@ -471,7 +480,11 @@ extern "C" int guffin_hip_h1_step(void* stream, const guffin_h1_desc* d, const u
     GUFFIN_TRY(validate_model(d->target));
     GUFFIN_TRY(validate_model(d->drafter));
     if (!d->target->head_tiles || !d->drafter->head_tiles) return fail(GUFFIN_E_ARG, "h1_step: models need packed head weights");
-    if (d->drafter->vocab != d->target->vocab) return fail(GUFFIN_E_SHAPE, "h1_step: drafter and target vocabularies must coincide");
+    if (d->drafter->vocab != d->target->vocab && !(d->draft_to_target && d->target_to_draft))
+        return fail(GUFFIN_E_SHAPE, "h1_step: drafter and target vocabularies must coincide unless a vocabulary map is given");
+    GUFFIN_TRY(check_ring_capacity(*d->target, d->target_position, 2, "h1_step: the verify rows do not fit the target's KV rings"));
+    GUFFIN_TRY(check_ring_capacity(*d->drafter, d->drafter_position, d->drafter_rows == 2 ? 2u : 1u,
+                                   "h1_step: the drafter's rows do not fit its KV rings"));
     if (reinterpret_cast<uintptr_t>(scratch) & 255u) return fail(GUFFIN_E_ALIGN, "h1_step: scratch must be 256-byte aligned");
     const guffin_model_desc& T = *d->target;
     const guffin_model_desc& D = *d->drafter;

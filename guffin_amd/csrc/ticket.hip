@@ -63,7 +63,7 @@ void clear_transaction(guffin_verify_ticket* t) {
 
 struct LayerRing { void* k; void* v; uint32_t mask; };
 LayerRing ring_of(const guffin_model_desc& m, uint32_t layer) {
-    const bool local = m.global_period == 0 || layer % m.global_period != m.global_period - 1;
+    const bool local = layer_is_local(m.global_period, layer);  // the same rule as the forward pass it commits for
     return {m.layers[layer].ring_k, m.layers[layer].ring_v, (local ? m.ring_local : m.ring_global) - 1u};
 }
 
@@ -99,7 +99,8 @@ extern "C" int guffin_hip_ticket_encode(guffin_verify_ticket* t, const uint32_t*
     if (rows == 0 || rows > kMaxTicketRows) return fail(GUFFIN_E_SHAPE, "ticket_encode: a pass has 1 or 2 rows");
     if (!m.head_tiles || !m.layers) return fail(GUFFIN_E_ARG, "ticket_encode: the target needs its head tiles and layers");
     if (reinterpret_cast<uintptr_t>(t->scratch) & 255u) return fail(GUFFIN_E_ALIGN, "ticket_encode: the arena must be 256-byte aligned");
-    if (t->retain == 0 || t->retain > 384) return fail(GUFFIN_E_CAPACITY, "ticket_encode: retain must be 1..384 candidates per row");
+    // the selection keeps at most 320 candidates per row (guffin_hip_select_candidates)
+    if (t->retain == 0 || t->retain > 320) return fail(GUFFIN_E_CAPACITY, "ticket_encode: retain must be 1..320 candidates per row");
     if (uint64_t(position) + rows > m.ring_global) return fail(GUFFIN_E_CAPACITY, "ticket_encode: the rows do not fit the global rings");
     if (t->scratch_bytes < arena_of(m, position, t->retain).total) return fail(GUFFIN_E_CAPACITY, "ticket_encode: scratch arena too small");
     t->rows = rows;

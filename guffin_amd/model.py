@@ -72,6 +72,9 @@ class Shape:
     dtypes: tuple = (Q4_K, Q4_K, Q6_K, Q4_K, Q4_K, Q4_K, Q6_K)   # q k v o gate up down
     embed_dtype: int = Q6_K
     eps: float = 1e-6
+    # per-block formats where they differ from `dtypes` (a Q4_K_M file keeps some blocks' attn_v and
+    # ffn_down in Q6_K and others in Q4_K): one 7-tuple per block, or None
+    layer_dtypes: tuple = None
 
     @property
     def q_width(self):
@@ -84,13 +87,19 @@ class Shape:
     def is_local(self, layer):
         return self.global_period > 1 and layer % self.global_period != self.global_period - 1
 
+    def dtypes_of(self, layer):
+        return self.layer_dtypes[layer] if self.layer_dtypes else self.dtypes
+
     def proj_shapes(self):
         """(K, N) of q, k, v, o, gate, up, down."""
         H, F, QW, KW = self.hidden, self.ffn, self.q_width, self.kv_width
         return [(H, QW), (H, KW), (H, KW), (QW, H), (H, F), (H, F), (F, H)]
 
-    def layer_weight_bytes(self):
-        return sum(synth.weight_bytes(d, K, N) for d, (K, N) in zip(self.dtypes, self.proj_shapes()))
+    def layer_weight_bytes(self, layer=0):
+        return sum(synth.weight_bytes(d, K, N) for d, (K, N) in zip(self.dtypes_of(layer), self.proj_shapes()))
+
+    def body_weight_bytes(self):
+        return sum(self.layer_weight_bytes(l) for l in range(self.layers))
 
     def head_bytes(self):
         return synth.weight_bytes(self.embed_dtype, self.hidden, self.vocab)
@@ -117,7 +126,7 @@ class HostModel:
         s = 1000 * seed
         for l in range(shape.layers):
             self.w.append([synth.make_weight(d, K, N, s + 16 * l + i)
-                           for i, (d, (K, N)) in enumerate(zip(shape.dtypes, shape.proj_shapes()))])
+                           for i, (d, (K, N)) in enumerate(zip(shape.dtypes_of(l), shape.proj_shapes()))])
             widths = [shape.hidden, shape.head_dim, shape.head_dim, shape.hidden, shape.hidden, shape.hidden]
             self.norm.append([(1.0 + rng.normal(0, gamma_sigma, w)).astype(np.float32) for w in widths])
             cap = shape.ring_local if shape.is_local(l) else shape.ring_global
@@ -133,24 +142,6 @@ class HostModel:
         self.embed = synth.make_weight(shape.embed_dtype, shape.hidden, shape.vocab, s + 999)
         self.out_norm = (1.0 + rng.normal(0, gamma_sigma, shape.hidden)).astype(np.float32)
 
-    def oracle_config(self, gfo):
-        sh = self.shape
-        return gfo.ModelConfig(sh.hidden, sh.ffn, sh.q_heads, sh.kv_heads, sh.head_dim, sh.layers, sh.vocab,
-                               sh.sliding_window, sh.global_period, sh.local_base, sh.global_base,
-                               sh.global_scale, sh.eps, sh.ring_local, sh.ring_global)
-
-    def oracle_layers(self, gfo):
-        arr = (gfo.Layer * self.shape.layers)()
-        for l in range(self.shape.layers):
-            for i in range(7):
-                arr[l].dtype[i] = self.shape.dtypes[i]
-                arr[l].w[i] = self.w[l][i].ctypes.data
-            for i in range(6):
-                arr[l].norm[i] = self.norm[l][i].ctypes.data
-            arr[l].ring_k = self.ring_k[l].ctypes.data
-            arr[l].ring_v = self.ring_v[l].ctypes.data
-        return arr
-
     def commit(self, pk, pv, position, rows):
         """Publishes the first `rows` private rows of a pass at `position` into the rings, like the device."""
         for l in range(self.shape.layers):
@@ -158,21 +149,6 @@ class HostModel:
             for r in range(rows):
                 self.ring_k[l][(position + r) & (cap - 1)] = pk[l, r].view(np.float16)
                 self.ring_v[l][(position + r) & (cap - 1)] = pv[l, r].view(np.float16)
-
-    def oracle_forward(self, gfo, tokens, position, threads=8):
-        sh = self.shape
-        rows = len(tokens)
-        tok = np.asarray(tokens, np.uint32)
-        pk = np.zeros((sh.layers, rows, sh.kv_width), np.uint16)
-        pv = np.zeros_like(pk)
-        out = np.zeros((rows, sh.hidden), np.float32)
-        cfg = self.oracle_config(gfo)
-        layers = self.oracle_layers(gfo)
-        gfo.lib().gfo_forward_rows(C.byref(cfg), layers, sh.embed_dtype, self.embed.ctypes.data_as(C.c_void_p),
-                                   self.out_norm.ctypes.data_as(C.c_void_p), tok.ctypes.data_as(C.c_void_p),
-                                   rows, position, pk.ctypes.data_as(C.c_void_p), pv.ctypes.data_as(C.c_void_p),
-                                   out.ctypes.data_as(C.c_void_p), threads)
-        return out, pk, pv
 
 
 class DeviceModel:
@@ -207,7 +183,7 @@ class DeviceModel:
         self = cls(host.shape)
         sh = host.shape
         for l in range(sh.layers):
-            for i, (dt, (K, N)) in enumerate(zip(sh.dtypes, sh.proj_shapes())):
+            for i, (dt, (K, N)) in enumerate(zip(sh.dtypes_of(l), sh.proj_shapes())):
                 canonical = torch.from_numpy(host.w[l][i]).cuda()
                 tiles = hip.repack(dt, canonical, K, N)
                 self.keep.append(tiles)
@@ -255,6 +231,11 @@ class DeviceModel:
                 raise ValueError("%s: tensor type %d is not a supported block format" % (name, t))
             return cls.GGUF_TYPES[t]
 
+        # every matrix is validated on its own, as the reference binds it (src/engine/gemma_model.cpp:140-148):
+        # a block's attn_v / ffn_down may be Q6_K where another block's is Q4_K
+        names = [["blk.%d.%s.weight" % (l, m) for m in cls.GGUF_MATRICES] for l in range(layers)]
+        per_layer = tuple(tuple(matrix_type(n) for n in row) for row in names)
+        uniform = all(row == per_layer[0] for row in per_layer)
         window = int(key("attention.sliding_window"))
         shape = Shape(hidden=hidden, ffn=int(key("feed_forward_length")), q_heads=int(key("attention.head_count")),
                       kv_heads=int(key("attention.head_count_kv")), head_dim=int(key("attention.key_length")),
@@ -263,9 +244,9 @@ class DeviceModel:
                       local_base=float(md.get(arch + ".rope.freq_base_swa", 10000.0)),
                       global_base=float(key("rope.freq_base")), global_scale=scale,
                       ring_local=ring_local or 1 << (window - 1).bit_length(), ring_global=ring_global,
-                      dtypes=tuple(matrix_type("blk.0.%s.weight" % m) for m in cls.GGUF_MATRICES),
-                      embed_dtype=matrix_type("token_embd.weight"),
-                      eps=float(key("attention.layer_norm_rms_epsilon")))
+                      dtypes=per_layer[0], embed_dtype=matrix_type("token_embd.weight"),
+                      eps=float(key("attention.layer_norm_rms_epsilon")),
+                      layer_dtypes=None if uniform else per_layer)
         self = cls(shape)
 
         def upload(name):
@@ -280,13 +261,15 @@ class DeviceModel:
         widths = [hidden, shape.head_dim, shape.head_dim, hidden, hidden, hidden]
         for l in range(layers):
             for i, (m, (K, N)) in enumerate(zip(cls.GGUF_MATRICES, shape.proj_shapes())):
-                name = "blk.%d.%s.weight" % (l, m)
-                t = reader.tensor(name)
-                if t["dims"] != [K, N] or matrix_type(name) != shape.dtypes[i]:
-                    raise ValueError("%s: expected a [%d, %d] matrix of the block format of block 0" % (name, K, N))
-                tiles = hip.repack(shape.dtypes[i], upload(name), K, N)
+                name = names[l][i]
+                dt = per_layer[l][i]
+                if reader.tensor(name)["dims"] != [K, N]:
+                    raise ValueError("%s: expected a [%d, %d] matrix" % (name, K, N))
+                if dt == Q8_0 and any(d != Q8_0 for d in per_layer[l]):
+                    raise ValueError("%s: a block mixes 32-weight and 256-weight formats" % name)
+                tiles = hip.repack(dt, upload(name), K, N)
                 self.keep.append(tiles)
-                self.layers[l].dtype[i] = shape.dtypes[i]
+                self.layers[l].dtype[i] = dt
                 self.layers[l].tiles[i] = tiles.data_ptr()
             for i, (n, w) in enumerate(zip(cls.GGUF_NORMS, widths)):
                 g = norm("blk.%d.%s.weight" % (l, n), w)
@@ -328,7 +311,7 @@ class DeviceModel:
             return raw.view(-1)
 
         for l in range(shape.layers):
-            for i, (dt, (K, N)) in enumerate(zip(shape.dtypes, shape.proj_shapes())):
+            for i, (dt, (K, N)) in enumerate(zip(shape.dtypes_of(l), shape.proj_shapes())):
                 tiles = hip.repack(dt, blocks(dt, K, N), K, N)
                 self.keep.append(tiles)
                 self.layers[l].dtype[i] = dt

@@ -304,3 +304,65 @@ def step_draws(seed, step):
     lib().gfo_step_draws(C.c_uint64(seed), C.c_uint64(step), C.byref(w), C.byref(a), C.byref(r),
                          C.byref(n))
     return w.value, a.value, r.value, n.value
+
+
+def model_config(host):
+    """ModelConfig of a synthetic host model (any object with a `.shape` of the benchmark's Shape fields)."""
+    sh = host.shape
+    return ModelConfig(sh.hidden, sh.ffn, sh.q_heads, sh.kv_heads, sh.head_dim, sh.layers, sh.vocab,
+                       sh.sliding_window, sh.global_period, sh.local_base, sh.global_base,
+                       sh.global_scale, sh.eps, sh.ring_local, sh.ring_global)
+
+
+def model_layers(host):
+    """The host model's canonical weights, norms and rings as the oracle's Layer array (views, not copies)."""
+    sh = host.shape
+    arr = (Layer * sh.layers)()
+    for l in range(sh.layers):
+        for i in range(7):
+            arr[l].dtype[i] = sh.dtypes_of(l)[i]
+            arr[l].w[i] = host.w[l][i].ctypes.data
+        for i in range(6):
+            arr[l].norm[i] = host.norm[l][i].ctypes.data
+        arr[l].ring_k = host.ring_k[l].ctypes.data
+        arr[l].ring_v = host.ring_v[l].ctypes.data
+    return arr
+
+
+def forward(host, tokens, position, threads=8):
+    """gfo_forward_rows on a host model: (output-normed rows, private K rows, private V rows)."""
+    sh = host.shape
+    rows = len(tokens)
+    tok = np.asarray(tokens, np.uint32)
+    pk = np.zeros((sh.layers, rows, sh.kv_width), np.uint16)
+    pv = np.zeros_like(pk)
+    out = np.zeros((rows, sh.hidden), np.float32)
+    cfg = model_config(host)
+    layers = model_layers(host)
+    lib().gfo_forward_rows(C.byref(cfg), layers, sh.embed_dtype, host.embed.ctypes.data_as(C.c_void_p),
+                           host.out_norm.ctypes.data_as(C.c_void_p), tok.ctypes.data_as(C.c_void_p),
+                           rows, position, pk.ctypes.data_as(C.c_void_p), pv.ctypes.data_as(C.c_void_p),
+                           out.ctypes.data_as(C.c_void_p), threads)
+    return out, pk, pv
+
+
+def correlating_map(q_logits, p_logits, protect, count=64):
+    """A draft -> target vocabulary permutation (and its inverse) under which the drafter's `count` best
+    tokens are the target's `count` best, rank by rank: two unrelated random models then propose tokens
+    the target gives mass to, so a test sees accepted and rejected proposals.  `protect` (the root) keeps
+    its id on both sides, so the drafter's input is what it was when q_logits were taken."""
+    q_logits, p_logits = np.asarray(q_logits), np.asarray(p_logits)
+    vocab = q_logits.size
+    assert p_logits.size == vocab
+    d2t = np.arange(vocab, dtype=np.int32)
+    t2d = np.arange(vocab, dtype=np.int32)
+    q_top = [int(t) for t in np.argsort(-q_logits, kind="stable") if t != protect][:count]
+    p_top = [int(t) for t in np.argsort(-p_logits, kind="stable") if t != protect][:count]
+    for a, b in zip(q_top, p_top):
+        c, other = int(d2t[a]), int(t2d[b])   # a -> c and other -> b become a -> b and other -> c
+        if other == protect or c == protect:
+            continue
+        d2t[a], d2t[other] = b, c
+        t2d[b], t2d[c] = a, other
+    assert d2t[protect] == protect and np.array_equal(d2t[t2d], np.arange(vocab))
+    return d2t, t2d

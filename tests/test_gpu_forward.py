@@ -55,7 +55,7 @@ def test_forward_rows_matches_oracle(hip, gfo, kind, rows, position):
     host = model.HostModel(shape, seed=3, position=position)
     devm = model.DeviceModel.from_host(host)
     tokens = np.array([17, 1999][:rows], np.uint32)
-    want, wk, wv = host.oracle_forward(gfo, tokens, position, threads=8)
+    want, wk, wv = gfo.forward(host, tokens, position, threads=8)
     hidden, sums, pk, pv, status = devm.forward(dev(tokens), position)
     assert int(status.item()) == 0
     assert rel_rms(hidden.cpu().numpy(), want) <= 1e-3
@@ -66,59 +66,73 @@ def test_forward_rows_matches_oracle(hip, gfo, kind, rows, position):
     assert np.allclose(sums.cpu().numpy(), ref_sums, rtol=0, atol=1e-4 * np.abs(h).max() * 4)
 
 
-def oracle_cycle(hip, gfo, plan, bufs, seed, step, top_k, opt_cpu):
-    """The oracle's decision for this cycle, evaluated on the GPU's logits."""
-    q_logits = bufs["q_logits"].cpu().numpy()
-    p_logits = bufs["p_logits"].cpu().numpy()
-    rc, law = gfo.draft_law_compact(q_logits, opt_cpu)
-    assert rc == 0
-    word, ua, ur, un = gfo.step_draws(seed, step)
-    proposal = gfo.lib().gfo_draft_select(C.byref(law), C.c_uint32(word))
-    r0 = gfo.select_candidates(p_logits[0], top_k)
-    r1 = gfo.select_candidates(p_logits[1], top_k)
-    rc, want = gfo.spec_accept(r0, r1, law, proposal, opt_cpu, ua, ur, un)
-    assert rc == 0
-    return proposal, want, law
-
-
 def run_h1(hip, gfo, t_shape, d_shape, t_pos, d_pos, steps, seed, threads=8):
+    """`steps` cycles from one root with the benchmark's sampler options.  The two random models are
+    unrelated, so the drafter reaches the target through a vocabulary map that lines its 64 best tokens
+    up with the target's (built from the first pass's logits): proposals then fall inside the target's
+    support and the run sees acceptances and rejections.  Returns the decisions among the rest."""
     import torch
     from guffin_amd import model
     t_host = model.HostModel(t_shape, seed=11, position=t_pos)
     d_host = model.HostModel(d_shape, seed=12, position=d_pos)
+    # these random models' logits reach 9e4 (target) and 1e3 (drafter): bring them to a sampler's range,
+    # so that both laws spread over many tokens
+    t_host.out_norm *= np.float32(1e-4)
+    d_host.out_norm *= np.float32(1e-2)
     target = model.DeviceModel.from_host(t_host)
     drafter = model.DeviceModel.from_host(d_host)
-    plan = model.H1Plan(target, drafter, t_pos, d_pos, seed=seed, publish=False)
-    opt_cpu = gfo.SamplerOptions(1.0, 64, 0.95, 0.0, 1.0)
     root = 123
+    probe = model.H1Plan(target, drafter, t_pos, d_pos, seed=seed, publish=False)
+    probe.root.fill_(root)
+    probe.step(0)
+    torch.cuda.synchronize()
+    assert int(probe.status.item()) == 0
+    d2t, t2d = gfo.correlating_map(probe.buffers()["q_logits"].cpu().numpy(), probe.buffers()["p_logits"].cpu().numpy()[0], root)
+    del probe
+    plan = model.H1Plan(target, drafter, t_pos, d_pos, seed=seed, publish=False, draft_to_target=d2t, target_to_draft=t2d)
+    opt_cpu = gfo.SamplerOptions(1.0, 64, 0.95, 0.0, 1.0)
+    none = np.zeros(0, np.uint32)
     plan.root.fill_(root)
-    accepted = 0
+    decisions, supports = [], []
     for step in range(steps):
         plan.step(step)
         torch.cuda.synchronize()
         bufs = plan.buffers()
         res = plan.read_result()
         assert int(plan.status.item()) == 0 and res["status"] == 0
-        proposal, want, _ = oracle_cycle(hip, gfo, plan, bufs, seed, step, 64, opt_cpu)
+        # the oracle's decision for this cycle, evaluated on the GPU's logits through the same map
+        rc, law = gfo.draft_law_compact_mapped(bufs["q_logits"].cpu().numpy(), opt_cpu, d2t)
+        assert rc == 0
+        word, ua, ur, un = gfo.step_draws(seed, step)
+        draft = gfo.lib().gfo_draft_select(C.byref(law), C.c_uint32(word))
+        proposal = int(d2t[draft])
+        p_logits = bufs["p_logits"].cpu().numpy()
+        r0, r1 = gfo.select_candidates(p_logits[0], 64), gfo.select_candidates(p_logits[1], 64)
+        rc, want = gfo.spec_accept_mapped(r0, none, r1, none, law, t2d, proposal, opt_cpu, ua, ur, un)
+        assert rc == 0
         assert res["proposal"] == proposal
         assert (res["accepted"], res["token"], res["next_root"]) == (want.accepted, want.token, want.next_root)
         assert abs(res["acceptance_probability"] - want.acceptance_probability) <= 1e-13
-        accepted += int(res["accepted"])
+        decisions.append(int(res["accepted"]))
+        supports.append((int(law.count), int(gfo.prepare(r0, opt_cpu)[1].count)))
         if step == 0:
             # numerical parity of both forwards and both heads against the CPU path
-            dh, _, _ = d_host.oracle_forward(gfo, [root], d_pos, threads=threads)
+            dh, _, _ = gfo.forward(d_host, [root], d_pos, threads=threads)
             assert rel_rms(bufs["drafter_hidden"].cpu().numpy()[None, :], dh) <= 1e-3
             ql = gfo.gemv(d_shape.embed_dtype, d_host.embed, dh, d_shape.vocab, threads=threads)
             assert rel_rms(bufs["q_logits"].cpu().numpy()[None, :], ql) <= 1e-3
             toks = bufs["tokens"].cpu().numpy().view(np.uint32)[:2]   # the verify pair: root, proposal
             assert toks[0] == root and toks[1] == proposal
-            th, wk, wv = t_host.oracle_forward(gfo, toks, t_pos, threads=threads)
+            th, wk, wv = gfo.forward(t_host, toks, t_pos, threads=threads)
             assert rel_rms(bufs["target_hidden"].cpu().numpy(), th) <= 1e-3
             pl = gfo.gemv(t_shape.embed_dtype, t_host.embed, th, t_shape.vocab, threads=threads)
             assert rel_rms(bufs["p_logits"].cpu().numpy(), pl) <= 1e-3
             check_private_rows(plan.t_pk, wk)
             check_private_rows(plan.t_pv, wv)
-    return accepted, plan, target, drafter, t_host
+    # both laws spread over many tokens, and the run took both branches of the acceptance test
+    assert min(q for q, p in supports) > 8 and min(p for q, p in supports) > 8, supports
+    assert 0 < sum(decisions) < steps, decisions
+    return decisions, plan, target, drafter, t_host
 
 
 def test_h1_cycle_small_models(hip, gfo):
@@ -267,7 +281,8 @@ def test_h1_commit_publishes_verified_rows(hip, gfo):
 def test_h1_cycle_full_size_models(hip, gfo):
     """Config 4 shapes: the 48-block 12B target at an 8192-token context with the 18-block drafter."""
     from guffin_amd import model
-    accepted, plan, *_ = run_h1(hip, gfo, model.GEMMA3_12B, model.GEMMA3_270M, 8190, 4096, steps=2, seed=1, threads=16)
+    decisions, plan, *_ = run_h1(hip, gfo, model.GEMMA3_12B, model.GEMMA3_270M, 8190, 4096, steps=10, seed=1, threads=16)
+    print("full-size decisions:", decisions)
 
 
 def test_h1_cycle_with_a_vocabulary_map(hip, gfo):
@@ -306,7 +321,7 @@ def test_h1_cycle_with_a_vocabulary_map(hip, gfo):
         toks = bufs["tokens"].cpu().numpy().view(np.uint32)
         assert toks[8] == t2d[root]                                        # the drafter's input row, in its ids
         if step == 0:   # the drafter really ran on that id
-            dh, _, _ = d_host.oracle_forward(gfo, [int(t2d[root])], 300, threads=8)
+            dh, _, _ = gfo.forward(d_host, [int(t2d[root])], 300, threads=8)
             assert rel_rms(bufs["drafter_hidden"].cpu().numpy()[None, :], dh) <= 1e-3
         scores = bufs["q_logits"].cpu().numpy().copy()
         hist_draft = t2d[history]

@@ -9,6 +9,7 @@ import numpy as np
 import pytest
 
 from guffin_amd import synth
+from bounds import assert_within_operator_bound
 
 pytestmark = pytest.mark.gpu
 
@@ -39,10 +40,11 @@ def check_gemv(hip, gfo, dtype, K, N, rows, seed):
     x = synth.make_activation(rows, K, seed + 1)
     y = hip.gemv(dtype, dev(w), dev(x), N).cpu().numpy()
     ref = gfo.gemv(dtype, w, x, N, threads=8)
-    dense_abs = None
     scale = np.sqrt((ref.astype(np.float64) ** 2).mean(axis=1, keepdims=True))
     err = np.abs(y.astype(np.float64) - ref)
     assert np.all(err <= 1e-3 * scale), (dtype, K, N, rows, float((err / scale).max()))
+    # the reference's own bar for this operator: a few 1e-6 of sum|x*w| against a double dot product
+    assert_within_operator_bound(gfo, dtype, w, x, y, K, N)
     return y
 
 

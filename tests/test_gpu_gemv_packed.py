@@ -9,6 +9,7 @@ import numpy as np
 import pytest
 
 from guffin_amd import synth
+from bounds import assert_within_operator_bound
 
 pytestmark = pytest.mark.gpu
 
@@ -94,6 +95,9 @@ def test_packed_gemv_parity(hip, gfo, dtype, K, N, rows):
     scale = np.sqrt((ref.astype(np.float64) ** 2).mean(axis=1, keepdims=True))
     err = np.abs(y.astype(np.float64) - ref)
     assert np.all(err <= 1e-3 * scale), float((err / scale).max())
+    # the reference's operator bound against a double dot product (a dropped low half of the operand
+    # or a wrong multiplier on one 32-group is orders of magnitude outside it)
+    assert_within_operator_bound(gfo, dtype, w, x, y, K, N)
     # and against the canonical-layout kernel: both are fp32 sums of the same products
     yc = hip.gemv(dtype, wd, xd, N).cpu().numpy()
     assert np.all(np.abs(y.astype(np.float64) - yc) <= 2e-5 * scale)

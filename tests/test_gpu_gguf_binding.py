@@ -36,7 +36,7 @@ def write_gguf(host, alignment=64):
     norms = ("attn_norm", "attn_q_norm", "attn_k_norm", "post_attention_norm", "ffn_norm", "post_ffw_norm")
     for l in range(sh.layers):
         for i, (n, (K, N)) in enumerate(zip(names, sh.proj_shapes())):
-            tensors.append(("blk.%d.%s.weight" % (l, n), [K, N], GGUF_TYPE[sh.dtypes[i]], host.w[l][i]))
+            tensors.append(("blk.%d.%s.weight" % (l, n), [K, N], GGUF_TYPE[sh.dtypes_of(l)[i]], host.w[l][i]))
         for i, n in enumerate(norms):
             tensors.append(("blk.%d.%s.weight" % (l, n), [host.norm[l][i].size], 0, host.norm[l][i]))
     out = bytearray(b"GGUF" + struct.pack("<IQQ", 3, len(tensors), len(md)))
@@ -86,6 +86,36 @@ def test_model_bound_from_a_gguf_image_runs_like_the_direct_binding(kind):
     assert int(got[4].item()) == 0 and int(want[4].item()) == 0
     for g, w in zip(got[:4], want[:4]):
         assert torch.equal(g.view(torch.uint8), w.view(torch.uint8))
+
+
+def test_blocks_of_mixed_formats_bind_matrix_by_matrix(gfo):
+    """A Q4_K_M file keeps attn_v and ffn_down in Q6_K in some blocks and in Q4_K in others; each matrix is
+    bound in its own format (src/engine/gemma_model.cpp:140-148) and the pass agrees with the oracle on the
+    same canonical weights."""
+    import torch
+    from guffin_amd import gguf, hip, model
+    hip.init(0)
+    Q4, Q6 = model.Q4_K, model.Q6_K
+    per_layer = ((Q4, Q4, Q6, Q4, Q4, Q4, Q6), (Q4, Q4, Q4, Q4, Q4, Q4, Q4), (Q4, Q4, Q6, Q4, Q4, Q4, Q4),
+                 (Q4, Q4, Q4, Q4, Q4, Q4, Q6), (Q4, Q4, Q4, Q4, Q6, Q4, Q6), (Q4, Q4, Q6, Q4, Q4, Q4, Q6))
+    shape = replace(model.GEMMA3_12B, layers=6, vocab=2048, ring_global=1024, layer_dtypes=per_layer)
+    host = model.HostModel(shape, seed=8, position=0)
+    bound = model.DeviceModel.from_gguf(gguf.Reader(write_gguf(host)), ring_local=shape.ring_local,
+                                        ring_global=shape.ring_global)
+    assert bound.shape.layer_dtypes == per_layer
+    assert [[bound.layers[l].dtype[i] for i in range(7)] for l in range(6)] == [list(r) for r in per_layer]
+    assert bound.shape.body_weight_bytes() == sum(host.w[l][i].size for l in range(6) for i in range(7))
+    tokens = torch.tensor([17, 1999], dtype=torch.int32, device="cuda")
+    got = bound.forward(tokens, 0)
+    torch.cuda.synchronize()
+    assert int(got[4].item()) == 0
+    want, wk, wv = gfo.forward(host, [17, 1999], 0, threads=8)
+    hidden = got[0].cpu().numpy().astype(np.float64)
+    scale = np.sqrt((want.astype(np.float64) ** 2).mean(-1, keepdims=True))
+    assert np.max(np.abs(hidden - want) / scale) <= 1e-3
+    direct = model.DeviceModel.from_host(host).forward(tokens, 0)
+    torch.cuda.synchronize()
+    assert torch.equal(got[0].view(torch.uint8), direct[0].view(torch.uint8))
 
 
 def test_binding_refuses_files_that_do_not_fit_the_model():

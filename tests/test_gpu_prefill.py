@@ -9,6 +9,7 @@ import numpy as np
 import pytest
 
 from guffin_amd import synth
+from bounds import assert_within_operator_bound
 
 pytestmark = pytest.mark.gpu
 
@@ -25,7 +26,8 @@ def dev(a):
     return torch.from_numpy(np.ascontiguousarray(a)).cuda()
 
 
-@pytest.mark.parametrize("dtype,K,N", [(1, 3840, 256), (2, 3840, 128), (0, 640, 256), (1, 256, 64), (2, 512, 192)])
+@pytest.mark.parametrize("dtype,K,N", [(1, 3840, 256), (2, 3840, 128), (0, 640, 256), (1, 256, 64), (2, 512, 192),
+                                       (1, 768, 320), (1, 512, 384), (1, 256, 448), (2, 256, 320)])
 @pytest.mark.parametrize("M", [1, 7, 33, 130])
 def test_prefill_gemm_parity(hip, gfo, dtype, K, N, M):
     w = synth.make_weight(dtype, K, N, seed=70 + dtype)
@@ -38,6 +40,7 @@ def test_prefill_gemm_parity(hip, gfo, dtype, K, N, M):
     ref = gfo.gemv(dtype, w, x, N, threads=8)
     scale = np.sqrt((ref.astype(np.float64) ** 2).mean(axis=1, keepdims=True))
     assert np.all(np.abs(y.astype(np.float64) - ref) <= 1e-3 * scale)
+    assert_within_operator_bound(gfo, dtype, w, x, y, K, N, matrix_path=True)   # the reference's bound for its matrix path
     # the decode GEMV on the same rows computes the same exact products
     for r in (0, M - 1):
         xr = xd[r:r + 1].contiguous()
@@ -58,10 +61,111 @@ def test_prefill_gemm_down_projection_shape(hip, gfo):
     ref = gfo.gemv(dtype, w, x, N, threads=8)
     scale = np.sqrt((ref.astype(np.float64) ** 2).mean(axis=1, keepdims=True))
     assert np.all(np.abs(y.astype(np.float64) - ref) <= 1e-3 * scale)
+    assert_within_operator_bound(gfo, dtype, w, x, y, K, N, matrix_path=True)
     for r in (0, 5, 24, M - 1):
         xr = xd[r:r + 1].contiguous()
         one = hip.gemv_packed(dtype, tiles, xr, hip.group_sums(xr), N).cpu().numpy()[0]
         assert np.all(np.abs(one.astype(np.float64) - y[r]) <= 2e-5 * scale[r])
+
+
+@pytest.mark.parametrize("dtype,K,N", [(1, 3840, 15360), (2, 15360, 3840)])
+def test_prefill_gemm_at_2048_rows(hip, gfo, dtype, K, N):
+    """The benchmark's prompt length on the gate (Q4_K) and down (Q6_K) shapes: 64 row chunks x every
+    column-tile group of the launch.  Rows sampled from the first, last and neighbouring chunks agree
+    with the decode GEMV on the same row to fp32 rounding, and with a double dot product within the
+    reference's bound for its matrix path (tests/tensor/gemma3_metal_tests.cpp:1280-1285)."""
+    import torch
+    M = 2048
+    w = synth.make_weight(dtype, K, N, seed=90 + dtype)
+    tiles = hip.repack(dtype, dev(w), K, N)
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(91)
+    xd = torch.randn((M, K), device="cuda", generator=gen)
+    xd[777] *= 300.0
+    y = hip.prefill_gemm(dtype, tiles, hip.prefill_pack(xd), M, K, N)
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(y).all())
+    rows = sorted(set([0, 1, 31, 32, 33, 63, 64, 127, 128, 1023, 1024, 1055, 1056, 2015, 2016, 2046, 2047]
+                      + list(np.random.default_rng(3).integers(0, M, 23))))
+    ys = y[rows].cpu().numpy().astype(np.float64)
+    scale = np.sqrt((ys ** 2).mean(axis=1, keepdims=True))
+    for i, r in enumerate(rows):
+        xr = xd[r:r + 1].contiguous()
+        one = hip.gemv_packed(dtype, tiles, xr, hip.group_sums(xr), N).cpu().numpy()[0]
+        assert np.all(np.abs(one.astype(np.float64) - ys[i]) <= 2e-5 * scale[i]), r
+    check = [0, 33, 1024, 1055, 2016, 2047, 777, rows[5]]
+    x_host = xd[check].cpu().numpy()
+    assert_within_operator_bound(gfo, dtype, w, x_host, y[check].cpu().numpy(), K, N, matrix_path=True)
+
+
+def test_prefill_rows_at_2048_rows_against_the_oracle_on_the_last_chunk(hip, gfo):
+    """2048 prompt tokens through two blocks of the 12B widths whose attention windows are 32 tokens: the
+    last 32 rows depend on the last 94 only, so the oracle's forward pass of those 94 rows (empty rings)
+    gives the expected rows 2016..2047 and their K/V (bars of tests/engine/gemma3_target_runtime_tests.cpp:
+    310-327).  The row chunks, the run-row indexing and the ring publication at 2048 rows are all in play."""
+    import torch
+    from dataclasses import replace
+    from guffin_amd import model
+    rows, window = 2048, 32
+    shape = replace(model.GEMMA3_12B, layers=2, vocab=2048, ring_global=2048, ring_local=64, sliding_window=window,
+                    global_period=3)   # both blocks local
+    host = model.HostModel(shape, seed=14, position=0)
+    devm = model.DeviceModel.from_host(host)
+    tokens = np.random.default_rng(10).integers(0, shape.vocab, rows).astype(np.uint32)
+    hidden, status = devm.prefill(dev(tokens), 0)
+    torch.cuda.synchronize()
+    assert int(status.item()) == 0
+    got = hidden.cpu().numpy().astype(np.float64)
+    assert np.isfinite(got).all()
+    start = rows - 1 - 3 * (window - 1)    # block 0 rows are right from start + 31 on, block 1 rows from start + 62 on
+    want, wk, wv = gfo.forward(host, tokens[start:], start, threads=8)
+    tail = np.arange(rows - window, rows)
+    scale = np.sqrt((want[tail - start].astype(np.float64) ** 2).mean(axis=-1, keepdims=True)) + 1e-30
+    assert np.max(np.abs(got[tail] - want[tail - start]) / scale) <= 1e-3
+    for l in range(shape.layers):
+        rk = devm.ring_k[l].view(torch.int16).cpu().numpy().view(np.uint16)
+        rv = devm.ring_v[l].view(torch.int16).cpu().numpy().view(np.uint16)
+        for r in tail:
+            assert np.mean(rk[r & (shape.ring_local - 1)] == wk[l, r - start]) >= 0.95, (l, r)
+            assert np.mean(rv[r & (shape.ring_local - 1)] == wv[l, r - start]) >= 0.95, (l, r)
+
+
+def test_prefill_rows_at_2048_rows_agree_with_the_decode_path(hip, gfo):
+    """The benchmark's prompt through one sliding-window block (window 1024) and one global block of the
+    12B widths.  The first rows are checked against the oracle; rows sampled from every part of the run
+    (chunk boundaries included) against the decode pass of the same token at the same position, which
+    reads the K/V the run published: hidden rows to fp32 rounding, the row's own K/V against the ring rows."""
+    import torch
+    from dataclasses import replace
+    from guffin_amd import model
+    rows = 2048
+    shape = replace(model.GEMMA3_12B, layers=2, vocab=2048, ring_global=2048, ring_local=2048, global_period=2)
+    host = model.HostModel(shape, seed=15, position=0)
+    devm = model.DeviceModel.from_host(host)
+    tokens = np.random.default_rng(11).integers(0, shape.vocab, rows).astype(np.uint32)
+    td = dev(tokens.view(np.int32))
+    hidden, status = devm.prefill(td, 0)
+    torch.cuda.synchronize()
+    assert int(status.item()) == 0
+    got = hidden.cpu().numpy().astype(np.float64)
+    assert np.isfinite(got).all()
+    head = 24
+    want, wk, wv = gfo.forward(host, tokens[:head], 0, threads=8)
+    scale = np.sqrt((want.astype(np.float64) ** 2).mean(axis=-1, keepdims=True)) + 1e-30
+    assert np.max(np.abs(got[:head] - want) / scale) <= 1e-3
+    sample = sorted(set([31, 32, 33, 127, 128, 1023, 1024, 1025, 1055, 1056, 2015, 2016, 2046, 2047]
+                        + list(np.random.default_rng(4).integers(40, rows, 18))))
+    rk = [t.view(torch.int16).cpu().numpy().view(np.uint16) for t in devm.ring_k]
+    rv = [t.view(torch.int16).cpu().numpy().view(np.uint16) for t in devm.ring_v]
+    for r in sample:
+        one, _, pk, pv, st = devm.forward(td[r:r + 1].contiguous(), int(r))
+        assert int(st.item()) == 0
+        row = one.cpu().numpy().astype(np.float64)[0]
+        assert np.max(np.abs(got[r] - row)) <= 2e-4 * np.sqrt((row ** 2).mean()), r
+        pk = pk.view(torch.int16).cpu().numpy().view(np.uint16)
+        pv = pv.view(torch.int16).cpu().numpy().view(np.uint16)
+        for l in range(shape.layers):
+            assert np.mean(rk[l][r] == pk[l, 0]) >= 0.95 and np.mean(rv[l][r] == pv[l, 0]) >= 0.95, (r, l)
 
 
 @pytest.mark.parametrize("matrix_core", [True, False])
@@ -122,7 +226,7 @@ def test_prefill_rows_match_oracle_forward(hip, gfo, kind, rows, position):
     host = model.HostModel(shape, seed=4, position=position)
     devm = model.DeviceModel.from_host(host)
     tokens = np.random.default_rng(9).integers(0, shape.vocab, rows).astype(np.uint32)
-    want, wk, wv = host.oracle_forward(gfo, tokens, position, threads=8)
+    want, wk, wv = gfo.forward(host, tokens, position, threads=8)
     hidden, status = devm.prefill(dev(tokens), position)
     assert int(status.item()) == 0
     got = hidden.cpu().numpy().astype(np.float64)

@@ -63,9 +63,9 @@ def test_session_generates_over_many_cycles(hip, gfo):
         assert emitted == ([proposal, want.next_root] if want.accepted else [want.token])
         # both passes against the oracle, teacher-forced, on the oracle's own mirrored caches
         d_tokens = [pending, root] if pending is not None else [root]
-        dh, dk, dv = d_host.oracle_forward(gfo, d_tokens, d_pos)
+        dh, dk, dv = gfo.forward(d_host, d_tokens, d_pos)
         assert rel_rms(bufs["drafter_hidden_rows"].cpu().numpy(), dh) <= 1e-3, cycle
-        th, tk, tv = t_host.oracle_forward(gfo, [root, proposal], t_pos)
+        th, tk, tv = gfo.forward(t_host, [root, proposal], t_pos)
         assert rel_rms(bufs["target_hidden"].cpu().numpy(), th) <= 1e-3, cycle
         d_host.commit(dk, dv, d_pos, len(d_tokens))
         t_host.commit(tk, tv, t_pos, 1 + want.accepted)

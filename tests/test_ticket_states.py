@@ -15,8 +15,8 @@ from guffin_amd import hip, model
 E_ARG, E_SHAPE, E_ALIGN, E_CAPACITY, E_STATE = -1, -2, -3, -4, -6
 
 
-def make_ticket(retain=64, scratch_bytes=1 << 34):
-    sh = replace(model.GEMMA3_12B, layers=6, vocab=2048, ring_global=2048)
+def make_ticket(retain=64, scratch_bytes=1 << 34, **shape_changes):
+    sh = replace(model.GEMMA3_12B, layers=6, vocab=2048, ring_global=2048, **shape_changes)
     desc = model.ModelDesc()
     for name in ("hidden", "ffn", "q_heads", "kv_heads", "head_dim", "vocab", "sliding_window", "global_period",
                  "local_base", "global_base", "global_scale", "eps", "ring_local", "ring_global"):
@@ -80,7 +80,7 @@ def test_encode_checks_its_arguments():
     assert lib.guffin_hip_ticket_discard(None, C.byref(t)) == 0
     small, keep2 = make_ticket(scratch_bytes=need - 1)
     assert lib.guffin_hip_ticket_encode(C.byref(small), tokens(1, 2), 2, 2046) == E_CAPACITY
-    wide, keep3 = make_ticket(retain=385)
+    wide, keep3 = make_ticket(retain=321)   # the selection keeps at most 320 candidates per row
     assert lib.guffin_hip_ticket_encode(C.byref(wide), tokens(1), 1, 0) == E_CAPACITY
     odd, keep4 = make_ticket()
     odd.scratch += 64
@@ -128,3 +128,42 @@ def test_a_poisoned_or_submitted_ticket_cannot_be_reused_or_discarded():
     c, keep3 = make_ticket()
     c.state, c.rows = model.TXN_COMPLETED, 2
     assert lib.guffin_hip_ticket_release(None, C.byref(c)) == 0 and c.state == model.TXN_IDLE
+
+
+def test_forward_entry_points_refuse_rows_beyond_the_ring_capacity():
+    """forward_rows, prefill_rows and h1_step check what ticket_encode checks: the rows must fit the
+    global rings, and a local ring must hold the window before a row (no GPU is reached)."""
+    lib = hip.lib()
+    t, (desc, layers) = make_ticket()
+    fake = C.c_void_p(0x7F0000000000)
+    big = C.c_uint64(1 << 40)
+    args = lambda rows, position: (None, C.byref(desc), fake, rows, position, fake, big, fake, fake, fake, fake, fake)
+    assert lib.guffin_hip_forward_rows(*args(2, 2047)) == E_CAPACITY
+    assert lib.guffin_hip_forward_rows(*args(1, 2048)) == E_CAPACITY
+    assert b"forward_rows" in lib.guffin_hip_last_error()
+    assert lib.guffin_hip_prefill_rows(None, C.byref(desc), fake, 100, 1949, fake, big, fake, fake) == E_CAPACITY
+    assert b"prefill_rows" in lib.guffin_hip_last_error()
+    narrow, (ndesc, nlayers) = make_ticket(ring_local=512)   # window 1024 needs 1023 ring rows
+    assert lib.guffin_hip_forward_rows(None, C.byref(ndesc), fake, 1, 0, fake, big, fake, fake, fake, fake, fake) == E_CAPACITY
+    h1 = model.H1Desc()
+    h1.target, h1.drafter = C.pointer(desc), C.pointer(desc)
+    h1.target_position, h1.drafter_position, h1.top_k = 2047, 0, 64
+    step = lambda: lib.guffin_hip_h1_step(None, C.byref(h1), fake, fake, big, fake, fake, fake, fake, fake, fake)
+    assert step() == E_CAPACITY and b"verify rows" in lib.guffin_hip_last_error()
+    h1.target_position, h1.drafter_position = 0, 2048
+    assert step() == E_CAPACITY and b"drafter" in lib.guffin_hip_last_error()
+
+
+@pytest.mark.parametrize("period", [0, 1])
+def test_a_model_without_local_layers_is_global_in_the_ticket_as_in_the_forward_pass(period):
+    """With a global period of 0 or 1 every layer is global (src/engine/model.cpp:607-610): the pass must
+    fit the global rings whatever the local capacity says, and the arena is the forward pass's."""
+    lib = hip.lib()
+    lib.guffin_hip_ticket_scratch_bytes.restype = C.c_uint64
+    lib.guffin_hip_forward_scratch_bytes.restype = C.c_uint64
+    t, (desc, layers) = make_ticket(global_period=period, ring_local=16)
+    assert lib.guffin_hip_ticket_encode(C.byref(t), tokens(1, 2), 2, 2046) == 0     # ring_local 16 is never used
+    assert lib.guffin_hip_ticket_discard(None, C.byref(t)) == 0
+    assert lib.guffin_hip_ticket_encode(C.byref(t), tokens(1, 2), 2, 2047) == E_CAPACITY
+    # every layer attends the whole context: the forward arena grows with the position on all six layers
+    assert lib.guffin_hip_forward_scratch_bytes(C.byref(desc), 2, 2000) > lib.guffin_hip_forward_scratch_bytes(C.byref(desc), 2, 10)
