@@ -29,7 +29,7 @@ int check_launch(const char* what) {
 
 int gemv_init(int cu_count);
 int ops_init(int cu_count);
-void gemv_packed_init(int cu_count);
+int gemv_packed_init(int device, int cu_count);
 int head_init();
 
 }  // namespace guffin
@@ -55,6 +55,7 @@ extern "C" int guffin_hip_init(int device) {
     }
     if (gemv_init(prop.multiProcessorCount) != 0 || ops_init(prop.multiProcessorCount) != 0 || head_init() != 0)
         return fail(GUFFIN_E_HIP, "init: could not raise a kernel's dynamic LDS limit");
-    gemv_packed_init(prop.multiProcessorCount);
+    if (gemv_packed_init(device, prop.multiProcessorCount) != 0)
+        return fail(GUFFIN_E_HIP, "init: could not take the address of the static scratch array on this device");
     return GUFFIN_OK;
 }

@@ -539,6 +539,14 @@ gateup_geglu_kernel(const uint8_t* __restrict__ gate_tiles, const uint8_t* __res
 
 int g_cus = 256;
 
+// Scratch of the entry point that allocates nothing (guffin_hip_gemv_packed_static): the partial
+// planes of one launch.  Every GPU the library runs on holds its own copy of this array at its own
+// address until the process ends; host code reaches it only through the pointer taken at init.
+constexpr uint32_t kStaticScratchFloats = 32768;   // 128 KiB: planes * rows * N of the largest supported launch
+static __device__ __align__(256) float scratch[kStaticScratchFloats];
+constexpr int kMaxDevices = 64;
+float* g_scratch_ptr[kMaxDevices] = {};
+
 // Work split of a launch over `tiles` column tiles of `nblk` blocks each: blocks per wave so
 // that the chip holds about four waves per SIMD, waves per workgroup (k-slices reduced in LDS,
 // at most max_w) and planes (k-slices left to the consumer), preferring one workgroup per CU.
@@ -595,7 +603,16 @@ int launch_packed(hipStream_t s, const uint8_t* w, const float* x, const float* 
 
 }  // namespace
 
-void gemv_packed_init(int cu_count) { g_cus = cu_count > 0 ? cu_count : 256; }
+// Called by guffin_hip_init with `device` current: the split heuristics' CU count and this device's
+// address of the static scratch array.
+int gemv_packed_init(int device, int cu_count) {
+    g_cus = cu_count > 0 ? cu_count : 256;
+    if (device < 0 || device >= kMaxDevices) return -1;
+    float* ptr = nullptr;
+    if (hipGetSymbolAddress(reinterpret_cast<void**>(&ptr), HIP_SYMBOL(scratch)) != hipSuccess || !ptr) return -1;
+    g_scratch_ptr[device] = ptr;
+    return 0;
+}
 
 }  // namespace guffin
 
@@ -768,4 +785,21 @@ extern "C" int guffin_hip_gemv_packed(void* stream, int dtype, const void* tiles
     const uint32_t count = rows * N;
     hipLaunchKernelGGL(reduce_partials_kernel, dim3((count + 255) / 256), dim3(256), 0, s, partials, y, S, count);
     return check_launch("reduce_partials");
+}
+
+extern "C" uint64_t guffin_hip_gemv_packed_static_limit(void) { return kStaticScratchFloats; }
+
+extern "C" int guffin_hip_gemv_packed_static(void* stream, int dtype, const void* tiles, const float* x, const float* xsums,
+                                             float* y, uint32_t rows, uint32_t K, uint32_t N) {
+    if (!tiles || !x || !xsums || !y) return fail(GUFFIN_E_ARG, "gemv_packed_static: null pointer");
+    if (int rc = check_packed_shape("gemv_packed_static: need K % block == 0 and N % 64 == 0", dtype, K, N)) return rc;
+    if (rows == 0 || rows > 2) return fail(GUFFIN_E_SHAPE, "gemv_packed_static: rows must be 1 or 2");
+    const uint32_t S = packed_plan(dtype, K / block_elems(dtype), N / kTileCols).sp.planes;
+    if (S > 1 && uint64_t(S) * rows * N > kStaticScratchFloats)
+        return fail(GUFFIN_E_CAPACITY, "gemv_packed_static: planes * rows * N exceeds the static scratch of 32768 floats");
+    int device = -1;
+    if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= kMaxDevices || !g_scratch_ptr[device])
+        return fail(GUFFIN_E_STATE, "gemv_packed_static: guffin_hip_init has not run for the current device");
+    // the kernels write every plane element they later read, so nothing needs clearing between calls
+    return guffin_hip_gemv_packed(stream, dtype, tiles, x, xsums, g_scratch_ptr[device], y, rows, K, N);
 }

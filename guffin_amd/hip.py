@@ -141,6 +141,14 @@ def gemv_packed(dtype, tiles, x, xsums, N, partials=None, out=None, reduce=True)
     return out if reduce else partials
 
 
+def gemv_packed_static(dtype, tiles, x, xsums, N, out):
+    """guffin_hip_gemv_packed_static: the packed GEMV with its partial planes in the library's static
+    device array; `out` is the caller's [rows, N] result."""
+    rows, K = x.shape
+    check(lib().guffin_hip_gemv_packed_static(_stream(), dtype, _p(tiles), _p(x), _p(xsums), _p(out), rows, K, N))
+    return out
+
+
 def _f32(shape, like):
     return torch.empty(shape, dtype=torch.float32, device=like.device)
 

@@ -109,6 +109,17 @@ uint32_t guffin_hip_gemv_packed_slices(int dtype, uint32_t K, uint32_t N);
 int guffin_hip_gemv_packed(void* stream, int dtype, const void* tiles, const float* x, const float* xsums,
                            float* partials, float* y, uint32_t rows, uint32_t K, uint32_t N);
 
+/* guffin_hip_gemv_packed for callers that cannot allocate device memory or carry a workspace (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc): the partial planes live in a
+ * static device array of the library (128 KiB per GPU, held until the process ends) instead of `partials`.
+ * No counterpart in the reference.  Refuses launches whose planes * rows * N exceed
+ * guffin_hip_gemv_packed_static_limit() floats (GUFFIN_E_CAPACITY) and devices guffin_hip_init has not
+ * seen (GUFFIN_E_STATE).  Calls no allocator.  All calls on one GPU share that GPU's array: calls that
+ * overlap on one GPU (two streams) race; calls on one stream do not. */
+uint64_t guffin_hip_gemv_packed_static_limit(void);
+int guffin_hip_gemv_packed_static(void* stream, int dtype, const void* tiles, const float* x, const float* xsums,
+                                  float* y, uint32_t rows, uint32_t K, uint32_t N);
+
 /* Up to three matrices that share the activation rows (q/k/v, gate/up) in one launch.  Each
  * matrix i writes partials[i] as [S][rows][N_i] with the one S = guffin_hip_gemv_packed_multi_slices
  * of the launch.  All matrices must share the block length (Q4_K and Q6_K mix, Q8_0 does not). */
@@ -592,7 +603,7 @@ typedef struct guffin_verify_ticket {
     uint32_t* selected;                      /* device u32[2]: the selected path */
     void* candidates;                        /* device, 2 candidate records */
     uint32_t* status;                        /* device u32[3]: the pass's status word, one selection status per row */
-    uint32_t retain;                         /* candidates kept per row (top_k), 1..384 */
+    uint32_t retain;                         /* candidates kept per row (top_k), 1..320 */
     uint32_t state;                          /* GUFFIN_TXN_* */
     uint32_t rows, position, provisional_count;
     uint32_t provisional_path[GUFFIN_TICKET_MAX_ROWS];
