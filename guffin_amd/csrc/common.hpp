@@ -22,6 +22,20 @@ __host__ __device__ inline bool layer_is_local(uint32_t global_period, uint32_t 
     return global_period > 1 && (layer % global_period) != global_period - 1;
 }
 
+// ---- resident forward pass (resident.hip), used by the block graph of plan.hip ------------------
+constexpr uint32_t kResidentLayers = 6;   // blocks per launch (their pointers travel as kernel arguments)
+extern uint32_t g_spin_limit;
+extern unsigned long long* g_resident_stamps;
+extern int g_forward_mode;
+bool resident_fits(const guffin_model_desc& m, uint32_t rows);
+uint64_t resident_scratch_bytes(const guffin_model_desc& m, uint32_t rows);
+uint32_t resident_sync_words(const guffin_model_desc& m);
+int resident_launch(hipStream_t stream, const guffin_model_desc& m, uint32_t rows, uint32_t first, uint32_t count,
+                    uint8_t* exchange, uint32_t* sync_words, const float* rope_local, const float* rope_global,
+                    const uint32_t* schedule, const uint32_t* ancestors, void* priv_k, void* priv_v, const float* x_in,
+                    const void* u_receipt_in, float* x_out, float* u_out, void* u_receipt_out, uint32_t max_ring_tokens,
+                    uint32_t* status);
+
 // ---- typed loads at the alignment a GGUF block stream guarantees ------------
 struct __attribute__((packed, aligned(4))) U4a4 { uint32_t x, y, z, w; };
 struct __attribute__((packed, aligned(2))) U4a2 { uint32_t x, y, z, w; };

@@ -99,13 +99,14 @@ __device__ __forceinline__ void hist_add(uint32_t* hist, bool valid, uint32_t bi
 template <int kMine>
 __global__ void __launch_bounds__(1024)
 topk_merge_kernel(const float* __restrict__ logits, const uint64_t* __restrict__ survivors, uint32_t n_survivors,
-                  uint32_t vocab, uint32_t retain, float divisor, const uint32_t* __restrict__ history,
+                  uint32_t tile_keep, uint32_t vocab, uint32_t retain, float divisor, const uint32_t* __restrict__ history,
                   const uint32_t* __restrict__ history_count, Candidates* __restrict__ result,
                   uint32_t* __restrict__ status) {
     __shared__ uint32_t hist[256];
     __shared__ uint64_t sel[512];
     __shared__ uint64_t keys[512];  // selected keys in candidate order
     __shared__ uint32_t s_bin, s_above, s_count, s_in_bin;
+    __shared__ uint64_t floor_key;
     const uint32_t row = blockIdx.x, lane = threadIdx.x & 63;
     const uint64_t* src = survivors + size_t(row) * n_survivors;
     // up to kMine keys per thread stay in registers (8 for the verify pass's lists, 34 for the 257 per
@@ -117,81 +118,126 @@ topk_merge_kernel(const float* __restrict__ logits, const uint64_t* __restrict__
         const uint32_t i = threadIdx.x + u * blockDim.x;
         mine[u] = cached && i < n_survivors ? src[i] : 0;
     }
-    uint64_t prefix = 0;
-    uint32_t remaining = retain;  // rank of the wanted key among the keys that match `prefix`
-    for (int pass = 0; pass < 8; ++pass) {
-        const int shift = 56 - 8 * pass;
-        for (uint32_t i = threadIdx.x; i < 256; i += blockDim.x) hist[i] = 0;
-        __syncthreads();
-        if (cached) {
+    // Shortcut for sorted tile lists (tile_keep > 0: the survivors are `tiles` descending lists of tile_keep
+    // keys): the retain-th largest of the tiles' first r keys (tiles * r >= retain of them) is a lower bound
+    // of the retain-th largest key overall, so only keys at or above it can be selected.  They are few (a
+    // little over `retain` unless the logits tie massively); a rank sort of them is the exact answer.
+    bool done = false;
+    if (cached && tile_keep > 0) {
+        const uint32_t tiles = n_survivors / tile_keep;
+        const uint32_t r = (retain + tiles - 1) / tiles;
+        const uint32_t heads = tiles * r;
+        if (r <= tile_keep && heads <= 512) {
+            for (uint32_t i = threadIdx.x; i < heads; i += blockDim.x) sel[i] = src[(i / r) * tile_keep + i % r];
+            if (threadIdx.x == 0) { s_count = 0; floor_key = 0; }   // a floor of zero lets every key through
+            __syncthreads();
+            for (uint32_t i = threadIdx.x; i < heads; i += blockDim.x) {
+                const uint64_t k = sel[i];
+                uint32_t rank = 0;
+                for (uint32_t j = 0; j < heads; ++j) rank += sel[j] > k;
+                if (rank == retain - 1) floor_key = k;   // real keys are unique; only the zero padding repeats
+            }
+            __syncthreads();
+            const uint64_t bound = floor_key;
+            __syncthreads();
 #pragma unroll
             for (int u = 0; u < kMine; ++u) {
-                const uint64_t k = mine[u];
-                hist_add(hist, threadIdx.x + u * blockDim.x < n_survivors && (pass == 0 || (k >> (shift + 8)) == prefix),
-                         static_cast<uint32_t>(k >> shift) & 255u, lane);
-            }
-        } else {
-            for (uint32_t i0 = 0; i0 < n_survivors; i0 += blockDim.x) {  // whole waves stay converged
-                const uint32_t i = i0 + threadIdx.x;
-                const uint64_t k = i < n_survivors ? src[i] : 0;
-                hist_add(hist, i < n_survivors && (pass == 0 || (k >> (shift + 8)) == prefix),
-                         static_cast<uint32_t>(k >> shift) & 255u, lane);
-            }
-        }
-        __syncthreads();
-        if (threadIdx.x < 64) {  // lane l owns bins 255-4l .. 252-4l, highest first
-            uint32_t c[4];
-#pragma unroll
-            for (int j = 0; j < 4; ++j) c[j] = hist[255 - 4 * lane - j];
-            const uint32_t own = c[0] + c[1] + c[2] + c[3];
-            uint32_t incl = own;
-#pragma unroll
-            for (int d = 1; d < 64; d <<= 1) {
-                const uint32_t o = __shfl_up(incl, d, kWave);
-                if (lane >= uint32_t(d)) incl += o;
-            }
-            uint32_t above = incl - own;
-            if (above < remaining && remaining <= incl) {
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    if (remaining <= above + c[j]) { s_bin = 255 - 4 * lane - j; s_above = above; s_in_bin = c[j]; break; }
-                    above += c[j];
+                if (threadIdx.x + u * blockDim.x < n_survivors && mine[u] >= bound) {
+                    const uint32_t at = atomicAdd(&s_count, 1u);
+                    if (at < 512) sel[at] = mine[u];
                 }
             }
+            __syncthreads();
+            const uint32_t n = s_count;
+            if (n <= 512) {   // else: too many ties at the bound, the general path below decides
+                for (uint32_t i = threadIdx.x; i < n; i += blockDim.x) {
+                    const uint64_t k = sel[i];
+                    uint32_t rank = 0;
+                    for (uint32_t j = 0; j < n; ++j) rank += sel[j] > k;
+                    if (rank < retain) keys[rank] = k;
+                }
+                done = true;
+            }
+            __syncthreads();
+        }
+    }
+    if (!done) {
+        uint64_t prefix = 0;
+        uint32_t remaining = retain;  // rank of the wanted key among the keys that match `prefix`
+        for (int pass = 0; pass < 8; ++pass) {
+            const int shift = 56 - 8 * pass;
+            for (uint32_t i = threadIdx.x; i < 256; i += blockDim.x) hist[i] = 0;
+            __syncthreads();
+            if (cached) {
+    #pragma unroll
+                for (int u = 0; u < kMine; ++u) {
+                    const uint64_t k = mine[u];
+                    hist_add(hist, threadIdx.x + u * blockDim.x < n_survivors && (pass == 0 || (k >> (shift + 8)) == prefix),
+                             static_cast<uint32_t>(k >> shift) & 255u, lane);
+                }
+            } else {
+                for (uint32_t i0 = 0; i0 < n_survivors; i0 += blockDim.x) {  // whole waves stay converged
+                    const uint32_t i = i0 + threadIdx.x;
+                    const uint64_t k = i < n_survivors ? src[i] : 0;
+                    hist_add(hist, i < n_survivors && (pass == 0 || (k >> (shift + 8)) == prefix),
+                             static_cast<uint32_t>(k >> shift) & 255u, lane);
+                }
+            }
+            __syncthreads();
+            if (threadIdx.x < 64) {  // lane l owns bins 255-4l .. 252-4l, highest first
+                uint32_t c[4];
+    #pragma unroll
+                for (int j = 0; j < 4; ++j) c[j] = hist[255 - 4 * lane - j];
+                const uint32_t own = c[0] + c[1] + c[2] + c[3];
+                uint32_t incl = own;
+    #pragma unroll
+                for (int d = 1; d < 64; d <<= 1) {
+                    const uint32_t o = __shfl_up(incl, d, kWave);
+                    if (lane >= uint32_t(d)) incl += o;
+                }
+                uint32_t above = incl - own;
+                if (above < remaining && remaining <= incl) {
+    #pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        if (remaining <= above + c[j]) { s_bin = 255 - 4 * lane - j; s_above = above; s_in_bin = c[j]; break; }
+                        above += c[j];
+                    }
+                }
+            }
+            __syncthreads();
+            prefix = (prefix << 8) | s_bin;
+            remaining -= s_above;
+            // the upper 32 bits are the logit: if every key that shares the threshold logit is wanted
+            // (no tie across the cut), the token bits need no passes
+            if (pass == 3 && s_in_bin == remaining) { prefix <<= 32; remaining = 0; break; }
+        }
+        // `prefix` is the retain-th largest key; keys above it are taken, then `remaining` copies of it
+        // (more than one only for the zero padding of a short last tile)
+        if (threadIdx.x == 0) s_count = 0;
+        __syncthreads();
+        if (cached) {
+    #pragma unroll
+            for (int u = 0; u < kMine; ++u)
+                if (threadIdx.x + u * blockDim.x < n_survivors && mine[u] > prefix) sel[atomicAdd(&s_count, 1u)] = mine[u];
+        } else {
+            for (uint32_t i = threadIdx.x; i < n_survivors; i += blockDim.x) {
+                const uint64_t k = src[i];
+                if (k > prefix) sel[atomicAdd(&s_count, 1u)] = k;
+            }
         }
         __syncthreads();
-        prefix = (prefix << 8) | s_bin;
-        remaining -= s_above;
-        // the upper 32 bits are the logit: if every key that shares the threshold logit is wanted
-        // (no tie across the cut), the token bits need no passes
-        if (pass == 3 && s_in_bin == remaining) { prefix <<= 32; remaining = 0; break; }
-    }
-    // `prefix` is the retain-th largest key; keys above it are taken, then `remaining` copies of it
-    // (more than one only for the zero padding of a short last tile)
-    if (threadIdx.x == 0) s_count = 0;
-    __syncthreads();
-    if (cached) {
-#pragma unroll
-        for (int u = 0; u < kMine; ++u)
-            if (threadIdx.x + u * blockDim.x < n_survivors && mine[u] > prefix) sel[atomicAdd(&s_count, 1u)] = mine[u];
-    } else {
-        for (uint32_t i = threadIdx.x; i < n_survivors; i += blockDim.x) {
-            const uint64_t k = src[i];
-            if (k > prefix) sel[atomicAdd(&s_count, 1u)] = k;
+        const uint32_t above_total = s_count;
+        for (uint32_t i = threadIdx.x; i < remaining; i += blockDim.x) sel[above_total + i] = prefix;
+        __syncthreads();
+        for (uint32_t i = threadIdx.x; i < retain; i += blockDim.x) {
+            const uint64_t k = sel[i];
+            uint32_t rank = 0;
+            for (uint32_t j = 0; j < retain; ++j) {
+                const uint64_t o = sel[j];
+                rank += (o > k) || (o == k && j < i);
+            }
+            keys[rank] = k;
         }
-    }
-    __syncthreads();
-    const uint32_t above_total = s_count;
-    for (uint32_t i = threadIdx.x; i < remaining; i += blockDim.x) sel[above_total + i] = prefix;
-    __syncthreads();
-    for (uint32_t i = threadIdx.x; i < retain; i += blockDim.x) {
-        const uint64_t k = sel[i];
-        uint32_t rank = 0;
-        for (uint32_t j = 0; j < retain; ++j) {
-            const uint64_t o = sel[j];
-            rank += (o > k) || (o == k && j < i);
-        }
-        keys[rank] = k;
     }
     __syncthreads();
     Candidates& out = result[row];
@@ -318,10 +364,10 @@ int guffin::select_candidates_scaled(hipStream_t s, const float* logits, uint32_
     hipLaunchKernelGGL(topk_tile_kernel, dim3(tiles, rows), dim3(1024), 0, s, logits, surv, vocab, keep, divisor, status, suppressed_ok);
     if (int rc = check_launch("select_candidates(tile)")) return rc;
     if (tiles * keep <= 8 * 1024)
-        hipLaunchKernelGGL(topk_merge_kernel<8>, dim3(rows), dim3(1024), 0, s, logits, surv, tiles * keep, vocab,
+        hipLaunchKernelGGL(topk_merge_kernel<8>, dim3(rows), dim3(1024), 0, s, logits, surv, tiles * keep, keep, vocab,
                            keep, divisor, history, history_count, static_cast<Candidates*>(result), status);
     else
-        hipLaunchKernelGGL(topk_merge_kernel<34>, dim3(rows), dim3(1024), 0, s, logits, surv, tiles * keep, vocab,
+        hipLaunchKernelGGL(topk_merge_kernel<34>, dim3(rows), dim3(1024), 0, s, logits, surv, tiles * keep, keep, vocab,
                            keep, divisor, history, history_count, static_cast<Candidates*>(result), status);
     return check_launch("select_candidates(merge)");
 }

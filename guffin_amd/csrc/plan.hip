@@ -41,6 +41,9 @@ struct Scratch {
     float *attn_out, *attn_ml;
     float *rope_local, *rope_global;          // [rows][head_dim/2][2] cos/sin per frequency base
     uint32_t *positions, *ancestors, *schedule;
+    uint8_t* exchange;        // the resident pass's exchange buffers (models it covers)
+    uint32_t* sync;           // its barrier counters, cleared by the row-staging kernel
+    uint32_t sync_words;
     uint64_t bytes;
 };
 
@@ -106,6 +109,11 @@ Scratch layout(const guffin_model_desc& m, uint32_t rows, uint32_t position, uin
     s.positions = ar.take<uint32_t>(rows);
     s.ancestors = ar.take<uint32_t>(rows);
     s.schedule = ar.take<uint32_t>(uint64_t(m.layer_count) * rows * 4);
+    if (resident_fits(m, rows)) {
+        s.exchange = ar.take<uint8_t>(resident_scratch_bytes(m, rows));
+        s.sync_words = resident_sync_words(m);
+        s.sync = ar.take<uint32_t>(s.sync_words);
+    }
     s.bytes = (ar.used + 255) & ~uint64_t{255};
     return s;
 }
@@ -115,8 +123,9 @@ Scratch layout(const guffin_model_desc& m, uint32_t rows, uint32_t position, uin
 __global__ void stage_rows_kernel(uint32_t* positions, uint32_t* ancestors, uint32_t* schedule, uint32_t rows,
                                   uint32_t position, uint32_t layers, uint32_t window, uint32_t global_period,
                                   float2* rope_local, float2* rope_global, uint32_t rope_dim, float local_base,
-                                  float global_base, float global_scale) {
+                                  float global_base, float global_scale, uint32_t* sync, uint32_t sync_words) {
     const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < sync_words) sync[i] = 0u;   // barrier counters of the resident pass start at zero
     const uint32_t half = rope_dim / 2;
     if (i < rows * half) {
         float c, s;
@@ -166,15 +175,36 @@ int forward_rows(hipStream_t stream, const guffin_model_desc& m, const uint32_t*
     void* st = stream;
     const uint32_t H = m.hidden, F = m.ffn, QW = m.q_heads * m.head_dim, KW = m.kv_heads * m.head_dim;
     const float attn_scale = 1.0f / std::sqrt(static_cast<float>(m.head_dim));
-    const uint32_t n_stage = std::max(m.layer_count * rows, rows * (m.head_dim / 2));
+    // the resident pass is the default where it is the faster one: models with a single KV head (the drafter's
+    // small blocks); it can be forced for any model it covers
+    const bool resident = s.exchange != nullptr && (g_forward_mode == 2 || (g_forward_mode == 0 && m.kv_heads == 1));
+    if (g_forward_mode == 2 && !resident) return fail(GUFFIN_E_SHAPE, "forward: the resident pass does not cover this model");
+    const uint32_t sync_words = resident ? s.sync_words : 0u;
+    const uint32_t n_stage = std::max({m.layer_count * rows, rows * (m.head_dim / 2), sync_words});
     hipLaunchKernelGGL(stage_rows_kernel, dim3((n_stage + 63) / 64), dim3(64), 0, stream, s.positions, s.ancestors,
                        s.schedule, rows, position, m.layer_count, m.sliding_window, m.global_period,
                        reinterpret_cast<float2*>(s.rope_local), reinterpret_cast<float2*>(s.rope_global), m.head_dim,
-                       m.local_base, m.global_base, m.global_scale);
+                       m.local_base, m.global_base, m.global_scale, s.sync, sync_words);
     GUFFIN_TRY(check_launch("stage_rows"));
     GUFFIN_TRY(guffin_hip_embed(st, m.embed_dtype, m.embed_rows, tokens, s.x, rows, H,
                                 std::sqrt(static_cast<float>(H)), m.vocab, status));
     GUFFIN_TRY(guffin_hip_rms_norm(st, s.x, 1, 0, m.layers[0].norm[0], nullptr, s.u, s.us, rows, H, m.eps, status));
+    if (resident) {
+        // groups of blocks, each one launch whose workgroups stay on the chip; the residual rows and the
+        // normalised rows' receipt pass from launch to launch through s.x / s.us
+        uint32_t ring_tokens = 0;
+        for (uint32_t l = 0; l < m.layer_count; ++l) ring_tokens = std::max(ring_tokens, max_tokens_for(m, l, position, rows) - rows);
+        const uint32_t words_per_launch = s.sync_words / ((m.layer_count + kResidentLayers - 1) / kResidentLayers);
+        for (uint32_t first = 0, n = 0; first < m.layer_count; first += kResidentLayers, ++n) {
+            const uint32_t count = std::min(kResidentLayers, m.layer_count - first);
+            const bool last = first + count == m.layer_count;
+            GUFFIN_TRY(resident_launch(stream, m, rows, first, count, s.exchange, s.sync + size_t(n) * words_per_launch,
+                                       s.rope_local, s.rope_global, s.schedule, s.ancestors, priv_k, priv_v, s.x, s.us, s.x,
+                                       last ? out_hidden : s.u, last ? static_cast<void*>(out_hidden_sums) : static_cast<void*>(s.us),
+                                       ring_tokens, status));
+        }
+        return GUFFIN_OK;
+    }
     for (uint32_t l = 0; l < m.layer_count; ++l) {
         const guffin_layer_desc& L = m.layers[l];
         const bool local = is_local(m, l);

@@ -85,8 +85,8 @@ __device__ __forceinline__ void emit_receipt_values(const float (&v)[8], uint32_
 // from vals[0 .. count) (LDS or global).  Called by every thread of a workgroup whose size is a
 // multiple of 64; four consecutive lanes share a group.
 __device__ __forceinline__ void emit_receipt(const float* vals, uint32_t k0, uint32_t count, uint32_t r, uint32_t rows,
-                                             uint32_t K, void* blob) {
-    for (uint32_t t = threadIdx.x; t < count / 8; t += blockDim.x) {
+                                             uint32_t K, void* blob, uint32_t tid = threadIdx.x, uint32_t nthreads = blockDim.x) {
+    for (uint32_t t = tid; t < count / 8; t += nthreads) {
         float v[8];
 #pragma unroll
         for (int i = 0; i < 8; ++i) v[i] = vals[t * 8 + i];

@@ -47,6 +47,16 @@ def init(device=0):
         _inited.add(device)
 
 
+def set_forward_mode(mode):
+    """0: resident pass where the model fits (default), 1: one launch per operator, 2: resident or an error."""
+    check(lib().guffin_hip_set_forward_mode(mode))
+
+
+def set_spin_limit(polls):
+    """Bound of every wait inside the resident pass, in polls of a counter (default 2**20)."""
+    check(lib().guffin_hip_set_spin_limit(C.c_uint32(polls)))
+
+
 def _stream():
     return C.c_void_p(torch.cuda.current_stream().cuda_stream)
 

@@ -117,7 +117,9 @@ def tiny(shape, layers, vocab):
 class HostModel:
     """Canonical-layout numpy weights (what the CPU oracle consumes)."""
 
-    def __init__(self, shape, seed, position, gamma_sigma=0.1):
+    def __init__(self, shape, seed, position, gamma_sigma=0.1, untied_head=False):
+        """untied_head: the output head is a matrix of its own (a GGUF file's output.weight) instead of the
+        embedding matrix; with random weights a tied head puts nearly all mass on the input token."""
         self.shape = shape
         rng = np.random.Generator(np.random.PCG64(seed))
         self.w = []      # [layer][7] canonical uint8
@@ -140,6 +142,7 @@ class HostModel:
             self.ring_k.append(k)
             self.ring_v.append(v)
         self.embed = synth.make_weight(shape.embed_dtype, shape.hidden, shape.vocab, s + 999)
+        self.head = synth.make_weight(shape.embed_dtype, shape.hidden, shape.vocab, s + 998) if untied_head else self.embed
         self.out_norm = (1.0 + rng.normal(0, gamma_sigma, shape.hidden)).astype(np.float32)
 
     def commit(self, pk, pv, position, rows):
@@ -174,6 +177,7 @@ class DeviceModel:
         d.layers = C.cast(self.layers, C.POINTER(LayerDesc))
         self.keep += [embed_rows, head_tiles, out_norm]
         self.head_tiles = head_tiles   # the packed head matrix (tied embedding)
+        self.out_norm = out_norm       # device gamma of the output norm (a test may rescale it in place)
         self.ring_k_table = torch.tensor([t.data_ptr() for t in self.ring_k], dtype=torch.int64, device="cuda")
         self.ring_v_table = torch.tensor([t.data_ptr() for t in self.ring_v], dtype=torch.int64, device="cuda")
         return self
@@ -198,7 +202,8 @@ class DeviceModel:
             self.ring_v.append(rv)
             self.layers[l].ring_k, self.layers[l].ring_v = rk.data_ptr(), rv.data_ptr()
         embed = torch.from_numpy(host.embed).cuda()
-        head = hip.repack(sh.embed_dtype, embed, sh.hidden, sh.vocab)
+        head = hip.repack(sh.embed_dtype, embed if host.head is host.embed else torch.from_numpy(host.head).cuda(),
+                          sh.hidden, sh.vocab)
         torch.cuda.synchronize()
         return self._finish(embed, head, torch.from_numpy(host.out_norm).cuda())
 

@@ -46,6 +46,7 @@ extern "C" {
 #define GUFFIN_STATUS_NONFINITE 2u       /* non-finite activation or logit */
 #define GUFFIN_STATUS_KV_NONFINITE 8u    /* non-finite value narrowed into the fp16 KV rows */
 #define GUFFIN_STATUS_LAW_INVALID 16u    /* proposal / target law could not be built */
+#define GUFFIN_STATUS_SYNC 64u           /* a workgroup of the resident forward pass gave up a bounded wait */
 
 const char* guffin_hip_last_error(void);
 /* Binds the calling thread to `device`, checks that it is a gfx950 and raises the
@@ -373,6 +374,25 @@ int guffin_hip_forward_rows(void* stream, const guffin_model_desc* model, const 
                             uint32_t rows, uint32_t position, void* scratch, uint64_t scratch_bytes,
                             void* priv_k, void* priv_v, float* out_hidden, float* out_hidden_sums,
                             uint32_t* status);
+/* How guffin_hip_forward_rows (and so guffin_hip_h1_step, the sessions and the tickets) runs the blocks:
+ * 0 (default) the resident pass for models with one KV head that fit it (measured faster there), else one
+ * launch per operator; 1 always one launch per operator; 2 the resident pass for every model it covers
+ * (1 or 8 KV heads of 256, hidden width <= 4096, one block length per model), else GUFFIN_E_SHAPE.  The resident pass keeps one workgroup per CU for a
+ * group of blocks, gives each of the 8 XCDs one KV head (models with 8 KV heads; one XCD for a single KV
+ * head) and moves a block's intermediate rows through that XCD's L2; only the two reductions of a block
+ * cross XCDs.  Every wait in it is bounded by the spin limit (polls of a counter): a workgroup that gives up
+ * raises GUFFIN_STATUS_SYNC in the status word and the launch still ends.  Same results as the
+ * per-operator path up to fp32 summation order; a row's arithmetic does not depend on the row count in
+ * the projections.  No counterpart in the reference (its command buffers are per operator). */
+int guffin_hip_set_forward_mode(int mode);
+int guffin_hip_set_spin_limit(uint32_t polls);
+/* Profiling aid: with a device buffer of 16 * blocks u64 words set, workgroup 0 of the resident pass stores the
+ * 100 MHz clock at the start of each block's q/k/v projection, attention, o-projection, first norm pair,
+ * gate/up, down projection, second norm pair, and at the block's end (words 0-7 of the block), and inside the
+ * first norm pair after the device-wide wait, the slice sums, the XCD-wide wait and the first row sum (words
+ * 8-11).  NULL (default) switches it off. */
+int guffin_hip_set_resident_stamps(void* device_words);
+
 /* Publishes private rows into the rings of every layer at slot (position + row) & mask: all
  * `rows` when accepted is NULL, else row 0 and, if *accepted != 0, row 1 (provisional commit,
  * src/engine/chain_chat.mm:473-479).  ring_k_table / ring_v_table: device arrays of the

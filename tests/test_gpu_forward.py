@@ -73,12 +73,9 @@ def run_h1(hip, gfo, t_shape, d_shape, t_pos, d_pos, steps, seed, threads=8):
     support and the run sees acceptances and rejections.  Returns the decisions among the rest."""
     import torch
     from guffin_amd import model
-    t_host = model.HostModel(t_shape, seed=11, position=t_pos)
-    d_host = model.HostModel(d_shape, seed=12, position=d_pos)
-    # these random models' logits reach 9e4 (target) and 1e3 (drafter): bring them to a sampler's range,
-    # so that both laws spread over many tokens
-    t_host.out_norm *= np.float32(1e-4)
-    d_host.out_norm *= np.float32(1e-2)
+    # heads of their own: a random tied head puts nearly all mass on the input token
+    t_host = model.HostModel(t_shape, seed=11, position=t_pos, untied_head=True)
+    d_host = model.HostModel(d_shape, seed=12, position=d_pos, untied_head=True)
     target = model.DeviceModel.from_host(t_host)
     drafter = model.DeviceModel.from_host(d_host)
     root = 123
@@ -87,8 +84,16 @@ def run_h1(hip, gfo, t_shape, d_shape, t_pos, d_pos, steps, seed, threads=8):
     probe.step(0)
     torch.cuda.synchronize()
     assert int(probe.status.item()) == 0
-    d2t, t2d = gfo.correlating_map(probe.buffers()["q_logits"].cpu().numpy(), probe.buffers()["p_logits"].cpu().numpy()[0], root)
+    q0, p0 = probe.buffers()["q_logits"].cpu().numpy(), probe.buffers()["p_logits"].cpu().numpy()[0]
     del probe
+    # these random models' logits have a spread in the thousands: the output norms are rescaled (on the
+    # host and on the device alike) so that both laws spread over many tokens; the ranking, and with it the
+    # map below, is unchanged by the positive factor
+    for host, devm, logits in ((t_host, target, p0), (d_host, drafter, q0)):
+        factor = np.float32(1.5 / logits.std())
+        host.out_norm *= factor
+        devm.out_norm.copy_(torch.from_numpy(host.out_norm))
+    d2t, t2d = gfo.correlating_map(q0, p0, root)
     plan = model.H1Plan(target, drafter, t_pos, d_pos, seed=seed, publish=False, draft_to_target=d2t, target_to_draft=t2d)
     opt_cpu = gfo.SamplerOptions(1.0, 64, 0.95, 0.0, 1.0)
     none = np.zeros(0, np.uint32)
@@ -119,13 +124,13 @@ def run_h1(hip, gfo, t_shape, d_shape, t_pos, d_pos, steps, seed, threads=8):
             # numerical parity of both forwards and both heads against the CPU path
             dh, _, _ = gfo.forward(d_host, [root], d_pos, threads=threads)
             assert rel_rms(bufs["drafter_hidden"].cpu().numpy()[None, :], dh) <= 1e-3
-            ql = gfo.gemv(d_shape.embed_dtype, d_host.embed, dh, d_shape.vocab, threads=threads)
+            ql = gfo.gemv(d_shape.embed_dtype, d_host.head, dh, d_shape.vocab, threads=threads)
             assert rel_rms(bufs["q_logits"].cpu().numpy()[None, :], ql) <= 1e-3
             toks = bufs["tokens"].cpu().numpy().view(np.uint32)[:2]   # the verify pair: root, proposal
             assert toks[0] == root and toks[1] == proposal
             th, wk, wv = gfo.forward(t_host, toks, t_pos, threads=threads)
             assert rel_rms(bufs["target_hidden"].cpu().numpy(), th) <= 1e-3
-            pl = gfo.gemv(t_shape.embed_dtype, t_host.embed, th, t_shape.vocab, threads=threads)
+            pl = gfo.gemv(t_shape.embed_dtype, t_host.head, th, t_shape.vocab, threads=threads)
             assert rel_rms(bufs["p_logits"].cpu().numpy(), pl) <= 1e-3
             check_private_rows(plan.t_pk, wk)
             check_private_rows(plan.t_pv, wv)

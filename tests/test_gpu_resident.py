@@ -1,0 +1,103 @@
+"""The resident forward pass (one launch per group of blocks, one KV head per XCD, hand-over through the
+XCD's L2) against the launch-per-operator pass on the same model and rows, and against the CPU oracle.
+
+Bars: hidden rows of the two passes within 1e-4 of the row RMS of each other (both are fp32 sums of the same
+exact products, in different orders); private K/V rows equal in at least 99 % of their fp16 bit patterns;
+hidden rows within 1e-3 of the oracle.  A wait that gives up raises GUFFIN_STATUS_SYNC and the launch ends.
+"""
+from dataclasses import replace
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+STATUS_SYNC = 64
+
+
+@pytest.fixture(scope="module")
+def hip():
+    from guffin_amd import hip as module
+    module.init(0)
+    yield module
+    module.set_forward_mode(0)
+    module.set_spin_limit(1 << 20)
+
+
+def rel_rms(got, want):
+    want = want.astype(np.float64)
+    scale = np.sqrt((want ** 2).mean(axis=-1, keepdims=True)) + 1e-30
+    return float(np.max(np.abs(got.astype(np.float64) - want) / scale))
+
+
+CASES = [("drafter", 3, 1, 700), ("drafter", 7, 2, 5), ("drafter", 2, 1, 0), ("drafter", 6, 1, 4000),
+         ("target", 2, 2, 1500), ("target", 7, 2, 40), ("target", 2, 1, 0), ("target", 6, 2, 2046)]
+
+
+@pytest.mark.parametrize("kind,layers,rows,position", CASES)
+def test_resident_pass_equals_the_per_operator_pass(hip, gfo, kind, layers, rows, position):
+    import torch
+    from guffin_amd import model
+    if kind == "drafter":
+        shape = replace(model.GEMMA3_270M, layers=layers, vocab=4096, ring_global=4096)
+    else:
+        shape = replace(model.GEMMA3_12B, layers=layers, vocab=2048, ring_global=2048)
+    host = model.HostModel(shape, seed=3 + layers, position=position)
+    devm = model.DeviceModel.from_host(host)
+    tokens = torch.tensor([17, 1999][:rows], dtype=torch.int32, device="cuda")
+    print("resident case", kind, layers, rows, position, flush=True)
+    hip.set_forward_mode(1)
+    want = devm.forward(tokens, position)
+    torch.cuda.synchronize()
+    hip.set_forward_mode(2)
+    got = devm.forward(tokens, position)
+    torch.cuda.synchronize()
+    hip.set_forward_mode(0)
+    assert int(want[4].item()) == 0 and int(got[4].item()) == 0, (int(want[4].item()), int(got[4].item()))
+    assert rel_rms(got[0].cpu().numpy(), want[0].cpu().numpy()) <= 1e-4
+    assert np.allclose(got[1].cpu().numpy()[:rows * (shape.hidden // 16 + shape.hidden // 32)],
+                       want[1].cpu().numpy()[:rows * (shape.hidden // 16 + shape.hidden // 32)], rtol=0,
+                       atol=1e-3 * float(want[0].abs().max()))
+    for g, w in ((got[2], want[2]), (got[3], want[3])):
+        gb, wb = g.view(torch.int16).cpu().numpy(), w.view(torch.int16).cpu().numpy()
+        assert np.mean(gb == wb) >= 0.99
+        d = np.abs(g.float().cpu().numpy() - w.float().cpu().numpy())
+        assert d.max() <= 2.0 ** -9 * float(w.float().abs().max()) + 1e-6
+    oracle, wk, wv = gfo.forward(host, tokens.cpu().numpy().view(np.uint32), position, threads=8)
+    assert rel_rms(got[0].cpu().numpy(), oracle) <= 1e-3
+
+
+def test_a_wait_that_gives_up_raises_the_status_bit_and_the_launch_ends(hip):
+    import torch
+    from guffin_amd import model
+    shape = replace(model.GEMMA3_270M, layers=2, vocab=4096, ring_global=1024)
+    devm = model.DeviceModel.from_host(model.HostModel(shape, seed=9, position=100))
+    tokens = torch.tensor([5], dtype=torch.int32, device="cuda")
+    hip.set_forward_mode(2)
+    hip.set_spin_limit(0)       # the first poll that finds the counter short gives up
+    out = devm.forward(tokens, 100)
+    torch.cuda.synchronize()
+    assert int(out[4].item()) & STATUS_SYNC
+    hip.set_spin_limit(1 << 20)
+    again = devm.forward(tokens, 100)
+    torch.cuda.synchronize()
+    hip.set_forward_mode(0)
+    assert int(again[4].item()) == 0
+    assert bool(torch.isfinite(again[0]).all())
+
+
+def test_models_the_resident_pass_does_not_cover_use_the_per_operator_pass(hip, gfo):
+    import torch
+    from guffin_amd import model
+    shape = replace(model.GEMMA3_12B, layers=2, vocab=2048, ring_global=2048, q_heads=8, kv_heads=4)   # 4 KV heads
+    host = model.HostModel(shape, seed=21, position=300)
+    devm = model.DeviceModel.from_host(host)
+    tokens = torch.tensor([17, 1999], dtype=torch.int32, device="cuda")
+    hip.set_forward_mode(2)
+    with pytest.raises(hip.GuffinError):
+        devm.forward(tokens, 300)
+    hip.set_forward_mode(0)
+    got = devm.forward(tokens, 300)
+    torch.cuda.synchronize()
+    oracle, _, _ = gfo.forward(host, [17, 1999], 300, threads=8)
+    assert int(got[4].item()) == 0 and rel_rms(got[0].cpu().numpy(), oracle) <= 1e-3
