@@ -15,6 +15,9 @@
 // A global top-R entry is necessarily a top-R entry of its own tile, so the two stages lose
 // nothing.
 #include "common.hpp"
+#include "selection_request.hpp"
+
+#include <cstddef>
 
 namespace guffin {
 namespace {
@@ -99,15 +102,22 @@ __device__ __forceinline__ void hist_add(uint32_t* hist, bool valid, uint32_t bi
 template <int kMine>
 __global__ void __launch_bounds__(1024)
 topk_merge_kernel(const float* __restrict__ logits, const uint64_t* __restrict__ survivors, uint32_t n_survivors,
-                  uint32_t tile_keep, uint32_t vocab, uint32_t retain, float divisor, const uint32_t* __restrict__ history,
-                  const uint32_t* __restrict__ history_count, Candidates* __restrict__ result,
-                  uint32_t* __restrict__ status) {
+                  uint32_t tile_keep, uint32_t vocab, uint32_t retain_cap, float divisor, const uint32_t* __restrict__ history,
+                  const uint32_t* __restrict__ history_count, const uint32_t* __restrict__ row_retain, uint32_t row_stride,
+                  uint32_t history_stride, Candidates* __restrict__ result, uint32_t* __restrict__ status) {
     __shared__ uint32_t hist[256];
     __shared__ uint64_t sel[512];
     __shared__ uint64_t keys[512];  // selected keys in candidate order
     __shared__ uint32_t s_bin, s_above, s_count, s_in_bin;
     __shared__ uint64_t floor_key;
     const uint32_t row = blockIdx.x, lane = threadIdx.x & 63;
+    // a row may ask for fewer than the launch's capacity (top_k plus ITS history count); history_count
+    // and row_retain are read `row_stride` words apart (1, or the stride of a resolved-request record)
+    uint32_t retain = retain_cap;
+    if (row_retain) {
+        const uint32_t want = row_retain[size_t(row) * row_stride];
+        retain = want < 1 ? 1 : (want < retain_cap ? want : retain_cap);
+    }
     const uint64_t* src = survivors + size_t(row) * n_survivors;
     // up to kMine keys per thread stay in registers (8 for the verify pass's lists, 34 for the 257 per
     // tile that the proposal law asks for); longer survivor lists are re-read from memory in every pass
@@ -241,7 +251,7 @@ topk_merge_kernel(const float* __restrict__ logits, const uint64_t* __restrict__
     }
     __syncthreads();
     Candidates& out = result[row];
-    const uint32_t hc = history_count ? history_count[row] : 0;
+    const uint32_t hc = history_count ? history_count[size_t(row) * row_stride] : 0;
     for (uint32_t i = threadIdx.x; i < retain; i += blockDim.x) {
         const uint32_t token = key_token(keys[i]);
         out.values[i].token = token;
@@ -249,7 +259,7 @@ topk_merge_kernel(const float* __restrict__ logits, const uint64_t* __restrict__
     }
     uint32_t st = 0;
     for (uint32_t i = threadIdx.x; i < hc; i += blockDim.x) {
-        const uint32_t token = history[row * 64 + i];
+        const uint32_t token = history[size_t(row) * history_stride + i];
         if (token >= vocab) {
             st |= GUFFIN_STATUS_BAD_TOKEN;
             out.values[retain + i].token = 0xFFFFFFFFu;
@@ -266,6 +276,29 @@ topk_merge_kernel(const float* __restrict__ logits, const uint64_t* __restrict__
     if (threadIdx.x == 0) {
         out.count = retain + hc;
         out.status = status ? status[row] : 0;
+    }
+}
+
+// ---- selection requests --------------------------------------------------------------------
+// One wave per row: the raw ring and suffix become the resolved record and the row's history list.
+__global__ void __launch_bounds__(64)
+selection_requests_kernel(const SelectionRow* __restrict__ raw, uint32_t vocab, uint32_t top_k, uint32_t repetition,
+                          ResolvedRow* __restrict__ resolved, uint32_t* __restrict__ histories,
+                          uint32_t* __restrict__ status) {
+    const uint32_t row = blockIdx.x, lane = threadIdx.x;
+    const SelectionRow& r = raw[row];
+    uint32_t token = 0, st = 0;
+    const uint32_t count = resolve_history(r.history_token_ids, r.history_head, r.history_length, r.history_window_limit,
+                                           r.suffix_token_ids, r.suffix_count, vocab, repetition != 0, lane, token, st);
+    ResolvedRow& out = resolved[row];
+    out.history_token_ids[lane] = token;
+    if (histories) histories[size_t(row) * kRequestHistory + lane] = token;
+    if (lane == 0) {
+        out.top_k = top_k;
+        out.base_candidate_count = top_k + count;
+        out.history_count = count;
+        out.reserved = 0;
+        if (st && status) atomicOr(status, st);
     }
 }
 
@@ -339,7 +372,8 @@ extern "C" uint64_t guffin_hip_select_workspace_bytes(uint32_t rows, uint32_t vo
 namespace guffin {
 int select_candidates_scaled(hipStream_t s, const float* logits, uint32_t rows, uint32_t vocab, uint32_t retain,
                              float divisor, const uint32_t* history, const uint32_t* history_count,
-                             void* workspace, void* result, uint32_t* status, bool suppressed_ok = false);
+                             void* workspace, void* result, uint32_t* status, bool suppressed_ok = false,
+                             const uint32_t* row_retain = nullptr, uint32_t row_stride = 1);
 }
 
 extern "C" int guffin_hip_select_candidates(void* stream, const float* logits, uint32_t rows, uint32_t vocab,
@@ -352,7 +386,7 @@ extern "C" int guffin_hip_select_candidates(void* stream, const float* logits, u
 int guffin::select_candidates_scaled(hipStream_t s, const float* logits, uint32_t rows, uint32_t vocab,
                                      uint32_t retain, float divisor, const uint32_t* history,
                                      const uint32_t* history_count, void* workspace, void* result, uint32_t* status,
-                                     bool suppressed_ok) {
+                                     bool suppressed_ok, const uint32_t* row_retain, uint32_t row_stride) {
     if (!logits || !workspace || !result) return fail(GUFFIN_E_ARG, "select_candidates: null pointer");
     if (rows == 0 || vocab == 0) return fail(GUFFIN_E_SHAPE, "select_candidates: empty shape");
     if (retain == 0 || retain > 320) return fail(GUFFIN_E_CAPACITY, "select_candidates: retain must be in [1, 320] (top_k <= 256 plus 64 history tokens)");
@@ -365,11 +399,40 @@ int guffin::select_candidates_scaled(hipStream_t s, const float* logits, uint32_
     if (int rc = check_launch("select_candidates(tile)")) return rc;
     if (tiles * keep <= 8 * 1024)
         hipLaunchKernelGGL(topk_merge_kernel<8>, dim3(rows), dim3(1024), 0, s, logits, surv, tiles * keep, keep, vocab,
-                           keep, divisor, history, history_count, static_cast<Candidates*>(result), status);
+                           keep, divisor, history, history_count, row_retain, row_stride, row_stride == 1 ? 64u : row_stride,
+                           static_cast<Candidates*>(result), status);
     else
         hipLaunchKernelGGL(topk_merge_kernel<34>, dim3(rows), dim3(1024), 0, s, logits, surv, tiles * keep, keep, vocab,
-                           keep, divisor, history, history_count, static_cast<Candidates*>(result), status);
+                           keep, divisor, history, history_count, row_retain, row_stride, row_stride == 1 ? 64u : row_stride,
+                           static_cast<Candidates*>(result), status);
     return check_launch("select_candidates(merge)");
+}
+
+extern "C" int guffin_hip_selection_requests(void* stream, const void* raw, uint32_t rows, uint32_t vocab, uint32_t top_k,
+                                             uint32_t repetition_enabled, void* resolved, uint32_t* histories,
+                                             uint32_t* status) {
+    if (!raw || !resolved) return fail(GUFFIN_E_ARG, "selection_requests: null pointer");
+    if (rows == 0 || vocab == 0) return fail(GUFFIN_E_SHAPE, "selection_requests: empty shape");
+    if (top_k == 0 || top_k > 256) return fail(GUFFIN_E_CAPACITY, "selection_requests: top_k must be in [1, 256]");
+    if ((reinterpret_cast<uintptr_t>(raw) | reinterpret_cast<uintptr_t>(resolved)) & 3u)
+        return fail(GUFFIN_E_ALIGN, "selection_requests: rows must be 4-byte aligned");
+    hipLaunchKernelGGL(selection_requests_kernel, dim3(rows), dim3(64), 0, as_stream(stream),
+                       static_cast<const SelectionRow*>(raw), vocab, top_k, repetition_enabled,
+                       static_cast<ResolvedRow*>(resolved), histories, status);
+    return check_launch("selection_requests");
+}
+
+extern "C" int guffin_hip_select_candidates_resolved(void* stream, const float* logits, uint32_t rows, uint32_t vocab,
+                                                     uint32_t retain_capacity, const void* resolved, void* workspace,
+                                                     void* result, uint32_t* status) {
+    if (!resolved) return fail(GUFFIN_E_ARG, "select_candidates_resolved: null pointer");
+    const uint32_t* words = static_cast<const uint32_t*>(resolved);
+    constexpr uint32_t stride = sizeof(ResolvedRow) / 4;
+    // history ids, their count and the row's retain all sit in the record; the ids are 68 words apart too
+    return select_candidates_scaled(as_stream(stream), logits, rows, vocab, retain_capacity, 1.0f,
+                                    words + offsetof(ResolvedRow, history_token_ids) / 4,
+                                    words + offsetof(ResolvedRow, history_count) / 4, workspace, result, status, false,
+                                    words + offsetof(ResolvedRow, base_candidate_count) / 4, stride);
 }
 
 extern "C" int guffin_hip_argmax(void* stream, const float* logits, uint32_t rows, uint32_t vocab, void* workspace,

@@ -13,6 +13,7 @@
 // caller can capture a whole step into a HIP graph.
 #include <cstddef>
 #include "common.hpp"
+#include "selection_request.hpp"
 #include "receipt.hpp"
 
 #include <algorithm>
@@ -278,15 +279,32 @@ __global__ void draft_history_kernel(const uint32_t* history, uint32_t count, co
     out[t] = d < 0 ? 0xFFFFFFFFu : static_cast<uint32_t>(d);
 }
 
-// row 0 keeps the caller's history, row 1 the same plus the proposal (oldest dropped at 64)
-__global__ void build_history_kernel(const uint32_t* history, uint32_t count, const uint32_t* proposal, uint32_t* out) {
-    const uint32_t t = threadIdx.x;
-    const uint32_t drop = count == kHistoryWindow ? 1u : 0u, count1 = count + 1 - drop;
-    if (t < kHistoryWindow) {
-        out[t] = t < count ? history[t] : 0u;
-        out[kHistoryWindow + t] = t + 1 < count1 ? history[t + drop] : (t + 1 == count1 ? *proposal : 0u);
+// The two verify rows' selection requests: row 0 sees the caller's history, row 1 the same after the
+// proposal has been observed (a full window drops its oldest token), each without duplicates as the
+// sampler lists them (src/engine/sampling.cpp:352-378).  out: two resolved records, then the two lists
+// [2][64], then the two counts.  A history token outside the vocabulary is skipped and flagged.
+constexpr uint32_t kHistLists = 2 * sizeof(ResolvedRow) / 4, kHistCounts = kHistLists + 2 * kHistoryWindow,
+                   kHistDraft = kHistCounts + 2, kHistWords = kHistDraft + kHistoryWindow;
+__global__ void __launch_bounds__(128)
+build_history_kernel(const uint32_t* history, uint32_t count, const uint32_t* proposal, uint32_t vocab, uint32_t top_k,
+                     uint32_t* out, uint32_t* status) {
+    __shared__ uint32_t suffix[1];
+    const uint32_t row = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    if (threadIdx.x == 0) suffix[0] = *proposal;
+    __syncthreads();
+    uint32_t token = 0, st = 0;
+    const uint32_t kept = resolve_history(history, 0, count, kHistoryWindow, suffix, row, vocab, true, lane, token, st);
+    ResolvedRow& record = reinterpret_cast<ResolvedRow*>(out)[row];
+    record.history_token_ids[lane] = token;
+    out[kHistLists + row * kHistoryWindow + lane] = token;
+    if (lane == 0) {
+        record.top_k = top_k;
+        record.base_candidate_count = top_k + kept;
+        record.history_count = kept;
+        record.reserved = 0;
+        out[kHistCounts + row] = kept;
+        if (st && status) atomicOr(status, GUFFIN_STATUS_BAD_TOKEN);
     }
-    if (t == 0) { out[2 * kHistoryWindow] = count; out[2 * kHistoryWindow + 1] = count1; }
 }
 
 // the step's token slots: [0] root, [1] proposal (written later), [8..] the drafter's input rows
@@ -485,7 +503,7 @@ StepBuffers carve_step(const guffin_h1_desc* d, void* scratch) {
     b.law = ar.take<uint8_t>(4096 + 2 * 3088);  // the compact law, then the two candidate rows
     b.cands = b.law ? b.law + 4096 : nullptr;
     b.words = ar.take<uint32_t>(16);
-    b.hist = ar.take<uint32_t>(3 * 64 + 2);  // then the same history in the drafter's ids (with a vocabulary map)
+    b.hist = ar.take<uint32_t>(kHistWords);  // resolved requests, lists, counts, then the history in the drafter's ids
     if (d->full_law) {
         b.any_ws = ar.take<uint8_t>(guffin_hip_draft_law_any_workspace_bytes(D.vocab));
         b.full_cdf = ar.take<uint64_t>(uint64_t(D.vocab) + 1);
@@ -558,9 +576,9 @@ extern "C" int guffin_hip_h1_step(void* stream, const guffin_h1_desc* d, const u
         const uint32_t* draft_hist = nullptr;
         if (with_history) {
             hipLaunchKernelGGL(draft_history_kernel, dim3(1), dim3(64), 0, s, d->history, d->history_count, d->target_to_draft,
-                               T.vocab, B.hist + 2 * kHistoryWindow + 2);
+                               T.vocab, B.hist + kHistDraft);
             GUFFIN_TRY(check_launch("draft_history"));
-            draft_hist = B.hist + 2 * kHistoryWindow + 2;
+            draft_hist = B.hist + kHistDraft;
         }
         GUFFIN_TRY(guffin_hip_draft_law_mapped(stream, q_logits, D.vocab, d->draft_to_target, draft_hist,
                                                with_history ? d->history_count : 0u, &opt, d->seed, d->step, nullptr, law_ws,
@@ -587,19 +605,21 @@ extern "C" int guffin_hip_h1_step(void* stream, const guffin_h1_desc* d, const u
                                       p_logits, 2, T.hidden, V));
     // candidates: the top_k best plus one per history token (a penalised token can fall out of the
     // top_k, src/engine/sampling.cpp:430-446), then the history tokens' own logits
-    uint32_t retain = d->top_k;
     const uint32_t* hist = nullptr;
     if (with_history) {
-        hipLaunchKernelGGL(build_history_kernel, dim3(1), dim3(64), 0, s, d->history, d->history_count, tokens + 1, B.hist);
+        hipLaunchKernelGGL(build_history_kernel, dim3(1), dim3(128), 0, s, d->history, d->history_count, tokens + 1, V,
+                           d->top_k, B.hist, status);
         GUFFIN_TRY(check_launch("build_history"));
-        hist = B.hist;
-        retain = std::min<uint64_t>(V, uint64_t(d->top_k) + std::min(d->history_count + 1, kHistoryWindow));
+        hist = B.hist + kHistLists;
+        // capacity of the launch; each row retains top_k + its own deduplicated count
+        const uint32_t capacity = std::min<uint64_t>(V, uint64_t(d->top_k) + std::min(d->history_count + 1, kHistoryWindow));
+        GUFFIN_TRY(guffin_hip_select_candidates_resolved(stream, p_logits, 2, V, capacity, B.hist, sel_ws, cands, sel_status));
+    } else {
+        GUFFIN_TRY(guffin_hip_select_candidates(stream, p_logits, 2, V, d->top_k, nullptr, nullptr, sel_ws, cands, sel_status));
     }
-    GUFFIN_TRY(guffin_hip_select_candidates(stream, p_logits, 2, V, retain, hist, hist ? hist + 2 * kHistoryWindow : nullptr,
-                                            sel_ws, cands, sel_status));
     // 3. accept x or draw from the residual; on acceptance draw the next root from row 1
     GUFFIN_TRY(guffin_hip_spec_accept_mapped(stream, cands, law, full_cdf, D.vocab, d->target_to_draft, hist,
-                                             hist ? hist + 2 * kHistoryWindow : nullptr, tokens + 1, &opt, d->seed, d->step,
+                                             hist ? B.hist + kHistCounts : nullptr, tokens + 1, &opt, d->seed, d->step,
                                              nullptr, result, status));
     // 4. publish: the target keeps row 0, and row 1 if x was accepted; the drafter keeps the root
     if (d->target_ring_k && d->target_ring_v) {

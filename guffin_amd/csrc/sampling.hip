@@ -660,7 +660,8 @@ spec_accept_kernel(const Candidates* __restrict__ rows, const DraftLaw* __restri
 
 int select_candidates_scaled(hipStream_t s, const float* logits, uint32_t rows, uint32_t vocab, uint32_t retain,
                              float divisor, const uint32_t* history, const uint32_t* history_count,
-                             void* workspace, void* result, uint32_t* status, bool suppressed_ok = false);
+                             void* workspace, void* result, uint32_t* status, bool suppressed_ok = false,
+                             const uint32_t* row_retain = nullptr, uint32_t row_stride = 1);
 
 }  // namespace guffin
 

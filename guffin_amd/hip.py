@@ -361,6 +361,41 @@ def select_candidates(logits, retain, history=None, history_count=None, status=N
     return result, status
 
 
+selection_row_dtype = _np.dtype([("history_token_ids", _np.uint32, 64), ("suffix_token_ids", _np.uint32, 23),
+                                ("history_head", _np.uint32), ("history_length", _np.uint32),
+                                ("history_window_limit", _np.uint32), ("suffix_count", _np.uint32)])
+resolved_row_dtype = _np.dtype([("top_k", _np.uint32), ("base_candidate_count", _np.uint32),
+                               ("history_count", _np.uint32), ("reserved", _np.uint32),
+                               ("history_token_ids", _np.uint32, 64)])
+
+
+def selection_requests(raw, vocab, top_k, repetition_enabled=True):
+    """raw: numpy array of selection_row_dtype records.  Returns (resolved rows on the device as bytes,
+    histories [rows][64] on the device, the status word on the device)."""
+    raw = _np.ascontiguousarray(raw, selection_row_dtype).reshape(-1)
+    rows = raw.size
+    d_raw = torch.from_numpy(raw.view(_np.uint8).copy()).cuda()
+    resolved = _bytes(rows * resolved_row_dtype.itemsize)
+    histories = torch.zeros(rows, 64, dtype=torch.int32, device="cuda")
+    status = torch.zeros(1, dtype=torch.int32, device="cuda")
+    check(lib().guffin_hip_selection_requests(_stream(), _p(d_raw), rows, vocab, top_k, 1 if repetition_enabled else 0,
+                                              _p(resolved), _p(histories), _p(status)))
+    return resolved, histories, status
+
+
+def select_candidates_resolved(logits, retain_capacity, resolved, status=None, result=None):
+    rows, vocab = logits.shape
+    lib().guffin_hip_select_workspace_bytes.restype = C.c_uint64
+    ws = _bytes(lib().guffin_hip_select_workspace_bytes(rows, vocab, retain_capacity))
+    if result is None:
+        result = _bytes(rows * candidates_dtype.itemsize)
+    if status is None:
+        status = torch.zeros(rows, dtype=torch.int32, device=logits.device)
+    check(lib().guffin_hip_select_candidates_resolved(_stream(), _p(logits), rows, vocab, retain_capacity, _p(resolved),
+                                                      _p(ws), _p(result), _p(status)))
+    return result, status
+
+
 def candidates_to_numpy(result):
     return result.cpu().numpy().view(candidates_dtype)
 

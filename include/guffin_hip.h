@@ -250,6 +250,39 @@ uint64_t guffin_hip_select_workspace_bytes(uint32_t rows, uint32_t vocab, uint32
 int guffin_hip_select_candidates(void* stream, const float* logits, uint32_t rows, uint32_t vocab,
                                  uint32_t retain, const uint32_t* history, const uint32_t* history_count,
                                  void* workspace, void* result, uint32_t* status);
+/* Selection requests of a verify pass, resolved on the device: per row the raw sampler history (a ring
+ * of history_window_limit slots with the oldest token at history_head) and the suffix of tokens observed
+ * before that row become the window after the appends, without later duplicates, and
+ * base_candidate_count = top_k + its length.  Replaces verifier_selection_request_resolve_kernel
+ * (src/tensor/backends/metal/metal_kernels.mm:2336-2404); on the host the reference computes the same
+ * with make_token_selection_request (src/engine/sampling.cpp:352-392).
+ * raw:      rows x guffin_selection_row  (VerifierDeviceSelectionRow,
+ *           include/local_gguf_engine/engine/target_verifier.hpp:114-121), device
+ * resolved: rows x guffin_resolved_row   (VerifierResolvedSelectionRow, metal_kernels.mm:91-97), device
+ * histories: rows x 64 token ids (the lists again, as the candidate kernels of the reference read them), or NULL
+ * status:   ONE word with the reference's bits, not the GUFFIN_STATUS_* of the other entry points:
+ *           GUFFIN_REQUEST_MALFORMED (window > 64, length > window, suffix > 23, a head outside the
+ *           window: the row resolves to top_k with no history) and GUFFIN_REQUEST_BAD_TOKEN (a history
+ *           or suffix token >= vocab: it is left out of the list).
+ * repetition_enabled == 0 (a penalty of exactly 1): rows resolve to top_k with no history. */
+#define GUFFIN_REQUEST_MALFORMED 2u
+#define GUFFIN_REQUEST_BAD_TOKEN 4u
+typedef struct {
+    uint32_t history_token_ids[64]; uint32_t suffix_token_ids[23];
+    uint32_t history_head, history_length, history_window_limit, suffix_count;
+} guffin_selection_row;
+typedef struct {
+    uint32_t top_k, base_candidate_count, history_count, reserved; uint32_t history_token_ids[64];
+} guffin_resolved_row;
+int guffin_hip_selection_requests(void* stream, const void* raw, uint32_t rows, uint32_t vocab, uint32_t top_k,
+                                  uint32_t repetition_enabled, void* resolved, uint32_t* histories,
+                                  uint32_t* status);
+/* guffin_hip_select_candidates on resolved requests: row r keeps its base_candidate_count best logits
+ * (at most retain_capacity, which sizes the workspace: guffin_hip_select_workspace_bytes(rows, vocab,
+ * retain_capacity)) and then the logits of its history_token_ids. */
+int guffin_hip_select_candidates_resolved(void* stream, const float* logits, uint32_t rows, uint32_t vocab,
+                                          uint32_t retain_capacity, const void* resolved, void* workspace,
+                                          void* result, uint32_t* status);
 /* Greedy token per row, strict '>' so the lowest id wins ties (src/tensor/ops/reduction.cpp:93-117).
  * workspace: rows * 256 * 8 bytes.  logit may be NULL. */
 int guffin_hip_argmax(void* stream, const float* logits, uint32_t rows, uint32_t vocab, void* workspace,

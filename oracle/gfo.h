@@ -104,6 +104,25 @@ int gfo_select_candidates(const float* logits, uint32_t vocab, uint32_t k,
                           const uint32_t* history, uint32_t history_count,
                           gfo_token_logit* out);
 
+/* ---- selection requests ------------------------------------------------ */
+/* One verify row's raw sampler history (a ring of `history_window_limit` slots, oldest at
+ * `history_head`) plus the hypothetical suffix of tokens before that row, and what the selection
+ * needs of it: the window after appending the suffix, without duplicates, first occurrence first.
+ * Layouts: VerifierDeviceSelectionRow (include/local_gguf_engine/engine/target_verifier.hpp:114-121)
+ * and VerifierResolvedSelectionRow (src/tensor/backends/metal/metal_kernels.mm:91-97). */
+typedef struct {
+    uint32_t history_token_ids[64]; uint32_t suffix_token_ids[23];
+    uint32_t history_head, history_length, history_window_limit, suffix_count;
+} gfo_selection_row;
+typedef struct {
+    uint32_t top_k, base_candidate_count, history_count, reserved; uint32_t history_token_ids[64];
+} gfo_resolved_row;
+/* append_sampler_history + make_token_selection_request (src/engine/sampling.cpp:329-378) with the
+ * status bits of the device version (metal_kernels.mm:2351-2371): 2 for a malformed row (the host
+ * version throws), 4 for a token outside the vocabulary (it is skipped).  Returns the status bits. */
+uint32_t gfo_selection_request(const gfo_selection_row* raw, uint32_t vocab, uint32_t top_k,
+                               int repetition_enabled, gfo_resolved_row* out);
+
 /* ---- sampling law ------------------------------------------------------ */
 typedef struct {
     float temperature; uint32_t top_k; float top_p; float min_p; float repetition_penalty;

@@ -14,6 +14,12 @@ BLOCK_BYTES = {Q8_0: 34, Q4_K: 144, Q6_K: 210}
 BLOCK_ELEMS = {Q8_0: 32, Q4_K: 256, Q6_K: 256}
 
 token_logit = np.dtype([("token", np.uint32), ("logit", np.float32)])
+# one verify row's raw sampler history and its resolved form (364 and 272 bytes, the reference's layouts)
+selection_row = np.dtype([("history_token_ids", np.uint32, 64), ("suffix_token_ids", np.uint32, 23),
+                          ("history_head", np.uint32), ("history_length", np.uint32),
+                          ("history_window_limit", np.uint32), ("suffix_count", np.uint32)])
+resolved_row = np.dtype([("top_k", np.uint32), ("base_candidate_count", np.uint32), ("history_count", np.uint32),
+                         ("reserved", np.uint32), ("history_token_ids", np.uint32, 64)])
 
 
 class SamplerOptions(C.Structure):
@@ -201,6 +207,24 @@ def select_candidates(logits, k, history=()):
     if n < 0:
         raise ValueError("non-finite selected logit")
     return out[:n]
+
+
+def selection_request(raw, vocab, top_k, repetition_enabled=True):
+    """raw: one selection_row record -> (resolved_row record, status bits)."""
+    raw = np.ascontiguousarray(raw, selection_row).reshape(1)
+    out = np.zeros(1, resolved_row)
+    fn = lib().gfo_selection_request
+    fn.restype = C.c_uint32
+    status = fn(_ptr(raw), C.c_uint32(vocab), C.c_uint32(top_k), C.c_int(1 if repetition_enabled else 0), _ptr(out))
+    return out[0], int(status)
+
+
+def ref_selection_request(raw, top_k, repetition_enabled=True):
+    """The compiled reference's make_token_selection_request; None where it throws."""
+    raw = np.ascontiguousarray(raw, selection_row).reshape(1)
+    out = np.zeros(1, resolved_row)
+    rc = ref().gfr_selection_request(_ptr(raw), C.c_uint32(top_k), C.c_int(1 if repetition_enabled else 0), _ptr(out))
+    return out[0] if rc == 0 else None
 
 
 def prepare(cands, opt, history=(), which=None):

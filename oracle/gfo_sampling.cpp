@@ -560,4 +560,45 @@ void gfo_step_draws(uint64_t seed, uint64_t step, uint32_t* word, double* u_acce
     *u_next = unit_double(b[2], b[3]);
 }
 
+uint32_t gfo_selection_request(const gfo_selection_row* raw, uint32_t vocab, uint32_t top_k,
+                               int repetition_enabled, gfo_resolved_row* out) {
+    std::memset(out, 0, sizeof *out);
+    out->top_k = top_k;
+    out->base_candidate_count = top_k;
+    const uint32_t limit = raw->history_window_limit;
+    if (limit > 64 || raw->history_length > limit || raw->suffix_count > 23
+        || (raw->history_length == 0 && raw->history_head != 0)
+        || (raw->history_length > 0 && raw->history_head >= limit))
+        return 2u;
+    uint32_t status = 0;
+    // the ring as the sampler keeps it: appending to a full window overwrites the oldest slot
+    uint32_t ring[64], head = raw->history_head, length = raw->history_length;
+    for (uint32_t i = 0; i < 64; ++i) ring[i] = raw->history_token_ids[i];
+    for (uint32_t i = 0; i < length; ++i)
+        if (ring[(head + i) % limit] >= vocab) status |= 4u;
+    for (uint32_t i = 0; i < raw->suffix_count; ++i) {
+        const uint32_t token = raw->suffix_token_ids[i];
+        if (token >= vocab) status |= 4u;
+        if (limit == 0) continue;
+        if (length < limit) {
+            ring[(head + length) % limit] = token;
+            ++length;
+        } else {
+            ring[head] = token;
+            head = (head + 1) % limit;
+        }
+    }
+    if (repetition_enabled) {
+        for (uint32_t i = 0; i < length; ++i) {
+            const uint32_t token = ring[(head + i) % limit];
+            if (token >= vocab) continue;
+            bool seen = false;
+            for (uint32_t j = 0; j < out->history_count; ++j) seen = seen || out->history_token_ids[j] == token;
+            if (!seen) out->history_token_ids[out->history_count++] = token;
+        }
+    }
+    out->base_candidate_count = top_k + out->history_count;
+    return status;
+}
+
 }  // extern "C"

@@ -240,4 +240,32 @@ int gfr_spec_accept(const gfo_token_logit* row0, uint32_t n0, const gfo_token_lo
     return 0;
 } catch (...) { return -1; }
 
+// make_token_selection_request(options, DeviceSelectionRequest) (sampling.cpp:380-392): the host
+// definition the device request resolver must reproduce.  Returns -1 where the reference throws.
+int gfr_selection_request(const gfo_selection_row* raw, uint32_t top_k, int repetition_enabled,
+                          gfo_resolved_row* out) try {
+    std::memset(out, 0, sizeof(*out));
+    e::TokenSamplerOptions options;
+    options.temperature = 0.8F;
+    options.top_k = top_k;
+    options.top_p = 1.0F;
+    options.min_p = 0.0F;
+    options.repetition_penalty = repetition_enabled ? 1.1F : 1.0F;
+    options.seed = 1;
+    options.repetition_window = raw->history_window_limit;
+    e::DeviceSelectionRequest request;
+    for (uint32_t i = 0; i < 64; ++i) request.history.token_ids[i] = raw->history_token_ids[i];
+    request.history.head = raw->history_head;
+    request.history.length = raw->history_length;
+    request.history.window_limit = raw->history_window_limit;
+    for (uint32_t i = 0; i < 23; ++i) request.suffix_token_ids[i] = raw->suffix_token_ids[i];
+    request.suffix_count = raw->suffix_count;
+    const auto resolved = e::make_token_selection_request(options, request);
+    out->top_k = resolved.top_k;
+    out->base_candidate_count = resolved.base_candidate_count;
+    out->history_count = resolved.history_token_count;
+    for (uint32_t i = 0; i < resolved.history_token_count; ++i) out->history_token_ids[i] = resolved.history_token_ids[i];
+    return 0;
+} catch (...) { return -1; }
+
 }  // extern "C"

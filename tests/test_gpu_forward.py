@@ -216,6 +216,7 @@ def test_h1_cycle_with_sampler_history(hip, gfo):
     differs = 0
     for count in (9, 64):
         history = np.concatenate([rng.integers(0, 8192, count - best.size).astype(np.uint32), best])
+        history[1] = history[0]   # a token seen twice is listed, penalised and counted once
         plan = model.H1Plan(target, drafter, 600, 600, temperature=1.0, top_k=32, seed=9, publish=False,
                             history=history.tolist(), repetition_penalty=1.9)
         opt_cpu = gfo.SamplerOptions(1.0, 32, 0.95, 0.0, 1.9)
@@ -237,10 +238,18 @@ def test_h1_cycle_with_sampler_history(hip, gfo):
             proposal = gfo.lib().gfo_draft_select(C.byref(law), C.c_uint32(word))
             assert res["proposal"] == proposal
             hist1 = np.concatenate([history, [proposal]]).astype(np.uint32)[-64:]
-            retain = 32 + min(count + 1, 64)
+            # each row retains top_k + its own count of distinct history tokens (base_candidate_count,
+            # src/engine/sampling.cpp:352-378) and then lists those tokens' logits, first occurrence first
+            uniq0, uniq1 = [np.array(list(dict.fromkeys(h.tolist())), np.uint32) for h in (history, hist1)]
             p_logits = bufs["p_logits"].cpu().numpy()
-            r0 = gfo.select_candidates(p_logits[0], retain, history)
-            r1 = gfo.select_candidates(p_logits[1], retain, hist1)
+            r0 = gfo.select_candidates(p_logits[0], 32 + uniq0.size, uniq0)
+            r1 = gfo.select_candidates(p_logits[1], 32 + uniq1.size, uniq1)
+            got = hip.candidates_to_numpy(bufs["candidates"])
+            for row, want_row in enumerate((r0, r1)):
+                assert got[row]["count"] == want_row.size
+                assert np.array_equal(got[row]["values"]["token"][:want_row.size], want_row["token"])
+                assert np.array_equal(got[row]["values"]["logit"][:want_row.size].view(np.uint32),
+                                      want_row["logit"].view(np.uint32))
             rc, want = gfo.spec_accept_history(r0, history, r1, hist1, law, proposal, opt_cpu, ua, ur, un)
             assert rc == 0
             assert (res["accepted"], res["token"], res["next_root"]) == (want.accepted, want.token, want.next_root)
