@@ -279,6 +279,13 @@ topk_merge_kernel(const float* __restrict__ logits, const uint64_t* __restrict__
     }
 }
 
+// ---- verify-row input validation --------------------------------------------------------------
+__global__ void input_validation_kernel(const uint32_t* __restrict__ actual, const uint32_t* __restrict__ expected,
+                                        uint32_t rows, uint32_t vocab, uint32_t* __restrict__ status) {
+    const uint32_t row = blockIdx.x * blockDim.x + threadIdx.x;
+    if (row < rows && (actual[row] >= vocab || actual[row] != expected[row])) atomicOr(status, GUFFIN_STATUS_BAD_TOKEN);
+}
+
 // ---- selection requests --------------------------------------------------------------------
 // One wave per row: the raw ring and suffix become the resolved record and the row's history list.
 __global__ void __launch_bounds__(64)
@@ -406,6 +413,15 @@ int guffin::select_candidates_scaled(hipStream_t s, const float* logits, uint32_
                            keep, divisor, history, history_count, row_retain, row_stride, row_stride == 1 ? 64u : row_stride,
                            static_cast<Candidates*>(result), status);
     return check_launch("select_candidates(merge)");
+}
+
+extern "C" int guffin_hip_input_validation(void* stream, const uint32_t* actual, const uint32_t* expected, uint32_t rows,
+                                           uint32_t vocab, uint32_t* status) {
+    if (!actual || !expected || !status) return fail(GUFFIN_E_ARG, "input_validation: null pointer");
+    if (rows == 0 || vocab == 0) return fail(GUFFIN_E_SHAPE, "input_validation: empty shape");
+    hipLaunchKernelGGL(input_validation_kernel, dim3((rows + 63) / 64), dim3(64), 0, as_stream(stream), actual, expected,
+                       rows, vocab, status);
+    return check_launch("input_validation");
 }
 
 extern "C" int guffin_hip_selection_requests(void* stream, const void* raw, uint32_t rows, uint32_t vocab, uint32_t top_k,

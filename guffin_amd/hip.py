@@ -369,6 +369,10 @@ resolved_row_dtype = _np.dtype([("top_k", _np.uint32), ("base_candidate_count", 
                                ("history_token_ids", _np.uint32, 64)])
 
 
+def input_validation(actual, expected, vocab, status):
+    check(lib().guffin_hip_input_validation(_stream(), _p(actual), _p(expected), actual.numel(), vocab, _p(status)))
+
+
 def selection_requests(raw, vocab, top_k, repetition_enabled=True):
     """raw: numpy array of selection_row_dtype records.  Returns (resolved rows on the device as bytes,
     histories [rows][64] on the device, the status word on the device)."""

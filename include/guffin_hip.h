@@ -250,6 +250,12 @@ uint64_t guffin_hip_select_workspace_bytes(uint32_t rows, uint32_t vocab, uint32
 int guffin_hip_select_candidates(void* stream, const float* logits, uint32_t rows, uint32_t vocab,
                                  uint32_t retain, const uint32_t* history, const uint32_t* history_count,
                                  void* workspace, void* result, uint32_t* status);
+/* The token ids a verify pass reads on the device against the ids the host planned: a row whose id is
+ * outside the vocabulary or differs sets GUFFIN_STATUS_BAD_TOKEN in the one status word.  Replaces
+ * encode_verifier_input_validation (metal_command_context.hpp:221; verifier_input_validate_u32_kernel,
+ * src/tensor/backends/metal/metal_kernels.mm:2323-2334, which sets the same bit 1). */
+int guffin_hip_input_validation(void* stream, const uint32_t* actual, const uint32_t* expected, uint32_t rows,
+                                uint32_t vocab, uint32_t* status);
 /* Selection requests of a verify pass, resolved on the device: per row the raw sampler history (a ring
  * of history_window_limit slots with the oldest token at history_head) and the suffix of tokens observed
  * before that row become the window after the appends, without later duplicates, and

@@ -85,3 +85,18 @@ def test_candidates_of_resolved_rows_keep_each_rows_own_count(hip, gfo):
         assert int(st[r]) == 0 and c[r]["count"] == want.size
         assert np.array_equal(c[r]["values"]["token"][:want.size], want["token"])
         assert np.array_equal(c[r]["values"]["logit"][:want.size].view(np.uint32), want["logit"].view(np.uint32))
+
+
+def test_input_validation_flags_a_foreign_or_changed_token(hip):
+    """verifier_input_validate_u32_kernel (metal_kernels.mm:2323-2334): bit 1 when a row's id is outside
+    the vocabulary or is not the id the host planned."""
+    import torch
+    def run(actual, expected, vocab=100):
+        status = torch.zeros(1, dtype=torch.int32, device="cuda")
+        hip.input_validation(torch.tensor(actual, dtype=torch.int32).cuda(), torch.tensor(expected, dtype=torch.int32).cuda(),
+                             vocab, status)
+        return int(status.item())
+    assert run([1, 2, 99], [1, 2, 99]) == 0
+    assert run([1, 2, 3], [1, 5, 3]) == 1
+    assert run([1, 100], [1, 100]) == 1
+    assert run(list(range(90)) + [7], list(range(90)) + [8]) == 1
