@@ -10,17 +10,21 @@ graph; `value` is the mean step latency in microseconds with every input residen
 Extra objects on the JSON line:
   roofline      the dominant kernel (2-row Q4_K gate+up GEMV fused with GeGLU, 66.4 MB of weights
                 per launch): algorithmic bytes / mean launch duration, measured with HIP events
-                around a graph of 48 back-to-back launches over the 48 blocks' own weights
-                (3.2 GB, far beyond the caches) on the launch stream.
+                around graphs of 48 back-to-back launches over the 48 blocks' own weights
+                (3.2 GB, far beyond the caches) on the launch stream; min / max over the replays and
+                over single launches; `traffic` is read from the committed counter profile.
+  rooflines     the same figures for the step's other streaming kernels worth watching: the local
+                layers' attention (the kernel furthest from its bound) and the down projection.
   configs       configs 0-3 on their own (one Q4_K GEMV at 1 row; one block's seven GEMVs at 2 rows;
                 the drafter's decode with head and argmax; the Q6_K head with selection and
                 acceptance): microseconds per unit as HIP graphs, algorithmic bytes, GB/s and the
                 fraction of the 8 TB/s HBM peak.
   prefill       config 4's second half: a 2048-token prompt through the same stack.
   cpu_baseline  the reference's own CPU row dot (oracle/_ref) or the oracle port timed on the
-                host cores on a bounded sample (one block's seven GEMVs at 2 rows, a column
-                subset), extrapolated to a whole step by weight count; `all_cores` is the oracle's
-                threaded row dot on the same GEMVs over the host's cores.  Reported, not a target.
+                host cores: configs 0 and 1 in full, config 3 on a vocabulary slice plus the oracle's
+                selection, law and acceptance in full, config 2 by weight count; the step is 48 blocks +
+                head + drafter from those.  Each config's figure also sits in configs[i].cpu_baseline.
+                `all_cores` is the oracle's threaded row dot over the host's cores.  Reported, not a target.
 """
 import argparse
 import json
@@ -53,8 +57,9 @@ def step_bytes(T, D, t_pos, d_pos):
     return model_bytes(T, 2, t_pos) + model_bytes(D, 1, d_pos)
 
 
-def timed_graph(fn, reps=10, warm=3):
-    """fn's launches captured as one HIP graph; microseconds per replay, from events on the launch stream."""
+def replay_times(fn, reps=10, warm=3):
+    """fn's launches captured as one HIP graph; microseconds of each of `reps` warmed replays, from event
+    pairs on the launch stream (recorded back to back, read after one synchronisation)."""
     import torch
     fn()
     torch.cuda.synchronize()
@@ -64,13 +69,84 @@ def timed_graph(fn, reps=10, warm=3):
     for _ in range(warm):
         graph.replay()
     stream = torch.cuda.current_stream()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record(stream)
-    for _ in range(reps):
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(reps + 1)]
+    marks[0].record(stream)
+    for i in range(reps):
         graph.replay()
-    e1.record(stream)
+        marks[i + 1].record(stream)
     torch.cuda.synchronize()
-    return e0.elapsed_time(e1) * 1e3 / reps
+    return [marks[i].elapsed_time(marks[i + 1]) * 1e3 for i in range(reps)]
+
+
+def timed_graph(fn, reps=10, warm=3):
+    """Mean microseconds per replay."""
+    times = replay_times(fn, reps, warm)
+    return sum(times) / len(times)
+
+
+def profile_traffic(kernel_prefix):
+    """HBM bytes per launch of a kernel from the committed counter profile (two rocprofv3 --pmc runs,
+    copy-calibrated): the line `FETCH_SIZE a KiB x f + WRITE_SIZE b KiB x g` under the kernel's name."""
+    import re
+    path = os.path.join(ROOT, "profiles", "gateup_geglu_q4k_hbm_traffic.txt")
+    if not os.path.exists(path):
+        return None, None
+    lines = open(path).read().splitlines()
+    for i, text in enumerate(lines[:-1]):
+        if text.startswith(kernel_prefix):
+            m = re.search(r"FETCH_SIZE ([0-9.]+) KiB x ([0-9.]+) \+ WRITE_SIZE ([0-9.]+) KiB x ([0-9.]+)", lines[i + 1])
+            if m:
+                a, f, b, g = (float(v) for v in m.groups())
+                return int(round((a * f + b * g) * 1024)), "profiles/gateup_geglu_q4k_hbm_traffic.txt"
+    return None, None
+
+
+def kernel_roofline(name, launch, layers, bytes_per_launch, traffic_prefix, replays=12):
+    """Roofline object of one streaming kernel.  launch(l) enqueues the kernel on block l's own operands, so
+    a graph of `layers` launches streams from HBM; sustained figures come from `replays` warmed replays
+    (layers * replays >= 100 launches), single-launch figures from event pairs around 3 * layers launches
+    enqueued back to back."""
+    import torch
+
+    def all_layers():
+        for l in layers:
+            launch(l)
+
+    per_replay = [t / len(layers) for t in replay_times(all_layers, reps=max(replays, -(-100 // len(layers))))]
+    launch_us = sum(per_replay) / len(per_replay)
+    stream = torch.cuda.current_stream()
+    count = 3 * len(layers)
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(count + 1)]
+    all_layers()                      # warm
+    torch.cuda.synchronize()
+    marks[0].record(stream)
+    for i in range(count):
+        launch(layers[i % len(layers)])
+        marks[i + 1].record(stream)
+    torch.cuda.synchronize()
+    single = sorted(marks[i].elapsed_time(marks[i + 1]) * 1e3 for i in range(count))
+    # the same kernel dispatched alone (one launch, then a wait): the reference's benchmark reports both an
+    # isolated and a sustained mode (include/local_gguf_engine/benchmarks/quick_benchmark.hpp:13-17)
+    isolated = []
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    for rep in range(len(layers)):
+        e0.record(stream)
+        launch(layers[rep])
+        e1.record(stream)
+        torch.cuda.synchronize()
+        isolated.append(e0.elapsed_time(e1) * 1e3)
+    achieved = bytes_per_launch / launch_us / 1e3  # GB/s
+    traffic, source = profile_traffic(traffic_prefix) if traffic_prefix else (None, None)
+    return {
+        "kernel": name, "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+        "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic, "traffic_source": source,
+        "bytes_per_launch": int(bytes_per_launch), "launch_us": round(launch_us, 3),
+        "launch_us_min": round(min(per_replay), 3), "launch_us_max": round(max(per_replay), 3),
+        "launches": len(per_replay) * len(layers), "sustained_dispatches": len(layers),
+        "single_launch_us": {"min": round(single[0], 3), "median": round(single[len(single) // 2], 3),
+                             "max": round(single[-1], 3), "launches": count},
+        "isolated_launch_us": round(sorted(isolated)[len(isolated) // 2], 3),
+    }
 
 
 def config_figures(target, drafter, T, D, d_pos):
@@ -167,62 +243,86 @@ def config_figures(target, drafter, T, D, d_pos):
     return out
 
 
-def cpu_baseline(T, D, budget_s=20.0):
-    """Times the CPU path on a bounded sample and extrapolates to one step by weight count."""
+def cpu_baseline(T, D):
+    """The CPU path on the host's cores, per config and for the step.  Configs 0 and 1 run in full, config 3's
+    head on a vocabulary slice (scaled) with the oracle's selection, law and acceptance in full, config 2 by
+    weight count from one drafter block and a slice of its head; the step is 48 blocks + head + drafter."""
+    import ctypes as C
     import numpy as np
     from guffin_amd import synth
     from oracle import gfo
     gfo.build()
     ref = gfo.ref()
     kind = "reference" if ref is not None else "port"
-    cores = 1 if ref is not None else (os.cpu_count() or 1)
+    cores = 1 if ref is not None else min(os.cpu_count() or 1, 16)
+    how = ("reference dot_q4_k_row_f32 / dot_q6_k_row_f32 (src/tensor/quantization.cpp), single thread" if ref is not None
+           else "oracle gfo_gemv_mt on %d host threads" % cores)
+    seeds = iter(range(10, 10 ** 6))
+
+    def gemv_seconds(dt, K, n, rows, threads=cores, which=ref):
+        w = synth.make_weight(dt, K, n, next(seeds))
+        x = synth.make_activation(rows, K, next(seeds))
+        t0 = time.perf_counter()
+        gfo.gemv(dt, w, x, n, threads=threads, which=which)
+        return time.perf_counter() - t0
+
+    def figure(seconds, sample):
+        return {"us": round(seconds * 1e6, 1), "cores": cores, "kind": kind, "sample": sample}
+
+    print("bench: cpu baseline, config 1 (one block in full, twice)", file=sys.stderr, flush=True)
     shapes = list(zip(T.dtypes, T.proj_shapes()))
-    # calibrate on a small slice, then size the sample to the budget
-    dt, (K, N) = shapes[0]
-    w = synth.make_weight(dt, K, 64, 1)
-    x = synth.make_activation(2, K, 2)
+    repeats = 2
+    block_s = sum(gemv_seconds(dt, K, N, 2) for _ in range(repeats) for dt, (K, N) in shapes) / repeats
+    print("bench: cpu baseline, configs 0, 3, 2", file=sys.stderr, flush=True)
+    gate_dt, (gK, gN) = shapes[4]
+    config0_s = gemv_seconds(gate_dt, gK, gN, 1)
+    # config 3: a 1/16 slice of the head's columns at 2 rows, then selection, law and acceptance on whole rows
+    slice_n = T.vocab // 16
+    head_s = gemv_seconds(T.embed_dtype, T.hidden, slice_n, 2) * (T.vocab / slice_n)
+    rng = np.random.default_rng(3)
+    p_logits = rng.normal(0, 2, (2, T.vocab)).astype(np.float32)
+    q_logits = rng.normal(0, 2, T.vocab).astype(np.float32)
+    opt = gfo.SamplerOptions(1.0, 64, 0.95, 0.0, 1.0)
     t0 = time.perf_counter()
-    gfo.gemv(dt, w, x, 64, threads=cores, which=ref)
-    per_weight = (time.perf_counter() - t0) / (K * 64)
-    layer_weights = sum(K * N for _, (K, N) in shapes)
-    frac = min(1.0, budget_s / (per_weight * layer_weights * 1.3))
-    done_weights, elapsed = 0, 0.0
-    # whole blocks' worth of GEMVs (fresh weights each time) until about half the budget is spent
-    repeats = max(1, int(0.6 * budget_s / max(per_weight * layer_weights * frac, 1e-9)))
-    for rep in range(repeats):
-        for i, (dt, (K, N)) in enumerate(shapes):
-            n = max(64, int(N * frac) // 64 * 64)
-            w = synth.make_weight(dt, K, n, 10 + i + 100 * rep)
-            x = synth.make_activation(2, K, 20 + i + 100 * rep)
-            t0 = time.perf_counter()
-            gfo.gemv(dt, w, x, n, threads=cores, which=ref)
-            elapsed += time.perf_counter() - t0
-            done_weights += K * n
-    step_weights = (T.layers * layer_weights + T.hidden * T.vocab
-                    + 0.5 * (D.layers * sum(K * N for K, N in D.proj_shapes()) + D.hidden * D.vocab))  # drafter: 1 row
-    value_us = elapsed / done_weights * step_weights * 1e6
+    r0, r1 = gfo.select_candidates(p_logits[0], 64), gfo.select_candidates(p_logits[1], 64)
+    rc, law = gfo.draft_law_compact(q_logits, opt)
+    word, ua, ur, un = gfo.step_draws(0, 0)
+    proposal = gfo.lib().gfo_draft_select(C.byref(law), C.c_uint32(word))
+    gfo.spec_accept(r0, r1, law, proposal, opt, ua, ur, un)
+    sampling_s = time.perf_counter() - t0
+    # config 2: one drafter block in full at 1 row, its head on a 1/16 slice, scaled by weight count
+    d_shapes = list(zip(D.dtypes, D.proj_shapes()))
+    d_block_s = sum(gemv_seconds(dt, K, N, 1) for dt, (K, N) in d_shapes)
+    d_head_s = gemv_seconds(D.embed_dtype, D.hidden, D.vocab // 16, 1) * 16
+    drafter_s = D.layers * d_block_s + d_head_s
+    step_s = T.layers * block_s + head_s + sampling_s + drafter_s
+    spent = repeats * block_s + config0_s + head_s / 16 + sampling_s + d_block_s + d_head_s / 16
+
     # the same rows spread over the host's cores (rows of W are independent; a row's arithmetic is
     # unchanged): the oracle's threaded row dot on one block's GEMVs
     many = min(os.cpu_count() or 1, 16)
-    par_weights, par_elapsed = 0, 0.0
-    for i, (dt, (K, N)) in enumerate(shapes):
-        n = max(64, int(N * min(1.0, 4.0 * frac)) // 64 * 64)
-        w = synth.make_weight(dt, K, n, 900 + i)
-        x = synth.make_activation(2, K, 920 + i)
-        t0 = time.perf_counter()
-        gfo.gemv(dt, w, x, n, threads=many)
-        par_elapsed += time.perf_counter() - t0
-        par_weights += K * n
+    par_s = sum(gemv_seconds(dt, K, N, 2, threads=many, which=None) for dt, (K, N) in shapes)
+    layer_weights = sum(K * N for _, (K, N) in shapes)
+    step_weights = (T.layers * layer_weights + T.hidden * T.vocab
+                    + 0.5 * (D.layers * sum(K * N for K, N in D.proj_shapes()) + D.hidden * D.vocab))  # drafter: 1 row
     return {
-        "value": round(value_us, 1), "unit": "us", "cores": cores, "kind": kind,
-        "all_cores": {"value": round(par_elapsed / par_weights * step_weights * 1e6, 1), "unit": "us", "cores": many,
-                      "kind": "port", "sample": "one 12B block's 7 GEMVs at 2 rows (%.2f s), oracle row dots on %d threads"
-                                                % (par_elapsed, many)},
-        "sample": "%d x one 12B block's 7 GEMVs at 2 rows, first %.1f%% of each matrix's columns (%.2f s of CPU work), "
-                  "scaled to the step's weight count; %s" % (
-                      repeats, 100 * frac, elapsed,
-                      "reference dot_q4_k_row_f32 / dot_q6_k_row_f32 (src/tensor/quantization.cpp), single thread"
-                      if ref is not None else "oracle gfo_gemv_mt on all host threads"),
+        "value": round(step_s * 1e6, 1), "unit": "us", "cores": cores, "kind": kind,
+        "sample": "%.1f s of CPU work: one 12B block's 7 GEMVs at 2 rows in full (x%d), the gate GEMV at 1 row, 1/16 of the "
+                  "head's columns at 2 rows, selection + law + acceptance on whole rows, one drafter block and 1/16 of its head "
+                  "at 1 row; step = 48 blocks + head + sampling + 18 drafter blocks + drafter head; %s" % (spent, repeats, how),
+        "all_cores": {"value": round(par_s / layer_weights * step_weights * 1e6, 1), "unit": "us", "cores": many,
+                      "kind": "port", "sample": "one 12B block's 7 GEMVs at 2 rows (%.2f s), oracle row dots on %d threads, "
+                                                "scaled to the step's weight count" % (par_s, many)},
+        "configs": {
+            "0": figure(config0_s, "the whole 3840 -> 15360 Q4_K GEMV at 1 row; " + how),
+            "1": figure(block_s, "the block's 7 GEMVs at 2 rows in full, mean of %d; %s" % (repeats, how)),
+            "2": figure(drafter_s, "one drafter block's 7 Q8_0 GEMVs at 1 row in full x 18, plus 1/16 of the head's columns x 16 "
+                                   "(by weight count; no attention or argmax); reference Q8_0 block decode, single thread"
+                        if ref is not None else "by weight count; " + how),
+            "3": figure(head_s + sampling_s, "1/16 of the Q6_K head's columns at 2 rows x 16 (%.2f s scaled), plus the oracle's "
+                                             "top-64 selection of 2 rows, compact law and acceptance on whole rows (%.3f s); %s"
+                        % (head_s, sampling_s, how)),
+        },
     }
 
 
@@ -237,11 +337,12 @@ def prefill_figure(target, T, tokens=2048):
     torch.cuda.synchronize()
     ms = (time.perf_counter() - t0) * 1e3
     macs = tokens * T.layers * sum(K * N for K, N in T.proj_shapes())
-    # every MAC is issued twice (fp16 hi and lo halves of the activation) on the f16 matrix pipe
-    issued_flops = 2 * 2 * macs
+    # mfma_frac counts the algorithmic flops (2 per weight and token); every MAC is issued twice on the f16 matrix
+    # pipe (fp16 hi and lo halves of the activation), which mfma_frac_issued counts
     return {"tokens": tokens, "ms": round(ms, 2), "tokens_per_s": round(tokens / ms * 1e3, 1),
             "model_tflops": round(2 * macs / ms / 1e9, 1), "bound": "mfma",
-            "mfma_frac": round(issued_flops / (ms * 1e-3) / 2.5e15, 4), "peak": "2.5 PFLOP/s f16 dense",
+            "mfma_frac": round(2 * macs / (ms * 1e-3) / 2.5e15, 4),
+            "mfma_frac_issued": round(2 * 2 * macs / (ms * 1e-3) / 2.5e15, 4), "peak": "2.5 PFLOP/s f16 dense",
             "status": int(status.item())}
 
 
@@ -295,54 +396,75 @@ def main():
     if (replayed["accepted"], replayed["token"], replayed["next_root"]) != (first["accepted"], first["token"], first["next_root"]):
         raise RuntimeError("graph replay changed the step's decision")
 
-    # ---- roofline of the dominant kernel: fused 2-row Q4_K gate+up GEMV + GeGLU, one launch per block -----
+    # ---- rooflines: the dominant kernel (fused 2-row Q4_K gate+up GEMV + GeGLU, one launch per block), then the
+    # local layers' attention and the down projection -----
     import ctypes as C
-    H, F = T.hidden, T.ffn
+    from guffin_amd import synth
+    H, F, QW, KW = T.hidden, T.ffn, T.q_width, T.kv_width
     x = torch.randn(2, H, device="cuda")
     xs = hip.group_sums(x)
     h_out = torch.empty(2, F, device="cuda")
     h_sums = hip._receipt(2, F, "cuda")
     lib = hip.lib()
+    every = list(range(T.layers))
 
-    def launch_all():
-        for l in range(T.layers):
-            L = target.layers[l]
-            # (ctypes passes a bare Python int as a 32-bit C int: pointers must be wrapped)
-            hip.check(lib.guffin_hip_gateup_geglu(hip._stream(), int(L.dtype[4]), C.c_void_p(L.tiles[4]), C.c_void_p(L.tiles[5]),
-                                                  hip._p(x), hip._p(xs), hip._p(h_out), hip._p(h_sums), 2, H, F))
-
-    launch_all()
-    torch.cuda.synchronize()
-    kgraph = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(kgraph):
-        launch_all()
-    for _ in range(3):
-        kgraph.replay()
-    stream = torch.cuda.current_stream()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    reps = 10
-    e0.record(stream)
-    for _ in range(reps):
-        kgraph.replay()
-    e1.record(stream)
-    torch.cuda.synchronize()
-    launch_us = e0.elapsed_time(e1) * 1e3 / (reps * T.layers)
-    # the same kernel dispatched alone (one launch, then a wait): the reference's benchmark reports both an
-    # isolated and a sustained mode (include/local_gguf_engine/benchmarks/quick_benchmark.hpp:13-17)
-    isolated = []
-    for rep in range(3 * T.layers):
-        L = target.layers[rep % T.layers]
-        e0.record(stream)
+    def gateup(l):
+        L = target.layers[l]
+        # (ctypes passes a bare Python int as a 32-bit C int: pointers must be wrapped)
         hip.check(lib.guffin_hip_gateup_geglu(hip._stream(), int(L.dtype[4]), C.c_void_p(L.tiles[4]), C.c_void_p(L.tiles[5]),
                                               hip._p(x), hip._p(xs), hip._p(h_out), hip._p(h_sums), 2, H, F))
-        e1.record(stream)
-        torch.cuda.synchronize()
-        isolated.append(e0.elapsed_time(e1) * 1e3)
-    isolated_us = sorted(isolated)[len(isolated) // 2]
-    from guffin_amd import synth
+
+    print("bench: timing the gate+up kernel", file=sys.stderr, flush=True)
     # weights once, activation rows in (fp32 rows are the operator's input; the kernel reads their receipt), h out
-    kernel_bytes = 2 * synth.weight_bytes(T.dtypes[4], H, F) + 2 * H * 4 + 2 * F * 4
-    achieved = kernel_bytes / launch_us / 1e3  # GB/s
+    gateup_bytes = 2 * synth.weight_bytes(T.dtypes[4], H, F) + 2 * H * 4 + 2 * F * 4
+    roofline = kernel_roofline("gateup_geglu_kernel<Q4_K, 2> (Q4_K gate+up GEMV + GeGLU, 2 rows, K=3840, N=2x15360)",
+                               gateup, every, gateup_bytes, "gateup_geglu_kernel<Q4_K, 2>")
+
+    print("bench: timing the down kernel", file=sys.stderr, flush=True)
+    xh = torch.randn(2, F, device="cuda")
+    xhs = hip.group_sums(xh)
+    down_dt = int(T.dtypes[6])
+    down_slices = hip.gemv_packed_slices(down_dt, F, H)
+    down_parts = torch.empty((down_slices, 2, H), device="cuda")
+
+    def down(l):
+        hip.check(lib.guffin_hip_gemv_packed(hip._stream(), down_dt, C.c_void_p(target.layers[l].tiles[6]), hip._p(xh), hip._p(xhs),
+                                             hip._p(down_parts), None, 2, F, H))
+
+    down_bytes = synth.weight_bytes(down_dt, F, H) + 2 * F * 4 + down_slices * 2 * H * 4
+    down_line = kernel_roofline("gemv_q6k_single_kernel<2> (Q6_K down GEMV, 2 rows, K=15360, N=3840, %d partial planes out)"
+                                % down_slices, down, [l for l in every if int(target.layers[l].dtype[6]) == down_dt],
+                                down_bytes, "gemv_q6k_single_kernel<2>")
+
+    print("bench: timing the local layers' attention", file=sys.stderr, flush=True)
+    # as the step runs it on a local layer: head norms, rotation, fp16 narrowing and attention of 2 rows over the
+    # 1024-token window in one launch, then the partition merge (its time is part of the figure, its bytes are not)
+    locals_ = [l for l in every if T.is_local(l)]
+    planes = 2
+    q_raw, k_raw, v_raw = (0.1 * torch.randn(planes, 2, w, device="cuda") for w in (QW, KW, KW))
+    q_norm, k_norm = torch.ones(T.head_dim, device="cuda"), torch.ones(T.head_dim, device="cuda")
+    positions = torch.tensor([t_pos, t_pos + 1], dtype=torch.int32, device="cuda")
+    table = hip.rope_table(positions, T.head_dim, T.local_base, 1.0)
+    sched_rows = []
+    for row in range(2):   # row r sees the last `window` positions up to its own: ring slots, then private rows
+        pos = t_pos + row
+        start = max(pos + 1 - T.sliding_window, 0)
+        base_start = min(t_pos, start)
+        first_private = max(start - t_pos, 0)
+        sched_rows.append([base_start, t_pos - base_start, first_private, row + 1 - first_private])
+    schedule = torch.tensor(sched_rows, dtype=torch.int32, device="cuda")
+    ancestors = torch.arange(2, dtype=torch.int32, device="cuda")
+    ring_tokens = max(r[0] + r[1] for r in sched_rows) - min(r[0] for r in sched_rows)
+
+    def local_attention(l):
+        hip.qkv_attention(q_raw, k_raw, v_raw, q_norm, k_norm, table, target.ring_k[l], target.ring_v[l], schedule, ancestors,
+                          ring_tokens + 2, T.ring_local - 1, T.q_heads, T.kv_heads, T.head_dim, T.head_dim ** -0.5)
+
+    # K and V rows of the window once per KV head, the projections' planes in, the attention rows out
+    attention_bytes = ring_tokens * KW * 2 * 2 + planes * 2 * (QW + 2 * KW) * 4 + 2 * QW * 4
+    attention_line = kernel_roofline("qkv attention of a local layer (2 rows, 16 query / 8 KV heads, %d-token window, fp16 K/V) "
+                                     "with its partition merge" % ring_tokens, local_attention, locals_, attention_bytes,
+                                     "attn_partial_kernel<2, 2, 256> (local layer")
 
     # a plain 256 MiB device copy: the reference reading for FETCH_SIZE / WRITE_SIZE counter runs
     cal_src = torch.empty(64 << 20, dtype=torch.float32, device="cuda").fill_(1.0)
@@ -365,22 +487,16 @@ def main():
             "step_hbm_frac": round(total_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
             "accepted": int(first["accepted"]),
         },
-        "roofline": {
-            "kernel": "gateup_geglu_kernel<Q4_K, 2> (Q4_K gate+up GEMV + GeGLU, 2 rows, K=3840, N=2x15360)",
-            "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": round(achieved / HBM_PEAK_GBS, 4),
-            # HBM bytes per launch from the FETCH_SIZE / WRITE_SIZE counter runs recorded in
-            # profiles/gateup_geglu_q4k_hbm_traffic.txt (copy-calibrated: fetch x 1.9997, write x 1)
-            "traffic": 67046400,
-            "bytes_per_launch": kernel_bytes, "launch_us": round(launch_us, 3),
-            "sustained_dispatches": T.layers, "isolated_launch_us": round(isolated_us, 3),
-        },
+        "roofline": roofline,
+        "rooflines": [attention_line, down_line],
     }
     line["configs"] = config_figures(target, drafter, T, D, d_pos)
     if not args.no_prefill:
         line["prefill"] = prefill_figure(target, T)
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(T, D)
+        for key, figure in line["cpu_baseline"].pop("configs").items():
+            line["configs"][key]["cpu_baseline"] = figure
     print(json.dumps(line))
 
 
