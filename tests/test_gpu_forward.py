@@ -66,6 +66,31 @@ def test_forward_rows_matches_oracle(hip, gfo, kind, rows, position):
     assert np.allclose(sums.cpu().numpy(), ref_sums, rtol=0, atol=1e-4 * np.abs(h).max() * 4)
 
 
+def test_drafter_greedy_token_at_full_size_equals_the_oracles_argmax(hip, gfo):
+    """The drafter's decode as the benchmark times it (18 blocks, a 4096-token cache, the 262144 x 640 Q8_0
+    head, argmax): the greedy token from the device's logits is the argmax of the ORACLE's logits, and the
+    oracle's best two logits are further apart than the two sides' logits differ."""
+    import torch
+    from guffin_amd import model
+    shape, position = model.GEMMA3_270M, 4096
+    host = model.HostModel(shape, seed=21, position=position, untied_head=True)   # a tied random head would elect the input token
+    devm = model.DeviceModel.from_host(host)
+    token = np.array([4242], np.uint32)
+    want_hidden, _, _ = gfo.forward(host, token, position, threads=8)
+    want = gfo.gemv(shape.embed_dtype, host.head, want_hidden, shape.vocab, threads=8)[0]
+    hidden, sums, _, _, status = devm.forward(dev(token), position)
+    logits = hip.gemv_packed(int(shape.embed_dtype), devm.head_tiles, hidden, sums, shape.vocab)
+    got_token, got_logit = hip.argmax(logits)
+    assert int(status.item()) == 0
+    best, second = np.argsort(-want, kind="stable")[:2]
+    margin = float(want[best] - want[second])
+    differ = float(np.max(np.abs(logits.cpu().numpy()[0] - want)))
+    print("drafter argmax %d, top-2 margin %.4g (logit std %.3g), device and oracle logits differ by at most %.3g"
+          % (best, margin, float(want.std()), differ))
+    assert margin > 4 * differ          # the election does not rest on the sides' rounding
+    assert int(got_token[0]) == int(best) == int(np.argmax(want))
+
+
 def run_h1(hip, gfo, t_shape, d_shape, t_pos, d_pos, steps, seed, threads=8):
     """`steps` cycles from one root with the benchmark's sampler options.  The two random models are
     unrelated, so the drafter reaches the target through a vocabulary map that lines its 64 best tokens

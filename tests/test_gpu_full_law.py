@@ -148,3 +148,37 @@ def test_accept_gathers_from_the_full_table(hip, gfo):
         assert (got["accepted"], got["token"], got["next_root"]) == (want.accepted, want.token, want.next_root), step
         accepted += want.accepted
     assert 0 < accepted < 200
+
+
+def test_device_laws_against_the_double_restatement(hip):
+    """Both law paths on the device against the rule restated in double precision (tests/law_brute.py), not
+    against the oracle: same supports, masses within 1e-6, on cases whose membership decisions are not
+    within 1e-5 of their edge."""
+    from law_brute import law, random_case
+    rng = np.random.default_rng(909)
+    compact = full = 0
+    while compact < 8 or full < 8:
+        logits, T, k, p, m = random_case(rng, 32768)
+        wide = bool(rng.integers(0, 2))
+        if wide:
+            k = int(rng.choice([100, 256]))
+        want, margin = law(logits, T, k, p, m)
+        if margin < 1e-5:
+            continue
+        head, cdf, proposal, status = full_law(hip, logits, opts(hip, T, k, p, m), int(rng.integers(0, 2 ** 32)))
+        assert status == 0
+        if head["count"] == 0xFFFFFFFF:
+            bins = np.diff(cdf.astype(np.int64))
+            got = {int(t): bins[t] / TOTAL for t in np.nonzero(bins)[0]}
+            tiny, full = 1e-6, full + 1
+        else:
+            n = int(head["count"])
+            got = {int(head["ids"][i]): (int(head["cdf"][i + 1]) - int(head["cdf"][i])) / TOTAL for i in range(n)}
+            got = {t: v for t, v in got.items() if v > 0}
+            tiny, compact = 2.0 ** -31, compact + 1
+        assert proposal in got
+        for token, mass in want.items():
+            if mass > tiny:
+                assert token in got, (T, k, p, m, token, mass)
+        for token, mass in got.items():
+            assert token in want and abs(mass - want[token]) <= 1e-6, (T, k, p, m, token, mass)

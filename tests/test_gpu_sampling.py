@@ -135,8 +135,32 @@ def test_draft_law_reference_fixtures(hip, gfo):
     assert int(status[0]) & 16
 
 
-def run_steps(hip, gfo, p_logits, q_logits, steps, seed, o_gpu, o_cpu):
-    """steps of draft-law + accept on the GPU against the oracle; returns (accepted, rejected)."""
+def cdf_margin(weights, draw):
+    """Relative distance of `draw` (in [0, total)) from the nearest bin edge of the running sum of `weights`:
+    how far a draw is from selecting a neighbouring token."""
+    edges = np.cumsum(np.asarray(weights, np.float64))
+    return float(np.min(np.abs(edges[:-1] - draw)) / edges[-1]) if edges.size > 1 else 1.0
+
+
+def decision_margins(gfo, prepared, law, want, ua, ur, un):
+    """(margin of the accept decision, margin of the token draw that follows it) for one step."""
+    total = float(1 << 32)
+    if want.accepted:
+        nxt = prepared[1]
+        weights = [nxt.sampling_weight[i] for i in range(nxt.count)]
+        return abs(ua - want.acceptance_probability), cdf_margin(weights, un * nxt.total_sampling_weight)
+    tgt = prepared[0]
+    mass = {law.ids[i]: (law.cdf[i + 1] - law.cdf[i]) / total for i in range(law.count)}
+    norm = sum(tgt.sampling_weight[i] for i in range(tgt.count))
+    residual = [tgt.sampling_weight[i] / norm - mass.get(tgt.token[i], 0.0) for i in range(tgt.count)]
+    residual = [d for d in residual if d > 0.0]
+    assert len(residual) == want.residual_count
+    return abs(ua - want.acceptance_probability), cdf_margin(residual, ur * sum(residual))
+
+
+def run_steps(hip, gfo, p_logits, q_logits, steps, seed, o_gpu, o_cpu, margins=None):
+    """steps of draft-law + accept on the GPU against the oracle; returns (accepted, rejected).  With a
+    `margins` list, the smallest accept and draw margins of the run are appended to it."""
     import torch
     sets = p_logits.shape[0]
     cands, laws_cpu, cands_cpu = [], [], []
@@ -152,6 +176,8 @@ def run_steps(hip, gfo, p_logits, q_logits, steps, seed, o_gpu, o_cpu):
             want = gfo.select_candidates(p_logits[s, row], o_gpu.top_k)
             assert np.array_equal(c[row]["values"]["token"][:want.size], want["token"])
         cands_cpu.append([gfo.select_candidates(p_logits[s, r], o_gpu.top_k) for r in range(2)])
+    prepared = [[gfo.prepare(cands_cpu[s][r], o_cpu)[1] for r in range(2)] for s in range(sets)]
+    least_accept = least_draw = 1.0
     q_dev = [dev(q_logits[s]) for s in range(sets)]
     results = torch.zeros(steps * hip.result_dtype.itemsize, dtype=torch.uint8, device="cuda")
     law = torch.zeros(hip.law_dtype.itemsize, dtype=torch.uint8, device="cuda")
@@ -183,6 +209,11 @@ def run_steps(hip, gfo, p_logits, q_logits, steps, seed, o_gpu, o_cpu):
         assert abs(got[step]["acceptance_probability"] - want.acceptance_probability) <= 1e-14
         accepted += want.accepted
         rejected += 1 - want.accepted
+        if margins is not None:
+            m_accept, m_draw = decision_margins(gfo, prepared[s], laws_cpu[s], want, ua, ur, un)
+            least_accept, least_draw = min(least_accept, m_accept), min(least_draw, m_draw)
+    if margins is not None:
+        margins += [least_accept, least_draw]
     return accepted, rejected
 
 
@@ -192,8 +223,14 @@ def test_ten_thousand_seeded_steps_bit_exact(hip, gfo):
     sets = 8
     p_logits = rng.normal(0, 3, (sets, 2, VOCAB)).astype(np.float32)
     q_logits = rng.normal(0, 2, (sets, VOCAB)).astype(np.float32)
-    a, r = run_steps(hip, gfo, p_logits, q_logits, 10000, 0, opts(hip), opts(gfo))
+    margins = []
+    a, r = run_steps(hip, gfo, p_logits, q_logits, 10000, 0, opts(hip), opts(gfo), margins)
     assert a + r == 10000
+    # "bit-exact decisions" must not rest on a near-tie: the device and the oracle agree on the laws' doubles
+    # to about 1e-15, and no draw of this run comes within 1e-9 of the edge it is compared with
+    print("10000 steps: %d accepted, %d rejected; least |u_accept - a| = %.3e, least draw-to-edge distance = %.3e"
+          % (a, r, margins[0], margins[1]))
+    assert margins[0] > 1e-9 and margins[1] > 1e-9, margins
 
 
 def test_correlated_drafter_mixes_accepts_and_rejections(hip, gfo):
@@ -201,8 +238,14 @@ def test_correlated_drafter_mixes_accepts_and_rejections(hip, gfo):
     sets = 8
     p_logits = rng.normal(0, 3, (sets, 2, VOCAB)).astype(np.float32)
     q_logits = (p_logits[:, 0] + rng.normal(0, 1.0, (sets, VOCAB))).astype(np.float32)
-    a, r = run_steps(hip, gfo, p_logits, q_logits, 3000, 17, opts(hip), opts(gfo))
+    margins = []
+    a, r = run_steps(hip, gfo, p_logits, q_logits, 3000, 17, opts(hip), opts(gfo), margins)
     assert a > 300 and r > 300, (a, r)
+    # here the acceptance probability is strictly between 0 and 1 on most steps: the accept decisions,
+    # the residual draws and the next-root draws all stay clear of their edges
+    print("3000 correlated steps: %d accepted, %d rejected; least |u_accept - a| = %.3e, least draw-to-edge distance = %.3e"
+          % (a, r, margins[0], margins[1]))
+    assert margins[0] > 1e-9 and margins[1] > 1e-9, margins
     a2, r2 = run_steps(hip, gfo, p_logits, q_logits, 500, 18, opts(hip, 0.8, 40, 0.9, 0.05), opts(gfo, 0.8, 40, 0.9, 0.05))
     assert a2 + r2 == 500
 
