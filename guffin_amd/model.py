@@ -576,3 +576,81 @@ class Session:
 
     def read_result(self):
         return self.result.cpu().numpy().view(hip.result_dtype)[0]
+
+
+class DraftPlanDesc(C.Structure):
+    _fields_ = [("model", C.c_void_p), ("workspace", C.c_void_p), ("workspace_bytes", C.c_uint64)] + \
+               [(n, C.c_uint32) for n in
+                ("position", "materialized", "pending_token", "has_pending", "transaction_active", "poisoned",
+                 "checkpoint_position", "checkpoint_materialized", "checkpoint_pending", "checkpoint_has_pending",
+                 "backup_end", "last_rows", "logits_valid", "hidden_valid", "checkpoint_hidden_valid",
+                 "checkpoint_last_rows")]
+
+
+class DraftPlan:
+    """The drafter between cycles, with the method names of the reference's Gemma3DraftPlan
+    (include/local_gguf_engine/engine/gemma3_draft.hpp:56-82) over guffin_hip_draft_plan_*.  State errors
+    raise hip.GuffinError with the C code (GUFFIN_E_STATE = -6, capacity -4, argument -1)."""
+
+    def __init__(self, drafter):
+        self.drafter = drafter
+        lib = hip.lib()
+        lib.guffin_hip_draft_plan_bytes.restype = C.c_uint64
+        need = lib.guffin_hip_draft_plan_bytes(C.byref(drafter.desc))
+        if need == 0:
+            raise ValueError("the model cannot carry a draft plan (head tiles and rings are required)")
+        self.workspace = torch.zeros(int(need), dtype=torch.uint8, device="cuda")
+        self.desc = DraftPlanDesc()
+        hip.check(lib.guffin_hip_draft_plan_init(hip._stream(), C.byref(self.desc), C.byref(drafter.desc),
+                                                 hip._p(self.workspace), C.c_uint64(need)))
+
+    position = property(lambda self: self.desc.position)
+    materialized_position = property(lambda self: self.desc.materialized)
+    transaction_active = property(lambda self: bool(self.desc.transaction_active))
+    poisoned = property(lambda self: bool(self.desc.poisoned))
+
+    def reset(self):
+        hip.check(hip.lib().guffin_hip_draft_plan_reset(hip._stream(), C.byref(self.desc)))
+
+    def begin_transaction(self):
+        hip.check(hip.lib().guffin_hip_draft_plan_begin_transaction(hip._stream(), C.byref(self.desc)))
+
+    def commit_prefix(self, position):
+        hip.check(hip.lib().guffin_hip_draft_plan_commit_prefix(hip._stream(), C.byref(self.desc), position))
+
+    def abort_transaction(self):
+        hip.check(hip.lib().guffin_hip_draft_plan_abort_transaction(hip._stream(), C.byref(self.desc)))
+
+    def can_truncate(self, position):
+        return bool(hip.lib().guffin_hip_draft_plan_can_truncate(C.byref(self.desc), position))
+
+    def truncate(self, position):
+        hip.check(hip.lib().guffin_hip_draft_plan_truncate(hip._stream(), C.byref(self.desc), position))
+
+    def append(self, tokens):
+        arr = (C.c_uint32 * len(tokens))(*[int(t) for t in tokens])
+        hip.check(hip.lib().guffin_hip_draft_plan_append(hip._stream(), C.byref(self.desc), arr, len(tokens)))
+
+    def restore_pending_token(self, token):
+        hip.check(hip.lib().guffin_hip_draft_plan_restore_pending_token(C.byref(self.desc), int(token)))
+
+    def propose(self, words, options, history=()):
+        h = len(words)
+        w = (C.c_uint32 * h)(*[int(x) for x in words])
+        hist = (C.c_uint32 * max(1, len(history)))(*[int(x) for x in history])
+        out = (C.c_uint32 * h)()
+        hip.check(hip.lib().guffin_hip_draft_plan_propose(hip._stream(), C.byref(self.desc), w, h, C.byref(options),
+                                                          hist if len(history) else None, len(history), out))
+        return list(out)
+
+    def read_logits(self):
+        out = np.empty(self.drafter.shape.vocab, np.float32)
+        hip.check(hip.lib().guffin_hip_draft_plan_read_logits(hip._stream(), C.byref(self.desc), out.ctypes.data_as(C.c_void_p)))
+        return out
+
+    def read_cache(self, layer, first_position, count):
+        width = self.drafter.shape.kv_width
+        k, v = np.empty((count, width), np.uint16), np.empty((count, width), np.uint16)
+        hip.check(hip.lib().guffin_hip_draft_plan_read_cache(hip._stream(), C.byref(self.desc), layer, first_position, count,
+                                                             k.ctypes.data_as(C.c_void_p), v.ctypes.data_as(C.c_void_p)))
+        return k, v

@@ -529,6 +529,49 @@ int guffin_hip_h1_buffers(const guffin_h1_desc* desc, void* scratch, float** dra
 /* The full-vocabulary table of the last step (desc->full_law != 0), else NULL. */
 int guffin_hip_h1_full_cdf(const guffin_h1_desc* desc, void* scratch, uint64_t** full_cdf);
 
+/* ---- drafter lifecycle --------------------------------------------------------------------
+ * The state machine of Gemma3DraftPlan (include/local_gguf_engine/engine/gemma3_draft.hpp:56-82;
+ * lifecycle cases tests/engine/gemma3_draft_tests.cpp:206-277) over guffin_hip_forward_rows and the model's
+ * rings: a prefix of `position` tokens of which `materialized` have K/V rows (a pending token, the drafter's
+ * last emission or one restored by the caller, is run only when the next input needs it), and transactions
+ * whose rows can be taken back.  Each call below names the method it replaces.  A transaction's rows go to
+ * the rings at once; the ring rows they overwrite are saved per position (at most 32 positions per
+ * transaction; the reference's arena holds 96 or 256) and copied back by abort, truncate and a commit of a
+ * shorter prefix.  Tokens run through the decode path one row per pass, so a token's rows and logits do not
+ * depend on how appends were grouped and a commit equals a replay bit for bit.  Every call returns when its device work is done; errors: GUFFIN_E_STATE for a call
+ * the state does not admit (nested transaction, truncation of published rows, a second pending token, a
+ * poisoned plan), GUFFIN_E_CAPACITY / GUFFIN_E_ARG raised before any state changes, GUFFIN_E_NUMERIC when a pass
+ * raises the device status (the plan is then poisoned until reset).  The struct is caller-owned; the fields
+ * after `workspace_bytes` belong to the library. */
+typedef struct guffin_draft_plan {
+    const guffin_model_desc* model;   /* the drafter, with head_tiles and every layer's rings */
+    void* workspace; uint64_t workspace_bytes;   /* device, guffin_hip_draft_plan_bytes(model), 256-byte aligned */
+    uint32_t position, materialized, pending_token, has_pending, transaction_active, poisoned;
+    uint32_t checkpoint_position, checkpoint_materialized, checkpoint_pending, checkpoint_has_pending;
+    uint32_t backup_end, last_rows, logits_valid, hidden_valid, checkpoint_hidden_valid, checkpoint_last_rows;
+} guffin_draft_plan;
+uint64_t guffin_hip_draft_plan_bytes(const guffin_model_desc* model);
+int guffin_hip_draft_plan_init(void* stream, guffin_draft_plan* plan, const guffin_model_desc* model, void* workspace,
+                               uint64_t workspace_bytes);
+int guffin_hip_draft_plan_reset(void* stream, guffin_draft_plan* plan);                        /* reset() */
+int guffin_hip_draft_plan_begin_transaction(void* stream, guffin_draft_plan* plan);                        /* begin_transaction() */
+int guffin_hip_draft_plan_commit_prefix(void* stream, guffin_draft_plan* plan, uint32_t position);   /* commit_prefix() */
+int guffin_hip_draft_plan_abort_transaction(void* stream, guffin_draft_plan* plan);            /* abort_transaction() */
+int guffin_hip_draft_plan_can_truncate(const guffin_draft_plan* plan, uint32_t position);      /* can_truncate(): 1 or 0 */
+int guffin_hip_draft_plan_truncate(void* stream, guffin_draft_plan* plan, uint32_t position);  /* truncate() */
+int guffin_hip_draft_plan_append(void* stream, guffin_draft_plan* plan, const uint32_t* tokens_host, uint32_t count);  /* append() */
+int guffin_hip_draft_plan_restore_pending_token(guffin_draft_plan* plan, uint32_t token);     /* restore_pending_token() */
+/* propose(): `horizon` (1..23) tokens from the given 32-bit words inside the open transaction; all but the last
+ * are run, the last stays pending.  options: the sampler options struct; history (host, <= 64 tokens, may be
+ * NULL) feeds the repetition penalty and grows by the drafted tokens.  drafted: host, `horizon` tokens. */
+int guffin_hip_draft_plan_propose(void* stream, guffin_draft_plan* plan, const uint32_t* words_host, uint32_t horizon,
+                                  const void* options, const uint32_t* history_host, uint32_t history_count,
+                                  uint32_t* drafted_host);
+int guffin_hip_draft_plan_read_logits(void* stream, guffin_draft_plan* plan, float* logits_host);   /* read_logits() */
+/* read_cache(): fp16 rows of `count` materialized positions of one layer, in position order. */
+int guffin_hip_draft_plan_read_cache(void* stream, const guffin_draft_plan* plan, uint32_t layer, uint32_t first_position,
+                                     uint32_t count, void* keys_host, void* values_host);
+
 /* ---- GGUF container reader (host only) ---------------------------------------------------
  * The validating reader of src/model_format/gguf_reader.cpp (types in
  * include/local_gguf_engine/model_format/gguf_{header,metadata,tensor,reader}.hpp): one pass over

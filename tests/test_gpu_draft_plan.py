@@ -1,0 +1,206 @@
+"""The drafter's lifecycle (guffin_hip_draft_plan_*) on the cases of the reference's transaction_lifecycle
+test (tests/engine/gemma3_draft_tests.cpp:206-277): aborted and truncated suffixes leave the caches as they
+were, a committed prefix followed by a different next root gives the logits and caches of a plain replay,
+bit for bit, and that replay agrees with the oracle run token by token over mirrored host caches."""
+from dataclasses import replace
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+PROMPT = 62            # two rows short of the local layers' 64-row ring, as the reference's 510 is of 512
+ROOT, NEXT_ROOT, CORRECTION = 55, 719, 111
+
+
+@pytest.fixture(scope="module")
+def hip():
+    from guffin_amd import hip as module
+    module.init(0)
+    return module
+
+
+@pytest.fixture(scope="module")
+def world(hip):
+    from guffin_amd import model
+    shape = replace(model.GEMMA3_270M, layers=3, global_period=3, vocab=4096, sliding_window=64, ring_local=64, ring_global=256)
+    host = model.HostModel(shape, seed=31, position=0, untied_head=True)
+    return shape, host, model.DeviceModel.from_host(host)
+
+
+def stream(n):
+    return [int((i * 37 + 11) % 4000) for i in range(n)]
+
+
+def greedy(hip):
+    return hip.SamplerOptions(0.0, 40, 0.95, 0.05, 1.0)
+
+
+def snapshot(plan, shape):
+    """Every materialized row each layer still holds, in position order."""
+    rows = []
+    for layer in range(shape.layers):
+        cap = shape.ring_local if shape.is_local(layer) else shape.ring_global
+        first = max(0, plan.materialized_position - cap)
+        rows.append((first,) + plan.read_cache(layer, first, plan.materialized_position - first))
+    return rows
+
+
+def same_caches(a, b):
+    return all(fa == fb and np.array_equal(ka, kb) and np.array_equal(va, vb) for (fa, ka, va), (fb, kb, vb) in zip(a, b))
+
+
+def refuses(hip, call, code):
+    with pytest.raises(hip.GuffinError) as info:
+        call()
+    assert info.value.code == code, info.value
+
+
+def oracle_replay(gfo, host, tokens):
+    """The oracle over host caches it fills itself, one token at a time: (logits after the last token, caches)."""
+    import copy
+    mirror = copy.copy(host)
+    mirror.ring_k = [np.zeros_like(r) for r in host.ring_k]
+    mirror.ring_v = [np.zeros_like(r) for r in host.ring_v]
+    hidden = None
+    for position, token in enumerate(tokens):
+        hidden, pk, pv = gfo.forward(mirror, np.array([token], np.uint32), position, threads=8)
+        mirror.commit(pk, pv, position, 1)
+    logits = gfo.gemv(host.shape.embed_dtype, host.head, hidden, host.shape.vocab, threads=8)[0]
+    return logits, mirror
+
+
+def test_transactions_leave_no_trace_and_commits_replay(hip, gfo, world):
+    from guffin_amd import model
+    shape, host, device = world
+    plan = model.DraftPlan(device)
+    prompt = stream(PROMPT)
+    plan.append(prompt)
+    before = snapshot(plan, shape)
+    words = [0] * 23
+
+    plan.begin_transaction()
+    plan.append([ROOT])
+    plan.propose(words[:3], greedy(hip))
+    plan.abort_transaction()
+    assert plan.position == PROMPT and same_caches(snapshot(plan, shape), before), "abort moved the prefix"
+
+    for accepted in range(4):
+        plan.begin_transaction()
+        plan.append([ROOT])
+        proposed = plan.propose(words[:3], greedy(hip))
+        assert plan.position == PROMPT + 4 and plan.materialized_position == PROMPT + 3, "the last draft is pending, not run"
+        plan.commit_prefix(PROMPT + 1 + accepted)
+        if accepted == 3:
+            pending_cache, old = snapshot(plan, shape), plan.materialized_position
+            plan.begin_transaction()
+            plan.append([NEXT_ROOT])
+            plan.propose(words[:1], greedy(hip))
+            plan.abort_transaction()
+            assert plan.position == PROMPT + 4 and plan.materialized_position == old
+            assert same_caches(snapshot(plan, shape), pending_cache), "abort lost the committed pending token"
+        plan.append([NEXT_ROOT])
+        actual, committed = plan.read_logits(), snapshot(plan, shape)
+        replay = prompt + [ROOT] + proposed[:accepted] + [NEXT_ROOT]
+        plan.reset()
+        plan.append(replay)
+        expected = plan.read_logits()
+        assert np.array_equal(actual.view(np.uint32), expected.view(np.uint32)), "commit + next root differs from a replay"
+        assert same_caches(snapshot(plan, shape), committed)
+        if accepted in (0, 3):     # the replay itself against the oracle over its own mirrored caches
+            want, mirror = oracle_replay(gfo, host, replay)
+            assert np.sqrt(np.mean((expected - want) ** 2)) <= 1e-3 * np.sqrt(np.mean(want ** 2))
+            assert int(np.argmax(expected)) == int(np.argmax(want))
+            for layer, (first, k, v) in enumerate(snapshot(plan, shape)):
+                cap = mirror.ring_k[layer].shape[0]
+                slots = (np.arange(first, len(replay)) & (cap - 1))
+                assert np.mean(k == mirror.ring_k[layer][slots].view(np.uint16)) >= 0.95
+                assert np.mean(v == mirror.ring_v[layer][slots].view(np.uint16)) >= 0.95
+        plan.reset()
+        plan.append(prompt)
+
+    # truncate an encoded speculative suffix before appending a correction
+    plan.begin_transaction()
+    plan.append([ROOT])
+    drafted = plan.propose(words[:3], greedy(hip))
+    plan.truncate(PROMPT + 2)
+    plan.append([CORRECTION])
+    plan.commit_prefix(PROMPT + 3)
+    assert not plan.can_truncate(PROMPT + 2)
+    refuses(hip, lambda: plan.truncate(PROMPT + 2), -6)
+    logits, corrected = plan.read_logits(), snapshot(plan, shape)
+    plan.reset()
+    plan.append(prompt + [ROOT, drafted[0], CORRECTION])
+    assert np.array_equal(logits.view(np.uint32), plan.read_logits().view(np.uint32)), "truncate + correction differs from a replay"
+    assert same_caches(snapshot(plan, shape), corrected)
+
+
+def test_horizons_capacity_and_pending_restoration(hip, world):
+    from guffin_amd import model
+    shape, host, device = world
+    plan = model.DraftPlan(device)
+    plan.append([ROOT])
+    for horizon in (1, 2, 3, 5, 23):
+        plan.begin_transaction()
+        drafted = plan.propose([7] * horizon, greedy(hip))
+        assert len(drafted) == horizon and plan.position == horizon + 1, "a requested horizon was narrowed"
+        plan.abort_transaction()
+        assert plan.position == 1
+    plan.begin_transaction()
+    refuses(hip, plan.begin_transaction, -6)                          # nested transaction
+    refuses(hip, lambda: plan.append(stream(33)), -4)                 # more rows than a transaction can take back
+    assert plan.position == 1, "a refused append changed the state"
+    plan.abort_transaction()
+    refuses(hip, lambda: plan.append(stream(shape.ring_global)), -4)  # context overflow
+    refuses(hip, lambda: plan.append([shape.vocab]), -1)              # token outside the vocabulary
+    refuses(hip, lambda: plan.propose([0], greedy(hip)), -6)          # proposals live inside a transaction
+    assert plan.position == 1 and not plan.poisoned
+
+    plan.reset()
+    plan.append([ROOT])
+    plan.restore_pending_token(CORRECTION)
+    assert plan.position == 2 and plan.materialized_position == 1, "a restored pending token was run eagerly"
+    refuses(hip, lambda: plan.restore_pending_token(CORRECTION), -6)
+    plan.begin_transaction()
+    refuses(hip, lambda: plan.restore_pending_token(ROOT), -6)
+    plan.append([NEXT_ROOT])
+    plan.abort_transaction()
+    assert plan.position == 2 and plan.materialized_position == 1, "abort changed the pending frontier"
+    plan.append([NEXT_ROOT])
+    logits = plan.read_logits()
+    plan.reset()
+    plan.append([ROOT, CORRECTION, NEXT_ROOT])
+    assert np.array_equal(logits.view(np.uint32), plan.read_logits().view(np.uint32)), "a restored pending token changed later logits"
+
+
+def test_sampled_proposals_follow_the_law_of_each_step(hip, gfo, world):
+    """With temperature and a repetition penalty, draft i is the oracle's selection from the law of the
+    logits the plan holds after draft i-1, with the history grown by the drafts so far."""
+    import ctypes as C
+    from guffin_amd import model
+    shape, host, device = world
+    plan = model.DraftPlan(device)
+    plan.append(stream(10))
+    history = [3, 4, 3]
+    rng = np.random.default_rng(4)
+    words = [int(w) for w in rng.integers(0, 2 ** 32, 4)]
+    options = hip.SamplerOptions(0.9, 40, 0.95, 0.02, 1.3)
+    plan.begin_transaction()
+    drafted = plan.propose(words, options, history)
+    plan.abort_transaction()
+    # replay the chain token by token through append / read_logits and build each law on the CPU
+    window = list(history)
+    for i, word in enumerate(words):
+        plan.begin_transaction()
+        if i:
+            plan.append(drafted[:i])
+        logits = plan.read_logits()
+        plan.abort_transaction()
+        scores = logits.copy()
+        hit = np.zeros(scores.size, bool)
+        hit[window] = True
+        scores[hit] = np.where(scores[hit] < 0, scores[hit] * np.float32(1.3), scores[hit] / np.float32(1.3))
+        rc, law = gfo.draft_law_compact(scores, gfo.SamplerOptions(0.9, 40, 0.95, 0.02, 1.0))
+        assert rc == 0
+        assert drafted[i] == gfo.lib().gfo_draft_select(C.byref(law), C.c_uint32(word))
+        window = (window + [drafted[i]])[-64:]
