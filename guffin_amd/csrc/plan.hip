@@ -17,6 +17,7 @@
 #include "receipt.hpp"
 
 #include <algorithm>
+#include <vector>
 #include <cmath>
 #include <cstring>
 
@@ -35,6 +36,9 @@ struct Arena {
         return p;
     }
 };
+
+// private rows a verify tree may hold (rows of one pass are at most 2; a tree takes several passes)
+constexpr uint32_t kMaxTreeSlots = 8;
 
 struct Scratch {
     float *x, *x1, *u, *us, *q, *a, *as, *h, *hs;
@@ -100,15 +104,20 @@ Scratch layout(const guffin_model_desc& m, uint32_t rows, uint32_t position, uin
     s.part_a = ar.take<float>(pa);
     s.part_b = ar.take<float>(pb);
     s.part_c = ar.take<float>(pc);
+    // partitions of the longest token list, and of any shorter one: the partition length shrinks with the list
+    // (down to 16 tokens, while fewer than 256 workgroups would run), so a shorter list can have more of them
     uint32_t max_parts = 1;
-    for (uint32_t l = 0; l < m.layer_count; ++l)
-        max_parts = std::max(max_parts, guffin_hip_attention_partitions(max_tokens_for(m, l, position, rows), m.kv_heads));
+    for (uint32_t l = 0; l < m.layer_count; ++l) {
+        const uint32_t longest = max_tokens_for(m, l, position, rows);
+        const uint32_t shorter = std::min((512u + m.kv_heads - 1) / m.kv_heads, (longest + 15) / 16);
+        max_parts = std::max({max_parts, guffin_hip_attention_partitions(longest, m.kv_heads), shorter});
+    }
     s.attn_out = ar.take<float>(uint64_t(rows) * m.q_heads * max_parts * m.head_dim);
     s.attn_ml = ar.take<float>(uint64_t(rows) * m.q_heads * max_parts * 2);
     s.rope_local = ar.take<float>(uint64_t(rows) * m.head_dim);
     s.rope_global = ar.take<float>(uint64_t(rows) * m.head_dim);
     s.positions = ar.take<uint32_t>(rows);
-    s.ancestors = ar.take<uint32_t>(rows);
+    s.ancestors = ar.take<uint32_t>(uint64_t(rows) * kMaxTreeSlots);   // a chain uses `rows` of them, a tree pass one list per row
     s.schedule = ar.take<uint32_t>(uint64_t(m.layer_count) * rows * 4);
     if (resident_fits(m, rows)) {
         s.exchange = ar.take<uint8_t>(resident_scratch_bytes(m, rows));
@@ -170,6 +179,37 @@ int check_ring_capacity(const guffin_model_desc& m, uint32_t position, uint32_t 
     return GUFFIN_OK;
 }
 
+// A block after its attention: o-projection, the two norm joints, gate/up with GeGLU, down.  s.a / s.as hold
+// the attention rows and their receipt, s.x the residual rows; leaves the next block's normalised rows in
+// s.u / s.us (the last block: the output-normed rows in out_hidden / out_hidden_sums).
+int block_tail(void* st, const guffin_model_desc& m, uint32_t l, const Scratch& s, uint32_t rows, float* out_hidden,
+               float* out_hidden_sums, uint32_t* status) {
+    const guffin_layer_desc& L = m.layers[l];
+    const uint32_t H = m.hidden, F = m.ffn, QW = m.q_heads * m.head_dim;
+    GUFFIN_TRY(guffin_hip_gemv_packed(st, L.dtype[3], L.tiles[3], s.a, s.as, s.part_a, nullptr, rows, QW, H));
+    // x1 = x + rms(o, post_attention_norm); u = rms(x1, ffn_norm)
+    GUFFIN_TRY(guffin_hip_rms_norm_add_norm(st, s.part_a, slices(L.dtype[3], QW, H), uint64_t(rows) * H, L.norm[3],
+                                            s.x, s.x1, L.norm[4], s.u, s.us, rows, H, m.eps, status));
+    if (L.dtype[4] == L.dtype[5] && L.dtype[4] != GUFFIN_Q6_K) {
+        GUFFIN_TRY(guffin_hip_gateup_geglu(st, L.dtype[4], L.tiles[4], L.tiles[5], s.u, s.us, s.h, s.hs, rows, H, F));
+    } else {
+        const int dt[2] = {L.dtype[4], L.dtype[5]};
+        const void* tl[2] = {L.tiles[4], L.tiles[5]};
+        const uint32_t n[2] = {F, F};
+        float* parts[2] = {s.part_a, s.part_b};
+        GUFFIN_TRY(guffin_hip_gemv_packed_multi(st, 2, dt, tl, n, parts, s.u, s.us, rows, H));
+        GUFFIN_TRY(guffin_hip_geglu(st, s.part_a, s.part_b, ffn_slices(L, H, F), uint64_t(rows) * F, s.h, s.hs, rows, F));
+    }
+    GUFFIN_TRY(guffin_hip_gemv_packed(st, L.dtype[6], L.tiles[6], s.h, s.hs, s.part_a, nullptr, rows, F, H));
+    // x = x1 + rms(down, post_ffw_norm); u = rms(x, next block's attn_norm | output_norm)
+    const bool last = l + 1 == m.layer_count;
+    const float* gamma_next = last ? m.out_norm : m.layers[l + 1].norm[0];
+    GUFFIN_TRY(guffin_hip_rms_norm_add_norm(st, s.part_a, slices(L.dtype[6], F, H), uint64_t(rows) * H, L.norm[5],
+                                            s.x1, s.x, gamma_next, last ? out_hidden : s.u,
+                                            last ? out_hidden_sums : s.us, rows, H, m.eps, status));
+    return GUFFIN_OK;
+}
+
 int forward_rows(hipStream_t stream, const guffin_model_desc& m, const uint32_t* tokens, uint32_t rows,
                  uint32_t position, const Scratch& s, void* priv_k, void* priv_v, float* out_hidden,
                  float* out_hidden_sums, uint32_t* status) {
@@ -228,27 +268,7 @@ int forward_rows(hipStream_t stream, const guffin_model_desc& m, const uint32_t*
                                                 s.attn_ml, rows, max_tokens_for(m, l, position, rows), ring_mask,
                                                 m.q_heads, m.kv_heads, m.head_dim, attn_scale, status));
         }
-        GUFFIN_TRY(guffin_hip_gemv_packed(st, L.dtype[3], L.tiles[3], s.a, s.as, s.part_a, nullptr, rows, QW, H));
-        // x1 = x + rms(o, post_attention_norm); u = rms(x1, ffn_norm)
-        GUFFIN_TRY(guffin_hip_rms_norm_add_norm(st, s.part_a, slices(L.dtype[3], QW, H), uint64_t(rows) * H, L.norm[3],
-                                                s.x, s.x1, L.norm[4], s.u, s.us, rows, H, m.eps, status));
-        if (L.dtype[4] == L.dtype[5] && L.dtype[4] != GUFFIN_Q6_K) {
-            GUFFIN_TRY(guffin_hip_gateup_geglu(st, L.dtype[4], L.tiles[4], L.tiles[5], s.u, s.us, s.h, s.hs, rows, H, F));
-        } else {
-            const int dt[2] = {L.dtype[4], L.dtype[5]};
-            const void* tl[2] = {L.tiles[4], L.tiles[5]};
-            const uint32_t n[2] = {F, F};
-            float* parts[2] = {s.part_a, s.part_b};
-            GUFFIN_TRY(guffin_hip_gemv_packed_multi(st, 2, dt, tl, n, parts, s.u, s.us, rows, H));
-            GUFFIN_TRY(guffin_hip_geglu(st, s.part_a, s.part_b, ffn_slices(L, H, F), uint64_t(rows) * F, s.h, s.hs, rows, F));
-        }
-        GUFFIN_TRY(guffin_hip_gemv_packed(st, L.dtype[6], L.tiles[6], s.h, s.hs, s.part_a, nullptr, rows, F, H));
-        // x = x1 + rms(down, post_ffw_norm); u = rms(x, next block's attn_norm | output_norm)
-        const bool last = l + 1 == m.layer_count;
-        const float* gamma_next = last ? m.out_norm : m.layers[l + 1].norm[0];
-        GUFFIN_TRY(guffin_hip_rms_norm_add_norm(st, s.part_a, slices(L.dtype[6], F, H), uint64_t(rows) * H, L.norm[5],
-                                                s.x1, s.x, gamma_next, last ? out_hidden : s.u,
-                                                last ? out_hidden_sums : s.us, rows, H, m.eps, status));
+        GUFFIN_TRY(block_tail(st, m, l, s, rows, out_hidden, out_hidden_sums, status));
     }
     return GUFFIN_OK;
 }
@@ -345,6 +365,95 @@ extern "C" int guffin_hip_forward_rows(void* stream, const guffin_model_desc* mo
     if (s.bytes > scratch_bytes) return fail(GUFFIN_E_CAPACITY, "forward_rows: scratch arena too small");
     return forward_rows(as_stream(stream), *model, tokens, rows, position, s, priv_k, priv_v, out_hidden,
                         out_hidden_sums, status);
+}
+
+// ---- rows of a verify tree -------------------------------------------------------------------
+// One pass of 1 or 2 rows whose parents may be any earlier row of the tree: a row's token list is the ring
+// below `base_position` (through the layer's window) followed by its ancestors among the tree's private
+// rows, itself last.  The rows' own K/V go to consecutive private slots; attention reads every slot an
+// ancestor list names, also those an earlier pass of the same tree wrote.
+extern "C" int guffin_hip_forward_tree_rows(void* stream, const guffin_model_desc* model, const uint32_t* tokens, uint32_t rows,
+                                            uint32_t base_position, const uint32_t* depths, const uint32_t* ancestor_lists,
+                                            const uint32_t* ancestor_counts, uint32_t first_slot, uint32_t slot_count,
+                                            void* scratch, uint64_t scratch_bytes, void* priv_k, void* priv_v,
+                                            float* out_hidden, float* out_hidden_sums, uint32_t* status) {
+    GUFFIN_TRY(validate_model(model));
+    if (!tokens || !depths || !ancestor_lists || !ancestor_counts || !scratch || !priv_k || !priv_v || !out_hidden || !status)
+        return fail(GUFFIN_E_ARG, "forward_tree_rows: null pointer");
+    if (rows == 0 || rows > 2) return fail(GUFFIN_E_SHAPE, "forward_tree_rows: a pass has 1 or 2 rows");
+    if (slot_count == 0 || slot_count > kMaxTreeSlots || first_slot + rows > slot_count)
+        return fail(GUFFIN_E_SHAPE, "forward_tree_rows: at most 8 private rows, the pass's slots among them");
+    const guffin_model_desc& m = *model;
+    if (m.global_period > 1 && m.sliding_window <= slot_count)
+        return fail(GUFFIN_E_SHAPE, "forward_tree_rows: the sliding window must exceed the tree's depth");
+    if (reinterpret_cast<uintptr_t>(scratch) & 255u) return fail(GUFFIN_E_ALIGN, "forward_tree_rows: scratch must be 256-byte aligned");
+    // host staging: positions, per-layer schedules, the concatenated ancestor lists
+    uint32_t positions[2] = {0, 0}, offsets[2] = {0, 0}, total = 0, deepest = 0;
+    for (uint32_t r = 0; r < rows; ++r) {
+        if (depths[r] >= slot_count) return fail(GUFFIN_E_ARG, "forward_tree_rows: a row lies deeper than the tree has rows");
+        const uint32_t n = ancestor_counts[r];
+        if (n == 0 || n > slot_count) return fail(GUFFIN_E_ARG, "forward_tree_rows: an ancestor list holds the row itself and at most every slot");
+        for (uint32_t i = 0; i < n; ++i)
+            if (ancestor_lists[total + i] >= slot_count) return fail(GUFFIN_E_ARG, "forward_tree_rows: ancestor outside the private rows");
+        if (ancestor_lists[total + n - 1] != first_slot + r) return fail(GUFFIN_E_ARG, "forward_tree_rows: a row's list ends with its own slot");
+        if (n != depths[r] + 1) return fail(GUFFIN_E_ARG, "forward_tree_rows: a row at depth d has d ancestors and itself");
+        positions[r] = base_position + depths[r];
+        offsets[r] = total;
+        total += n;
+        deepest = std::max(deepest, depths[r]);
+    }
+    GUFFIN_TRY(check_ring_capacity(m, base_position, deepest + 1, "forward_tree_rows: the rows do not fit the KV rings"));
+    // the arena of a chain pass at the deepest position covers this pass: its longest token list is the same
+    const Scratch s = layout(m, rows, base_position + slot_count, static_cast<uint8_t*>(scratch));
+    if (s.bytes > scratch_bytes) return fail(GUFFIN_E_CAPACITY, "forward_tree_rows: scratch arena too small");
+    std::vector<uint32_t> schedule(size_t(m.layer_count) * rows * 4);
+    for (uint32_t l = 0; l < m.layer_count; ++l)
+        for (uint32_t r = 0; r < rows; ++r) {
+            const bool local = is_local(m, l);
+            const uint32_t p = positions[r];
+            const uint32_t window_start = (local && p >= m.sliding_window) ? p + 1 - m.sliding_window : 0;
+            const uint32_t base_first = std::min(window_start, base_position);
+            uint32_t* e = schedule.data() + (size_t(l) * rows + r) * 4;
+            e[0] = base_first; e[1] = base_position - base_first; e[2] = offsets[r]; e[3] = ancestor_counts[r];
+        }
+    hipStream_t hs = as_stream(stream);
+    if (hipMemcpyAsync(s.positions, positions, rows * 4, hipMemcpyHostToDevice, hs) != hipSuccess
+        || hipMemcpyAsync(s.ancestors, ancestor_lists, total * 4, hipMemcpyHostToDevice, hs) != hipSuccess
+        || hipMemcpyAsync(s.schedule, schedule.data(), schedule.size() * 4, hipMemcpyHostToDevice, hs) != hipSuccess)
+        return fail(GUFFIN_E_HIP, "forward_tree_rows: upload failed");
+    const uint32_t H = m.hidden, QW = m.q_heads * m.head_dim, KW = m.kv_heads * m.head_dim;
+    const float attn_scale = 1.0f / std::sqrt(static_cast<float>(m.head_dim));
+    if (m.global_period > 1) GUFFIN_TRY(guffin_hip_rope_table(stream, s.positions, s.rope_local, rows, m.head_dim, m.local_base, 1.0f));
+    GUFFIN_TRY(guffin_hip_rope_table(stream, s.positions, s.rope_global, rows, m.head_dim, m.global_base, m.global_scale));
+    GUFFIN_TRY(guffin_hip_embed(stream, m.embed_dtype, m.embed_rows, tokens, s.x, rows, H, std::sqrt(static_cast<float>(H)), m.vocab, status));
+    GUFFIN_TRY(guffin_hip_rms_norm(stream, s.x, 1, 0, m.layers[0].norm[0], nullptr, s.u, s.us, rows, H, m.eps, status));
+    for (uint32_t l = 0; l < m.layer_count; ++l) {
+        const guffin_layer_desc& L = m.layers[l];
+        const bool local = is_local(m, l);
+        const uint32_t ring_mask = (local ? m.ring_local : m.ring_global) - 1;
+        uint16_t* layer_k = static_cast<uint16_t*>(priv_k) + size_t(l) * slot_count * KW;
+        uint16_t* layer_v = static_cast<uint16_t*>(priv_v) + size_t(l) * slot_count * KW;
+        const int dt[3] = {L.dtype[0], L.dtype[1], L.dtype[2]};
+        const void* tl[3] = {L.tiles[0], L.tiles[1], L.tiles[2]};
+        const uint32_t n[3] = {QW, KW, KW};
+        float* parts[3] = {s.part_a, s.part_b, s.part_c};
+        GUFFIN_TRY(guffin_hip_gemv_packed_multi(stream, 3, dt, tl, n, parts, s.u, s.us, rows, H));
+        const uint32_t sq = qkv_slices(L, H, QW, KW);
+        if (sq == 0) return fail(GUFFIN_E_SHAPE, "forward_tree_rows: q, k and v must share the block length");
+        // head norms, rotation and fp16 narrowing into the rows' own slots, then attention over ring and slots
+        GUFFIN_TRY(guffin_hip_qkv_post(stream, s.part_a, s.part_b, s.part_c, sq, sq, sq, uint64_t(rows) * QW, uint64_t(rows) * KW,
+                                       uint64_t(rows) * KW, L.norm[1], L.norm[2], s.positions, s.q, layer_k + size_t(first_slot) * KW,
+                                       layer_v + size_t(first_slot) * KW, rows, m.q_heads, m.kv_heads, m.head_dim, m.head_dim,
+                                       local ? m.local_base : m.global_base, local ? 1.0f : m.global_scale, m.eps,
+                                       local ? s.rope_local : s.rope_global, status));
+        const uint32_t ring_tokens = max_tokens_for(m, l, base_position + deepest, 1) - 1;   // the widest ring range of the pass
+        GUFFIN_TRY(guffin_hip_attention_decode(stream, s.q, L.ring_k, L.ring_v, layer_k, layer_v, s.schedule + size_t(l) * rows * 4,
+                                               s.ancestors, s.a, s.as, s.attn_out, s.attn_ml, rows, slot_count,
+                                               std::min(ring_tokens, base_position) + slot_count, ring_mask, m.q_heads, m.kv_heads,
+                                               m.head_dim, attn_scale, status));
+        GUFFIN_TRY(block_tail(stream, m, l, s, rows, out_hidden, out_hidden_sums, status));
+    }
+    return GUFFIN_OK;
 }
 
 extern "C" int guffin_hip_commit_rows(void* stream, const guffin_model_desc* model, const void* priv_k,

@@ -10,9 +10,11 @@
 // with the states of VerifierTransactionState (include/local_gguf_engine/engine/gemma2_metal_plan.hpp:
 // 208-215).  The pass keeps its K/V in private rows; a provisional commit first copies the ring rows
 // it is about to overwrite into the backup rows, then scatters the selected private rows into the
-// rings; finalize keeps a prefix of them and restores the rest.  The rows of a pass are a chain
-// (row r's parent is row r - 1), which is what the block graph here runs, so the only causal paths
-// are {0} and {0, 1}.  Nothing is allocated: every buffer is the caller's.
+// rings; finalize keeps a prefix of them and restores the rest.  The rows of a pass are a chain of 1 or
+// 2 rows (one launch sequence of the block graph) or a tree of up to 4 rows in topological order (row r's
+// parent is any earlier row), which runs in passes of 2 rows whose attention reads the earlier rows'
+// private K/V; a provisional commit takes any root-to-node path.  Nothing is allocated: every buffer is
+// the caller's.
 #include <cstddef>
 #include "common.hpp"
 #include "receipt.hpp"
@@ -29,7 +31,7 @@ constexpr uint64_t kAlign = 256;
 uint64_t aligned(uint64_t n) { return (n + kAlign - 1) & ~(kAlign - 1); }
 
 struct Arena {
-    uint64_t forward, hidden, parts, logits, select, total;
+    uint64_t forward, hidden, parts, pass_receipt, logits, select, total;
     uint64_t hidden_receipt;  // floats from the hidden rows to their receipt
 };
 
@@ -37,11 +39,15 @@ Arena arena_of(const guffin_model_desc& m, uint32_t position, uint32_t retain) {
     Arena a {};
     const uint32_t rows = kMaxTicketRows;
     uint64_t off = 0;
-    a.forward = off; off += aligned(guffin_hip_forward_scratch_bytes(&m, rows, position));
+    // a pass has at most 2 rows; a tree pass sizes its arena at the deepest position a row can take
+    a.forward = off; off += aligned(std::max({guffin_hip_forward_scratch_bytes(&m, 2, position),
+                                              guffin_hip_forward_scratch_bytes(&m, 2, position + kMaxTicketRows),
+                                              guffin_hip_forward_scratch_bytes(&m, 1, position + kMaxTicketRows)}));
     a.hidden_receipt = (uint64_t(rows) * m.hidden + 63) & ~uint64_t{63};
     a.hidden = off; off += aligned(a.hidden_receipt * 4 + receipt_layout(rows, m.hidden).bytes);
     const uint32_t slices = guffin_hip_gemv_packed_slices(m.head_dtype, m.hidden, m.vocab);
     a.parts = off; off += aligned(uint64_t(slices) * rows * m.vocab * 4);
+    a.pass_receipt = off; off += aligned(receipt_layout(2, m.hidden).bytes);
     a.logits = off; off += aligned(uint64_t(rows) * m.vocab * 4);
     a.select = off; off += aligned(guffin_hip_select_workspace_bytes(rows, m.vocab, retain));
     a.total = off;
@@ -90,25 +96,56 @@ extern "C" uint64_t guffin_hip_ticket_scratch_bytes(const guffin_verify_ticket* 
     return arena_of(*t->target, last_position, t->retain).total;
 }
 
-extern "C" int guffin_hip_ticket_encode(guffin_verify_ticket* t, const uint32_t* row_tokens, uint32_t rows, uint32_t position) {
+namespace {
+int encode(guffin_verify_ticket* t, const uint32_t* row_tokens, const uint32_t* parents, uint32_t rows, uint32_t position,
+           uint32_t max_rows, const char* too_many) {
     GUFFIN_TRY(ticket_ready(t, "ticket_encode: null pointer"));
     if (!row_tokens) return fail(GUFFIN_E_ARG, "ticket_encode: null pointer");
     if (t->state == GUFFIN_TXN_POISONED) return fail(GUFFIN_E_STATE, "ticket_encode: the ticket is poisoned");
     if (t->state != GUFFIN_TXN_IDLE) return fail(GUFFIN_E_STATE, "ticket_encode: a verify pass is already pending");
     const guffin_model_desc& m = *t->target;
-    if (rows == 0 || rows > kMaxTicketRows) return fail(GUFFIN_E_SHAPE, "ticket_encode: a pass has 1 or 2 rows");
+    if (rows == 0 || rows > max_rows) return fail(GUFFIN_E_SHAPE, too_many);
     if (!m.head_tiles || !m.layers) return fail(GUFFIN_E_ARG, "ticket_encode: the target needs its head tiles and layers");
     if (reinterpret_cast<uintptr_t>(t->scratch) & 255u) return fail(GUFFIN_E_ALIGN, "ticket_encode: the arena must be 256-byte aligned");
     // the selection keeps at most 320 candidates per row (guffin_hip_select_candidates)
     if (t->retain == 0 || t->retain > 320) return fail(GUFFIN_E_CAPACITY, "ticket_encode: retain must be 1..320 candidates per row");
-    if (uint64_t(position) + rows > m.ring_global) return fail(GUFFIN_E_CAPACITY, "ticket_encode: the rows do not fit the global rings");
+    uint32_t depths[kMaxTicketRows] = {}, deepest = 0;
+    for (uint32_t r = 0; r < rows; ++r) {
+        const uint32_t parent = parents ? parents[r] : (r == 0 ? GUFFIN_TICKET_ROOT : r - 1);
+        if ((r == 0) != (parent == GUFFIN_TICKET_ROOT) || (r > 0 && parent >= r))
+            return fail(GUFFIN_E_ARG, "ticket_encode: rows come in topological order under one root");
+        depths[r] = r == 0 ? 0u : depths[parent] + 1;
+        deepest = std::max(deepest, depths[r]);
+    }
+    if (uint64_t(position) + deepest + 1 > m.ring_global) return fail(GUFFIN_E_CAPACITY, "ticket_encode: the rows do not fit the global rings");
     if (t->scratch_bytes < arena_of(m, position, t->retain).total) return fail(GUFFIN_E_CAPACITY, "ticket_encode: scratch arena too small");
     t->rows = rows;
     t->position = position;
     t->provisional_count = 0;
-    for (uint32_t r = 0; r < kMaxTicketRows; ++r) t->row_tokens[r] = r < rows ? row_tokens[r] : 0u;
+    for (uint32_t r = 0; r < kMaxTicketRows; ++r) {
+        t->row_tokens[r] = r < rows ? row_tokens[r] : 0u;
+        t->parents[r] = r < rows ? (parents ? parents[r] : (r == 0 ? GUFFIN_TICKET_ROOT : r - 1)) : 0u;
+        t->depths[r] = r < rows ? depths[r] : 0u;
+    }
     t->state = GUFFIN_TXN_ENCODED;
     return GUFFIN_OK;
+}
+
+bool is_chain(const guffin_verify_ticket* t) {
+    for (uint32_t r = 1; r < t->rows; ++r)
+        if (t->parents[r] != r - 1) return false;
+    return true;
+}
+}  // namespace
+
+extern "C" int guffin_hip_ticket_encode(guffin_verify_ticket* t, const uint32_t* row_tokens, uint32_t rows, uint32_t position) {
+    return encode(t, row_tokens, nullptr, rows, position, 2, "ticket_encode: a pass has 1 or 2 rows");
+}
+
+extern "C" int guffin_hip_ticket_encode_tree(guffin_verify_ticket* t, const uint32_t* row_tokens, const uint32_t* parents,
+                                             uint32_t rows, uint32_t position) {
+    if (!parents) return fail(GUFFIN_E_ARG, "ticket_encode_tree: null pointer");
+    return encode(t, row_tokens, parents, rows, position, kMaxTicketRows, "ticket_encode_tree: a tree has 1 to 4 rows");
 }
 
 extern "C" int guffin_hip_ticket_submit(void* stream, guffin_verify_ticket* t) {
@@ -128,11 +165,33 @@ extern "C" int guffin_hip_ticket_submit(void* stream, guffin_verify_ticket* t) {
     if (hipMemcpyAsync(t->tokens, t->row_tokens, t->rows * sizeof(uint32_t), hipMemcpyHostToDevice, hs) != hipSuccess
         || hipMemcpyAsync(t->status, kZero, sizeof(kZero), hipMemcpyHostToDevice, hs) != hipSuccess)
         rc = fail(GUFFIN_E_HIP, "ticket_submit: upload failed");
-    if (rc == GUFFIN_OK)
-        rc = guffin_hip_forward_rows(stream, &m, t->tokens, t->rows, t->position, base + a.forward, a.hidden - a.forward, t->priv_k,
-                                     t->priv_v, hidden, hidden_sums, t->status);
-    if (rc == GUFFIN_OK)
-        rc = guffin_hip_gemv_packed(stream, m.head_dtype, m.head_tiles, hidden, hidden_sums, parts, logits, t->rows, m.hidden, m.vocab);
+    if (t->rows <= 2 && is_chain(t)) {
+        if (rc == GUFFIN_OK)
+            rc = guffin_hip_forward_rows(stream, &m, t->tokens, t->rows, t->position, base + a.forward, a.hidden - a.forward, t->priv_k,
+                                         t->priv_v, hidden, hidden_sums, t->status);
+        if (rc == GUFFIN_OK)
+            rc = guffin_hip_gemv_packed(stream, m.head_dtype, m.head_tiles, hidden, hidden_sums, parts, logits, t->rows, m.hidden, m.vocab);
+    } else {
+        // passes of two rows in row order; a row's ancestor list is its path from the root, itself last
+        float* pass_receipt = reinterpret_cast<float*>(base + a.pass_receipt);
+        for (uint32_t first = 0; rc == GUFFIN_OK && first < t->rows; first += 2) {
+            const uint32_t n = std::min(2u, t->rows - first);
+            uint32_t lists[2 * kMaxTicketRows], counts[2], used = 0;
+            for (uint32_t r = 0; r < n; ++r) {
+                uint32_t path[kMaxTicketRows], len = 0;
+                for (uint32_t node = first + r; node != GUFFIN_TICKET_ROOT; node = t->parents[node]) path[len++] = node;
+                for (uint32_t i = 0; i < len; ++i) lists[used + i] = path[len - 1 - i];
+                counts[r] = len;
+                used += len;
+            }
+            rc = guffin_hip_forward_tree_rows(stream, &m, t->tokens + first, n, t->position, t->depths + first, lists, counts, first,
+                                              t->rows, base + a.forward, a.hidden - a.forward, t->priv_k, t->priv_v,
+                                              hidden + size_t(first) * m.hidden, pass_receipt, t->status);
+            if (rc == GUFFIN_OK)
+                rc = guffin_hip_gemv_packed(stream, m.head_dtype, m.head_tiles, hidden + size_t(first) * m.hidden, pass_receipt, parts,
+                                            logits + size_t(first) * m.vocab, n, m.hidden, m.vocab);
+        }
+    }
     if (rc == GUFFIN_OK)
         rc = guffin_hip_select_candidates(stream, logits, t->rows, m.vocab, t->retain, nullptr, nullptr, base + a.select,
                                           t->candidates, t->status + 1);
@@ -173,8 +232,8 @@ extern "C" int guffin_hip_ticket_provisional_commit(void* stream, guffin_verify_
     if (t->state != GUFFIN_TXN_COMPLETED) return fail(GUFFIN_E_STATE, "ticket_provisional_commit: requires completion");
     if (!path || count == 0 || count > t->rows) return fail(GUFFIN_E_ARG, "ticket_provisional_commit: selected path extent is invalid");
     for (uint32_t i = 0; i < count; ++i) {
-        // row 0 is the root of the pass; row r's parent is row r - 1
-        if (path[i] >= t->rows || (i == 0 && path[i] != 0) || (i > 0 && path[i] != path[i - 1] + 1))
+        // row 0 is the root of the pass; every further node is a child of the one before it
+        if (path[i] >= t->rows || (i == 0 && path[i] != 0) || (i > 0 && t->parents[path[i]] != path[i - 1]))
             return fail(GUFFIN_E_ARG, "ticket_provisional_commit: selected nodes are not one causal path");
     }
     const guffin_model_desc& m = *t->target;

@@ -460,7 +460,8 @@ class VerifyTicketDesc(C.Structure):
                 ("priv_k", C.c_void_p), ("priv_v", C.c_void_p), ("backup_k", C.c_void_p), ("backup_v", C.c_void_p),
                 ("tokens", C.c_void_p), ("selected", C.c_void_p), ("candidates", C.c_void_p), ("status", C.c_void_p),
                 ("retain", C.c_uint32), ("state", C.c_uint32), ("rows", C.c_uint32), ("position", C.c_uint32),
-                ("provisional_count", C.c_uint32), ("provisional_path", C.c_uint32 * 2), ("row_tokens", C.c_uint32 * 2)]
+                ("provisional_count", C.c_uint32), ("provisional_path", C.c_uint32 * 4), ("row_tokens", C.c_uint32 * 4),
+                ("parents", C.c_uint32 * 4), ("depths", C.c_uint32 * 4)]
 
 
 TXN_IDLE, TXN_ENCODED, TXN_SUBMITTED, TXN_COMPLETED, TXN_PROVISIONAL, TXN_POISONED = range(6)
@@ -481,12 +482,12 @@ class VerifyTicket:
         if nbytes == 0:
             raise hip.GuffinError(-1, "ticket: no arena size for this target")
         self.scratch = torch.zeros(nbytes, dtype=torch.uint8, device="cuda")
-        self.priv_k, self.priv_v = target.private_rows(2)
-        self.backup_k, self.backup_v = target.private_rows(2)
-        self.tokens = torch.zeros(2, dtype=torch.int32, device="cuda")
-        self.selected = torch.zeros(2, dtype=torch.int32, device="cuda")
-        self.candidates = torch.zeros(2 * hip.candidates_dtype.itemsize, dtype=torch.uint8, device="cuda")
-        self.status = torch.zeros(3, dtype=torch.int32, device="cuda")
+        self.priv_k, self.priv_v = target.private_rows(4)
+        self.backup_k, self.backup_v = target.private_rows(4)
+        self.tokens = torch.zeros(4, dtype=torch.int32, device="cuda")
+        self.selected = torch.zeros(4, dtype=torch.int32, device="cuda")
+        self.candidates = torch.zeros(4 * hip.candidates_dtype.itemsize, dtype=torch.uint8, device="cuda")
+        self.status = torch.zeros(5, dtype=torch.int32, device="cuda")
         t.scratch, t.scratch_bytes = self.scratch.data_ptr(), nbytes
         t.priv_k, t.priv_v = self.priv_k.data_ptr(), self.priv_v.data_ptr()
         t.backup_k, t.backup_v = self.backup_k.data_ptr(), self.backup_v.data_ptr()
@@ -501,6 +502,14 @@ class VerifyTicket:
     def encode(self, row_tokens, position):
         arr = (C.c_uint32 * len(row_tokens))(*row_tokens)
         hip.check(hip.lib().guffin_hip_ticket_encode(C.byref(self.desc), arr, len(row_tokens), position))
+
+    ROOT = 0xFFFFFFFF
+
+    def encode_tree(self, row_tokens, parents, position):
+        """parents[r]: the row whose child row r is (None for the root)."""
+        arr = (C.c_uint32 * len(row_tokens))(*row_tokens)
+        par = (C.c_uint32 * len(parents))(*[self.ROOT if p is None else p for p in parents])
+        hip.check(hip.lib().guffin_hip_ticket_encode_tree(C.byref(self.desc), arr, par, len(row_tokens), position))
 
     def submit(self):
         hip.check(hip.lib().guffin_hip_ticket_submit(hip._stream(), C.byref(self.desc)))

@@ -413,6 +413,20 @@ int guffin_hip_forward_rows(void* stream, const guffin_model_desc* model, const 
                             uint32_t rows, uint32_t position, void* scratch, uint64_t scratch_bytes,
                             void* priv_k, void* priv_v, float* out_hidden, float* out_hidden_sums,
                             uint32_t* status);
+/* One pass of 1 or 2 rows of a verify tree (rows whose parent is any earlier row, siblings included): row r sits
+ * at cache position base_position + depths[r] and attends the rings below base_position (through the layer's
+ * window) and then the private rows its ancestor list names, its own slot last (the list of row r has depths[r] + 1
+ * entries; the lists are concatenated in ancestor_lists, host memory like depths and ancestor_counts).  The rows'
+ * K/V go to slots first_slot.. of priv_k / priv_v, laid out [layer][slot_count][kv_heads*head_dim] (slot_count <= 8);
+ * slots written by earlier passes of the same tree are read where a list names them.  Operator order of
+ * guffin_hip_forward_rows with encode_verifier_kv_store and encode_verifier_attention as separate steps
+ * (metal_command_context.hpp:250, 267: the general `ancestors` form).  scratch: guffin_hip_forward_scratch_bytes(model,
+ * rows, base_position + slot_count) bytes. */
+int guffin_hip_forward_tree_rows(void* stream, const guffin_model_desc* model, const uint32_t* tokens, uint32_t rows,
+                                 uint32_t base_position, const uint32_t* depths, const uint32_t* ancestor_lists,
+                                 const uint32_t* ancestor_counts, uint32_t first_slot, uint32_t slot_count,
+                                 void* scratch, uint64_t scratch_bytes, void* priv_k, void* priv_v,
+                                 float* out_hidden, float* out_hidden_sums, uint32_t* status);
 /* How guffin_hip_forward_rows (and so guffin_hip_h1_step, the sessions and the tickets) runs the blocks:
  * 0 (default) the resident pass for models with one KV head that fit it (measured faster there), else one
  * launch per operator; 1 always one launch per operator; 2 the resident pass for every model it covers
@@ -695,26 +709,36 @@ int guffin_hip_session_complete(void* stream, guffin_h1_session* session, uint32
 #define GUFFIN_TXN_ENCODED 1u
 #define GUFFIN_TXN_COMPLETED 3u
 #define GUFFIN_TXN_PROVISIONAL 4u
-#define GUFFIN_TICKET_MAX_ROWS 2u
+#define GUFFIN_TICKET_MAX_ROWS 4u
 typedef struct guffin_verify_ticket {
     const guffin_model_desc* target;         /* with head_tiles */
     void* scratch; uint64_t scratch_bytes;   /* device arena, >= guffin_hip_ticket_scratch_bytes */
     void* priv_k; void* priv_v;              /* device, [blocks][rows][kv width] fp16: the pass's own rows */
-    void* backup_k; void* backup_v;          /* device, [blocks][2][kv width] fp16: ring rows a commit overwrites */
-    uint32_t* tokens;                        /* device u32[2]: the rows' tokens */
-    uint32_t* selected;                      /* device u32[2]: the selected path */
-    void* candidates;                        /* device, 2 candidate records */
-    uint32_t* status;                        /* device u32[3]: the pass's status word, one selection status per row */
+    void* backup_k; void* backup_v;          /* device, [blocks][4][kv width] fp16: ring rows a commit overwrites */
+    uint32_t* tokens;                        /* device u32[4]: the rows' tokens */
+    uint32_t* selected;                      /* device u32[4]: the selected path */
+    void* candidates;                        /* device, 4 candidate records */
+    uint32_t* status;                        /* device u32[5]: the pass's status word, one selection status per row */
     uint32_t retain;                         /* candidates kept per row (top_k), 1..320 */
     uint32_t state;                          /* GUFFIN_TXN_* */
     uint32_t rows, position, provisional_count;
     uint32_t provisional_path[GUFFIN_TICKET_MAX_ROWS];
     uint32_t row_tokens[GUFFIN_TICKET_MAX_ROWS];
+    uint32_t parents[GUFFIN_TICKET_MAX_ROWS];   /* row r's parent row (row 0: GUFFIN_TICKET_ROOT); a chain has r - 1 */
+    uint32_t depths[GUFFIN_TICKET_MAX_ROWS];    /* row r sits at cache position `position` + depths[r] */
 } guffin_verify_ticket;
+#define GUFFIN_TICKET_ROOT 0xFFFFFFFFu
 /* Arena size that covers every pass up to the given cache position. */
 uint64_t guffin_hip_ticket_scratch_bytes(const guffin_verify_ticket* ticket, uint32_t last_position);
-/* Host only: validates and records the pass (row tokens are host memory). */
+/* Host only: validates and records the pass (row tokens are host memory).  A chain of 1 or 2 rows. */
 int guffin_hip_ticket_encode(guffin_verify_ticket* ticket, const uint32_t* row_tokens, uint32_t rows, uint32_t position);
+/* The same for a tree of up to 4 rows in topological order (VerifierTopologyDescriptor,
+ * include/local_gguf_engine/engine/target_verifier.hpp): parents[0] = GUFFIN_TICKET_ROOT, parents[r] < r.  Row r is
+ * verified at cache position `position` + its depth and attends the ring and its ancestors among the rows.  A chain
+ * of 1 or 2 rows runs as guffin_hip_ticket_encode runs it (one pass); any other tree runs in passes of 2 rows
+ * through guffin_hip_forward_tree_rows.  guffin_hip_ticket_provisional_commit then takes any root-to-node path. */
+int guffin_hip_ticket_encode_tree(guffin_verify_ticket* ticket, const uint32_t* row_tokens, const uint32_t* parents,
+                                  uint32_t rows, uint32_t position);
 int guffin_hip_ticket_submit(void* stream, guffin_verify_ticket* ticket);
 /* Blocks on the stream.  device_status (may be NULL) receives the OR of the status words. */
 int guffin_hip_ticket_complete(void* stream, guffin_verify_ticket* ticket, uint32_t* device_status);

@@ -140,3 +140,88 @@ def test_a_raised_status_word_drops_the_transaction(hip, target):
     pk, pv = run_pass(hip, target, ticket, [17, 1999], POSITION)   # and the ticket is usable again
     ticket.discard()
     assert ticket.state == model.TXN_IDLE
+
+
+def oracle_candidates(gfo, host, tokens, position, row, retain=64):
+    """Top `retain` candidates of chain row `row` from the oracle's forward pass and head."""
+    hidden, pk, pv = gfo.forward(host, np.array(tokens, np.uint32), position, threads=8)
+    logits = gfo.gemv(host.shape.embed_dtype, host.head, hidden[row:row + 1], host.shape.vocab, threads=8)[0]
+    return gfo.select_candidates(logits, retain), pk[:, row], pv[:, row]
+
+
+def same_tokens_close_logits(got, want, scale, rel=1e-3):
+    """The device and the oracle sum in different orders: candidates agree as sets of tokens down to the
+    point where two logits are closer than the sides differ, and in value within 1e-3 of the logit scale."""
+    n = want.size
+    g = {int(t): float(l) for t, l in zip(got["values"]["token"][:n], got["values"]["logit"][:n])}
+    w = {int(t): float(l) for t, l in zip(want["token"], want["logit"])}
+    tol = rel * scale
+    for token, logit in w.items():
+        if token in g:
+            assert abs(g[token] - logit) <= tol
+        else:
+            assert logit <= float(want["logit"][-1]) + 2 * tol, "a clear member of the oracle's top is missing"
+    assert len(set(g) & set(w)) >= n - 2
+
+
+def test_three_row_tree_against_the_oracle_and_every_path(hip, gfo):
+    """Rows [root, A, B] with A and B both children of the root (two proposals for the same position):
+    row 1 equals row 1 of the chain [root, A] and row 2 equals row 1 of the chain [root, B], in the oracle's
+    arithmetic and on the device's own chain pass; a provisional commit publishes any root-to-node path."""
+    import torch
+    from guffin_amd import model
+    shape = replace(model.GEMMA3_12B, layers=6, vocab=2048, ring_global=2048)
+    host = model.HostModel(shape, seed=5, position=POSITION, untied_head=True)
+    target = model.DeviceModel.from_host(host)
+    ticket = model.VerifyTicket(target, POSITION + 4)
+    root, a, b = 17, 1999, 42
+    before = rings(target)
+    ticket.encode_tree([root, a, b], [None, 0, 0], POSITION)
+    ticket.submit()
+    assert ticket.complete() == 0 and ticket.state == model.TXN_COMPLETED
+    assert_rings(target, before)
+    got = ticket.read_candidates()
+    kvw = shape.kv_width
+    priv_k = ticket.priv_k.view(-1)[:shape.layers * 3 * kvw].view(shape.layers, 3, kvw)
+    priv_v = ticket.priv_v.view(-1)[:shape.layers * 3 * kvw].view(shape.layers, 3, kvw)
+    # (1) the oracle, chain by chain
+    for row, (chain, chain_row) in enumerate([((root, a), 0), ((root, a), 1), ((root, b), 1)]):
+        want, wk, wv = oracle_candidates(gfo, host, chain, POSITION, chain_row)
+        assert int(got[row]["count"]) == 64 and int(got[row]["status"]) == 0
+        same_tokens_close_logits(got[row], want, float(np.abs(want["logit"]).max()))
+        k = priv_k[:, row].view(torch.int16).cpu().numpy().view(np.uint16)
+        v = priv_v[:, row].view(torch.int16).cpu().numpy().view(np.uint16)
+        assert np.mean(k == wk) >= 0.95 and np.mean(v == wv) >= 0.95
+    # (2) the device's own two-row chain passes (fused attention) give the same rows up to summation order
+    for row, chain in ((1, (root, a)), (2, (root, b))):
+        hidden, sums, pk, pv, status = target.forward(torch.tensor(chain, dtype=torch.int32, device="cuda"), POSITION)
+        logits = hip.gemv_packed(int(shape.embed_dtype), target.head_tiles, hidden, sums, shape.vocab)
+        want = hip.candidates_to_numpy(hip.select_candidates(logits, 64)[0])[1]
+        assert np.array_equal(got[row]["values"]["token"][:8], want["values"]["token"][:8])
+        assert np.allclose(got[row]["values"]["logit"][:64], want["values"]["logit"][:64], rtol=0, atol=1e-3 * float(np.abs(want["values"]["logit"][:64]).max()))
+        assert np.mean((priv_k[:, row] == pk[:, 1]).cpu().numpy()) >= 0.97
+    # (3) paths: [0, 2] publishes the root and B; keeping one row restores B's slot; [0, 1, 2] is no path
+    with pytest.raises(hip.GuffinError):
+        ticket.provisional_commit([0, 1, 2])
+    ticket.provisional_commit([0, 2])
+    want = rings_copy(before)
+    publish(want, target, priv_k, priv_v, POSITION, [0, 2])
+    assert_rings(target, want)
+    ticket.finalize(1)
+    kept = rings_copy(before)
+    publish(kept, target, priv_k, priv_v, POSITION, [0])
+    assert_rings(target, kept)
+    # a four-row tree with a grandchild: [root, A, A's child, B]
+    ticket.encode_tree([a, b, 7, root], [None, 0, 1, 0], POSITION + 1)
+    ticket.submit()
+    assert ticket.complete() == 0
+    got = ticket.read_candidates()
+    host.commit(np.stack([priv_k[:, 0].view(torch.int16).cpu().numpy().view(np.uint16)] * 1, axis=1),
+                np.stack([priv_v[:, 0].view(torch.int16).cpu().numpy().view(np.uint16)] * 1, axis=1), POSITION, 1)
+    # the ring row below this tree is the device's own (published above), so the sides start a little apart
+    for row, (chain, chain_row) in ((1, ((a, b), 1)), (3, ((a, root), 1))):
+        want, _, _ = oracle_candidates(gfo, host, chain, POSITION + 1, chain_row)
+        same_tokens_close_logits(got[row], want, float(np.abs(want["logit"]).max()), rel=2e-3)
+    ticket.provisional_commit([0, 1, 2])
+    ticket.discard()
+    assert_rings(target, kept)

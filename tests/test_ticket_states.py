@@ -40,6 +40,9 @@ def make_ticket(retain=64, scratch_bytes=1 << 34, **shape_changes):
     return t, (desc, layers)
 
 
+ROOT = 0xFFFFFFFF
+
+
 def tokens(*values):
     return (C.c_uint32 * len(values))(*values)
 
@@ -55,7 +58,8 @@ def test_calls_out_of_order_are_refused_and_change_nothing():
     assert lib.guffin_hip_ticket_discard(None, C.byref(t)) == 0      # an idle ticket has nothing to discard
     assert lib.guffin_hip_ticket_release(None, C.byref(t)) == 0
     assert lib.guffin_hip_ticket_encode(C.byref(t), tokens(5, 6), 2, 100) == 0
-    assert (t.state, t.rows, t.position, list(t.row_tokens)) == (model.TXN_ENCODED, 2, 100, [5, 6])
+    assert (t.state, t.rows, t.position, list(t.row_tokens)[:2]) == (model.TXN_ENCODED, 2, 100, [5, 6])
+    assert list(t.parents)[:2] == [ROOT, 0] and list(t.depths)[:2] == [0, 1]
     assert lib.guffin_hip_ticket_encode(C.byref(t), tokens(5, 6), 2, 100) == E_STATE   # one pass at a time
     assert lib.guffin_hip_ticket_complete(None, C.byref(t), None) == E_STATE
     assert lib.guffin_hip_ticket_provisional_commit(None, C.byref(t), tokens(0), 1) == E_STATE
@@ -97,12 +101,37 @@ def test_selected_path_must_be_one_causal_path(path):
     lib = hip.lib()
     t, keep = make_ticket()
     t.state, t.rows, t.position = model.TXN_COMPLETED, 2, 40   # as guffin_hip_ticket_complete leaves it
+    t.parents[0], t.parents[1] = ROOT, 0
     arr = tokens(*path) if path else tokens(0)
     assert lib.guffin_hip_ticket_provisional_commit(None, C.byref(t), arr, len(path)) == E_ARG
     assert t.state == model.TXN_COMPLETED and t.provisional_count == 0
     one, keep1 = make_ticket()
     one.state, one.rows = model.TXN_COMPLETED, 1
     assert lib.guffin_hip_ticket_provisional_commit(None, C.byref(one), tokens(0, 1), 2) == E_ARG   # row 1 was not in the pass
+
+
+def test_trees_are_encoded_in_topological_order_and_paths_follow_parents():
+    """A verify tree (VerifierTopologyDescriptor): one root, parents before children, at most 4 rows; a
+    provisional commit takes a root-to-node path and nothing else."""
+    lib = hip.lib()
+    t, keep = make_ticket()
+    enc = lambda toks, parents, position=100: lib.guffin_hip_ticket_encode_tree(C.byref(t), tokens(*toks), tokens(*parents), len(toks), position)
+    assert enc((5, 6, 7), (ROOT, 0, 0)) == 0
+    assert (t.state, t.rows, list(t.parents)[:3], list(t.depths)[:3]) == (model.TXN_ENCODED, 3, [ROOT, 0, 0], [0, 1, 1])
+    assert lib.guffin_hip_ticket_discard(None, C.byref(t)) == 0
+    assert enc((5, 6, 7, 8), (ROOT, 0, 1, 0)) == 0 and list(t.depths) == [0, 1, 2, 1]
+    assert lib.guffin_hip_ticket_discard(None, C.byref(t)) == 0
+    for parents in ((0, 0, 0), (ROOT, ROOT, 0), (ROOT, 1, 0), (ROOT, 0, 2), (ROOT, 0, 5)):
+        assert enc((5, 6, 7), parents) == E_ARG and t.state == model.TXN_IDLE, parents
+    assert enc((1, 2, 3, 4, 5), (ROOT, 0, 1, 2, 3)) == E_SHAPE                  # more rows than a ticket holds
+    assert lib.guffin_hip_ticket_encode(C.byref(t), tokens(1, 2, 3), 3, 100) == E_SHAPE   # a chain pass has 1 or 2 rows
+    assert enc((5, 6, 7), (ROOT, 0, 1), 2046) == E_CAPACITY                  # depth 2 at position 2046 of 2048
+    assert enc((5, 6, 7), (ROOT, 0, 0), 2046) == 0                           # depth 1 fits
+    t.state = model.TXN_COMPLETED
+    for path in ((0, 1, 2), (2,), (0, 2, 1), (1, 2), (0, 3)):
+        arr = tokens(*path)
+        assert lib.guffin_hip_ticket_provisional_commit(None, C.byref(t), arr, len(path)) == E_ARG, path
+    assert t.state == model.TXN_COMPLETED
 
 
 def test_finalize_cannot_retain_an_uncommitted_row():
