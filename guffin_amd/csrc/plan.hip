@@ -670,7 +670,6 @@ extern "C" int guffin_hip_h1_step(void* stream, const guffin_h1_desc* d, const u
     if (dr == 2 && !d->pending_token) return fail(GUFFIN_E_ARG, "h1_step: two drafter rows need the pending token");
     const bool mapped = d->draft_to_target != nullptr;
     if (mapped != (d->target_to_draft != nullptr)) return fail(GUFFIN_E_ARG, "h1_step: the vocabulary map needs its inverse");
-    if (mapped && d->full_law) return fail(GUFFIN_E_ARG, "h1_step: the vocabulary map goes with the compact law only");
     hipLaunchKernelGGL(set_step_tokens_kernel, dim3(1), dim3(1), 0, s, root_token, dr == 2 ? d->pending_token : nullptr, tokens,
                        d->target_to_draft, T.vocab, status);
     GUFFIN_TRY(check_launch("set_step_tokens"));
@@ -689,9 +688,14 @@ extern "C" int guffin_hip_h1_step(void* stream, const guffin_h1_desc* d, const u
             GUFFIN_TRY(check_launch("draft_history"));
             draft_hist = B.hist + kHistDraft;
         }
-        GUFFIN_TRY(guffin_hip_draft_law_mapped(stream, q_logits, D.vocab, d->draft_to_target, draft_hist,
-                                               with_history ? d->history_count : 0u, &opt, d->seed, d->step, nullptr, law_ws,
-                                               q_parts, law, tokens + 2, tokens + 1, status));
+        if (d->full_law)
+            GUFFIN_TRY(guffin_hip_draft_law_any_mapped(stream, q_logits, D.vocab, d->draft_to_target, draft_hist,
+                                                       with_history ? d->history_count : 0u, &opt, d->seed, d->step, nullptr, any_ws,
+                                                       q_parts, law, full_cdf, tokens + 2, tokens + 1, status));
+        else
+            GUFFIN_TRY(guffin_hip_draft_law_mapped(stream, q_logits, D.vocab, d->draft_to_target, draft_hist,
+                                                   with_history ? d->history_count : 0u, &opt, d->seed, d->step, nullptr, law_ws,
+                                                   q_parts, law, tokens + 2, tokens + 1, status));
     } else if (with_history && d->repetition_penalty != 1.0f) {
         // the proposal law sees the same history as the verify pass's first row (the head's partial
         // planes are summed by now: their buffer takes the penalised scores)

@@ -239,7 +239,7 @@ __global__ void law_begin_kernel(DraftLaw* law, uint32_t* proposal, uint32_t* er
 
 // score = logit / T (gd_process), then 2048-token tiles sorted by (score desc, token asc)
 __global__ void __launch_bounds__(1024)
-law_sort_tile_kernel(const float* __restrict__ logits, uint32_t vocab, float temperature, bool sort,
+law_sort_tile_kernel(const float* __restrict__ logits, uint32_t vocab, float temperature, bool sort, bool suppressed_ok,
                      const uint32_t* __restrict__ guard, FullLawWs ws, uint32_t* __restrict__ status) {
     if (guarded_off(guard)) return;
     __shared__ uint64_t keys[kSortTile];
@@ -248,9 +248,14 @@ law_sort_tile_kernel(const float* __restrict__ logits, uint32_t vocab, float tem
         uint64_t key = 0;  // padding sorts behind every real entry
         if (token < vocab) {
             float score = logits[token];
-            if (!isfinite(score)) { law_fail(status, ws.error, GUFFIN_STATUS_LAW_INVALID | GUFFIN_STATUS_NONFINITE); score = 0.f; }
-            if (temperature > 0.f) score = __fdiv_rn(score, temperature);
-            if (!isfinite(score)) { law_fail(status, ws.error, GUFFIN_STATUS_LAW_INVALID | GUFFIN_STATUS_NONFINITE); score = 0.f; }
+            // a score of -inf marks a draft token the vocabulary map gives no target token (its raw logit was
+            // validated where the scores were made): it stays out of every sum and sorts last
+            const bool suppressed = suppressed_ok && score == -INFINITY;
+            if (!suppressed) {
+                if (!isfinite(score)) { law_fail(status, ws.error, GUFFIN_STATUS_LAW_INVALID | GUFFIN_STATUS_NONFINITE); score = 0.f; }
+                if (temperature > 0.f) score = __fdiv_rn(score, temperature);
+                if (!isfinite(score)) { law_fail(status, ws.error, GUFFIN_STATUS_LAW_INVALID | GUFFIN_STATUS_NONFINITE); score = 0.f; }
+            }
             ws.scores[token] = score;
             key = score_key(score, token);
         }
@@ -722,11 +727,11 @@ int launch_compact_law(hipStream_t s, const float* logits, uint32_t vocab, const
 // the full-vocabulary kernels in the reference's dispatch order (src/engine/gemma3_draft.mm:1040-1166)
 int launch_full_law(hipStream_t s, const float* logits, uint32_t vocab, const SamplerOptions& opt, uint64_t seed,
                     uint64_t step, const void* injected_draws, const uint32_t* guard, const FullLawWs& ws,
-                    uint64_t* cdf, uint32_t* proposal, uint32_t* status) {
+                    uint64_t* cdf, uint32_t* proposal, uint32_t* status, bool suppressed_ok = false) {
     const bool greedy = opt.temperature == 0.f;
     const uint32_t padded = padded_vocab(vocab);
     hipLaunchKernelGGL(law_sort_tile_kernel, dim3(padded / kSortTile), dim3(1024), 0, s, logits, vocab, opt.temperature,
-                       !greedy, guard, ws, status);
+                       !greedy, suppressed_ok, guard, ws, status);
     if (!greedy) {
         const uint64_t* sorted = ws.keys_a;
         uint64_t* other = ws.keys_b;
@@ -840,9 +845,10 @@ extern "C" uint64_t guffin_hip_draft_law_any_workspace_bytes(uint32_t vocab) {
     return compact_ws_bytes(vocab) + full_ws_bytes(vocab);
 }
 
-extern "C" int guffin_hip_draft_law_any(void* stream, const float* logits, uint32_t vocab, const void* options,
-                                        uint64_t seed, uint64_t step, const void* injected_draws, void* workspace,
-                                        void* law, uint64_t* full_cdf, uint32_t* proposal, uint32_t* status) {
+namespace {
+int draft_law_any(void* stream, const float* logits, uint32_t vocab, const void* options, uint64_t seed, uint64_t step,
+                  const void* injected_draws, void* workspace, void* law, uint64_t* full_cdf, uint32_t* proposal,
+                  uint32_t* status, bool suppressed_ok) {
     if (!logits || !options || !workspace || !law || !full_cdf || !proposal || !status)
         return fail(GUFFIN_E_ARG, "draft_law_any: null pointer");
     if (vocab < kLawTile || vocab % kLawTile != 0)
@@ -860,12 +866,43 @@ extern "C" int guffin_hip_draft_law_any(void* stream, const float* logits, uint3
     if (compact_options(opt)) {
         // the compact law; its kernel hands over to the guarded full-vocabulary kernels when more
         // than 256 tokens tie into the support
-        if (int rc = launch_compact_law(s, logits, vocab, opt, seed, step, injected_draws, base, law, proposal, status, ws.error))
+        if (int rc = launch_compact_law(s, logits, vocab, opt, seed, step, injected_draws, base, law, proposal, status, ws.error, suppressed_ok))
             return rc;
-        return launch_full_law(s, logits, vocab, opt, seed, step, injected_draws, &slot->count, ws, full_cdf, proposal, status);
+        return launch_full_law(s, logits, vocab, opt, seed, step, injected_draws, &slot->count, ws, full_cdf, proposal, status, suppressed_ok);
     }
     hipLaunchKernelGGL(law_begin_kernel, dim3(1), dim3(1), 0, s, slot, proposal, ws.error);
-    return launch_full_law(s, logits, vocab, opt, seed, step, injected_draws, nullptr, ws, full_cdf, proposal, status);
+    return launch_full_law(s, logits, vocab, opt, seed, step, injected_draws, nullptr, ws, full_cdf, proposal, status, suppressed_ok);
+}
+}  // namespace
+
+
+extern "C" int guffin_hip_draft_law_any(void* stream, const float* logits, uint32_t vocab, const void* options,
+                                        uint64_t seed, uint64_t step, const void* injected_draws, void* workspace,
+                                        void* law, uint64_t* full_cdf, uint32_t* proposal, uint32_t* status) {
+    return draft_law_any(stream, logits, vocab, options, seed, step, injected_draws, workspace, law, full_cdf, proposal, status, false);
+}
+
+extern "C" int guffin_hip_draft_law_any_mapped(void* stream, const float* logits, uint32_t vocab, const int32_t* draft_to_target,
+                                               const uint32_t* history, uint32_t history_count, const void* options,
+                                               uint64_t seed, uint64_t step, const void* injected_draws, void* workspace,
+                                               float* scores, void* law, uint64_t* full_cdf, uint32_t* draft_proposal,
+                                               uint32_t* target_proposal, uint32_t* status) {
+    if (!logits || !draft_to_target || !options || !scores || !draft_proposal || !target_proposal || !status || (history_count && !history))
+        return fail(GUFFIN_E_ARG, "draft_law_any_mapped: null pointer");
+    if (vocab == 0) return fail(GUFFIN_E_SHAPE, "draft_law_any_mapped: empty vocabulary");
+    if (history_count > kHistoryCap) return fail(GUFFIN_E_CAPACITY, "draft_law_any_mapped: at most 64 history tokens");
+    const SamplerOptions opt = *static_cast<const SamplerOptions*>(options);
+    if (!std::isfinite(opt.repetition_penalty) || !(opt.repetition_penalty > 0.f)) return fail(GUFFIN_E_ARG, "draft_law_any_mapped: the penalty must be positive");
+    hipStream_t s = as_stream(stream);
+    const uint32_t blocks = std::min<uint32_t>((vocab + 255) / 256, 1024);
+    hipLaunchKernelGGL(draft_process_kernel, dim3(blocks), dim3(256), 0, s, logits, vocab, history, history_count,
+                       opt.repetition_penalty, draft_to_target, scores, status);
+    if (int rc = check_launch("draft_process")) return rc;
+    if (int rc = draft_law_any(stream, scores, vocab, options, seed, step, injected_draws, workspace, law, full_cdf, draft_proposal,
+                               status, true))
+        return rc;
+    hipLaunchKernelGGL(map_proposal_kernel, dim3(1), dim3(1), 0, s, draft_to_target, vocab, draft_proposal, target_proposal);
+    return check_launch("map_proposal");
 }
 
 extern "C" int guffin_hip_spec_accept_mapped(void* stream, const void* target_candidates, const void* law,

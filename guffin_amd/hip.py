@@ -455,10 +455,30 @@ def draft_law_mapped(logits, draft_to_target, options, history=None, seed=0, ste
     return law, draft, target, status
 
 
+def draft_law_any_mapped(logits, draft_to_target, options, history=None, seed=0, step=0, draws=None, status=None):
+    """draft_law_mapped by whichever path the options need: (law, full table, draft proposal, target proposal, status)."""
+    vocab = logits.numel()
+    lib().guffin_hip_draft_law_any_workspace_bytes.restype = C.c_uint64
+    workspace = _bytes(lib().guffin_hip_draft_law_any_workspace_bytes(vocab))
+    scores = torch.empty_like(logits)
+    law = _bytes(law_dtype.itemsize)
+    cdf = torch.zeros(vocab + 1, dtype=torch.int64, device=logits.device)
+    draft = torch.zeros(1, dtype=torch.int32, device=logits.device)
+    target = torch.zeros(1, dtype=torch.int32, device=logits.device)
+    if status is None:
+        status = torch.zeros(1, dtype=torch.int32, device=logits.device)
+    check(lib().guffin_hip_draft_law_any_mapped(_stream(), _p(logits), vocab, _p(draft_to_target), _p(history),
+                                                0 if history is None else history.numel(), C.byref(options),
+                                                C.c_uint64(seed), C.c_uint64(step), _p(draws), _p(workspace), _p(scores),
+                                                _p(law), _p(cdf), _p(draft), _p(target), _p(status)))
+    return law, cdf, draft, target, status
+
+
 def spec_accept_mapped(cands, law, target_to_draft, proposal, options, history=None, history_count=None, seed=0,
-                       step=0, draws=None, status=None):
+                       step=0, draws=None, status=None, full_cdf=None, vocab=0):
+    """full_cdf / vocab: the drafter's full table and its vocabulary when the law is held as one."""
     result = _bytes(result_dtype.itemsize)
-    check(lib().guffin_hip_spec_accept_mapped(_stream(), _p(cands), _p(law), None, 0, _p(target_to_draft), _p(history),
+    check(lib().guffin_hip_spec_accept_mapped(_stream(), _p(cands), _p(law), _p(full_cdf), vocab, _p(target_to_draft), _p(history),
                                               _p(history_count), _p(proposal), C.byref(options), C.c_uint64(seed),
                                               C.c_uint64(step), _p(draws), _p(result), _p(status)))
     return result

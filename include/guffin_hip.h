@@ -372,6 +372,14 @@ int guffin_hip_draft_law_mapped(void* stream, const float* logits, uint32_t voca
                                 uint64_t seed, uint64_t step, const void* injected_draws, void* workspace,
                                 float* scores, void* law, uint32_t* draft_proposal, uint32_t* target_proposal,
                                 uint32_t* status);
+/* guffin_hip_draft_law_mapped by whichever path the options and the scores need (guffin_hip_draft_law_any on the
+ * processed scores): the full-vocabulary kernels keep suppressed tokens (-inf) out of every sum, so a token without
+ * a target id has an empty bin.  workspace: guffin_hip_draft_law_any_workspace_bytes(vocab). */
+int guffin_hip_draft_law_any_mapped(void* stream, const float* logits, uint32_t vocab, const int32_t* draft_to_target,
+                                    const uint32_t* history, uint32_t history_count, const void* options,
+                                    uint64_t seed, uint64_t step, const void* injected_draws, void* workspace,
+                                    float* scores, void* law, uint64_t* full_cdf, uint32_t* draft_proposal,
+                                    uint32_t* target_proposal, uint32_t* status);
 int guffin_hip_spec_accept_mapped(void* stream, const void* target_candidates, const void* law,
                                   const uint64_t* full_cdf, uint32_t vocab, const int32_t* target_to_draft,
                                   const uint32_t* history, const uint32_t* history_count,
@@ -528,8 +536,7 @@ typedef struct guffin_h1_desc {
     const uint32_t* history; uint32_t history_count; float repetition_penalty;
     /* The drafter's vocabulary map and its inverse (device; see guffin_hip_draft_law_mapped): both or
      * neither.  With them the root, the pending token and the history reach the drafter in its own ids,
-     * its law lives in its ids, and the proposal enters the verify pass in the target's.  Only with the
-     * compact law (full_law == 0). */
+     * its law lives in its ids, and the proposal enters the verify pass in the target's (with either law). */
     const int32_t* draft_to_target; const int32_t* target_to_draft;
 } guffin_h1_desc;
 uint64_t guffin_hip_h1_scratch_bytes(const guffin_h1_desc* desc);

@@ -158,6 +158,8 @@ int gfo_draft_law_compact_mapped(const float* logits, uint32_t vocab, const gfo_
 /* full-vocabulary law: cdf has vocab+1 entries */
 int gfo_draft_law_full(const float* logits, uint32_t vocab, const gfo_sampler_options* opt,
                        uint64_t* cdf);
+int gfo_draft_law_full_mapped(const float* logits, uint32_t vocab, const gfo_sampler_options* opt,
+                              const int32_t* draft_to_target, uint64_t* cdf);
 uint32_t gfo_draft_select(const gfo_draft_law* law, uint32_t word);
 uint32_t gfo_draft_select_full(const uint64_t* cdf, uint32_t vocab, uint32_t word);
 
@@ -191,6 +193,10 @@ int gfo_spec_accept_mapped(const gfo_token_logit* row0, uint32_t n0, const uint3
                            const gfo_draft_law* law, const int32_t* target_to_draft, uint32_t proposal,
                            const gfo_sampler_options* opt, double u_accept, double u_residual, double u_next,
                            gfo_spec_result* out);
+int gfo_spec_accept_full_mapped(const gfo_token_logit* row0, uint32_t n0, const gfo_token_logit* row1,
+                                uint32_t n1, const uint64_t* cdf, uint32_t vocab, const int32_t* target_to_draft,
+                                uint32_t proposal, const gfo_sampler_options* opt, double u_accept,
+                                double u_residual, double u_next, gfo_spec_result* out);
 int gfo_spec_accept_full(const gfo_token_logit* row0, uint32_t n0, const gfo_token_logit* row1,
                          uint32_t n1, const uint64_t* cdf, uint32_t vocab, uint32_t proposal,
                          const gfo_sampler_options* opt, double u_accept, double u_residual,

@@ -296,6 +296,26 @@ def spec_accept_mapped(row0, hist0, row1, hist1, law, target_to_draft, proposal,
     return rc, out
 
 
+def draft_law_full_mapped(logits, opt, draft_to_target):
+    logits = np.ascontiguousarray(logits, np.float32)
+    d2t = np.ascontiguousarray(draft_to_target, np.int32)
+    cdf = np.zeros(logits.size + 1, np.uint64)
+    rc = lib().gfo_draft_law_full_mapped(_ptr(logits), logits.size, C.byref(opt), _ptr(d2t), _ptr(cdf))
+    return rc, cdf
+
+
+def spec_accept_full_mapped(row0, row1, cdf, target_to_draft, proposal, opt, u_accept, u_residual, u_next):
+    row0 = np.ascontiguousarray(row0, token_logit)
+    row1 = np.ascontiguousarray(row1, token_logit)
+    cdf = np.ascontiguousarray(cdf, np.uint64)
+    t2d = np.ascontiguousarray(target_to_draft, np.int32)
+    out = SpecResult()
+    rc = lib().gfo_spec_accept_full_mapped(_ptr(row0), row0.size, _ptr(row1), row1.size, _ptr(cdf),
+                                           C.c_uint32(cdf.size - 1), _ptr(t2d), C.c_uint32(proposal), C.byref(opt),
+                                           C.c_double(u_accept), C.c_double(u_residual), C.c_double(u_next), C.byref(out))
+    return rc, out
+
+
 def spec_accept_full(row0, row1, cdf, proposal, opt, u_accept, u_residual, u_next):
     row0 = np.ascontiguousarray(row0, token_logit)
     row1 = np.ascontiguousarray(row1, token_logit)

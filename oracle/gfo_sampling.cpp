@@ -294,8 +294,24 @@ static int compact_law(const float* logits, uint32_t vocab, const gfo_sampler_op
     return 0;
 }
 
+static int full_law(const float* logits, uint32_t vocab, const gfo_sampler_options* opt,
+                    const int32_t* draft_to_target, uint64_t* cdf);
+
 int gfo_draft_law_full(const float* logits, uint32_t vocab, const gfo_sampler_options* opt,
                        uint64_t* cdf) {
+    return full_law(logits, vocab, opt, nullptr, cdf);
+}
+
+// with the drafter's vocabulary map: gd_process gives a token without a target id the score -inf before
+// either law is built (src/engine/gemma3_draft.mm:191-204), so it sorts last, weighs nothing and keeps an
+// empty bin; its raw logit is validated all the same
+int gfo_draft_law_full_mapped(const float* logits, uint32_t vocab, const gfo_sampler_options* opt,
+                              const int32_t* draft_to_target, uint64_t* cdf) {
+    return full_law(logits, vocab, opt, draft_to_target, cdf);
+}
+
+static int full_law(const float* logits, uint32_t vocab, const gfo_sampler_options* opt,
+                    const int32_t* draft_to_target, uint64_t* cdf) {
     // Full-vocabulary law (gemma3_draft.mm:295-395 in the dispatch order of :1040-1166), entered
     // when top_k > 64, when drafting greedily, or when the compact support overflows:
     // tiles of 256 tokens, f32 prefix inside a tile, f32 running offsets across tiles.
@@ -303,17 +319,20 @@ int gfo_draft_law_full(const float* logits, uint32_t vocab, const gfo_sampler_op
     if (opt->temperature == 0.0f) {
         // greedy drafting: no transform, no filter; all mass on the lowest-id maximum
         // (gd_max / gd_max_finish, then gd_cdf's step function, gemma3_draft.mm:338-379)
-        uint32_t best = 0;
+        uint32_t best = 0xFFFFFFFFu;
         for (uint32_t i = 0; i < vocab; ++i) {
             if (!std::isfinite(logits[i])) return -10;
-            if (logits[i] > logits[best]) best = i;
+            if (draft_to_target && draft_to_target[i] < 0) continue;
+            if (best == 0xFFFFFFFFu || logits[i] > logits[best]) best = i;
         }
+        if (best == 0xFFFFFFFFu) return -6;
         for (uint32_t i = 0; i <= vocab; ++i) cdf[i] = i <= best ? 0 : kMassTotal;
         return 0;
     }
     std::vector<float> score(vocab);
     for (uint32_t i = 0; i < vocab; ++i) {
         if (!std::isfinite(logits[i])) return -10;
+        if (draft_to_target && draft_to_target[i] < 0) { score[i] = -std::numeric_limits<float>::infinity(); continue; }
         score[i] = logits[i] / opt->temperature;
         if (!std::isfinite(score[i])) return -11;
     }
@@ -515,6 +534,14 @@ int gfo_spec_accept_mapped(const gfo_token_logit* row0, uint32_t n0, const uint3
     const RowHistory h {{history0, history1}, {count0, count1}};
     return spec_accept(row0, n0, row1, n1, LawView{law, nullptr, 0, target_to_draft}, proposal, opt, u_accept, u_residual,
                        u_next, out, h);
+}
+
+int gfo_spec_accept_full_mapped(const gfo_token_logit* row0, uint32_t n0, const gfo_token_logit* row1,
+                                uint32_t n1, const uint64_t* cdf, uint32_t vocab, const int32_t* target_to_draft,
+                                uint32_t proposal, const gfo_sampler_options* opt, double u_accept,
+                                double u_residual, double u_next, gfo_spec_result* out) {
+    return spec_accept(row0, n0, row1, n1, LawView{nullptr, cdf, vocab, target_to_draft}, proposal, opt, u_accept, u_residual,
+                       u_next, out);
 }
 
 int gfo_spec_accept_full(const gfo_token_logit* row0, uint32_t n0, const gfo_token_logit* row1,

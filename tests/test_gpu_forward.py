@@ -380,6 +380,27 @@ def test_h1_cycle_with_a_vocabulary_map(hip, gfo):
         rc, want = gfo.spec_accept_mapped(r0, history, r1, hist1, law, t2d, int(d2t[draft]), opt_cpu, ua, ur, un)
         assert rc == 0
         assert (res["accepted"], res["token"], res["next_root"]) == (want.accepted, want.token, want.next_root)
+    # the same map with a law that needs the full table (top_k beyond the compact law's 64)
+    wide = model.H1Plan(target, drafter, 300, 300, temperature=1.0, top_k=100, seed=4, publish=False, full_law=True,
+                        draft_to_target=d2t, target_to_draft=t2d)
+    wide_cpu = gfo.SamplerOptions(1.0, 100, 0.95, 0.0, 1.0)
+    wide.root.fill_(root)
+    for step in range(4):
+        wide.step(step)
+        torch.cuda.synchronize()
+        bufs, res = wide.buffers(), wide.read_result()
+        assert int(wide.status.item()) == 0 and res["status"] == 0
+        rc, cdf = gfo.draft_law_full_mapped(bufs["q_logits"].cpu().numpy(), wide_cpu, d2t)
+        assert rc == 0 and np.array_equal(bufs["full_cdf"].cpu().numpy().view(np.uint64), cdf)
+        word, ua, ur, un = gfo.step_draws(4, step)
+        draft = gfo.draft_select_full(cdf, word)
+        toks = bufs["tokens"].cpu().numpy().view(np.uint32)
+        assert toks[2] == draft and toks[1] == d2t[draft] and res["proposal"] == d2t[draft]
+        p_logits = bufs["p_logits"].cpu().numpy()
+        rc, want = gfo.spec_accept_full_mapped(gfo.select_candidates(p_logits[0], 100), gfo.select_candidates(p_logits[1], 100),
+                                               cdf, t2d, int(d2t[draft]), wide_cpu, ua, ur, un)
+        assert rc == 0
+        assert (res["accepted"], res["token"], res["next_root"]) == (want.accepted, want.token, want.next_root)
     # a root the drafter does not have raises the bad-token bit instead of reading outside its table
     orphan = int(np.nonzero(t2d < 0)[0][0])
     plan.root.fill_(orphan)

@@ -182,3 +182,46 @@ def test_device_laws_against_the_double_restatement(hip):
                 assert token in got, (T, k, p, m, token, mass)
         for token, mass in got.items():
             assert token in want and abs(mass - want[token]) <= 1e-6, (T, k, p, m, token, mass)
+
+
+def test_full_law_behind_a_vocabulary_map_is_the_oracles_table(hip, gfo):
+    """guffin_hip_draft_law_any_mapped: the table, the proposal in both id spaces and the greedy case, bit for
+    bit against the oracle's mapped full law; acceptance gathers q through the inverse map from the full table."""
+    import torch
+    vocab = 32768
+    rng = np.random.default_rng(21)
+    d2t = rng.permutation(vocab).astype(np.int32)
+    d2t[rng.choice(vocab, 2000, replace=False)] = -1
+    t2d = np.full(vocab, -1, np.int32)
+    t2d[d2t[d2t >= 0]] = np.nonzero(d2t >= 0)[0].astype(np.int32)
+    logits = rng.normal(0, 2, vocab).astype(np.float32)
+    logits[np.nonzero(d2t < 0)[0][:4]] = 40.0
+    for t, k, p, m in ((1.0, 128, 0.9, 0.0), (0.8, 256, 1.0, 0.02), (0.0, 1, 1.0, 0.0)):
+        word = int(rng.integers(0, 2 ** 32))
+        law, cdf, draft, target, status = hip.draft_law_any_mapped(dev(logits), dev(d2t), opts(hip, t, k, p, m),
+                                                                   draws=draws_for(hip, word))
+        rc, want = gfo.draft_law_full_mapped(logits, opts(gfo, t, k, p, m), d2t)
+        assert rc == 0 and int(status[0]) == 0
+        assert law.cpu().numpy().view(hip.law_dtype)[0]["count"] == 0xFFFFFFFF
+        assert np.array_equal(cdf.cpu().numpy().view(np.uint64), want)
+        pick = gfo.draft_select_full(want, word)
+        assert int(draft[0]) == pick and int(target[0]) == d2t[pick] and d2t[pick] >= 0
+        if t > 0:
+            # acceptance with this table: the target's candidates are in its ids, q comes through the inverse map
+            p_logits = rng.normal(0, 3, (2, vocab)).astype(np.float32)
+            p_logits[0, d2t[pick]] += 6.0          # the proposal sits in the target's support
+            cands, _ = hip.select_candidates(dev(p_logits), 64)
+            o_gpu, o_cpu = opts(hip, t, 64, p, m), opts(gfo, t, 64, p, m)
+            out = hip.spec_accept_mapped(cands, law, dev(t2d), target, o_gpu, seed=5, step=3, full_cdf=cdf, vocab=vocab)
+            got = out.cpu().numpy().view(hip.result_dtype)[0]
+            _, ua, ur, un = gfo.step_draws(5, 3)
+            rc, ref = gfo.spec_accept_full_mapped(gfo.select_candidates(p_logits[0], 64), gfo.select_candidates(p_logits[1], 64),
+                                                  want, t2d, int(d2t[pick]), o_cpu, ua, ur, un)
+            assert rc == 0 and got["status"] == 0
+            assert (got["accepted"], got["token"], got["next_root"]) == (ref.accepted, ref.token, ref.next_root)
+            assert abs(got["acceptance_probability"] - ref.acceptance_probability) <= 1e-14
+    # an unmapped token's NaN still poisons the law
+    broken = logits.copy()
+    broken[np.nonzero(d2t < 0)[0][0]] = np.nan
+    *_, status = hip.draft_law_any_mapped(dev(broken), dev(d2t), opts(hip, 1.0, 128, 0.9, 0.0))
+    assert int(status[0]) != 0

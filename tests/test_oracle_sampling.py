@@ -388,3 +388,43 @@ def test_mapped_law_reference_case(gfo):
     assert right == 511 and d2t[right] == 511
     logits[0] = np.nan
     assert gfo.draft_law_compact_mapped(logits, opt, d2t)[0] == -10
+
+
+def test_full_mapped_law_suppresses_unmapped_tokens_and_agrees_with_the_compact_one(gfo):
+    """The full-vocabulary law behind a vocabulary map: the reference's mapped case (an excluded control token
+    with the best logit gets no mass; a NaN in an excluded raw logit still refuses), the compact mapped law as a
+    second path to the same masses, the double-precision rule over the mapped tokens only, and greedy drafting
+    landing on the best MAPPED token."""
+    from law_brute import law as brute_law
+    vocab = 4096
+    rng = np.random.default_rng(12)
+    d2t = rng.permutation(vocab).astype(np.int32)
+    d2t[rng.choice(vocab, 300, replace=False)] = -1
+    logits = rng.normal(0, 2, vocab).astype(np.float32)
+    logits[np.nonzero(d2t < 0)[0][:3]] = 50.0          # unmapped tokens with the best logits by far
+    for t, k, p, m in ((0.8, 40, 0.9, 0.0), (1.0, 64, 1.0, 0.05), (1.2, 200, 0.95, 0.0), (0.7, 256, 1.0, 0.0)):
+        o = opts(gfo, t=t, k=k, p=p, m=m)
+        rc, cdf = gfo.draft_law_full_mapped(logits, o, d2t)
+        assert rc == 0
+        mass = np.diff(cdf.astype(np.int64))
+        assert mass.sum() == TOTAL and not mass[d2t < 0].any()
+        mapped = np.nonzero(d2t >= 0)[0]
+        want, margin = brute_law(logits[mapped], t, k, p, m)       # the rule over the tokens that exist
+        assert margin > 1e-5
+        for i, w in want.items():
+            assert abs(mass[mapped[i]] / TOTAL - w) <= 1e-6
+        assert np.count_nonzero(mass) <= len(want)
+        if k <= 64:
+            rc, law = gfo.draft_law_compact_mapped(logits, o, d2t)
+            assert rc == 0
+            ids = np.array(law.ids[:law.count])
+            cm = np.diff(np.array(law.cdf[:law.count + 1], dtype=np.int64))
+            assert list(np.nonzero(mass)[0]) == list(ids[cm > 0])
+            assert np.max(np.abs(mass[ids] - cm)) / TOTAL < 1e-6
+    rc, cdf = gfo.draft_law_full_mapped(logits, opts(gfo, t=0.0, k=1, p=1.0, m=0.0), d2t)
+    best_mapped = mapped[np.argmax(logits[mapped])]
+    assert rc == 0 and gfo.draft_select_full(cdf, 12345) == best_mapped and d2t[best_mapped] >= 0
+    broken = logits.copy()
+    broken[np.nonzero(d2t < 0)[0][0]] = np.nan
+    assert gfo.draft_law_full_mapped(broken, opts(gfo, k=100), d2t)[0] == -10
+    assert gfo.draft_law_full_mapped(logits, opts(gfo, k=100), np.full(vocab, -1, np.int32))[0] != 0   # nothing left to propose
