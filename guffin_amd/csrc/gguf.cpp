@@ -11,6 +11,7 @@
 #include <cstring>
 #include <limits>
 #include <new>
+#include <cmath>
 #include <string>
 #include <vector>
 
@@ -334,4 +335,107 @@ extern "C" int guffin_gguf_find_tensor(const guffin_gguf* g, const char* name, u
     for (size_t i = 0; i < g->tensors.size(); ++i)
         if (g->tensors[i].name == name) { *index = i; return GUFFIN_OK; }
     return GUFFIN_E_ARG;
+}
+
+// ---- weight binding ---------------------------------------------------------------------------
+// bind_gemma_model_weights + validate_gemma3_model_weights (src/engine/gemma_model.cpp:72-177): every tensor
+// a Gemma 3 block graph needs is looked up by its GGUF name and checked against the configuration before
+// anything is uploaded.  The detail string of a refusal follows the reference's wording.
+namespace {
+thread_local std::string g_bind_detail;
+
+int refuse(int code, std::string detail) {
+    g_bind_detail = std::move(detail);
+    return code;
+}
+
+constexpr const char* kMatrixNames[7] = {"attn_q", "attn_k", "attn_v", "attn_output", "ffn_gate", "ffn_up", "ffn_down"};
+constexpr const char* kNormNames[6] = {"attn_norm", "attn_q_norm", "attn_k_norm", "post_attention_norm", "ffn_norm", "post_ffw_norm"};
+constexpr uint32_t kTypeF32 = 0, kTypeQ8 = 8, kTypeQ4K = 12, kTypeQ6K = 14;
+
+std::string block_name(uint32_t block, const char* suffix) {
+    return "blk." + std::to_string(block) + "." + suffix + ".weight";
+}
+}  // namespace
+
+extern "C" const char* guffin_gguf_bind_detail(void) { return g_bind_detail.c_str(); }
+
+extern "C" int guffin_gguf_bind_gemma3(const guffin_gguf* g, const guffin_gemma3_config* c, guffin_gemma3_binding* out,
+                                       guffin_gemma3_block* blocks) {
+    if (!g || !c || !out || !blocks) return GUFFIN_E_ARG;
+    g_bind_detail.clear();
+    const auto finite_positive = [](float v) { return std::isfinite(v) && v > 0.0f; };
+    // the execution configuration (:106-119)
+    if (!c->uses_qk_norm || c->attention_global_layer_period != 6 || c->embedding_length == 0 || c->feed_forward_length == 0
+        || c->block_count == 0 || c->vocab_size == 0 || c->attention_head_count == 0 || c->attention_head_count_kv == 0
+        || c->attention_head_count % c->attention_head_count_kv != 0 || c->attention_key_length == 0
+        || c->attention_key_length % 2 != 0 || c->attention_key_length != c->attention_value_length
+        || !finite_positive(c->rms_norm_epsilon) || c->attention_logit_softcap != 0.0f || c->final_logit_softcap != 0.0f
+        || !finite_positive(c->rope_freq_base) || !finite_positive(c->local_rope_freq_base) || !finite_positive(c->rope_freq_scale))
+        return refuse(GUFFIN_BIND_INVALID_TENSOR, "Gemma 3 execution configuration");
+    // the target's geometry (:120-124); the drafter (4 query heads on 1 KV head, Q8_0 blocks) is bound without it
+    if (c->target_geometry
+        && (c->attention_key_length != 256 || uint64_t(c->attention_head_count) != 2 * uint64_t(c->attention_head_count_kv)
+            || c->block_count > 64))
+        return refuse(GUFFIN_BIND_INVALID_TENSOR, "Gemma 3 target requires 256-wide paired GQA heads and at most 64 layers");
+    if (c->context_length < c->sliding_window)
+        return refuse(GUFFIN_BIND_INVALID_TENSOR, "Gemma 3 runtime context must cover the local attention window");
+    const uint64_t query_width = uint64_t(c->attention_head_count) * c->attention_key_length;
+    const uint64_t kv_width = uint64_t(c->attention_head_count_kv) * c->attention_key_length;
+    if (query_width > 0xFFFFFFFFull || kv_width > 0xFFFFFFFFull)
+        return refuse(GUFFIN_BIND_INVALID_TENSOR, "Gemma 3 attention width exceeds 32-bit indexing range");
+
+    int rc = GUFFIN_OK;
+    const auto find = [&](const std::string& name, uint64_t* index, bool required) {
+        for (size_t i = 0; i < g->tensors.size(); ++i)
+            if (g->tensors[i].name == name) { *index = i; return true; }
+        if (required && rc == GUFFIN_OK) rc = refuse(GUFFIN_BIND_MISSING_TENSOR, name);
+        return false;
+    };
+    const auto norm = [&](const std::string& name, uint64_t width, uint64_t* index) {
+        if (rc != GUFFIN_OK || !find(name, index, true)) return;
+        const Tensor& t = g->tensors[static_cast<size_t>(*index)];
+        if (t.n_dims != 1 || t.dims[0] != width || t.type_id != kTypeF32)
+            rc = refuse(GUFFIN_BIND_INVALID_TENSOR, name + ": expected F32 norm with width " + std::to_string(width));
+    };
+    const auto matrix = [&](const std::string& name, uint64_t input, uint64_t output, uint64_t* index, bool head) {
+        if (rc != GUFFIN_OK || !find(name, index, true)) return;
+        const Tensor& t = g->tensors[static_cast<size_t>(*index)];
+        const bool kquant = head && c->target_geometry ? t.type_id == kTypeQ6K : (t.type_id == kTypeQ4K || t.type_id == kTypeQ6K);
+        const bool q8 = !c->target_geometry && t.type_id == kTypeQ8;
+        if (t.n_dims != 2 || t.dims[0] != input || t.dims[1] != output || !(kquant || q8) || input % (q8 ? 32 : 256) != 0)
+            rc = refuse(GUFFIN_BIND_INVALID_TENSOR, name + ": expected native " + (c->target_geometry ? (head ? "Q6_K" : "Q4_K/Q6_K") : "Q8_0/Q4_K/Q6_K")
+                            + " GGUF matrix [" + std::to_string(input) + ", " + std::to_string(output) + "]");
+    };
+    matrix("token_embd.weight", c->embedding_length, c->vocab_size, &out->token_embedding, true);
+    // output_weight_or_tied_embedding (:26-34): output.weight when the file has one, else the embedding
+    out->tied_output = 1;
+    out->output = out->token_embedding;
+    uint64_t own = 0;
+    if (rc == GUFFIN_OK && find("output.weight", &own, false)) {
+        matrix("output.weight", c->embedding_length, c->vocab_size, &out->output, true);
+        out->tied_output = 0;
+    }
+    if (rc == GUFFIN_OK && c->uses_tied_output_weight && !out->tied_output)
+        rc = refuse(GUFFIN_BIND_INVALID_TENSOR, "Gemma 3 tied output must alias token_embd.weight");
+    norm("output_norm.weight", c->embedding_length, &out->output_norm);
+    const uint64_t in_out[7][2] = {{c->embedding_length, query_width}, {c->embedding_length, kv_width}, {c->embedding_length, kv_width},
+                                   {query_width, c->embedding_length}, {c->embedding_length, c->feed_forward_length},
+                                   {c->embedding_length, c->feed_forward_length}, {c->feed_forward_length, c->embedding_length}};
+    const uint64_t widths[6] = {c->embedding_length, c->attention_key_length, c->attention_key_length, c->embedding_length,
+                                c->embedding_length, c->embedding_length};
+    for (uint32_t b = 0; rc == GUFFIN_OK && b < c->block_count; ++b) {
+        for (int i = 0; i < 6; ++i) norm(block_name(b, kNormNames[i]), widths[i], &blocks[b].norm[i]);
+        bool any_q8 = false, any_kquant = false;
+        for (int i = 0; i < 7; ++i) {
+            matrix(block_name(b, kMatrixNames[i]), in_out[i][0], in_out[i][1], &blocks[b].matrix[i], false);
+            if (rc != GUFFIN_OK) break;
+            blocks[b].type_id[i] = g->tensors[static_cast<size_t>(blocks[b].matrix[i])].type_id;
+            (blocks[b].type_id[i] == kTypeQ8 ? any_q8 : any_kquant) = true;
+        }
+        // the kernels of one block share an activation image: 32-weight and 256-weight formats do not mix in it
+        if (rc == GUFFIN_OK && any_q8 && any_kquant)
+            rc = refuse(GUFFIN_BIND_INVALID_TENSOR, block_name(b, "attn_q") + ": a block mixes 32-weight and 256-weight formats");
+    }
+    return rc;
 }

@@ -31,6 +31,34 @@ class TensorInfo(C.Structure):
                 ("offset", C.c_uint64), ("file_offset", C.c_uint64), ("byte_count", C.c_uint64)]
 
 
+class Gemma3Config(C.Structure):
+    """The GemmaModelConfig fields the weight validation reads (guffin_gemma3_config)."""
+    _fields_ = [(n, C.c_uint32) for n in
+                ("block_count", "embedding_length", "feed_forward_length", "vocab_size", "attention_head_count",
+                 "attention_head_count_kv", "attention_key_length", "attention_value_length", "sliding_window",
+                 "context_length", "attention_global_layer_period", "uses_qk_norm", "uses_tied_output_weight",
+                 "target_geometry")] + \
+               [(n, C.c_float) for n in ("rms_norm_epsilon", "attention_logit_softcap", "final_logit_softcap",
+                                         "rope_freq_base", "local_rope_freq_base", "rope_freq_scale")]
+
+
+class Gemma3Block(C.Structure):
+    _fields_ = [("matrix", C.c_uint64 * 7), ("norm", C.c_uint64 * 6), ("type_id", C.c_uint32 * 7), ("pad", C.c_uint32)]
+
+
+class Gemma3Binding(C.Structure):
+    _fields_ = [("token_embedding", C.c_uint64), ("output_norm", C.c_uint64), ("output", C.c_uint64),
+                ("tied_output", C.c_uint32), ("pad", C.c_uint32)]
+
+
+class BindError(ValueError):
+    """missing_tensor / invalid_tensor of the reference's EngineModelError, with its detail string."""
+    def __init__(self, code, detail):
+        self.code = {-120: "missing_tensor", -121: "invalid_tensor"}.get(code, code)
+        self.detail = detail
+        super().__init__("%s: %s" % (self.code, detail))
+
+
 class ReadError(Exception):
     def __init__(self, code, expected, actual, magic):
         self.code = ERRORS[-100 - code] if -114 <= code <= -100 else code
@@ -108,6 +136,22 @@ class Reader:
             raise KeyError(name)
         hip.lib().guffin_gguf_tensor(self._h, index, C.byref(t))
         return {"name": name, "dims": [int(t.dims[d]) for d in range(t.n_dims)], "type_id": t.type_id,
+                "offset": t.offset, "file_offset": t.file_offset, "byte_count": t.byte_count}
+
+    def bind_gemma3(self, config):
+        """guffin_gguf_bind_gemma3: (binding, blocks) of tensor indices, or BindError."""
+        lib = hip.lib()
+        lib.guffin_gguf_bind_detail.restype = C.c_char_p
+        binding, blocks = Gemma3Binding(), (Gemma3Block * max(1, config.block_count))()
+        rc = lib.guffin_gguf_bind_gemma3(self._h, C.byref(config), C.byref(binding), blocks)
+        if rc != 0:
+            raise BindError(rc, lib.guffin_gguf_bind_detail().decode())
+        return binding, blocks
+
+    def tensor_at(self, index):
+        t = TensorInfo()
+        assert hip.lib().guffin_gguf_tensor(self._h, C.c_uint64(index), C.byref(t)) == 0
+        return {"name": t.name.decode(), "dims": [int(t.dims[d]) for d in range(t.n_dims)], "type_id": t.type_id,
                 "offset": t.offset, "file_offset": t.file_offset, "byte_count": t.byte_count}
 
     def payload(self, name):

@@ -219,6 +219,7 @@ class DeviceModel:
         (src/engine/model.cpp:330-390), matrices uploaded as they lie in the file ([input, output] with
         the input dimension contiguous, i.e. blocks per output column) and repacked on the device, tied
         head when there is no output.weight.  Rings start empty."""
+        from . import gguf as gguf_module
         md = reader.metadata()
         key = lambda k: md[arch + "." + k]
         scale = 1.0
@@ -226,22 +227,33 @@ class DeviceModel:
             scale = 1.0 / float(key("rope.scaling.factor"))
         embed_info = reader.tensor("token_embd.weight")
         hidden, vocab = embed_info["dims"]
-        if hidden != key("embedding_length"):
-            raise ValueError("token_embd.weight does not match " + arch + ".embedding_length")
         layers = int(key("block_count"))
+        window = int(key("attention.sliding_window"))
+        # names, shapes and formats are checked by the library before anything is uploaded
+        # (guffin_gguf_bind_gemma3: bind_gemma_model_weights + validate_gemma3_model_weights of the reference)
+        cfg = gguf_module.Gemma3Config()
+        cfg.block_count, cfg.embedding_length, cfg.vocab_size = layers, int(key("embedding_length")), vocab
+        cfg.feed_forward_length = int(key("feed_forward_length"))
+        cfg.attention_head_count, cfg.attention_head_count_kv = int(key("attention.head_count")), int(key("attention.head_count_kv"))
+        cfg.attention_key_length, cfg.attention_value_length = int(key("attention.key_length")), int(key("attention.value_length"))
+        cfg.sliding_window, cfg.context_length = window, int(md.get(arch + ".context_length", ring_global))
+        cfg.attention_global_layer_period = int(md.get(arch + ".attention.sliding_window_pattern", 6))
+        cfg.uses_qk_norm, cfg.uses_tied_output_weight = 1, 0
+        cfg.target_geometry = 1 if cfg.attention_head_count == 2 * cfg.attention_head_count_kv and embed_info["type_id"] != 8 else 0
+        cfg.rms_norm_epsilon = float(key("attention.layer_norm_rms_epsilon"))
+        cfg.attention_logit_softcap = float(md.get(arch + ".attn_logit_softcapping", 0.0))
+        cfg.final_logit_softcap = float(md.get(arch + ".final_logit_softcapping", 0.0))
+        cfg.rope_freq_base = float(key("rope.freq_base"))
+        cfg.local_rope_freq_base = float(md.get(arch + ".rope.freq_base_swa", 10000.0))
+        cfg.rope_freq_scale = scale
+        binding, blocks = reader.bind_gemma3(cfg)
 
         def matrix_type(name):
-            t = reader.tensor(name)["type_id"]
-            if t not in cls.GGUF_TYPES:
-                raise ValueError("%s: tensor type %d is not a supported block format" % (name, t))
-            return cls.GGUF_TYPES[t]
+            return cls.GGUF_TYPES[reader.tensor(name)["type_id"]]
 
-        # every matrix is validated on its own, as the reference binds it (src/engine/gemma_model.cpp:140-148):
-        # a block's attn_v / ffn_down may be Q6_K where another block's is Q4_K
         names = [["blk.%d.%s.weight" % (l, m) for m in cls.GGUF_MATRICES] for l in range(layers)]
-        per_layer = tuple(tuple(matrix_type(n) for n in row) for row in names)
+        per_layer = tuple(tuple(cls.GGUF_TYPES[blocks[l].type_id[i]] for i in range(7)) for l in range(layers))
         uniform = all(row == per_layer[0] for row in per_layer)
-        window = int(key("attention.sliding_window"))
         shape = Shape(hidden=hidden, ffn=int(key("feed_forward_length")), q_heads=int(key("attention.head_count")),
                       kv_heads=int(key("attention.head_count_kv")), head_dim=int(key("attention.key_length")),
                       layers=layers, vocab=vocab, sliding_window=window,
@@ -258,9 +270,6 @@ class DeviceModel:
             return torch.from_numpy(np.array(reader.payload(name))).cuda()   # staged through a writable copy
 
         def norm(name, width):
-            t = reader.tensor(name)
-            if t["type_id"] != 0 or t["dims"] != [width]:
-                raise ValueError("%s: expected an F32 norm of width %d" % (name, width))
             return upload(name).view(torch.float32)
 
         widths = [hidden, shape.head_dim, shape.head_dim, hidden, hidden, hidden]
@@ -268,10 +277,6 @@ class DeviceModel:
             for i, (m, (K, N)) in enumerate(zip(cls.GGUF_MATRICES, shape.proj_shapes())):
                 name = names[l][i]
                 dt = per_layer[l][i]
-                if reader.tensor(name)["dims"] != [K, N]:
-                    raise ValueError("%s: expected a [%d, %d] matrix" % (name, K, N))
-                if dt == Q8_0 and any(d != Q8_0 for d in per_layer[l]):
-                    raise ValueError("%s: a block mixes 32-weight and 256-weight formats" % name)
                 tiles = hip.repack(dt, upload(name), K, N)
                 self.keep.append(tiles)
                 self.layers[l].dtype[i] = dt
@@ -287,7 +292,7 @@ class DeviceModel:
             self.ring_v.append(rv)
             self.layers[l].ring_k, self.layers[l].ring_v = rk.data_ptr(), rv.data_ptr()
         embed = upload("token_embd.weight")
-        head_name = "output.weight" if any(t["name"] == "output.weight" for t in reader.tensors()) else "token_embd.weight"
+        head_name = "token_embd.weight" if binding.tied_output else "output.weight"
         head = hip.repack(matrix_type(head_name), embed if head_name == "token_embd.weight" else upload(head_name),
                           hidden, vocab)
         torch.cuda.synchronize()

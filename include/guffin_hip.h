@@ -654,6 +654,36 @@ int guffin_gguf_find_entry(const guffin_gguf* gguf, const char* key, uint64_t* i
 int guffin_gguf_tensor(const guffin_gguf* gguf, uint64_t index, guffin_gguf_tensor_info* out);
 int guffin_gguf_find_tensor(const guffin_gguf* gguf, const char* name, uint64_t* index);
 
+/* Weight binding of a Gemma 3 shaped file: bind_gemma_model_weights + validate_gemma3_model_weights
+ * (src/engine/gemma_model.cpp:72-177).  Every tensor the block graph needs is looked up by its GGUF name
+ * (token_embd, output_norm, output or the tied embedding, per block the 7 matrices and 6 norms) and checked
+ * against the configuration: norms F32 of the right width, matrices native block formats of shape
+ * [input, output] with input a whole number of blocks.  target_geometry != 0 adds the target's rules (:120-124,
+ * :150-158): 256-wide heads, two query heads per KV head, at most 64 blocks, Q4_K / Q6_K matrices, a Q6_K head;
+ * without it the drafter's geometry and Q8_0 blocks are admitted (one block length per block).  Returns 0 and the
+ * tensor indices (for guffin_gguf_tensor), GUFFIN_BIND_MISSING_TENSOR (EngineModelErrorCode::missing_tensor) or
+ * GUFFIN_BIND_INVALID_TENSOR (::invalid_tensor) with the reference's detail string from guffin_gguf_bind_detail
+ * (per thread).  `blocks`: caller array of block_count records. */
+#define GUFFIN_BIND_MISSING_TENSOR (-120)
+#define GUFFIN_BIND_INVALID_TENSOR (-121)
+typedef struct guffin_gemma3_config {   /* the GemmaModelConfig fields the validation reads */
+    uint32_t block_count, embedding_length, feed_forward_length, vocab_size;
+    uint32_t attention_head_count, attention_head_count_kv, attention_key_length, attention_value_length;
+    uint32_t sliding_window, context_length, attention_global_layer_period;
+    uint32_t uses_qk_norm, uses_tied_output_weight, target_geometry;
+    float rms_norm_epsilon, attention_logit_softcap, final_logit_softcap;
+    float rope_freq_base, local_rope_freq_base, rope_freq_scale;
+} guffin_gemma3_config;
+typedef struct guffin_gemma3_block {
+    uint64_t matrix[7];    /* q, k, v, o, gate, up, down */
+    uint64_t norm[6];      /* attn_norm, attn_q_norm, attn_k_norm, post_attention_norm, ffn_norm, post_ffw_norm */
+    uint32_t type_id[7]; uint32_t pad;
+} guffin_gemma3_block;
+typedef struct guffin_gemma3_binding { uint64_t token_embedding, output_norm, output; uint32_t tied_output, pad; } guffin_gemma3_binding;
+int guffin_gguf_bind_gemma3(const guffin_gguf* gguf, const guffin_gemma3_config* config, guffin_gemma3_binding* binding,
+                            guffin_gemma3_block* blocks);
+const char* guffin_gguf_bind_detail(void);
+
 /* ---- consecutive cycles ---------------------------------------------------------------------
  * Host-side lifecycle around guffin_hip_h1_step for generation over many cycles.  It keeps what
  * the reference keeps between cycles: the verify pass's transaction state (VerifierTransactionState,
