@@ -10,8 +10,9 @@
 // candidate order and keys are unique, so selection is a pure comparison network and the
 // result is exact including ties.
 //   stage 1  every workgroup sorts a 2048-logit tile in LDS (bitonic) and keeps its best R
-//   stage 2  one workgroup per row picks the best `retain` of the G*R survivors (radix select
-//            plus a rank sort), then appends the logits of the history tokens
+//   stage 2  one workgroup per row picks the best `retain` of the G*R survivors (a threshold from
+//            the sorted tile lists' heads plus a rank sort; a radix select where that does not
+//            apply), then appends the logits of the history tokens
 // A global top-R entry is necessarily a top-R entry of its own tile, so the two stages lose
 // nothing.
 #include "common.hpp"
@@ -96,9 +97,10 @@ __device__ __forceinline__ void hist_add(uint32_t* hist, bool valid, uint32_t bi
     if ((todo >> lane) & 1u) atomicAdd(&hist[bin], 1u);
 }
 
-// Stage 2: exact selection of the best `retain` of n unique keys by an 8-pass radix select
-// (one byte per pass, most significant first: a 256-bin histogram in LDS, then the bin that
-// holds the retain-th largest key), followed by a rank sort of the selected keys.
+// Stage 2: exact selection of the best `retain` of n unique keys.  Sorted tile lists take the
+// threshold shortcut below; otherwise an 8-pass radix select (one byte per pass, most significant
+// first: a 256-bin histogram in LDS, then the bin that holds the retain-th largest key).  Either
+// way a rank sort of the selected keys follows.
 template <int kMine>
 __global__ void __launch_bounds__(1024)
 topk_merge_kernel(const float* __restrict__ logits, const uint64_t* __restrict__ survivors, uint32_t n_survivors,
