@@ -119,19 +119,34 @@ draft_law_kernel(const Candidates* __restrict__ top, SamplerOptions opt, uint64_
     // full_error != nullptr: the full-vocabulary kernels follow, guarded by law->count; a support of
     // more than 256 ties then hands over to them instead of failing
     __shared__ uint64_t keys[256];
-    __shared__ float score[256], weight[256];
-    __shared__ uint32_t s_n;
+    __shared__ float score[256], weight[256], running[256];
+    __shared__ uint64_t edge[257];
+    __shared__ uint32_t s_n, s_first, s_bad, s_chosen;
     const uint32_t t = threadIdx.x;
     const uint32_t avail = top->count;
+    // every thread fetches its own entry once; the single-lane sections below work on LDS only
+    const bool usable = options_valid(opt) && opt.temperature > 0.f && opt.top_k <= 64 && avail >= 1;
+    const uint32_t k = usable ? (opt.top_k < avail ? opt.top_k : avail) : 1u;
+    const float cutoff = usable ? top->values[k - 1].logit : 0.f;
+    const float first_logit = usable ? top->values[0].logit : 0.f;
+    const float my_logit = t < avail ? top->values[t].logit : -INFINITY;
+    const uint32_t my_token = t < avail ? top->values[t].token : 0u;
+    if (t == 0) { s_first = 256u; s_bad = 0; s_chosen = 0xFFFFFFFFu; }
+    __syncthreads();
+    // entries are sorted by (score desc, token asc): the support is a prefix, its length the first
+    // entry that is below the cutoff or -inf
+    if (!(t < avail && !(my_logit < cutoff) && my_logit != -INFINITY)) atomicMin(&s_first, t);
+    __syncthreads();
     if (t == 0) {
         uint32_t st = 0, n = 0;
-        if (!options_valid(opt) || opt.temperature <= 0.f || opt.top_k > 64 || avail < 1) st = GUFFIN_STATUS_LAW_INVALID;
+        if (!usable) st = GUFFIN_STATUS_LAW_INVALID;
         if (top->status & GUFFIN_STATUS_NONFINITE) st = GUFFIN_STATUS_LAW_INVALID | GUFFIN_STATUS_NONFINITE;
         if (!st) {
-            const uint32_t k = opt.top_k < avail ? opt.top_k : avail;
-            const float cutoff = top->values[k - 1].logit;
-            // entries are sorted by (score desc, token asc): the support is a prefix
-            while (n < avail && !(top->values[n].logit < cutoff) && top->values[n].logit != -INFINITY) ++n;
+            n = s_first;
+            if (n == 256u && avail > 256u) {   // all 256 are in: a 257th eligible entry overflows the compact law
+                const float more = top->values[256].logit;
+                if (!(more < cutoff) && more != -INFINITY) n = 257u;
+            }
             if (n == 0) st = GUFFIN_STATUS_LAW_INVALID;  // nothing eligible
             if (n > 256) st = GUFFIN_STATUS_LAW_INVALID | 32u;  // support overflow: needs the full-vocabulary law
         }
@@ -143,24 +158,27 @@ draft_law_kernel(const Candidates* __restrict__ top, SamplerOptions opt, uint64_
     __syncthreads();
     const uint32_t n = s_n;
     if (n == 0) return;
-    score[t] = t < n ? top->values[t].logit : -INFINITY;
-    weight[t] = t < n ? law_exp(top->values[t].logit - top->values[0].logit) : 0.f;
+    score[t] = t < n ? my_logit : -INFINITY;
+    weight[t] = t < n ? law_exp(my_logit - first_logit) : 0.f;
     __syncthreads();
     if (t == 0) {  // descending-tail top-p / min-p in the reference's sequential order
         float total = 0.f, tail = 0.f;
         for (uint32_t j = n; j > 0; --j) total = __fadd_rn(total, weight[j - 1]);
         for (uint32_t j = n; j > 0; --j) {
-            const uint32_t i = j - 1;
-            tail = __fadd_rn(tail, weight[i]);
-            const bool keep = i == 0
-                || ((opt.top_p >= 1.0f || __fdiv_rn(tail, total) > __fsub_rn(1.0f, opt.top_p))
-                    && (opt.min_p <= 0.0f || weight[i] >= opt.min_p));
-            if (!keep) score[i] = -INFINITY;
+            tail = __fadd_rn(tail, weight[j - 1]);
+            running[j - 1] = tail;
         }
+        running[0] = total;   // slot 0 is always kept; it carries the total to the other lanes
+    }
+    __syncthreads();
+    if (t > 0 && t < n) {
+        const bool keep = (opt.top_p >= 1.0f || __fdiv_rn(running[t], running[0]) > __fsub_rn(1.0f, opt.top_p))
+                          && (opt.min_p <= 0.0f || weight[t] >= opt.min_p);
+        if (!keep) score[t] = -INFINITY;
     }
     __syncthreads();
     // ascending token id; the score rides in the low half of the key
-    keys[t] = t < n ? (uint64_t(top->values[t].token) << 32) | __float_as_uint(score[t]) : ~uint64_t{0};
+    keys[t] = t < n ? (uint64_t(my_token) << 32) | __float_as_uint(score[t]) : ~uint64_t{0};
     bitonic(keys, 256, false);
     const float s = __uint_as_float(static_cast<uint32_t>(keys[t]));
     score[t] = t < n ? s : -INFINITY;
@@ -175,30 +193,36 @@ draft_law_kernel(const Candidates* __restrict__ top, SamplerOptions opt, uint64_
     __syncthreads();
     weight[t] = t < n ? law_exp(__fsub_rn(score[t], maximum)) : 0.f;
     __syncthreads();
-    if (t == 0) {
-        float total = 0.f;
-        for (uint32_t i = 0; i < n; ++i) total = __fadd_rn(total, weight[i]);
-        uint32_t st = 0;
-        if (!(total > 0.f) || !isfinite(total)) st = GUFFIN_STATUS_LAW_INVALID;
-        const StepDraws d = injected ? *injected : step_draws(seed, step);
+    if (t == 0) {   // the f32 running sums in token order; the quotients and edges are per-lane work
         float prefix = 0.f;
-        uint64_t last = 0;
-        uint32_t chosen = 0xFFFFFFFFu;
+        for (uint32_t i = 0; i < n; ++i) { prefix = __fadd_rn(prefix, weight[i]); running[i] = prefix; }
+        edge[0] = 0;
+    }
+    __syncthreads();
+    const float total = running[n - 1];
+    const bool total_ok = total > 0.f && isfinite(total);
+    uint64_t next = 0;
+    if (t < n) {
+        float scaled = __fmul_rn(__fdiv_rn(running[t], total), 4294967296.0f);
+        scaled = fminf(fmaxf(scaled, 0.0f), 4294967296.0f);
+        next = static_cast<uint64_t>(scaled);
+        edge[t + 1] = next;
+    }
+    __syncthreads();
+    const StepDraws d = injected ? *injected : step_draws(seed, step);
+    if (t < n) {
+        const uint64_t last = edge[t];
+        if (next < last || next > kMassTotal || (t == n - 1 && next != kMassTotal)) s_bad = 1;
+        if (uint64_t(d.word) >= last && uint64_t(d.word) < next) s_chosen = static_cast<uint32_t>(keys[t] >> 32);
+        law->ids[t] = static_cast<uint32_t>(keys[t] >> 32);
+        law->cdf[t + 1] = next;
+    }
+    __syncthreads();
+    if (t == 0) {
         law->count = n; law->pad = 0; law->cdf[0] = 0;
-        for (uint32_t i = 0; i < n && !st; ++i) {
-            law->ids[i] = static_cast<uint32_t>(keys[i] >> 32);
-            prefix = __fadd_rn(prefix, weight[i]);
-            float scaled = __fmul_rn(__fdiv_rn(prefix, total), 4294967296.0f);
-            scaled = fminf(fmaxf(scaled, 0.0f), 4294967296.0f);
-            const uint64_t next = static_cast<uint64_t>(scaled);
-            law->cdf[i + 1] = next;
-            if (next < last || next > kMassTotal) st = GUFFIN_STATUS_LAW_INVALID;
-            if (uint64_t(d.word) >= last && uint64_t(d.word) < next) chosen = law->ids[i];
-            last = next;
-        }
-        if (!st && last != kMassTotal) st = GUFFIN_STATUS_LAW_INVALID;
-        if (st) { atomicOr(status, st); chosen = 0xFFFFFFFFu; }
-        *proposal = chosen;
+        const bool bad = !total_ok || s_bad;
+        if (bad) atomicOr(status, GUFFIN_STATUS_LAW_INVALID);
+        *proposal = bad ? 0xFFFFFFFFu : s_chosen;
     }
 }
 
@@ -425,10 +449,18 @@ struct Scratch {
     uint64_t keys[512];
     float logit[512];
     double w[kMaxTopK];
+    double run[kMaxTopK];            // running sums of w, taken by one lane in index order
+    uint32_t tok[kMaxCandidates];    // the candidate record, staged once
+    float raw[kMaxCandidates];
+    uint32_t hist[kHistoryCap];
+    uint32_t kept, cut;              // ends of the top-p and min-p prefixes
+    uint32_t flag;
+    double value;
     int err;
 };
 
-// returns 0 or a negative error; result in `out` (shared); uses all threads
+// returns 0 or a negative error; result in `out` (shared); uses all threads.  Sums whose order matters are
+// taken by one lane over LDS; divisions, comparisons and exponentials are spread over the lanes.
 __device__ int prepare_distribution(const Candidates* cand, const SamplerOptions& opt, const uint32_t* history,
                                     uint32_t history_count, Scratch& sc, Prepared& out) {
     const uint32_t t = threadIdx.x, n = cand->count;
@@ -436,34 +468,38 @@ __device__ int prepare_distribution(const Candidates* cand, const SamplerOptions
     __syncthreads();
     if (sc.err) return sc.err;
     const uint32_t request_top_k = opt.temperature == 0.f ? 1u : opt.top_k;
+    if (t < n) { sc.tok[t] = cand->values[t].token; sc.raw[t] = cand->values[t].logit; }
+    if (t < history_count) sc.hist[t] = history[t];
+    __syncthreads();
     // dedup (a later duplicate must carry the same logit), repetition penalty, sort key
     uint64_t key = 0;
     if (t < n) {
-        const uint32_t token = cand->values[t].token;
-        float logit = cand->values[t].logit;
+        const uint32_t token = sc.tok[t];
+        float logit = sc.raw[t];
         bool dup = false;
         if (!isfinite(logit)) atomicMin(&sc.err, -4);
         for (uint32_t j = 0; j < t; ++j)
-            if (cand->values[j].token == token) {
+            if (sc.tok[j] == token) {
                 dup = true;
-                if (cand->values[j].logit != logit) atomicMin(&sc.err, -5);
+                if (sc.raw[j] != logit) atomicMin(&sc.err, -5);
             }
         if (!dup) {
             for (uint32_t h = 0; h < history_count; ++h)
-                if (history[h] == token) {
+                if (sc.hist[h] == token) {
                     logit = logit < 0.f ? __fmul_rn(logit, opt.repetition_penalty) : __fdiv_rn(logit, opt.repetition_penalty);
                     break;
                 }
             key = score_key(logit, token);
-            sc.logit[t] = logit;
         }
     }
     if (t < 512) sc.keys[t] = key;
     __syncthreads();
     if (sc.err) return sc.err;
-    bitonic(sc.keys, 512, true);
+    uint32_t span = 64;   // the sort covers the record only (a real key is never 0, the padding is)
+    while (span < n) span <<= 1;
+    bitonic(sc.keys, span, true);
     // unique count = number of non-zero keys (a real key is never 0: ordered(logit) has a set bit)
-    uint32_t mine = (t < 512 && sc.keys[t] != 0) ? 1u : 0u;
+    uint32_t mine = (t < span && sc.keys[t] != 0) ? 1u : 0u;
     const uint32_t unique = __syncthreads_count(mine);
     if (unique < request_top_k) return -6;
     uint32_t count = unique < request_top_k ? unique : request_top_k;
@@ -483,29 +519,27 @@ __device__ int prepare_distribution(const Candidates* cand, const SamplerOptions
     if (t < count) sc.w[t] = exp(static_cast<double>(__fsub_rn(sc.logit[t], max_logit)));
     __syncthreads();
     if (t == 0) {
-        double total = 0.0;
-        for (uint32_t i = 0; i < count; ++i) total += sc.w[i];
-        double retained = 0.0;
-        uint32_t kept = 0;
-        do {
-            retained += sc.w[kept++];
-        } while (kept < count && retained / total < static_cast<double>(opt.top_p));
-        uint32_t c = kept;
-        if (opt.min_p > 0.f) {
-            uint32_t m = 1;
-            while (m < c && sc.w[m] >= static_cast<double>(opt.min_p)) ++m;
-            c = m;
-        }
-        out.count = c;
+        double running = 0.0;
+        for (uint32_t i = 0; i < count; ++i) { running += sc.w[i]; sc.run[i] = running; }
+        sc.kept = count; sc.cut = count;
     }
     __syncthreads();
-    count = out.count;
+    {
+        // top-p keeps entries up to and including the first whose running share reaches top_p; min-p then
+        // keeps the leading entries (the first always) whose weight is at least min_p
+        const double total = sc.run[count - 1];
+        if (t + 1 < count && !(sc.run[t] / total < static_cast<double>(opt.top_p))) atomicMin(&sc.kept, t + 1);
+        if (opt.min_p > 0.f && t >= 1 && t < count && !(sc.w[t] >= static_cast<double>(opt.min_p))) atomicMin(&sc.cut, t);
+    }
+    __syncthreads();
+    count = sc.kept < sc.cut ? sc.kept : sc.cut;
     if (t < count)
         out.weight[t] = exp(static_cast<double>(__fsub_rn(sc.logit[t], max_logit)) / static_cast<double>(opt.temperature));
     __syncthreads();
     if (t == 0) {
         double norm = 0.0;
         for (uint32_t i = 0; i < count; ++i) norm += out.weight[i];
+        out.count = count;
         out.total = norm;
         sc.err = (!isfinite(norm) || norm <= 0.0) ? -7 : 0;
     }
@@ -513,22 +547,40 @@ __device__ int prepare_distribution(const Candidates* cand, const SamplerOptions
     return sc.err;
 }
 
-// Neumaier-compensated total with the reference's consistency checks; one lane.
-__device__ double validated_total(const Prepared& p) {
-    if (p.count == 0 || p.count > kMaxTopK || !isfinite(p.total) || p.total <= 0.0) return -1.0;
-    double total = 0.0, correction = 0.0;
-    for (uint32_t i = 0; i < p.count; ++i) {
-        const double w = p.weight[i];
-        const double prob = w / p.total;  // the stored probability is exactly this quotient
-        if (!isfinite(prob) || prob < 0.0 || prob > 1.0 || !isfinite(w) || w < 0.0) return -1.0;
-        const double sum = total + w;
-        correction += total >= w ? (total - sum) + w : (w - sum) + total;
-        total = sum;
+// Neumaier-compensated total with the reference's consistency checks; all threads call it (the quotients
+// are checked per lane, the compensated sum is one lane's), every thread gets the result: -1 when invalid.
+__device__ double validated_total(const Prepared& p, Scratch& sc) {
+    const uint32_t t = threadIdx.x;
+    __syncthreads();
+    const uint32_t count = p.count;
+    const double stored = p.total;
+    const bool shape_ok = !(count == 0 || count > kMaxTopK || !isfinite(stored) || stored <= 0.0);
+    if (t == 0) sc.flag = 0;
+    __syncthreads();
+    if (shape_ok && t < count) {
+        const double w = p.weight[t];
+        const double prob = w / stored;  // the stored probability is exactly this quotient
+        if (!isfinite(prob) || prob < 0.0 || prob > 1.0 || !isfinite(w) || w < 0.0) sc.flag = 1;
     }
-    total += correction;
-    const double tol = static_cast<double>(p.count) * 2.220446049250313e-16 * total;
-    if (!isfinite(total) || total <= 0.0 || fabs(total - p.total) > tol) return -1.0;
-    return total;
+    __syncthreads();
+    if (t == 0) {
+        double result = -1.0;
+        if (shape_ok && !sc.flag) {
+            double total = 0.0, correction = 0.0;
+            for (uint32_t i = 0; i < count; ++i) {
+                const double w = p.weight[i];
+                const double sum = total + w;
+                correction += total >= w ? (total - sum) + w : (w - sum) + total;
+                total = sum;
+            }
+            total += correction;
+            const double tol = static_cast<double>(count) * 2.220446049250313e-16 * total;
+            if (isfinite(total) && total > 0.0 && !(fabs(total - stored) > tol)) result = total;
+        }
+        sc.value = result;
+    }
+    __syncthreads();
+    return sc.value;
 }
 
 __device__ uint32_t select_prepared(const Prepared& p, double draw) {
@@ -574,8 +626,10 @@ spec_accept_kernel(const Candidates* __restrict__ rows, const DraftLaw* __restri
     __shared__ Scratch sc;
     __shared__ Prepared target, residual;
     __shared__ uint64_t q[kMaxTopK];
+    __shared__ double diff[kMaxTopK];
+    __shared__ double s_proposed, s_acceptance;
     __shared__ int s_code;
-    __shared__ uint32_t s_accepted;
+    __shared__ uint32_t s_accepted, s_draw_residual;
     const uint32_t t = threadIdx.x;
     const uint32_t proposal = *proposal_ptr;
     const StepDraws d = injected ? *injected : step_draws(seed, step);
@@ -587,13 +641,13 @@ spec_accept_kernel(const Candidates* __restrict__ rows, const DraftLaw* __restri
     // history: [2][64] token ids and their counts per row (null: no repetition history)
     int rc = prepare_distribution(&rows[0], opt, history, history ? history_count[0] : 0u, sc, target);
     if (!rc && t < target.count) q[t] = law_mass(law, full_cdf, vocab, target.token[t], nullptr, target_to_draft);
+    const double normalization = rc ? -1.0 : validated_total(target, sc);
     __syncthreads();
     if (t == 0) {
         int code = rc;
         auto unit = [](double u) { return isfinite(u) && u >= 0.0 && u < 1.0; };
         if (!code && (!unit(d.u_accept) || !unit(d.u_residual) || !unit(d.u_next))) code = -20;
-        double normalization = 0.0;
-        if (!code) { normalization = validated_total(target); if (normalization < 0.0) code = -21; }
+        if (!code && normalization < 0.0) code = -21;
         uint64_t begin = 0, proposal_mass = 0;
         if (!code) {
             proposal_mass = law_mass(law, full_cdf, vocab, proposal, &begin, target_to_draft);
@@ -609,20 +663,32 @@ spec_accept_kernel(const Candidates* __restrict__ rows, const DraftLaw* __restri
             }
             if (!code && !in_target && proposal_mass > kMassTotal - gathered) code = -24;
         }
-        uint32_t accepted = 0;
-        if (!code) {
-            const double proposed = static_cast<double>(proposal_mass) / static_cast<double>(kMassTotal);
-            double acceptance = 0.0;
+        s_code = code;
+        s_accepted = 0;
+        s_draw_residual = 0;
+        s_acceptance = 0.0;
+        s_proposed = static_cast<double>(proposal_mass) / static_cast<double>(kMassTotal);
+    }
+    __syncthreads();
+    if (s_code == 0) {
+        // p, p / q of the proposal and p - q per lane; the residual's order and sum stay one lane's
+        if (t < target.count) {
+            const double p = target.weight[t] / normalization;
+            if (target.token[t] == proposal) s_acceptance = fmin(1.0, p / s_proposed);   // tokens are distinct
+            diff[t] = p - static_cast<double>(q[t]) / static_cast<double>(kMassTotal);
+        }
+        __syncthreads();
+        if (t == 0) {
+            int code = 0;
+            const double acceptance = s_acceptance;
             residual.count = 0; residual.total = 0.0;
             for (uint32_t i = 0; i < target.count; ++i) {
-                const double p = target.weight[i] / normalization;
-                if (target.token[i] == proposal) acceptance = fmin(1.0, p / proposed);
-                const double diff = p - static_cast<double>(q[i]) / static_cast<double>(kMassTotal);
-                if (diff <= 0.0) continue;
+                const double excess = diff[i];
+                if (excess <= 0.0) continue;
                 residual.token[residual.count] = target.token[i];
-                residual.weight[residual.count] = diff;
+                residual.weight[residual.count] = excess;
                 ++residual.count;
-                residual.total += diff;
+                residual.total += excess;
             }
             if (residual.count == 0 && acceptance < 1.0) code = -25;
             result->acceptance_probability = acceptance;
@@ -630,20 +696,28 @@ spec_accept_kernel(const Candidates* __restrict__ rows, const DraftLaw* __restri
             result->residual_count = residual.count;
             if (!code) {
                 if (d.u_accept < acceptance) {
-                    accepted = 1;
+                    s_accepted = 1;
                     result->accepted = 1; result->token = proposal; result->next_root = proposal;
-                } else if (validated_total(residual) < 0.0) {
-                    code = -26;
+                } else {
+                    s_draw_residual = 1;
+                }
+            }
+            s_code = code;
+        }
+        __syncthreads();
+        if (s_draw_residual) {
+            const double residual_total = validated_total(residual, sc);
+            if (t == 0) {
+                if (residual_total < 0.0) {
+                    s_code = -26;
                 } else {
                     const uint32_t tok = select_prepared(residual, d.u_residual * residual.total);
                     result->token = tok; result->next_root = tok;
                 }
             }
+            __syncthreads();
         }
-        s_code = code;
-        s_accepted = accepted;
     }
-    __syncthreads();
     if (s_code == 0 && s_accepted) {
         // a fully accepted chain leaves row 1's candidates to seed the next root
         rc = prepare_distribution(&rows[1], opt, history ? history + 64 : nullptr, history ? history_count[1] : 0u, sc, target);
