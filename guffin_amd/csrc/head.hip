@@ -97,6 +97,42 @@ __device__ __forceinline__ void hist_add(uint32_t* hist, bool valid, uint32_t bi
     if ((todo >> lane) & 1u) atomicAdd(&hist[bin], 1u);
 }
 
+// Writes one row of the result from its `retain` selected keys (candidate order) and appends the logits of
+// the row's history tokens; all threads of the workgroup call it after the keys are complete.
+__device__ void emit_candidates(const uint64_t* keys, uint32_t retain, uint32_t row, const float* __restrict__ logits,
+                                uint32_t vocab, float divisor, const uint32_t* __restrict__ history,
+                                const uint32_t* __restrict__ history_count, uint32_t row_stride, uint32_t history_stride,
+                                Candidates* __restrict__ result, uint32_t* __restrict__ status) {
+    __syncthreads();
+    Candidates& out = result[row];
+    const uint32_t hc = history_count ? history_count[size_t(row) * row_stride] : 0;
+    for (uint32_t i = threadIdx.x; i < retain; i += blockDim.x) {
+        const uint32_t token = key_token(keys[i]);
+        out.values[i].token = token;
+        out.values[i].logit = logits[size_t(row) * vocab + token] / divisor;  // the native value, not the key's
+    }
+    uint32_t st = 0;
+    for (uint32_t i = threadIdx.x; i < hc; i += blockDim.x) {
+        const uint32_t token = history[size_t(row) * history_stride + i];
+        if (token >= vocab) {
+            st |= GUFFIN_STATUS_BAD_TOKEN;
+            out.values[retain + i].token = 0xFFFFFFFFu;
+            out.values[retain + i].logit = -INFINITY;
+        } else {
+            const float v = logits[size_t(row) * vocab + token] / divisor;
+            if (!isfinite(v)) st |= GUFFIN_STATUS_NONFINITE;
+            out.values[retain + i].token = token;
+            out.values[retain + i].logit = v;
+        }
+    }
+    if (st && status) atomicOr(status + row, st);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        out.count = retain + hc;
+        out.status = status ? status[row] : 0;
+    }
+}
+
 // Stage 2: exact selection of the best `retain` of n unique keys.  Sorted tile lists take the
 // threshold shortcut below; otherwise an 8-pass radix select (one byte per pass, most significant
 // first: a 256-bin histogram in LDS, then the bin that holds the retain-th largest key).  Either
@@ -251,34 +287,205 @@ topk_merge_kernel(const float* __restrict__ logits, const uint64_t* __restrict__
             keys[rank] = k;
         }
     }
-    __syncthreads();
-    Candidates& out = result[row];
-    const uint32_t hc = history_count ? history_count[size_t(row) * row_stride] : 0;
-    for (uint32_t i = threadIdx.x; i < retain; i += blockDim.x) {
-        const uint32_t token = key_token(keys[i]);
-        out.values[i].token = token;
-        out.values[i].logit = logits[size_t(row) * vocab + token] / divisor;  // the native value, not the key's
-    }
-    uint32_t st = 0;
-    for (uint32_t i = threadIdx.x; i < hc; i += blockDim.x) {
-        const uint32_t token = history[size_t(row) * history_stride + i];
-        if (token >= vocab) {
-            st |= GUFFIN_STATUS_BAD_TOKEN;
-            out.values[retain + i].token = 0xFFFFFFFFu;
-            out.values[retain + i].logit = -INFINITY;
-        } else {
-            const float v = logits[size_t(row) * vocab + token] / divisor;
-            if (!isfinite(v)) st |= GUFFIN_STATUS_NONFINITE;
-            out.values[retain + i].token = token;
-            out.values[retain + i].logit = v;
+    emit_candidates(keys, retain, row, logits, vocab, divisor, history, history_count, row_stride, history_stride, result, status);
+}
+
+// ---- selection by threshold ------------------------------------------------------------------
+// For large vocabularies the sort of every tile is more work than the answer needs.  The maxima of the
+// 256-logit segments give a bound first: with at least `retain` segments, the retain-th largest segment
+// maximum is at or below the retain-th largest logit of the row, so only logits at or above it can be
+// selected, and on anything but massively tied rows they are few more than `retain`.  Two launches:
+//   segment_max_kernel       the ordered score bits of every segment's maximum; clears the row's counters
+//   threshold_select_kernel  every workgroup finds the bound for itself (a 4-pass radix select over at most
+//                            1024 words), collects the keys of its 4096 logits that reach it into the row's
+//                            list, and the workgroup that finishes last sorts the list and writes the row
+// The list and the counters move with device-scope accesses (the workgroups sit on different L2s), every
+// workgroup waits for its own stores before it counts itself done, and nobody waits for anybody: the last
+// arrival is whoever draws the last ticket.  A row whose list overflows (more than kCollectCap logits tie
+// into the bound) is selected exactly, and slowly, by a radix select over the whole row in that workgroup.
+constexpr uint32_t kSeg = 256, kMaxSegs = 1024, kCollectTile = 4096, kCollectCap = 2048;
+constexpr uint32_t kThresholdRowWords = kMaxSegs + 4 + 2 * kCollectCap;   // segment maxima, counter, done, pad, list
+
+__device__ __forceinline__ uint32_t ordered_bits(float v) {
+    const uint32_t b = __float_as_uint(v + 0.0f);
+    return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
+}
+
+__global__ void __launch_bounds__(256)
+segment_max_kernel(const float* __restrict__ logits, uint32_t vocab, uint32_t segs, float divisor, uint32_t* __restrict__ ws) {
+    const uint32_t row = blockIdx.y, lane = threadIdx.x & 63;
+    const uint32_t seg = blockIdx.x * 4 + (threadIdx.x >> 6);
+    uint32_t* row_ws = ws + size_t(row) * kThresholdRowWords;
+    if (blockIdx.x == 0 && threadIdx.x < 4) row_ws[kMaxSegs + threadIdx.x] = 0;
+    if (seg >= segs) return;
+    const float* lr = logits + size_t(row) * vocab;
+    uint32_t best = 0;
+#pragma unroll
+    for (uint32_t u = 0; u < kSeg / 64; ++u) {
+        const uint32_t t = seg * kSeg + u * 64 + lane;
+        if (t < vocab) {
+            const uint32_t o = ordered_bits(lr[t] / divisor);
+            best = o > best ? o : best;
         }
     }
-    if (st && status) atomicOr(status + row, st);
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        out.count = retain + hc;
-        out.status = status ? status[row] : 0;
+#pragma unroll
+    for (int sft = 32; sft > 0; sft >>= 1) {
+        const uint32_t o = __shfl_xor(best, sft, kWave);
+        best = o > best ? o : best;
     }
+    if (lane == 0) row_ws[seg] = best;
+}
+
+// the bin (highest first) that holds the `remaining`-th largest entry of a 256-bin histogram; first wave only
+__device__ __forceinline__ void find_bin(const uint32_t* hist, uint32_t remaining, uint32_t lane, uint32_t& s_bin,
+                                         uint32_t& s_above) {
+    uint32_t c[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) c[j] = hist[255 - 4 * lane - j];
+    const uint32_t own = c[0] + c[1] + c[2] + c[3];
+    uint32_t incl = own;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        const uint32_t o = __shfl_up(incl, d, kWave);
+        if (lane >= uint32_t(d)) incl += o;
+    }
+    uint32_t above = incl - own;
+    if (above < remaining && remaining <= incl) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            if (remaining <= above + c[j]) { s_bin = 255 - 4 * lane - j; s_above = above; break; }
+            above += c[j];
+        }
+    }
+}
+
+__global__ void __launch_bounds__(1024)
+threshold_select_kernel(const float* __restrict__ logits, uint32_t vocab, uint32_t segs, uint32_t retain_cap, float divisor,
+                        const uint32_t* __restrict__ history, const uint32_t* __restrict__ history_count,
+                        const uint32_t* __restrict__ row_retain, uint32_t row_stride, uint32_t history_stride,
+                        uint32_t* __restrict__ ws, Candidates* __restrict__ result, uint32_t* __restrict__ status,
+                        bool suppressed_ok) {
+    __shared__ uint32_t hist[256];
+    __shared__ uint64_t sel[kCollectCap];
+    __shared__ uint64_t keys[512];
+    __shared__ uint32_t s_bin, s_above, s_last, s_count;
+    const uint32_t row = blockIdx.y, tid = threadIdx.x, lane = tid & 63;
+    uint32_t retain = retain_cap;
+    if (row_retain) {
+        const uint32_t want = row_retain[size_t(row) * row_stride];
+        retain = want < 1 ? 1 : (want < retain_cap ? want : retain_cap);
+    }
+    uint32_t* row_ws = ws + size_t(row) * kThresholdRowWords;
+    uint32_t* counter = row_ws + kMaxSegs;
+    uint32_t* done = counter + 1;
+    uint64_t* list = reinterpret_cast<uint64_t*>(row_ws + kMaxSegs + 4);
+    const float* lr = logits + size_t(row) * vocab;
+    // this workgroup's logits are requested before the bound is worked out
+    float mine[kCollectTile / 1024];
+#pragma unroll
+    for (uint32_t u = 0; u < kCollectTile / 1024; ++u) {
+        const uint32_t t = blockIdx.x * kCollectTile + u * 1024 + tid;
+        mine[u] = t < vocab ? lr[t] : 0.f;
+    }
+    // ---- the bound: the retain-th largest segment maximum (segs >= retain by the launch's condition) ----
+    const uint32_t word = tid < segs ? row_ws[tid] : 0u;
+    uint32_t prefix = 0, remaining = retain;
+    for (int pass = 0; pass < 4; ++pass) {
+        const int shift = 24 - 8 * pass;
+        if (tid < 256) hist[tid] = 0;
+        __syncthreads();
+        hist_add(hist, tid < segs && (pass == 0 || (word >> (shift + 8)) == prefix), (word >> shift) & 255u, lane);
+        __syncthreads();
+        if (tid < 64) find_bin(hist, remaining, lane, s_bin, s_above);
+        __syncthreads();
+        prefix = (prefix << 8) | s_bin;
+        remaining -= s_above;
+    }
+    const uint32_t bound = prefix;
+    // ---- collect ----------------------------------------------------------------------------------
+    bool bad = false;
+#pragma unroll
+    for (uint32_t u = 0; u < kCollectTile / 1024; ++u) {
+        const uint32_t t = blockIdx.x * kCollectTile + u * 1024 + tid;
+        bool hit = false;
+        uint64_t key = 0;
+        if (t < vocab) {
+            const float v = mine[u] / divisor;
+            bad |= (!isfinite(v) || !isfinite(mine[u])) && !(suppressed_ok && mine[u] == -INFINITY);
+            key = make_key(v, t);
+            hit = static_cast<uint32_t>(key >> 32) >= bound;
+        }
+        const uint64_t mask = __ballot(hit);
+        if (mask) {
+            const int leader = __ffsll(static_cast<long long>(mask)) - 1;
+            uint32_t base = 0;
+            if (lane == uint32_t(leader))
+                base = __hip_atomic_fetch_add(counter, static_cast<uint32_t>(__popcll(mask)), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            base = __shfl(base, leader, kWave);
+            const uint32_t at = base + static_cast<uint32_t>(__popcll(mask & ((uint64_t{1} << lane) - 1)));
+            if (hit && at < kCollectCap) __hip_atomic_store(list + at, key, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+    if (bad && status) atomicOr(status + row, GUFFIN_STATUS_NONFINITE);
+    // ---- the last workgroup of the row to get here finishes it -----------------------------------------
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    if (tid == 0) {
+        const uint32_t before = __hip_atomic_fetch_add(done, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        s_last = before + 1 == gridDim.x;
+        s_count = 0;
+    }
+    __syncthreads();
+    if (!s_last) return;
+    const uint32_t n = __hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (n <= kCollectCap) {
+        for (uint32_t i = tid; i < n; i += blockDim.x) sel[i] = __hip_atomic_load(list + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (n <= 512) {
+            __syncthreads();
+            for (uint32_t i = tid; i < n; i += blockDim.x) {
+                const uint64_t k = sel[i];
+                uint32_t rank = 0;
+                for (uint32_t j = 0; j < n; ++j) rank += sel[j] > k;
+                if (rank < retain) keys[rank] = k;
+            }
+        } else {
+            for (uint32_t i = n + tid; i < kCollectCap; i += blockDim.x) sel[i] = 0;
+            bitonic_desc(sel, kCollectCap);
+            for (uint32_t i = tid; i < retain; i += blockDim.x) keys[i] = sel[i];
+        }
+    } else {
+        // more ties than the list holds: an 8-pass radix select over the whole row's keys, exact and slow
+        uint64_t kprefix = 0;
+        uint32_t left = retain;
+        for (int pass = 0; pass < 8; ++pass) {
+            const int shift = 56 - 8 * pass;
+            if (tid < 256) hist[tid] = 0;
+            __syncthreads();
+            for (uint32_t i0 = 0; i0 < vocab; i0 += blockDim.x) {   // whole waves stay converged
+                const uint32_t i = i0 + tid;
+                const uint64_t k = i < vocab ? make_key(lr[i] / divisor, i) : 0;
+                hist_add(hist, i < vocab && (pass == 0 || (k >> (shift + 8)) == kprefix), static_cast<uint32_t>(k >> shift) & 255u, lane);
+            }
+            __syncthreads();
+            if (tid < 64) find_bin(hist, left, lane, s_bin, s_above);
+            __syncthreads();
+            kprefix = (kprefix << 8) | s_bin;
+            left -= s_above;
+        }
+        // kprefix is the retain-th largest key (keys are unique): everything above it, then it
+        for (uint32_t i = tid; i < vocab; i += blockDim.x) {
+            const uint64_t k = make_key(lr[i] / divisor, i);
+            if (k >= kprefix) sel[atomicAdd(&s_count, 1u)] = k;
+        }
+        __syncthreads();
+        for (uint32_t i = tid; i < retain; i += blockDim.x) {
+            const uint64_t k = sel[i];
+            uint32_t rank = 0;
+            for (uint32_t j = 0; j < retain; ++j) rank += sel[j] > k;
+            keys[rank] = k;
+        }
+    }
+    emit_candidates(keys, retain, row, logits, vocab, divisor, history, history_count, row_stride, history_stride, result, status);
 }
 
 // ---- verify-row input validation --------------------------------------------------------------
@@ -375,7 +582,8 @@ using namespace guffin;
 extern "C" uint64_t guffin_hip_select_workspace_bytes(uint32_t rows, uint32_t vocab, uint32_t retain) {
     const uint64_t tiles = (uint64_t(vocab) + kTile - 1) / kTile;
     const uint64_t keep = retain < kTile ? retain : kTile;
-    return rows * tiles * keep * 8;
+    const uint64_t sorted_tiles = rows * tiles * keep * 8, by_threshold = uint64_t(rows) * kThresholdRowWords * 4;
+    return sorted_tiles > by_threshold ? sorted_tiles : by_threshold;   // either path may serve the call
 }
 
 namespace guffin {
@@ -403,6 +611,16 @@ int guffin::select_candidates_scaled(hipStream_t s, const float* logits, uint32_
     if (reinterpret_cast<uintptr_t>(workspace) & 7u) return fail(GUFFIN_E_ALIGN, "select_candidates: workspace must be 8-byte aligned");
     const uint32_t keep = retain < vocab ? retain : vocab;
     const uint32_t tiles = (vocab + kTile - 1) / kTile;
+    const uint32_t segs = (vocab + kSeg - 1) / kSeg;
+    if (segs <= kMaxSegs && segs >= 2 * keep) {   // large vocabulary: a bound from the segment maxima, then one pass
+        uint32_t* words = static_cast<uint32_t*>(workspace);
+        hipLaunchKernelGGL(segment_max_kernel, dim3((segs + 3) / 4, rows), dim3(256), 0, s, logits, vocab, segs, divisor, words);
+        if (int rc = check_launch("select_candidates(segment maxima)")) return rc;
+        hipLaunchKernelGGL(threshold_select_kernel, dim3((vocab + kCollectTile - 1) / kCollectTile, rows), dim3(1024), 0, s,
+                           logits, vocab, segs, keep, divisor, history, history_count, row_retain, row_stride,
+                           row_stride == 1 ? 64u : row_stride, words, static_cast<Candidates*>(result), status, suppressed_ok);
+        return check_launch("select_candidates(threshold)");
+    }
     uint64_t* surv = static_cast<uint64_t*>(workspace);
     hipLaunchKernelGGL(topk_tile_kernel, dim3(tiles, rows), dim3(1024), 0, s, logits, surv, vocab, keep, divisor, status, suppressed_ok);
     if (int rc = check_launch("select_candidates(tile)")) return rc;

@@ -747,9 +747,8 @@ int select_candidates_scaled(hipStream_t s, const float* logits, uint32_t rows, 
 using namespace guffin;
 
 extern "C" uint64_t guffin_hip_draft_law_workspace_bytes(uint32_t vocab) {
-    // survivors of the 257-best selection plus the sorted candidate row
-    const uint64_t tiles = (uint64_t(vocab) + 2047) / 2048;
-    return tiles * 257 * 8 + sizeof(Candidates) + 16;
+    // workspace of the 257-best selection plus the sorted candidate row
+    return ((guffin_hip_select_workspace_bytes(1, vocab, 257) + 15) & ~uint64_t{15}) + sizeof(Candidates) + 16;
 }
 
 namespace {
@@ -785,9 +784,8 @@ bool compact_options(const SamplerOptions& o) { return o.temperature > 0.f && o.
 int launch_compact_law(hipStream_t s, const float* logits, uint32_t vocab, const SamplerOptions& opt, uint64_t seed,
                        uint64_t step, const void* injected_draws, void* workspace, void* law, uint32_t* proposal,
                        uint32_t* status, uint32_t* full_error, bool suppressed_ok = false) {
-    const uint64_t tiles = (uint64_t(vocab) + 2047) / 2048;
     uint8_t* ws = static_cast<uint8_t*>(workspace);
-    Candidates* top = reinterpret_cast<Candidates*>(ws + ((tiles * 257 * 8 + 15) & ~uint64_t{15}));
+    Candidates* top = reinterpret_cast<Candidates*>(ws + ((guffin_hip_select_workspace_bytes(1, vocab, 257) + 15) & ~uint64_t{15}));
     // the k-th best score and every tie with it: the best 257 scores decide both
     if (int rc = select_candidates_scaled(s, logits, 1, vocab, vocab < 257 ? vocab : 257, opt.temperature, nullptr,
                                           nullptr, ws, top, status, suppressed_ok))

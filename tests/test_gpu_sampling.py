@@ -69,11 +69,68 @@ def test_selection_matches_oracle_on_full_vocabulary(hip, gfo, retain):
     assert [int(t) for t in tok] == [gfo.lib().gfo_argmax(logits[r].ctypes, VOCAB) for r in range(2)]
 
 
+@pytest.mark.parametrize("vocab,retain,shape", [
+    (VOCAB, 64, "uniform"),          # every logit ties: the collected list overflows, the whole-row select decides
+    (VOCAB, 64, "plateau1500"),      # 1500 logits tie at the top: the list is sorted as a whole
+    (VOCAB, 257, "plateau1500"),
+    (200003, 64, "normal"),          # a ragged last segment and a ragged last tile
+    (200003, 100, "clustered"),      # the best logits sit in a few segments: the bound is loose
+    (131072, 256, "normal"),         # exactly twice as many segments as kept entries
+    (65536, 128, "normal"),
+    (65536, 129, "normal"),          # one entry too many for the bound: sorted tiles serve the call
+])
+def test_selection_paths_of_large_vocabularies(hip, gfo, vocab, retain, shape):
+    rng = np.random.default_rng(vocab + retain)
+    logits = rng.normal(0, 3, (2, vocab)).astype(np.float32)
+    if shape == "uniform":
+        logits[0, :] = 1.25
+        logits[1, :] = -0.0
+        logits[1, ::2] = 0.0          # both zeros order as one value, ties go to the lower id
+    elif shape == "plateau1500":
+        logits[0, rng.choice(vocab, 1500, replace=False)] = 40.0
+        logits[1, 1000:2500] = 40.0
+    elif shape == "clustered":
+        logits[0, 5000:5600] += 30.0
+        logits[1, vocab - 700:] += 30.0
+    res, status = hip.select_candidates(dev(logits), retain)
+    c = hip.candidates_to_numpy(res)
+    assert int(status[0]) == 0 and int(status[1]) == 0
+    for row in range(2):
+        want = gfo.select_candidates(logits[row], retain)
+        assert c[row]["count"] == retain
+        assert np.array_equal(c[row]["values"]["token"][:retain], want["token"])
+        assert np.array_equal(c[row]["values"]["logit"][:retain].view(np.uint32), want["logit"].view(np.uint32))
+
+
+def test_selection_of_a_large_vocabulary_with_histories_and_row_counts(hip, gfo):
+    """Rows that keep different numbers of entries and append their own history tokens' logits, twice in a
+    row on one workspace-sized call each (the counters of the first call must not leak into the second)."""
+    rng = np.random.default_rng(77)
+    for trial in range(2):
+        logits = rng.normal(0, 2, (2, VOCAB)).astype(np.float32)
+        hist = np.zeros((2, 64), np.uint32)
+        counts = np.array([5, 64], np.uint32)
+        hist[0, :5] = rng.integers(0, VOCAB, 5)
+        hist[1] = rng.integers(0, VOCAB, 64)
+        res, status = hip.select_candidates(dev(logits), 64 + trial, history=dev(hist), history_count=dev(counts))
+        c = hip.candidates_to_numpy(res)
+        for row in range(2):
+            want = gfo.select_candidates(logits[row], 64 + trial, hist[row, :counts[row]])
+            n = 64 + trial + int(counts[row])
+            assert c[row]["count"] == n and int(status[row]) == 0
+            assert np.array_equal(c[row]["values"]["token"][:n], want["token"])
+            assert np.array_equal(c[row]["values"]["logit"][:n].view(np.uint32), want["logit"].view(np.uint32))
+
+
 def test_selection_flags_non_finite_logits(hip):
     logits = np.zeros((2, 4096), np.float32)
     logits[1, 77] = np.inf
     _, status = hip.select_candidates(dev(logits), 8)
     assert int(status[0]) == 0 and int(status[1]) & 2
+    logits = np.zeros((2, VOCAB), np.float32)
+    logits[0, VOCAB - 1] = np.nan
+    _, status = hip.select_candidates(dev(logits), 8)
+    assert int(status[0]) & 2 and int(status[1]) == 0
 
 
 def law_np(hip, law):
