@@ -179,7 +179,9 @@ draft_law_kernel(const Candidates* __restrict__ top, SamplerOptions opt, uint64_
     __syncthreads();
     // ascending token id; the score rides in the low half of the key
     keys[t] = t < n ? (uint64_t(my_token) << 32) | __float_as_uint(score[t]) : ~uint64_t{0};
-    bitonic(keys, 256, false);
+    uint32_t span = 64;   // entries beyond the support are all-ones keys already in their final place
+    while (span < n) span <<= 1;
+    bitonic(keys, span, false);
     const float s = __uint_as_float(static_cast<uint32_t>(keys[t]));
     score[t] = t < n ? s : -INFINITY;
     __syncthreads();
@@ -595,26 +597,30 @@ __device__ uint32_t select_prepared(const Prepared& p, double draw) {
 // target_to_draft: null when both sides share one vocabulary; else the law lives in draft ids and a
 // target token's mass is that of the draft token mapped to it, if any (Gemma3DraftPlan::gather,
 // src/engine/gemma3_draft.mm:1570-1578)
-__device__ uint64_t law_mass(const DraftLaw* law, const uint64_t* full_cdf, uint32_t vocab, uint32_t token,
+// The compact law as the acceptance kernel keeps it in LDS (ids ascending, cdf[i] .. cdf[i + 1] the mass of ids[i]).
+struct LawCopy { uint32_t count; uint32_t ids[256]; uint64_t cdf[257]; };
+
+__device__ uint64_t law_mass(const LawCopy& law, const uint64_t* full_cdf, uint32_t vocab, uint32_t token,
                              uint64_t* begin, const int32_t* target_to_draft = nullptr) {
     if (target_to_draft) {
         const int32_t draft = target_to_draft[token];
         if (draft < 0) { if (begin) *begin = 0; return 0; }
         token = static_cast<uint32_t>(draft);
     }
-    if (law->count == kLawFull) {  // gather from the full table (src/engine/gemma3_draft.mm:1544-1545)
+    if (law.count == kLawFull) {  // gather from the full table (src/engine/gemma3_draft.mm:1544-1545)
         if (!full_cdf || token >= vocab) { if (begin) *begin = 0; return 0; }
         if (begin) *begin = full_cdf[token];
         return full_cdf[token + 1] - full_cdf[token];
     }
-    uint32_t lo = 0, hi = law->count;
+    const uint32_t count = law.count < 256u ? law.count : 256u;
+    uint32_t lo = 0, hi = count;
     while (lo < hi) {
         const uint32_t mid = (lo + hi) >> 1;
-        if (law->ids[mid] < token) lo = mid + 1; else hi = mid;
+        if (law.ids[mid] < token) lo = mid + 1; else hi = mid;
     }
-    if (lo == law->count || law->ids[lo] != token) { if (begin) *begin = 0; return 0; }
-    if (begin) *begin = law->cdf[lo];
-    return law->cdf[lo + 1] - law->cdf[lo];
+    if (lo == count || law.ids[lo] != token) { if (begin) *begin = 0; return 0; }
+    if (begin) *begin = law.cdf[lo];
+    return law.cdf[lo + 1] - law.cdf[lo];
 }
 
 __global__ void __launch_bounds__(512)
@@ -630,9 +636,14 @@ spec_accept_kernel(const Candidates* __restrict__ rows, const DraftLaw* __restri
     __shared__ double s_proposed, s_acceptance;
     __shared__ int s_code;
     __shared__ uint32_t s_accepted, s_draw_residual;
+    __shared__ LawCopy q_law;
     const uint32_t t = threadIdx.x;
     const uint32_t proposal = *proposal_ptr;
     const StepDraws d = injected ? *injected : step_draws(seed, step);
+    // the compact law comes in once, every word by its own lane (the record is always whole in memory):
+    // the gathers below search it in LDS instead of through a chain of dependent trips to memory
+    if (t < 256) { q_law.ids[t] = law->ids[t]; q_law.cdf[t] = law->cdf[t]; }
+    if (t == 256) { q_law.cdf[256] = law->cdf[256]; q_law.count = law->count; }
     if (t == 0) {
         result->accepted = 0; result->token = 0xFFFFFFFFu; result->next_root = 0xFFFFFFFFu; result->status = 0;
         result->acceptance_probability = 0.0; result->residual_total = 0.0; result->residual_count = 0;
@@ -640,7 +651,7 @@ spec_accept_kernel(const Candidates* __restrict__ rows, const DraftLaw* __restri
     }
     // history: [2][64] token ids and their counts per row (null: no repetition history)
     int rc = prepare_distribution(&rows[0], opt, history, history ? history_count[0] : 0u, sc, target);
-    if (!rc && t < target.count) q[t] = law_mass(law, full_cdf, vocab, target.token[t], nullptr, target_to_draft);
+    if (!rc && t < target.count) q[t] = law_mass(q_law, full_cdf, vocab, target.token[t], nullptr, target_to_draft);
     const double normalization = rc ? -1.0 : validated_total(target, sc);
     __syncthreads();
     if (t == 0) {
@@ -650,7 +661,7 @@ spec_accept_kernel(const Candidates* __restrict__ rows, const DraftLaw* __restri
         if (!code && normalization < 0.0) code = -21;
         uint64_t begin = 0, proposal_mass = 0;
         if (!code) {
-            proposal_mass = law_mass(law, full_cdf, vocab, proposal, &begin, target_to_draft);
+            proposal_mass = law_mass(q_law, full_cdf, vocab, proposal, &begin, target_to_draft);
             if (proposal_mass == 0 || proposal_mass > kMassTotal || begin > kMassTotal - proposal_mass) code = -22;
         }
         bool in_target = false;
