@@ -331,6 +331,48 @@ __device__ __forceinline__ void run_blocks_at(const uint8_t* __restrict__ tiles,
     }
 }
 
+// The first two Q8_0 tiles of a wave's run, requested ahead of time (before a wait that the operand needs
+// and the weights do not), and the run itself starting from them.
+struct Q8Ahead { Q8Tile t[2]; };
+
+__device__ __forceinline__ void load_ahead(Q8Ahead& ahead, const uint8_t* __restrict__ tiles, uint32_t count, uint32_t lane) {
+    constexpr uint32_t TB = kTileCols * block_bytes(GUFFIN_Q8_0);
+    const uint8_t* tp = tiles + lane * 16;
+    ahead.t[0] = Q8Tile{};
+    ahead.t[1] = Q8Tile{};
+    if (count > 0) load_tile(ahead.t[0], tp, lane);
+    if (count > 1) load_tile(ahead.t[1], tp + TB, lane);
+}
+
+template <int R>
+__device__ __forceinline__ void run_blocks_ahead(const Q8Ahead& ahead, const uint8_t* __restrict__ tiles,
+                                                 const float* __restrict__ xsums, uint32_t K, uint32_t ob0, uint32_t count,
+                                                 float (&acc)[R], uint32_t lane = threadIdx.x & 63) {
+    constexpr uint32_t TB = kTileCols * block_bytes(GUFFIN_Q8_0);
+    const uint32_t n16 = K / 16, per_row = n16 + K / 32;
+    const float* xs = xsums + n16;
+    const uint8_t* tp = tiles + lane * 16;
+#pragma unroll
+    for (int r = 0; r < R; ++r) acc[r] = 0.f;
+    const ReceiptLayout L = receipt_layout(R, K);
+    const uint8_t* blob = reinterpret_cast<const uint8_t*>(xsums);
+    const float* mult = reinterpret_cast<const float*>(blob + L.mult_off);
+    const uint8_t* image = blob + L.image_off + (lane & 3u) * 64u + (lane >> 4) * 16u;
+    const uint32_t ob1 = ob0 + count;
+    auto operand = [&](uint32_t b) { return __builtin_bit_cast(half8_t, *reinterpret_cast<const uint4*>(image + size_t(b) * 256u)); };
+    Q8Tile cur = ahead.t[0], nxt = ahead.t[1], far = Q8Tile{};
+    half8_t a = {}, an = {};
+    if (count) a = operand(ob0);
+    for (uint32_t b = ob0; b < ob1; ++b) {
+        if (b + 1 < ob1) an = operand(b + 1);
+        if (b + 2 < ob1) load_tile(far, tp + size_t(b + 2 - ob0) * TB, lane);
+        compute_tile<R>(cur, a, mult + b, K / 32, xs + b, per_row, lane >> 4, acc);
+        cur = nxt;
+        nxt = far;
+        a = an;
+    }
+}
+
 // One wave: blocks [b0, b1) of column tile `ct` of a whole matrix whose operand is the receipt of its K inputs.
 template <int DTYPE, int R, bool SINGLE = false>
 __device__ __forceinline__ void run_blocks(const uint8_t* __restrict__ wt, const float* __restrict__ x,

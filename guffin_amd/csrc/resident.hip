@@ -191,12 +191,16 @@ __device__ __forceinline__ uint32_t tile_bytes(uint32_t dtype) { return kTileCol
 
 // One wave's run of blocks against the operand receipt at the start of the dynamic LDS.
 // KQ: 256-element formats (Q4_K or Q6_K by the matrix's dtype), else Q8_0.
-template <bool KQ, int R>
+template <bool KQ, int R, bool AHEAD = false>
 __device__ __forceinline__ void wave_blocks(const Ctx& c, uint32_t dtype, const uint8_t* tiles, uint32_t K, uint32_t ob0,
-                                            uint32_t count, float (&acc)[R]) {
+                                            uint32_t count, float (&acc)[R], const Q8Ahead& ahead = Q8Ahead{}) {
     const uint32_t lane = c.tid & 63;
     extern __shared__ __attribute__((aligned(256))) uint8_t dyn[];
     const float* opnd = reinterpret_cast<const float*>(dyn);
+    if constexpr (!KQ && AHEAD) {
+        run_blocks_ahead<R>(ahead, tiles, opnd, K, ob0, count, acc, lane);
+        return;
+    }
     if constexpr (KQ) {
         if (dtype == GUFFIN_Q4_K) {
             run_blocks_at<GUFFIN_Q4_K, R>(tiles, opnd, K, ob0, count, acc, lane);
@@ -272,13 +276,22 @@ __device__ __forceinline__ WaveRun ksplit_wave(const Ctx& c, const KSplit ks, ui
     return {tile, wb0, cnt};
 }
 
+// The first tiles of this wave's run in a K-split projection, requested ahead of the wait before it.
+__device__ __forceinline__ void ksplit_ahead(const Ctx& c, Q8Ahead& ahead, const uint8_t* tiles, uint32_t dtype, uint32_t ntiles,
+                                             uint32_t nblk_total, uint32_t first_block, uint32_t nbp, const KSplit ks,
+                                             uint32_t tg, bool active) {
+    const WaveRun wr = ksplit_wave(c, ks, tg, ntiles, nbp, active);
+    const uint8_t* tp = tiles + (size_t(wr.cnt ? wr.tile : 0u) * nblk_total + first_block + wr.wb0) * tile_bytes(dtype);
+    load_ahead(ahead, tp, wr.cnt, c.tid & 63);
+}
+
 // Projection of the LDS operand (R rows of `count` inputs, blocks relative to the part) with the part's
 // column tiles; partial plane `plane` of `out` ([planes][R][N]) receives the sums.
-template <bool KQ, int R>
+template <bool KQ, int R, bool AHEAD = false>
 __device__ __forceinline__ void ksplit_project(Ctx& c, const uint8_t* tiles, uint32_t dtype, uint32_t ntiles,
                                                uint32_t nblk_total, uint32_t first_block, uint32_t nbp, uint32_t Kp,
                                                const KSplit ks, uint32_t tg, bool active, float* out, uint32_t plane,
-                                               uint32_t N) {
+                                               uint32_t N, const Q8Ahead& ahead = Q8Ahead{}) {
     const uint32_t wave = __builtin_amdgcn_readfirstlane(c.tid >> 6), lane = c.tid & 63;
     const uint32_t wpt = kWaves / ks.tpw;
     const WaveRun wr = ksplit_wave(c, ks, tg, ntiles, nbp, active);
@@ -286,7 +299,7 @@ __device__ __forceinline__ void ksplit_project(Ctx& c, const uint8_t* tiles, uin
     float acc[R];
     if (cnt > 0) {
         const uint8_t* tp = tiles + (size_t(tile) * nblk_total + first_block + wb0) * tile_bytes(dtype);
-        wave_blocks<KQ, R>(c, dtype, tp, Kp, wb0, cnt, acc);
+        wave_blocks<KQ, R, AHEAD>(c, dtype, tp, Kp, wb0, cnt, acc, ahead);
     } else {
 #pragma unroll
         for (int r = 0; r < R; ++r) acc[r] = 0.f;
@@ -789,6 +802,13 @@ __global__ void __launch_bounds__(kThreads) resident_blocks_kernel(const RArgs a
         return LL.tiles[m] + (size_t(ct) * nbH + g_wb0) * tile_bytes(dtype_of(LL, m));
     };
 
+    // Q8_0 models: the first two tiles of a wave's next run of blocks are requested before the wait that
+    // precedes the run (the weights do not depend on the pass) and held in registers across it, so that the
+    // trip to memory overlaps the hand-over instead of following it.  The 256-element formats' tiles are
+    // too large to hold across the norms.
+    Q8Ahead ahead = {};
+    if constexpr (!KQ) load_ahead(ahead, q_tiles(a.layer[0]), q_cnt, lane);
+
     for (uint32_t l = 0; l < a.layers; ++l) {
         const RLayer& L = a.layer[l];
         stamp(c, l, 0);
@@ -797,7 +817,7 @@ __global__ void __launch_bounds__(kThreads) resident_blocks_kernel(const RArgs a
             const uint32_t dtype = dtype_of(L, qm);
             float acc[R];
             if (q_cnt > 0) {
-                wave_blocks<KQ, R>(c, dtype, q_tiles(L), H, qb0 + q_wb0, q_cnt, acc);
+                wave_blocks<KQ, R, !KQ>(c, dtype, q_tiles(L), H, qb0 + q_wb0, q_cnt, acc, ahead);
             } else {
 #pragma unroll
                 for (int r = 0; r < R; ++r) acc[r] = 0.f;
@@ -812,7 +832,13 @@ __global__ void __launch_bounds__(kThreads) resident_blocks_kernel(const RArgs a
                 a.qkv_part[((size_t(c.x) * PA + qkp) * R + r) * CW + qt * 64 + lane] = s;
             }
         }
-        xcd_barrier(c);
+        if constexpr (!KQ) {   // the o-projection's tiles travel while attention runs
+            __builtin_amdgcn_s_waitcnt(0);
+            ksplit_ahead(c, ahead, L.tiles[3], dtype_of(L, 3), H / 64, o_nblk, o_first, onbp, oks, otg, o_active);
+            xcd_barrier(c, true);
+        } else {
+            xcd_barrier(c);
+        }
         stamp(c, l, 1);
         // ---- attention over this workgroup's partition of the tokens ------------------------------
         attention_partition<R, G>(c, L, PA);
@@ -828,12 +854,16 @@ __global__ void __launch_bounds__(kThreads) resident_blocks_kernel(const RArgs a
                 for (int r = 0; r < R; ++r) emit_receipt(vals + size_t(r) * onbp * BE, 0, onbp * BE, r, R, Kp, dyn, c.tid, kThreads);
             }
             __syncthreads();
-            ksplit_project<KQ, R>(c, L.tiles[3], dtype_of(L, 3), H / 64, o_nblk, o_first, onbp, Kp, oks, otg, o_active,
-                                  a.o_planes, c.x * oks.kparts + okp, H);
+            ksplit_project<KQ, R, !KQ>(c, L.tiles[3], dtype_of(L, 3), H / 64, o_nblk, o_first, onbp, Kp, oks, otg, o_active,
+                                       a.o_planes, c.x * oks.kparts + okp, H, ahead);
         }
         stamp(c, l, 3);
+        if constexpr (!KQ) {   // this workgroup's first gate / up tiles
+            __builtin_amdgcn_s_waitcnt(0);
+            load_ahead(ahead, g_tiles(L, fs.tile0 + (c.slot < fs.tiles ? c.slot : 0u)), g_cnt, lane);
+        }
         // ---- x1 = x + rms(o, post_attention_norm); u = rms(x1, ffn_norm) -------------------------------
-        norm_pair<R>(c, a.o_planes, c.X * oks.kparts, L.norm[3], L.norm[4], xr, false, false, l, 8);
+        norm_pair<R>(c, a.o_planes, c.X * oks.kparts, L.norm[3], L.norm[4], xr, false, !KQ, l, 8);
         stamp(c, l, 4);
         // ---- gate and up columns of this XCD's slice of the FFN width, GeGLU, its receipt --------------
         for (uint32_t pair = c.slot; pair < fs.tiles; pair += kGroups) {
@@ -841,7 +871,8 @@ __global__ void __launch_bounds__(kThreads) resident_blocks_kernel(const RArgs a
             const uint32_t dtype = dtype_of(L, g_is_up ? 5 : 4);
             float acc[R];
             if (g_cnt > 0) {
-                wave_blocks<KQ, R>(c, dtype, g_tiles(L, ct), H, g_wb0, g_cnt, acc);
+                if (!KQ && pair == c.slot) wave_blocks<KQ, R, !KQ>(c, dtype, g_tiles(L, ct), H, g_wb0, g_cnt, acc, ahead);
+                else wave_blocks<KQ, R>(c, dtype, g_tiles(L, ct), H, g_wb0, g_cnt, acc);
             } else {
 #pragma unroll
                 for (int r = 0; r < R; ++r) acc[r] = 0.f;
@@ -859,20 +890,30 @@ __global__ void __launch_bounds__(kThreads) resident_blocks_kernel(const RArgs a
 #pragma unroll
             for (int r = 0; r < R; ++r) emit_receipt(sh.vals + r * 64, ct * kTileCols, kTileCols, r, R, F, a.h_receipt, c.tid, kThreads);
         }
-        xcd_barrier(c);
+        if constexpr (!KQ) {   // the down projection's first tiles
+            __builtin_amdgcn_s_waitcnt(0);
+            ksplit_ahead(c, ahead, L.tiles[6], dtype_of(L, 6), H / 64, d_nblk, d_first, dnbp, dks, dtg, d_active);
+            xcd_barrier(c, true);
+        } else {
+            xcd_barrier(c);
+        }
         stamp(c, l, 5);
         // ---- down projection over this XCD's slice of the FFN width -----------------------------------
         {
             const uint32_t Kp = max(dnbp, 1u) * BE;
             if (d_active && dnbp) copy_receipt<R>(c, a.h_receipt, F, fs.tile0 * 64 + dpb0 * BE, dnbp * BE, dyn);
             __syncthreads();
-            ksplit_project<KQ, R>(c, L.tiles[6], dtype_of(L, 6), H / 64, d_nblk, d_first, dnbp, Kp, dks, dtg, d_active,
-                                  a.d_planes, c.x * d_planes_per_xcd + dkp, H);
+            ksplit_project<KQ, R, !KQ>(c, L.tiles[6], dtype_of(L, 6), H / 64, d_nblk, d_first, dnbp, Kp, dks, dtg, d_active,
+                                       a.d_planes, c.x * d_planes_per_xcd + dkp, H, ahead);
         }
         stamp(c, l, 6);
         const bool more = l + 1 < a.layers;
+        if constexpr (!KQ) {   // the next block's q / k / v tiles
+            __builtin_amdgcn_s_waitcnt(0);
+            if (more) load_ahead(ahead, q_tiles(a.layer[l + 1]), q_cnt, lane);
+        }
         // ---- x = x1 + rms(down, post_ffw_norm); u = rms(x, next block's attn_norm or the output norm) ----
-        norm_pair<R>(c, a.d_planes, c.X * d_planes_per_xcd, L.norm[5], L.gamma_next, xr, !more, false);
+        norm_pair<R>(c, a.d_planes, c.X * d_planes_per_xcd, L.norm[5], L.gamma_next, xr, !more, !KQ);
         stamp(c, l, 7);
     }
 }
