@@ -105,6 +105,35 @@ def test_provisional_commit_then_keep_one_row(hip, target):
     assert_rings(target, one)
 
 
+@pytest.mark.parametrize("accepted", [0, 1])
+def test_commit_and_finalize_leave_the_rings_as_commit_rows_does(hip, target, accepted):
+    """The H1 step publishes after the decision (commit_rows with the accept word); a host that keeps the
+    reference's protocol publishes both rows and finalizes 1 + accepted of them.  Both must leave every ring,
+    local (1024 slots, wrapping here) and global (2048 slots), with the same bytes."""
+    import ctypes as C
+    import torch
+    from guffin_amd import model
+    ticket = model.VerifyTicket(target, POSITION + 4)
+    before = rings(target)
+    pk, pv = run_pass(hip, target, ticket, [17, 1999], POSITION)
+    # commit_rows on copies of the rings
+    copies = rings_copy(before)
+    k_table = torch.tensor([k.data_ptr() for k, _ in copies], dtype=torch.int64, device="cuda")
+    v_table = torch.tensor([v.data_ptr() for _, v in copies], dtype=torch.int64, device="cuda")
+    word = torch.tensor([accepted], dtype=torch.int32, device="cuda")
+    hip.check(hip.lib().guffin_hip_commit_rows(
+        hip._stream(), C.byref(target.desc), C.c_void_p(pk.data_ptr()),
+        C.c_void_p(pv.data_ptr()), C.c_void_p(k_table.data_ptr()), C.c_void_p(v_table.data_ptr()),
+        C.c_void_p(word.data_ptr()), C.c_uint32(POSITION), C.c_uint32(2)))
+    torch.cuda.synchronize()
+    ticket.provisional_commit([0, 1])
+    ticket.finalize(1 + accepted)
+    assert ticket.state == model.TXN_IDLE
+    assert_rings(target, copies)
+    changed = sum(int((k != b[0]).any(dim=-1).sum()) for (k, _), b in zip(copies, before))
+    assert changed == (1 + accepted) * target.shape.layers   # one slot per published row and layer (random rows differ)
+
+
 def rings_copy(src):
     return [(k.clone(), v.clone()) for k, v in src]
 
