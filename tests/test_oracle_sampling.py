@@ -159,6 +159,58 @@ def test_near_equal_residual_and_full_support(gfo):
     assert spec(gfo, p, q, 1, 1.0, 0.1)[0] < 0
 
 
+def uniform_table(vocabulary):
+    """The reference's 32 000-token proposal law: endpoint(i) = i * 2^32 / vocabulary, integer division."""
+    return (np.arange(vocabulary + 1, dtype=np.uint64) * np.uint64(1 << 32)) // np.uint64(vocabulary)
+
+
+def sparse_target(gfo):
+    """p = {0: 0.125, 999: 0.375, 40000: 0.5} as logits (token 40000 lies outside the 32 000-token draft
+    vocabulary); top-k 3, no nucleus, T = 1."""
+    pairs = [(0, math.log(0.125)), (999, math.log(0.375)), (40000, math.log(0.5))]
+    return cands(gfo, pairs), opts(gfo, 1.0, 3, 1.0, 0.0)
+
+
+def test_gathered_full_table_recovers_the_target_marginal(gfo):
+    """tests/engine/lossless_sampling_tests.cpp:375-432: over every proposal of a 32 000-token law with sparse
+    lookups of q on p's support, sum_x q(x) [a(x) 1{x = t} + (1 - a(x)) r_x(t)] = p(t) — the acceptance is
+    lossless — and the residual is never renormalised over the vocabulary intersection."""
+    vocabulary = 32000
+    cdf = uniform_table(vocabulary)
+    row, o = sparse_target(gfo)
+    rc, p = gfo.prepare(row, o)
+    assert rc == 0 and p.count == 3
+    tokens = [p.token[i] for i in range(3)]
+    prob = {p.token[i]: p.probability[i] for i in range(3)}
+    assert abs(prob[0] - 0.125) < 1e-7 and abs(prob[999] - 0.375) < 1e-7 and abs(prob[40000] - 0.5) < 1e-7
+    total = float(1 << 32)
+    mass = lambda t: float(int(cdf[t + 1]) - int(cdf[t])) if t < vocabulary else 0.0
+    marginal = {t: 0.0 for t in tokens}
+    for x in range(vocabulary):
+        rc, got = gfo.spec_accept_full(row, row, cdf, x, o, 0.0, 0.99, 0.5)
+        assert rc == 0, (x, rc)
+        qx = mass(x) / total
+        # the residual this proposal leaves: max(p - q, 0) over p's support in p's order, q not renormalised
+        residual = [max(prob[t] - mass(t) / total, 0.0) for t in tokens]
+        assert got.residual_count == sum(1 for r in residual if r > 0.0)
+        assert abs(got.residual_total - sum(residual)) <= 4e-16
+        if x in prob:
+            assert abs(got.acceptance_probability - min(1.0, prob[x] / qx)) <= 1e-15
+        else:
+            assert got.acceptance_probability == 0.0
+            assert not got.accepted and got.token == tokens[-1]   # u_residual 0.99 lands in the last entry
+        for i, t in enumerate(tokens):
+            inside = qx * got.acceptance_probability if t == x else 0.0
+            marginal[t] += inside + qx * (1.0 - got.acceptance_probability) * residual[i] / got.residual_total
+        if x == 17:
+            assert abs(got.residual_total - (1.0 - (mass(0) + mass(999)) / total)) <= 1e-15
+            # the correction can select a target token that the draft vocabulary does not have
+            rc, first = gfo.spec_accept_full(row, row, cdf, x, o, 0.0, 0.0, 0.5)
+            assert rc == 0 and tokens[0] == 40000 and not first.accepted and first.token == 40000
+    for t in tokens:
+        assert abs(marginal[t] - prob[t]) <= 1e-11, (t, marginal[t], prob[t])
+
+
 def test_prepare_matches_compiled_reference_bit_exact(gfo, ref):
     if ref is None:
         pytest.skip("oracle/_ref not built")
