@@ -131,6 +131,56 @@ def test_packed_unit_vectors_recover_columns(hip, gfo, dtype):
         assert np.allclose(y, dense[:, k], rtol=2e-6, atol=2e-6), k
 
 
+def f32_information_case(dtype, rows, width, columns):
+    """tests/tensor/gemma3_metal_tests.cpp:1419-1499: one non-zero per row, 1 + (row + 1) 2^-20, which a half
+    cannot hold, against weights whose first block scale is the half 0x3555 (about 1/3, not a power of two), so
+    that neither operand survives narrowing to 16 bits; returns (weights, activations, inner index per row)."""
+    w = synth.make_weight(dtype, width, columns, seed=51 if dtype == 1 else 71)
+    bb, scale_offset = (144, 0) if dtype == 1 else (210, 208)
+    for column in range(columns):
+        at = column * (width // 256) * bb + scale_offset
+        w[at], w[at + 1] = 0x55, 0x35
+    x = np.zeros((rows, width), np.float32)
+    inner = [(row % 8) * 33 for row in range(rows)]
+    for row in range(rows):
+        x[row, inner[row]] = np.float32(1.0 + (row + 1) * 2.0 ** -20)
+    return w, x, inner
+
+
+def assert_f32_information(gfo, dtype, w, x, inner, y, width, columns):
+    """The reference's bound is 4 eps |x w| + 1e-6.  Q4_K meets it as written.  For Q6_K the kernels form
+    d s (sum q x - 32 sum x) with q the stored 0..63 (the matrix core takes unsigned quants), not d s sum (q - 32) x:
+    both terms are exact to fp32, but their difference carries their rounding, so the bound here is 4 eps on the
+    two terms, |x w| + 32 |d s x| — wider than the reference's by at most (q + 32) / |q - 32|, still far below what
+    a half-staged operand loses (2^-11)."""
+    dense = gfo.dequant(dtype, w).reshape(columns, width)
+    discriminates = False
+    d_half = np.float32(np.array([0x3555], np.uint16).view(np.float16)[0])
+    for row, k in enumerate(inner):
+        expected = (x[row, k] * dense[:, k]).astype(np.float32)
+        terms = np.abs(expected)
+        if dtype == 2:
+            scales = np.array([np.int8(w[c * (width // 256) * 210 + 192 + k // 16]) for c in range(columns)], np.float32)
+            terms = terms + 32.0 * np.abs(d_half * scales * x[row, k])
+        bound = 4.0 * np.finfo(np.float32).eps * terms + 1e-6
+        assert np.all(np.abs(y[row] - expected) <= bound), (row, float(np.max(np.abs(y[row] - expected) / bound)))
+        narrowed = np.float32(np.float16(x[row, k])) * dense[:, k].astype(np.float16).astype(np.float32)
+        discriminates |= bool(np.any(np.abs(expected - narrowed) > 16.0 * bound))
+    assert discriminates          # the fixture must be able to tell half operands from fp32 ones
+
+
+@pytest.mark.parametrize("dtype", [1, 2])
+def test_packed_gemv_keeps_all_f32_operand_information(hip, gfo, dtype):
+    width, columns = 3840, 64
+    w, x, inner = f32_information_case(dtype, 33, width, columns)
+    tiles = hip.repack(dtype, dev(w), width, columns)
+    got = np.zeros((33, columns), np.float32)
+    for r0 in range(0, 33, 2):                       # rows in pairs (and one single row), as a verify pass sees them
+        xr = dev(x[r0:r0 + 2])
+        got[r0:r0 + 2] = hip.gemv_packed(dtype, tiles, xr, hip.group_sums(xr), columns).cpu().numpy()
+    assert_f32_information(gfo, dtype, w, x, inner, got, width, columns)
+
+
 def test_packed_partials_sum_in_slice_order(hip):
     dtype, K, N = 1, 3840, 1024
     w = hip.repack(dtype, dev(synth.make_weight(dtype, K, N, 11)), K, N)

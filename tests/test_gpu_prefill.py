@@ -48,6 +48,18 @@ def test_prefill_gemm_parity(hip, gfo, dtype, K, N, M):
         assert np.all(np.abs(one.astype(np.float64) - y[r]) <= 2e-5 * scale[r])
 
 
+@pytest.mark.parametrize("dtype", [1, 2])
+def test_prefill_gemm_keeps_all_f32_operand_information(hip, gfo, dtype):
+    """tests/tensor/gemma3_metal_tests.cpp:1419-1499 on the matrix path: 33 rows (a ragged row group), operands
+    that a half cannot hold."""
+    from test_gpu_gemv_packed import assert_f32_information, f32_information_case
+    width, columns = 3840, 64
+    w, x, inner = f32_information_case(dtype, 33, width, columns)
+    tiles = hip.repack(dtype, dev(w), width, columns)
+    y = hip.prefill_gemm(dtype, tiles, hip.prefill_pack(dev(x)), 33, width, columns).cpu().numpy()
+    assert_f32_information(gfo, dtype, w, x, inner, y, width, columns)
+
+
 def test_prefill_gemm_down_projection_shape(hip, gfo):
     """Q6_K at the down projection's K = 15360 (60 blocks per column, the longest chain of LDS
     stages and weight prefetches) with an odd number of column tiles and rows in every row group."""
