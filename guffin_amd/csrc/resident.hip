@@ -10,8 +10,9 @@
 //   gate/up columns and the down projection over the same slice of the FFN width             -> XCD h
 // so that everything between two projections stays inside one L2 and only the two reductions of a
 // block (after the o-projection and after the down projection) cross XCDs.  Inside an XCD workgroups
-// hand data over through that L2: plain stores, a counter in the L2 (atomics execute there), and an
-// L1 invalidate before the reads.  Across XCDs the partial planes are written through (sc1 stores)
+// hand data over through that L2: plain stores, a counter in the L2 (atomics execute there), and reads of
+// addresses this CU has not read before in the launch (a set of exchange buffers per block, so that no line
+// of the L1 can be stale).  Across XCDs the partial planes are written through (sc1 stores)
 // and read with sc1 loads after a two-level barrier (XCD counter, then one device counter).
 // A model with one KV head (the drafter) runs on the 32 CUs of XCD 0; the others leave at once.
 //
@@ -67,6 +68,7 @@ struct RArgs {
     const uint32_t* ancestors;
     uint32_t* status;
     uint32_t spin_limit, opnd_bytes;
+    uint32_t set_floats, vec_floats;   // floats between the exchange buffers of consecutive blocks; floats of one `vec`
     unsigned long long* stamps;   // profiling aid: 8 clock readings per block from workgroup 0, or null
 };
 
@@ -106,6 +108,9 @@ struct Ctx {
     uint32_t X;
     const RArgs* a;
     uint32_t tid;         // the thread index
+    // this block's exchange buffers
+    float *qkv_part, *attn_out, *attn_ml, *o_planes, *d_planes, *vec;
+    uint8_t* h_receipt;
 };
 
 // clock reading `phase` of block `layer` (first workgroup of XCD 0 only; 100 MHz constant clock)
@@ -119,7 +124,13 @@ __device__ __forceinline__ void give_up(Ctx& c) {
 }
 
 // Barrier of the 32 workgroups of this XCD.  Stores issued before it are in the L2 when it opens
-// (the wait for the memory counters precedes the arrival); the L1 is invalidated after it.
+// (the wait for the memory counters precedes the arrival).  Nothing invalidates this CU's L1 here: a
+// device-scope invalidate also sweeps the XCD's L2 (14 us per barrier, measured), and one of workgroup scope
+// does nothing for data from other CUs.  Instead no address of the exchange buffers is read twice during a
+// launch -- every block of a launch has its own set of them (RArgs::set_floats), the two norm joints of a block
+// their own slice buffers -- so a line in the L1 is never older than the data it stands for; the L1 starts
+// every launch empty.  (With one set for all blocks a small model, whose weight stream does not sweep the L1
+// between blocks, read rows of the block before: the reference's six-block fixture caught that.)
 // drained: the caller has already waited for its stores (and then asked for data it does not need before
 // the barrier opens: such loads stay in flight across the wait).
 __device__ __forceinline__ void xcd_barrier(Ctx& c, bool drained = false) {
@@ -136,7 +147,7 @@ __device__ __forceinline__ void xcd_barrier(Ctx& c, bool drained = false) {
         }
     }
     __syncthreads();
-    asm volatile("buffer_inv sc0" ::: "memory");
+    asm volatile("" ::: "memory");
 }
 
 // Barrier of all participating workgroups: arrival at the XCD's counter, the last arrival of an XCD
@@ -169,7 +180,7 @@ __device__ __forceinline__ void device_barrier(Ctx& c, bool drained = false) {
         }
     }
     __syncthreads();
-    asm volatile("buffer_inv sc0" ::: "memory");
+    asm volatile("" ::: "memory");
 }
 
 // sum over one row's threads (waves 8r .. 8r+7), the same order for every row index
@@ -326,7 +337,7 @@ __device__ __forceinline__ void ksplit_project(Ctx& c, const uint8_t* tiles, uin
 template <int R>
 __device__ __forceinline__ void norm_pair(Ctx& c, const float* planes, uint32_t P, const float* gamma_post,
                                           const float* gamma_next, float (&xr)[kRowItems][8], bool last, bool drained,
-                                          uint32_t stamp_layer = 0, uint32_t stamp_base = 0) {
+                                          float* vec, uint32_t stamp_layer = 0, uint32_t stamp_base = 0) {
     const RArgs& a = *c.a;
     const uint32_t H = a.H, r = c.tid / kRowThreads, t0 = c.tid % kRowThreads;
     bool on[kRowItems];
@@ -365,7 +376,7 @@ __device__ __forceinline__ void norm_pair(Ctx& c, const float* planes, uint32_t 
 #pragma unroll
                 for (uint32_t i = 0; i < 8; ++i) if (p0 + i < P) s = p0 + i == 0 ? t[i] : s + t[i];
             }
-            a.vec[(size_t(c.x) * R + rr) * H + cc] = s;
+            vec[(size_t(c.x) * R + rr) * H + cc] = s;
         }
         if (stamp_base) stamp(c, stamp_layer, stamp_base + 1);
         xcd_barrier(c);
@@ -373,7 +384,7 @@ __device__ __forceinline__ void norm_pair(Ctx& c, const float* planes, uint32_t 
 #pragma unroll
         for (uint32_t k = 0; k < kRowItems; ++k) {
             if (on[k]) {
-                const float* src = a.vec + (size_t(c.x) * R + r) * H + col[k];
+                const float* src = vec + (size_t(c.x) * R + r) * H + col[k];
                 const f4_t lo = xld4(src), hi = xld4(src + 4);
                 v[k][0] = lo.x; v[k][1] = lo.y; v[k][2] = lo.z; v[k][3] = lo.w;
                 v[k][4] = hi.x; v[k][5] = hi.y; v[k][6] = hi.z; v[k][7] = hi.w;
@@ -470,7 +481,7 @@ __device__ __forceinline__ void attention_partition(Ctx& c, const RLayer& L, uin
     Shared& sh = *c.sh;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(c.tid >> 6), lane = c.tid & 63;
     const uint32_t row_stride = a.kv_heads * kHd;   // halves between ring rows
-    const float* part = a.qkv_part + size_t(c.x) * PA * R * CW;   // [PA][R][CW]
+    const float* part = c.qkv_part + size_t(c.x) * PA * R * CW;   // [PA][R][CW]
     const size_t pstride = size_t(R) * CW;
 
     // token list: union of the rows' ring ranges, then the private rows
@@ -670,8 +681,8 @@ __device__ __forceinline__ void attention_partition(Ctx& c, const RLayer& L, uin
     }
     __syncthreads();
     // waves that had no token hold zeros: every wave's slot is summed, in wave order
-    float* po = a.attn_out + (size_t(c.x) * kGroups + c.slot) * NQ * kHd;
-    float* pml = a.attn_ml + (size_t(c.x) * kGroups + c.slot) * NQ * 2;
+    float* po = c.attn_out + (size_t(c.x) * kGroups + c.slot) * NQ * kHd;
+    float* pml = c.attn_ml + (size_t(c.x) * kGroups + c.slot) * NQ * 2;
     for (uint32_t i = c.tid; i < uint32_t(NQ) * kHd; i += kThreads) {
         const uint32_t n = i / kHd, d = i % kHd;
         float v = merge[(0 * NQ + n) * kHd + d];
@@ -689,8 +700,8 @@ __device__ __forceinline__ void merge_attention(Ctx& c, uint32_t e0, uint32_t co
     constexpr int NQ = R * G;
     const RArgs& a = *c.a;
     Shared& sh = *c.sh;
-    const float* pml = a.attn_ml + size_t(c.x) * kGroups * NQ * 2;
-    const float* po = a.attn_out + size_t(c.x) * kGroups * NQ * kHd;
+    const float* pml = c.attn_ml + size_t(c.x) * kGroups * NQ * 2;
+    const float* po = c.attn_out + size_t(c.x) * kGroups * NQ * kHd;
     // weights of the 32 partitions per query: half a wave per query
     if (c.tid < uint32_t(NQ) * kGroups) {
         const uint32_t n = c.tid / kGroups, p = c.tid % kGroups;
@@ -737,7 +748,7 @@ __global__ void __launch_bounds__(kThreads) resident_blocks_kernel(const RArgs a
         sh.slot = blockIdx.x / 8;
     }
     __syncthreads();
-    Ctx c {&sh, dyn, sh.xcd, sh.slot, 0, 0, a.kv_heads, &a, threadIdx.x};
+    Ctx c {&sh, dyn, sh.xcd, sh.slot, 0, 0, a.kv_heads, &a, threadIdx.x, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
     if (c.x >= c.X) return;            // a model with fewer KV heads than XCDs leaves the others idle
     if (c.slot >= kGroups) return;
     const uint32_t H = a.H, F = a.F, nbH = H / BE;
@@ -811,6 +822,12 @@ __global__ void __launch_bounds__(kThreads) resident_blocks_kernel(const RArgs a
 
     for (uint32_t l = 0; l < a.layers; ++l) {
         const RLayer& L = a.layer[l];
+        {
+            const size_t at = size_t(l) * a.set_floats;
+            c.qkv_part = a.qkv_part + at; c.attn_out = a.attn_out + at; c.attn_ml = a.attn_ml + at;
+            c.o_planes = a.o_planes + at; c.d_planes = a.d_planes + at; c.vec = a.vec + at;
+            c.h_receipt = static_cast<uint8_t*>(a.h_receipt) + at * 4;
+        }
         stamp(c, l, 0);
         // ---- q, k, v columns of this XCD's KV head -------------------------------------------------
         {
@@ -829,7 +846,7 @@ __global__ void __launch_bounds__(kThreads) resident_blocks_kernel(const RArgs a
                 const uint32_t r = c.tid >> 6;
                 float s = sh.red[r * 64 + lane];
                 for (uint32_t w = 1; w < kWaves; ++w) s += sh.red[(w * R + r) * 64 + lane];
-                a.qkv_part[((size_t(c.x) * PA + qkp) * R + r) * CW + qt * 64 + lane] = s;
+                c.qkv_part[((size_t(c.x) * PA + qkp) * R + r) * CW + qt * 64 + lane] = s;
             }
         }
         if constexpr (!KQ) {   // the o-projection's tiles travel while attention runs
@@ -855,7 +872,7 @@ __global__ void __launch_bounds__(kThreads) resident_blocks_kernel(const RArgs a
             }
             __syncthreads();
             ksplit_project<KQ, R, !KQ>(c, L.tiles[3], dtype_of(L, 3), H / 64, o_nblk, o_first, onbp, Kp, oks, otg, o_active,
-                                       a.o_planes, c.x * oks.kparts + okp, H, ahead);
+                                       c.o_planes, c.x * oks.kparts + okp, H, ahead);
         }
         stamp(c, l, 3);
         if constexpr (!KQ) {   // this workgroup's first gate / up tiles
@@ -863,7 +880,7 @@ __global__ void __launch_bounds__(kThreads) resident_blocks_kernel(const RArgs a
             load_ahead(ahead, g_tiles(L, fs.tile0 + (c.slot < fs.tiles ? c.slot : 0u)), g_cnt, lane);
         }
         // ---- x1 = x + rms(o, post_attention_norm); u = rms(x1, ffn_norm) -------------------------------
-        norm_pair<R>(c, a.o_planes, c.X * oks.kparts, L.norm[3], L.norm[4], xr, false, !KQ, l, 8);
+        norm_pair<R>(c, c.o_planes, c.X * oks.kparts, L.norm[3], L.norm[4], xr, false, !KQ, c.vec, l, 8);
         stamp(c, l, 4);
         // ---- gate and up columns of this XCD's slice of the FFN width, GeGLU, its receipt --------------
         for (uint32_t pair = c.slot; pair < fs.tiles; pair += kGroups) {
@@ -888,7 +905,7 @@ __global__ void __launch_bounds__(kThreads) resident_blocks_kernel(const RArgs a
             }
             __syncthreads();
 #pragma unroll
-            for (int r = 0; r < R; ++r) emit_receipt(sh.vals + r * 64, ct * kTileCols, kTileCols, r, R, F, a.h_receipt, c.tid, kThreads);
+            for (int r = 0; r < R; ++r) emit_receipt(sh.vals + r * 64, ct * kTileCols, kTileCols, r, R, F, c.h_receipt, c.tid, kThreads);
         }
         if constexpr (!KQ) {   // the down projection's first tiles
             __builtin_amdgcn_s_waitcnt(0);
@@ -901,10 +918,10 @@ __global__ void __launch_bounds__(kThreads) resident_blocks_kernel(const RArgs a
         // ---- down projection over this XCD's slice of the FFN width -----------------------------------
         {
             const uint32_t Kp = max(dnbp, 1u) * BE;
-            if (d_active && dnbp) copy_receipt<R>(c, a.h_receipt, F, fs.tile0 * 64 + dpb0 * BE, dnbp * BE, dyn);
+            if (d_active && dnbp) copy_receipt<R>(c, c.h_receipt, F, fs.tile0 * 64 + dpb0 * BE, dnbp * BE, dyn);
             __syncthreads();
             ksplit_project<KQ, R, !KQ>(c, L.tiles[6], dtype_of(L, 6), H / 64, d_nblk, d_first, dnbp, Kp, dks, dtg, d_active,
-                                       a.d_planes, c.x * d_planes_per_xcd + dkp, H, ahead);
+                                       c.d_planes, c.x * d_planes_per_xcd + dkp, H, ahead);
         }
         stamp(c, l, 6);
         const bool more = l + 1 < a.layers;
@@ -913,7 +930,7 @@ __global__ void __launch_bounds__(kThreads) resident_blocks_kernel(const RArgs a
             if (more) load_ahead(ahead, q_tiles(a.layer[l + 1]), q_cnt, lane);
         }
         // ---- x = x1 + rms(down, post_ffw_norm); u = rms(x, next block's attn_norm or the output norm) ----
-        norm_pair<R>(c, a.d_planes, c.X * d_planes_per_xcd, L.norm[5], L.gamma_next, xr, !more, !KQ);
+        norm_pair<R>(c, c.d_planes, c.X * d_planes_per_xcd, L.norm[5], L.gamma_next, xr, !more, !KQ, c.vec + a.vec_floats);
         stamp(c, l, 7);
     }
 }
@@ -951,7 +968,7 @@ bool resident_fits(const guffin_model_desc& m, uint32_t rows) {
     return resident_lds_bytes(m, rows, m.ring_global) <= 140u * 1024u;
 }
 
-struct ResidentSizes { uint64_t qkv, attn_out, attn_ml, o_planes, d_planes, vec, h_receipt, sync, total; uint32_t opnd, lds; };
+struct ResidentSizes { uint64_t qkv, attn_out, attn_ml, o_planes, d_planes, vec, h_receipt, set, sync, total; uint32_t opnd, lds; };
 
 static ResidentSizes resident_sizes(const guffin_model_desc& m, uint32_t rows, uint32_t max_ring_tokens) {
     ResidentSizes s {};
@@ -972,7 +989,9 @@ static ResidentSizes resident_sizes(const guffin_model_desc& m, uint32_t rows, u
     s.h_receipt = al(receipt_layout(rows, F).bytes);
     const uint32_t launches = (m.layer_count + kResidentLayers - 1) / kResidentLayers;
     s.sync = al(uint64_t(launches) * kSyncWords * 4);
-    s.total = s.qkv + s.attn_out + s.attn_ml + s.o_planes + s.d_planes + s.vec + s.h_receipt + s.sync;
+    // one set of exchange buffers per block of a launch (two `vec`: one per norm joint): no address is read twice
+    s.set = s.qkv + s.attn_out + s.attn_ml + s.o_planes + s.d_planes + 2 * s.vec + s.h_receipt;
+    s.total = s.set * kResidentLayers + s.sync;
     // LDS: the operand receipt of the widest K a workgroup sees (the hidden width, or a K part of o / down),
     // then that part's fp32 values (the merged attention rows); or the attention scratch
     const uint32_t kp_o = ko.bpp * BE, kp_d = kd.bpp * BE;
@@ -1047,12 +1066,13 @@ int resident_launch(hipStream_t stream, const guffin_model_desc& m, uint32_t row
     a.attn_ml = reinterpret_cast<float*>(p); p += s.attn_ml;
     a.o_planes = reinterpret_cast<float*>(p); p += s.o_planes;
     a.d_planes = reinterpret_cast<float*>(p); p += s.d_planes;
-    a.vec = reinterpret_cast<float*>(p); p += s.vec;
+    a.vec = reinterpret_cast<float*>(p); p += 2 * s.vec;
     a.h_receipt = p; p += s.h_receipt;
     a.sync = sync_words;
     a.x_in = x_in; a.u_receipt_in = u_receipt_in; a.x_out = x_out; a.u_out = u_out; a.u_receipt_out = u_receipt_out;
     a.ancestors = ancestors; a.status = status;
     a.spin_limit = g_spin_limit; a.opnd_bytes = s.opnd;
+    a.set_floats = static_cast<uint32_t>(s.set / 4); a.vec_floats = static_cast<uint32_t>(s.vec / 4);
     a.stamps = g_resident_stamps ? g_resident_stamps + size_t(first) * 16 : nullptr;
     const uint32_t G = m.q_heads / m.kv_heads;
     const bool kq = m.layers[0].dtype[0] != GUFFIN_Q8_0;

@@ -1,0 +1,150 @@
+"""The target on the device against the reference's dyadic six-block fixture (tests/target_fixture.py), on the
+sequences of the reference's own target tests (tests/engine/gemma3_target_runtime_tests.cpp):
+  :353-386  twelve tokens one at a time, then the same twelve as one prefill and a continuation, across the wrap
+            of the 8-row local rings: logits and cache rows against the independent evaluation, replays bit-equal
+  :515-572  a two-row verify pass at position 7: rows bit-equal to one-row passes, close to the evaluation; both
+            rows published and 0, 1 or 2 of them kept: every cache byte as a plain run leaves it, and a decode
+            step after the rollback."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import target_fixture as fx
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def hip():
+    from guffin_amd import hip as module
+    module.init(0)
+    return module
+
+
+@pytest.fixture(scope="module")
+def fixture():
+    return fx.Fixture()
+
+
+def fresh(fixture):
+    from guffin_amd import model
+    return model.DeviceModel.from_host(fixture.host_model(model))
+
+
+def logits_of(hip, device, hidden, sums):
+    sh = device.shape
+    return hip.gemv_packed(int(sh.embed_dtype), device.head_tiles, hidden, sums, sh.vocab).cpu().numpy()[:, :fx.VOCAB]
+
+
+def commit(hip, device, pk, pv, position, rows):
+    hip.check(hip.lib().guffin_hip_commit_rows(hip._stream(), C.byref(device.desc), C.c_void_p(pk.data_ptr()),
+                                               C.c_void_p(pv.data_ptr()), C.c_void_p(device.ring_k_table.data_ptr()),
+                                               C.c_void_p(device.ring_v_table.data_ptr()), None, C.c_uint32(position),
+                                               C.c_uint32(rows)))
+
+
+def decode(hip, device, token, position):
+    """One ordinary step: a one-row pass, its row published; returns the logits."""
+    import torch
+    hidden, sums, pk, pv, status = device.forward(torch.tensor([token], dtype=torch.int32, device="cuda"), position)
+    commit(hip, device, pk, pv, position, 1)
+    torch.cuda.synchronize()
+    assert int(status.item()) == 0
+    return logits_of(hip, device, hidden, sums)[0]
+
+
+def prefill(hip, device, tokens, position):
+    import torch
+    hidden, status = device.prefill(torch.tensor(list(tokens), dtype=torch.int32, device="cuda"), position)
+    torch.cuda.synchronize()
+    assert int(status.item()) == 0
+    last = hidden[-1:].contiguous()
+    return logits_of(hip, device, last, hip.group_sums(last))[0]
+
+
+def reader(device):
+    def read(layer, position):
+        cap = device.ring_k[layer].shape[0]
+        return (device.ring_k[layer][position & (cap - 1)].float().cpu().numpy().reshape(-1),
+                device.ring_v[layer][position & (cap - 1)].float().cpu().numpy().reshape(-1))
+    return read
+
+
+def caches(device):
+    return [(k.clone(), v.clone()) for k, v in zip(device.ring_k, device.ring_v)]
+
+
+def same_caches(a, b):
+    import torch
+    return all(torch.equal(ka, kb) and torch.equal(va, vb) for (ka, va), (kb, vb) in zip(a, b))
+
+
+def test_complete_synthetic_reference_and_wrapped_batch(hip, fixture):
+    ref = fx.Reference(fixture)
+    scalar = fresh(fixture)
+    worst = 0.0
+    for i in range(12):
+        expected = ref.append(fx.TOKENS[i])
+        print("target fixture: scalar token", i, flush=True)
+        worst = max(worst, fx.assert_close(decode(hip, scalar, fx.TOKENS[i], i), expected, "scalar logits of token %d" % i))
+        if i in (6, 7, 8, 11):
+            fx.assert_cache(scalar, ref, i + 1, reader(scalar))
+    print("device vs dense evaluation: worst logit error %.2f of the budget" % worst, flush=True)
+    batch = fresh(fixture)
+    fx.assert_close(prefill(hip, batch, fx.TOKENS[:12], 0), ref.logits[-1], "twelve-row batched logits")
+    fx.assert_cache(batch, ref, 12, reader(batch))
+    expected = ref.append(fx.TOKENS[12])
+    last = prefill(hip, batch, fx.TOKENS[12:], 12)
+    fx.assert_close(last, expected, "continuation after the wrapped batch")
+    fx.assert_cache(batch, ref, 13, reader(batch))
+    replay = fresh(fixture)
+    prefill(hip, replay, fx.TOKENS[:12], 0)
+    again = prefill(hip, replay, fx.TOKENS[12:], 12)
+    assert np.array_equal(again.view(np.uint32), last.view(np.uint32)), "segmented replay changed the logits"
+    assert same_caches(caches(replay), caches(batch))
+
+
+def test_width_two_prefix_publication_and_rollback(hip, fixture):
+    import torch
+    from guffin_amd import model
+    tokens = fx.TOKENS[:9]
+    ref = fx.Reference(fixture)
+    for token in tokens:
+        ref.append(token)
+    ordinary = fresh(fixture)
+    prefill(hip, ordinary, tokens[:7], 0)
+    ordinary_logits = [decode(hip, ordinary, tokens[7 + i], 7 + i) for i in range(2)]
+    for retained in range(3):
+        print("target fixture: width two, retained", retained, flush=True)
+        plan = fresh(fixture)
+        prefill(hip, plan, tokens[:7], 0)
+        before = caches(plan)
+        ticket = model.VerifyTicket(plan, 7 + 4)
+        ticket.encode(list(tokens[7:9]), 7)
+        ticket.submit()
+        assert ticket.complete() == 0
+        assert same_caches(caches(plan), before), "a completed pass touched the caches"
+        # the pass's rows through the plain entry point: logits of both rows
+        hidden, sums, pk, pv, status = plan.forward(torch.tensor(list(tokens[7:9]), dtype=torch.int32, device="cuda"), 7)
+        logits = logits_of(hip, plan, hidden, sums)
+        for row in range(2):
+            assert np.array_equal(logits[row].view(np.uint32), ordinary_logits[row].view(np.uint32)), \
+                "width-two target conditionals differ from ordinary logits"
+            fx.assert_close(logits[row], ref.logits[7 + row], "verifier row %d" % row)
+        kvw = plan.shape.kv_width
+        assert torch.equal(ticket.priv_k.view(-1)[:pk.numel()].view(-1, 2, kvw), pk)
+        ticket.provisional_commit([0, 1])
+        ticket.finalize(retained)
+        assert ticket.state == model.TXN_IDLE
+        if retained == 0:
+            assert same_caches(caches(plan), before), "full rejection did not restore every slot across the wrap"
+        fx.assert_cache(plan, ref, 7 + retained, reader(plan))
+        check = fresh(fixture)
+        prefill(hip, check, tokens[:7], 0)
+        for i in range(retained):
+            decode(hip, check, tokens[7 + i], 7 + i)
+        assert same_caches(caches(plan), caches(check)), "kept rows differ from a plain run's"
+        if retained < 2:
+            fx.assert_close(decode(hip, plan, tokens[7 + retained], 7 + retained), ref.logits[7 + retained],
+                            "decode after the suffix was rolled back")
