@@ -98,9 +98,9 @@ class Fixture:
                 full = prefix + name + ".weight"
                 self.packed[full], self.dense[full] = (q6k_tensor if six else q4k_tensor)(full, o, i)
 
-    def host_model(self, model):
+    def host_model(self, model, ring_global=32):
         """A guffin_amd.model.HostModel with these weights, empty caches, rings of 8 (local) and 32 (global) rows."""
-        shape = model.Shape(WIDTH, 256, 2, 1, 256, LAYERS, PADDED_VOCAB, WINDOW, 6, 1e4, 1e6, 0.125, 8, 32)
+        shape = model.Shape(WIDTH, 256, 2, 1, 256, LAYERS, PADDED_VOCAB, WINDOW, 6, 1e4, 1e6, 0.125, 8, ring_global)
         host = object.__new__(model.HostModel)
         host.shape = shape
         host.w, host.norm, host.ring_k, host.ring_v = [], [], [], []

@@ -2,6 +2,9 @@
 sequences of the reference's own target tests (tests/engine/gemma3_target_runtime_tests.cpp):
   :353-386  twelve tokens one at a time, then the same twelve as one prefill and a continuation, across the wrap
             of the 8-row local rings: logits and cache rows against the independent evaluation, replays bit-equal
+  :388-462  prompts of 127, 128, 129 and 257 tokens as one prefill and as chunks of 32: last-row logits and every
+            cache row still held agree, rows beyond the prompt keep the NaN pattern the caches were filled with, and a
+            decode step continues from either
   :515-572  a two-row verify pass at position 7: rows bit-equal to one-row passes, close to the evaluation; both
             rows published and 0, 1 or 2 of them kept: every cache byte as a plain run leaves it, and a decode
             step after the rollback."""
@@ -27,9 +30,9 @@ def fixture():
     return fx.Fixture()
 
 
-def fresh(fixture):
+def fresh(fixture, ring_global=32):
     from guffin_amd import model
-    return model.DeviceModel.from_host(fixture.host_model(model))
+    return model.DeviceModel.from_host(fixture.host_model(model, ring_global))
 
 
 def logits_of(hip, device, hidden, sums):
@@ -148,3 +151,40 @@ def test_width_two_prefix_publication_and_rollback(hip, fixture):
         if retained < 2:
             fx.assert_close(decode(hip, plan, tokens[7 + retained], 7 + retained), ref.logits[7 + retained],
                             "decode after the suffix was rolled back")
+
+
+@pytest.mark.parametrize("count", [127, 128, 129, 257])
+def test_bulk_prefill_cache_across_chunk_partitions(hip, fixture, count):
+    import torch
+    tokens = [(i * 19 + i // 7 + 2) % 32 for i in range(258)]
+    batch, segmented = fresh(fixture, 512), fresh(fixture, 512)
+    for plan in (batch, segmented):
+        for k, v in zip(plan.ring_k, plan.ring_v):
+            k.view(torch.int16).fill_(0x7e00)
+            v.view(torch.int16).fill_(0x7e00)
+    whole = prefill(hip, batch, tokens[:count], 0)
+    first = 0
+    while first < count:
+        rows = min(32, count - first)
+        last = prefill(hip, segmented, tokens[first:first + rows], first)
+        first += rows
+    fx.assert_close(whole, last, "chunk partition logits")
+
+    def check(committed):
+        for layer in range(fx.LAYERS):
+            cap = batch.ring_k[layer].shape[0]
+            held = range(max(0, committed - cap), committed)
+            for a, b in ((batch.ring_k[layer], segmented.ring_k[layer]), (batch.ring_v[layer], segmented.ring_v[layer])):
+                a, b = a.float().cpu().numpy().reshape(cap, -1), b.float().cpu().numpy().reshape(cap, -1)
+                for position in held:
+                    fx.assert_close(a[position & (cap - 1)], b[position & (cap - 1)], "committed row %d of block %d" % (position, layer),
+                                    3e-4, 3e-4 + 2.0 ** -10)
+            if committed < cap:
+                for ring in (batch.ring_k[layer], batch.ring_v[layer], segmented.ring_k[layer], segmented.ring_v[layer]):
+                    rest = ring.view(torch.int16).reshape(cap, -1)[committed:]
+                    assert bool((rest == 0x7e00).all()), "a row beyond the prompt was written"
+
+    check(count)
+    fx.assert_close(decode(hip, batch, tokens[count], count), decode(hip, segmented, tokens[count], count),
+                    "ordinary decode after the partitioned prompt")
+    check(count + 1)
