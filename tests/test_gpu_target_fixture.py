@@ -5,6 +5,8 @@ sequences of the reference's own target tests (tests/engine/gemma3_target_runtim
   :388-462  prompts of 127, 128, 129 and 257 tokens as one prefill and as chunks of 32: last-row logits and every
             cache row still held agree, rows beyond the prompt keep the NaN pattern the caches were filled with, and a
             decode step continues from either
+  :719-790  a V projection scaled from 2^-11 to 2^11: the row's fp32 values are finite, their binary16 narrowing is not;
+            the plain pass raises the status bit, the width-two transaction ends and leaves every cache bit
   :515-572  a two-row verify pass at position 7: rows bit-equal to one-row passes, close to the evaluation; both
             rows published and 0, 1 or 2 of them kept: every cache byte as a plain run leaves it, and a decode
             step after the rollback."""
@@ -188,3 +190,43 @@ def test_bulk_prefill_cache_across_chunk_partitions(hip, fixture, count):
     fx.assert_close(decode(hip, batch, tokens[count], count), decode(hip, segmented, tokens[count], count),
                     "ordinary decode after the partitioned prompt")
     check(count + 1)
+
+
+def test_f16_cache_overflow_preserves_transaction_boundaries(hip, fixture):
+    import copy
+    import torch
+    from guffin_amd import model
+    KV_NONFINITE = 8
+    broken = copy.copy(fixture)
+    broken.packed = dict(fixture.packed)
+    embd = fixture.packed["token_embd.weight"].copy()
+    embd[:210] = 0                                      # token 0 embeds to zero: a prefix with finite zero K/V
+    broken.packed["token_embd.weight"] = embd
+    v = fixture.packed["blk.0.attn_v.weight"].copy().reshape(-1, 210)
+    v[:, 208], v[:, 209] = 0x00, 0x68                   # d = 2^11 instead of 2^-11
+    broken.packed["blk.0.attn_v.weight"] = v.reshape(-1)
+    host = broken.host_model(model)
+
+    def plan_with_prefix():
+        plan = model.DeviceModel.from_host(host)
+        prefill(hip, plan, [0], 0)
+        for k, vv in zip(plan.ring_k, plan.ring_v):
+            assert float(k[0].float().abs().max()) == 0.0 and float(vv[0].float().abs().max()) == 0.0
+        return plan
+
+    plan = plan_with_prefix()
+    hidden, sums, pk, pv, status = plan.forward(torch.tensor([2], dtype=torch.int32, device="cuda"), 1)
+    torch.cuda.synchronize()
+    assert int(status.item()) & KV_NONFINITE, "a non-finite narrowed V row went unreported"
+    assert not bool(torch.isfinite(pv[0].float()).all())
+
+    plan = plan_with_prefix()
+    before = caches(plan)
+    ticket = model.VerifyTicket(plan, 8)
+    ticket.encode([2, 7], 1)
+    ticket.submit()
+    with pytest.raises(hip.GuffinError) as err:
+        ticket.complete()
+    assert err.value.code == -7                          # numerical fault: the transaction is dropped
+    assert ticket.state == model.TXN_IDLE
+    assert same_caches(caches(plan), before), "the overflowing pass changed a cache bit"
