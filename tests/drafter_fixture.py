@@ -89,7 +89,10 @@ class Reference:
         r = np.arange(outputs)
         return (np.float32(0.125) * np.asarray(x, np.float32)[(r * 7 + 11 + matrix * 3) % len(x)]).astype(np.float32)
 
-    def step(self, token):
+    def step(self, token, zero_prefix=False):
+        """zero_prefix: every earlier position of the caches holds zero keys and values (the reference's
+        seed_zero_cache_prefix_for_testing): their scores are 0, so the current token's weight is
+        1 / (1 + n exp(-s)) over the n earlier positions in reach and the output that weight times its value."""
         j = np.arange(WIDTH, dtype=np.int64)
         emb = ((((token * 17 + j * 13) % 53) - 26) / 64.0).astype(np.float32)
         x = (emb * np.float32(math.sqrt(np.float32(WIDTH)))).astype(np.float32)
@@ -115,13 +118,19 @@ class Reference:
             self.keys[layer].append(k)
             self.values[layer].append(v)
             first = pos - 511 if local and pos >= 511 else 0
-            K = np.stack(self.keys[layer][first:pos + 1]).astype(np.float64)
-            V = np.stack(self.values[layer][first:pos + 1]).astype(np.float64)
             attended = np.zeros(1024, np.float32)
-            for head in range(4):
-                scores = K @ q[head * HEAD:(head + 1) * HEAD].astype(np.float64) / 16.0
-                w = np.exp(scores - scores.max())
-                attended[head * HEAD:(head + 1) * HEAD] = ((w / w.sum()) @ V).astype(np.float32)
+            if zero_prefix:
+                for head in range(4):
+                    score = float(q[head * HEAD:(head + 1) * HEAD].astype(np.float64) @ k.astype(np.float64))
+                    current = 1.0 / (1.0 + (pos - first) * math.exp(-score / 16.0))
+                    attended[head * HEAD:(head + 1) * HEAD] = (current * v.astype(np.float64)).astype(np.float32)
+            else:
+                K = np.stack(self.keys[layer][first:pos + 1]).astype(np.float64)
+                V = np.stack(self.values[layer][first:pos + 1]).astype(np.float64)
+                for head in range(4):
+                    scores = K @ q[head * HEAD:(head + 1) * HEAD].astype(np.float64) / 16.0
+                    w = np.exp(scores - scores.max())
+                    attended[head * HEAD:(head + 1) * HEAD] = ((w / w.sum()) @ V).astype(np.float32)
             x = x + self.norm(self.linear(attended, WIDTH, 3), WIDTH)
             nf = self.norm(x, WIDTH)
             gate = self.linear(nf, FF, 4).astype(np.float64)
