@@ -59,3 +59,23 @@ extern "C" int guffin_hip_init(int device) {
         return fail(GUFFIN_E_HIP, "init: could not take the address of the static scratch array on this device");
     return GUFFIN_OK;
 }
+
+extern "C" int guffin_vocab_map_invert(const int32_t* draft_to_target, uint32_t draft_vocab, uint32_t target_vocab,
+                                       int32_t* target_to_draft, uint32_t* mapped_count) {
+    if (!draft_to_target || !target_to_draft) return fail(GUFFIN_E_ARG, "vocab_map_invert: null pointer");
+    if (draft_vocab == 0 || target_vocab == 0) return fail(GUFFIN_E_SHAPE, "vocab_map_invert: empty vocabulary");
+    for (uint32_t t = 0; t < target_vocab; ++t) target_to_draft[t] = -1;
+    uint32_t mapped = 0;
+    for (uint32_t d = 0; d < draft_vocab; ++d) {
+        const int32_t t = draft_to_target[d];
+        if (t < -1 || (t >= 0 && static_cast<uint32_t>(t) >= target_vocab))
+            return fail(GUFFIN_E_ARG, "vocab_map_invert: map token is out of bounds");
+        if (t < 0) continue;
+        if (target_to_draft[t] != -1) return fail(GUFFIN_E_ARG, "vocab_map_invert: map is not injective");
+        target_to_draft[t] = static_cast<int32_t>(d);
+        ++mapped;
+    }
+    if (mapped == 0) return fail(GUFFIN_E_ARG, "vocab_map_invert: intersection is empty");
+    if (mapped_count) *mapped_count = mapped;
+    return GUFFIN_OK;
+}

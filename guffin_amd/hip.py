@@ -437,6 +437,16 @@ def draft_process(logits, history, repetition_penalty):
     return scores
 
 
+def vocab_map_invert(draft_to_target, target_vocab):
+    """Host check of a draft -> target vocabulary map; returns (target_to_draft, number of mapped tokens)."""
+    d2t = _np.ascontiguousarray(draft_to_target, _np.int32)
+    t2d = _np.empty(target_vocab, _np.int32)
+    mapped = C.c_uint32(0)
+    check(lib().guffin_vocab_map_invert(d2t.ctypes.data_as(C.c_void_p), d2t.size, target_vocab,
+                                        t2d.ctypes.data_as(C.c_void_p), C.byref(mapped)))
+    return t2d, mapped.value
+
+
 def draft_law_mapped(logits, draft_to_target, options, history=None, seed=0, step=0, draws=None, status=None):
     """(law in draft ids, draft proposal, target proposal, status) with the drafter's vocabulary map."""
     vocab = logits.numel()

@@ -367,6 +367,14 @@ int guffin_hip_spec_accept_history(void* stream, const void* target_candidates, 
  * guffin_hip_draft_law.  guffin_hip_spec_accept_mapped is guffin_hip_spec_accept_history with the
  * candidates and the proposal in target ids and masses gathered through target_to_draft
  * (Gemma3DraftPlan::gather, :1528-1581); NULL maps mean one shared vocabulary. */
+/* Host only, no GPU call: checks a vocabulary map as the reference's drafter does when it is built
+ * (src/engine/gemma3_draft.mm:655-675) and writes its inverse.  draft_to_target: draft_vocab host words;
+ * target_to_draft: target_vocab host words, out.  GUFFIN_E_ARG with the reference's reasons: a target id
+ * below -1 or at or beyond target_vocab ("out of bounds"), two draft tokens on one target token ("not
+ * injective"), no mapped token at all ("intersection is empty"); mapped_count (may be NULL) receives the
+ * number of mapped tokens. */
+int guffin_vocab_map_invert(const int32_t* draft_to_target, uint32_t draft_vocab, uint32_t target_vocab,
+                            int32_t* target_to_draft, uint32_t* mapped_count);
 int guffin_hip_draft_law_mapped(void* stream, const float* logits, uint32_t vocab, const int32_t* draft_to_target,
                                 const uint32_t* history, uint32_t history_count, const void* options,
                                 uint64_t seed, uint64_t step, const void* injected_draws, void* workspace,
