@@ -99,6 +99,40 @@ def test_attention_closed_forms(hip):
     assert np.array_equal(out1, want1)
 
 
+def test_attention_extreme_finite_scores(hip):
+    """tests/tensor/gemma3_metal_tests.cpp:882-936: scores of exactly +-1024 and +-2048 against fp16 values of
+    +-65504.  A stable fp32 softmax discards the losing exponentials, maxima of different partitions stay finite,
+    and every output element is exact: the winning private row's 65504 / -65504, or the plain mean of 256 equal
+    value rows."""
+    rows, heads, kv_heads, width, capacity = 2, 16, 8, 256, 512
+    q = np.zeros((rows, heads, width), np.float32)
+    q[:, 0::2, 0], q[:, 1::2, 0] = 1024.0, -1024.0
+    pk = np.zeros((rows, kv_heads, width), np.float16)
+    pk[0, :, 0], pk[1, :, 0] = 32.0, -32.0
+    pv = np.zeros((rows, kv_heads, width), np.float16)
+    pv[0], pv[1] = 65504.0, -65504.0
+    k = np.zeros((capacity, kv_heads, width), np.float16)
+    k[0::2, :, 0], k[1::2, :, 0] = 16.0, -16.0
+    v = np.zeros((capacity, kv_heads, width), np.float16)
+    v[:] = (np.arange(kv_heads, dtype=np.float32)[:, None] + np.arange(width, dtype=np.float32)[None, :] * 0.25)[None]
+    sched = np.array([[0, capacity, 0, 1], [0, capacity, 1, 2]], np.uint32)
+    ancestors = np.array([0, 0, 1], np.uint32)
+    flat = lambda a: dev(a.reshape(a.shape[0], -1))
+    for want_sums in (False, True):
+        got = hip.attention_decode(flat(q), flat(k), flat(v), flat(pk), flat(pv), dev(sched), dev(ancestors), capacity + rows,
+                                   capacity - 1, heads, kv_heads, width, 1.0 / 16.0, want_sums=want_sums)
+        out = (got[0] if want_sums else got).cpu().numpy().reshape(rows, heads, width)
+        for row in range(rows):
+            for head in range(heads):
+                if head % 2 == 0:
+                    expected = np.full(width, 65504.0, np.float32)
+                elif row == 1:
+                    expected = np.full(width, -65504.0, np.float32)
+                else:
+                    expected = (head // 2 + np.arange(width) * 0.25).astype(np.float32)
+                assert np.array_equal(out[row, head], expected), (row, head, out[row, head][:4], expected[:4])
+
+
 def test_attention_rejects_bad_shapes(hip):
     import torch
     z = torch.zeros(4096, dtype=torch.float32, device="cuda")
