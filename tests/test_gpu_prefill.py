@@ -213,6 +213,69 @@ def test_prefill_attention_matches_double_softmax(hip, q_heads, kv_heads, rows, 
     assert np.max(np.abs(out - want)) <= 2e-6 * max(1.0, np.abs(want).max())
 
 
+REFERENCE_ATTENTION_CASES = (
+    [(rows, 0, rows, 256, 4, 2, False, False) for rows in (8, 9, 31, 32, 33, 127, 128)]
+    + [(rows, 141, 8, 32, 4, 2, False, False) for rows in (8, 9, 31, 32, 33, 127, 128)]
+    + [(9, 1021, 1024, 1024, 16, 8, False, False), (33, 257, 290, 512, 16, 8, False, False),
+       (9, 141, 32, 32, 16, 8, True, False), (8, 0, 8, 16, 4, 2, False, True)])
+
+
+@pytest.mark.parametrize("matrix_core", [True, False])
+@pytest.mark.parametrize("rows,origin,window,capacity,q_heads,kv_heads,large_scores,sensitive_query", REFERENCE_ATTENTION_CASES)
+def test_prefill_attention_reference_cases(hip, rows, origin, window, capacity, q_heads, kv_heads, large_scores,
+                                           sensitive_query, matrix_core):
+    """tests/tensor/gemma3_metal_tests.cpp:940-1077: dyadic key / value / query patterns, NaN in every ring slot
+    and beyond every row that must not be read, causal tails of 8..128 rows from an empty cache and behind an
+    unaligned origin whose chunk wraps the ring, the target's head geometry, large scores, and a query whose
+    information is lost if it is rounded to fp16 (row 1's two scores then cancel and the output is 0 instead of
+    about 0.0016).  Bar: the reference's 4e-4 against a double softmax."""
+    hd = 256
+    width = kv_heads * hd
+    end = origin + rows
+    first = origin + 1 - window if origin + 1 > window else 0
+    pos = np.arange(end)[:, None, None]
+    head = np.arange(kv_heads)[None, :, None]
+    col = np.arange(hd)[None, None, :]
+    if sensitive_query:
+        logical_k = np.where(pos == 0, 1.0, -1.0) * np.ones((1, kv_heads, hd))
+        logical_v = logical_k.copy()
+    else:
+        logical_k = (((pos * 97 + head * 19 + col * 37) % 251) - 125) / 64.0
+        logical_v = (((pos * 41 + head * 29 + col * 11) % 127) - 63) / 64.0
+    logical_k = logical_k.astype(np.float32).reshape(end, width)
+    logical_v = logical_v.astype(np.float32).reshape(end, width)
+    r = np.arange(rows)[:, None, None]
+    h = np.arange(q_heads)[None, :, None]
+    if sensitive_query:
+        q = np.where(col < 128, np.float32(1.0002), np.float32(-1.0)) * np.ones((rows, q_heads, 1), np.float32)
+    else:
+        q = ((((r * 43 + h * 23 + col * 17) % 257) - 128).astype(np.float32) * np.float32(0.500173 if large_scores else 0.0078173)
+             + (h % 3).astype(np.float32) * np.float32(0.000173))
+    q = q.astype(np.float32).reshape(rows, q_heads * hd)
+    ring_k = np.full((capacity, width), np.nan, np.float16)
+    ring_v = np.full((capacity, width), np.nan, np.float16)
+    for p in range(first, origin):
+        ring_k[p & (capacity - 1)], ring_v[p & (capacity - 1)] = logical_k[p], logical_v[p]
+    run_k, run_v = logical_k[origin:end].astype(np.float16), logical_v[origin:end].astype(np.float16)
+    out = hip.prefill_attention(dev(q), dev(ring_k), dev(ring_v), dev(run_k), dev(run_v), origin, window, capacity - 1,
+                                q_heads, kv_heads, hd, 0.0625, matrix_core=matrix_core).cpu().numpy()
+    group = q_heads // kv_heads
+    worst = 0.0
+    for row in range(rows):
+        position = origin + row
+        start = position + 1 - window if position + 1 > window else 0
+        K = logical_k[start:position + 1].astype(np.float64).reshape(-1, kv_heads, hd)
+        V = logical_v[start:position + 1].astype(np.float64).reshape(-1, kv_heads, hd)
+        for hq in range(q_heads):
+            scores = K[:, hq // group] @ q[row, hq * hd:(hq + 1) * hd].astype(np.float64) / 16.0
+            w = np.exp(scores - scores.max())
+            expected = (w / w.sum()) @ V[:, hq // group]
+            worst = max(worst, float(np.abs(out[row, hq * hd:(hq + 1) * hd] - expected).max()))
+    assert np.all(np.isfinite(out)) and worst <= 4e-4, worst
+    if sensitive_query:
+        assert abs(float(out[1, 0]) ) > 1e-3       # the retained fp32 query decides row 1
+
+
 def test_publish_run_keeps_the_newest_rows(hip):
     import torch
     rows, width, cap, position = 40, 256, 16, 9
