@@ -242,20 +242,27 @@ struct GroupA { half8_t a[4]; };
 template <int CH>
 __device__ __forceinline__ void q4_chunk(const GroupA& lo, const GroupA& hi, const uint4 (&q)[8], const uint32_t (&scw)[4],
                                          float4_t (&D)[4][4]) {
+    constexpr uint32_t M = 0x000F000Fu;
+    // all low-nibble groups first, then all high-nibble groups: an accumulator is used again 16
+    // matrix instructions later rather than 4
 #pragma unroll
     for (int cg = 0; cg < 4; ++cg) {
         // the scale byte in both 16-bit fields
         const uint32_t pair_lo = __builtin_amdgcn_perm(0u, scw[cg], (CH & 1) ? 0x0c020c02u : 0x0c000c00u);
+        const uint4 piece = q[2 * cg + (CH >> 1)];
+        const uint32_t w0 = (CH & 1) ? piece.z : piece.x, w1 = (CH & 1) ? piece.w : piece.y;
+        const half8_t blo = as_half8(pk_mul(w0 & M, pair_lo), pk_mul((w0 >> 8) & M, pair_lo),
+                                     pk_mul(w1 & M, pair_lo), pk_mul((w1 >> 8) & M, pair_lo));
+#pragma unroll
+        for (int rg = 0; rg < 4; ++rg) D[cg][rg] = __builtin_amdgcn_mfma_f32_16x16x32_f16(lo.a[rg], blo, D[cg][rg], 0, 0, 0);
+    }
+#pragma unroll
+    for (int cg = 0; cg < 4; ++cg) {
         const uint32_t pair_hi = __builtin_amdgcn_perm(0u, scw[cg], (CH & 1) ? 0x0c030c03u : 0x0c010c01u);
         const uint4 piece = q[2 * cg + (CH >> 1)];
         const uint32_t w0 = (CH & 1) ? piece.z : piece.x, w1 = (CH & 1) ? piece.w : piece.y;
-        constexpr uint32_t M = 0x000F000Fu;
-        const half8_t blo = as_half8(pk_mul(w0 & M, pair_lo), pk_mul((w0 >> 8) & M, pair_lo),
-                                     pk_mul(w1 & M, pair_lo), pk_mul((w1 >> 8) & M, pair_lo));
         const half8_t bhi = as_half8(pk_mul((w0 >> 4) & M, pair_hi), pk_mul((w0 >> 12) & M, pair_hi),
                                      pk_mul((w1 >> 4) & M, pair_hi), pk_mul((w1 >> 12) & M, pair_hi));
-#pragma unroll
-        for (int rg = 0; rg < 4; ++rg) D[cg][rg] = __builtin_amdgcn_mfma_f32_16x16x32_f16(lo.a[rg], blo, D[cg][rg], 0, 0, 0);
 #pragma unroll
         for (int rg = 0; rg < 4; ++rg) D[cg][rg] = __builtin_amdgcn_mfma_f32_16x16x32_f16(hi.a[rg], bhi, D[cg][rg], 0, 0, 0);
     }
