@@ -495,6 +495,23 @@ __device__ __forceinline__ void attention_partition(Ctx& c, const RLayer& L, uin
     const TokenList tl = token_list<R>(L, c.slot);
     const uint32_t u_first = tl.u_first, n_ring = tl.n_ring, tp = tl.tp, t0 = tl.t0, t1 = tl.t1;
 
+    const uint32_t half = lane >> 5, l32 = lane & 31;            // token slot of the wave's round, 8-dim segment
+    constexpr int U = 4;                                         // rounds of loads in flight
+    // ring rows of this wave's first rounds: their addresses need the schedule only, so the keys travel while
+    // the queries are prepared and the values while the softmax runs (private rows come from LDS at use)
+    const uint32_t tb_first = t0 + wave * 2 + half;
+    auto load_ring = [&](const uint16_t* ring, uint32_t tb, uint4 (&dst)[U]) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const uint32_t t = tb + 2 * kWaves * u;
+            dst[u] = make_uint4(0, 0, 0, 0);
+            if (t < t1 && t < n_ring)
+                dst[u] = *reinterpret_cast<const uint4*>(ring + size_t((u_first + t) & L.ring_mask) * row_stride + c.x * kHd + l32 * 8);
+        }
+    };
+    uint4 kk[U], vv[U];
+    load_ring(L.ring_k, tb_first, kk);
+
     // item n < NQ is query row n; items NQ .. NQ + 2R - 1 are the private rows' key and value, prepared when
     // this partition holds them (head norm, rotation, fp16 rounding after rotation); a wave takes items
     // wave, wave + 8, ..
@@ -559,8 +576,6 @@ __device__ __forceinline__ void attention_partition(Ctx& c, const RLayer& L, uin
 
     float* sc = reinterpret_cast<float*>(c.dyn);                 // [NQ][tp] scores, then probabilities
     float* merge = sc + ((size_t(NQ) * tp + 63) & ~size_t{63});  // [waves][NQ][256]
-    const uint32_t half = lane >> 5, l32 = lane & 31;            // token slot of the wave's round, 8-dim segment
-    constexpr int U = 4;                                         // rounds of loads in flight
     // ---- scores: a half wave per token, 8 dims per lane -----------------------------------------
     {
         float qv[NQ][8];
@@ -568,17 +583,12 @@ __device__ __forceinline__ void attention_partition(Ctx& c, const RLayer& L, uin
         for (int n = 0; n < NQ; ++n)
 #pragma unroll
             for (int i = 0; i < 8; ++i) qv[n][i] = sh.q_s[n * kHd + l32 * 8 + i];
-        const uint32_t tb_first = t0 + wave * 2 + half;
         for (uint32_t tb = tb_first; tb < t1; tb += 2 * kWaves * U) {
-            uint4 kk[U];
+            if (tb != tb_first) load_ring(L.ring_k, tb, kk);
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 const uint32_t t = tb + 2 * kWaves * u;
-                kk[u] = make_uint4(0, 0, 0, 0);
-                if (t < t1) {
-                    if (t >= n_ring) kk[u] = *reinterpret_cast<const uint4*>(&sh.k_s[t - n_ring][l32 * 8]);
-                    else kk[u] = *reinterpret_cast<const uint4*>(L.ring_k + size_t((u_first + t) & L.ring_mask) * row_stride + c.x * kHd + l32 * 8);
-                }
+                if (t < t1 && t >= n_ring) kk[u] = *reinterpret_cast<const uint4*>(&sh.k_s[t - n_ring][l32 * 8]);
             }
 #pragma unroll
             for (int u = 0; u < U; ++u) {
@@ -614,6 +624,7 @@ __device__ __forceinline__ void attention_partition(Ctx& c, const RLayer& L, uin
             }
         }
     }
+    load_ring(L.ring_v, tb_first, vv);
     __syncthreads();
     // ---- softmax over the partition, one wave per query ------------------------------------------
     const uint32_t np = t1 - t0;
@@ -639,17 +650,12 @@ __device__ __forceinline__ void attention_partition(Ctx& c, const RLayer& L, uin
         for (int n = 0; n < NQ; ++n)
 #pragma unroll
             for (int i = 0; i < 8; ++i) acc[n][i] = 0.f;
-        const uint32_t tb_first = t0 + wave * 2 + half;
         for (uint32_t tb = tb_first; tb < t1; tb += 2 * kWaves * U) {
-            uint4 vv[U];
+            if (tb != tb_first) load_ring(L.ring_v, tb, vv);
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 const uint32_t t = tb + 2 * kWaves * u;
-                vv[u] = make_uint4(0, 0, 0, 0);
-                if (t < t1) {
-                    if (t >= n_ring) vv[u] = *reinterpret_cast<const uint4*>(&sh.v_s[t - n_ring][l32 * 8]);
-                    else vv[u] = *reinterpret_cast<const uint4*>(L.ring_v + size_t((u_first + t) & L.ring_mask) * row_stride + c.x * kHd + l32 * 8);
-                }
+                if (t < t1 && t >= n_ring) vv[u] = *reinterpret_cast<const uint4*>(&sh.v_s[t - n_ring][l32 * 8]);
             }
 #pragma unroll
             for (int u = 0; u < U; ++u) {
