@@ -76,7 +76,7 @@ __device__ __forceinline__ void compute_tile(const Q4Tile& t, const Q4Operand& o
     const uint32_t sc_a = s0 & 0x3F3F3F3Fu, mn_a = s1 & 0x3F3F3F3Fu;
     const uint32_t sc_b = (s2 & 0x0F0F0F0Fu) | ((s0 >> 2) & 0x30303030u);
     const uint32_t mn_b = ((s2 >> 4) & 0x0F0F0F0Fu) | ((s1 >> 2) & 0x30303030u);
-    const float d_hi = d * 0.0625f;  // high nibbles enter as 16*q
+    const float d_q = d * 0.0625f;  // nibbles enter as 16 q
     float mt[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) mt[r] = 0.f;
@@ -88,9 +88,14 @@ __device__ __forceinline__ void compute_tile(const Q4Tile& t, const Q4Operand& o
         for (int cg = 0; cg < 4; ++cg) {
             const uint4 piece = t.q[2 * cg + (ch >> 1)];
             const uint32_t w0 = (ch & 1) ? piece.z : piece.x, w1 = (ch & 1) ? piece.w : piece.y;
-            const uint32_t v0 = w0 >> 8, v1 = w1 >> 8;
-            const half8_t blo = as_half8(w0 & 0x000F000Fu, v0 & 0x000F000Fu, w1 & 0x000F000Fu, v1 & 0x000F000Fu);
-            const half8_t bhi = as_half8(w0 & 0x00F000F0u, v0 & 0x00F000F0u, w1 & 0x00F000F0u, v1 & 0x00F000F0u);
+            // every nibble sits in bits 4-7 of its half (16 q as a bit pattern below 2048, which reads as
+            // 16 q 2^-24): the matrix instruction does not normalise such operands, so a pattern with leading
+            // zeros loses that many bits of every product it meets once the products of a sum are aligned.
+            // (In bits 0-3 the low nibbles cost up to 200 eps of a group's sum|q x| on activations with a wide
+            // range inside the group; bits 6-9 would gain two more bits for one more shift per word.)
+            constexpr uint32_t M = 0x00F000F0u;
+            const half8_t blo = as_half8((w0 << 4) & M, (w0 >> 4) & M, (w1 << 4) & M, (w1 >> 4) & M);
+            const half8_t bhi = as_half8(w0 & M, (w0 >> 8) & M, w1 & M, (w1 >> 8) & M);
             const float4_t dlo = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[2 * ch], blo, zero, 0, 0, 0);
             const float4_t dhi = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[2 * ch + 1], bhi, zero, 0, 0, 0);
             if (lane_group == uint32_t(cg)) { lo = dlo; hi = dhi; }
@@ -98,7 +103,7 @@ __device__ __forceinline__ void compute_tile(const Q4Tile& t, const Q4Operand& o
         const uint32_t scw = ch < 2 ? sc_a : sc_b, mnw = ch < 2 ? mn_a : mn_b;
         const float sc_lo = (ch & 1) ? ub2(scw) : ub0(scw), sc_hi = (ch & 1) ? ub3(scw) : ub1(scw);
         const float mn_lo = (ch & 1) ? ub2(mnw) : ub0(mnw), mn_hi = (ch & 1) ? ub3(mnw) : ub1(mnw);
-        const float f_lo = d * sc_lo, f_hi = d_hi * sc_hi;
+        const float f_lo = d_q * sc_lo, f_hi = d_q * sc_hi;
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             const float m_lo = mult[r * per_mult + 2 * ch], m_hi = mult[r * per_mult + 2 * ch + 1];
@@ -170,12 +175,13 @@ __device__ __forceinline__ void compute_tile(const Q6Tile& t, const uint8_t* __r
 #pragma unroll
             for (int k = 0; k < 2; ++k) {
                 const uint32_t w = k ? w1 : w0, h = k ? h1 : h0;
-                const uint32_t lo0 = (w >> ls) & 0x000F000Fu, lo1 = (w >> (ls + 8)) & 0x000F000Fu;
-                // 2-bit field of quadrant qd moved to bits 4-5 of each half
-                const uint32_t hs0 = qd == 0 ? h << 4 : qd == 1 ? h << 2 : qd == 2 ? h : h >> 2;
-                const uint32_t hs1 = h >> (4 + 2 * qd);
-                b[2 * k] = (hs0 & 0x00300030u) | lo0;
-                b[2 * k + 1] = (hs1 & 0x00300030u) | lo1;
+                // the 6-bit quant sits in bits 4-9 of its half (16 q as a bit pattern: see the Q4_K tile)
+                const uint32_t lo0 = (ls ? w : w << 4) & 0x00F000F0u, lo1 = (w >> (ls + 4)) & 0x00F000F0u;
+                // 2-bit field of quadrant qd moved to bits 8-9 of each half
+                const uint32_t hs0 = h << (8 - 2 * qd);
+                const uint32_t hs1 = qd == 0 ? h : h >> (2 * qd);
+                b[2 * k] = (hs0 & 0x03000300u) | lo0;
+                b[2 * k + 1] = (hs1 & 0x03000300u) | lo1;
             }
             D[cg] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, as_half8(b[0], b[1], b[2], b[3]), zero, 0, 0, 0);
         }
@@ -204,7 +210,7 @@ __device__ __forceinline__ void compute_tile(const Q6Tile& t, const uint8_t* __r
     for (int c = 0; c < 2; ++c) {
         const float d = h2f(t.d[c]);
 #pragma unroll
-        for (int r = 0; r < R; ++r) acc[c][r] = fmaf(d, fmaf(-32.0f, off[c][r], part[c][r]), acc[c][r]);
+        for (int r = 0; r < R; ++r) acc[c][r] = fmaf(d, fmaf(-32.0f, off[c][r], 0.0625f * part[c][r]), acc[c][r]);
     }
 }
 
@@ -245,14 +251,15 @@ __device__ __forceinline__ void compute_tile(const Q8Tile& t, const half8_t a,
     for (int cg = 0; cg < 4; ++cg) {
         const uint4 piece = t.q[cg >> 1];
         const uint32_t w0 = ((cg & 1) ? piece.z : piece.x) ^ 0x80808080u, w1 = ((cg & 1) ? piece.w : piece.y) ^ 0x80808080u;
+        // the biased byte sits in bits 3-10 of its half (8 (q + 128) as a bit pattern: see the Q4_K tile)
         const float4_t d4 = __builtin_amdgcn_mfma_f32_16x16x32_f16(
-            a, as_half8(even_bytes(w0), odd_bytes(w0), even_bytes(w1), odd_bytes(w1)), zero, 0, 0, 0);
+            a, as_half8(even_bytes(w0) << 3, odd_bytes(w0) << 3, even_bytes(w1) << 3, odd_bytes(w1) << 3), zero, 0, 0, 0);
         if (lane_group == uint32_t(cg)) own = d4;
     }
     const float d = h2f(t.d);
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-        const float v = fmaf(mult[r * per_mult], own[2 * r] + own[2 * r + 1], -128.0f * xs32[r * per_row]);
+        const float v = fmaf(0.125f * mult[r * per_mult], own[2 * r] + own[2 * r + 1], -128.0f * xs32[r * per_row]);
         acc[r] = fmaf(d, v, acc[r]);
     }
 }

@@ -7,11 +7,12 @@ with the reference's own criteria:
                                                 sqrt(hidden)) and as head (3e-5 of a double dot)
   tests/tensor/gemma3_metal_tests.cpp:1290-1365  Q4_K weights that are the difference of two terms 1365 times larger,
                                                 against signed activations, within the same gamma bound on the SMALL
-                                                weights: the canonical-layout GEMV meets it; the packed GEMV, which keeps
-                                                d sc sum(q x) and dmin m sum(x) apart until the end of a group, is held to
-                                                twice the bound (measured: up to 1.13 of it on 2 of 10 rows at K = 3840,
-                                                0.14-0.37 at K = 15360) -- a stated deviation, far inside the 1e-3 relative
-                                                that the logits are asked to keep
+                                                weights: both the canonical-layout GEMV and the packed GEMV (which keeps
+                                                d sc sum(q x) and dmin m sum(x) apart until the end of a group) meet it
+                                                (measured: 0.45 and 0.28 of it at K = 3840, 0.13 and 0.06 at K = 15360)
+  tests/tensor/tensor_backend_tests.cpp:964-1158 the 17 small-batch / tile-boundary cases and the 17 parallel-projection
+                                                cases (12B block counts, odd column counts, a head that starts inside the
+                                                input), activations with a 512-fold range inside every 32-group
 Column counts are padded to the 64-column tiles of the packed layout with zero blocks."""
 import math
 
@@ -121,4 +122,140 @@ def test_q4k_scale_min_cancellation(hip, width):
         worst["canonical"] = max(worst["canonical"], float((np.abs(canonical - reference) / bound).max()))
     print("cancellation fixture, K = %d: packed %.2f, canonical %.2f of the reference's bound" % (width, worst["packed"], worst["canonical"]), flush=True)
     assert worst["canonical"] <= 1.0
-    assert worst["packed"] <= 2.0
+    assert worst["packed"] <= 1.0
+
+
+# tests/tensor/tensor_backend_tests.cpp:964-1067: the reference's 17 (rows, 256-blocks of K, columns) cases around its
+# small-batch / tile boundaries, production block counts and the 64-column boundary, on the stress matrices, with
+# every 17th activation 16 times and every 13th 1/32 of its pattern value.
+PROJECTION_CASES = [(2, 1, 1), (2, 14, 3), (2, 16, 4), (2, 56, 5), (3, 2, 2), (4, 14, 3), (5, 16, 4), (6, 56, 5), (7, 1, 63),
+                    (8, 2, 64), (9, 14, 65), (15, 16, 5), (16, 56, 4), (17, 1, 3), (31, 2, 2), (32, 14, 1), (33, 16, 5)]
+
+
+@pytest.mark.parametrize("dtype", [1, 2])
+@pytest.mark.parametrize("rows,blocks,columns", PROJECTION_CASES)
+def test_small_batch_and_tiled_projection_cases(hip, gfo, dtype, rows, blocks, columns):
+    """The reference holds its backend to 0.05-2.0 absolute + 1e-5..2e-2 relative of a float reference here and,
+    up to 8 rows, to bit-equality with one-row calls.  Here every row of the matrix path is held to the operator
+    bound gamma / (1 - gamma) sum|x w| + 1e-6 of a double dot, and the decode path (one- and two-row calls) is
+    bit-equal row by row and within 2e-5 of the row RMS of the matrix path."""
+    K = blocks * 256
+    x = rg.projection_values(rows, K).reshape(-1)
+    i = np.arange(x.size)
+    x = np.where(i % 17 == 0, x * np.float32(16.0), np.where(i % 13 == 0, x * np.float32(0.03125), x)).astype(np.float32)
+    x = x.reshape(rows, K)
+    w = rg.q4k_stress(K, columns, rows) if dtype == 1 else rg.q6k_stress(K, columns, rows)
+    N = (columns + 63) // 64 * 64
+    dense = gfo.dequant(dtype, w).reshape(columns, K).astype(np.float64)
+    tiles = hip.repack(dtype, dev(padded(w, dtype, K, columns, N)), K, N)
+    xd = dev(x)
+    y = hip.prefill_gemm(dtype, tiles, hip.prefill_pack(xd), rows, K, N).cpu().numpy()
+    assert np.all(y[:, columns:] == 0)
+    gamma = (K // 32 + 32) * np.finfo(np.float32).eps
+    products = np.abs(dense)[None, :, :] * np.abs(x.astype(np.float64))[:, None, :]
+    bound = gamma / (1.0 - gamma) * products.sum(2) + 1e-6
+    exact = x.astype(np.float64) @ dense.T
+    worst = float((np.abs(y[:, :columns] - exact) / bound).max())
+    assert worst <= 1.0, worst
+    rms = np.sqrt((exact ** 2).mean(1)) + 1e-30
+    for r in (0, 1, rows - 1):
+        one = dev(x[r:r + 1])
+        single = hip.gemv_packed(dtype, tiles, one, hip.group_sums(one), N).cpu().numpy()[0]
+        assert float((np.abs(single[:columns] - exact[r]) / bound[r]).max()) <= 1.0
+        assert np.all(np.abs(single[:columns].astype(np.float64) - y[r, :columns]) <= 2e-5 * rms[r])
+        if r + 1 < rows:
+            two = dev(x[r:r + 2])
+            both = hip.gemv_packed(dtype, tiles, two, hip.group_sums(two), N).cpu().numpy()
+            assert np.array_equal(both[0].view(np.uint32), single.view(np.uint32)), "one-row and two-row calls differ"
+    print("rows %d blocks %d columns %d dtype %d: matrix path at %.3f of the bound" % (rows, blocks, columns, dtype, worst), flush=True)
+
+
+# tests/tensor/tensor_backend_tests.cpp:1069-1158: the 12B model's K dimensions (15, 16 and 60 blocks) with odd column
+# counts, batches of 1-8 rows and a head that starts `head_offset` rows into the input.
+PARALLEL_CASES = [(2, 1, 1, 1), (1, 15, 3, 0), (2, 15, 5, 1), (3, 15, 7, 3), (4, 15, 33, 4), (5, 15, 65, 5), (1, 16, 5, 1),
+                  (2, 16, 67, 3), (3, 16, 3, 4), (4, 16, 4, 5), (5, 16, 7, 1), (1, 60, 3, 3), (2, 60, 4, 4), (3, 60, 5, 5),
+                  (4, 60, 5, 1), (5, 60, 7, 3), (8, 60, 3, 1)]
+
+
+@pytest.mark.parametrize("dtype", [1, 2])
+@pytest.mark.parametrize("rows,blocks,columns,head_offset", PARALLEL_CASES)
+def test_parallel_projection_keeps_scalar_bits(hip, gfo, dtype, rows, blocks, columns, head_offset):
+    """A batch of verify rows (here: calls of at most two rows, the width of a verify pass) and a head over rows
+    that start `head_offset` into the input give, row by row, the bits of one-row calls; every value is finite and
+    within the reference's 0.05 (Q4_K) / 0.1 (Q6_K) + 1e-5 |e| of a double dot; the row after the batch in the
+    output keeps its NaN pattern.  (The reference compares with a sequential fp32 sum.  At these magnitudes --
+    sum|x w| around 2e5 at 15 blocks -- that sum's own rounding error reaches 0.1, more than the tolerance: it
+    passes there because the reference's kernel shares most of the sum's order.  The oracle's sequential sum is
+    printed beside the kernel's error for comparison.)"""
+    import torch
+    K = blocks * 256
+    input_rows = rows + head_offset
+    i = np.arange(input_rows * K)
+    x = rg.projection_values(input_rows, K).reshape(-1)
+    x = (x * np.where(i % 17 == 0, np.float32(16.0), np.where(i % 13 == 0, np.float32(0.03125), np.float32(1.0))).astype(np.float32)
+         + np.float32(0.00037) * (i % 11).astype(np.float32)).astype(np.float32).reshape(input_rows, K)
+    w = rg.q4k_stress(K, columns, rows) if dtype == 1 else rg.q6k_stress(K, columns, rows)
+    N = (columns + 63) // 64 * 64
+    tiles = hip.repack(dtype, dev(padded(w, dtype, K, columns, N)), K, N)
+    sequential = gfo.gemv(dtype, padded(w, dtype, K, columns, N), x, N, threads=4)[:, :columns]
+    dense = gfo.dequant(dtype, w).reshape(columns, K).astype(np.float64)
+    expected = x.astype(np.float64) @ dense.T
+    xd = dev(x)
+    worst = 0.0
+
+    def one(r):
+        xr = xd[r:r + 1].contiguous()
+        return hip.gemv_packed(dtype, tiles, xr, hip.group_sums(xr), N).cpu().numpy()[0]
+
+    scalar = [one(r) for r in range(input_rows)]
+    for first in (0, head_offset):
+        out = torch.full((rows + 1, N), float("nan"), dtype=torch.float32, device="cuda")
+        out.view(torch.int32)[...] = 0x7fc00000
+        for r in range(0, rows, 2):
+            n = min(2, rows - r)
+            xr = xd[first + r:first + r + n].contiguous()
+            hip.gemv_packed(dtype, tiles, xr, hip.group_sums(xr), N, out=out[r:r + n])
+        got = out.cpu().numpy()
+        assert np.all(got[rows].view(np.uint32) == 0x7fc00000), "the row after the batch was written"
+        for r in range(rows):
+            assert np.all(np.isfinite(got[r]))
+            assert np.array_equal(got[r].view(np.uint32), scalar[first + r].view(np.uint32)), (first, r)
+            e = expected[first + r]
+            tol = (0.05 if dtype == 1 else 0.1) + 1e-5 * np.abs(e)
+            assert np.all(np.abs(got[r, :columns] - e) <= tol), float(np.abs(got[r, :columns] - e).max())
+            worst = max(worst, float(np.abs(got[r, :columns] - e).max()))
+    print("rows %d blocks %d columns %d dtype %d: worst error %.2e, the sequential fp32 sum's %.2e"
+          % (rows, blocks, columns, dtype, worst, float(np.abs(sequential - expected).max())), flush=True)
+
+
+@pytest.mark.parametrize("dtype,width", [(0, 640), (0, 2048), (1, 256), (1, 3840), (1, 15360), (2, 3840), (2, 15360)])
+def test_range_inside_a_group_costs_no_precision(hip, gfo, dtype, width):
+    """Activations whose magnitudes span 2^9 inside every 32-group and use all their mantissa bits: the packed GEMV
+    and the prefill GEMM stay within 2 eps sum|x w| of a double dot (the canonical-layout GEMV: 0.1-0.5).  The
+    quants enter the matrix instruction as fp16 bit patterns below 2048, which it does not normalise: with the
+    pattern's leading zeros in place (a nibble in bits 0-3) every product loses that many bits once a sum's
+    products are aligned, and these operands came out 70 times worse than the canonical kernel (up to 200 eps
+    on a single group); the quants therefore sit near the top of the 11-bit window (bits 4-7 for Q4_K, 4-9
+    for Q6_K, 3-10 for the biased Q8_0 byte; the prefill GEMM's scaled quants reach it by themselves)."""
+    from guffin_amd import synth
+    columns, rows = 64, 4
+    i = np.arange(rows * width)
+    x = rg.projection_values(rows, width).reshape(-1)
+    x = (x * np.where(i % 17 == 0, np.float32(16.0), np.where(i % 13 == 0, np.float32(0.03125), np.float32(1.0))).astype(np.float32)
+         + np.float32(0.00037) * (i % 11).astype(np.float32)).astype(np.float32).reshape(rows, width)
+    w = (synth.make_weight(0, width, columns, 3) if dtype == 0 else
+         rg.q4k_stress(width, columns, 2) if dtype == 1 else rg.q6k_stress(width, columns, 2))
+    dense = gfo.dequant(dtype, w).reshape(columns, width).astype(np.float64)
+    stream = dev(w)
+    tiles = hip.repack(dtype, stream, width, columns)
+    xd = dev(x)
+    exact = x.astype(np.float64) @ dense.T
+    unit = np.finfo(np.float32).eps * (np.abs(x.astype(np.float64)) @ np.abs(dense).T)
+    two = xd[:2].contiguous()
+    packed = hip.gemv_packed(dtype, tiles, two, hip.group_sums(two), columns).cpu().numpy()
+    canonical = hip.gemv(dtype, stream, two, columns).cpu().numpy()
+    matrix = hip.prefill_gemm(dtype, tiles, hip.prefill_pack(xd), rows, width, columns).cpu().numpy()
+    worst = [float((np.abs(packed - exact[:2]) / unit[:2]).max()), float((np.abs(matrix - exact) / unit).max()),
+             float((np.abs(canonical - exact[:2]) / unit[:2]).max())]
+    print("dtype %d K %d: packed %.2f, matrix path %.2f, canonical %.2f eps sum|x w|" % (dtype, width, *worst), flush=True)
+    assert worst[0] <= 2.0 and worst[1] <= 2.0, worst
