@@ -97,3 +97,19 @@ def pattern(count, scale=0.15):
     a = np.sin((i % 8191).astype(np.float32) * np.float32(0.071)).astype(np.float32) * scale
     b = np.cos((i % 997).astype(np.float32) * np.float32(0.027)).astype(np.float32) * scale * np.float32(0.37)
     return (a + b).astype(np.float32)
+
+
+def q8_0_from_values(values):
+    """quantize_f16_gguf_weight_q8_0 (src/tensor/quantization.cpp:634-676) of a [shared][columns] value table
+    stored the way tensor_f16_gguf_matrix stores it (a column's `shared` halves contiguous): per 32 elements the
+    scale is max|v| / 127 in float, kept as a half, and the quants are round-half-away(v / scale)."""
+    shared, columns = values.shape
+    v = values.astype(np.float16).astype(np.float32).T.reshape(columns, shared // 32, 32)
+    scale = (np.abs(v).max(2) / np.float32(127.0)).astype(np.float32)
+    inverse = np.where(scale == 0, np.float32(0), np.float32(1.0) / np.where(scale == 0, np.float32(1), scale)).astype(np.float32)
+    scaled = (v * inverse[:, :, None]).astype(np.float32)
+    quants = (np.sign(scaled) * np.floor(np.abs(scaled) + np.float32(0.5))).astype(np.int8)
+    blocks = np.zeros((columns, shared // 32, 34), np.uint8)
+    blocks[:, :, 0:2] = np.ascontiguousarray(scale.astype(np.float16)).view(np.uint8).reshape(columns, shared // 32, 2)
+    blocks[:, :, 2:] = np.ascontiguousarray(quants).view(np.uint8)
+    return blocks.reshape(-1)

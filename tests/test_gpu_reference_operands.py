@@ -13,6 +13,8 @@ with the reference's own criteria:
   tests/tensor/tensor_backend_tests.cpp:964-1158 the 17 small-batch / tile-boundary cases and the 17 parallel-projection
                                                 cases (12B block counts, odd column counts, a head that starts inside the
                                                 input), activations with a 512-fold range inside every 32-group
+  tests/tensor/tensor_backend_tests.cpp:1352-1472 one-row decode at the reference's block and column counts; the Q8_0
+                                                output projection on weights through the reference's quantiser
 Column counts are padded to the 64-column tiles of the packed layout with zero blocks."""
 import math
 
@@ -267,3 +269,53 @@ def test_range_inside_a_group_costs_no_precision(hip, gfo, dtype, width):
              float((np.abs(canonical - exact[:2]) / unit[:2]).max())]
     print("dtype %d K %d: packed %.2f, matrix path %.2f, canonical %.2f eps sum|x w|" % (dtype, width, *worst), flush=True)
     assert worst[0] <= 2.0 and worst[1] <= 2.0, worst
+
+
+@pytest.mark.parametrize("dtype", [1, 2])
+@pytest.mark.parametrize("blocks", [1, 2, 14, 16, 56])
+def test_decode_boundary_cases(hip, gfo, dtype, blocks):
+    """tests/tensor/tensor_backend_tests.cpp:1352-1392: one row against 1-7 columns of the stress matrices at the
+    reference's block counts, every 17th activation times -8 and every 11th times 1/8; the reference's tolerance
+    (0.1 for Q4_K, 0.25 for Q6_K, + 1e-5 |e|), here against a double dot."""
+    K = blocks * 256
+    x = rg.projection_values(1, K).reshape(-1)
+    i = np.arange(K)
+    x = np.where(i % 17 == 0, x * np.float32(-8.0), np.where(i % 11 == 0, x * np.float32(0.125), x)).astype(np.float32).reshape(1, K)
+    xd = dev(x)
+    receipt = hip.group_sums(xd)
+    for columns in (1, 2, 3, 4, 5, 7):
+        w = rg.q4k_stress(K, columns, blocks) if dtype == 1 else rg.q6k_stress(K, columns, blocks)
+        dense = gfo.dequant(dtype, w).reshape(columns, K).astype(np.float64)
+        tiles = hip.repack(dtype, dev(padded(w, dtype, K, columns)), K, 64)
+        y = hip.gemv_packed(dtype, tiles, xd, receipt, 64).cpu().numpy()[0]
+        exact = dense @ x[0].astype(np.float64)
+        assert np.all(y[columns:] == 0)
+        assert np.all(np.abs(y[:columns] - exact) <= (0.1 if dtype == 1 else 0.25) + 1e-5 * np.abs(exact))
+
+
+@pytest.mark.parametrize("shared", [64, 3584])
+def test_q8_0_output_projection(hip, gfo, shared):
+    """tests/tensor/tensor_backend_tests.cpp:1423-1472: weights ((i % 31) - 15) / 37 through the reference's Q8_0
+    quantiser, activations ((i % 17) - 8) / 9, one and two rows within 2e-4 of the CPU path (here the oracle's
+    sequential GEMV); rows of the two-row call equal the one-row calls (bit for bit here, 2e-4 there)."""
+    columns = 5
+    a = ((np.arange(2 * shared) % 17).astype(np.float32) - 8) / np.float32(9.0)
+    wv = (((np.arange(shared * columns) % 31).astype(np.float32) - 15) / np.float32(37.0)).reshape(shared, columns)
+    w = rg.q8_0_from_values(wv)
+    stream = np.concatenate([w, np.zeros((64 - columns) * (shared // 32) * 34, np.uint8)])
+    dense = gfo.dequant(0, w).reshape(columns, shared)
+    assert np.abs(dense - wv.T).max() <= np.abs(wv).max() / 127.0        # the quantiser restated: half a step at most
+    tiles = hip.repack(0, dev(stream), shared, 64)
+    x = a.reshape(2, shared).astype(np.float32)
+    both = None
+    for rows in (1, 2):
+        xd = dev(x[:rows])
+        got = hip.gemv_packed(0, tiles, xd, hip.group_sums(xd), 64).cpu().numpy()
+        cpu = gfo.gemv(0, stream, x[:rows], 64, threads=1)
+        assert np.all(np.abs(got[:, :columns] - cpu[:, :columns]) <= 2e-4)
+        if rows == 2:
+            both = got
+    for row in range(2):
+        xr = dev(x[row:row + 1])
+        single = hip.gemv_packed(0, tiles, xr, hip.group_sums(xr), 64).cpu().numpy()[0]
+        assert np.array_equal(single.view(np.uint32), both[row].view(np.uint32))

@@ -35,3 +35,22 @@ def test_plain_matrices_and_patterns(gfo):
     assert v[0, 0] == -0.25 and set(np.unique(v * 8)) <= set(range(-5, 6))
     p = rg.pattern(10, 0.03)
     assert abs(p[0] - 0.03 * 0.37) < 1e-7 and np.abs(p).max() < 0.03 * 1.37 + 1e-6
+
+
+def test_q8_0_quantiser_restated(gfo):
+    """The Q8_0 quantiser of the reference's tests: a block's largest element maps to +-127, every decoded value is
+    within half a step of its source, the scale is the half nearest max / 127, and a zero block stays zero."""
+    shared, columns = 128, 5
+    values = (((np.arange(shared * columns) % 31).astype(np.float32) - 15) / np.float32(37.0)).reshape(shared, columns)
+    values[32:64, 2] = 0.0
+    stream = rg.q8_0_from_values(values)
+    blocks = stream.reshape(columns, shared // 32, 34)
+    quants = blocks[:, :, 2:].view(np.int8)
+    scales = np.ascontiguousarray(blocks[:, :, 0:2]).view(np.float16).reshape(columns, shared // 32).astype(np.float32)
+    source = values.astype(np.float16).astype(np.float32).T.reshape(columns, shared // 32, 32)
+    peak = np.abs(source).max(2)
+    assert np.array_equal(scales, (peak / np.float32(127.0)).astype(np.float16).astype(np.float32))
+    assert np.all(np.abs(quants).max(2)[peak > 0] == 127) and np.all(quants[2, 1] == 0) and scales[2, 1] == 0
+    decoded = gfo.dequant(0, stream).reshape(columns, shared // 32, 32)
+    step = (peak / 127.0)[:, :, None]
+    assert np.all(np.abs(decoded - source) <= 0.5 * step * (1 + 2.0 ** -10) + 1e-12)
