@@ -41,7 +41,7 @@ struct AttnArgs {
     const uint32_t* ancestors;
     float* part_out;             // [rows][q_heads][partitions][hd]
     float* part_ml;              // [rows][q_heads][partitions][2]
-    uint32_t rows, q_heads, kv_heads, hd, ring_mask, tp, partitions, private_rows;
+    uint32_t rows, q_heads, kv_heads, hd, ring_mask, tp, span, partitions, private_rows;   // span: tokens the last partition may hold (>= tp)
     float scale;
     // fused mode: q, k, v arrive as the projections' partial planes; every workgroup prepares
     // the query heads it serves (head norm, rotation) and the partition that holds a private
@@ -51,6 +51,9 @@ struct AttnArgs {
     const float* q_norm; const float* k_norm; const float2* rope;   // rope: [rows][hd/2] (cos, sin)
     uint16_t* priv_k_out; uint16_t* priv_v_out;
     float eps; uint32_t* status;
+    // the rows' schedule words and ancestor masks when the host knows them (contiguous rows at a host-known
+    // position): they arrive with the launch arguments instead of through two dependent trips to memory
+    uint32_t inline_schedule, sched[kMaxRows][4], amask[kMaxRows];
 };
 
 // One head row (hd = 256) by one wave, in registers: lane l holds columns l, l+64, l+128, l+192.
@@ -89,6 +92,12 @@ __device__ __forceinline__ void finish_head_row(HeadRow& h, bool norm, bool rota
     }
 }
 
+// A workgroup barrier for data that moves through LDS: it waits for this wave's LDS operations only.
+// (__syncthreads() also waits for every vector load in flight -- here the key rows requested before the
+// queries are prepared and the value rows requested before the softmax, which are meant to stay in flight
+// across it.)  Nothing a wave stores to global memory in this kernel is read by another wave of the launch.
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
 __device__ __forceinline__ float dot2(float acc, uint32_t packed_half2, float a, float b) {
     const half2_t h = __builtin_bit_cast(half2_t, packed_half2);
     acc = fmaf(static_cast<float>(h.x), a, acc);
@@ -101,7 +110,7 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(AttnArgs a) {
     constexpr int NQ = ROWS * GROUP;
     extern __shared__ float lds[];
     float* sc = lds;                          // [NQ][tp] scores, then probabilities
-    float* merge = lds + NQ * a.tp;           // [4][NQ][HD]
+    float* merge = lds + NQ * a.span;         // [4][NQ][HD]
     float* q_s = merge + 4 * NQ * HD;         // fused: [NQ][HD] prepared queries
     __shared__ float s_max[NQ], s_sum[NQ];
     __shared__ __attribute__((aligned(16))) uint16_t k_s[FUSED ? ROWS : 1][HD], v_s[FUSED ? ROWS : 1][HD];
@@ -133,7 +142,11 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(AttnArgs a) {
 #pragma unroll
     for (int r = 0; r < ROWS; ++r) {
         bfirst[r] = 0; bend[r] = 0; amask[r] = 0;
-        {
+        if (a.inline_schedule) {
+            bfirst[r] = a.sched[r][0]; bend[r] = a.sched[r][0] + a.sched[r][1];
+            if (a.sched[r][1]) { u_first = min(u_first, bfirst[r]); u_end = max(u_end, bend[r]); }
+            amask[r] = a.amask[r];
+        } else {
             const uint32_t* s = a.schedule + 4 * r;
             bfirst[r] = s[0]; bend[r] = s[0] + s[1];
             if (s[1]) { u_first = min(u_first, s[0]); u_end = max(u_end, s[0] + s[1]); }
@@ -142,7 +155,9 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(AttnArgs a) {
     }
     if (u_end == 0) { u_first = 0; }
     const uint32_t n_ring = u_end - u_first, n_total = n_ring + a.private_rows;
-    const uint32_t t0 = part * a.tp, t1 = min(t0 + a.tp, n_total);
+    // the last partition takes what is left (at most `span` tokens: the launch has one partition fewer when a
+    // handful of tokens -- the private rows -- would otherwise need a workgroup of their own on a full chip)
+    const uint32_t t0 = part * a.tp, t1 = part + 1 == a.partitions ? min(t0 + a.span, n_total) : min(t0 + a.tp, n_total);
 
     // ---- keys: four rounds of loads are issued before their dot products so that a wave keeps
     // 16 key rows (8 KB) in flight; in fused mode the first batch travels during the preparation
@@ -220,7 +235,7 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(AttnArgs a) {
             }
             if (bad && a.status) atomicOr(a.status, GUFFIN_STATUS_KV_NONFINITE);
         }
-        __syncthreads();
+        lds_barrier();
     }
     // ---- pass 1: scores ------------------------------------------------------------
     {
@@ -233,12 +248,12 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(AttnArgs a) {
 #pragma unroll
             for (int i = 0; i < 16; ++i) qv[n][i] = qp[i] * a.scale;
         }
-        for (uint32_t tb = tb_first; tb < t0 + a.tp; tb += 16 * U) {
+        for (uint32_t tb = tb_first; tb < t0 + a.span; tb += 16 * U) {
             if (!FUSED || tb != tb_first) load_keys(tb);
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 const uint32_t t = tb + 16 * u;
-                if (t >= t0 + a.tp) break;
+                if (t >= t0 + a.span) break;
                 const bool in_range = t < t1, is_priv = t >= n_ring;
                 const uint32_t pos = u_first + t, prow = t - n_ring;
                 if (FUSED && in_range && is_priv) {
@@ -252,10 +267,7 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(AttnArgs a) {
                     s[n] = 0.f;
 #pragma unroll
                     for (int i = 0; i < 8; ++i) s[n] = dot2(s[n], kw[i], qv[n][2 * i], qv[n][2 * i + 1]);
-                    s[n] += __shfl_xor(s[n], 8, kWave);
-                    s[n] += __shfl_xor(s[n], 4, kWave);
-                    s[n] += __shfl_xor(s[n], 2, kWave);
-                    s[n] += __shfl_xor(s[n], 1, kWave);
+                    s[n] = row16_sum(s[n]);
                 }
                 if (seg == 0) {
 #pragma unroll
@@ -263,31 +275,31 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(AttnArgs a) {
                         const uint32_t r = n / group;
                         const bool valid = in_range && (is_priv ? ((amask[r] >> prow) & 1u) != 0
                                                                 : (pos >= bfirst[r] && pos < bend[r]));
-                        sc[n * a.tp + (t - t0)] = valid ? s[n] : -INFINITY;
+                        sc[n * a.span + (t - t0)] = valid ? s[n] : -INFINITY;
                     }
                 }
             }
         }
     }
     if constexpr (FUSED) load_values(vb_first);  // in flight during the softmax
-    __syncthreads();
+    lds_barrier();
 
     // ---- softmax over the partition, one wave per query ----------------------------------
     for (uint32_t n = wv; n < NQ; n += 4) {
         float m = -INFINITY;
-        for (uint32_t i = lane; i < a.tp; i += 64) m = fmaxf(m, sc[n * a.tp + i]);
+        for (uint32_t i = lane; i < a.span; i += 64) m = fmaxf(m, sc[n * a.span + i]);
         m = wave_max(m);
         float l = 0.f;
-        for (uint32_t i = lane; i < a.tp; i += 64) {
-            const float v = sc[n * a.tp + i];
+        for (uint32_t i = lane; i < a.span; i += 64) {
+            const float v = sc[n * a.span + i];
             const float p = v == -INFINITY ? 0.f : expf(v - m);
-            sc[n * a.tp + i] = p;
+            sc[n * a.span + i] = p;
             l += p;
         }
         l = wave_sum(l);
         if (lane == 0) { s_max[n] = m; s_sum[n] = l; }
     }
-    __syncthreads();
+    lds_barrier();
     // ---- pass 2: values; halves are combined by a lane exchange, waves via LDS ------------
     {
         float acc[NQ][8];
@@ -305,7 +317,7 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(AttnArgs a) {
                 const uint32_t w4[4] = {vv[u].x, vv[u].y, vv[u].z, vv[u].w};
 #pragma unroll
                 for (int n = 0; n < NQ; ++n) {
-                    const float p = sc[n * a.tp + (t - t0)];
+                    const float p = sc[n * a.span + (t - t0)];
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
                         const half2_t h = __builtin_bit_cast(half2_t, w4[i]);
@@ -326,7 +338,7 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(AttnArgs a) {
             }
         }
     }
-    __syncthreads();
+    lds_barrier();
     for (uint32_t i = threadIdx.x; i < NQ * HD; i += 256) {
         const uint32_t n = i / HD, d = i % HD;
         const float v = (merge[(0 * NQ + n) * HD + d] + merge[(1 * NQ + n) * HD + d])
@@ -412,7 +424,7 @@ template <int ROWS, int GROUP>
 int launch_partial(hipStream_t s, const AttnArgs& a) {
     constexpr int NQ = ROWS * GROUP;
     const bool fused = a.q_raw != nullptr;
-    const size_t lds = (size_t(NQ) * a.tp + size_t(4) * NQ * 256 + (fused ? size_t(NQ) * 256 : 0)) * sizeof(float);
+    const size_t lds = (size_t(NQ) * a.span + size_t(4) * NQ * 256 + (fused ? size_t(NQ) * 256 : 0)) * sizeof(float);
     if (fused)
         hipLaunchKernelGGL((attn_partial_kernel<ROWS, GROUP, 256, true>), dim3(a.partitions, a.kv_heads), dim3(256), lds, s, a);
     else
@@ -425,15 +437,33 @@ int launch_partial(hipStream_t s, const AttnArgs& a) {
 
 using namespace guffin;
 
+namespace {
+struct AttentionSplit { uint32_t partitions, tp, span; };
+AttentionSplit attention_split(uint32_t max_tokens, uint32_t kv_heads) {
+    uint32_t tp = 128;
+    const uint32_t floor_tp = ((max_tokens + 31) / 32) * kv_heads < 64 ? 16u : 32u;
+    while (tp > floor_tp && ((max_tokens + tp - 1) / tp) * kv_heads < 256) tp >>= 1;
+    uint32_t partitions = (max_tokens + tp - 1) / tp;
+    tp = (((max_tokens + partitions - 1) / partitions) + 15u) & ~15u;   // whole rounds of 16 tokens per workgroup
+    partitions = (max_tokens + tp - 1) / tp;
+    uint32_t span = tp;
+    // A last partition of at most 16 tokens that alone pushes the launch past one workgroup per CU (1025 tokens
+    // on 8 KV heads: 33 x 8 = 264) is folded into the one before it: the eight workgroups that would share a
+    // CU with another finish 2 us after everybody else.
+    if (partitions > 1) {
+        const uint32_t rem = max_tokens - (partitions - 1) * tp;
+        if (rem <= 16 && partitions * kv_heads > 256 && (partitions - 1) * kv_heads <= 256) { partitions -= 1; span = tp + 16; }
+    }
+    return {partitions, tp, span};
+}
+}  // namespace
+
 extern "C" uint32_t guffin_hip_attention_partitions(uint32_t max_tokens, uint32_t kv_heads) {
     // tokens per partition: aim at >= 256 workgroups, between 32 and 128 tokens each; a context so
     // small that 32-token partitions give fewer than 64 workgroups (the drafter's window) is cut into
     // 16-token partitions, which shortens every workgroup's chain of dependent steps
     if (max_tokens == 0 || kv_heads == 0) return 0;
-    uint32_t tp = 128;
-    const uint32_t floor_tp = ((max_tokens + 31) / 32) * kv_heads < 64 ? 16u : 32u;
-    while (tp > floor_tp && ((max_tokens + tp - 1) / tp) * kv_heads < 256) tp >>= 1;
-    return (max_tokens + tp - 1) / tp;
+    return attention_split(max_tokens, kv_heads).partitions;
 }
 
 namespace {
@@ -447,7 +477,7 @@ int attention_decode(void* stream, const float* q, const FusedInputs* fused, con
                      void* priv_k, void* priv_v, const uint32_t* schedule, const uint32_t* ancestors, float* out,
                      float* out_sums, float* partial_out, float* partial_ml, uint32_t rows, uint32_t private_rows,
                      uint32_t max_tokens, uint32_t ring_mask, uint32_t q_heads, uint32_t kv_heads, uint32_t head_dim,
-                     float scale, uint32_t* status) {
+                     float scale, uint32_t* status, const uint32_t* host_schedule = nullptr, const uint32_t* host_amask = nullptr) {
     if ((!q && !fused) || !ring_k || !ring_v || !priv_k || !priv_v || !schedule || !ancestors || !out || !partial_out || !partial_ml)
         return fail(GUFFIN_E_ARG, "attention_decode: null pointer");
     if (rows == 0 || rows > kMaxRows || private_rows > 32) return fail(GUFFIN_E_SHAPE, "attention_decode: rows must be 1 or 2, private rows <= 32");
@@ -467,10 +497,16 @@ int attention_decode(void* stream, const float* q, const FusedInputs* fused, con
     a.priv_k = static_cast<const uint16_t*>(priv_k); a.priv_v = static_cast<const uint16_t*>(priv_v);
     a.schedule = schedule; a.ancestors = ancestors; a.part_out = partial_out; a.part_ml = partial_ml;
     a.rows = rows; a.q_heads = q_heads; a.kv_heads = kv_heads; a.hd = head_dim; a.ring_mask = ring_mask;
-    a.partitions = guffin_hip_attention_partitions(max_tokens, kv_heads);
-    a.tp = (max_tokens + a.partitions - 1) / a.partitions;
-    a.tp = (a.tp + 15u) & ~15u;  // whole rounds of 16 tokens per workgroup
+    const AttentionSplit split = attention_split(max_tokens, kv_heads);
+    a.partitions = split.partitions; a.tp = split.tp; a.span = split.span;
     a.private_rows = private_rows; a.scale = scale;
+    if (host_schedule && host_amask) {
+        a.inline_schedule = 1;
+        for (uint32_t r = 0; r < rows; ++r) {
+            for (int k = 0; k < 4; ++k) a.sched[r][k] = host_schedule[4 * r + k];
+            a.amask[r] = host_amask[r];
+        }
+    }
     if (fused) {
         if (!fused->q_raw || !fused->k_raw || !fused->v_raw || !fused->rope)
             return fail(GUFFIN_E_ARG, "qkv_attention: null pointer");
@@ -514,6 +550,24 @@ extern "C" int guffin_hip_attention_decode(void* stream, const float* q, const v
                             schedule, ancestors, out, out_sums, partial_out, partial_ml, rows, private_rows, max_tokens,
                             ring_mask, q_heads, kv_heads, head_dim, scale, status);
 }
+
+// guffin_hip_qkv_attention for contiguous rows whose schedule the host knows: the same words the device copy
+// holds (`schedule`, still passed) travel as launch arguments.
+namespace guffin {
+int qkv_attention_scheduled(void* stream, const float* q_raw, const float* k_raw, const float* v_raw, uint32_t planes,
+                            uint64_t q_plane_stride, uint64_t k_plane_stride, uint64_t v_plane_stride, const float* q_norm,
+                            const float* k_norm, const float* rope_table, float eps, const void* ring_k, const void* ring_v,
+                            void* priv_k, void* priv_v, const uint32_t* schedule, const uint32_t* ancestors,
+                            const uint32_t* host_schedule, const uint32_t* host_amask, float* out, float* out_sums,
+                            float* partial_out, float* partial_ml, uint32_t rows, uint32_t max_tokens, uint32_t ring_mask,
+                            uint32_t q_heads, uint32_t kv_heads, uint32_t head_dim, float scale, uint32_t* status) {
+    const FusedInputs f {q_raw, k_raw, v_raw, planes, q_plane_stride, k_plane_stride, v_plane_stride, q_norm, k_norm,
+                         rope_table, eps};
+    return attention_decode(stream, nullptr, &f, ring_k, ring_v, priv_k, priv_v, schedule, ancestors, out, out_sums,
+                            partial_out, partial_ml, rows, rows, max_tokens, ring_mask, q_heads, kv_heads, head_dim,
+                            scale, status, host_schedule, host_amask);
+}
+}  // namespace guffin
 
 extern "C" int guffin_hip_qkv_attention(void* stream, const float* q_raw, const float* k_raw, const float* v_raw,
                                         uint32_t planes, uint64_t q_plane_stride, uint64_t k_plane_stride,

@@ -36,6 +36,15 @@ int resident_launch(hipStream_t stream, const guffin_model_desc& m, uint32_t row
                     const void* u_receipt_in, float* x_out, float* u_out, void* u_receipt_out, uint32_t max_ring_tokens,
                     uint32_t* status);
 
+// ---- attention with a host-known schedule (attention.hip), used by the block graph of plan.hip --------
+int qkv_attention_scheduled(void* stream, const float* q_raw, const float* k_raw, const float* v_raw, uint32_t planes,
+                            uint64_t q_plane_stride, uint64_t k_plane_stride, uint64_t v_plane_stride, const float* q_norm,
+                            const float* k_norm, const float* rope_table, float eps, const void* ring_k, const void* ring_v,
+                            void* priv_k, void* priv_v, const uint32_t* schedule, const uint32_t* ancestors,
+                            const uint32_t* host_schedule, const uint32_t* host_amask, float* out, float* out_sums,
+                            float* partial_out, float* partial_ml, uint32_t rows, uint32_t max_tokens, uint32_t ring_mask,
+                            uint32_t q_heads, uint32_t kv_heads, uint32_t head_dim, float scale, uint32_t* status);
+
 // ---- typed loads at the alignment a GGUF block stream guarantees ------------
 struct __attribute__((packed, aligned(4))) U4a4 { uint32_t x, y, z, w; };
 struct __attribute__((packed, aligned(2))) U4a2 { uint32_t x, y, z, w; };
@@ -80,15 +89,37 @@ __device__ __forceinline__ float sb1(uint32_t v) { return static_cast<float>(sta
 __device__ __forceinline__ float sb2(uint32_t v) { return static_cast<float>(static_cast<int8_t>(v >> 16)); }
 __device__ __forceinline__ float sb3(uint32_t v) { return static_cast<float>(static_cast<int8_t>(v >> 24)); }
 
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int s = 32; s > 0; s >>= 1) v += __shfl_xor(v, s, kWave);
+// Sums and maxima over the 16 lanes of a row on the vector unit's lane-crossing modifiers (two quad permutations,
+// then the mirror of 8 and of 16 lanes: every lane ends with the row's total), and over the wave with two more
+// steps through the LDS crossbar.  A crossbar shuffle costs a wave that is alone on its SIMD more than a hundred
+// cycles, and the reductions sit in dependent chains; every lane of the wave must be active.
+template <int CTRL>
+__device__ __forceinline__ float lane_cross(float v) {   // a lane outside the modifier's reach reads 0
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+__device__ __forceinline__ float row16_sum(float v) {
+    v += lane_cross<0xB1>(v);    // quad_perm [1,0,3,2]
+    v += lane_cross<0x4E>(v);    // quad_perm [2,3,0,1]
+    v += lane_cross<0x141>(v);   // row_half_mirror
+    v += lane_cross<0x140>(v);   // row_mirror
     return v;
 }
-__device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int s = 32; s > 0; s >>= 1) v = fmaxf(v, __shfl_xor(v, s, kWave));
+__device__ __forceinline__ float row16_max(float v) {
+    v = fmaxf(v, lane_cross<0xB1>(v));
+    v = fmaxf(v, lane_cross<0x4E>(v));
+    v = fmaxf(v, lane_cross<0x141>(v));
+    v = fmaxf(v, lane_cross<0x140>(v));
     return v;
+}
+__device__ __forceinline__ float wave_sum(float v) {
+    v = row16_sum(v);
+    v += __shfl_xor(v, 16, kWave);
+    return v + __shfl_xor(v, 32, kWave);
+}
+__device__ __forceinline__ float wave_max(float v) {
+    v = row16_max(v);
+    v = fmaxf(v, __shfl_xor(v, 16, kWave));
+    return fmaxf(v, __shfl_xor(v, 32, kWave));
 }
 
 // Sum of `planes` partial planes in plane order; loads are issued four at a time so that the

@@ -128,6 +128,22 @@ Scratch layout(const guffin_model_desc& m, uint32_t rows, uint32_t position, uin
     return s;
 }
 
+// The schedule words of row `row` of a pass of contiguous rows at `position`: first ring position, ring count,
+// first private row, private row count.
+__host__ __device__ inline void row_schedule_words(bool local, uint32_t window, uint32_t position, uint32_t row, uint32_t (&s)[4]) {
+    const uint32_t p = position + row;
+    const uint32_t window_start = (local && p >= window) ? p + 1 - window : 0;
+    const uint32_t base_start = position < window_start ? position : window_start;
+    const uint32_t private_start = window_start > position ? window_start - position : 0;
+    s[0] = base_start; s[1] = position - base_start; s[2] = private_start; s[3] = row + 1 - private_start;
+}
+// the same on the host, with a bit per private row the row attends (a contiguous pass's ancestor list is 0, 1, 2, ..)
+void row_schedule(const guffin_model_desc& m, uint32_t layer, uint32_t position, uint32_t row, uint32_t (&s)[4], uint32_t& amask) {
+    row_schedule_words(layer_is_local(m.global_period, layer), m.sliding_window, position, row, s);
+    amask = 0;
+    for (uint32_t i = 0; i < s[3]; ++i) amask |= 1u << (s[2] + i);
+}
+
 // positions, ancestors, the per-layer attention schedule of `rows` contiguous rows and the two
 // rotation tables (local and global frequency base) of the pass
 __global__ void stage_rows_kernel(uint32_t* positions, uint32_t* ancestors, uint32_t* schedule, uint32_t rows,
@@ -148,13 +164,11 @@ __global__ void stage_rows_kernel(uint32_t* positions, uint32_t* ancestors, uint
     }
     if (i < rows) { positions[i] = position + i; ancestors[i] = i; }
     if (i >= layers * rows) return;
-    const uint32_t layer = i / rows, row = i % rows, p = position + row;
-    const bool local = layer_is_local(global_period, layer);
-    const uint32_t window_start = (local && p >= window) ? p + 1 - window : 0;
-    const uint32_t base_start = position < window_start ? position : window_start;
-    const uint32_t private_start = window_start > position ? window_start - position : 0;
+    const uint32_t layer = i / rows, row = i % rows;
+    uint32_t words[4];
+    row_schedule_words(layer_is_local(global_period, layer), window, position, row, words);
     uint32_t* s = schedule + 4 * i;
-    s[0] = base_start; s[1] = position - base_start; s[2] = private_start; s[3] = row + 1 - private_start;
+    s[0] = words[0]; s[1] = words[1]; s[2] = words[2]; s[3] = words[3];
 }
 
 int validate_model(const guffin_model_desc* m) {
@@ -260,13 +274,17 @@ int forward_rows(hipStream_t stream, const guffin_model_desc& m, const uint32_t*
             GUFFIN_TRY(guffin_hip_gemv_packed_multi(st, 3, dt, tl, n, parts, s.u, s.us, rows, H));
             const uint32_t sq = qkv_slices(L, H, QW, KW);
             if (sq == 0) return fail(GUFFIN_E_SHAPE, "forward: q, k and v must share the block length");
-            // head norms, rotation, fp16 K/V rows and the attention itself in one pass over the planes
-            GUFFIN_TRY(guffin_hip_qkv_attention(st, s.part_a, s.part_b, s.part_c, sq, uint64_t(rows) * QW, uint64_t(rows) * KW,
-                                                uint64_t(rows) * KW, L.norm[1], L.norm[2],
-                                                local ? s.rope_local : s.rope_global, m.eps, L.ring_k, L.ring_v, pk, pv,
-                                                s.schedule + size_t(l) * rows * 4, s.ancestors, s.a, s.as, s.attn_out,
-                                                s.attn_ml, rows, max_tokens_for(m, l, position, rows), ring_mask,
-                                                m.q_heads, m.kv_heads, m.head_dim, attn_scale, status));
+            // head norms, rotation, fp16 K/V rows and the attention itself in one pass over the planes; the
+            // rows are contiguous and the position is the host's, so the schedule words stage_rows_kernel
+            // writes are known here too and travel with the launch
+            uint32_t host_schedule[2][4], host_amask[2];
+            for (uint32_t row = 0; row < rows; ++row) row_schedule(m, l, position, row, host_schedule[row], host_amask[row]);
+            GUFFIN_TRY(qkv_attention_scheduled(st, s.part_a, s.part_b, s.part_c, sq, uint64_t(rows) * QW, uint64_t(rows) * KW,
+                                               uint64_t(rows) * KW, L.norm[1], L.norm[2],
+                                               local ? s.rope_local : s.rope_global, m.eps, L.ring_k, L.ring_v, pk, pv,
+                                               s.schedule + size_t(l) * rows * 4, s.ancestors, &host_schedule[0][0], host_amask,
+                                               s.a, s.as, s.attn_out, s.attn_ml, rows, max_tokens_for(m, l, position, rows),
+                                               ring_mask, m.q_heads, m.kv_heads, m.head_dim, attn_scale, status));
         }
         GUFFIN_TRY(block_tail(st, m, l, s, rows, out_hidden, out_hidden_sums, status));
     }

@@ -46,10 +46,11 @@ __device__ __forceinline__ void emit_receipt_values(const float (&v)[8], uint32_
         float sum = v[0], m = fabsf(v[0]);
 #pragma unroll
         for (int i = 1; i < 8; ++i) { sum += v[i]; m = fmaxf(m, fabsf(v[i])); }
-        m = fmaxf(m, __shfl_xor(m, 1, kWave));
-        m = fmaxf(m, __shfl_xor(m, 2, kWave));
-        const float sum16 = sum + __shfl_xor(sum, 1, kWave);
-        const float sum32 = sum16 + __shfl_xor(sum16, 2, kWave);
+        // the four lanes of the group exchange inside their quad (lane ^ 1, then lane ^ 2)
+        m = fmaxf(m, lane_cross<0xB1>(m));
+        m = fmaxf(m, lane_cross<0x4E>(m));
+        const float sum16 = sum + lane_cross<0xB1>(sum);
+        const float sum32 = sum16 + lane_cross<0x4E>(sum16);
         // biased exponent of the group maximum, clamped so that both scale factors are normal floats
         uint32_t eb = __float_as_uint(m) >> 23;
         eb = eb < 14u ? 14u : eb > 244u ? 244u : eb;

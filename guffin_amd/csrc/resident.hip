@@ -605,11 +605,8 @@ __device__ __forceinline__ void attention_partition(Ctx& c, const RLayer& L, uin
                         s[n] = fmaf(static_cast<float>(h2.x), qv[n][2 * i], s[n]);
                         s[n] = fmaf(static_cast<float>(h2.y), qv[n][2 * i + 1], s[n]);
                     }
+                    s[n] = row16_sum(s[n]);
                     s[n] += __shfl_xor(s[n], 16, kWave);
-                    s[n] += __shfl_xor(s[n], 8, kWave);
-                    s[n] += __shfl_xor(s[n], 4, kWave);
-                    s[n] += __shfl_xor(s[n], 2, kWave);
-                    s[n] += __shfl_xor(s[n], 1, kWave);
                 }
                 if (l32 == 0) {
                     const bool is_priv = t >= n_ring;
