@@ -111,6 +111,30 @@ __device__ __forceinline__ float row16_max(float v) {
     v = fmaxf(v, lane_cross<0x140>(v));
     return v;
 }
+// Inclusive prefix sum over the 64 lanes, the same way: four shifts inside the rows of 16 (a lane past the row's
+// start reads 0), then lane 15's total into the next row and lane 31's into the upper half.
+template <int CTRL, int ROWS>
+__device__ __forceinline__ uint32_t lane_cross_u32(uint32_t v) {
+    return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), CTRL, ROWS, 0xF, ROWS == 0xF));
+}
+__device__ __forceinline__ uint32_t wave_inclusive_scan(uint32_t v) {
+    v += lane_cross_u32<0x111, 0xF>(v);   // row_shr:1
+    v += lane_cross_u32<0x112, 0xF>(v);   // row_shr:2
+    v += lane_cross_u32<0x114, 0xF>(v);   // row_shr:4
+    v += lane_cross_u32<0x118, 0xF>(v);   // row_shr:8
+    v += lane_cross_u32<0x142, 0xA>(v);   // row_bcast:15 into rows 1 and 3
+    v += lane_cross_u32<0x143, 0xC>(v);   // row_bcast:31 into rows 2 and 3
+    return v;
+}
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
+    v = max(v, lane_cross_u32<0xB1, 0xF>(v));
+    v = max(v, lane_cross_u32<0x4E, 0xF>(v));
+    v = max(v, lane_cross_u32<0x141, 0xF>(v));
+    v = max(v, lane_cross_u32<0x140, 0xF>(v));
+    v = max(v, static_cast<uint32_t>(__shfl_xor(static_cast<int>(v), 16, kWave)));
+    return max(v, static_cast<uint32_t>(__shfl_xor(static_cast<int>(v), 32, kWave)));
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
     v = row16_sum(v);
     v += __shfl_xor(v, 16, kWave);

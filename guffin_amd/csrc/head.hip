@@ -237,12 +237,7 @@ topk_merge_kernel(const float* __restrict__ logits, const uint64_t* __restrict__
     #pragma unroll
                 for (int j = 0; j < 4; ++j) c[j] = hist[255 - 4 * lane - j];
                 const uint32_t own = c[0] + c[1] + c[2] + c[3];
-                uint32_t incl = own;
-    #pragma unroll
-                for (int d = 1; d < 64; d <<= 1) {
-                    const uint32_t o = __shfl_up(incl, d, kWave);
-                    if (lane >= uint32_t(d)) incl += o;
-                }
+                const uint32_t incl = wave_inclusive_scan(own);
                 uint32_t above = incl - own;
                 if (above < remaining && remaining <= incl) {
     #pragma unroll
@@ -328,11 +323,7 @@ segment_max_kernel(const float* __restrict__ logits, uint32_t vocab, uint32_t se
             best = o > best ? o : best;
         }
     }
-#pragma unroll
-    for (int sft = 32; sft > 0; sft >>= 1) {
-        const uint32_t o = __shfl_xor(best, sft, kWave);
-        best = o > best ? o : best;
-    }
+    best = wave_max_u32(best);
     if (lane == 0) row_ws[seg] = best;
 }
 
@@ -343,12 +334,7 @@ __device__ __forceinline__ void find_bin(const uint32_t* hist, uint32_t remainin
 #pragma unroll
     for (int j = 0; j < 4; ++j) c[j] = hist[255 - 4 * lane - j];
     const uint32_t own = c[0] + c[1] + c[2] + c[3];
-    uint32_t incl = own;
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-        const uint32_t o = __shfl_up(incl, d, kWave);
-        if (lane >= uint32_t(d)) incl += o;
-    }
+    const uint32_t incl = wave_inclusive_scan(own);
     uint32_t above = incl - own;
     if (above < remaining && remaining <= incl) {
 #pragma unroll
