@@ -103,6 +103,37 @@ __device__ __forceinline__ void bitonic(uint64_t* keys, uint32_t n, bool desc) {
     __syncthreads();
 }
 
+// Sort of the first n keys in LDS by rank, n at most the workgroup's size: every thread counts the keys that go
+// before its own (all lanes read the same word: a broadcast) and drops its key at that place.  Three barriers
+// instead of the bitonic network's one per stage (28 for 128 keys, 45 for 512).
+// Distinct keys, ascending: a permutation of the n places.
+__device__ __forceinline__ void rank_sort_ascending(uint64_t* keys, uint32_t n) {
+    __syncthreads();
+    const uint32_t t = threadIdx.x;
+    const uint64_t mine = t < n ? keys[t] : 0;
+    uint32_t rank = 0;
+    if (t < n)
+        for (uint32_t j = 0; j < n; ++j) rank += keys[j] < mine;
+    __syncthreads();
+    if (t < n) keys[rank] = mine;
+    __syncthreads();
+}
+// Descending, keys distinct except for zeros (padding and dropped duplicates), which end up behind the others in
+// the first `span` places.
+__device__ __forceinline__ void rank_sort_descending(uint64_t* keys, uint32_t n, uint32_t span) {
+    __syncthreads();
+    const uint32_t t = threadIdx.x;
+    const uint64_t mine = t < n ? keys[t] : 0;
+    uint32_t rank = 0;
+    if (mine != 0)
+        for (uint32_t j = 0; j < n; ++j) rank += keys[j] > mine;
+    __syncthreads();
+    if (t < span) keys[t] = 0;
+    __syncthreads();
+    if (mine != 0) keys[rank] = mine;
+    __syncthreads();
+}
+
 __device__ __forceinline__ uint64_t score_key(float score, uint32_t token) {
     const uint32_t b = __float_as_uint(score + 0.0f);
     const uint32_t ordered = (b & 0x80000000u) ? ~b : (b | 0x80000000u);
@@ -179,9 +210,7 @@ draft_law_kernel(const Candidates* __restrict__ top, SamplerOptions opt, uint64_
     __syncthreads();
     // ascending token id; the score rides in the low half of the key
     keys[t] = t < n ? (uint64_t(my_token) << 32) | __float_as_uint(score[t]) : ~uint64_t{0};
-    uint32_t span = 64;   // entries beyond the support are all-ones keys already in their final place
-    while (span < n) span <<= 1;
-    bitonic(keys, span, false);
+    rank_sort_ascending(keys, n);   // entries beyond the support are all-ones keys already in their final place
     const float s = __uint_as_float(static_cast<uint32_t>(keys[t]));
     score[t] = t < n ? s : -INFINITY;
     __syncthreads();
@@ -499,7 +528,7 @@ __device__ int prepare_distribution(const Candidates* cand, const SamplerOptions
     if (sc.err) return sc.err;
     uint32_t span = 64;   // the sort covers the record only (a real key is never 0, the padding is)
     while (span < n) span <<= 1;
-    bitonic(sc.keys, span, true);
+    rank_sort_descending(sc.keys, n, span);
     // unique count = number of non-zero keys (a real key is never 0: ordered(logit) has a set bit)
     uint32_t mine = (t < span && sc.keys[t] != 0) ? 1u : 0u;
     const uint32_t unique = __syncthreads_count(mine);
