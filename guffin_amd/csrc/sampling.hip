@@ -193,13 +193,13 @@ draft_law_kernel(const Candidates* __restrict__ top, SamplerOptions opt, uint64_
     weight[t] = t < n ? law_exp(my_logit - first_logit) : 0.f;
     __syncthreads();
     if (t == 0) {  // descending-tail top-p / min-p in the reference's sequential order
-        float total = 0.f, tail = 0.f;
-        for (uint32_t j = n; j > 0; --j) total = __fadd_rn(total, weight[j - 1]);
+        // the tail sums from the last entry down; the last of them, in slot 0 (always kept), is the total: the
+        // same adds in the same order
+        float tail = 0.f;
         for (uint32_t j = n; j > 0; --j) {
             tail = __fadd_rn(tail, weight[j - 1]);
             running[j - 1] = tail;
         }
-        running[0] = total;   // slot 0 is always kept; it carries the total to the other lanes
     }
     __syncthreads();
     if (t > 0 && t < n) {
@@ -214,13 +214,12 @@ draft_law_kernel(const Candidates* __restrict__ top, SamplerOptions opt, uint64_
     const float s = __uint_as_float(static_cast<uint32_t>(keys[t]));
     score[t] = t < n ? s : -INFINITY;
     __syncthreads();
-    if (t == 0) {
-        float maximum = -INFINITY;
-        for (uint32_t i = 0; i < n; ++i) maximum = fmaxf(maximum, score[i]);
-        weight[0] = maximum;  // broadcast slot
+    {   // the maximum of the support (a maximum does not depend on the order it is taken in)
+        const float wave_best = wave_max(t < n ? score[t] : -INFINITY);
+        if ((t & 63u) == 0) weight[t >> 6] = wave_best;
     }
     __syncthreads();
-    const float maximum = weight[0];
+    const float maximum = fmaxf(fmaxf(weight[0], weight[1]), fmaxf(weight[2], weight[3]));
     __syncthreads();
     weight[t] = t < n ? law_exp(__fsub_rn(score[t], maximum)) : 0.f;
     __syncthreads();
