@@ -705,7 +705,10 @@ __device__ __forceinline__ void merge_attention(Ctx& c, uint32_t e0, uint32_t co
     Shared& sh = *c.sh;
     const float* pml = c.attn_ml + size_t(c.x) * kGroups * NQ * 2;
     const float* po = c.attn_out + size_t(c.x) * kGroups * NQ * kHd;
-    // weights of the 32 partitions per query: half a wave per query
+    // weights of the 32 partitions per query: half a wave per query.  The two reductions stay xor butterflies
+    // (not the quad-and-mirror tree of row16_sum): a row's tokens sit one partition further along as the second
+    // row of a two-row pass than when the row is decoded alone, and the butterfly's pairing keeps the sum's bits
+    // under that shift where the tree does not (the width-two verify pass must reproduce the one-row bits).
     if (c.tid < uint32_t(NQ) * kGroups) {
         const uint32_t n = c.tid / kGroups, p = c.tid % kGroups;
         const float m = xld(pml + (size_t(p) * NQ + n) * 2), l = xld(pml + (size_t(p) * NQ + n) * 2 + 1);
