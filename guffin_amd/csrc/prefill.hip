@@ -967,16 +967,12 @@ prefill_attention_mfma_kernel(const float* __restrict__ q, const uint16_t* __res
                     const bool visible = kp <= pos_r[r] && kp >= first_r[r] && kp <= hi_pos;
                     sv[c] = visible ? S[g][c][r] : -INFINITY;
                 }
-                float tmax = fmaxf(sv[0], sv[1]);
-#pragma unroll
-                for (int o = 8; o > 0; o >>= 1) tmax = fmaxf(tmax, __shfl_xor(tmax, o, kWave));
+                const float tmax = row16_max(fmaxf(sv[0], sv[1]));
                 const float new_m = fmaxf(m[g][r], tmax);
                 const float resc = new_m == -INFINITY ? 1.f : expf(m[g][r] - new_m);
                 const float p0 = sv[0] == -INFINITY ? 0.f : expf(sv[0] - new_m);
                 const float p1 = sv[1] == -INFINITY ? 0.f : expf(sv[1] - new_m);
-                float add = p0 + p1;
-#pragma unroll
-                for (int o = 8; o > 0; o >>= 1) add += __shfl_xor(add, o, kWave);
+                const float add = row16_sum(p0 + p1);
                 l[g][r] = l[g][r] * resc + add;
                 m[g][r] = new_m;
 #pragma unroll
