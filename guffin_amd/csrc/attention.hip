@@ -104,14 +104,20 @@ __device__ __forceinline__ float dot2(float acc, uint32_t packed_half2, float a,
     return fmaf(static_cast<float>(h.y), b, acc);
 }
 
+// waves of a partition's workgroup: two per SIMD.  With eight the queries and the private rows' key / value are
+// prepared by different waves, and a 32-token partition is one round of keys and two of values per wave.
+// (Eight query rows keep four waves: their per-wave output slots would not fit 64 KB of LDS otherwise.)
+constexpr int attention_waves(int queries) { return queries <= 4 ? 8 : 4; }
+
 template <int ROWS, int GROUP, int HD, bool FUSED>
-__global__ void __launch_bounds__(256) attn_partial_kernel(AttnArgs a) {
+__global__ void __launch_bounds__(64 * attention_waves(ROWS * GROUP)) attn_partial_kernel(AttnArgs a) {
     static_assert(HD == 256, "head dimension 256 (16 lanes x 16 dims)");
     constexpr int NQ = ROWS * GROUP;
+    constexpr int kAW = attention_waves(NQ);
     extern __shared__ float lds[];
     float* sc = lds;                          // [NQ][tp] scores, then probabilities
-    float* merge = lds + NQ * a.span;         // [4][NQ][HD]
-    float* q_s = merge + 4 * NQ * HD;         // fused: [NQ][HD] prepared queries
+    float* merge = lds + NQ * a.span;         // [kAW][NQ][HD]
+    float* q_s = merge + kAW * NQ * HD;       // fused: [NQ][HD] prepared queries
     __shared__ float s_max[NQ], s_sum[NQ];
     __shared__ __attribute__((aligned(16))) uint16_t k_s[FUSED ? ROWS : 1][HD], v_s[FUSED ? ROWS : 1][HD];
 
@@ -120,14 +126,14 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(AttnArgs a) {
     constexpr uint32_t group = GROUP;
     const uint32_t row_stride = a.kv_heads * HD;  // in halves
 
-    // fused: the query rows of this wave (w, w+4, ..) are requested first; their addresses need
+    // fused: the query rows of this wave (w, w+kAW, ..) are requested first; their addresses need
     // nothing but the launch arguments, so they travel together with the schedule below
-    constexpr int QI = (NQ + 3) / 4;
+    constexpr int QI = (NQ + kAW - 1) / kAW;
     HeadRow qr[FUSED ? QI : 1];
     if constexpr (FUSED) {
 #pragma unroll
         for (int i = 0; i < QI; ++i) {
-            const uint32_t item = wv + 4 * i;
+            const uint32_t item = wv + kAW * i;
             if (item < NQ) {
                 const uint32_t r = item / group, head = kvh * group + item % group;
                 load_head_row(qr[i], a.q_raw + (size_t(r) * a.q_heads + head) * HD, a.planes, a.q_stride, a.q_norm,
@@ -160,7 +166,8 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(AttnArgs a) {
     const uint32_t t0 = part * a.tp, t1 = part + 1 == a.partitions ? min(t0 + a.span, n_total) : min(t0 + a.tp, n_total);
 
     // ---- keys: four rounds of loads are issued before their dot products so that a wave keeps
-    // 16 key rows (8 KB) in flight; in fused mode the first batch travels during the preparation
+    // 16 key rows (8 KB) in flight (a round is 4 tokens per wave, 4 kAW per workgroup); in fused mode the first
+    // batch travels during the preparation
     constexpr int U = 4;
     const uint32_t slot = lane >> 4, seg = lane & 15;  // token slot in the wave, 16-dim segment
     const uint32_t tb_first = t0 + wv * 4 + slot;
@@ -168,7 +175,7 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(AttnArgs a) {
     auto load_keys = [&](uint32_t tb) {
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            const uint32_t t = tb + 16 * u;
+            const uint32_t t = tb + 4 * kAW * u;
             k0[u] = make_uint4(0, 0, 0, 0); k1[u] = k0[u];
             if (t < t1) {
                 const bool is_priv = t >= n_ring;
@@ -190,7 +197,7 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(AttnArgs a) {
     auto load_values = [&](uint32_t tb) {
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            const uint32_t t = tb + 8 * u;
+            const uint32_t t = tb + 2 * kAW * u;
             vv[u] = make_uint4(0, 0, 0, 0);
             if (t < t1) {
                 const bool is_priv = t >= n_ring;
@@ -203,19 +210,20 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(AttnArgs a) {
     };
 
     if constexpr (FUSED) {
-        // wave w prepares query rows w, w+4, .. and one of the private rows' key / value (row w/2,
-        // key for even w) when this partition holds it; every load is issued before any arithmetic
+        // wave w prepares query rows w, w+kAW, ..; the last 2 ROWS waves prepare the private rows' key / value
+        // (row i/2, key for even i) when this partition holds it; every load is issued before any arithmetic
         HeadRow kvr;
-        const uint32_t pr = wv >> 1, pt = n_ring + pr;
-        const bool is_key = (wv & 1u) == 0;
-        const bool mine = pr < ROWS && pr < a.private_rows && pt >= t0 && pt < t1;
+        const uint32_t ki = wv - (kAW - 2 * ROWS);   // wraps for the waves below: pr >= ROWS then
+        const uint32_t pr = ki >> 1, pt = n_ring + pr;
+        const bool is_key = (ki & 1u) == 0;
+        const bool mine = wv >= uint32_t(kAW - 2 * ROWS) && pr < ROWS && pr < a.private_rows && pt >= t0 && pt < t1;
         const size_t kv_off = (size_t(pr) * a.kv_heads + kvh) * HD;
         if (mine)
             load_head_row(kvr, (is_key ? a.k_raw : a.v_raw) + kv_off, a.planes, is_key ? a.k_stride : a.v_stride,
                           is_key ? a.k_norm : nullptr, is_key ? a.rope + size_t(pr) * (HD / 2) : nullptr, lane);
 #pragma unroll
         for (int i = 0; i < QI; ++i) {
-            const uint32_t item = wv + 4 * i;
+            const uint32_t item = wv + kAW * i;
             if (item < NQ) {
                 finish_head_row(qr[i], a.q_norm != nullptr, true, a.eps);
 #pragma unroll
@@ -248,11 +256,11 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(AttnArgs a) {
 #pragma unroll
             for (int i = 0; i < 16; ++i) qv[n][i] = qp[i] * a.scale;
         }
-        for (uint32_t tb = tb_first; tb < t0 + a.span; tb += 16 * U) {
+        for (uint32_t tb = tb_first; tb < t0 + a.span; tb += 4 * kAW * U) {
             if (!FUSED || tb != tb_first) load_keys(tb);
 #pragma unroll
             for (int u = 0; u < U; ++u) {
-                const uint32_t t = tb + 16 * u;
+                const uint32_t t = tb + 4 * kAW * u;
                 if (t >= t0 + a.span) break;
                 const bool in_range = t < t1, is_priv = t >= n_ring;
                 const uint32_t pos = u_first + t, prow = t - n_ring;
@@ -285,7 +293,7 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(AttnArgs a) {
     lds_barrier();
 
     // ---- softmax over the partition, one wave per query ----------------------------------
-    for (uint32_t n = wv; n < NQ; n += 4) {
+    for (uint32_t n = wv; n < NQ; n += kAW) {
         float m = -INFINITY;
         for (uint32_t i = lane; i < a.span; i += 64) m = fmaxf(m, sc[n * a.span + i]);
         m = wave_max(m);
@@ -307,11 +315,11 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(AttnArgs a) {
         for (int n = 0; n < NQ; ++n)
 #pragma unroll
             for (int i = 0; i < 8; ++i) acc[n][i] = 0.f;
-        for (uint32_t tb = vb_first; tb < t1; tb += 8 * U) {
+        for (uint32_t tb = vb_first; tb < t1; tb += 2 * kAW * U) {
             if (!FUSED || tb != vb_first) load_values(tb);
 #pragma unroll
             for (int u = 0; u < U; ++u) {
-                const uint32_t t = tb + 8 * u;
+                const uint32_t t = tb + 2 * kAW * u;
                 if (t >= t1) break;
                 if (FUSED && t >= n_ring) vv[u] = *reinterpret_cast<const uint4*>(&v_s[t - n_ring][dl]);
                 const uint32_t w4[4] = {vv[u].x, vv[u].y, vv[u].z, vv[u].w};
@@ -339,10 +347,14 @@ __global__ void __launch_bounds__(256) attn_partial_kernel(AttnArgs a) {
         }
     }
     lds_barrier();
-    for (uint32_t i = threadIdx.x; i < NQ * HD; i += 256) {
+    for (uint32_t i = threadIdx.x; i < NQ * HD; i += 64 * kAW) {
         const uint32_t n = i / HD, d = i % HD;
-        const float v = (merge[(0 * NQ + n) * HD + d] + merge[(1 * NQ + n) * HD + d])
-            + (merge[(2 * NQ + n) * HD + d] + merge[(3 * NQ + n) * HD + d]);
+        float pair[kAW / 2];   // waves in pairs, the pairs in order
+#pragma unroll
+        for (int w = 0; w < kAW; w += 2) pair[w / 2] = merge[(w * NQ + n) * HD + d] + merge[((w + 1) * NQ + n) * HD + d];
+        float v = pair[0] + pair[1];
+#pragma unroll
+        for (int w = 2; w < kAW / 2; w += 2) v += pair[w] + pair[w + 1];
         const uint32_t r = n / group, g = n % group, head = kvh * group + g;
         const size_t slot = (size_t(r) * a.q_heads + head) * a.partitions + part;
         a.part_out[slot * HD + d] = v;
@@ -423,12 +435,13 @@ attn_merge_kernel(const float* __restrict__ part_out, const float* __restrict__ 
 template <int ROWS, int GROUP>
 int launch_partial(hipStream_t s, const AttnArgs& a) {
     constexpr int NQ = ROWS * GROUP;
+    constexpr int kAW = attention_waves(NQ);
     const bool fused = a.q_raw != nullptr;
-    const size_t lds = (size_t(NQ) * a.span + size_t(4) * NQ * 256 + (fused ? size_t(NQ) * 256 : 0)) * sizeof(float);
+    const size_t lds = (size_t(NQ) * a.span + size_t(kAW) * NQ * 256 + (fused ? size_t(NQ) * 256 : 0)) * sizeof(float);
     if (fused)
-        hipLaunchKernelGGL((attn_partial_kernel<ROWS, GROUP, 256, true>), dim3(a.partitions, a.kv_heads), dim3(256), lds, s, a);
+        hipLaunchKernelGGL((attn_partial_kernel<ROWS, GROUP, 256, true>), dim3(a.partitions, a.kv_heads), dim3(64 * kAW), lds, s, a);
     else
-        hipLaunchKernelGGL((attn_partial_kernel<ROWS, GROUP, 256, false>), dim3(a.partitions, a.kv_heads), dim3(256), lds, s, a);
+        hipLaunchKernelGGL((attn_partial_kernel<ROWS, GROUP, 256, false>), dim3(a.partitions, a.kv_heads), dim3(64 * kAW), lds, s, a);
     return check_launch("attention_partial");
 }
 
