@@ -368,6 +368,7 @@ __global__ void __launch_bounds__(64 * attention_waves(ROWS * GROUP)) attn_parti
 // meet a zero weight), so up to 64 partitions cost one trip to memory; weights and denominators
 // terms are formed once, in parallel, in LDS.
 constexpr int kMergeAhead = 64;
+template <int AHEAD>
 __global__ void __launch_bounds__(256)
 attn_merge_kernel(const float* __restrict__ part_out, const float* __restrict__ part_ml, float* __restrict__ out,
                   float* __restrict__ out_sums, uint32_t partitions, uint32_t hd, uint32_t q_heads,
@@ -377,14 +378,14 @@ attn_merge_kernel(const float* __restrict__ part_out, const float* __restrict__ 
     __shared__ float rowbuf[1024];
     const uint32_t rh = blockIdx.x;  // row * q_heads + head
     const uint32_t lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
-    const uint32_t slots = partitions > uint32_t(kMergeAhead) ? partitions : uint32_t(kMergeAhead);
+    const uint32_t slots = partitions > uint32_t(AHEAD) ? partitions : uint32_t(AHEAD);
     float* lsum = wgt + slots;
     const float* ml = part_ml + size_t(rh) * partitions * 2;
     const float* po = part_out + size_t(rh) * partitions * hd;
     const uint32_t d0 = threadIdx.x;
-    float pre[kMergeAhead];
+    float pre[AHEAD];
 #pragma unroll
-    for (int p = 0; p < kMergeAhead; ++p) {
+    for (int p = 0; p < AHEAD; ++p) {
         const uint32_t q = uint32_t(p) < partitions ? uint32_t(p) : partitions - 1;
         pre[p] = d0 < hd ? po[size_t(q) * hd + d0] : 0.f;
     }
@@ -402,16 +403,16 @@ attn_merge_kernel(const float* __restrict__ part_out, const float* __restrict__ 
     __syncthreads();
     float denom = 0.f, acc0 = 0.f;
 #pragma unroll
-    for (int q = 0; q < kMergeAhead; ++q) {
+    for (int q = 0; q < AHEAD; ++q) {
         denom = fmaf(wgt[q], lsum[q], denom);
         acc0 = fmaf(wgt[q], pre[q], acc0);
     }
-    for (uint32_t p = kMergeAhead; p < partitions; ++p) denom = fmaf(wgt[p], lsum[p], denom);
+    for (uint32_t p = AHEAD; p < partitions; ++p) denom = fmaf(wgt[p], lsum[p], denom);
     bool bad = false;
     for (uint32_t d = threadIdx.x; d < hd; d += blockDim.x) {
         float acc = 0.f;
         uint32_t p = 0;
-        if (d == d0) { acc = acc0; p = partitions < uint32_t(kMergeAhead) ? partitions : uint32_t(kMergeAhead); }
+        if (d == d0) { acc = acc0; p = partitions < uint32_t(AHEAD) ? partitions : uint32_t(AHEAD); }
         for (; p + 4 <= partitions; p += 4) {
             const float v0 = po[size_t(p) * hd + d], v1 = po[size_t(p + 1) * hd + d], v2 = po[size_t(p + 2) * hd + d],
                         v3 = po[size_t(p + 3) * hd + d];
@@ -545,8 +546,13 @@ int attention_decode(void* stream, const float* q, const FusedInputs* fused, con
         default: return fail(GUFFIN_E_SHAPE, "attention_decode: q_heads / kv_heads must be 1, 2 or 4");
     }
     if (rc) return rc;
-    hipLaunchKernelGGL(attn_merge_kernel, dim3(rows * q_heads), dim3(256), 2 * std::max<uint32_t>(a.partitions, kMergeAhead) * sizeof(float), s, partial_out, partial_ml, out,
-                       out_sums, a.partitions, head_dim, q_heads, status);
+    // the outputs requested ahead: 32 when the partitions are that few (a local layer), else 64
+    if (a.partitions <= 32)
+        hipLaunchKernelGGL(attn_merge_kernel<32>, dim3(rows * q_heads), dim3(256), 2 * 32 * sizeof(float), s, partial_out, partial_ml, out,
+                           out_sums, a.partitions, head_dim, q_heads, status);
+    else
+        hipLaunchKernelGGL(attn_merge_kernel<kMergeAhead>, dim3(rows * q_heads), dim3(256), 2 * std::max<uint32_t>(a.partitions, kMergeAhead) * sizeof(float), s, partial_out, partial_ml, out,
+                           out_sums, a.partitions, head_dim, q_heads, status);
     return check_launch("attention_merge");
 }
 }  // namespace
