@@ -14,7 +14,8 @@ Extra objects on the JSON line:
                 (3.2 GB, far beyond the caches) on the launch stream; min / max over the replays and
                 over single launches; `traffic` is read from the committed counter profile.
   rooflines     the same figures for the step's other streaming kernels worth watching: the local
-                layers' attention (the kernel furthest from its bound) and the down projection.
+                layers' attention (the kernel furthest from its bound), the down projection, the q/k/v
+                launch and the o projection.
   configs       configs 0-3 on their own (one Q4_K GEMV at 1 row; one block's seven GEMVs at 2 rows;
                 the drafter's decode with head and argmax; the Q6_K head with selection and
                 acceptance): microseconds per unit as HIP graphs, algorithmic bytes, GB/s and the
@@ -436,6 +437,43 @@ def main():
                                 % down_slices, down, [l for l in every if int(target.layers[l].dtype[6]) == down_dt],
                                 down_bytes, "gemv_q6k_single_kernel<2>")
 
+    print("bench: timing the q/k/v and o projections", file=sys.stderr, flush=True)
+    qkv_dt = [int(d) for d in T.dtypes[:3]]
+    qkv_n = [QW, KW, KW]
+    c_dt, c_n = (C.c_int * 3)(*qkv_dt), (C.c_uint32 * 3)(*qkv_n)
+    lib.guffin_hip_gemv_packed_multi_slices.restype = C.c_uint32
+    qkv_slices = int(lib.guffin_hip_gemv_packed_multi_slices(3, c_dt, c_n, H))
+    if qkv_slices == 0:
+        raise RuntimeError("q/k/v split: " + lib.guffin_hip_last_error().decode())
+    qkv_parts = [torch.empty((qkv_slices, 2, n), device="cuda") for n in qkv_n]
+    c_parts = (C.c_void_p * 3)(*[p.data_ptr() for p in qkv_parts])
+
+    def qkv(l):
+        L = target.layers[l]
+        hip.check(lib.guffin_hip_gemv_packed_multi(hip._stream(), 3, c_dt, (C.c_void_p * 3)(*[L.tiles[i] for i in range(3)]), c_n,
+                                                   c_parts, hip._p(x), hip._p(xs), 2, H))
+
+    same_qkv = [l for l in every if [int(d) for d in target.layers[l].dtype[:3]] == qkv_dt]
+    qkv_bytes = (sum(synth.weight_bytes(dt, H, n) for dt, n in zip(qkv_dt, qkv_n)) + 2 * H * 4
+                 + qkv_slices * 2 * sum(qkv_n) * 4)
+    qkv_line = kernel_roofline("gemv_packed_multi_kernel<2, 3, mixed> (q/k/v GEMVs of one block in one launch, 2 rows, K=3840, "
+                               "N=4096+2048+2048, %d partial planes out)" % qkv_slices, qkv, same_qkv, qkv_bytes,
+                               "gemv_packed_multi_kernel<2, 3, mixed>")
+    xo = torch.randn(2, QW, device="cuda")
+    xos = hip.group_sums(xo)
+    o_dt = int(T.dtypes[3])
+    o_slices = hip.gemv_packed_slices(o_dt, QW, H)
+    o_parts = torch.empty((o_slices, 2, H), device="cuda")
+
+    def o_proj(l):
+        hip.check(lib.guffin_hip_gemv_packed(hip._stream(), o_dt, C.c_void_p(target.layers[l].tiles[3]), hip._p(xo), hip._p(xos),
+                                             hip._p(o_parts), None, 2, QW, H))
+
+    o_bytes = synth.weight_bytes(o_dt, QW, H) + 2 * QW * 4 + o_slices * 2 * H * 4
+    o_line = kernel_roofline("gemv_packed_kernel<Q4_K, 2> (o projection, 2 rows, K=4096, N=3840, %d partial planes out)" % o_slices,
+                             o_proj, [l for l in every if int(target.layers[l].dtype[3]) == o_dt], o_bytes,
+                             "gemv_packed_kernel<Q4_K, 2> (o")
+
     print("bench: timing the local layers' attention", file=sys.stderr, flush=True)
     # as the step runs it on a local layer: head norms, rotation, fp16 narrowing and attention of 2 rows over the
     # 1024-token window in one launch, then the partition merge (its time is part of the figure, its bytes are not)
@@ -488,7 +526,7 @@ def main():
             "accepted": int(first["accepted"]),
         },
         "roofline": roofline,
-        "rooflines": [attention_line, down_line],
+        "rooflines": [attention_line, down_line, qkv_line, o_line],
     }
     line["configs"] = config_figures(target, drafter, T, D, d_pos)
     if not args.no_prefill:
