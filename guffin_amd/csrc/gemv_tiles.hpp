@@ -47,10 +47,14 @@ __device__ __forceinline__ uint4 stream_load(const uint8_t* p) {
 
 struct Q4Tile { uint4 q[8]; uint4 hdr; };
 
+// Loads come back in the order of their requests: the scales and the pieces of the first four sub-blocks go
+// first, so that their products run while the other half of the tile is still on its way.
 __device__ __forceinline__ void load_tile(Q4Tile& t, const uint8_t* p) {
-#pragma unroll
-    for (int i = 0; i < 8; ++i) t.q[i] = stream_load(p + 1024 * i);
     t.hdr = stream_load(p + 8192);
+#pragma unroll
+    for (int i = 0; i < 8; i += 2) t.q[i] = stream_load(p + 1024 * i);
+#pragma unroll
+    for (int i = 1; i < 8; i += 2) t.q[i] = stream_load(p + 1024 * i);
 }
 
 __device__ __forceinline__ half8_t as_half8(uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
@@ -127,9 +131,13 @@ __device__ __forceinline__ void compute_tile(const Q4Tile& t, const Q4Operand& o
 // groups 2*(g/2) and 2*(g/2)+1, and the two k-halves are added across lanes at the end.
 struct Q6Tile { uint4 ql[8]; uint4 qh[4]; uint4 sc[2]; uint32_t d[2]; };
 
+// EARLY: the request order of the Q4_K tile (what the first 128 elements need, then the low nibbles of the other
+// half).  It pays where the operand groups are requested ahead of the tile; the one-tile-at-a-time walk reads
+// them behind the tile, where a group's wait covers every earlier request anyway, and is slower with it.
+template <bool EARLY>
 __device__ __forceinline__ void load_tile(Q6Tile& t, const uint8_t* p, uint32_t lane) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) t.ql[i] = stream_load(p + 1024 * i);
+    for (int i = 0; i < 8; i += EARLY ? 2 : 1) t.ql[i] = stream_load(p + 1024 * i);
 #pragma unroll
     for (int i = 0; i < 4; ++i) t.qh[i] = stream_load(p + 8192 + 1024 * i);
     const uint8_t* base = p - lane * 16;
@@ -138,6 +146,10 @@ __device__ __forceinline__ void load_tile(Q6Tile& t, const uint8_t* p, uint32_t 
     for (int c = 0; c < 2; ++c) {
         t.sc[c] = *reinterpret_cast<const uint4*>(base + 12288 + (col + 16 * c) * 16);
         t.d[c] = *reinterpret_cast<const uint16_t*>(base + 13312 + (col + 16 * c) * 2);
+    }
+    if constexpr (EARLY) {
+#pragma unroll
+        for (int i = 1; i < 8; i += 2) t.ql[i] = stream_load(p + 1024 * i);
     }
 }
 
@@ -311,14 +323,14 @@ __device__ __forceinline__ void run_blocks_at(const uint8_t* __restrict__ tiles,
         if constexpr (SINGLE) {  // one tile in registers at a time: 16 waves fit a workgroup
             for (uint32_t b = ob0; b < ob1; ++b) {
                 Q6Tile cur;
-                load_tile(cur, tp + size_t(b - ob0) * TB, lane);
+                load_tile<false>(cur, tp + size_t(b - ob0) * TB, lane);
                 compute_tile<R>(cur, image + size_t(b) * 2048u, keep, mult + b * 8u, K / 32, xs + b * 16u, per_row, lane, acc2);
             }
         } else {
             Q6Tile cur, nxt;
-            if (count) load_tile(cur, tp, lane);
+            if (count) load_tile<true>(cur, tp, lane);
             for (uint32_t b = ob0; b < ob1; ++b) {
-                if (b + 1 < ob1) load_tile(nxt, tp + size_t(b + 1 - ob0) * TB, lane);
+                if (b + 1 < ob1) load_tile<true>(nxt, tp + size_t(b + 1 - ob0) * TB, lane);
                 compute_tile<R>(cur, image + size_t(b) * 2048u, keep, mult + b * 8u, K / 32, xs + b * 16u, per_row, lane, acc2);
                 cur = nxt;
             }
