@@ -13,8 +13,9 @@
 // then every private row) with a per-row validity mask.
 //
 // Workgroup = (partition of TP consecutive virtual tokens, KV head), 256 threads.
-//   pass 1  scores: 16 lanes split the head dimension of one token (coalesced 512-byte K
-//           rows), four tokens per wave at a time; fp16 keys enter v_fma_mix_f32 directly;
+//   pass 1  scores: 16 lanes split the head dimension of one token (512-byte K rows, each of a
+//           lane's two requests part of 256 contiguous bytes), four tokens per wave at a time;
+//           fp16 keys enter v_fma_mix_f32 directly;
 //           a 4-step exchange inside each 16-lane group finishes the dot product.
 //   softmax per query over the partition in LDS (max, exp, sum).
 //   pass 2  values: a half wave owns one token (a lane eight output dims, 16-byte loads);
@@ -169,7 +170,9 @@ __global__ void __launch_bounds__(64 * attention_waves(ROWS * GROUP)) attn_parti
     // 16 key rows (8 KB) in flight (a round is 4 tokens per wave, 4 kAW per workgroup); in fused mode the first
     // batch travels during the preparation
     constexpr int U = 4;
-    const uint32_t slot = lane >> 4, seg = lane & 15;  // token slot in the wave, 16-dim segment
+    // (a lane's 16 dimensions are 8 seg .. 8 seg + 7 of each half of the row: either request of a row's 16 lanes
+    // then covers 256 contiguous bytes -- with 32 contiguous bytes per lane both requests touch every line of the row)
+    const uint32_t slot = lane >> 4, seg = lane & 15;  // token slot in the wave, segment of the head dimension
     const uint32_t tb_first = t0 + wv * 4 + slot;
     uint4 k0[U], k1[U];
     auto load_keys = [&](uint32_t tb) {
@@ -182,8 +185,8 @@ __global__ void __launch_bounds__(64 * attention_waves(ROWS * GROUP)) attn_parti
                 if (FUSED && is_priv) continue;  // taken from LDS once prepared
                 const uint16_t* kp = is_priv ? a.priv_k + size_t(t - n_ring) * row_stride
                                              : a.ring_k + size_t((u_first + t) & a.ring_mask) * row_stride;
-                kp += kvh * HD + seg * 16;
-                k0[u] = *reinterpret_cast<const uint4*>(kp); k1[u] = *reinterpret_cast<const uint4*>(kp + 8);
+                kp += kvh * HD + seg * 8;
+                k0[u] = *reinterpret_cast<const uint4*>(kp); k1[u] = *reinterpret_cast<const uint4*>(kp + HD / 2);
             }
         }
     };
@@ -251,10 +254,10 @@ __global__ void __launch_bounds__(64 * attention_waves(ROWS * GROUP)) attn_parti
 #pragma unroll
         for (int n = 0; n < NQ; ++n) {
             const uint32_t r = n / group, g = n % group;
-            const float* qp = FUSED ? q_s + n * HD + seg * 16
-                                    : a.q + (size_t(r) * a.q_heads + kvh * group + g) * HD + seg * 16;
+            const float* qp = FUSED ? q_s + n * HD + seg * 8
+                                    : a.q + (size_t(r) * a.q_heads + kvh * group + g) * HD + seg * 8;
 #pragma unroll
-            for (int i = 0; i < 16; ++i) qv[n][i] = qp[i] * a.scale;
+            for (int i = 0; i < 8; ++i) { qv[n][i] = qp[i] * a.scale; qv[n][8 + i] = qp[HD / 2 + i] * a.scale; }
         }
         for (uint32_t tb = tb_first; tb < t0 + a.span; tb += 4 * kAW * U) {
             if (!FUSED || tb != tb_first) load_keys(tb);
@@ -265,8 +268,8 @@ __global__ void __launch_bounds__(64 * attention_waves(ROWS * GROUP)) attn_parti
                 const bool in_range = t < t1, is_priv = t >= n_ring;
                 const uint32_t pos = u_first + t, prow = t - n_ring;
                 if (FUSED && in_range && is_priv) {
-                    const uint16_t* kp = &k_s[prow][seg * 16];
-                    k0[u] = *reinterpret_cast<const uint4*>(kp); k1[u] = *reinterpret_cast<const uint4*>(kp + 8);
+                    const uint16_t* kp = &k_s[prow][seg * 8];
+                    k0[u] = *reinterpret_cast<const uint4*>(kp); k1[u] = *reinterpret_cast<const uint4*>(kp + HD / 2);
                 }
                 const uint32_t kw[8] = {k0[u].x, k0[u].y, k0[u].z, k0[u].w, k1[u].x, k1[u].y, k1[u].z, k1[u].w};
                 float s[NQ];
