@@ -69,6 +69,23 @@ __device__ __forceinline__ void load_head_row(HeadRow& h, const float* src, uint
     for (int i = 0; i < 4; ++i) h.gm[i] = gamma ? gamma[lane + 64 * i] : 1.f;
     h.rp[0] = rope_row ? rope_row[lane] : make_float2(1.f, 0.f);
     h.rp[1] = rope_row ? rope_row[lane + 64] : make_float2(1.f, 0.f);
+    // up to four planes: every plane of every column is requested before the first add (a loop over a
+    // run-time plane count waits for each plane of each column in turn: eight dependent trips for two planes)
+    if (planes <= 4) {
+        float t[4][4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int s = 0; s < 4; ++s) t[i][s] = uint32_t(s) < planes ? src[lane + 64 * i + s * stride] : 0.f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            float v = t[i][0];
+#pragma unroll
+            for (int s = 1; s < 4; ++s) v = uint32_t(s) < planes ? v + t[i][s] : v;   // plane order, as load_planes
+            h.v[i] = v;
+        }
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < 4; ++i) h.v[i] = load_planes(src + lane + 64 * i, planes, stride);
 }
@@ -125,6 +142,16 @@ __global__ void __launch_bounds__(64 * attention_waves(ROWS * GROUP)) attn_parti
     const uint32_t part = blockIdx.x, kvh = blockIdx.y;
     const uint32_t lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
     constexpr uint32_t group = GROUP;
+    // Every launch argument is asked for here, in one go: left to their first uses, the scalar loads of a
+    // 300-byte argument block are spread over the blocks of the prologue, one dependent trip each.
+    asm volatile("" :: "s"(a.q), "s"(a.ring_k), "s"(a.ring_v), "s"(a.priv_k), "s"(a.priv_v), "s"(a.schedule), "s"(a.ancestors),
+                 "s"(a.part_out), "s"(a.part_ml), "s"(a.rows), "s"(a.q_heads), "s"(a.kv_heads), "s"(a.ring_mask), "s"(a.tp),
+                 "s"(a.span), "s"(a.partitions), "s"(a.private_rows), "s"(a.scale), "s"(a.q_raw), "s"(a.k_raw), "s"(a.v_raw),
+                 "s"(a.planes), "s"(a.q_stride), "s"(a.k_stride), "s"(a.v_stride), "s"(a.q_norm), "s"(a.k_norm), "s"(a.rope),
+                 "s"(a.priv_k_out), "s"(a.priv_v_out));
+    asm volatile("" :: "s"(a.eps), "s"(a.status), "s"(a.inline_schedule), "s"(a.sched[0][0]), "s"(a.sched[0][1]),
+                 "s"(a.sched[0][2]), "s"(a.sched[0][3]), "s"(a.sched[kMaxRows - 1][0]), "s"(a.sched[kMaxRows - 1][1]),
+                 "s"(a.sched[kMaxRows - 1][2]), "s"(a.sched[kMaxRows - 1][3]), "s"(a.amask[0]), "s"(a.amask[kMaxRows - 1]));
     const uint32_t row_stride = a.kv_heads * HD;  // in halves
 
     // fused: the query rows of this wave (w, w+kAW, ..) are requested first; their addresses need
