@@ -413,21 +413,25 @@ attn_merge_kernel(const float* __restrict__ part_out, const float* __restrict__ 
     const float* ml = part_ml + size_t(rh) * partitions * 2;
     const float* po = part_out + size_t(rh) * partitions * hd;
     const uint32_t d0 = threadIdx.x;
+    // this thread's (maximum, denominator) pair, requested first and once: the maximum and the weights below
+    // would otherwise each fetch the two words one after the other
+    const float2 own = threadIdx.x < partitions ? reinterpret_cast<const float2*>(ml)[threadIdx.x] : make_float2(0.f, 0.f);
     float pre[AHEAD];
 #pragma unroll
     for (int p = 0; p < AHEAD; ++p) {
         const uint32_t q = uint32_t(p) < partitions ? uint32_t(p) : partitions - 1;
         pre[p] = d0 < hd ? po[size_t(q) * hd + d0] : 0.f;
     }
-    float m = -INFINITY;
-    for (uint32_t p = threadIdx.x; p < partitions; p += 256) if (ml[2 * p + 1] > 0.f) m = fmaxf(m, ml[2 * p]);
+    float m = own.y > 0.f ? own.x : -INFINITY;
+    for (uint32_t p = threadIdx.x + 256; p < partitions; p += 256) if (ml[2 * p + 1] > 0.f) m = fmaxf(m, ml[2 * p]);
     m = wave_max(m);
     if (lane == 0) red[wv] = m;
     __syncthreads();
     const float M = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
     for (uint32_t p = threadIdx.x; p < slots; p += 256) {
-        const float l = p < partitions ? ml[2 * p + 1] : 0.f;
-        wgt[p] = l > 0.f ? expf(ml[2 * p] - M) : 0.f;
+        const bool first = p == threadIdx.x;
+        const float l = first ? own.y : p < partitions ? ml[2 * p + 1] : 0.f;
+        wgt[p] = l > 0.f ? expf((first ? own.x : ml[2 * p]) - M) : 0.f;
         lsum[p] = l;
     }
     __syncthreads();
