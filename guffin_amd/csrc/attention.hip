@@ -488,7 +488,7 @@ using namespace guffin;
 namespace {
 struct AttentionSplit { uint32_t partitions, tp, span; };
 AttentionSplit attention_split(uint32_t max_tokens, uint32_t kv_heads) {
-    uint32_t tp = 128;
+    uint32_t tp = 256;
     const uint32_t floor_tp = ((max_tokens + 31) / 32) * kv_heads < 64 ? 16u : 32u;
     while (tp > floor_tp && ((max_tokens + tp - 1) / tp) * kv_heads < 256) tp >>= 1;
     uint32_t partitions = (max_tokens + tp - 1) / tp;
@@ -507,7 +507,7 @@ AttentionSplit attention_split(uint32_t max_tokens, uint32_t kv_heads) {
 }  // namespace
 
 extern "C" uint32_t guffin_hip_attention_partitions(uint32_t max_tokens, uint32_t kv_heads) {
-    // tokens per partition: aim at >= 256 workgroups, between 32 and 128 tokens each; a context so
+    // tokens per partition: aim at >= 256 workgroups, between 32 and 256 tokens each; a context so
     // small that 32-token partitions give fewer than 64 workgroups (the drafter's window) is cut into
     // 16-token partitions, which shortens every workgroup's chain of dependent steps
     if (max_tokens == 0 || kv_heads == 0) return 0;
