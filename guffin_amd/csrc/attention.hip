@@ -474,9 +474,9 @@ int launch_partial(hipStream_t s, const AttnArgs& a) {
     const bool fused = a.q_raw != nullptr;
     const size_t lds = (size_t(NQ) * a.span + size_t(kAW) * NQ * 256 + (fused ? size_t(NQ) * 256 : 0)) * sizeof(float);
     if (fused)
-        hipLaunchKernelGGL((attn_partial_kernel<ROWS, GROUP, 256, true>), dim3(a.partitions, a.kv_heads), dim3(64 * kAW), lds, s, a);
+        launch((attn_partial_kernel<ROWS, GROUP, 256, true>), dim3(a.partitions, a.kv_heads), dim3(64 * kAW), lds, s, a);
     else
-        hipLaunchKernelGGL((attn_partial_kernel<ROWS, GROUP, 256, false>), dim3(a.partitions, a.kv_heads), dim3(64 * kAW), lds, s, a);
+        launch((attn_partial_kernel<ROWS, GROUP, 256, false>), dim3(a.partitions, a.kv_heads), dim3(64 * kAW), lds, s, a);
     return check_launch("attention_partial");
 }
 
@@ -582,10 +582,10 @@ int attention_decode(void* stream, const float* q, const FusedInputs* fused, con
     if (rc) return rc;
     // the outputs requested ahead: 32 when the partitions are that few (a local layer), else 64
     if (a.partitions <= 32)
-        hipLaunchKernelGGL(attn_merge_kernel<32>, dim3(rows * q_heads), dim3(256), 2 * 32 * sizeof(float), s, partial_out, partial_ml, out,
+        launch(attn_merge_kernel<32>, dim3(rows * q_heads), dim3(256), 2 * 32 * sizeof(float), s, partial_out, partial_ml, out,
                            out_sums, a.partitions, head_dim, q_heads, status);
     else
-        hipLaunchKernelGGL(attn_merge_kernel<kMergeAhead>, dim3(rows * q_heads), dim3(256), 2 * std::max<uint32_t>(a.partitions, kMergeAhead) * sizeof(float), s, partial_out, partial_ml, out,
+        launch(attn_merge_kernel<kMergeAhead>, dim3(rows * q_heads), dim3(256), 2 * std::max<uint32_t>(a.partitions, kMergeAhead) * sizeof(float), s, partial_out, partial_ml, out,
                            out_sums, a.partitions, head_dim, q_heads, status);
     return check_launch("attention_merge");
 }

@@ -4,6 +4,7 @@
 #include <stdint.h>
 
 #include "../../include/guffin_hip.h"
+#include "chain.hpp"
 
 namespace guffin {
 

@@ -527,8 +527,8 @@ template <int R>
 int launch_q4k(hipStream_t s, const uint8_t* w, const float* x, float* y, uint32_t K, uint32_t N) {
     const KPlan p = plan_kquant(R, K, N, 16, 4096, 256);
     if (p.lds > kMaxLds) return fail(GUFFIN_E_CAPACITY, "gemv_q4k: activation rows do not fit in LDS");
-    if (p.C == 4) hipLaunchKernelGGL((gemv_q4k_kernel<R, 4>), dim3(p.grid), dim3(p.threads), p.lds, s, w, x, y, p.dm);
-    else hipLaunchKernelGGL((gemv_q4k_kernel<R, 2>), dim3(p.grid), dim3(p.threads), p.lds, s, w, x, y, p.dm);
+    if (p.C == 4) launch((gemv_q4k_kernel<R, 4>), dim3(p.grid), dim3(p.threads), p.lds, s, w, x, y, p.dm);
+    else launch((gemv_q4k_kernel<R, 2>), dim3(p.grid), dim3(p.threads), p.lds, s, w, x, y, p.dm);
     return check_launch("gemv_q4k");
 }
 
@@ -536,8 +536,8 @@ template <int R>
 int launch_q6k(hipStream_t s, const uint8_t* w, const float* x, float* y, uint32_t K, uint32_t N) {
     const KPlan p = plan_kquant(R, K, N, 8, 2048, 128);
     if (p.lds > kMaxLds) return fail(GUFFIN_E_CAPACITY, "gemv_q6k: activation rows do not fit in LDS");
-    if (p.C == 4) hipLaunchKernelGGL((gemv_q6k_kernel<R, 4>), dim3(p.grid), dim3(p.threads), p.lds, s, w, x, y, p.dm);
-    else hipLaunchKernelGGL((gemv_q6k_kernel<R, 2>), dim3(p.grid), dim3(p.threads), p.lds, s, w, x, y, p.dm);
+    if (p.C == 4) launch((gemv_q6k_kernel<R, 4>), dim3(p.grid), dim3(p.threads), p.lds, s, w, x, y, p.dm);
+    else launch((gemv_q6k_kernel<R, 2>), dim3(p.grid), dim3(p.threads), p.lds, s, w, x, y, p.dm);
     return check_launch("gemv_q6k");
 }
 
@@ -555,7 +555,7 @@ int launch_q80(hipStream_t s, const uint8_t* w, const float* x, float* y, uint32
     uint32_t grid = (ntiles + waves - 1) / waves;
     const uint32_t max_grid = g_cu_count * 8;
     if (grid > max_grid) grid = max_grid;
-    hipLaunchKernelGGL((gemv_q80_kernel<R>), dim3(grid), dim3(waves * 64), lds, s, w, x, y, K, N, nblk, CT, ntiles);
+    launch((gemv_q80_kernel<R>), dim3(grid), dim3(waves * 64), lds, s, w, x, y, K, N, nblk, CT, ntiles);
     return check_launch("gemv_q80");
 }
 
@@ -585,9 +585,9 @@ extern "C" int guffin_hip_dequant(void* stream, int dtype, const void* blocks, u
     const uint32_t grid = static_cast<uint32_t>(n / 256 < 65535 ? (n + 255) / 256 : 65535);
     const uint8_t* b = static_cast<const uint8_t*>(blocks);
     hipStream_t s = as_stream(stream);
-    if (dtype == GUFFIN_Q8_0) hipLaunchKernelGGL(dequant_kernel<GUFFIN_Q8_0>, dim3(grid), dim3(256), 0, s, b, n, out);
-    else if (dtype == GUFFIN_Q4_K) hipLaunchKernelGGL(dequant_kernel<GUFFIN_Q4_K>, dim3(grid), dim3(256), 0, s, b, n, out);
-    else hipLaunchKernelGGL(dequant_kernel<GUFFIN_Q6_K>, dim3(grid), dim3(256), 0, s, b, n, out);
+    if (dtype == GUFFIN_Q8_0) launch(dequant_kernel<GUFFIN_Q8_0>, dim3(grid), dim3(256), 0, s, b, n, out);
+    else if (dtype == GUFFIN_Q4_K) launch(dequant_kernel<GUFFIN_Q4_K>, dim3(grid), dim3(256), 0, s, b, n, out);
+    else launch(dequant_kernel<GUFFIN_Q6_K>, dim3(grid), dim3(256), 0, s, b, n, out);
     return check_launch("dequant");
 }
 

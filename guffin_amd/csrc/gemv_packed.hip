@@ -271,13 +271,13 @@ int launch_packed(hipStream_t s, const uint8_t* w, const float* x, const float* 
     const dim3 grid(N / kTileCols, sp.planes), block(sp.W * 64);
     if constexpr (DTYPE == GUFFIN_Q6_K) {
         if (plan.single) {
-            if (rows == 2) hipLaunchKernelGGL((gemv_q6k_single_kernel<2>), grid, block, 0, s, w, x, xsums, part, N, c);
-            else hipLaunchKernelGGL((gemv_q6k_single_kernel<1>), grid, block, 0, s, w, x, xsums, part, N, c);
+            if (rows == 2) launch((gemv_q6k_single_kernel<2>), grid, block, 0, s, w, x, xsums, part, N, c);
+            else launch((gemv_q6k_single_kernel<1>), grid, block, 0, s, w, x, xsums, part, N, c);
             return check_launch("gemv_packed");
         }
     }
-    if (rows == 2) hipLaunchKernelGGL((gemv_packed_kernel<DTYPE, 2>), grid, block, 0, s, w, x, xsums, part, N, c);
-    else hipLaunchKernelGGL((gemv_packed_kernel<DTYPE, 1>), grid, block, 0, s, w, x, xsums, part, N, c);
+    if (rows == 2) launch((gemv_packed_kernel<DTYPE, 2>), grid, block, 0, s, w, x, xsums, part, N, c);
+    else launch((gemv_packed_kernel<DTYPE, 1>), grid, block, 0, s, w, x, xsums, part, N, c);
     return check_launch("gemv_packed");
 }
 
@@ -321,8 +321,8 @@ static int repack_common(void* stream, int dtype, const void* src, void* dst, ui
     uint16_t* d16 = static_cast<uint16_t*>(dst);
     hipStream_t s = as_stream(stream);
 #define GUFFIN_REPACK(DT)                                                                                   \
-    if (to_tiles) hipLaunchKernelGGL((repack_kernel<DT, true>), dim3(grid), dim3(256), 0, s, s16, d16, nblk, words); \
-    else hipLaunchKernelGGL((repack_kernel<DT, false>), dim3(grid), dim3(256), 0, s, s16, d16, nblk, words)
+    if (to_tiles) launch((repack_kernel<DT, true>), dim3(grid), dim3(256), 0, s, s16, d16, nblk, words); \
+    else launch((repack_kernel<DT, false>), dim3(grid), dim3(256), 0, s, s16, d16, nblk, words)
     if (dtype == GUFFIN_Q4_K) { GUFFIN_REPACK(GUFFIN_Q4_K); }
     else if (dtype == GUFFIN_Q6_K) { GUFFIN_REPACK(GUFFIN_Q6_K); }
     else { GUFFIN_REPACK(GUFFIN_Q8_0); }
@@ -342,7 +342,7 @@ extern "C" int guffin_hip_group_sums(void* stream, const float* x, float* xsums,
     if (!x || !xsums) return fail(GUFFIN_E_ARG, "group_sums: null pointer");
     if (rows == 0 || rows > 2 || K == 0 || K % 32 != 0) return fail(GUFFIN_E_SHAPE, "group_sums: K must be a positive multiple of 32, rows 1 or 2");
     if (reinterpret_cast<uintptr_t>(xsums) & 255u) return fail(GUFFIN_E_ALIGN, "group_sums: the receipt must be 256-byte aligned");
-    hipLaunchKernelGGL(group_sums_kernel, dim3(rows), dim3(256), 0, as_stream(stream), x, xsums, K, rows);
+    launch(group_sums_kernel, dim3(rows), dim3(256), 0, as_stream(stream), x, xsums, K, rows);
     return check_launch("group_sums");
 }
 
@@ -406,7 +406,7 @@ extern "C" int guffin_hip_gemv_packed_multi(void* stream, uint32_t count, const 
     const PackedCfg c {K, K / block_elems(dtypes[0]), sp.bps, sp.W};
     const dim3 grid(tile_end, sp.planes), block(sp.W * 64);
     hipStream_t s = as_stream(stream);
-#define GUFFIN_MULTI(R_, C_, M_) hipLaunchKernelGGL((gemv_packed_multi_kernel<R_, C_, M_>), grid, block, 0, s, t[0], t[1], t[2], p[0], p[1], p[2], x, xsums, m, c)
+#define GUFFIN_MULTI(R_, C_, M_) launch((gemv_packed_multi_kernel<R_, C_, M_>), grid, block, 0, s, t[0], t[1], t[2], p[0], p[1], p[2], x, xsums, m, c)
 #define GUFFIN_MULTI_MODE(R_, C_) do { \
         if (mode == GUFFIN_Q4_K) GUFFIN_MULTI(R_, C_, GUFFIN_Q4_K); else if (mode == GUFFIN_Q6_K) GUFFIN_MULTI(R_, C_, GUFFIN_Q6_K); \
         else if (mode == GUFFIN_Q8_0) GUFFIN_MULTI(R_, C_, GUFFIN_Q8_0); else GUFFIN_MULTI(R_, C_, kMixed); } while (0)
@@ -438,7 +438,7 @@ extern "C" int guffin_hip_gateup_geglu(void* stream, int dtype, const void* gate
     hipStream_t s = as_stream(stream);
     const uint8_t* g = static_cast<const uint8_t*>(gate_tiles);
     const uint8_t* u = static_cast<const uint8_t*>(up_tiles);
-#define GUFFIN_GU(D_, R_) hipLaunchKernelGGL((gateup_geglu_kernel<D_, R_>), grid, block, 0, s, g, u, x, xsums, h, h_sums, F, c)
+#define GUFFIN_GU(D_, R_) launch((gateup_geglu_kernel<D_, R_>), grid, block, 0, s, g, u, x, xsums, h, h_sums, F, c)
     if (dtype == GUFFIN_Q4_K) { if (rows == 2) GUFFIN_GU(GUFFIN_Q4_K, 2); else GUFFIN_GU(GUFFIN_Q4_K, 1); }
     else { if (rows == 2) GUFFIN_GU(GUFFIN_Q8_0, 2); else GUFFIN_GU(GUFFIN_Q8_0, 1); }
 #undef GUFFIN_GU
@@ -463,7 +463,7 @@ extern "C" int guffin_hip_gemv_packed(void* stream, int dtype, const void* tiles
     else rc = launch_packed<GUFFIN_Q8_0>(s, w, x, xsums, out, rows, K, N);
     if (rc || !y || S == 1) return rc;
     const uint32_t count = rows * N;
-    hipLaunchKernelGGL(reduce_partials_kernel, dim3((count + 255) / 256), dim3(256), 0, s, partials, y, S, count);
+    launch(reduce_partials_kernel, dim3((count + 255) / 256), dim3(256), 0, s, partials, y, S, count);
     return check_launch("reduce_partials");
 }
 

@@ -600,22 +600,22 @@ int guffin::select_candidates_scaled(hipStream_t s, const float* logits, uint32_
     const uint32_t segs = (vocab + kSeg - 1) / kSeg;
     if (segs <= kMaxSegs && segs >= 2 * keep) {   // large vocabulary: a bound from the segment maxima, then one pass
         uint32_t* words = static_cast<uint32_t*>(workspace);
-        hipLaunchKernelGGL(segment_max_kernel, dim3((segs + 3) / 4, rows), dim3(256), 0, s, logits, vocab, segs, divisor, words);
+        launch(segment_max_kernel, dim3((segs + 3) / 4, rows), dim3(256), 0, s, logits, vocab, segs, divisor, words);
         if (int rc = check_launch("select_candidates(segment maxima)")) return rc;
-        hipLaunchKernelGGL(threshold_select_kernel, dim3((vocab + kCollectTile - 1) / kCollectTile, rows), dim3(1024), 0, s,
+        launch(threshold_select_kernel, dim3((vocab + kCollectTile - 1) / kCollectTile, rows), dim3(1024), 0, s,
                            logits, vocab, segs, keep, divisor, history, history_count, row_retain, row_stride,
                            row_stride == 1 ? 64u : row_stride, words, static_cast<Candidates*>(result), status, suppressed_ok);
         return check_launch("select_candidates(threshold)");
     }
     uint64_t* surv = static_cast<uint64_t*>(workspace);
-    hipLaunchKernelGGL(topk_tile_kernel, dim3(tiles, rows), dim3(1024), 0, s, logits, surv, vocab, keep, divisor, status, suppressed_ok);
+    launch(topk_tile_kernel, dim3(tiles, rows), dim3(1024), 0, s, logits, surv, vocab, keep, divisor, status, suppressed_ok);
     if (int rc = check_launch("select_candidates(tile)")) return rc;
     if (tiles * keep <= 8 * 1024)
-        hipLaunchKernelGGL(topk_merge_kernel<8>, dim3(rows), dim3(1024), 0, s, logits, surv, tiles * keep, keep, vocab,
+        launch(topk_merge_kernel<8>, dim3(rows), dim3(1024), 0, s, logits, surv, tiles * keep, keep, vocab,
                            keep, divisor, history, history_count, row_retain, row_stride, row_stride == 1 ? 64u : row_stride,
                            static_cast<Candidates*>(result), status);
     else
-        hipLaunchKernelGGL(topk_merge_kernel<34>, dim3(rows), dim3(1024), 0, s, logits, surv, tiles * keep, keep, vocab,
+        launch(topk_merge_kernel<34>, dim3(rows), dim3(1024), 0, s, logits, surv, tiles * keep, keep, vocab,
                            keep, divisor, history, history_count, row_retain, row_stride, row_stride == 1 ? 64u : row_stride,
                            static_cast<Candidates*>(result), status);
     return check_launch("select_candidates(merge)");
@@ -625,7 +625,7 @@ extern "C" int guffin_hip_input_validation(void* stream, const uint32_t* actual,
                                            uint32_t vocab, uint32_t* status) {
     if (!actual || !expected || !status) return fail(GUFFIN_E_ARG, "input_validation: null pointer");
     if (rows == 0 || vocab == 0) return fail(GUFFIN_E_SHAPE, "input_validation: empty shape");
-    hipLaunchKernelGGL(input_validation_kernel, dim3((rows + 63) / 64), dim3(64), 0, as_stream(stream), actual, expected,
+    launch(input_validation_kernel, dim3((rows + 63) / 64), dim3(64), 0, as_stream(stream), actual, expected,
                        rows, vocab, status);
     return check_launch("input_validation");
 }
@@ -638,7 +638,7 @@ extern "C" int guffin_hip_selection_requests(void* stream, const void* raw, uint
     if (top_k == 0 || top_k > 256) return fail(GUFFIN_E_CAPACITY, "selection_requests: top_k must be in [1, 256]");
     if ((reinterpret_cast<uintptr_t>(raw) | reinterpret_cast<uintptr_t>(resolved)) & 3u)
         return fail(GUFFIN_E_ALIGN, "selection_requests: rows must be 4-byte aligned");
-    hipLaunchKernelGGL(selection_requests_kernel, dim3(rows), dim3(64), 0, as_stream(stream),
+    launch(selection_requests_kernel, dim3(rows), dim3(64), 0, as_stream(stream),
                        static_cast<const SelectionRow*>(raw), vocab, top_k, repetition_enabled,
                        static_cast<ResolvedRow*>(resolved), histories, status);
     return check_launch("selection_requests");
@@ -665,8 +665,8 @@ extern "C" int guffin_hip_argmax(void* stream, const float* logits, uint32_t row
     const uint32_t blocks = vocab / 1024 < 1 ? 1 : (vocab / 1024 > 256 ? 256 : vocab / 1024);
     hipStream_t s = as_stream(stream);
     uint64_t* part = static_cast<uint64_t*>(workspace);  // rows * 256 keys at most
-    hipLaunchKernelGGL(argmax_tile_kernel, dim3(blocks, rows), dim3(256), 0, s, logits, part, vocab, status);
+    launch(argmax_tile_kernel, dim3(blocks, rows), dim3(256), 0, s, logits, part, vocab, status);
     if (int rc = check_launch("argmax(tile)")) return rc;
-    hipLaunchKernelGGL(argmax_final_kernel, dim3(rows), dim3(256), 0, s, part, blocks, token, logit);
+    launch(argmax_final_kernel, dim3(rows), dim3(256), 0, s, part, blocks, token, logit);
     return check_launch("argmax(final)");
 }

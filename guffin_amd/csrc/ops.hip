@@ -466,7 +466,7 @@ extern "C" int guffin_hip_rms_norm(void* stream, const float* x, uint32_t planes
     if (!aligned4(x) || !aligned4(y) || !aligned4(gamma)) return fail(GUFFIN_E_ALIGN, "rms_norm: fp32 pointers must be 4-byte aligned");
     const size_t lds = (size_t(width) + 16) * 4;
     if (lds > 160 * 1024) return fail(GUFFIN_E_CAPACITY, "rms_norm: row does not fit in LDS");
-    hipLaunchKernelGGL(rms_norm_kernel, dim3(rows), dim3(norm_threads(width)), lds, as_stream(stream), x, planes,
+    launch(rms_norm_kernel, dim3(rows), dim3(norm_threads(width)), lds, as_stream(stream), x, planes,
                        static_cast<size_t>(plane_stride), gamma, residual, y, y_sums, width, eps, status);
     return check_launch("rms_norm");
 }
@@ -485,14 +485,14 @@ extern "C" int guffin_hip_rms_norm_add_norm(void* stream, const float* x, uint32
     if (planes <= uint32_t(kFastPlanes) && width % 8 == 0 && width / 8 <= 1024 && (!out_sums || width % 32 == 0)
         && plane_stride % 4 == 0 && a16(x) && a16(gamma_post) && a16(residual) && a16(out_residual) && a16(gamma_next) && a16(out_norm)) {
         const uint32_t threads = (width / 8 + 63) / 64 * 64;
-        hipLaunchKernelGGL(rms_norm_add_norm_regs_kernel, dim3(rows), dim3(threads), 0, as_stream(stream), x, planes,
+        launch(rms_norm_add_norm_regs_kernel, dim3(rows), dim3(threads), 0, as_stream(stream), x, planes,
                            static_cast<size_t>(plane_stride), gamma_post, residual, out_residual, gamma_next, out_norm,
                            out_sums, width, eps, status);
         return check_launch("rms_norm_add_norm");
     }
     const size_t lds = (size_t(width) + 16) * 4;
     if (lds > 160 * 1024) return fail(GUFFIN_E_CAPACITY, "rms_norm_add_norm: row does not fit in LDS");
-    hipLaunchKernelGGL(rms_norm_add_norm_kernel, dim3(rows), dim3(norm_threads(width)), lds, as_stream(stream), x, planes,
+    launch(rms_norm_add_norm_kernel, dim3(rows), dim3(norm_threads(width)), lds, as_stream(stream), x, planes,
                        static_cast<size_t>(plane_stride), gamma_post, residual, out_residual, gamma_next,
                        out_norm, out_sums, width, eps, status);
     return check_launch("rms_norm_add_norm");
@@ -503,7 +503,7 @@ extern "C" int guffin_hip_head_rms_norm(void* stream, const float* x, const floa
     if (!x || !gamma || !y) return fail(GUFFIN_E_ARG, "head_rms_norm: null pointer");
     if (rows == 0 || heads == 0 || head_dim == 0) return fail(GUFFIN_E_SHAPE, "head_rms_norm: empty shape");
     if (!(eps > 0.f)) return fail(GUFFIN_E_ARG, "head_rms_norm: epsilon must be positive");
-    hipLaunchKernelGGL(head_rms_norm_kernel, dim3(rows * heads), dim3(64), 0, as_stream(stream), x, gamma, y, head_dim, eps);
+    launch(head_rms_norm_kernel, dim3(rows * heads), dim3(64), 0, as_stream(stream), x, gamma, y, head_dim, eps);
     return check_launch("head_rms_norm");
 }
 
@@ -514,7 +514,7 @@ static int launch_qkv(void* stream, const QkvArgs& a) {
     if (a.rope_dim && !a.rope_table && !(a.base > 0.f)) return fail(GUFFIN_E_ARG, "rope/kv: frequency base must be positive");
     const uint32_t blocks = a.rows * (a.q_heads + 2 * a.kv_heads);
     if (blocks == 0) return fail(GUFFIN_E_SHAPE, "rope/kv: no heads");
-    hipLaunchKernelGGL(qkv_post_kernel, dim3(blocks), dim3(64), a.head_dim * sizeof(float), as_stream(stream), a);
+    launch(qkv_post_kernel, dim3(blocks), dim3(64), a.head_dim * sizeof(float), as_stream(stream), a);
     return check_launch("qkv_post");
 }
 
@@ -570,7 +570,7 @@ extern "C" int guffin_hip_rope_table(void* stream, const uint32_t* positions, fl
     if (rows == 0 || rope_dim == 0 || rope_dim % 2) return fail(GUFFIN_E_SHAPE, "rope_table: rope_dim must be even and rows >= 1");
     if (reinterpret_cast<uintptr_t>(table) & 7u) return fail(GUFFIN_E_ALIGN, "rope_table: table must be 8-byte aligned");
     const uint32_t n = rows * (rope_dim / 2);
-    hipLaunchKernelGGL(rope_table_kernel, dim3((n + 63) / 64), dim3(64), 0, as_stream(stream), positions,
+    launch(rope_table_kernel, dim3((n + 63) / 64), dim3(64), 0, as_stream(stream), positions,
                        reinterpret_cast<float2*>(table), rows, rope_dim, freq_base, freq_scale);
     return check_launch("rope_table");
 }
@@ -585,7 +585,7 @@ extern "C" int guffin_hip_geglu(void* stream, const float* gate, const float* up
     const uint32_t chunk = 512, chunks = (width + chunk - 1) / chunk;
     const uint32_t per = out_sums ? chunk : (width + chunks - 1) / chunks;
     const uint32_t gx = (width + per - 1) / per;
-    hipLaunchKernelGGL(geglu_kernel, dim3(gx, rows), dim3(256), out_sums ? per * sizeof(float) : 0, as_stream(stream),
+    launch(geglu_kernel, dim3(gx, rows), dim3(256), out_sums ? per * sizeof(float) : 0, as_stream(stream),
                        gate, up, planes, static_cast<size_t>(plane_stride), out, out_sums, width);
     return check_launch("geglu");
 }
@@ -599,9 +599,9 @@ extern "C" int guffin_hip_embed(void* stream, int dtype, const void* w, const ui
     if (reinterpret_cast<uintptr_t>(w) & 1u) return fail(GUFFIN_E_ALIGN, "embed: weights must be 2-byte aligned");
     const uint8_t* wb = static_cast<const uint8_t*>(w);
     hipStream_t s = as_stream(stream);
-    if (dtype == GUFFIN_Q8_0) hipLaunchKernelGGL(embed_kernel<GUFFIN_Q8_0>, dim3(rows), dim3(256), 0, s, wb, tokens, out, width, scale, vocab, status);
-    else if (dtype == GUFFIN_Q4_K) hipLaunchKernelGGL(embed_kernel<GUFFIN_Q4_K>, dim3(rows), dim3(256), 0, s, wb, tokens, out, width, scale, vocab, status);
-    else hipLaunchKernelGGL(embed_kernel<GUFFIN_Q6_K>, dim3(rows), dim3(256), 0, s, wb, tokens, out, width, scale, vocab, status);
+    if (dtype == GUFFIN_Q8_0) launch(embed_kernel<GUFFIN_Q8_0>, dim3(rows), dim3(256), 0, s, wb, tokens, out, width, scale, vocab, status);
+    else if (dtype == GUFFIN_Q4_K) launch(embed_kernel<GUFFIN_Q4_K>, dim3(rows), dim3(256), 0, s, wb, tokens, out, width, scale, vocab, status);
+    else launch(embed_kernel<GUFFIN_Q6_K>, dim3(rows), dim3(256), 0, s, wb, tokens, out, width, scale, vocab, status);
     return check_launch("embed");
 }
 
@@ -611,7 +611,7 @@ extern "C" int guffin_hip_kv_scatter(void* stream, const void* priv_k, const voi
     if (!priv_k || !priv_v || !selected || !ring_k || !ring_v) return fail(GUFFIN_E_ARG, "kv_scatter: null pointer");
     if (rows == 0 || row_width == 0) return fail(GUFFIN_E_SHAPE, "kv_scatter: empty shape");
     if ((ring_mask & (ring_mask + 1)) != 0) return fail(GUFFIN_E_ARG, "kv_scatter: ring capacity must be a power of two");
-    hipLaunchKernelGGL(kv_scatter_kernel, dim3((row_width + 255) / 256, rows), dim3(256), 0, as_stream(stream),
+    launch(kv_scatter_kernel, dim3((row_width + 255) / 256, rows), dim3(256), 0, as_stream(stream),
                        static_cast<const uint16_t*>(priv_k), static_cast<const uint16_t*>(priv_v), selected,
                        static_cast<uint16_t*>(ring_k), static_cast<uint16_t*>(ring_v), position, rows, row_width, ring_mask);
     return check_launch("kv_scatter");

@@ -236,7 +236,7 @@ int forward_rows(hipStream_t stream, const guffin_model_desc& m, const uint32_t*
     if (g_forward_mode == 2 && !resident) return fail(GUFFIN_E_SHAPE, "forward: the resident pass does not cover this model");
     const uint32_t sync_words = resident ? s.sync_words : 0u;
     const uint32_t n_stage = std::max({m.layer_count * rows, rows * (m.head_dim / 2), sync_words});
-    hipLaunchKernelGGL(stage_rows_kernel, dim3((n_stage + 63) / 64), dim3(64), 0, stream, s.positions, s.ancestors,
+    launch(stage_rows_kernel, dim3((n_stage + 63) / 64), dim3(64), 0, stream, s.positions, s.ancestors,
                        s.schedule, rows, position, m.layer_count, m.sliding_window, m.global_period,
                        reinterpret_cast<float2*>(s.rope_local), reinterpret_cast<float2*>(s.rope_global), m.head_dim,
                        m.local_base, m.global_base, m.global_scale, s.sync, sync_words);
@@ -481,7 +481,7 @@ extern "C" int guffin_hip_commit_rows(void* stream, const guffin_model_desc* mod
     if (!priv_k || !priv_v || !ring_k_table || !ring_v_table) return fail(GUFFIN_E_ARG, "commit_rows: null pointer");
     if (rows == 0 || rows > 2) return fail(GUFFIN_E_SHAPE, "commit_rows: rows must be 1 or 2");
     const uint32_t KW = model->kv_heads * model->head_dim;
-    hipLaunchKernelGGL(commit_rows_kernel, dim3((KW + 255) / 256, model->layer_count, rows), dim3(256), 0,
+    launch(commit_rows_kernel, dim3((KW + 255) / 256, model->layer_count, rows), dim3(256), 0,
                        as_stream(stream), static_cast<const uint16_t*>(priv_k), static_cast<const uint16_t*>(priv_v),
                        reinterpret_cast<uint16_t* const*>(ring_k_table), reinterpret_cast<uint16_t* const*>(ring_v_table),
                        accepted, position, rows, KW, model->ring_local - 1, model->ring_global - 1, model->global_period);
@@ -551,7 +551,7 @@ extern "C" int guffin_hip_prefill_rows(void* stream, const guffin_model_desc* mo
     hipStream_t hs = as_stream(stream);
     const uint32_t H = m.hidden, F = m.ffn, QW = m.q_heads * m.head_dim, KW = m.kv_heads * m.head_dim;
     const float attn_scale = 1.0f / std::sqrt(static_cast<float>(m.head_dim));
-    hipLaunchKernelGGL(fill_positions_kernel, dim3((rows + 255) / 256), dim3(256), 0, hs, s.positions, rows, position);
+    launch(fill_positions_kernel, dim3((rows + 255) / 256), dim3(256), 0, hs, s.positions, rows, position);
     GUFFIN_TRY(check_launch("prefill positions"));
     GUFFIN_TRY(guffin_hip_rope_table(stream, s.positions, s.rope_local, rows, m.head_dim, m.local_base, 1.0f));
     GUFFIN_TRY(guffin_hip_rope_table(stream, s.positions, s.rope_global, rows, m.head_dim, m.global_base, m.global_scale));
@@ -688,7 +688,7 @@ extern "C" int guffin_hip_h1_step(void* stream, const guffin_h1_desc* d, const u
     if (dr == 2 && !d->pending_token) return fail(GUFFIN_E_ARG, "h1_step: two drafter rows need the pending token");
     const bool mapped = d->draft_to_target != nullptr;
     if (mapped != (d->target_to_draft != nullptr)) return fail(GUFFIN_E_ARG, "h1_step: the vocabulary map needs its inverse");
-    hipLaunchKernelGGL(set_step_tokens_kernel, dim3(1), dim3(1), 0, s, root_token, dr == 2 ? d->pending_token : nullptr, tokens,
+    launch(set_step_tokens_kernel, dim3(1), dim3(1), 0, s, root_token, dr == 2 ? d->pending_token : nullptr, tokens,
                        d->target_to_draft, T.vocab, status);
     GUFFIN_TRY(check_launch("set_step_tokens"));
     GUFFIN_TRY(guffin_hip_forward_rows(stream, &D, tokens + 8, dr, d->drafter_position, d_scratch, d_bytes, drafter_priv_k,
@@ -701,7 +701,7 @@ extern "C" int guffin_hip_h1_step(void* stream, const guffin_h1_desc* d, const u
         // drafter's ids, tokens[1] carries it to the verify pass in the target's
         const uint32_t* draft_hist = nullptr;
         if (with_history) {
-            hipLaunchKernelGGL(draft_history_kernel, dim3(1), dim3(64), 0, s, d->history, d->history_count, d->target_to_draft,
+            launch(draft_history_kernel, dim3(1), dim3(64), 0, s, d->history, d->history_count, d->target_to_draft,
                                T.vocab, B.hist + kHistDraft);
             GUFFIN_TRY(check_launch("draft_history"));
             draft_hist = B.hist + kHistDraft;
@@ -738,7 +738,7 @@ extern "C" int guffin_hip_h1_step(void* stream, const guffin_h1_desc* d, const u
     // top_k, src/engine/sampling.cpp:430-446), then the history tokens' own logits
     const uint32_t* hist = nullptr;
     if (with_history) {
-        hipLaunchKernelGGL(build_history_kernel, dim3(1), dim3(128), 0, s, d->history, d->history_count, tokens + 1, V,
+        launch(build_history_kernel, dim3(1), dim3(128), 0, s, d->history, d->history_count, tokens + 1, V,
                            d->top_k, B.hist, status);
         GUFFIN_TRY(check_launch("build_history"));
         hist = B.hist + kHistLists;

@@ -1098,7 +1098,7 @@ extern "C" int guffin_hip_kv_cache_copy(void* stream, const void* src_k, const v
           | reinterpret_cast<uintptr_t>(dst_v)) & 15u) != 0)
         return fail(GUFFIN_E_ALIGN, "kv_cache_copy: rows must be 16-byte aligned");
     const uint64_t n = uint64_t(tokens) * (row_width / 8);
-    hipLaunchKernelGGL(kv_cache_copy_kernel, dim3(static_cast<uint32_t>((n + 255) / 256)), dim3(256), 0, as_stream(stream),
+    launch(kv_cache_copy_kernel, dim3(static_cast<uint32_t>((n + 255) / 256)), dim3(256), 0, as_stream(stream),
                        static_cast<const uint4*>(src_k), static_cast<const uint4*>(src_v), static_cast<uint4*>(dst_k),
                        static_cast<uint4*>(dst_v), tokens, position, src_mask, dst_mask, row_width / 8);
     return check_launch("kv_cache_copy");
@@ -1111,7 +1111,7 @@ extern "C" int guffin_hip_publish_run(void* stream, const void* run_k, const voi
     if ((ring_mask & (ring_mask + 1)) != 0) return fail(GUFFIN_E_ARG, "publish_run: ring capacity must be a power of two");
     const uint32_t first = rows > ring_mask + 1 ? rows - (ring_mask + 1) : 0;  // older rows would be overwritten anyway
     const uint64_t n = uint64_t(rows - first) * (row_width / 8);
-    hipLaunchKernelGGL(publish_run_kernel, dim3(static_cast<uint32_t>((n + 255) / 256)), dim3(256), 0, as_stream(stream),
+    launch(publish_run_kernel, dim3(static_cast<uint32_t>((n + 255) / 256)), dim3(256), 0, as_stream(stream),
                        static_cast<const uint4*>(run_k), static_cast<const uint4*>(run_v), static_cast<uint4*>(ring_k),
                        static_cast<uint4*>(ring_v), rows, first, position, ring_mask, row_width / 8);
     return check_launch("publish_run");
@@ -1128,7 +1128,7 @@ extern "C" int guffin_hip_prefill_pack(void* stream, const float* x, void* image
     if (reinterpret_cast<uintptr_t>(image) & 255u) return fail(GUFFIN_E_ALIGN, "prefill_pack: the image must be 256-byte aligned");
     const ImageLayout L = image_layout(M, K);
     const uint64_t threads = uint64_t(L.mpad) * (K / 32) * 4;
-    hipLaunchKernelGGL(prefill_pack_kernel, dim3(static_cast<uint32_t>((threads + 255) / 256)), dim3(256), 0,
+    launch(prefill_pack_kernel, dim3(static_cast<uint32_t>((threads + 255) / 256)), dim3(256), 0,
                        as_stream(stream), x, static_cast<uint8_t*>(image), M, K);
     return check_launch("prefill_pack");
 }
@@ -1149,10 +1149,10 @@ extern "C" int guffin_hip_prefill_gemm(void* stream, int dtype, const void* tile
     const uint8_t* t = static_cast<const uint8_t*>(tiles);
     const uint8_t* im = static_cast<const uint8_t*>(image);
     if (dtype == GUFFIN_Q4_K)
-        hipLaunchKernelGGL(prefill_gemm_q4k_kernel, dim3(L.mpad / kWaveRows, (N / kCols + 3) / 4), block, 0, s, t, im, y, M, K, N);
+        launch(prefill_gemm_q4k_kernel, dim3(L.mpad / kWaveRows, (N / kCols + 3) / 4), block, 0, s, t, im, y, M, K, N);
     else if (dtype == GUFFIN_Q6_K)
-        hipLaunchKernelGGL(prefill_gemm_q6k_kernel, dim3(L.mpad / kWaveRows, (N / kCols + 1) / 2), block, 0, s, t, im, y, M, K, N);
-    else hipLaunchKernelGGL(prefill_gemm_kernel<GUFFIN_Q8_0>, grid, block, 0, s, t, im, y, M, K, N);
+        launch(prefill_gemm_q6k_kernel, dim3(L.mpad / kWaveRows, (N / kCols + 1) / 2), block, 0, s, t, im, y, M, K, N);
+    else launch(prefill_gemm_kernel<GUFFIN_Q8_0>, grid, block, 0, s, t, im, y, M, K, N);
     return check_launch("prefill_gemm");
 }
 
@@ -1198,19 +1198,19 @@ extern "C" int guffin_hip_prefill_attention(void* stream, const float* q, const 
         // matrix-core path: V^T first, then scores and values as MFMA chains
         const ValueSpan vs = value_span(rows, position, window);
         uint16_t* vt = static_cast<uint16_t*>(workspace);
-        hipLaunchKernelGGL(transpose_values_kernel, dim3(vs.T / 32, kv_heads), dim3(256), 0, s, rv, uv, vt, vs.base32, vs.T,
+        launch(transpose_values_kernel, dim3(vs.T / 32, kv_heads), dim3(256), 0, s, rv, uv, vt, vs.base32, vs.T,
                            vs.first_visible, position, position + rows, ring_mask, kv_heads);
         if (int rc = check_launch("transpose_values")) return rc;
         const size_t lds = size_t(group) * 16384 + size_t(4) * group * 16 * 32 * 4 + size_t(group) * 16 * 2 * 4;
         if (group == 1)
-            hipLaunchKernelGGL(prefill_attention_mfma_kernel<1>, grid, block, lds, s, q, rk, uk, vt, out, rows, position, window,
+            launch(prefill_attention_mfma_kernel<1>, grid, block, lds, s, q, rk, uk, vt, out, rows, position, window,
                                ring_mask, q_heads, kv_heads, scale, vs.base32, vs.T);
         else
-            hipLaunchKernelGGL(prefill_attention_mfma_kernel<2>, grid, block, lds, s, q, rk, uk, vt, out, rows, position, window,
+            launch(prefill_attention_mfma_kernel<2>, grid, block, lds, s, q, rk, uk, vt, out, rows, position, window,
                                ring_mask, q_heads, kv_heads, scale, vs.base32, vs.T);
         return check_launch("prefill_attention_mfma");
     }
-#define GUFFIN_PA(G_) hipLaunchKernelGGL(prefill_attention_kernel<G_>, grid, block, 0, s, q, rk, rv, uk, uv, out, rows, \
+#define GUFFIN_PA(G_) launch(prefill_attention_kernel<G_>, grid, block, 0, s, q, rk, rv, uk, uv, out, rows, \
                                          position, window, ring_mask, q_heads, kv_heads, scale)
     if (group == 1) GUFFIN_PA(1); else if (group == 2) GUFFIN_PA(2); else if (group == 4) GUFFIN_PA(4);
     else return fail(GUFFIN_E_SHAPE, "prefill_attention: q_heads / kv_heads must be 1, 2 or 4");

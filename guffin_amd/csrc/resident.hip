@@ -1031,7 +1031,7 @@ static int launch_resident(hipStream_t stream, const RArgs& args, uint32_t lds) 
             return fail(GUFFIN_E_HIP, "resident forward: could not raise the dynamic LDS limit");
         raised = true;
     }
-    hipLaunchKernelGGL(kernel, dim3(kGrid), dim3(kThreads), lds, stream, args);
+    launch(kernel, dim3(kGrid), dim3(kThreads), lds, stream, args);
     return check_launch("resident_blocks");
 }
 

@@ -829,7 +829,7 @@ int launch_compact_law(hipStream_t s, const float* logits, uint32_t vocab, const
     if (int rc = select_candidates_scaled(s, logits, 1, vocab, vocab < 257 ? vocab : 257, opt.temperature, nullptr,
                                           nullptr, ws, top, status, suppressed_ok))
         return rc;
-    hipLaunchKernelGGL(draft_law_kernel, dim3(1), dim3(256), 0, s, top, opt, seed, step,
+    launch(draft_law_kernel, dim3(1), dim3(256), 0, s, top, opt, seed, step,
                        static_cast<const StepDraws*>(injected_draws), static_cast<DraftLaw*>(law), proposal, status,
                        full_error);
     return check_launch("draft_law");
@@ -841,22 +841,22 @@ int launch_full_law(hipStream_t s, const float* logits, uint32_t vocab, const Sa
                     uint64_t* cdf, uint32_t* proposal, uint32_t* status, bool suppressed_ok = false) {
     const bool greedy = opt.temperature == 0.f;
     const uint32_t padded = padded_vocab(vocab);
-    hipLaunchKernelGGL(law_sort_tile_kernel, dim3(padded / kSortTile), dim3(1024), 0, s, logits, vocab, opt.temperature,
+    launch(law_sort_tile_kernel, dim3(padded / kSortTile), dim3(1024), 0, s, logits, vocab, opt.temperature,
                        !greedy, suppressed_ok, guard, ws, status);
     if (!greedy) {
         const uint64_t* sorted = ws.keys_a;
         uint64_t* other = ws.keys_b;
         for (uint32_t width = kSortTile; width < padded; width <<= 1) {
-            hipLaunchKernelGGL(law_merge_kernel, dim3(padded / 256), dim3(256), 0, s, sorted, other, width, padded, guard);
+            launch(law_merge_kernel, dim3(padded / 256), dim3(256), 0, s, sorted, other, width, padded, guard);
             const uint64_t* done = other;
             other = const_cast<uint64_t*>(sorted);
             sorted = done;
         }
-        hipLaunchKernelGGL(law_filter_prefix_kernel, dim3(1), dim3(1024), 0, s, sorted, vocab, opt.top_k, guard, ws);
-        hipLaunchKernelGGL(law_filter_apply_kernel, dim3((vocab + 255) / 256), dim3(256), 0, s, sorted, vocab, opt, guard, ws);
+        launch(law_filter_prefix_kernel, dim3(1), dim3(1024), 0, s, sorted, vocab, opt.top_k, guard, ws);
+        launch(law_filter_apply_kernel, dim3((vocab + 255) / 256), dim3(256), 0, s, sorted, vocab, opt, guard, ws);
     }
-    hipLaunchKernelGGL(law_weights_kernel, dim3(1), dim3(1024), 0, s, vocab, greedy, guard, ws, status);
-    hipLaunchKernelGGL(law_cdf_select_kernel, dim3(vocab / 256 + 1), dim3(256), 0, s, vocab, greedy, seed, step,
+    launch(law_weights_kernel, dim3(1), dim3(1024), 0, s, vocab, greedy, guard, ws, status);
+    launch(law_cdf_select_kernel, dim3(vocab / 256 + 1), dim3(256), 0, s, vocab, greedy, seed, step,
                        static_cast<const StepDraws*>(injected_draws), guard, ws, cdf, proposal, status);
     return check_launch("draft_law_full");
 }
@@ -919,7 +919,7 @@ extern "C" int guffin_hip_draft_process(void* stream, const float* logits, uint3
     if (history_count > kHistoryCap) return fail(GUFFIN_E_CAPACITY, "draft_process: at most 64 history tokens");
     if (!std::isfinite(repetition_penalty) || !(repetition_penalty > 0.f)) return fail(GUFFIN_E_ARG, "draft_process: the penalty must be positive");
     const uint32_t blocks = std::min<uint32_t>((vocab + 255) / 256, 1024);
-    hipLaunchKernelGGL(draft_process_kernel, dim3(blocks), dim3(256), 0, as_stream(stream), logits, vocab, history,
+    launch(draft_process_kernel, dim3(blocks), dim3(256), 0, as_stream(stream), logits, vocab, history,
                        history_count, repetition_penalty, static_cast<const int32_t*>(nullptr), scores,
                        static_cast<uint32_t*>(nullptr));
     return check_launch("draft_process");
@@ -942,13 +942,13 @@ extern "C" int guffin_hip_draft_law_mapped(void* stream, const float* logits, ui
     if (!std::isfinite(opt.repetition_penalty) || !(opt.repetition_penalty > 0.f)) return fail(GUFFIN_E_ARG, "draft_law_mapped: the penalty must be positive");
     hipStream_t s = as_stream(stream);
     const uint32_t blocks = std::min<uint32_t>((vocab + 255) / 256, 1024);
-    hipLaunchKernelGGL(draft_process_kernel, dim3(blocks), dim3(256), 0, s, logits, vocab, history, history_count,
+    launch(draft_process_kernel, dim3(blocks), dim3(256), 0, s, logits, vocab, history, history_count,
                        opt.repetition_penalty, draft_to_target, scores, status);
     if (int rc = check_launch("draft_process")) return rc;
     if (int rc = launch_compact_law(s, scores, vocab, opt, seed, step, injected_draws, workspace, law, draft_proposal, status,
                                     nullptr, true))
         return rc;
-    hipLaunchKernelGGL(map_proposal_kernel, dim3(1), dim3(1), 0, s, draft_to_target, vocab, draft_proposal, target_proposal);
+    launch(map_proposal_kernel, dim3(1), dim3(1), 0, s, draft_to_target, vocab, draft_proposal, target_proposal);
     return check_launch("map_proposal");
 }
 
@@ -981,7 +981,7 @@ int draft_law_any(void* stream, const float* logits, uint32_t vocab, const void*
             return rc;
         return launch_full_law(s, logits, vocab, opt, seed, step, injected_draws, &slot->count, ws, full_cdf, proposal, status, suppressed_ok);
     }
-    hipLaunchKernelGGL(law_begin_kernel, dim3(1), dim3(1), 0, s, slot, proposal, ws.error);
+    launch(law_begin_kernel, dim3(1), dim3(1), 0, s, slot, proposal, ws.error);
     return launch_full_law(s, logits, vocab, opt, seed, step, injected_draws, nullptr, ws, full_cdf, proposal, status, suppressed_ok);
 }
 }  // namespace
@@ -1006,13 +1006,13 @@ extern "C" int guffin_hip_draft_law_any_mapped(void* stream, const float* logits
     if (!std::isfinite(opt.repetition_penalty) || !(opt.repetition_penalty > 0.f)) return fail(GUFFIN_E_ARG, "draft_law_any_mapped: the penalty must be positive");
     hipStream_t s = as_stream(stream);
     const uint32_t blocks = std::min<uint32_t>((vocab + 255) / 256, 1024);
-    hipLaunchKernelGGL(draft_process_kernel, dim3(blocks), dim3(256), 0, s, logits, vocab, history, history_count,
+    launch(draft_process_kernel, dim3(blocks), dim3(256), 0, s, logits, vocab, history, history_count,
                        opt.repetition_penalty, draft_to_target, scores, status);
     if (int rc = check_launch("draft_process")) return rc;
     if (int rc = draft_law_any(stream, scores, vocab, options, seed, step, injected_draws, workspace, law, full_cdf, draft_proposal,
                                status, true))
         return rc;
-    hipLaunchKernelGGL(map_proposal_kernel, dim3(1), dim3(1), 0, s, draft_to_target, vocab, draft_proposal, target_proposal);
+    launch(map_proposal_kernel, dim3(1), dim3(1), 0, s, draft_to_target, vocab, draft_proposal, target_proposal);
     return check_launch("map_proposal");
 }
 
@@ -1024,7 +1024,7 @@ extern "C" int guffin_hip_spec_accept_mapped(void* stream, const void* target_ca
     if (!target_candidates || !law || !proposal || !options || !result) return fail(GUFFIN_E_ARG, "spec_accept: null pointer");
     if ((history == nullptr) != (history_count == nullptr)) return fail(GUFFIN_E_ARG, "spec_accept: history needs its counts");
     const SamplerOptions opt = *static_cast<const SamplerOptions*>(options);
-    hipLaunchKernelGGL(spec_accept_kernel, dim3(1), dim3(512), 0, as_stream(stream),
+    launch(spec_accept_kernel, dim3(1), dim3(512), 0, as_stream(stream),
                        static_cast<const Candidates*>(target_candidates), static_cast<const DraftLaw*>(law), full_cdf,
                        vocab, history, history_count, proposal, opt, seed, step,
                        static_cast<const StepDraws*>(injected_draws), static_cast<SpecResult*>(result), status,

@@ -57,6 +57,54 @@ def set_spin_limit(polls):
     check(lib().guffin_hip_set_spin_limit(C.c_uint32(polls)))
 
 
+
+class Chain:
+    """Recorded launches replayed as AQL packets (guffin_hip_chain_*).  Usage:
+        chain = Chain(chained=True)
+        with chain:                 # every library call on the current stream is recorded, not run
+            plan.step(0)
+        chain.launch(); chain.wait()
+    """
+
+    def __init__(self, chained=True):
+        self.handle = C.c_void_p()
+        self.chained = chained
+        self.stream = _stream()
+
+    def __enter__(self):
+        check(lib().guffin_hip_chain_begin(self.stream, 1 if self.chained else 0, C.byref(self.handle)))
+        return self
+
+    def __exit__(self, exc_type, exc, tb):
+        if exc_type is not None:
+            lib().guffin_hip_chain_destroy(self.handle)
+            self.handle = C.c_void_p()
+            return False
+        check(lib().guffin_hip_chain_end(self.handle))
+        return False
+
+    def launch(self):
+        check(lib().guffin_hip_chain_launch(self.handle))
+
+    def wait(self):
+        check(lib().guffin_hip_chain_wait(self.handle))
+
+    def info(self):
+        a, b, c = C.c_uint32(), C.c_uint32(), C.c_uint32()
+        check(lib().guffin_hip_chain_info(self.handle, C.byref(a), C.byref(b), C.byref(c)))
+        return {"launches": a.value, "chained": b.value, "unbarriered": c.value}
+
+    def close(self):
+        if self.handle:
+            lib().guffin_hip_chain_destroy(self.handle)
+            self.handle = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
 def _stream():
     return C.c_void_p(torch.cuda.current_stream().cuda_stream)
 
