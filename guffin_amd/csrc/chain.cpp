@@ -2,7 +2,7 @@
 // objects (guffin_amd/hsaco/*.hsaco, built from the same sources with the same flags), and recorded launches
 // replayed as AQL dispatch packets.  chain.hpp describes the role and the ordering protocol.
 //
-// A replay allocates nothing: kernel arguments, counters and packets are laid down once by chain_end.
+// A replay allocates nothing: kernel arguments and packets are laid down once by chain_end.
 #include "common.hpp"
 
 #include <dirent.h>
@@ -20,14 +20,9 @@
 #include <vector>
 
 namespace guffin {
-
-void chain_clear_counters(hipStream_t stream, uint32_t* counters, uint32_t words);   // chain_kernels.hip
-
 namespace chain {
 namespace {
 
-constexpr uint32_t kMaxLinks = 4096;       // chained launches per chain
-constexpr uint32_t kCounterStride = 32;    // words between counters: one 128-byte line each
 constexpr uint32_t kHiddenBytes = 256;     // implicit kernel arguments behind the explicit ones (code object v5)
 constexpr uint64_t kWaitNanoseconds = 30ull * 1000 * 1000 * 1000;
 
@@ -154,6 +149,9 @@ int engine_init() {
     const uint32_t size = std::min<uint32_t>(max_size ? max_size : 4096u, 16384u);
     rc = hsa_queue_create(e.gpu, size, HSA_QUEUE_TYPE_SINGLE, nullptr, nullptr, UINT32_MAX, UINT32_MAX, &e.queue);
     if (rc != HSA_STATUS_SUCCESS) return engine_fail("chain: hsa_queue_create: " + hsa_text(rc));
+    // dispatch timestamps for the packets that carry a signal (the first and the last of a replay)
+    rc = hsa_amd_profiling_set_profiler_enabled(e.queue, 1);
+    if (rc != HSA_STATUS_SUCCESS) return engine_fail("chain: dispatch timestamps: " + hsa_text(rc));
     const std::string dir = library_directory() + "/hsaco";
     DIR* d = opendir(dir.c_str());
     if (!d) return engine_fail("chain: no code objects under " + dir + " (run the build)");
@@ -177,8 +175,6 @@ struct Launch {
     dim3 grid, block;
     uint32_t lds;
     std::vector<uint8_t> args;
-    bool chained;    // the kernel follows the ChainLink protocol
-    bool waits;      // ... and is ordered after its (chained) predecessor by that one's counter: no packet barrier
 };
 
 }  // namespace
@@ -188,23 +184,16 @@ struct Recorder {
     bool recording = false, built = false;
     std::string error;
     std::vector<Launch> launches;
-    // links handed out by next_link; the pending one belongs to the launch that follows
-    uint32_t links = 0;
-    bool last_chained = false, pending_waits = false;
-    uint32_t last_link = 0, last_arrivals = 0, pending_link = 0, pending_arrivals = 0;
-    uint32_t* counters = nullptr;          // device, kMaxLinks * kCounterStride words
     uint8_t* kernargs = nullptr;           // device
     std::vector<hsa_kernel_dispatch_packet_t> packets;   // headers zero (invalid) until they are copied into the ring
     std::vector<uint16_t> headers;
-    hsa_signal_t done {};
+    hsa_signal_t done {}, started {};   // completion signals of the last and of the first packet
     bool have_signal = false;
-    bool allow_chaining = true;
-    uint32_t unbarriered = 0;
+    uint64_t replays = 0;
 };
 
 namespace {
 Recorder* g_active = nullptr;
-bool g_chaining_enabled = true;
 }  // namespace
 
 Recorder* recorder_for(hipStream_t stream) {
@@ -212,21 +201,8 @@ Recorder* recorder_for(hipStream_t stream) {
     return (r && r->recording && r->stream == stream) ? r : nullptr;
 }
 
-ChainLink next_link(Recorder* r, uint32_t arrivals, uint32_t* status) {
-    ChainLink link {nullptr, 0, 0, 0, g_spin_limit, status};
-    if (!r || !r->allow_chaining) return link;
-    if (r->links >= kMaxLinks) { r->error = "chain: more chained launches than the chain has counters"; return link; }
-    link.counters = r->counters;
-    link.signal_index = r->links++;
-    r->pending_link = link.signal_index;
-    r->pending_arrivals = arrivals;
-    r->pending_waits = r->last_chained;
-    if (r->last_chained) { link.wait_index = r->last_link; link.wait_count = r->last_arrivals; }
-    return link;
-}
-
 void record(Recorder* r, const void* host_function, dim3 grid, dim3 block, uint32_t lds_bytes, const void* args,
-            uint32_t arg_bytes, bool chained) {
+            uint32_t arg_bytes) {
     if (!r->error.empty()) return;
     Engine& e = g_engine;
     const KernelInfo* k = nullptr;
@@ -246,13 +222,8 @@ void record(Recorder* r, const void* host_function, dim3 grid, dim3 block, uint3
                  + std::to_string(k->explicit_end) + " bytes)";
         return;
     }
-    const bool linked = chained && r->allow_chaining;
-    Launch l {k, grid, block, lds_bytes, std::vector<uint8_t>(static_cast<const uint8_t*>(args), static_cast<const uint8_t*>(args) + arg_bytes),
-              linked, linked && r->pending_waits};
-    r->launches.push_back(std::move(l));
-    r->last_chained = linked;
-    if (linked) { r->last_link = r->pending_link; r->last_arrivals = r->pending_arrivals; }
-    r->pending_waits = false;
+    r->launches.push_back(Launch {k, grid, block, lds_bytes,
+                                  std::vector<uint8_t>(static_cast<const uint8_t*>(args), static_cast<const uint8_t*>(args) + arg_bytes)});
 }
 
 namespace {
@@ -296,11 +267,11 @@ int build(Recorder& r) {
     if (hipMalloc(reinterpret_cast<void**>(&r.kernargs), total) != hipSuccess) return fail(GUFFIN_E_HIP, "chain_end: kernel argument buffer");
     if (hipMemcpy(r.kernargs, host.data(), total, hipMemcpyHostToDevice) != hipSuccess) return fail(GUFFIN_E_HIP, "chain_end: kernel argument upload");
     hsa_status_t rc = hsa_signal_create(0, 0, nullptr, &r.done);
+    if (rc == HSA_STATUS_SUCCESS) rc = hsa_signal_create(0, 0, nullptr, &r.started);
     if (rc != HSA_STATUS_SUCCESS) return engine_fail("chain_end: signal: " + hsa_text(rc));
     r.have_signal = true;
     r.packets.assign(r.launches.size(), hsa_kernel_dispatch_packet_t {});
     r.headers.assign(r.launches.size(), 0);
-    r.unbarriered = 0;
     for (size_t i = 0; i < r.launches.size(); ++i) {
         const Launch& l = r.launches[i];
         hsa_kernel_dispatch_packet_t& p = r.packets[i];
@@ -317,13 +288,9 @@ int build(Recorder& r) {
         p.completion_signal.handle = 0;
         const bool last = i + 1 == r.launches.size();
         if (last) p.completion_signal = r.done;
-        // A launch that keeps its own order with its predecessor carries no barrier and skips the cache invalidation at
-        // its start (what it reads of the chain's data, it reads with device-coherent loads); every launch writes its
-        // results back at its end, and the last one to the host as well.
-        const bool free_running = l.waits;
-        r.unbarriered += free_running ? 1u : 0u;
-        r.headers[i] = packet_header(!free_running, free_running ? HSA_FENCE_SCOPE_NONE : HSA_FENCE_SCOPE_AGENT,
-                                     last ? HSA_FENCE_SCOPE_SYSTEM : HSA_FENCE_SCOPE_AGENT);
+        else if (i == 0) p.completion_signal = r.started;   // carries the replay's first timestamp
+        // the order and visibility of a stream: barrier bit, agent-scope fences; the last launch releases to the host
+        r.headers[i] = packet_header(true, HSA_FENCE_SCOPE_AGENT, last ? HSA_FENCE_SCOPE_SYSTEM : HSA_FENCE_SCOPE_AGENT);
     }
     r.built = true;
     return GUFFIN_OK;
@@ -336,21 +303,14 @@ int build(Recorder& r) {
 using namespace guffin;
 using namespace guffin::chain;
 
-extern "C" int guffin_hip_chain_begin(void* stream, int chained, void** out) {
+extern "C" int guffin_hip_chain_begin(void* stream, void** out) {
     if (!out) return fail(GUFFIN_E_ARG, "chain_begin: null pointer");
     if (g_active && g_active->recording) return fail(GUFFIN_E_STATE, "chain_begin: another chain is being recorded");
     if (int rc = engine_init()) return rc;
     auto* r = new Recorder();
     r->stream = as_stream(stream);
-    r->allow_chaining = chained != 0 && g_chaining_enabled;
-    if (hipMalloc(reinterpret_cast<void**>(&r->counters), size_t(kMaxLinks) * kCounterStride * 4) != hipSuccess) {
-        delete r;
-        return fail(GUFFIN_E_HIP, "chain_begin: counter buffer");
-    }
     r->recording = true;
     g_active = r;
-    // the first launch of every replay clears the counters (a kernel: it orders itself with the rest of the queue)
-    chain_clear_counters(r->stream, r->counters, kMaxLinks * kCounterStride);
     *out = r;
     return GUFFIN_OK;
 }
@@ -379,6 +339,8 @@ extern "C" int guffin_hip_chain_launch(void* chain) {
         if (++spins > (1ull << 34)) return fail(GUFFIN_E_HIP, "chain_launch: the queue does not drain");
     }
     hsa_signal_add_relaxed(r->done, 1);
+    if (n > 1) hsa_signal_add_relaxed(r->started, 1);
+    r->replays += 1;
     auto* ring = static_cast<hsa_kernel_dispatch_packet_t*>(q->base_address);
     const uint64_t mask = q->size - 1;
     for (uint64_t i = 0; i < n; ++i) {
@@ -400,14 +362,29 @@ extern "C" int guffin_hip_chain_wait(void* chain) {
     return GUFFIN_OK;
 }
 
-extern "C" int guffin_hip_chain_info(void* chain, uint32_t* launches, uint32_t* chained, uint32_t* unbarriered) {
+// Device time of the last replay, from the start of its first dispatch to the end of its last (the reference's
+// gpu_duration_ns of a command buffer, metal_command_context.hpp:19-45: GPUEndTime - GPUStartTime).
+extern "C" int guffin_hip_chain_gpu_ns(void* chain, uint64_t* nanoseconds) {
     auto* r = static_cast<Recorder*>(chain);
-    if (!r) return fail(GUFFIN_E_ARG, "chain_info: null pointer");
-    uint32_t c = 0;
-    for (const auto& l : r->launches) c += l.chained ? 1u : 0u;
-    if (launches) *launches = static_cast<uint32_t>(r->launches.size());
-    if (chained) *chained = c;
-    if (unbarriered) *unbarriered = r->unbarriered;
+    if (!r || !nanoseconds) return fail(GUFFIN_E_ARG, "chain_gpu_ns: null pointer");
+    if (!r->built || r->replays == 0) return fail(GUFFIN_E_STATE, "chain_gpu_ns: no replay has run");
+    if (hsa_signal_load_scacquire(r->done) >= 1) return fail(GUFFIN_E_STATE, "chain_gpu_ns: a replay is still running (wait first)");
+    hsa_amd_profiling_dispatch_time_t first {}, last {};
+    hsa_status_t rc = hsa_amd_profiling_get_dispatch_time(g_engine.gpu, r->done, &last);
+    if (rc == HSA_STATUS_SUCCESS) rc = r->packets.size() > 1 ? hsa_amd_profiling_get_dispatch_time(g_engine.gpu, r->started, &first) : rc;
+    if (rc != HSA_STATUS_SUCCESS) return engine_fail("chain_gpu_ns: " + hsa_text(rc));
+    if (r->packets.size() == 1) first = last;
+    uint64_t frequency = 0;
+    hsa_system_get_info(HSA_SYSTEM_INFO_TIMESTAMP_FREQUENCY, &frequency);
+    if (frequency == 0 || last.end < first.start) return fail(GUFFIN_E_HIP, "chain_gpu_ns: no usable timestamps");
+    *nanoseconds = static_cast<uint64_t>(static_cast<double>(last.end - first.start) * 1e9 / static_cast<double>(frequency));
+    return GUFFIN_OK;
+}
+
+extern "C" int guffin_hip_chain_info(void* chain, uint32_t* launches) {
+    auto* r = static_cast<Recorder*>(chain);
+    if (!r || !launches) return fail(GUFFIN_E_ARG, "chain_info: null pointer");
+    *launches = static_cast<uint32_t>(r->launches.size());
     return GUFFIN_OK;
 }
 
@@ -416,8 +393,7 @@ extern "C" int guffin_hip_chain_destroy(void* chain) {
     if (!r) return GUFFIN_OK;
     if (r->recording) { r->recording = false; if (g_active == r) g_active = nullptr; }
     if (r->built) hsa_signal_wait_scacquire(r->done, HSA_SIGNAL_CONDITION_LT, 1, kWaitNanoseconds, HSA_WAIT_STATE_BLOCKED);
-    if (r->have_signal) hsa_signal_destroy(r->done);
-    if (r->counters) (void)hipFree(r->counters);
+    if (r->have_signal) { hsa_signal_destroy(r->done); hsa_signal_destroy(r->started); }
     if (r->kernargs) (void)hipFree(r->kernargs);
     delete r;
     return GUFFIN_OK;

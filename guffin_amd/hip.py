@@ -60,19 +60,18 @@ def set_spin_limit(polls):
 
 class Chain:
     """Recorded launches replayed as AQL packets (guffin_hip_chain_*).  Usage:
-        chain = Chain(chained=True)
+        chain = Chain()
         with chain:                 # every library call on the current stream is recorded, not run
             plan.step(0)
         chain.launch(); chain.wait()
     """
 
-    def __init__(self, chained=True):
+    def __init__(self):
         self.handle = C.c_void_p()
-        self.chained = chained
         self.stream = _stream()
 
     def __enter__(self):
-        check(lib().guffin_hip_chain_begin(self.stream, 1 if self.chained else 0, C.byref(self.handle)))
+        check(lib().guffin_hip_chain_begin(self.stream, C.byref(self.handle)))
         return self
 
     def __exit__(self, exc_type, exc, tb):
@@ -89,10 +88,15 @@ class Chain:
     def wait(self):
         check(lib().guffin_hip_chain_wait(self.handle))
 
-    def info(self):
-        a, b, c = C.c_uint32(), C.c_uint32(), C.c_uint32()
-        check(lib().guffin_hip_chain_info(self.handle, C.byref(a), C.byref(b), C.byref(c)))
-        return {"launches": a.value, "chained": b.value, "unbarriered": c.value}
+    def gpu_ns(self):
+        ns = C.c_uint64()
+        check(lib().guffin_hip_chain_gpu_ns(self.handle, C.byref(ns)))
+        return ns.value
+
+    def launches(self):
+        n = C.c_uint32()
+        check(lib().guffin_hip_chain_info(self.handle, C.byref(n)))
+        return n.value
 
     def close(self):
         if self.handle:
@@ -104,6 +108,7 @@ class Chain:
             self.close()
         except Exception:
             pass
+
 
 def _stream():
     return C.c_void_p(torch.cuda.current_stream().cuda_stream)

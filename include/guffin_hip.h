@@ -797,25 +797,25 @@ int guffin_hip_ticket_release(void* stream, guffin_verify_ticket* ticket);
 /* ---- recorded launch chains ---------------------------------------------------------------------------------
  * The command buffer of the reference: MetalCommandContext encodes a whole pass and commits it once
  * (src/tensor/backends/metal/metal_command_context.hpp:346-353, commit / wait_until_completed / commit_and_wait).
- * Between guffin_hip_chain_begin(stream, ...) and guffin_hip_chain_end every kernel this library would enqueue on
- * `stream` is recorded instead of run (guffin_hip_h1_step, guffin_hip_forward_rows, ... are called as usual);
- * guffin_hip_chain_launch replays the recorded launches as AQL dispatch packets on a hardware queue of the
- * library's own and returns at once, guffin_hip_chain_wait blocks until every replay has completed.  Buffers and
- * arguments are the recorded ones: a replay reads its inputs (root token, step draws) from device memory.
- * `chained` != 0 lets kernels that keep their own order with their predecessor (a counter raised by the
- * predecessor's workgroups once their stores have landed, polled with the spin limit as bound) run without the
- * packet barrier, so that their first weight tiles travel while the predecessor drains; a wait that gives up
- * raises GUFFIN_STATUS_SYNC and the replay still ends.  With chained == 0 every packet carries the barrier and
- * agent-scope fences, which is what a stream does.  Results are those of the same calls made directly, bit for
- * bit.  guffin_hip_chain_launch first waits for the work already enqueued on `stream`; work enqueued on any HIP
- * stream afterwards is not ordered after the replay: call guffin_hip_chain_wait first.  One chain records at a
- * time; begin / end allocate (counters, kernel arguments), launch and wait do not. */
-int guffin_hip_chain_begin(void* stream, int chained, void** chain);
+ * Between guffin_hip_chain_begin(stream, ..) and guffin_hip_chain_end every kernel this library would enqueue on
+ * `stream` is recorded instead of run (guffin_hip_h1_step, guffin_hip_forward_rows, .. are called as usual; calls
+ * that copy or synchronise are not recordable); guffin_hip_chain_launch replays the recorded launches as AQL dispatch
+ * packets on a hardware queue of the library's own and returns at once, guffin_hip_chain_wait blocks until every
+ * replay has completed.  Buffers and arguments are the recorded ones: a replay reads its inputs (root token, step
+ * draws) from device memory.  Every packet carries the barrier bit and agent-scope fences, the last one a
+ * system-scope release: the order and visibility of a stream, and the results of the same calls made directly, bit
+ * for bit.  guffin_hip_chain_launch first waits for the work already enqueued on `stream`; work enqueued on any HIP
+ * stream afterwards is not ordered after the replay: call guffin_hip_chain_wait first.  One chain records at a time;
+ * begin / end allocate (kernel arguments), launch and wait do not. */
+int guffin_hip_chain_begin(void* stream, void** chain);
 int guffin_hip_chain_end(void* chain);
 int guffin_hip_chain_launch(void* chain);
 int guffin_hip_chain_wait(void* chain);
-/* launches recorded, how many of them follow the counter protocol, how many run without the packet barrier */
-int guffin_hip_chain_info(void* chain, uint32_t* launches, uint32_t* chained, uint32_t* unbarriered);
+/* Device time of the last replay in nanoseconds, first dispatch's start to last dispatch's end: MetalCommandStats'
+ * gpu_duration_ns (metal_command_context.hpp:19-45).  After guffin_hip_chain_wait. */
+int guffin_hip_chain_gpu_ns(void* chain, uint64_t* nanoseconds);
+/* launches recorded */
+int guffin_hip_chain_info(void* chain, uint32_t* launches);
 int guffin_hip_chain_destroy(void* chain);
 
 #ifdef __cplusplus
