@@ -29,6 +29,14 @@ extern uint32_t g_spin_limit;
 extern unsigned long long* g_resident_stamps;
 extern int g_forward_mode;
 bool resident_fits(const guffin_model_desc& m, uint32_t rows);
+// Whether forward_rows runs the resident pass for this model now: the model fits, the mode asks for it (2) or leaves
+// the choice open (0) for a model with one KV head, and no earlier pass of this process gave up a wait.
+bool resident_chosen(const guffin_model_desc& m, uint32_t rows);
+// Host code that reads a device status word reports it here: GUFFIN_STATUS_SYNC switches the automatic choice of
+// the resident pass off for the rest of the process (a device shared with other work, or one whose dispatcher does
+// not place the workgroups as the pass assumes, would raise it on every pass).
+void resident_note_status(uint32_t status_word);
+int resident_init(int cu_count);
 uint64_t resident_scratch_bytes(const guffin_model_desc& m, uint32_t rows);
 uint32_t resident_sync_words(const guffin_model_desc& m);
 int resident_launch(hipStream_t stream, const guffin_model_desc& m, uint32_t rows, uint32_t first, uint32_t count,

@@ -55,6 +55,7 @@ extern "C" int guffin_hip_init(int device) {
     }
     if (gemv_init(prop.multiProcessorCount) != 0 || ops_init(prop.multiProcessorCount) != 0 || head_init() != 0)
         return fail(GUFFIN_E_HIP, "init: could not raise a kernel's dynamic LDS limit");
+    resident_init(prop.multiProcessorCount);
     if (gemv_packed_init(device, prop.multiProcessorCount) != 0)
         return fail(GUFFIN_E_HIP, "init: could not take the address of the static scratch array on this device");
     return GUFFIN_OK;

@@ -124,8 +124,26 @@ int forward(hipStream_t s, guffin_draft_plan* p, const Buffers& b, uint32_t rows
         GUFFIN_TRY(move_rows(s, p, b, first, at + rows, true));
         p->backup_end = at + rows;
     }
+    // The resident pass can give up a wait (a device shared with other work): its rows, and whatever else it
+    // raised in the status word, are then not to be trusted.  These calls are host-synchronous anyway: the status
+    // word is read before and after such a pass and, if the bit came up, put back, the resident form is switched
+    // off for the process and the pass runs again, one launch per operator.
+    const bool watched = resident_chosen(m, rows) && g_forward_mode == 0;
+    uint32_t before = 0, after = 0;
+    if (watched && (hipStreamSynchronize(s) != hipSuccess || hipMemcpy(&before, b.status, 4, hipMemcpyDeviceToHost) != hipSuccess))
+        return fail(GUFFIN_E_HIP, "draft_plan: the stream failed");
     GUFFIN_TRY(guffin_hip_forward_rows(s, &m, b.tokens, rows, at, b.forward, b.forward_bytes, b.priv_k, b.priv_v, b.hidden,
                                        b.hidden_sums, b.status));
+    if (watched) {
+        if (hipStreamSynchronize(s) != hipSuccess || hipMemcpy(&after, b.status, 4, hipMemcpyDeviceToHost) != hipSuccess)
+            return fail(GUFFIN_E_HIP, "draft_plan: the pass failed");
+        if ((after & GUFFIN_STATUS_SYNC) && !(before & GUFFIN_STATUS_SYNC)) {
+            resident_note_status(after);
+            if (hipMemcpy(b.status, &before, 4, hipMemcpyHostToDevice) != hipSuccess) return fail(GUFFIN_E_HIP, "draft_plan: the pass failed");
+            GUFFIN_TRY(guffin_hip_forward_rows(s, &m, b.tokens, rows, at, b.forward, b.forward_bytes, b.priv_k, b.priv_v, b.hidden,
+                                               b.hidden_sums, b.status));
+        }
+    }
     GUFFIN_TRY(guffin_hip_commit_rows(s, &m, b.priv_k, b.priv_v, b.ring_k_table, b.ring_v_table, nullptr, at, rows));
     p->materialized = at + rows;
     p->last_rows = rows;

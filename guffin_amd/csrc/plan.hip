@@ -232,7 +232,7 @@ int forward_rows(hipStream_t stream, const guffin_model_desc& m, const uint32_t*
     const float attn_scale = 1.0f / std::sqrt(static_cast<float>(m.head_dim));
     // the resident pass is the default where it is the faster one: models with a single KV head (the drafter's
     // small blocks); it can be forced for any model it covers
-    const bool resident = s.exchange != nullptr && (g_forward_mode == 2 || (g_forward_mode == 0 && m.kv_heads == 1));
+    const bool resident = s.exchange != nullptr && resident_chosen(m, rows);
     if (g_forward_mode == 2 && !resident) return fail(GUFFIN_E_SHAPE, "forward: the resident pass does not cover this model");
     const uint32_t sync_words = resident ? s.sync_words : 0u;
     const uint32_t n_stage = std::max({m.layer_count * rows, rows * (m.head_dim / 2), sync_words});
@@ -868,6 +868,7 @@ extern "C" int guffin_hip_session_complete(void* stream, guffin_h1_session* s, u
         return fail(GUFFIN_E_HIP, "session_complete: read-back failed");
     }
     *emitted_count = 0;
+    resident_note_status(status);   // a wait that gave up: later cycles of this process run one launch per operator
     if (status != 0 || r.status != 0) {
         // a numerical fault or a refused law: the rows of this cycle may already be in the caches
         s->state = GUFFIN_TXN_POISONED;

@@ -946,6 +946,24 @@ __global__ void __launch_bounds__(kThreads) resident_blocks_kernel(const RArgs a
 uint32_t g_spin_limit = 1u << 20;
 unsigned long long* g_resident_stamps = nullptr;
 int g_forward_mode = 0;   // 0: resident where the model fits, 1: one launch per operator, 2: resident or an error
+namespace {
+int g_device_cus = 0;          // CU count of the device guffin_hip_init saw (0: not initialised yet)
+bool g_resident_off = false;   // a pass gave up a wait: the automatic mode uses one launch per operator from then on
+}  // namespace
+
+int resident_init(int cu_count) {
+    g_device_cus = cu_count;
+    return 0;
+}
+
+void resident_note_status(uint32_t status_word) {
+    if (status_word & GUFFIN_STATUS_SYNC) g_resident_off = true;
+}
+
+bool resident_chosen(const guffin_model_desc& m, uint32_t rows) {
+    if (!resident_fits(m, rows)) return false;
+    return g_forward_mode == 2 || (g_forward_mode == 0 && m.kv_heads == 1 && !g_resident_off);
+}
 
 }  // namespace guffin
 
@@ -958,6 +976,9 @@ uint32_t resident_lds_bytes(const guffin_model_desc& m, uint32_t rows, uint32_t 
 // Whether the resident kernel covers this model: one KV head per XCD (1 or 8 heads of 256), rows of the
 // residual in 512 threads, formats of one block length per model.
 bool resident_fits(const guffin_model_desc& m, uint32_t rows) {
+    // the placement the pass relies on (256 workgroups, one per CU, dealt to 8 XCDs of 32 CUs in turn) is this part's:
+    // on a device with another CU count the per-operator path runs
+    if (g_device_cus != 0 && g_device_cus != static_cast<int>(kGrid)) return false;
     if (rows < 1 || rows > 2 || m.head_dim != 256) return false;
     if (m.kv_heads != 1 && m.kv_heads != 8) return false;
     const uint32_t G = m.q_heads / m.kv_heads;
@@ -1100,8 +1121,11 @@ int resident_launch(hipStream_t stream, const guffin_model_desc& m, uint32_t row
 extern "C" int guffin_hip_set_forward_mode(int mode) {
     if (mode < 0 || mode > 2) return fail(GUFFIN_E_ARG, "set_forward_mode: 0 (automatic), 1 (one launch per operator) or 2 (resident only)");
     g_forward_mode = mode;
+    g_resident_off = false;   // the caller chose again: an earlier give-up no longer decides
     return GUFFIN_OK;
 }
+
+extern "C" int guffin_hip_resident_enabled(void) { return g_resident_off ? 0 : 1; }
 
 extern "C" int guffin_hip_set_spin_limit(uint32_t polls) {
     g_spin_limit = polls;

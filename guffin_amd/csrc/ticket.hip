@@ -213,6 +213,7 @@ extern "C" int guffin_hip_ticket_complete(void* stream, guffin_verify_ticket* t,
         t->state = GUFFIN_TXN_POISONED;  // the pass may still be running over the private rows
         return fail(GUFFIN_E_HIP, "ticket_complete: wait or read-back failed, the ticket is poisoned");
     }
+    resident_note_status(status[0]);
     uint32_t raised = status[0];
     for (uint32_t r = 0; r < t->rows; ++r) raised |= status[1 + r];
     if (device_status) *device_status = raised;

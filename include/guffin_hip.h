@@ -452,8 +452,14 @@ int guffin_hip_forward_tree_rows(void* stream, const guffin_model_desc* model, c
  * cross XCDs.  Every wait in it is bounded by the spin limit (polls of a counter): a workgroup that gives up
  * raises GUFFIN_STATUS_SYNC in the status word and the launch still ends.  Same results as the
  * per-operator path up to fp32 summation order; a row's arithmetic does not depend on the row count in
- * the projections.  No counterpart in the reference (its command buffers are per operator). */
+ * the projections.  No counterpart in the reference (its command buffers are per operator).
+ * The resident pass assumes this part's placement (256 CUs; a device with another CU count always runs one launch
+ * per operator).  When host code of this library reads a status word with GUFFIN_STATUS_SYNC up (a session or
+ * ticket completing, a drafter plan's pass), the automatic mode stops choosing the resident pass for the rest of the
+ * process -- guffin_hip_resident_enabled() then returns 0 -- until guffin_hip_set_forward_mode is called again; a
+ * drafter plan, whose calls are host-synchronous, also runs the pass that gave up once more, per operator. */
 int guffin_hip_set_forward_mode(int mode);
+int guffin_hip_resident_enabled(void);
 int guffin_hip_set_spin_limit(uint32_t polls);
 /* Profiling aid: with a device buffer of 16 * blocks u64 words set, workgroup 0 of the resident pass stores the
  * 100 MHz clock at the start of each block's q/k/v projection, attention, o-projection, first norm pair,

@@ -145,11 +145,32 @@ private:
     return buffer;
 }
 
-struct HipCommandStats {   // the subset of MetalCommandStats (metal_command_context.hpp:19-46) with a meaning here
+// MetalCommandStats (metal_command_context.hpp:19-46) with the fields that have a meaning here.  One in-order stream
+// stands for the command buffer and its encoders; projections are counted by weight format and row count
+// (decode = one row, width_two = two rows, small_batch = the pairs of a longer run, generic_tiled = the
+// matrix-core GEMM of a prefill chunk); gpu_duration_ns is the device time between the batch's first encode
+// and its commit (hipEvent pair, read by wait_until_completed).
+struct HipCommandStats {
+    std::uint32_t command_buffer_count = 0;
     std::uint32_t commit_count = 0;
     std::uint32_t synchronous_wait_count = 0;
     std::uint32_t compute_dispatch_count = 0;
+    std::uint32_t memory_barrier_count = 0;
     std::uint32_t transient_buffer_allocation_count = 0;   // stays 0: nothing is allocated after construction
+    std::uint64_t gpu_duration_ns = 0;
+    std::uint32_t q4_decode_projection_count = 0;
+    std::uint32_t q8_decode_projection_count = 0;
+    std::uint32_t q8_width_two_projection_count = 0;
+    std::uint32_t q4_small_batch_projection_count = 0;
+    std::uint32_t q4_width_two_projection_count = 0;
+    std::uint32_t q4_generic_tiled_projection_count = 0;
+    std::uint32_t q6_decode_projection_count = 0;
+    std::uint32_t q6_small_batch_projection_count = 0;
+    std::uint32_t q6_width_two_projection_count = 0;
+    std::uint32_t q6_generic_tiled_projection_count = 0;
+    std::uint32_t decode_attention_dispatch_count = 0;      // verify / decode attention encodes
+    std::uint32_t decode_attention_partition_count = 0;     // token partitions of those launches
+    std::uint64_t decode_attention_token_count = 0;         // tokens their longest rows attend
 };
 
 // ---- the context ----------------------------------------------------------------------------
@@ -162,6 +183,8 @@ public:
         : label_(label), scratch_floats_(scratch_floats) {
         check(guffin_hip_init(device));
         check_hip(hipStreamCreate(&stream_), "stream creation failed");
+        check_hip(hipEventCreate(&batch_start_), "event creation failed");
+        check_hip(hipEventCreate(&batch_end_), "event creation failed");
         check_hip(hipMalloc(&scratch_, scratch_floats * sizeof(float)), "allocation failed");
         check_hip(hipMalloc(&receipt_, scratch_floats * sizeof(float)), "allocation failed");
         check_hip(hipMalloc(&meta_, kMetaWords * sizeof(std::uint32_t)), "allocation failed");
@@ -172,6 +195,8 @@ public:
         (void)hipFree(scratch_);
         (void)hipFree(receipt_);
         (void)hipFree(meta_);
+        if (batch_start_) (void)hipEventDestroy(batch_start_);
+        if (batch_end_) (void)hipEventDestroy(batch_end_);
         if (stream_) (void)hipStreamDestroy(stream_);
     }
     HipCommandContext(const HipCommandContext&) = delete;
@@ -180,7 +205,7 @@ public:
     // Makes a completed context encodable again (:61): the stream is reused as it is.
     void restart() {
         if (submitted_ && !completed_) throw std::logic_error("HIP command context restarted before completion");
-        submitted_ = completed_ = false;
+        submitted_ = completed_ = started_ = false;
     }
     [[nodiscard]] hipStream_t stream() const noexcept { return stream_; }
 
@@ -233,6 +258,8 @@ public:
             check(guffin_hip_prefill_pack(stream_, f32(input), receipt_, row_count, K));
             check(guffin_hip_prefill_gemm(stream_, dtype, dev(weight), receipt_, f32(output), row_count, K, N));
             stats_.compute_dispatch_count += 2;
+            if (dtype == GUFFIN_Q4_K) ++stats_.q4_generic_tiled_projection_count;
+            if (dtype == GUFFIN_Q6_K) ++stats_.q6_generic_tiled_projection_count;
             return;
         }
         for (std::uint32_t row = 0; row < row_count; row += 2U) {
@@ -246,6 +273,7 @@ public:
                 sums = make_receipt(x, rows, K);
             }
             gemv(dtype, dev(weight), x, sums, f32(output) + std::size_t(row) * N, rows, K, N);
+            count_projection(dtype, rows, row_count > 2U);
         }
     }
     // Logit rows of the output head (:103): the same GEMV on the head's tiles.
@@ -263,6 +291,7 @@ public:
         const float* x = f32(input) + std::size_t(input_row_start) * K;
         gemv(guffin_dtype(weight.descriptor().dtype), dev(weight), x, make_receipt(x, row_count, K), f32(logits_tile),
              row_count, K, N);
+        count_projection(guffin_dtype(weight.descriptor().dtype), row_count, false);
     }
 
     void encode_head_rms_norm(const BackendBuffer& input, const BackendBuffer& weight, const BackendBuffer& output,
@@ -360,6 +389,9 @@ public:
                                           private_rows, max_tokens, cache_row_mask, query_head_count, kv_head_count, key_dimension,
                                           scale, status_word()));
         stats_.compute_dispatch_count += 2;
+        ++stats_.decode_attention_dispatch_count;
+        stats_.decode_attention_partition_count += partitions;
+        stats_.decode_attention_token_count += max_tokens;
     }
     void encode_verifier_kv_scatter(const BackendBuffer& private_key, const BackendBuffer& private_value,
                                     const BackendBuffer& selected_nodes, const BackendBuffer& resident_key,
@@ -484,12 +516,13 @@ public:
         return 2U;
     }
 
-    void encode_memory_barrier() {}   // one in-order stream
+    void encode_memory_barrier() { require_encodable(); ++stats_.memory_barrier_count; }   // one in-order stream: nothing to enqueue
     void push_debug_group(std::string_view) {}
     void pop_debug_group() {}
 
     HipCommandStats commit() {
         require_encodable();
+        check_hip(hipEventRecord(batch_end_, stream_), "event record failed");
         submitted_ = true;
         ++stats_.commit_count;
         return stats_;
@@ -497,6 +530,13 @@ public:
     HipCommandStats wait_until_completed() {
         if (!submitted_) throw std::logic_error("HIP command context waited before commit");
         if (hipStreamSynchronize(stream_) != hipSuccess) throw_hip("the stream failed");
+        if (!completed_) {
+            float ms = 0.0F;
+            if (started_ && hipEventElapsedTime(&ms, batch_start_, batch_end_) == hipSuccess)
+                stats_.gpu_duration_ns = static_cast<std::uint64_t>(static_cast<double>(ms) * 1e6);
+            else
+                stats_.gpu_duration_ns = 0;
+        }
         completed_ = true;
         ++stats_.synchronous_wait_count;
         return stats_;
@@ -547,8 +587,14 @@ private:
     // meta_: [0] operator status, [1..2] per-row selection status, [16..] two resolved requests of host-side calls
     static constexpr std::uint32_t kMetaRowStatus = 1, kMetaResolved = 16, kMetaWords = 16 + 2 * 68;
 
-    void require_encodable() const {
+    // every encode passes here first: the batch's first one also marks its start on the stream
+    void require_encodable() {
         if (submitted_) throw std::logic_error("HIP command context is already committed");
+        if (!started_) {
+            check_hip(hipEventRecord(batch_start_, stream_), "event record failed");
+            started_ = true;
+            ++stats_.command_buffer_count;
+        }
     }
     void require_completed(const char* what) const {
         if (!completed_) throw std::logic_error(std::string("HIP ") + what + " cannot be read before completion");
@@ -563,6 +609,11 @@ private:
         const auto v = d.shape.dimension(index);
         if (v > UINT32_MAX) throw std::invalid_argument("HIP backend: dimension exceeds 32 bits");
         return static_cast<std::uint32_t>(v);
+    }
+    void count_projection(int dtype, std::uint32_t rows, bool part_of_a_batch) {
+        if (dtype == GUFFIN_Q4_K) ++(part_of_a_batch ? stats_.q4_small_batch_projection_count : rows == 2U ? stats_.q4_width_two_projection_count : stats_.q4_decode_projection_count);
+        else if (dtype == GUFFIN_Q6_K) ++(part_of_a_batch ? stats_.q6_small_batch_projection_count : rows == 2U ? stats_.q6_width_two_projection_count : stats_.q6_decode_projection_count);
+        else ++(rows == 2U ? stats_.q8_width_two_projection_count : stats_.q8_decode_projection_count);
     }
     [[nodiscard]] std::uint32_t* status_word() const { return meta_; }
     [[nodiscard]] std::uint32_t* row_status(std::uint32_t rows) {
@@ -665,7 +716,8 @@ private:
     void* receipt_ = nullptr;    // self-made activation receipt / prefill operand image
     std::uint32_t* meta_ = nullptr;
     std::size_t scratch_floats_;
-    bool submitted_ = false, completed_ = false;
+    hipEvent_t batch_start_ = nullptr, batch_end_ = nullptr;
+    bool submitted_ = false, completed_ = false, started_ = false;
     HipCommandStats stats_;
 };
 

@@ -182,3 +182,34 @@ def test_attention_from_projection_planes_equals_the_separate_passes(hip, rows, 
     assert torch.equal(gk.view(torch.int16), pk.view(torch.int16)) and torch.equal(gv.view(torch.int16), pv.view(torch.int16))
     assert torch.equal(got.view(torch.int32), want.view(torch.int32))
     assert torch.equal(got_sums.view(torch.int32), want_sums.view(torch.int32))
+
+
+@pytest.mark.parametrize("offset_bytes", [4, 12])
+def test_kv_views_at_any_word_offset(hip, offset_bytes):
+    """K/V buffers may be views that start at any 4-byte offset of their allocation (the reference's case uses a
+    12-byte one, tests/tensor/gemma3_metal_tests.cpp:765-774): the same bits as from 16-byte aligned rows, through
+    the separate pass and through the pass that prepares q/k/v itself."""
+    import torch
+    rows, q_heads, kv_heads, hd, cap, position = 2, 16, 8, 256, 2048, 1500
+    rng = np.random.default_rng(77)
+    ring_k = rng.normal(0, 1, (cap, kv_heads * hd)).astype(np.float16)
+    ring_v = rng.normal(0, 1, (cap, kv_heads * hd)).astype(np.float16)
+    pk = rng.normal(0, 1, (rows, kv_heads * hd)).astype(np.float16)
+    pv = rng.normal(0, 1, (rows, kv_heads * hd)).astype(np.float16)
+    q = dev(rng.normal(0, 1, (rows, q_heads * hd)).astype(np.float32))
+    sched = dev(contiguous_schedule(position, rows, 1024))
+    anc = dev(np.arange(rows, dtype=np.uint32))
+
+    def shifted(a):
+        pad = offset_bytes // 2
+        parent = torch.zeros(a.size + pad + 8, dtype=torch.float16, device="cuda")
+        view = parent[pad:pad + a.size].view(a.shape)
+        view.copy_(dev(a))
+        assert view.data_ptr() % 16 == offset_bytes % 16
+        return view
+
+    args = (1023 + rows, cap - 1, q_heads, kv_heads, hd, 0.0625)
+    want = hip.attention_decode(q, dev(ring_k), dev(ring_v), dev(pk), dev(pv), sched, anc, *args)
+    got = hip.attention_decode(q, shifted(ring_k), shifted(ring_v), shifted(pk), shifted(pv), sched, anc, *args)
+    torch.cuda.synchronize()
+    assert torch.equal(got, want)

@@ -246,3 +246,30 @@ def test_sampled_proposals_follow_the_law_of_each_step(hip, gfo, scaled_world):
         assert rc == 0
         assert drafted[i] == gfo.lib().gfo_draft_select(C.byref(law), C.c_uint32(word))
         window = (window + [drafted[i]])[-64:]
+
+
+def test_a_pass_that_gives_up_a_wait_is_run_again_per_operator(hip, scaled_world):
+    """The resident pass bounds every wait; when one gives up (forced here from the host: a spin limit of 0), the
+    drafter plan takes GUFFIN_STATUS_SYNC down, switches the resident form off for the process and runs the pass
+    again with one launch per operator: same logits and caches as a plan that ran per operator from the start."""
+    from guffin_amd import model
+    shape, host, device = scaled_world
+    tokens = stream(9)
+    hip.set_forward_mode(1)
+    plain = model.DraftPlan(device)
+    plain.append(tokens)
+    want_logits, want_caches = plain.read_logits().copy(), snapshot(plain, shape)
+    hip.set_forward_mode(0)
+    assert hip.lib().guffin_hip_resident_enabled() == 1
+    hip.set_spin_limit(0)
+    try:
+        print("draft plan with a spin limit of 0", flush=True)
+        plan = model.DraftPlan(device)
+        plan.append(tokens)                      # no exception: the pass was redone
+        assert hip.lib().guffin_hip_resident_enabled() == 0
+        assert np.array_equal(plan.read_logits(), want_logits)
+        assert same_caches(snapshot(plan, shape), want_caches)
+    finally:
+        hip.set_spin_limit(1 << 20)
+        hip.set_forward_mode(0)                  # an explicit choice enables the resident form again
+    assert hip.lib().guffin_hip_resident_enabled() == 1
