@@ -168,7 +168,7 @@ int ingest(hipStream_t s, guffin_draft_plan* p, const Buffers& b, const uint32_t
     if (p->has_pending) input.push_back(p->pending_token);
     input.insert(input.end(), tokens, tokens + count);
     for (size_t i = 0; i < input.size(); ++i) {
-        if (hipMemcpyAsync(b.tokens, input.data() + i, 4, hipMemcpyHostToDevice, s) != hipSuccess)
+        if (hipMemcpyWithStream(b.tokens, input.data() + i, 4, hipMemcpyHostToDevice, s) != hipSuccess)
             return poison(p, GUFFIN_E_HIP, "draft_plan: token upload failed");
         if (int rc = forward(s, p, b, 1)) { p->poisoned = 1; return rc; }
     }
@@ -279,7 +279,9 @@ extern "C" int guffin_hip_draft_plan_begin_transaction(void* stream, guffin_draf
 
 extern "C" int guffin_hip_draft_plan_abort_transaction(void* stream, guffin_draft_plan* plan) {
     GUFFIN_TRY(usable(plan, "draft_plan_abort_transaction: null pointer"));
-    if (!plan->transaction_active) return GUFFIN_OK;   // abort_transaction() is noexcept and idempotent in the reference
+    // outside a transaction the reference's abort poisons the plan (gemma3_draft.mm:1305-1312): there is nothing to
+    // go back to, and the caller's ledger is out of step with the plan's
+    if (!plan->transaction_active) { plan->poisoned = 1; return fail(GUFFIN_E_STATE, "draft_plan_abort_transaction: no transaction is open; the plan is poisoned"); }
     const Buffers b = carve(*plan->model, plan->workspace, nullptr);
     hipStream_t s = as_stream(stream);
     if (int rc = move_rows(s, plan, b, plan->checkpoint_materialized, plan->backup_end, false)) { plan->poisoned = 1; return rc; }
@@ -298,10 +300,11 @@ extern "C" int guffin_hip_draft_plan_abort_transaction(void* stream, guffin_draf
     return GUFFIN_OK;
 }
 
-// 1 if truncate(position) would be admitted: only rows of the open transaction can be taken back
+// 1 if truncate(position) would be admitted: the current position always (nothing changes), and inside a transaction
+// any position down to where it began (gemma3_draft.mm:1283-1288)
 extern "C" int guffin_hip_draft_plan_can_truncate(const guffin_draft_plan* plan, uint32_t position) {
-    return plan && plan->model && !plan->poisoned && plan->transaction_active && position >= plan->checkpoint_position
-        && position <= plan->position;
+    if (!plan || !plan->model || plan->poisoned || position > plan->position) return 0;
+    return position == plan->position || (plan->transaction_active && position >= plan->checkpoint_position);
 }
 
 extern "C" int guffin_hip_draft_plan_truncate(void* stream, guffin_draft_plan* plan, uint32_t position) {
@@ -385,7 +388,7 @@ extern "C" int guffin_hip_draft_plan_propose(void* stream, guffin_draft_plan* pl
     if (plan->has_pending) GUFFIN_TRY(ingest(s, plan, b, nullptr, 0));
     std::vector<Draws> draws(horizon);
     for (uint32_t i = 0; i < horizon; ++i) draws[i] = {words[i], 0, 0.5, 0.5, 0.5};
-    if (hipMemcpyAsync(b.draws, draws.data(), horizon * sizeof(Draws), hipMemcpyHostToDevice, s) != hipSuccess)
+    if (hipMemcpyWithStream(b.draws, draws.data(), horizon * sizeof(Draws), hipMemcpyHostToDevice, s) != hipSuccess)
         return poison(plan, GUFFIN_E_HIP, "draft_plan_propose: upload failed");
     std::vector<uint32_t> window(history, history + history_count);
     const bool penalise = opt.repetition_penalty != 1.0f;
@@ -395,7 +398,7 @@ extern "C" int guffin_hip_draft_plan_propose(void* stream, guffin_draft_plan* pl
         if (int rc = ensure_logits(s, plan, b)) { plan->poisoned = 1; return rc; }
         const float* logits = b.logits + uint64_t(plan->last_rows - 1) * m.vocab;
         if (penalise && !window.empty()) {
-            if (hipMemcpyAsync(b.history, window.data(), window.size() * 4, hipMemcpyHostToDevice, s) != hipSuccess)
+            if (hipMemcpyWithStream(b.history, window.data(), window.size() * 4, hipMemcpyHostToDevice, s) != hipSuccess)
                 return poison(plan, GUFFIN_E_HIP, "draft_plan_propose: upload failed");
             if (int rc = guffin_hip_draft_process(s, logits, m.vocab, b.history, static_cast<uint32_t>(window.size()),
                                                   opt.repetition_penalty, b.scores)) { plan->poisoned = 1; return rc; }

@@ -435,9 +435,9 @@ extern "C" int guffin_hip_forward_tree_rows(void* stream, const guffin_model_des
             e[0] = base_first; e[1] = base_position - base_first; e[2] = offsets[r]; e[3] = ancestor_counts[r];
         }
     hipStream_t hs = as_stream(stream);
-    if (hipMemcpyAsync(s.positions, positions, rows * 4, hipMemcpyHostToDevice, hs) != hipSuccess
-        || hipMemcpyAsync(s.ancestors, ancestor_lists, total * 4, hipMemcpyHostToDevice, hs) != hipSuccess
-        || hipMemcpyAsync(s.schedule, schedule.data(), schedule.size() * 4, hipMemcpyHostToDevice, hs) != hipSuccess)
+    if (hipMemcpyWithStream(s.positions, positions, rows * 4, hipMemcpyHostToDevice, hs) != hipSuccess
+        || hipMemcpyWithStream(s.ancestors, ancestor_lists, total * 4, hipMemcpyHostToDevice, hs) != hipSuccess
+        || hipMemcpyWithStream(s.schedule, schedule.data(), schedule.size() * 4, hipMemcpyHostToDevice, hs) != hipSuccess)
         return fail(GUFFIN_E_HIP, "forward_tree_rows: upload failed");
     const uint32_t H = m.hidden, QW = m.q_heads * m.head_dim, KW = m.kv_heads * m.head_dim;
     const float attn_scale = 1.0f / std::sqrt(static_cast<float>(m.head_dim));

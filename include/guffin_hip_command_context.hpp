@@ -210,11 +210,11 @@ public:
     [[nodiscard]] hipStream_t stream() const noexcept { return stream_; }
 
     void write_u32(const BackendBuffer& destination, std::uint32_t value) { write_u32s(destination, 0, {&value, 1}); }
-    // Pageable source memory is staged by the runtime before hipMemcpyAsync returns, so `values` may die.
+    // hipMemcpyWithStream: ordered on the stream, and back only when the source has been read (`values` may die).
     void write_u32s(const BackendBuffer& destination, std::uint32_t element_offset, std::span<const std::uint32_t> values) {
         require_encodable();
         require_capacity(destination, (std::uint64_t(element_offset) + values.size()) * 4, "write_u32s destination");
-        check_hip(hipMemcpyAsync(u32(destination) + element_offset, values.data(), values.size_bytes(),
+        check_hip(hipMemcpyWithStream(u32(destination) + element_offset, values.data(), values.size_bytes(),
                                  hipMemcpyHostToDevice, stream_), "write_u32s failed");
     }
 
@@ -681,7 +681,7 @@ private:
         capacity = std::min(capacity, vocab);
         require_capacity(workspace.candidate_runs_a, guffin_hip_select_workspace_bytes(rows, vocab, capacity), "candidate selection workspace");
         require_capacity(workspace.compact_result, std::uint64_t(rows) * kResultStride, "candidate results");
-        check_hip(hipMemcpyAsync(meta_ + kMetaResolved, resolved.data(), rows * sizeof(guffin_resolved_row), hipMemcpyHostToDevice,
+        check_hip(hipMemcpyWithStream(meta_ + kMetaResolved, resolved.data(), rows * sizeof(guffin_resolved_row), hipMemcpyHostToDevice,
                                  stream_), "request upload failed");
         check(guffin_hip_select_candidates_resolved(stream_, f32(logits), rows, vocab, capacity, meta_ + kMetaResolved,
                                                     dev(workspace.candidate_runs_a), dev(workspace.compact_result), row_status(rows)));

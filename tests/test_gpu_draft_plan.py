@@ -273,3 +273,24 @@ def test_a_pass_that_gives_up_a_wait_is_run_again_per_operator(hip, scaled_world
         hip.set_spin_limit(1 << 20)
         hip.set_forward_mode(0)                  # an explicit choice enables the resident form again
     assert hip.lib().guffin_hip_resident_enabled() == 1
+
+
+def test_truncate_and_abort_outside_a_transaction(hip, scaled_world):
+    """gemma3_draft.mm:1283-1312: truncating to the current position is always admitted and changes nothing; an
+    abort with no transaction open poisons the plan."""
+    from guffin_amd import model
+    shape, host, device = scaled_world
+    plan = model.DraftPlan(device)
+    plan.append(stream(5))
+    before = snapshot(plan, shape)
+    assert plan.can_truncate(5) and not plan.can_truncate(4) and not plan.can_truncate(6)
+    plan.truncate(5)
+    assert plan.position == 5 and same_caches(snapshot(plan, shape), before)
+    refuses(hip, lambda: plan.truncate(4), -6)
+    assert not plan.poisoned
+    refuses(hip, plan.abort_transaction, -6)
+    assert plan.poisoned
+    refuses(hip, lambda: plan.append([ROOT]), -6)
+    plan.reset()
+    plan.append([ROOT])
+    assert plan.position == 1 and not plan.poisoned
