@@ -202,21 +202,23 @@ __global__ void __launch_bounds__(64 * attention_waves(ROWS * GROUP)) attn_parti
     const uint32_t slot = lane >> 4, seg = lane & 15;  // token slot in the wave, segment of the head dimension
     const uint32_t tb_first = t0 + wv * 4 + slot;
     uint4 k0[U], k1[U];
+    // one round's key row of this lane group: token tb + 4 kAW u, into slot u
+    auto load_key_round = [&](int u, uint32_t tb) {
+        const uint32_t t = tb + 4 * kAW * u;
+        k0[u] = make_uint4(0, 0, 0, 0); k1[u] = k0[u];
+        if (t < t1) {
+            const bool is_priv = t >= n_ring;
+            if (FUSED && is_priv) return;  // taken from LDS once prepared
+            const uint16_t* kp = is_priv ? a.priv_k + size_t(t - n_ring) * row_stride
+                                         : a.ring_k + size_t((u_first + t) & a.ring_mask) * row_stride;
+            kp += kvh * HD + seg * 8;
+            // (4-byte aligned requests: a caller's K/V view may start at any word of its parent allocation)
+            k0[u] = ld16_a4(reinterpret_cast<const uint8_t*>(kp)); k1[u] = ld16_a4(reinterpret_cast<const uint8_t*>(kp + HD / 2));
+        }
+    };
     auto load_keys = [&](uint32_t tb) {
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const uint32_t t = tb + 4 * kAW * u;
-            k0[u] = make_uint4(0, 0, 0, 0); k1[u] = k0[u];
-            if (t < t1) {
-                const bool is_priv = t >= n_ring;
-                if (FUSED && is_priv) continue;  // taken from LDS once prepared
-                const uint16_t* kp = is_priv ? a.priv_k + size_t(t - n_ring) * row_stride
-                                             : a.ring_k + size_t((u_first + t) & a.ring_mask) * row_stride;
-                kp += kvh * HD + seg * 8;
-                // (4-byte aligned requests: a caller's K/V view may start at any word of its parent allocation)
-                k0[u] = ld16_a4(reinterpret_cast<const uint8_t*>(kp)); k1[u] = ld16_a4(reinterpret_cast<const uint8_t*>(kp + HD / 2));
-            }
-        }
+        for (int u = 0; u < U; ++u) load_key_round(u, tb);
     };
     if constexpr (FUSED) load_keys(tb_first);
     // ---- values: a half wave covers one value row (32 lanes x 8 dims, 16-byte loads), a wave two
@@ -224,20 +226,22 @@ __global__ void __launch_bounds__(64 * attention_waves(ROWS * GROUP)) attn_parti
     // the softmax runs
     const uint32_t hsel = lane >> 5, dl = (lane & 31) * 8;
     const uint32_t vb_first = t0 + wv * 2 + hsel;
-    uint4 vv[U];
+    constexpr int UV = 8;   // value rounds in flight: a round is half a key round's bytes (16 per lane)
+    uint4 vv[UV];
+    auto load_value_round = [&](int u, uint32_t tb) {
+        const uint32_t t = tb + 2 * kAW * u;
+        vv[u] = make_uint4(0, 0, 0, 0);
+        if (t < t1) {
+            const bool is_priv = t >= n_ring;
+            if (FUSED && is_priv) return;  // taken from LDS once prepared
+            const uint16_t* vp = is_priv ? a.priv_v + size_t(t - n_ring) * row_stride
+                                         : a.ring_v + size_t((u_first + t) & a.ring_mask) * row_stride;
+            vv[u] = ld16_a4(reinterpret_cast<const uint8_t*>(vp + kvh * HD + dl));
+        }
+    };
     auto load_values = [&](uint32_t tb) {
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const uint32_t t = tb + 2 * kAW * u;
-            vv[u] = make_uint4(0, 0, 0, 0);
-            if (t < t1) {
-                const bool is_priv = t >= n_ring;
-                if (FUSED && is_priv) continue;  // taken from LDS once prepared
-                const uint16_t* vp = is_priv ? a.priv_v + size_t(t - n_ring) * row_stride
-                                             : a.ring_v + size_t((u_first + t) & a.ring_mask) * row_stride;
-                vv[u] = ld16_a4(reinterpret_cast<const uint8_t*>(vp + kvh * HD + dl));
-            }
-        }
+        for (int u = 0; u < UV; ++u) load_value_round(u, tb);
     };
 
     if constexpr (FUSED) {
@@ -287,8 +291,10 @@ __global__ void __launch_bounds__(64 * attention_waves(ROWS * GROUP)) attn_parti
 #pragma unroll
             for (int i = 0; i < 8; ++i) { qv[n][i] = qp[i] * a.scale; qv[n][8 + i] = qp[HD / 2 + i] * a.scale; }
         }
+        // U rounds stay in flight for the whole walk: a slot is asked for its next row (U rounds on) as soon as its
+        // row has been read, so a long partition streams instead of filling and draining once per batch
+        if constexpr (!FUSED) load_keys(tb_first);
         for (uint32_t tb = tb_first; tb < t0 + a.span; tb += 4 * kAW * U) {
-            if (!FUSED || tb != tb_first) load_keys(tb);
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 const uint32_t t = tb + 4 * kAW * u;
@@ -300,6 +306,7 @@ __global__ void __launch_bounds__(64 * attention_waves(ROWS * GROUP)) attn_parti
                     k0[u] = *reinterpret_cast<const uint4*>(kp); k1[u] = *reinterpret_cast<const uint4*>(kp + HD / 2);
                 }
                 const uint32_t kw[8] = {k0[u].x, k0[u].y, k0[u].z, k0[u].w, k1[u].x, k1[u].y, k1[u].z, k1[u].w};
+                if (tb + 4 * kAW * U < t0 + a.span) load_key_round(u, tb + 4 * kAW * U);
                 float s[NQ];
 #pragma unroll
                 for (int n = 0; n < NQ; ++n) {
@@ -346,14 +353,15 @@ __global__ void __launch_bounds__(64 * attention_waves(ROWS * GROUP)) attn_parti
         for (int n = 0; n < NQ; ++n)
 #pragma unroll
             for (int i = 0; i < 8; ++i) acc[n][i] = 0.f;
-        for (uint32_t tb = vb_first; tb < t1; tb += 2 * kAW * U) {
-            if (!FUSED || tb != vb_first) load_values(tb);
+        if constexpr (!FUSED) load_values(vb_first);
+        for (uint32_t tb = vb_first; tb < t1; tb += 2 * kAW * UV) {
 #pragma unroll
-            for (int u = 0; u < U; ++u) {
+            for (int u = 0; u < UV; ++u) {
                 const uint32_t t = tb + 2 * kAW * u;
                 if (t >= t1) break;
                 if (FUSED && t >= n_ring) vv[u] = *reinterpret_cast<const uint4*>(&v_s[t - n_ring][dl]);
                 const uint32_t w4[4] = {vv[u].x, vv[u].y, vv[u].z, vv[u].w};
+                if (tb + 2 * kAW * UV < t1) load_value_round(u, tb + 2 * kAW * UV);
 #pragma unroll
                 for (int n = 0; n < NQ; ++n) {
                     const float p = sc[n * a.span + (t - t0)];
