@@ -20,6 +20,9 @@ Extra objects on the JSON line:
                 the drafter's decode with head and argmax; the Q6_K head with selection and
                 acceptance): microseconds per unit as HIP graphs, algorithmic bytes, GB/s and the
                 fraction of the 8 TB/s HBM peak.
+  chain         the same step recorded once and replayed as dispatch packets on the library's own queue
+                (guffin_hip_chain_*): wall microseconds per replay with its wait, and the device's clock
+                between the first packet's start and the last packet's end.
   prefill       config 4's second half: a 2048-token prompt through the same stack.
   cpu_baseline  the reference's own CPU row dot (oracle/_ref) or the oracle port timed on the
                 host cores: configs 0 and 1 in full, config 3 on a vocabulary slice plus the oracle's
@@ -397,6 +400,29 @@ def main():
     if (replayed["accepted"], replayed["token"], replayed["next_root"]) != (first["accepted"], first["token"], first["next_root"]):
         raise RuntimeError("graph replay changed the step's decision")
 
+    # the same step once more as a recorded chain (the library's own command buffer: AQL packets on its own queue);
+    # wall time per replay and the device's own clock between the first and the last packet
+    chain = hip.Chain()
+    with chain:
+        plan.step(0)
+    for _ in range(2):
+        chain.launch()
+        chain.wait()
+    chain_steps = min(args.steps, 20)
+    t0 = time.perf_counter()
+    device_ns = 0
+    for _ in range(chain_steps):
+        chain.launch()
+        chain.wait()
+        device_ns += chain.gpu_ns()
+    chain_us = (time.perf_counter() - t0) * 1e6 / chain_steps
+    chained = plan.read_result()
+    if (chained["accepted"], chained["token"], chained["next_root"]) != (first["accepted"], first["token"], first["next_root"]):
+        raise RuntimeError("chain replay changed the step's decision")
+    chain_figure = {"launches": chain.launches(), "replays": chain_steps, "us_per_replay_wall": round(chain_us, 1),
+                    "us_per_replay_device": round(device_ns / chain_steps / 1e3, 1)}
+    chain.close()
+
     # ---- rooflines: the dominant kernel (fused 2-row Q4_K gate+up GEMV + GeGLU, one launch per block), then the
     # local layers' attention and the down projection -----
     import ctypes as C
@@ -527,6 +553,7 @@ def main():
         },
         "roofline": roofline,
         "rooflines": [attention_line, down_line, qkv_line, o_line],
+        "chain": chain_figure,
     }
     line["configs"] = config_figures(target, drafter, T, D, d_pos)
     if not args.no_prefill:
