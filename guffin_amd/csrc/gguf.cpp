@@ -364,8 +364,40 @@ extern "C" int guffin_gguf_bind_gemma3(const guffin_gguf* g, const guffin_gemma3
                                        guffin_gemma3_block* blocks) {
     if (!g || !c || !out || !blocks) return GUFFIN_E_ARG;
     g_bind_detail.clear();
+    const auto find = [&](const std::string& name, uint64_t* index) {
+        for (size_t i = 0; i < g->tensors.size(); ++i)
+            if (g->tensors[i].name == name) { *index = i; return true; }
+        return false;
+    };
+    // bind_gemma_model_weights (:72-103): every tensor is looked up before anything is validated, the blocks first
+    // and inside a block in the order of the reference's initialisers (:38-68), so the first name that is absent in
+    // that order is the refusal whatever else is wrong with the file or the configuration.
+    enum { kAttnNorm = 0, kQNorm = 1, kKNorm = 2, kPostAttnNorm = 3, kFfnNorm = 4, kPostFfwNorm = 5 };
+    for (uint32_t b = 0; b < c->block_count; ++b) {
+        guffin_gemma3_block& blk = blocks[b];
+        const auto need_norm = [&](int i) { return find(block_name(b, kNormNames[i]), &blk.norm[i]) ? 0 : refuse(GUFFIN_BIND_MISSING_TENSOR, block_name(b, kNormNames[i])); };
+        const auto need_matrix = [&](int i) { return find(block_name(b, kMatrixNames[i]), &blk.matrix[i]) ? 0 : refuse(GUFFIN_BIND_MISSING_TENSOR, block_name(b, kMatrixNames[i])); };
+        if (int rc = need_norm(kAttnNorm)) return rc;
+        if (int rc = need_norm(kPostAttnNorm)) return rc;
+        for (int i = 0; i < 4; ++i)
+            if (int rc = need_matrix(i)) return rc;
+        if (c->uses_qk_norm) {
+            if (int rc = need_norm(kQNorm)) return rc;
+            if (int rc = need_norm(kKNorm)) return rc;
+        }
+        if (int rc = need_norm(kFfnNorm)) return rc;
+        if (int rc = need_norm(kPostFfwNorm)) return rc;
+        for (int i = 4; i < 7; ++i)
+            if (int rc = need_matrix(i)) return rc;
+    }
+    if (!find("token_embd.weight", &out->token_embedding)) return refuse(GUFFIN_BIND_MISSING_TENSOR, "token_embd.weight");
+    if (!find("output_norm.weight", &out->output_norm)) return refuse(GUFFIN_BIND_MISSING_TENSOR, "output_norm.weight");
+    // output_weight_or_tied_embedding (:26-34): output.weight when the file has one, else the embedding
+    out->tied_output = find("output.weight", &out->output) ? 0u : 1u;
+    if (out->tied_output) out->output = out->token_embedding;
+
+    // validate_gemma3_model_weights (:105-177), in its order.  The execution configuration (:106-119):
     const auto finite_positive = [](float v) { return std::isfinite(v) && v > 0.0f; };
-    // the execution configuration (:106-119)
     if (!c->uses_qk_norm || c->attention_global_layer_period != 6 || c->embedding_length == 0 || c->feed_forward_length == 0
         || c->block_count == 0 || c->vocab_size == 0 || c->attention_head_count == 0 || c->attention_head_count_kv == 0
         || c->attention_head_count % c->attention_head_count_kv != 0 || c->attention_key_length == 0
@@ -382,60 +414,54 @@ extern "C" int guffin_gguf_bind_gemma3(const guffin_gguf* g, const guffin_gemma3
         return refuse(GUFFIN_BIND_INVALID_TENSOR, "Gemma 3 runtime context must cover the local attention window");
     const uint64_t query_width = uint64_t(c->attention_head_count) * c->attention_key_length;
     const uint64_t kv_width = uint64_t(c->attention_head_count_kv) * c->attention_key_length;
-    if (query_width > 0xFFFFFFFFull || kv_width > 0xFFFFFFFFull)
-        return refuse(GUFFIN_BIND_INVALID_TENSOR, "Gemma 3 attention width exceeds 32-bit indexing range");
+    if (query_width > 0xFFFFFFFFull || kv_width > 0xFFFFFFFFull)   // the reference's wording, whatever the device
+        return refuse(GUFFIN_BIND_INVALID_TENSOR, "Gemma 3 attention width exceeds Metal indexing range");
 
-    int rc = GUFFIN_OK;
-    const auto find = [&](const std::string& name, uint64_t* index, bool required) {
-        for (size_t i = 0; i < g->tensors.size(); ++i)
-            if (g->tensors[i].name == name) { *index = i; return true; }
-        if (required && rc == GUFFIN_OK) rc = refuse(GUFFIN_BIND_MISSING_TENSOR, name);
-        return false;
-    };
-    const auto norm = [&](const std::string& name, uint64_t width, uint64_t* index) {
-        if (rc != GUFFIN_OK || !find(name, index, true)) return;
-        const Tensor& t = g->tensors[static_cast<size_t>(*index)];
+    const auto norm = [&](uint64_t index, uint64_t width, const std::string& name) {
+        const Tensor& t = g->tensors[static_cast<size_t>(index)];
         if (t.n_dims != 1 || t.dims[0] != width || t.type_id != kTypeF32)
-            rc = refuse(GUFFIN_BIND_INVALID_TENSOR, name + ": expected F32 norm with width " + std::to_string(width));
+            return refuse(GUFFIN_BIND_INVALID_TENSOR, name + ": expected F32 norm with width " + std::to_string(width));
+        return 0;
     };
-    const auto matrix = [&](const std::string& name, uint64_t input, uint64_t output, uint64_t* index, bool head) {
-        if (rc != GUFFIN_OK || !find(name, index, true)) return;
-        const Tensor& t = g->tensors[static_cast<size_t>(*index)];
+    const auto matrix = [&](uint64_t index, uint64_t input, uint64_t output, const std::string& name, bool head) {
+        const Tensor& t = g->tensors[static_cast<size_t>(index)];
         const bool kquant = head && c->target_geometry ? t.type_id == kTypeQ6K : (t.type_id == kTypeQ4K || t.type_id == kTypeQ6K);
         const bool q8 = !c->target_geometry && t.type_id == kTypeQ8;
         if (t.n_dims != 2 || t.dims[0] != input || t.dims[1] != output || !(kquant || q8) || input % (q8 ? 32 : 256) != 0)
-            rc = refuse(GUFFIN_BIND_INVALID_TENSOR, name + ": expected native " + (c->target_geometry ? (head ? "Q6_K" : "Q4_K/Q6_K") : "Q8_0/Q4_K/Q6_K")
-                            + " GGUF matrix [" + std::to_string(input) + ", " + std::to_string(output) + "]");
+            return refuse(GUFFIN_BIND_INVALID_TENSOR, name + ": expected native " + (c->target_geometry ? (head ? "Q6_K" : "Q4_K/Q6_K") : "Q8_0/Q4_K/Q6_K")
+                              + " GGUF matrix [" + std::to_string(input) + ", " + std::to_string(output) + "]");
+        return 0;
     };
-    matrix("token_embd.weight", c->embedding_length, c->vocab_size, &out->token_embedding, true);
-    // output_weight_or_tied_embedding (:26-34): output.weight when the file has one, else the embedding
-    out->tied_output = 1;
-    out->output = out->token_embedding;
-    uint64_t own = 0;
-    if (rc == GUFFIN_OK && find("output.weight", &own, false)) {
-        matrix("output.weight", c->embedding_length, c->vocab_size, &out->output, true);
-        out->tied_output = 0;
-    }
-    if (rc == GUFFIN_OK && c->uses_tied_output_weight && !out->tied_output)
-        rc = refuse(GUFFIN_BIND_INVALID_TENSOR, "Gemma 3 tied output must alias token_embd.weight");
-    norm("output_norm.weight", c->embedding_length, &out->output_norm);
+    if (int rc = matrix(out->token_embedding, c->embedding_length, c->vocab_size, "token_embd.weight", true)) return rc;
+    if (int rc = matrix(out->output, c->embedding_length, c->vocab_size, "output.weight", true)) return rc;
+    if (c->uses_tied_output_weight && !out->tied_output)
+        return refuse(GUFFIN_BIND_INVALID_TENSOR, "Gemma 3 tied output must alias token_embd.weight");
+    if (int rc = norm(out->output_norm, c->embedding_length, "output_norm.weight")) return rc;
     const uint64_t in_out[7][2] = {{c->embedding_length, query_width}, {c->embedding_length, kv_width}, {c->embedding_length, kv_width},
                                    {query_width, c->embedding_length}, {c->embedding_length, c->feed_forward_length},
                                    {c->embedding_length, c->feed_forward_length}, {c->feed_forward_length, c->embedding_length}};
-    const uint64_t widths[6] = {c->embedding_length, c->attention_key_length, c->attention_key_length, c->embedding_length,
-                                c->embedding_length, c->embedding_length};
-    for (uint32_t b = 0; rc == GUFFIN_OK && b < c->block_count; ++b) {
-        for (int i = 0; i < 6; ++i) norm(block_name(b, kNormNames[i]), widths[i], &blocks[b].norm[i]);
+    for (uint32_t b = 0; b < c->block_count; ++b) {
+        guffin_gemma3_block& blk = blocks[b];
+        const auto check_norm = [&](int i, uint64_t width) { return norm(blk.norm[i], width, block_name(b, kNormNames[i])); };
+        const auto check_matrix = [&](int i) { return matrix(blk.matrix[i], in_out[i][0], in_out[i][1], block_name(b, kMatrixNames[i]), false); };
+        if (int rc = check_norm(kAttnNorm, c->embedding_length)) return rc;
+        if (int rc = check_norm(kPostAttnNorm, c->embedding_length)) return rc;
+        if (int rc = check_norm(kQNorm, c->attention_key_length)) return rc;
+        if (int rc = check_norm(kKNorm, c->attention_key_length)) return rc;
+        for (int i = 0; i < 4; ++i)
+            if (int rc = check_matrix(i)) return rc;
+        if (int rc = check_norm(kFfnNorm, c->embedding_length)) return rc;
+        if (int rc = check_norm(kPostFfwNorm, c->embedding_length)) return rc;
+        for (int i = 4; i < 7; ++i)
+            if (int rc = check_matrix(i)) return rc;
         bool any_q8 = false, any_kquant = false;
         for (int i = 0; i < 7; ++i) {
-            matrix(block_name(b, kMatrixNames[i]), in_out[i][0], in_out[i][1], &blocks[b].matrix[i], false);
-            if (rc != GUFFIN_OK) break;
-            blocks[b].type_id[i] = g->tensors[static_cast<size_t>(blocks[b].matrix[i])].type_id;
-            (blocks[b].type_id[i] == kTypeQ8 ? any_q8 : any_kquant) = true;
+            blk.type_id[i] = g->tensors[static_cast<size_t>(blk.matrix[i])].type_id;
+            (blk.type_id[i] == kTypeQ8 ? any_q8 : any_kquant) = true;
         }
         // the kernels of one block share an activation image: 32-weight and 256-weight formats do not mix in it
-        if (rc == GUFFIN_OK && any_q8 && any_kquant)
-            rc = refuse(GUFFIN_BIND_INVALID_TENSOR, block_name(b, "attn_q") + ": a block mixes 32-weight and 256-weight formats");
+        if (any_q8 && any_kquant)
+            return refuse(GUFFIN_BIND_INVALID_TENSOR, block_name(b, "attn_q") + ": a block mixes 32-weight and 256-weight formats");
     }
-    return rc;
+    return GUFFIN_OK;
 }

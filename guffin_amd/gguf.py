@@ -138,6 +138,10 @@ class Reader:
         return {"name": name, "dims": [int(t.dims[d]) for d in range(t.n_dims)], "type_id": t.type_id,
                 "offset": t.offset, "file_offset": t.file_offset, "byte_count": t.byte_count}
 
+    def has_tensor(self, name):
+        index = C.c_uint64()
+        return hip.lib().guffin_gguf_find_tensor(self._h, name.encode(), C.byref(index)) == 0
+
     def bind_gemma3(self, config):
         """guffin_gguf_bind_gemma3: (binding, blocks) of tensor indices, or BindError."""
         lib = hip.lib()

@@ -214,11 +214,17 @@ class DeviceModel:
     GGUF_TYPES = {8: Q8_0, 12: Q4_K, 14: Q6_K}
 
     @classmethod
-    def from_gguf(cls, reader, ring_local=None, ring_global=8192, arch="gemma3"):
+    def from_gguf(cls, reader, ring_local=None, ring_global=8192, arch="gemma3", role="target"):
         """Binds a parsed GGUF file (guffin_amd.gguf.Reader): shape from the `<arch>.*` metadata keys
         (src/engine/model.cpp:330-390), matrices uploaded as they lie in the file ([input, output] with
         the input dimension contiguous, i.e. blocks per output column) and repacked on the device, tied
-        head when there is no output.weight.  Rings start empty."""
+        head when there is no output.weight (model.cpp:328).  Rings start empty.
+
+        `role` is the caller's statement of what the file is: "target" binds under the reference's target rules
+        (256-wide paired GQA heads, K-quant matrices, Q6_K head: gemma_model.cpp:120-124, 137-147), "drafter"
+        without the geometry rule and with Q8_0 matrices allowed.  A file that does not fit its role is refused."""
+        if role not in ("target", "drafter"):
+            raise ValueError("from_gguf: role is 'target' or 'drafter'")
         from . import gguf as gguf_module
         md = reader.metadata()
         key = lambda k: md[arch + "." + k]
@@ -238,8 +244,9 @@ class DeviceModel:
         cfg.attention_key_length, cfg.attention_value_length = int(key("attention.key_length")), int(key("attention.value_length"))
         cfg.sliding_window, cfg.context_length = window, int(md.get(arch + ".context_length", ring_global))
         cfg.attention_global_layer_period = int(md.get(arch + ".attention.sliding_window_pattern", 6))
-        cfg.uses_qk_norm, cfg.uses_tied_output_weight = 1, 0
-        cfg.target_geometry = 1 if cfg.attention_head_count == 2 * cfg.attention_head_count_kv and embed_info["type_id"] != 8 else 0
+        cfg.uses_qk_norm = 1
+        cfg.uses_tied_output_weight = 0 if reader.has_tensor("output.weight") else 1
+        cfg.target_geometry = 1 if role == "target" else 0
         cfg.rms_norm_epsilon = float(key("attention.layer_norm_rms_epsilon"))
         cfg.attention_logit_softcap = float(md.get(arch + ".attn_logit_softcapping", 0.0))
         cfg.final_logit_softcap = float(md.get(arch + ".final_logit_softcapping", 0.0))

@@ -672,8 +672,12 @@ int guffin_gguf_find_tensor(const guffin_gguf* gguf, const char* name, uint64_t*
  * (src/engine/gemma_model.cpp:72-177).  Every tensor the block graph needs is looked up by its GGUF name
  * (token_embd, output_norm, output or the tied embedding, per block the 7 matrices and 6 norms) and checked
  * against the configuration: norms F32 of the right width, matrices native block formats of shape
- * [input, output] with input a whole number of blocks.  target_geometry != 0 adds the target's rules (:120-124,
- * :150-158): 256-wide heads, two query heads per KV head, at most 64 blocks, Q4_K / Q6_K matrices, a Q6_K head;
+ * [input, output] with input a whole number of blocks.  As in the reference every name is looked up before
+ * anything is validated (blocks first, in the order of its initialisers), so a missing tensor is reported
+ * whatever else is wrong; validation then follows the reference's order (configuration, token_embd, output,
+ * output_norm, blocks).  uses_tied_output_weight is what the reference's loader sets when the file has no
+ * output.weight (src/engine/model.cpp:328).  target_geometry is the caller's statement of what the file is:
+ * != 0 adds the target's rules (:120-124, :150-158): 256-wide heads, two query heads per KV head, at most 64 blocks, Q4_K / Q6_K matrices, a Q6_K head;
  * without it the drafter's geometry and Q8_0 blocks are admitted (one block length per block).  Returns 0 and the
  * tensor indices (for guffin_gguf_tensor), GUFFIN_BIND_MISSING_TENSOR (EngineModelErrorCode::missing_tensor) or
  * GUFFIN_BIND_INVALID_TENSOR (::invalid_tensor) with the reference's detail string from guffin_gguf_bind_detail

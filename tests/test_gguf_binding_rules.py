@@ -76,7 +76,11 @@ def test_the_references_refusals(world):
                 dict(uses_qk_norm=0), dict(rms_norm_epsilon=0.0), dict(local_rope_freq_base=-1.0),
                 dict(rope_freq_scale=float("nan")), dict(attention_value_length=128), dict(block_count=0)):
         refused(gguf, image, good(**bad), "invalid_tensor", "Gemma 3 execution configuration")
-    refused(gguf, image, good(block_count=65), "invalid_tensor", "at most 64 layers")
+    # more blocks in the configuration than in the file: the lookup fails first; a file that has them is refused by the rule
+    refused(gguf, image, good(block_count=65), "missing_tensor", "blk.2.attn_norm.weight")
+    deep = replace(shape, layers=65)
+    refused(gguf, write_gguf(model.HostModel(deep, seed=2, position=0)), config_for(gguf, deep, True), "invalid_tensor",
+            "at most 64 layers")
 
 
 def test_tensor_formats_and_widths(world):
@@ -96,3 +100,56 @@ def test_tensor_formats_and_widths(world):
     wide = replace(d_shape, hidden=512, ffn=1024, layer_dtypes=((0,) * 7, (1, 0, 0, 0, 0, 0, 0)))   # block 1: a Q4_K attn_q among Q8_0
     refused(gguf, write_gguf(model.HostModel(wide, seed=3, position=0)), config_for(gguf, wide, target=False), "invalid_tensor",
             "mixes 32-weight and 256-weight formats")
+
+
+def test_which_refusal_wins_when_two_things_are_wrong(world):
+    """bind_gemma_model_weights looks every tensor up before validate_gemma3_model_weights sees anything
+    (src/engine/gemma_model.cpp:72-103): a missing tensor wins over any invalid one and over the configuration,
+    blocks are looked up before token_embd / output_norm and inside a block in the order of the reference's
+    initialisers (:38-68: attn_norm, post_attention_norm, q, k, v, o, q_norm, k_norm, ffn_norm, post_ffw_norm,
+    gate, up, down).  Validation then runs token_embd, output, output_norm, and per block attn_norm,
+    post_attention_norm, q_norm, k_norm, q, k, v, o, ffn_norm, post_ffw_norm, gate, up, down (:149-175)."""
+    gguf, model, shape, host = world
+    good = lambda **kw: config_for(gguf, shape, True, **kw)
+    # missing beats invalid, wherever each sits
+    refused(gguf, write_gguf(host, drop=("blk.1.ffn_down.weight",), retype={"token_embd.weight": 12}), good(),
+            "missing_tensor", "blk.1.ffn_down.weight")
+    refused(gguf, write_gguf(host, drop=("output_norm.weight",), reshape={"blk.0.attn_q_norm.weight": [128]}), good(),
+            "missing_tensor", "output_norm.weight")
+    # missing beats a configuration that would be refused
+    refused(gguf, write_gguf(host, drop=("blk.0.attn_v.weight",)), good(attention_logit_softcap=50.0),
+            "missing_tensor", "blk.0.attn_v.weight")
+    refused(gguf, write_gguf(host, drop=("token_embd.weight",)), good(context_length=4), "missing_tensor", "token_embd.weight")
+    # two missing tensors: blocks before the model's own tensors, block 0 before block 1, initialiser order inside a block
+    refused(gguf, write_gguf(host, drop=("token_embd.weight", "blk.1.ffn_up.weight")), good(), "missing_tensor", "blk.1.ffn_up.weight")
+    refused(gguf, write_gguf(host, drop=("blk.1.attn_norm.weight", "blk.0.ffn_down.weight")), good(), "missing_tensor", "blk.0.ffn_down.weight")
+    refused(gguf, write_gguf(host, drop=("blk.0.attn_q_norm.weight", "blk.0.attn_output.weight")), good(),
+            "missing_tensor", "blk.0.attn_output.weight")
+    refused(gguf, write_gguf(host, drop=("blk.0.attn_q_norm.weight", "blk.0.ffn_norm.weight")), good(),
+            "missing_tensor", "blk.0.attn_q_norm.weight")
+    refused(gguf, write_gguf(host, drop=("blk.0.post_attention_norm.weight", "blk.0.attn_q.weight")), good(),
+            "missing_tensor", "blk.0.post_attention_norm.weight")
+    # without Q/K norms in the configuration their names are not looked up: the configuration is what is refused
+    refused(gguf, write_gguf(host, drop=("blk.0.attn_q_norm.weight",)), good(uses_qk_norm=0), "invalid_tensor",
+            "Gemma 3 execution configuration")
+    # the configuration beats any invalid tensor; among invalid tensors the validation order decides
+    refused(gguf, write_gguf(host, retype={"token_embd.weight": 12}), good(rms_norm_epsilon=0.0), "invalid_tensor",
+            "Gemma 3 execution configuration")
+    refused(gguf, write_gguf(host, retype={"token_embd.weight": 12, "blk.0.attn_norm.weight": 1}), good(), "invalid_tensor",
+            "token_embd.weight: expected native Q6_K")
+    k_shape = list(shape.proj_shapes()[1])
+    refused(gguf, write_gguf(host, reshape={"blk.0.attn_q.weight": k_shape, "blk.0.attn_k_norm.weight": [128]}), good(),
+            "invalid_tensor", "blk.0.attn_k_norm.weight: expected F32 norm")
+    refused(gguf, write_gguf(host, reshape={"blk.0.attn_q.weight": k_shape}, retype={"blk.0.ffn_norm.weight": 1}), good(),
+            "invalid_tensor", "blk.0.attn_q.weight: expected native")
+    refused(gguf, write_gguf(host, retype={"blk.0.post_ffw_norm.weight": 1, "blk.1.attn_norm.weight": 1}), good(),
+            "invalid_tensor", "blk.0.post_ffw_norm.weight")
+    refused(gguf, write_gguf(host, retype={"output_norm.weight": 1, "blk.0.attn_norm.weight": 1}), good(), "invalid_tensor",
+            "output_norm.weight: expected F32 norm")
+
+
+def test_the_width_refusal_keeps_the_references_wording(world):
+    gguf, model, shape, host = world
+    wide = config_for(gguf, shape, False, attention_head_count=1 << 25, attention_head_count_kv=1 << 25,
+                      attention_key_length=256, attention_value_length=256)
+    refused(gguf, write_gguf(host), wide, "invalid_tensor", "Gemma 3 attention width exceeds Metal indexing range")

@@ -24,7 +24,7 @@ def test_model_bound_from_a_gguf_image_runs_like_the_direct_binding(kind):
     reader = gguf.Reader(image)
     assert reader.info.alignment == 64 and reader.metadata()["general.architecture"] == "gemma3"
     assert len(reader.tensors()) == 2 + 13 * shape.layers
-    bound = model.DeviceModel.from_gguf(reader, ring_local=shape.ring_local, ring_global=shape.ring_global)
+    bound = model.DeviceModel.from_gguf(reader, ring_local=shape.ring_local, ring_global=shape.ring_global, role=kind)
     direct = model.DeviceModel.from_host(host)
     assert replace(bound.shape, eps=shape.eps) == shape and abs(bound.shape.eps - shape.eps) < 1e-12
     tokens = torch.tensor([17, 1999], dtype=torch.int32, device="cuda")
@@ -73,4 +73,17 @@ def test_binding_refuses_files_that_do_not_fit_the_model():
     host = model.HostModel(shape, seed=6, position=0)
     host.norm[1][0] = host.norm[1][0][:-1].copy()          # a norm of the wrong width
     with pytest.raises(ValueError):
-        model.DeviceModel.from_gguf(gguf.Reader(write_gguf(host)), ring_global=512)
+        model.DeviceModel.from_gguf(gguf.Reader(write_gguf(host)), ring_global=512, role="drafter")
+
+
+def test_a_file_bound_as_target_must_have_the_targets_geometry():
+    """The caller says what the file is; a drafter-shaped file (4 query heads on 1 KV head, Q8_0) given as the
+    target is refused by the geometry rule (src/engine/gemma_model.cpp:120-124), not bound under other rules."""
+    from guffin_amd import gguf, hip, model
+    hip.init(0)
+    shape = replace(model.GEMMA3_270M, layers=2, vocab=512, ring_global=512)
+    image = write_gguf(model.HostModel(shape, seed=6, position=0))
+    with pytest.raises(gguf.BindError) as refusal:
+        model.DeviceModel.from_gguf(gguf.Reader(image), ring_global=512, role="target")
+    assert "Gemma 3 target requires 256-wide paired GQA heads" in str(refusal.value)
+    model.DeviceModel.from_gguf(gguf.Reader(image), ring_global=512, role="drafter")
