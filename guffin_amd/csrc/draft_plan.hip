@@ -11,9 +11,12 @@
 // The reference keeps a transaction's rows in a private arena that attention reads beside the ring.  Here a
 // transaction's rows go to the rings at once, where the ring attention of guffin_hip_forward_rows sees them,
 // and the ring rows they overwrite (a local layer's slot (position & mask) held position - window) are first
-// saved per position in a backup arena of kTransactionRows rows per layer; abort, truncate and a commit of a
-// shorter prefix copy them back.  Same observable behaviour: an aborted or truncated suffix leaves every ring
-// row as it was, and logits after a commit equal those of a plain replay of the kept tokens.
+// saved per position in a backup arena per layer (the plan's transaction capacity, a constructor argument as in
+// the reference, rounded up to a power of two); abort, truncate and a commit of a shorter prefix copy them back.
+// The final normalised row of every position a transaction runs is kept as well (the reference's private_norm,
+// gemma3_draft.mm:966-968, 984-992), so that logits can be projected at a frontier a truncate or a shorter commit
+// went back to.  Same observable behaviour: an aborted or truncated suffix leaves every ring row as it was, and
+// logits after a commit equal those of a plain replay of the kept tokens.
 //
 // Every call is host-synchronous (it returns when its device work is done); the path that is timed is
 // guffin_hip_h1_step, which needs none of this.
@@ -28,7 +31,7 @@
 namespace guffin {
 namespace {
 
-constexpr uint32_t kTransactionRows = 32;   // positions a transaction may write (the reference's arena: 96 or 256)
+constexpr uint32_t kDefaultTransactionRows = 32;   // when the caller names none (the reference's callers use 96 or 256)
 constexpr uint32_t kMaxHorizon = 23;        // external_speculation_max_horizon
 constexpr uint64_t kLawBytes = 8 + 256 * 4 + 257 * 8;
 struct Draws { uint32_t word, pad; double u_accept, u_residual, u_next; };
@@ -46,7 +49,7 @@ struct Carve {
 struct Buffers {
     uint8_t* forward; uint64_t forward_bytes;
     uint16_t *priv_k, *priv_v, *backup_k, *backup_v;
-    float *hidden, *hidden_sums, *hidden_saved, *sums_saved, *logits, *parts, *scores;
+    float *hidden, *hidden_sums, *hidden_saved, *sums_saved, *txn_hidden, *logits, *parts, *scores;
     uint32_t *tokens, *drafted, *history, *status, *proposal;
     Draws* draws;
     uint8_t *law_ws, *law;
@@ -54,7 +57,13 @@ struct Buffers {
     void **ring_k_table, **ring_v_table;
 };
 
-Buffers carve(const guffin_model_desc& m, void* workspace, uint64_t* total) {
+uint32_t arena_rows(uint32_t transaction_rows) {
+    uint32_t rows = 1;
+    while (rows < transaction_rows) rows <<= 1;
+    return rows;
+}
+
+Buffers carve(const guffin_model_desc& m, uint32_t arena, void* workspace, uint64_t* total) {
     Carve c {static_cast<uint8_t*>(workspace), 0};
     Buffers b {};
     const uint64_t kvw = uint64_t(m.kv_heads) * m.head_dim;
@@ -62,12 +71,13 @@ Buffers carve(const guffin_model_desc& m, void* workspace, uint64_t* total) {
     b.forward = c.take<uint8_t>(b.forward_bytes);
     b.priv_k = c.take<uint16_t>(uint64_t(m.layer_count) * 2 * kvw);
     b.priv_v = c.take<uint16_t>(uint64_t(m.layer_count) * 2 * kvw);
-    b.backup_k = c.take<uint16_t>(uint64_t(m.layer_count) * kTransactionRows * kvw);
-    b.backup_v = c.take<uint16_t>(uint64_t(m.layer_count) * kTransactionRows * kvw);
+    b.backup_k = c.take<uint16_t>(uint64_t(m.layer_count) * arena * kvw);
+    b.backup_v = c.take<uint16_t>(uint64_t(m.layer_count) * arena * kvw);
     b.hidden = c.take<float>(2 * uint64_t(m.hidden));
     b.hidden_sums = c.take<float>(guffin_hip_receipt_bytes(2, m.hidden) / 4);
     b.hidden_saved = c.take<float>(2 * uint64_t(m.hidden));
     b.sums_saved = c.take<float>(guffin_hip_receipt_bytes(2, m.hidden) / 4);
+    b.txn_hidden = c.take<float>(uint64_t(arena) * m.hidden);
     b.logits = c.take<float>(2 * uint64_t(m.vocab));
     b.parts = c.take<float>(uint64_t(std::max(1u, guffin_hip_gemv_packed_slices(m.head_dtype, m.hidden, m.vocab))) * 2 * m.vocab);
     b.scores = c.take<float>(m.vocab);
@@ -85,6 +95,8 @@ Buffers carve(const guffin_model_desc& m, void* workspace, uint64_t* total) {
     if (total) *total = (c.used + 255) & ~uint64_t{255};
     return b;
 }
+
+Buffers carve(const guffin_draft_plan* p) { return carve(*p->model, p->transaction_arena, p->workspace, nullptr); }
 
 int usable(const guffin_draft_plan* p, const char* what) {
     if (!p || !p->model || !p->workspace) return fail(GUFFIN_E_ARG, what);
@@ -104,12 +116,13 @@ int move_rows(hipStream_t s, const guffin_draft_plan* p, const Buffers& b, uint3
     const uint64_t kvw = uint64_t(m.kv_heads) * m.head_dim;
     for (uint32_t l = 0; l < m.layer_count; ++l) {
         const uint32_t ring_mask = (layer_is_local(m.global_period, l) ? m.ring_local : m.ring_global) - 1;
-        void* bk = b.backup_k + uint64_t(l) * kTransactionRows * kvw;
-        void* bv = b.backup_v + uint64_t(l) * kTransactionRows * kvw;
+        const uint32_t arena = p->transaction_arena;
+        void* bk = b.backup_k + uint64_t(l) * arena * kvw;
+        void* bv = b.backup_v + uint64_t(l) * arena * kvw;
         void* rk = m.layers[l].ring_k;
         void* rv = m.layers[l].ring_v;
-        const int rc = save ? guffin_hip_kv_cache_copy(s, rk, rv, bk, bv, first, end - first, ring_mask, kTransactionRows - 1, kvw)
-                            : guffin_hip_kv_cache_copy(s, bk, bv, rk, rv, first, end - first, kTransactionRows - 1, ring_mask, kvw);
+        const int rc = save ? guffin_hip_kv_cache_copy(s, rk, rv, bk, bv, first, end - first, ring_mask, arena - 1, kvw)
+                            : guffin_hip_kv_cache_copy(s, bk, bv, rk, rv, first, end - first, arena - 1, ring_mask, kvw);
         if (rc) return rc;
     }
     return GUFFIN_OK;
@@ -145,6 +158,10 @@ int forward(hipStream_t s, guffin_draft_plan* p, const Buffers& b, uint32_t rows
         }
     }
     GUFFIN_TRY(guffin_hip_commit_rows(s, &m, b.priv_k, b.priv_v, b.ring_k_table, b.ring_v_table, nullptr, at, rows));
+    if (p->transaction_active   // the rows' final normalised states, by their place in the transaction
+        && hipMemcpyAsync(b.txn_hidden + uint64_t(at - p->checkpoint_materialized) * m.hidden, b.hidden, uint64_t(rows) * m.hidden * 4,
+                          hipMemcpyDeviceToDevice, s) != hipSuccess)
+        return fail(GUFFIN_E_HIP, "draft_plan: keeping the rows' final states failed");
     p->materialized = at + rows;
     p->last_rows = rows;
     p->logits_valid = 0;
@@ -191,8 +208,8 @@ int ensure_logits(hipStream_t s, guffin_draft_plan* p, const Buffers& b) {
 int capacity_check(const guffin_draft_plan* p, uint32_t new_rows, const char* what) {
     const guffin_model_desc& m = *p->model;
     if (uint64_t(p->materialized) + new_rows > m.ring_global) return fail(GUFFIN_E_CAPACITY, what);
-    if (p->transaction_active && uint64_t(p->materialized) + new_rows - p->checkpoint_materialized > kTransactionRows)
-        return fail(GUFFIN_E_CAPACITY, "draft_plan: a transaction writes at most 32 rows");
+    if (p->transaction_active && uint64_t(p->materialized) + new_rows - p->checkpoint_materialized > p->transaction_rows)
+        return fail(GUFFIN_E_CAPACITY, "draft_plan: the transaction would write more rows than the plan was prepared for");
     return GUFFIN_OK;
 }
 
@@ -201,28 +218,36 @@ int capacity_check(const guffin_draft_plan* p, uint32_t new_rows, const char* wh
 
 using namespace guffin;
 
-extern "C" uint64_t guffin_hip_draft_plan_bytes(const guffin_model_desc* model) {
-    if (!model || !model->layers || !model->head_tiles || model->ring_global < 4) return 0;
+// transaction_rows: 0 = 32; otherwise at least the largest horizon + 2 (gemma3_draft.mm:654-655) and no more than a ring holds
+static bool transaction_rows_fit(const guffin_model_desc& m, uint32_t& transaction_rows) {
+    if (transaction_rows == 0) transaction_rows = kDefaultTransactionRows;
+    return transaction_rows >= kMaxHorizon + 2 && arena_rows(transaction_rows) <= m.ring_local && arena_rows(transaction_rows) <= m.ring_global;
+}
+
+extern "C" uint64_t guffin_hip_draft_plan_bytes(const guffin_model_desc* model, uint32_t transaction_rows) {
+    if (!model || !model->layers || !model->head_tiles || model->ring_global < 4 || !transaction_rows_fit(*model, transaction_rows)) return 0;
     uint64_t total = 0;
-    carve(*model, nullptr, &total);
+    carve(*model, arena_rows(transaction_rows), nullptr, &total);
     return total;
 }
 
 extern "C" int guffin_hip_draft_plan_init(void* stream, guffin_draft_plan* plan, const guffin_model_desc* model, void* workspace,
-                                          uint64_t workspace_bytes) {
+                                          uint64_t workspace_bytes, uint32_t transaction_rows) {
     if (!plan || !model || !model->layers || !workspace) return fail(GUFFIN_E_ARG, "draft_plan_init: null pointer");
     if (!model->head_tiles) return fail(GUFFIN_E_ARG, "draft_plan_init: the model needs its head tiles");
     if (model->vocab % 256 != 0) return fail(GUFFIN_E_SHAPE, "draft_plan_init: the law kernels need a vocabulary that is a multiple of 256");
-    if (model->ring_local < kTransactionRows || model->ring_global < kTransactionRows)
-        return fail(GUFFIN_E_SHAPE, "draft_plan_init: rings must hold at least 32 rows");
-    const uint64_t need = guffin_hip_draft_plan_bytes(model);
+    if (!transaction_rows_fit(*model, transaction_rows))
+        return fail(GUFFIN_E_SHAPE, "draft_plan_init: a transaction holds at least 25 rows (the largest horizon + 2) and, rounded up to a power of two, no more than the smallest ring");
+    const uint64_t need = guffin_hip_draft_plan_bytes(model, transaction_rows);
     if (need == 0 || workspace_bytes < need) return fail(GUFFIN_E_CAPACITY, "draft_plan_init: workspace below guffin_hip_draft_plan_bytes");
     if (reinterpret_cast<uintptr_t>(workspace) & 255u) return fail(GUFFIN_E_ALIGN, "draft_plan_init: workspace must be 256-byte aligned");
     std::memset(plan, 0, sizeof(*plan));
     plan->model = model;
     plan->workspace = workspace;
     plan->workspace_bytes = workspace_bytes;
-    const Buffers b = carve(*model, workspace, nullptr);
+    plan->transaction_rows = transaction_rows;
+    plan->transaction_arena = arena_rows(transaction_rows);
+    const Buffers b = carve(plan);
     std::vector<void*> rk(model->layer_count), rv(model->layer_count);
     for (uint32_t l = 0; l < model->layer_count; ++l) {
         if (!model->layers[l].ring_k || !model->layers[l].ring_v) return fail(GUFFIN_E_ARG, "draft_plan_init: every layer needs its rings");
@@ -240,15 +265,17 @@ extern "C" int guffin_hip_draft_plan_init(void* stream, guffin_draft_plan* plan,
 // Forgets the prefix (reset(), gemma3_draft.hpp:63): ring contents stay but no row of them is referenced.
 extern "C" int guffin_hip_draft_plan_reset(void* stream, guffin_draft_plan* plan) {
     if (!plan || !plan->model || !plan->workspace) return fail(GUFFIN_E_ARG, "draft_plan_reset: null pointer");
-    const Buffers b = carve(*plan->model, plan->workspace, nullptr);
+    const Buffers b = carve(plan);
     hipStream_t s = as_stream(stream);
     if (hipMemsetAsync(b.status, 0, 4, s) != hipSuccess || hipStreamSynchronize(s) != hipSuccess)
         return fail(GUFFIN_E_HIP, "draft_plan_reset: clearing the status failed");
     const guffin_model_desc* model = plan->model;
     void* workspace = plan->workspace;
     const uint64_t bytes = plan->workspace_bytes;
+    const uint32_t rows = plan->transaction_rows, arena = plan->transaction_arena;
     std::memset(plan, 0, sizeof(*plan));
     plan->model = model; plan->workspace = workspace; plan->workspace_bytes = bytes;
+    plan->transaction_rows = rows; plan->transaction_arena = arena;
     return GUFFIN_OK;
 }
 
@@ -265,7 +292,7 @@ static int copy_frontier(hipStream_t s, const guffin_model_desc& m, const Buffer
 extern "C" int guffin_hip_draft_plan_begin_transaction(void* stream, guffin_draft_plan* plan) {
     GUFFIN_TRY(usable(plan, "draft_plan_begin_transaction: null pointer"));
     if (plan->transaction_active) return fail(GUFFIN_E_STATE, "draft_plan_begin_transaction: a transaction is already open");
-    if (plan->hidden_valid) GUFFIN_TRY(copy_frontier(as_stream(stream), *plan->model, carve(*plan->model, plan->workspace, nullptr), true));
+    if (plan->hidden_valid) GUFFIN_TRY(copy_frontier(as_stream(stream), *plan->model, carve(plan), true));
     plan->checkpoint_hidden_valid = plan->hidden_valid;
     plan->checkpoint_last_rows = plan->last_rows;
     plan->checkpoint_position = plan->position;
@@ -282,7 +309,7 @@ extern "C" int guffin_hip_draft_plan_abort_transaction(void* stream, guffin_draf
     // outside a transaction the reference's abort poisons the plan (gemma3_draft.mm:1305-1312): there is nothing to
     // go back to, and the caller's ledger is out of step with the plan's
     if (!plan->transaction_active) { plan->poisoned = 1; return fail(GUFFIN_E_STATE, "draft_plan_abort_transaction: no transaction is open; the plan is poisoned"); }
-    const Buffers b = carve(*plan->model, plan->workspace, nullptr);
+    const Buffers b = carve(plan);
     hipStream_t s = as_stream(stream);
     if (int rc = move_rows(s, plan, b, plan->checkpoint_materialized, plan->backup_end, false)) { plan->poisoned = 1; return rc; }
     GUFFIN_TRY(finish(s, plan, b, "draft_plan_abort_transaction: restoring the ring rows failed"));
@@ -313,13 +340,28 @@ extern "C" int guffin_hip_draft_plan_truncate(void* stream, guffin_draft_plan* p
         return fail(GUFFIN_E_STATE, "draft_plan_truncate: only rows written inside the open transaction can be dropped");
     if (position == plan->position) return GUFFIN_OK;
     if (position < plan->materialized) {
-        const Buffers b = carve(*plan->model, plan->workspace, nullptr);
+        const Buffers b = carve(plan);
         hipStream_t s = as_stream(stream);
         if (int rc = move_rows(s, plan, b, position, plan->backup_end, false)) { plan->poisoned = 1; return rc; }
         GUFFIN_TRY(finish(s, plan, b, "draft_plan_truncate: restoring the ring rows failed"));
         plan->backup_end = std::min(plan->backup_end, position);
         plan->materialized = position;
         plan->hidden_valid = plan->logits_valid = 0;
+        // the frontier's final state: a row this transaction ran, or the one the transaction began on
+        const guffin_model_desc& m = *plan->model;
+        if (position > plan->checkpoint_materialized) {
+            const float* kept = b.txn_hidden + uint64_t(position - 1 - plan->checkpoint_materialized) * m.hidden;
+            if (hipMemcpyAsync(b.hidden, kept, uint64_t(m.hidden) * 4, hipMemcpyDeviceToDevice, s) != hipSuccess)
+                return poison(plan, GUFFIN_E_HIP, "draft_plan_truncate: restoring the frontier's state failed");
+            if (int rc = guffin_hip_group_sums(s, b.hidden, b.hidden_sums, 1, m.hidden)) { plan->poisoned = 1; return rc; }
+            plan->last_rows = 1;
+            plan->hidden_valid = 1;
+        } else if (plan->checkpoint_hidden_valid) {
+            if (int rc = copy_frontier(s, m, b, false)) { plan->poisoned = 1; return rc; }
+            plan->last_rows = plan->checkpoint_last_rows;
+            plan->hidden_valid = 1;
+        }
+        GUFFIN_TRY(finish(s, plan, b, "draft_plan_truncate: restoring the frontier's state failed"));
     }
     plan->has_pending = 0;    // position <= materialized now: whatever was pending lay beyond it
     plan->position = position;
@@ -344,7 +386,7 @@ extern "C" int guffin_hip_draft_plan_append(void* stream, guffin_draft_plan* pla
     for (uint32_t i = 0; i < count; ++i)
         if (tokens[i] >= plan->model->vocab) return fail(GUFFIN_E_ARG, "draft_plan_append: token outside the vocabulary");
     GUFFIN_TRY(capacity_check(plan, count + (plan->has_pending ? 1u : 0u), "draft_plan_append: the context is full"));
-    const Buffers b = carve(*plan->model, plan->workspace, nullptr);
+    const Buffers b = carve(plan);
     hipStream_t s = as_stream(stream);
     GUFFIN_TRY(ingest(s, plan, b, tokens, count));
     return finish(s, plan, b, "draft_plan_append: the pass raised the device status");
@@ -378,12 +420,14 @@ extern "C" int guffin_hip_draft_plan_propose(void* stream, guffin_draft_plan* pl
     if (horizon == 0 || horizon > kMaxHorizon) return fail(GUFFIN_E_CAPACITY, "draft_plan_propose: the horizon must be in [1, 23]");
     if (history_count > 64 || (history_count && !history)) return fail(GUFFIN_E_ARG, "draft_plan_propose: at most 64 history tokens");
     if (plan->materialized == 0) return fail(GUFFIN_E_STATE, "draft_plan_propose: no prefix to draft from");
+    if (!plan->has_pending && !plan->hidden_valid && !plan->logits_valid)   // a state error, not a fault: nothing is poisoned
+        return fail(GUFFIN_E_STATE, "draft_plan_propose: no pass stands at the current frontier (append a token first)");
     GUFFIN_TRY(capacity_check(plan, horizon - 1 + (plan->has_pending ? 1u : 0u), "draft_plan_propose: the context is full"));
     struct Options { float temperature; uint32_t top_k; float top_p, min_p, repetition_penalty; };
     Options opt;
     std::memcpy(&opt, options, sizeof(opt));
     const guffin_model_desc& m = *plan->model;
-    const Buffers b = carve(m, plan->workspace, nullptr);
+    const Buffers b = carve(plan);
     hipStream_t s = as_stream(stream);
     if (plan->has_pending) GUFFIN_TRY(ingest(s, plan, b, nullptr, 0));
     std::vector<Draws> draws(horizon);
@@ -427,7 +471,7 @@ extern "C" int guffin_hip_draft_plan_propose(void* stream, guffin_draft_plan* pl
 extern "C" int guffin_hip_draft_plan_read_logits(void* stream, guffin_draft_plan* plan, float* logits_host) {
     GUFFIN_TRY(usable(plan, "draft_plan_read_logits: null pointer"));
     if (!logits_host) return fail(GUFFIN_E_ARG, "draft_plan_read_logits: null pointer");
-    const Buffers b = carve(*plan->model, plan->workspace, nullptr);
+    const Buffers b = carve(plan);
     hipStream_t s = as_stream(stream);
     GUFFIN_TRY(ensure_logits(s, plan, b));
     GUFFIN_TRY(finish(s, plan, b, "draft_plan_read_logits: the head raised the device status"));

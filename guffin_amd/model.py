@@ -605,7 +605,7 @@ class DraftPlanDesc(C.Structure):
                 ("position", "materialized", "pending_token", "has_pending", "transaction_active", "poisoned",
                  "checkpoint_position", "checkpoint_materialized", "checkpoint_pending", "checkpoint_has_pending",
                  "backup_end", "last_rows", "logits_valid", "hidden_valid", "checkpoint_hidden_valid",
-                 "checkpoint_last_rows")]
+                 "checkpoint_last_rows", "transaction_rows", "transaction_arena")]
 
 
 class DraftPlan:
@@ -613,17 +613,20 @@ class DraftPlan:
     (include/local_gguf_engine/engine/gemma3_draft.hpp:56-82) over guffin_hip_draft_plan_*.  State errors
     raise hip.GuffinError with the C code (GUFFIN_E_STATE = -6, capacity -4, argument -1)."""
 
-    def __init__(self, drafter):
+    def __init__(self, drafter, transaction_rows=0):
+        """transaction_rows: positions one transaction may write (the reference's constructor argument,
+        src/engine/gemma3_draft.mm:648-657); 0 = 32."""
         self.drafter = drafter
         lib = hip.lib()
         lib.guffin_hip_draft_plan_bytes.restype = C.c_uint64
-        need = lib.guffin_hip_draft_plan_bytes(C.byref(drafter.desc))
+        need = lib.guffin_hip_draft_plan_bytes(C.byref(drafter.desc), C.c_uint32(transaction_rows))
         if need == 0:
-            raise ValueError("the model cannot carry a draft plan (head tiles and rings are required)")
+            raise ValueError("the model cannot carry a draft plan of this transaction capacity (head tiles and rings "
+                             "are required; a transaction holds 25 rows or more and fits the smallest ring)")
         self.workspace = torch.zeros(int(need), dtype=torch.uint8, device="cuda")
         self.desc = DraftPlanDesc()
         hip.check(lib.guffin_hip_draft_plan_init(hip._stream(), C.byref(self.desc), C.byref(drafter.desc),
-                                                 hip._p(self.workspace), C.c_uint64(need)))
+                                                 hip._p(self.workspace), C.c_uint64(need), C.c_uint32(transaction_rows)))
 
     position = property(lambda self: self.desc.position)
     materialized_position = property(lambda self: self.desc.materialized)

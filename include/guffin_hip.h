@@ -570,9 +570,13 @@ int guffin_hip_h1_full_cdf(const guffin_h1_desc* desc, void* scratch, uint64_t**
  * rings: a prefix of `position` tokens of which `materialized` have K/V rows (a pending token, the drafter's
  * last emission or one restored by the caller, is run only when the next input needs it), and transactions
  * whose rows can be taken back.  Each call below names the method it replaces.  A transaction's rows go to
- * the rings at once; the ring rows they overwrite are saved per position (at most 32 positions per
- * transaction; the reference's arena holds 96 or 256) and copied back by abort, truncate and a commit of a
- * shorter prefix.  Tokens run through the decode path one row per pass, so a token's rows and logits do not
+ * the rings at once; the ring rows they overwrite are saved per position and copied back by abort, truncate
+ * and a commit of a shorter prefix, and the final normalised row of every position a transaction runs is kept
+ * (the reference's private_norm, src/engine/gemma3_draft.mm:966-968, 984-992), so logits can be read and
+ * proposals drafted at a frontier that a truncate or a shorter commit went back to.  transaction_rows is the
+ * reference's constructor argument of that name (:648-657): how many positions one transaction may write, at
+ * least the largest horizon + 2 = 25 and, rounded up to a power of two, at most the smallest ring; 0 = 32.
+ * Tokens run through the decode path one row per pass, so a token's rows and logits do not
  * depend on how appends were grouped and a commit equals a replay bit for bit.  Every call returns when its device work is done; errors: GUFFIN_E_STATE for a call
  * the state does not admit (nested transaction, truncation of published rows, a second pending token, a
  * poisoned plan), GUFFIN_E_CAPACITY / GUFFIN_E_ARG raised before any state changes, GUFFIN_E_NUMERIC when a pass
@@ -580,14 +584,15 @@ int guffin_hip_h1_full_cdf(const guffin_h1_desc* desc, void* scratch, uint64_t**
  * after `workspace_bytes` belong to the library. */
 typedef struct guffin_draft_plan {
     const guffin_model_desc* model;   /* the drafter, with head_tiles and every layer's rings */
-    void* workspace; uint64_t workspace_bytes;   /* device, guffin_hip_draft_plan_bytes(model), 256-byte aligned */
+    void* workspace; uint64_t workspace_bytes;   /* device, guffin_hip_draft_plan_bytes(model, transaction_rows), 256-byte aligned */
     uint32_t position, materialized, pending_token, has_pending, transaction_active, poisoned;
     uint32_t checkpoint_position, checkpoint_materialized, checkpoint_pending, checkpoint_has_pending;
     uint32_t backup_end, last_rows, logits_valid, hidden_valid, checkpoint_hidden_valid, checkpoint_last_rows;
+    uint32_t transaction_rows, transaction_arena;
 } guffin_draft_plan;
-uint64_t guffin_hip_draft_plan_bytes(const guffin_model_desc* model);
+uint64_t guffin_hip_draft_plan_bytes(const guffin_model_desc* model, uint32_t transaction_rows);   /* 0: not a model or a capacity a plan can have */
 int guffin_hip_draft_plan_init(void* stream, guffin_draft_plan* plan, const guffin_model_desc* model, void* workspace,
-                               uint64_t workspace_bytes);
+                               uint64_t workspace_bytes, uint32_t transaction_rows);
 int guffin_hip_draft_plan_reset(void* stream, guffin_draft_plan* plan);                        /* reset() */
 int guffin_hip_draft_plan_begin_transaction(void* stream, guffin_draft_plan* plan);                        /* begin_transaction() */
 int guffin_hip_draft_plan_commit_prefix(void* stream, guffin_draft_plan* plan, uint32_t position);   /* commit_prefix() */

@@ -294,3 +294,87 @@ def test_truncate_and_abort_outside_a_transaction(hip, scaled_world):
     plan.reset()
     plan.append([ROOT])
     assert plan.position == 1 and not plan.poisoned
+
+
+def test_logits_and_proposals_at_a_frontier_a_transaction_went_back_to(hip, scaled_world):
+    """gemma3_draft.mm:984-992: inside a transaction the head projects from the kept final state of the row at the
+    frontier, so after a truncate or a shorter commit logits can be read and proposals drafted without another
+    token; each equals a plain replay of the kept tokens bit for bit."""
+    from guffin_amd import model
+    shape, host, device = scaled_world
+    prompt = stream(20)
+    words = [0] * 23
+    replica = model.DeviceModel.from_host(host)         # the same weights over rings of its own, for the replays
+
+    def replay_logits(tokens):
+        fresh = model.DraftPlan(replica)
+        fresh.append(tokens)
+        return fresh.read_logits().copy(), fresh
+
+    plan = model.DraftPlan(device)
+    plan.append(prompt)
+    plan.begin_transaction()
+    plan.append([ROOT])
+    drafted = plan.propose(words[:4], greedy(hip))
+    assert plan.materialized_position == 24 and plan.position == 25
+    plan.truncate(23)                                   # keeps ROOT and two drafts, all of them run
+    assert plan.position == 23 and plan.materialized_position == 23 and not plan.poisoned
+    want, fresh = replay_logits(prompt + [ROOT] + drafted[:2])
+    assert np.array_equal(plan.read_logits().view(np.uint32), want.view(np.uint32))
+    fresh.begin_transaction()
+    again = plan.propose(words[:2], greedy(hip))        # drafts from the truncated frontier
+    assert again == fresh.propose(words[:2], greedy(hip)) and again[0] == drafted[2]
+    plan.truncate(21)                                   # back to ROOT alone
+    want, _ = replay_logits(prompt + [ROOT])
+    assert np.array_equal(plan.read_logits().view(np.uint32), want.view(np.uint32))
+    plan.truncate(20)                                   # back to where the transaction began
+    want, _ = replay_logits(prompt)
+    assert np.array_equal(plan.read_logits().view(np.uint32), want.view(np.uint32))
+    plan.append([ROOT])
+    drafted = plan.propose(words[:3], greedy(hip))
+    plan.commit_prefix(22)                              # a shorter commit: ROOT and the first draft
+    assert not plan.transaction_active and plan.position == 22 and plan.materialized_position == 22
+    want, _ = replay_logits(prompt + [ROOT, drafted[0]])
+    assert np.array_equal(plan.read_logits().view(np.uint32), want.view(np.uint32))
+    plan.begin_transaction()
+    assert plan.propose(words[:1], greedy(hip)) == [drafted[1]]
+    plan.abort_transaction()
+    assert np.array_equal(plan.read_logits().view(np.uint32), want.view(np.uint32)) and not plan.poisoned
+
+
+def test_a_frontier_with_no_pass_is_a_state_error_that_poisons_nothing(hip, scaled_world):
+    from guffin_amd import model
+    shape, host, device = scaled_world
+    plan = model.DraftPlan(device)
+    plan.begin_transaction()
+    refuses(hip, lambda: plan.propose([0], greedy(hip)), -6)      # nothing materialized
+    refuses(hip, plan.read_logits, -6)
+    assert not plan.poisoned
+    plan.append([ROOT])
+    assert plan.propose([0, 0], greedy(hip)) and not plan.poisoned
+
+
+def test_the_transaction_capacity_is_the_callers(hip, scaled_world):
+    """The reference's constructor takes the transaction capacity (gemma3_draft.mm:648-657: at least the horizon
+    + 2); here it also has to fit the smallest ring, 64 rows in this world."""
+    from guffin_amd import model
+    shape, host, device = scaled_world
+    for rows in (24, 65, 1 << 20):
+        with pytest.raises(ValueError):
+            model.DraftPlan(device, transaction_rows=rows)
+    plan = model.DraftPlan(device, transaction_rows=48)
+    plan.append(stream(70))                              # beyond the local window: the transaction overwrites live ring rows
+    before, logits = snapshot(plan, shape), plan.read_logits().copy()
+    plan.begin_transaction()
+    plan.append(stream(40))
+    refuses(hip, lambda: plan.append(stream(9)), -4)     # 49 rows
+    plan.append(stream(8))
+    assert plan.position == 118
+    plan.truncate(100)
+    want = model.DraftPlan(model.DeviceModel.from_host(host))     # the same weights over rings of its own
+    want.append(stream(70) + stream(40)[:30])
+    assert np.array_equal(plan.read_logits().view(np.uint32), want.read_logits().view(np.uint32))
+    assert same_caches(snapshot(plan, shape), snapshot(want, shape))
+    plan.abort_transaction()
+    assert plan.position == 70 and same_caches(snapshot(plan, shape), before)
+    assert np.array_equal(plan.read_logits().view(np.uint32), logits.view(np.uint32))
