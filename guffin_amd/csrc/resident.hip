@@ -1031,6 +1031,24 @@ static ResidentSizes resident_sizes(const guffin_model_desc& m, uint32_t rows, u
     return s;
 }
 
+// Where the regions of one block's set start: q/k/v parts, attention outputs, attention (maximum, denominator)
+// pairs, o planes, down planes, the two norm joints' vectors, the GeGLU receipt.  Regions are handed over in
+// different phases, between CUs whose L1 nothing invalidates: each starts on a 256-byte boundary of the set
+// (two cache lines), so no line holds words of two regions.
+struct ResidentLayout { uint64_t offset[8], bytes[8]; };
+
+static ResidentLayout resident_layout(const ResidentSizes& s) {
+    ResidentLayout at {};
+    const uint64_t sizes[8] = {s.qkv, s.attn_out, s.attn_ml, s.o_planes, s.d_planes, s.vec, s.vec, s.h_receipt};
+    uint64_t p = 0;
+    for (int i = 0; i < 8; ++i) {
+        at.offset[i] = p;
+        at.bytes[i] = sizes[i];
+        p += sizes[i];
+    }
+    return at;
+}
+
 uint32_t resident_lds_bytes(const guffin_model_desc& m, uint32_t rows, uint32_t max_ring_tokens) {
     return resident_sizes(m, rows, max_ring_tokens).lds;
 }
@@ -1087,14 +1105,14 @@ int resident_launch(hipStream_t stream, const guffin_model_desc& m, uint32_t row
     }
     a.layers = count; a.H = m.hidden; a.F = m.ffn; a.kv_heads = m.kv_heads;
     a.eps = m.eps; a.scale = 1.0f / std::sqrt(static_cast<float>(m.head_dim));
-    uint8_t* p = exchange;
-    a.qkv_part = reinterpret_cast<float*>(p); p += s.qkv;
-    a.attn_out = reinterpret_cast<float*>(p); p += s.attn_out;
-    a.attn_ml = reinterpret_cast<float*>(p); p += s.attn_ml;
-    a.o_planes = reinterpret_cast<float*>(p); p += s.o_planes;
-    a.d_planes = reinterpret_cast<float*>(p); p += s.d_planes;
-    a.vec = reinterpret_cast<float*>(p); p += 2 * s.vec;
-    a.h_receipt = p; p += s.h_receipt;
+    const ResidentLayout at = resident_layout(s);
+    a.qkv_part = reinterpret_cast<float*>(exchange + at.offset[0]);
+    a.attn_out = reinterpret_cast<float*>(exchange + at.offset[1]);
+    a.attn_ml = reinterpret_cast<float*>(exchange + at.offset[2]);
+    a.o_planes = reinterpret_cast<float*>(exchange + at.offset[3]);
+    a.d_planes = reinterpret_cast<float*>(exchange + at.offset[4]);
+    a.vec = reinterpret_cast<float*>(exchange + at.offset[5]);     // the second joint's follows at vec_floats
+    a.h_receipt = exchange + at.offset[7];
     a.sync = sync_words;
     a.x_in = x_in; a.u_receipt_in = u_receipt_in; a.x_out = x_out; a.u_out = u_out; a.u_receipt_out = u_receipt_out;
     a.ancestors = ancestors; a.status = status;
@@ -1126,6 +1144,21 @@ extern "C" int guffin_hip_set_forward_mode(int mode) {
 }
 
 extern "C" int guffin_hip_resident_enabled(void) { return g_resident_off ? 0 : 1; }
+
+extern "C" int guffin_hip_resident_layout(const guffin_model_desc* model, uint32_t rows, uint64_t* offsets, uint64_t* bytes,
+                                          uint64_t* set_bytes, uint32_t* sets, uint64_t* total_bytes) {
+    if (!model || !model->layers || !offsets || !bytes || !set_bytes || !sets || !total_bytes || rows < 1 || rows > 2)
+        return fail(GUFFIN_E_ARG, "resident_layout: null pointer or rows outside [1, 2]");
+    if (model->kv_heads == 0 || model->q_heads % model->kv_heads != 0 || model->hidden % 64 != 0)
+        return fail(GUFFIN_E_SHAPE, "resident_layout: not a shape the resident pass is laid out for");
+    const ResidentSizes s = resident_sizes(*model, rows, model->ring_global);
+    const ResidentLayout at = resident_layout(s);
+    for (int i = 0; i < 8; ++i) { offsets[i] = at.offset[i]; bytes[i] = at.bytes[i]; }
+    *set_bytes = s.set;
+    *sets = kResidentLayers;
+    *total_bytes = s.total;
+    return GUFFIN_OK;
+}
 
 extern "C" int guffin_hip_set_spin_limit(uint32_t polls) {
     g_spin_limit = polls;

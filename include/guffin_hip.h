@@ -460,6 +460,13 @@ int guffin_hip_forward_tree_rows(void* stream, const guffin_model_desc* model, c
  * drafter plan, whose calls are host-synchronous, also runs the pass that gave up once more, per operator. */
 int guffin_hip_set_forward_mode(int mode);
 int guffin_hip_resident_enabled(void);
+/* Host only: where the resident pass puts the eight exchange regions of one block inside its scratch (q/k/v
+ * parts, attention outputs, attention maxima and denominators, o planes, down planes, the two norm joints'
+ * vectors, the GeGLU receipt), how long one block's set is, how many sets a launch has (one per block it runs,
+ * so that no address is read twice in a launch) and the whole scratch.  Regions are handed over between CUs in
+ * different phases, so each starts on a 256-byte boundary; tests hold the layout to that. */
+int guffin_hip_resident_layout(const guffin_model_desc* model, uint32_t rows, uint64_t* offsets /* [8] */, uint64_t* bytes /* [8] */,
+                               uint64_t* set_bytes, uint32_t* sets, uint64_t* total_bytes);
 int guffin_hip_set_spin_limit(uint32_t polls);
 /* Profiling aid: with a device buffer of 16 * blocks u64 words set, workgroup 0 of the resident pass stores the
  * 100 MHz clock at the start of each block's q/k/v projection, attention, o-projection, first norm pair,
