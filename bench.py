@@ -14,8 +14,8 @@ Extra objects on the JSON line:
                 (3.2 GB, far beyond the caches) on the launch stream; min / max over the replays and
                 over single launches; `traffic` is read from the committed counter profile.
   rooflines     the same figures for the step's other streaming kernels worth watching: the local
-                layers' attention (the kernel furthest from its bound), the down projection, the q/k/v
-                launch and the o projection.
+                layers' attention (the kernel furthest from its bound) and the global layers', the down
+                projection, the q/k/v launch, the o projection and the two head GEMVs.
   configs       configs 0-3 on their own (one Q4_K GEMV at 1 row; one block's seven GEMVs at 2 rows;
                 the drafter's decode with head and argmax; the Q6_K head with selection and
                 acceptance): microseconds per unit as HIP graphs, algorithmic bytes, GB/s and the
@@ -530,6 +530,39 @@ def main():
                                      "with its partition merge" % ring_tokens, local_attention, locals_, attention_bytes,
                                      "attn_partial_kernel<2, 2, 256> (local layer")
 
+    print("bench: timing the global layers' attention and the two heads", file=sys.stderr, flush=True)
+    globals_ = [l for l in every if not T.is_local(l)]
+    g_table = hip.rope_table(positions, T.head_dim, T.global_base, T.global_scale)
+    g_schedule = torch.tensor([[0, t_pos, 0, row + 1] for row in range(2)], dtype=torch.int32, device="cuda")
+
+    def global_attention(l):
+        hip.qkv_attention(q_raw, k_raw, v_raw, q_norm, k_norm, g_table, target.ring_k[l], target.ring_v[l], g_schedule, ancestors,
+                          t_pos + 2, T.ring_global - 1, T.q_heads, T.kv_heads, T.head_dim, T.head_dim ** -0.5)
+
+    g_attention_bytes = t_pos * KW * 2 * 2 + planes * 2 * (QW + 2 * KW) * 4 + 2 * QW * 4
+    g_attention_line = kernel_roofline("qkv attention of a global layer (2 rows, 16 query / 8 KV heads, %d tokens, fp16 K/V) with its "
+                                       "partition merge" % t_pos, global_attention, globals_, g_attention_bytes,
+                                       "attn_partial_kernel<2, 2, 256> (global layer")
+    # the two heads: one matrix each (far larger than the caches), so the graph launches it eight times over
+    xt = torch.randn(2, H, device="cuda")
+    xts = hip.group_sums(xt)
+    t_logits = torch.empty(2, T.vocab, device="cuda")
+    head_dt = int(T.embed_dtype)
+    t_parts = torch.empty((hip.gemv_packed_slices(head_dt, H, T.vocab), 2, T.vocab), device="cuda")
+    t_head_line = kernel_roofline("gemv_packed_kernel<Q6_K, 2> (target head, 262144 x 3840, 2 rows)",
+                                  lambda l: hip.check(lib.guffin_hip_gemv_packed(hip._stream(), head_dt, hip._p(target.head_tiles), hip._p(xt),
+                                                                                 hip._p(xts), hip._p(t_parts), hip._p(t_logits), 2, H, T.vocab)),
+                                  [0] * 8, T.head_bytes() + 2 * H * 4 + 2 * T.vocab * 4, "gemv_packed_kernel<Q6_K, 2> (target head")
+    xd = torch.randn(1, D.hidden, device="cuda")
+    xds = hip.group_sums(xd)
+    d_logits = torch.empty(1, D.vocab, device="cuda")
+    d_head_dt = int(D.embed_dtype)
+    d_parts = torch.empty((hip.gemv_packed_slices(d_head_dt, D.hidden, D.vocab), 1, D.vocab), device="cuda")
+    d_head_line = kernel_roofline("gemv_packed_kernel<Q8_0, 1> (drafter head, 262144 x 640, 1 row)",
+                                  lambda l: hip.check(lib.guffin_hip_gemv_packed(hip._stream(), d_head_dt, hip._p(drafter.head_tiles), hip._p(xd),
+                                                                                 hip._p(xds), hip._p(d_parts), hip._p(d_logits), 1, D.hidden, D.vocab)),
+                                  [0] * 8, D.head_bytes() + D.hidden * 4 + D.vocab * 4, "gemv_packed_kernel<Q8_0, 1> (drafter head")
+
     # a plain 256 MiB device copy: the reference reading for FETCH_SIZE / WRITE_SIZE counter runs
     cal_src = torch.empty(64 << 20, dtype=torch.float32, device="cuda").fill_(1.0)
     cal_dst = torch.empty_like(cal_src)
@@ -552,7 +585,7 @@ def main():
             "accepted": int(first["accepted"]),
         },
         "roofline": roofline,
-        "rooflines": [attention_line, down_line, qkv_line, o_line],
+        "rooflines": [attention_line, g_attention_line, down_line, qkv_line, o_line, t_head_line, d_head_line],
         "chain": chain_figure,
     }
     line["configs"] = config_figures(target, drafter, T, D, d_pos)
