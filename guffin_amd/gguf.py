@@ -115,7 +115,7 @@ class Reader:
                                  else _scalar(e.element_type, bits.value))
             else:
                 value = _scalar(e.type, e.bits)
-            out.append((e.key.decode(), e.type, value))
+            out.append((e.key.decode("utf-8", "replace"), e.type, value))
         return out
 
     def metadata(self):
@@ -126,7 +126,7 @@ class Reader:
         for i in range(self.info.parsed_tensors):
             t = TensorInfo()
             assert lib.guffin_gguf_tensor(self._h, C.c_uint64(i), C.byref(t)) == 0
-            out.append({"name": t.name.decode(), "dims": [int(t.dims[d]) for d in range(t.n_dims)], "type_id": t.type_id,
+            out.append({"name": t.name.decode("utf-8", "replace"), "dims": [int(t.dims[d]) for d in range(t.n_dims)], "type_id": t.type_id,
                         "offset": t.offset, "file_offset": t.file_offset, "byte_count": t.byte_count})
         return out
 
@@ -155,7 +155,7 @@ class Reader:
     def tensor_at(self, index):
         t = TensorInfo()
         assert hip.lib().guffin_gguf_tensor(self._h, C.c_uint64(index), C.byref(t)) == 0
-        return {"name": t.name.decode(), "dims": [int(t.dims[d]) for d in range(t.n_dims)], "type_id": t.type_id,
+        return {"name": t.name.decode("utf-8", "replace"), "dims": [int(t.dims[d]) for d in range(t.n_dims)], "type_id": t.type_id,
                 "offset": t.offset, "file_offset": t.file_offset, "byte_count": t.byte_count}
 
     def payload(self, name):

@@ -165,3 +165,52 @@ def test_arguments(gguf):
     assert hip.lib().guffin_gguf_open(None, C.c_uint64(0), 7, C.byref(handle)) == -1
     with pytest.raises(gguf.ReadError):
         gguf.Reader(np.zeros(0, np.uint8), gguf.STAGE_HEADER)
+
+
+def test_damaged_images_end_in_a_defined_error(gguf):
+    """The reader validates every count and offset before it uses it (src/model_format/gguf_reader.cpp walks the
+    file the same way): flipped bytes, truncations and oversized counts anywhere in the header, metadata and
+    tensor directory of a small model image give one of the 15 error codes or a parse that can be listed and bound
+    (or refused) - never a fault."""
+    from dataclasses import replace
+    from guffin_amd import model
+    from gguf_image import write_gguf
+    shape = replace(model.GEMMA3_270M, layers=1, vocab=256, hidden=64, ffn=128)
+    image = np.array(write_gguf(model.HostModel(shape, seed=1, position=0)))
+    meta_end = int(gguf.Reader(image).info.metadata_end_offset)
+    config = gguf.Gemma3Config()
+    config.block_count, config.embedding_length, config.feed_forward_length, config.vocab_size = 1, 64, 128, 256
+    config.attention_head_count, config.attention_head_count_kv = 4, 1
+    config.attention_key_length = config.attention_value_length = 256
+    config.sliding_window, config.context_length, config.attention_global_layer_period, config.uses_qk_norm = 512, 8192, 6, 1
+    config.rms_norm_epsilon, config.rope_freq_base, config.local_rope_freq_base, config.rope_freq_scale = 1e-6, 1e6, 1e4, 1.0
+    gguf.Reader(image).bind_gemma3(config)
+    rng = np.random.default_rng(0)
+    seen = set()
+    for case in range(3000):
+        data = image.copy()
+        kind = case % 4
+        if kind == 0:
+            for _ in range(rng.integers(1, 4)):
+                data[rng.integers(0, meta_end + 4096)] = rng.integers(0, 256)
+        elif kind == 1:
+            data = data[:rng.integers(0, meta_end + 8192)]
+        elif kind == 2:
+            at = int(rng.integers(0, meta_end))
+            data[at:at + 8] = 0xFF
+        else:
+            data[rng.integers(0, meta_end)] = rng.integers(0, 256)
+            data = data[:rng.integers(meta_end // 2, data.size)]
+        try:
+            reader = gguf.Reader(np.ascontiguousarray(data))
+        except gguf.ReadError as error:
+            assert error.code in gguf.ERRORS, error.code
+            seen.add(error.code)
+            continue
+        assert len(reader.entries()) == reader.info.parsed_entries and len(reader.tensors()) == reader.info.parsed_tensors
+        try:
+            reader.bind_gemma3(config)
+        except gguf.BindError as error:
+            assert error.code in ("missing_tensor", "invalid_tensor")
+            seen.add(error.code)
+    assert {"truncated_metadata", "truncated_tensor_payload", "invalid_metadata_value_type", "truncated_tensor_directory"} <= seen
