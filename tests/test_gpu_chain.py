@@ -87,3 +87,29 @@ def test_calls_out_of_order_are_refused(hip):
     ns = C.c_uint64()
     assert lib.guffin_hip_chain_gpu_ns(chain.handle, C.byref(ns)) == -6      # no replay has run
     chain.close()
+
+
+def test_a_kernel_that_spills_runs_in_a_chain(hip):
+    """The canonical two-row Q4_K GEMV at four columns per wave keeps part of its state in scratch memory (a private
+    segment of 96 bytes per lane); the library's queue gets that memory from the runtime on demand, as a stream's
+    queue does."""
+    import torch
+    from guffin_amd import synth
+    K, N = 4096, 8192
+    w = torch.from_numpy(synth.make_weight(hip.Q4_K, K, N, seed=9)).cuda()
+    x = torch.from_numpy(synth.make_activation(2, K, seed=10)).cuda()
+    want = hip.gemv(hip.Q4_K, w, x, N)
+    torch.cuda.synchronize()
+    out = torch.zeros_like(want)
+    chain = hip.Chain()
+    with chain:
+        hip.gemv(hip.Q4_K, w, x, N, out=out)
+    assert chain.launches() == 1
+    for replay in range(2):
+        out.zero_()
+        torch.cuda.synchronize()
+        print("chain with a private segment, replay", replay, flush=True)
+        chain.launch()
+        chain.wait()
+        assert torch.equal(out, want)
+    chain.close()
