@@ -1057,9 +1057,11 @@ prefill_attention_mfma_kernel(const float* __restrict__ q, const uint16_t* __res
     }
 }
 
-// ring[(position + row) & mask] = run[row] for the rows that survive in a ring of this capacity
-__global__ void publish_run_kernel(const uint4* __restrict__ run_k, const uint4* __restrict__ run_v,
-                                   uint4* __restrict__ ring_k, uint4* __restrict__ ring_v, uint32_t rows,
+// ring[(position + row) & mask] = run[row] for the rows that survive in a ring of this capacity.
+// Rows move as 16-byte pieces asked for at 4-byte alignment: a ring may be a view that starts at any word of its
+// allocation (the reference's caches are, tests/tensor/gemma3_metal_tests.cpp:765-774).
+__global__ void publish_run_kernel(const U4a4* __restrict__ run_k, const U4a4* __restrict__ run_v,
+                                   U4a4* __restrict__ ring_k, U4a4* __restrict__ ring_v, uint32_t rows,
                                    uint32_t first_row, uint32_t position, uint32_t ring_mask, uint32_t row_vec) {
     const uint64_t i = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x;
     if (i >= uint64_t(rows - first_row) * row_vec) return;
@@ -1070,8 +1072,8 @@ __global__ void publish_run_kernel(const uint4* __restrict__ run_k, const uint4*
 }
 
 // dst[(position + t) & dst_mask] = src[(position + t) & src_mask], keys and values
-__global__ void kv_cache_copy_kernel(const uint4* __restrict__ src_k, const uint4* __restrict__ src_v,
-                                     uint4* __restrict__ dst_k, uint4* __restrict__ dst_v, uint32_t tokens,
+__global__ void kv_cache_copy_kernel(const U4a4* __restrict__ src_k, const U4a4* __restrict__ src_v,
+                                     U4a4* __restrict__ dst_k, U4a4* __restrict__ dst_v, uint32_t tokens,
                                      uint32_t position, uint32_t src_mask, uint32_t dst_mask, uint32_t row_vec) {
     const uint64_t i = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x;
     if (i >= uint64_t(tokens) * row_vec) return;
@@ -1095,12 +1097,12 @@ extern "C" int guffin_hip_kv_cache_copy(void* stream, const void* src_k, const v
         return fail(GUFFIN_E_ARG, "kv_cache_copy: row masks must be a power of two minus one");
     if (tokens > src_mask + 1 || tokens > dst_mask + 1) return fail(GUFFIN_E_CAPACITY, "kv_cache_copy: more tokens than rows on one side");
     if (((reinterpret_cast<uintptr_t>(src_k) | reinterpret_cast<uintptr_t>(src_v) | reinterpret_cast<uintptr_t>(dst_k)
-          | reinterpret_cast<uintptr_t>(dst_v)) & 15u) != 0)
-        return fail(GUFFIN_E_ALIGN, "kv_cache_copy: rows must be 16-byte aligned");
+          | reinterpret_cast<uintptr_t>(dst_v)) & 3u) != 0)
+        return fail(GUFFIN_E_ALIGN, "kv_cache_copy: rows must be 4-byte aligned");
     const uint64_t n = uint64_t(tokens) * (row_width / 8);
     launch(kv_cache_copy_kernel, dim3(static_cast<uint32_t>((n + 255) / 256)), dim3(256), 0, as_stream(stream),
-                       static_cast<const uint4*>(src_k), static_cast<const uint4*>(src_v), static_cast<uint4*>(dst_k),
-                       static_cast<uint4*>(dst_v), tokens, position, src_mask, dst_mask, row_width / 8);
+                       static_cast<const U4a4*>(src_k), static_cast<const U4a4*>(src_v), static_cast<U4a4*>(dst_k),
+                       static_cast<U4a4*>(dst_v), tokens, position, src_mask, dst_mask, row_width / 8);
     return check_launch("kv_cache_copy");
 }
 
@@ -1109,11 +1111,14 @@ extern "C" int guffin_hip_publish_run(void* stream, const void* run_k, const voi
     if (!run_k || !run_v || !ring_k || !ring_v) return fail(GUFFIN_E_ARG, "publish_run: null pointer");
     if (rows == 0 || row_width == 0 || row_width % 8 != 0) return fail(GUFFIN_E_SHAPE, "publish_run: row width must be a multiple of 8 halves");
     if ((ring_mask & (ring_mask + 1)) != 0) return fail(GUFFIN_E_ARG, "publish_run: ring capacity must be a power of two");
+    if (((reinterpret_cast<uintptr_t>(run_k) | reinterpret_cast<uintptr_t>(run_v) | reinterpret_cast<uintptr_t>(ring_k)
+          | reinterpret_cast<uintptr_t>(ring_v)) & 3u) != 0)
+        return fail(GUFFIN_E_ALIGN, "publish_run: rows must be 4-byte aligned");
     const uint32_t first = rows > ring_mask + 1 ? rows - (ring_mask + 1) : 0;  // older rows would be overwritten anyway
     const uint64_t n = uint64_t(rows - first) * (row_width / 8);
     launch(publish_run_kernel, dim3(static_cast<uint32_t>((n + 255) / 256)), dim3(256), 0, as_stream(stream),
-                       static_cast<const uint4*>(run_k), static_cast<const uint4*>(run_v), static_cast<uint4*>(ring_k),
-                       static_cast<uint4*>(ring_v), rows, first, position, ring_mask, row_width / 8);
+                       static_cast<const U4a4*>(run_k), static_cast<const U4a4*>(run_v), static_cast<U4a4*>(ring_k),
+                       static_cast<U4a4*>(ring_v), rows, first, position, ring_mask, row_width / 8);
     return check_launch("publish_run");
 }
 

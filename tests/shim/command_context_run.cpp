@@ -211,10 +211,92 @@ int main(int argc, char** argv) {
              << "\nattention_partitions " << stats.decode_attention_partition_count << "\nattention_tokens " << stats.decode_attention_token_count
              << "\n";
 
-        // ---- error paths: the exception classes the engine expects ------------------------------------------------------
+        // ---- a second command buffer: the operators around the pass ----------------------------------------------------
+        // (residual norm, the projections on more than two rows, K/V scatter into the 12-byte views and copy out of them,
+        // prefill attention over them, candidate selection from host-side requests of one and of two rows)
         bool ok = true;
         ok &= throws<std::logic_error>("encode after commit", [&] { context.encode_memory_barrier(); });
         context.restart();
+        constexpr std::uint32_t P = 5;   // rows of the prefill-shaped calls
+        const auto upload_rows = [&](const std::string& name, std::uint64_t n_rows, std::uint64_t width, DType dtype) {
+            const auto bytes = read_file(name);
+            BackendBuffer b = hipctx::allocate_hip_buffer(TensorDescriptor::from(Shape::from({n_rows, width}), dtype));
+            if (bytes.size() != b.descriptor().byte_count) throw std::runtime_error("input has the wrong size: " + name);
+            hipctx::check_hip(hipMemcpy(hipctx::storage(b).device(), bytes.data(), bytes.size(), hipMemcpyHostToDevice), "upload failed");
+            return b;
+        };
+        const BackendBuffer xp = upload_rows("xp.f32", P, H, DType::f32), qp = upload_rows("qp.f32", P, QW, DType::f32);
+        const BackendBuffer chunk_k = upload_rows("chunk_k.f16", P, KW, DType::f16), chunk_v = upload_rows("chunk_v.f16", P, KW, DType::f16);
+        const BackendBuffer selected = upload_words(read_file("selected.u32"));
+        const BackendBuffer y_add = hipctx::allocate_hip_buffer(f32_rows(rows, H));
+        const BackendBuffer yp_matrix = hipctx::allocate_hip_buffer(f32_rows(P, QW)), yp_pairs = hipctx::allocate_hip_buffer(f32_rows(P, QW));
+        const BackendBuffer yv_matrix = hipctx::allocate_hip_buffer(f32_rows(P, KW));
+        const auto copy_desc = TensorDescriptor::from(Shape::from({16, KW}), DType::f16);
+        const BackendBuffer copy_k = hipctx::allocate_hip_buffer(copy_desc), copy_v = hipctx::allocate_hip_buffer(copy_desc);
+        hipctx::check_hip(hipMemset(hipctx::storage(copy_k).device(), 0, copy_desc.byte_count), "clearing failed");
+        hipctx::check_hip(hipMemset(hipctx::storage(copy_v).device(), 0, copy_desc.byte_count), "clearing failed");
+        const BackendBuffer pattn = hipctx::allocate_hip_buffer(f32_rows(P, QW)), pattn_window = hipctx::allocate_hip_buffer(f32_rows(P, QW));
+        const BackendBuffer marks = hipctx::allocate_hip_buffer(words(4));
+        struct SelectionWorkspace { BackendBuffer candidate_runs_a, compact_result; };   // engine::TokenSelectionWorkspace's members
+        const SelectionWorkspace sw {candidate_runs, hipctx::allocate_hip_buffer(words(2 * (8 + 384 * 8) / 4))};
+        std::array<lge::engine::TokenSelectionRequest, 2> requests;
+        requests[0].top_k = 40; requests[0].history_token_count = 3; requests[0].base_candidate_count = 43;
+        requests[0].history_token_ids[0] = 3; requests[0].history_token_ids[1] = 9; requests[0].history_token_ids[2] = 70;
+        requests[1].top_k = 1; requests[1].history_token_count = 0; requests[1].base_candidate_count = 1;
+
+        context.write_u32(marks, 0xC0FFEEu);
+        context.encode_rms_norm_add(u, attn_norm, x0, y_add, eps, rows);
+        context.encode_verifier_matmul(xp, wq, yp_matrix, P, true);     // the matrix-core path
+        context.encode_verifier_matmul(xp, wv, yv_matrix, P, true);     // ... on Q6_K tiles
+        context.encode_verifier_matmul(xp, wq, yp_pairs, P, false);     // pairs of rows through the decode GEMV
+        context.encode_verifier_kv_scatter(priv_k, priv_v, selected, ring_k, ring_v, 40, rows, KW, cap - 1);
+        context.encode_memory_barrier();
+        context.encode_gemma2_kv_cache_copy(ring_k, ring_v, copy_k, copy_v, 30, 12, cap - 1, 15);
+        context.encode_f16_prefill_attention(qp, ring_k, ring_v, chunk_k, chunk_v, pattn, 42, 16, 8, 256, 256, 42 + P, 0.0625F, 0.0F,
+                                             cap - 1, P, true, 42);
+        context.encode_f16_prefill_attention(qp, ring_k, ring_v, chunk_k, chunk_v, pattn_window, 42, 16, 8, 256, 256, 16, 0.0625F, 0.0F,
+                                             cap - 1, P, true, 42);
+        const std::uint32_t launches_two = context.encode_token_candidates_width_two(ws.logits_tile, sw, requests, 0.0F);
+        const hipctx::HipCommandStats second = context.commit_and_wait();
+        const auto pair = context.read_token_candidates_width_two(sw);
+        dump("y_add.out", y_add); dump("yp_matrix.out", yp_matrix); dump("yv_matrix.out", yv_matrix); dump("yp_pairs.out", yp_pairs);
+        dump("ring_k_after.out", ring_k); dump("ring_v_after.out", ring_v); dump("copy_k.out", copy_k); dump("copy_v.out", copy_v);
+        dump("pattn.out", pattn); dump("pattn_window.out", pattn_window); dump("marks.out", marks);
+        const auto write_candidates = [&](const std::string& name, const lge::engine::CompactTokenCandidates& c) {
+            std::vector<std::uint32_t> flat {c.count};
+            for (std::uint32_t i = 0; i < c.count; ++i) {
+                flat.push_back(c.values[i].token);
+                std::uint32_t logit_bits;
+                std::memcpy(&logit_bits, &c.values[i].logit, 4);
+                flat.push_back(logit_bits);
+            }
+            write_file(name, flat.data(), flat.size() * 4);
+        };
+        write_candidates("pair0.out", pair[0]);
+        write_candidates("pair1.out", pair[1]);
+        // a third one: a single row
+        context.restart();
+        const std::uint32_t launches_one = context.encode_token_candidates(ws.logits_tile, sw, requests[0], 0.0F);
+        const hipctx::HipCommandStats third = context.commit_and_wait();
+        write_candidates("single.out", context.read_token_candidates(sw));
+        text << "launches_two " << launches_two << "\nlaunches_one " << launches_one
+             << "\nsecond_command_buffers " << second.command_buffer_count << "\nsecond_commits " << second.commit_count
+             << "\nq4_generic_tiled " << second.q4_generic_tiled_projection_count << "\nq6_generic_tiled " << second.q6_generic_tiled_projection_count
+             << "\nq4_small_batch " << second.q4_small_batch_projection_count << "\nthird_commits " << third.commit_count
+             << "\nthird_gpu_duration_ns " << third.gpu_duration_ns << "\n";
+
+        // ---- error paths: the exception classes the engine expects ------------------------------------------------------
+        ok &= throws<std::logic_error>("encode after the third commit", [&] { context.encode_memory_barrier(); });
+        context.restart();
+        ok &= throws<std::invalid_argument>("prefill attention without a staged chunk", [&] {
+            context.encode_f16_prefill_attention(qp, ring_k, ring_v, chunk_k, chunk_v, pattn, 42, 16, 8, 256, 256, 42 + P, 0.0625F, 0.0F,
+                                                 cap - 1, P, false, 42);
+        });
+        ok &= throws<std::invalid_argument>("a request outside product bounds", [&] {
+            auto bad = requests[0];
+            bad.base_candidate_count = 40;   // not top_k + history
+            (void)context.encode_token_candidates(ws.logits_tile, sw, bad, 0.0F);
+        });
         ok &= throws<std::invalid_argument>("zero rows", [&] { context.encode_verifier_matmul(u, wq, q, 0); });
         ok &= throws<std::invalid_argument>("mismatched inner dimension", [&] { context.encode_verifier_matmul(q, wk, k, rows); });
         ok &= throws<std::invalid_argument>("output too small", [&] { context.encode_verifier_matmul(u, wq, k, rows); });

@@ -4,7 +4,10 @@ operators through HipCommandContext on buffers made by allocate_hip_buffer / vie
 -- embedding, norm with a receipt, the projections with the producer's receipt and with the context's own, head
 norms, rotation, K/V narrowing, attention over K/V views that start 12 bytes into their allocations
 (tests/tensor/gemma3_metal_tests.cpp:765-774), GeGLU, the tied head, request resolution, candidate selection and
-the candidate read-back -- and writes every result to a directory.  Here every result is compared, bit for bit,
+the candidate read-back; then, in a second and a third command buffer, the operators around the pass (residual norm,
+projections on five rows by the matrix path and by pairs of rows, K/V scatter into those views and copy out of them,
+prefill attention over them with and without a window, candidate selection from host-side requests of two rows and of
+one) -- and writes every result to a directory.  Here every result is compared, bit for bit,
 with the same operator called through the C entry points (ctypes) on the same inputs, and with the oracle where a
 tolerance says more than equality.  The program itself checks the exception classes of the error paths."""
 import os
@@ -61,6 +64,16 @@ def test_the_command_context_runs_a_verify_pass(tmp_path):
         raw(os.path.join(d, n + ".f32"), g)
     raw(os.path.join(d, "ring_k.f16"), ring_k); raw(os.path.join(d, "ring_v.f16"), ring_v)
     raw(os.path.join(d, "requests.raw"), requests)
+    # the second command buffer's inputs: five rows for the calls with more than two, a chunk of keys and values
+    P = 5
+    xp = rng.standard_normal((P, H)).astype(np.float32)
+    qp = rng.standard_normal((P, QW)).astype(np.float32)
+    chunk_k = rng.standard_normal((P, KW)).astype(np.float16)
+    chunk_v = rng.standard_normal((P, KW)).astype(np.float16)
+    selected = np.array([1, 0], np.uint32)
+    raw(os.path.join(d, "xp.f32"), xp); raw(os.path.join(d, "qp.f32"), qp)
+    raw(os.path.join(d, "chunk_k.f16"), chunk_k); raw(os.path.join(d, "chunk_v.f16"), chunk_v)
+    raw(os.path.join(d, "selected.u32"), selected)
 
     print("running the command context", flush=True)
     run = subprocess.run([RUNNER, d], capture_output=True, text=True, timeout=120)
@@ -128,3 +141,51 @@ def test_the_command_context_runs_a_verify_pass(tmp_path):
     want_q = gfo.gemv(synth.Q4_K, host["wq.q4k"], u.cpu().numpy(), QW)
     scale = np.sqrt((want_q.astype(np.float64) ** 2).mean())
     assert np.max(np.abs(out("q.out", np.float32).reshape(2, QW) - want_q)) <= 1e-3 * scale
+
+
+    # ---- the second and third command buffers ------------------------------------------------------------------------
+    assert int(stats["launches_two"]) == 2 and int(stats["launches_one"]) == 2
+    assert int(stats["second_command_buffers"]) == 2 and int(stats["second_commits"]) == 2 and int(stats["third_commits"]) == 3
+    assert int(stats["q4_generic_tiled"]) == 1 and int(stats["q6_generic_tiled"]) == 1 and int(stats["q4_small_batch"]) == 3
+    assert int(stats["third_gpu_duration_ns"]) > 0
+    assert int(out("marks.out", np.uint32)[0]) == 0xC0FFEE
+    t_xp, t_qp = torch.from_numpy(xp).cuda(), torch.from_numpy(qp).cuda()
+    y_add = hip.rms_norm(u, gam["attn_norm"], residual=x0, status=status)
+    image = hip.prefill_pack(t_xp)
+    yp_matrix = hip.prefill_gemm(synth.Q4_K, tiles["wq.q4k"], image, P, H, QW)
+    yv_matrix = hip.prefill_gemm(synth.Q6_K, tiles["wv.q6k"], image, P, H, KW)
+    yp_pairs = torch.cat([hip.gemv_packed(synth.Q4_K, tiles["wq.q4k"], t_xp[r:r + 2].contiguous(), hip.group_sums(t_xp[r:r + 2].contiguous()), QW)
+                          for r in range(0, P, 2)])
+    rk, rv = torch.from_numpy(ring_k).cuda(), torch.from_numpy(ring_v).cuda()
+    hip.kv_scatter(priv_k, priv_v, torch.from_numpy(selected.view(np.int32)).cuda(), rk, rv, 40, KW, CAP - 1)
+    ck, cv = torch.zeros((16, KW), dtype=torch.float16, device="cuda"), torch.zeros((16, KW), dtype=torch.float16, device="cuda")
+    hip.kv_cache_copy(rk, rv, ck, cv, 30, 12, CAP - 1, 15)
+    t_ck, t_cv = torch.from_numpy(chunk_k).cuda(), torch.from_numpy(chunk_v).cuda()
+    pattn = hip.prefill_attention(t_qp, rk, rv, t_ck, t_cv, 42, 0, CAP - 1, 16, 8, 256, 0.0625, matrix_core=False)
+    pattn_window = hip.prefill_attention(t_qp, rk, rv, t_ck, t_cv, 42, 16, CAP - 1, 16, 8, 256, 0.0625, matrix_core=False)
+    host_requests = np.zeros(2, hip.resolved_row_dtype)
+    host_requests[0]["top_k"], host_requests[0]["base_candidate_count"], host_requests[0]["history_count"] = 40, 43, 3
+    host_requests[0]["history_token_ids"][:3] = [3, 9, 70]
+    host_requests[1]["top_k"], host_requests[1]["base_candidate_count"] = 1, 1
+    d_requests = torch.from_numpy(host_requests.view(np.uint8).copy()).cuda()
+    pair, pair_status = hip.select_candidates_resolved(logits, 43, d_requests)
+    single, single_status = hip.select_candidates_resolved(logits[:1].contiguous(), 43, d_requests[:hip.resolved_row_dtype.itemsize].contiguous())
+    torch.cuda.synchronize()
+    assert int(status.item()) == 0 and int(pair_status.abs().sum()) == 0 and int(single_status.abs().sum()) == 0
+    assert torch.equal(rk[40], priv_k[1]) and torch.equal(rk[41], priv_k[0]) and torch.equal(ck[(30 + 11) & 15], rk[41])
+    second = {"y_add": y_add, "yp_matrix": yp_matrix, "yv_matrix": yv_matrix, "yp_pairs": yp_pairs, "ring_k_after": rk,
+              "ring_v_after": rv, "copy_k": ck, "copy_v": cv, "pattn": pattn, "pattn_window": pattn_window}
+    for name, tensor in second.items():
+        assert out(name + ".out").tobytes() == bits(tensor), name
+    # rows of the matrix path agree with the decode path's to the operator bound, and the window changes the answer
+    assert float((yp_matrix - yp_pairs).abs().max()) <= 1e-3 * float(yp_pairs.abs().max())
+    assert not torch.equal(pattn, pattn_window)
+    for name, record in (("pair0", hip.candidates_to_numpy(pair)[0]), ("pair1", hip.candidates_to_numpy(pair)[1]),
+                         ("single", hip.candidates_to_numpy(single)[0])):
+        flat = out(name + ".out", np.uint32)
+        count = int(flat[0])
+        assert count == int(record["count"]) and count >= 1
+        assert np.array_equal(flat[1:1 + 2 * count:2], record["values"]["token"][:count])
+        assert np.array_equal(flat[2:2 + 2 * count:2], record["values"]["logit"][:count].view(np.uint32))
+    assert int(out("pair1.out", np.uint32)[0]) == 1 and int(out("pair0.out", np.uint32)[0]) >= 40
+    assert out("single.out").tobytes() == out("pair0.out").tobytes()

@@ -294,3 +294,48 @@ def test_kv_cache_copy_backs_ring_rows_up_and_restores_them(hip):
         hip.kv_cache_copy(ring_k, ring_v, backup_k, backup_v, position, 3, cap - 1, 1)   # three tokens, two rows
     with pytest.raises(hip.GuffinError):
         hip.kv_cache_copy(ring_k, ring_v, backup_k, backup_v, position, 2, 5, 1)         # not a row mask
+
+
+@pytest.mark.parametrize("offset_bytes", [4, 12])
+def test_kv_rows_move_between_views_at_any_word_offset(hip, offset_bytes):
+    """The reference's K/V caches may be views that start at any word of their allocation
+    (tests/tensor/gemma3_metal_tests.cpp:765-774 uses 12 bytes): copies and publications between such views give
+    the bytes the aligned calls give, and touch nothing outside the views; half a word off is refused."""
+    import torch
+    rng = np.random.default_rng(12)
+    cap, width, position = 8, 2048, 6
+    pad = offset_bytes // 2
+
+    def view(rows, fill):
+        parent = torch.full((rows * width + 16,), fill, dtype=torch.float16, device="cuda")
+        return parent, parent[pad:pad + rows * width].view(rows, width)
+
+    ring = rng.normal(0, 1, (2, cap, width)).astype(np.float16)
+    run = rng.normal(0, 1, (2, 3, width)).astype(np.float16)
+    pk, ring_k = view(cap, 7.0)
+    pv, ring_v = view(cap, 7.0)
+    ring_k.copy_(dev(ring[0])); ring_v.copy_(dev(ring[1]))
+    assert ring_k.data_ptr() % 16 == offset_bytes % 16
+    pbk, backup_k = view(4, 5.0)
+    pbv, backup_v = view(4, 5.0)
+    hip.kv_cache_copy(ring_k, ring_v, backup_k, backup_v, position, 3, cap - 1, 3)        # rows 6, 7, 8 -> slots 2, 3, 0
+    _, run_k = view(3, 0.0)
+    _, run_v = view(3, 0.0)
+    run_k.copy_(dev(run[0])); run_v.copy_(dev(run[1]))
+    hip.publish_run(run_k, run_v, ring_k, ring_v, position, cap - 1)
+    # the same on aligned tensors
+    a_ring_k, a_ring_v = dev(ring[0]), dev(ring[1])
+    a_backup_k, a_backup_v = torch.full((4, width), 5.0, dtype=torch.float16, device="cuda"), torch.full((4, width), 5.0, dtype=torch.float16, device="cuda")
+    hip.kv_cache_copy(a_ring_k, a_ring_v, a_backup_k, a_backup_v, position, 3, cap - 1, 3)
+    hip.publish_run(dev(run[0]), dev(run[1]), a_ring_k, a_ring_v, position, cap - 1)
+    torch.cuda.synchronize()
+    assert torch.equal(ring_k, a_ring_k) and torch.equal(ring_v, a_ring_v)
+    assert torch.equal(backup_k, a_backup_k) and torch.equal(backup_v, a_backup_v)
+    assert torch.equal(ring_k[6], dev(run[0][0])) and torch.equal(ring_k[0], dev(run[0][2]))
+    for parent, fill, rows in ((pk, 7.0, cap), (pv, 7.0, cap), (pbk, 5.0, 4), (pbv, 5.0, 4)):
+        assert float((parent[:pad] - fill).abs().sum()) == 0.0 and float((parent[pad + rows * width:] - fill).abs().sum()) == 0.0
+    half_word = pk[1:1 + cap * width].view(cap, width)
+    with pytest.raises(hip.GuffinError):
+        hip.kv_cache_copy(half_word, ring_v, backup_k, backup_v, position, 2, cap - 1, 3)
+    with pytest.raises(hip.GuffinError):
+        hip.publish_run(run_k, run_v, half_word, ring_v, position, cap - 1)
